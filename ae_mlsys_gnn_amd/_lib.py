@@ -1,0 +1,174 @@
+"""ctypes binding of libfgnn_hip.so (the C ABI declared in include/fgnn.h).
+
+There is no CPU fallback: every operator of this package runs the HIP kernels or raises."""
+from __future__ import annotations
+
+import collections
+import ctypes
+import os
+from ctypes import c_float, c_int, c_int64, c_size_t, c_void_p
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libfgnn_hip.so")
+
+_lib = None
+
+
+class FgnnError(RuntimeError):
+    pass
+
+
+_SIGNATURES = {
+    "fgnn_version": (c_int, []),
+    "fgnn_last_error": (ctypes.c_char_p, []),
+    "fgnn_schedule_create": (c_int, [c_void_p, c_int, c_int, c_void_p, ctypes.POINTER(c_void_p)]),
+    "fgnn_schedule_destroy": (None, [c_void_p]),
+    "fgnn_schedule_num_items": (c_int, [c_void_p]),
+    "fgnn_schedule_num_partials": (c_int, [c_void_p]),
+    "fgnn_schedule_num_edges": (c_int64, [c_void_p]),
+    "fgnn_gat_forward_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int]),
+    "fgnn_gat_forward": (c_int, [c_int, c_int64, c_int, c_int] + [c_void_p] * 4 + [c_float] + [c_void_p] * 8
+                         + [c_void_p, c_void_p, c_size_t, c_void_p]),
+    "fgnn_gat_backward_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_void_p, c_void_p, c_int]),
+    "fgnn_gat_backward": (c_int, [c_int, c_int64, c_int, c_int, c_float] + [c_void_p] * 19
+                          + [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "fgnn_edgeconv_forward": (c_int, [c_int, c_int, c_int, c_int] + [c_void_p] * 5 + [c_void_p]),
+    "fgnn_edgeconv_backward": (c_int, [c_int, c_int, c_int] + [c_void_p] * 3 + [c_void_p]),
+    "fgnn_gmm_forward_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int]),
+    "fgnn_gmm_forward": (c_int, [c_int, c_int64, c_int, c_int, c_int] + [c_void_p] * 9
+                         + [c_void_p, c_void_p, c_size_t, c_void_p]),
+    "fgnn_gmm_backward_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int, c_int]),
+    "fgnn_gmm_backward": (c_int, [c_int, c_int64, c_int, c_int, c_int] + [c_void_p] * 12
+                          + [c_void_p, c_void_p, c_size_t, c_void_p]),
+    "fgnn_gaussian": (c_int, [c_int64, c_int, c_int] + [c_void_p] * 4 + [c_void_p]),
+    "fgnn_gaussian_backward": (c_int, [c_int64, c_int, c_int] + [c_void_p] * 7 + [c_void_p]),
+    "fgnn_mhspmm_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int]),
+    "fgnn_mhspmm": (c_int, [c_int, c_int64, c_int, c_int] + [c_void_p] * 6 + [c_void_p, c_void_p, c_size_t, c_void_p]),
+    "fgnn_mhsddmm": (c_int, [c_int, c_int64, c_int, c_int] + [c_void_p] * 5 + [c_void_p]),
+    "fgnn_gather_rows": (c_int, [c_int64, c_int] + [c_void_p] * 3 + [c_void_p]),
+    "fgnn_edge_softmax": (c_int, [c_int, c_int64, c_int] + [c_void_p] * 3 + [c_void_p]),
+    "fgnn_edge_softmax_backward": (c_int, [c_int, c_int64, c_int] + [c_void_p] * 4 + [c_void_p]),
+    "fgnn_u_add_v": (c_int, [c_int, c_int64, c_int] + [c_void_p] * 5 + [c_void_p]),
+    "fgnn_u_add_v_backward": (c_int, [c_int, c_int64, c_int] + [c_void_p] * 5 + [c_void_p]),
+    "fgnn_csr2csc_workspace_bytes": (c_size_t, [c_int, c_int, c_int64]),
+    "fgnn_csr2csc": (c_int, [c_int, c_int, c_int64] + [c_void_p] * 5 + [c_void_p, c_size_t, c_void_p]),
+}
+
+
+def exported_symbols():
+    """Names the C ABI must export (kept in step with include/fgnn.h)."""
+    return sorted(_SIGNATURES)
+
+
+def lib():
+    """The loaded library; raises when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FgnnError(
+                "libfgnn_hip.so is missing at %s; build it with "
+                "`python -m ae_mlsys_gnn_amd.build` (needs hipcc)" % LIB_PATH)
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(rc: int, what: str):
+    if rc != 0:
+        msg = lib().fgnn_last_error().decode("utf-8", "replace")
+        raise FgnnError("%s failed (code %d): %s" % (what, rc, msg))
+
+
+def ptr(t):
+    """Device pointer of a tensor (None -> NULL)."""
+    if t is None:
+        return None
+    return c_void_p(t.data_ptr())
+
+
+def stream_ptr():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def require_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise FgnnError("fgnn operators run on the GPU only (got a %s tensor); there is no CPU path" % t.device)
+
+
+def as_f32(t):
+    if t.dtype != torch.float32:
+        raise FgnnError("expected float32, got %s" % t.dtype)
+    return t.contiguous()
+
+
+def as_i32(t):
+    if t.dtype != torch.int32:
+        raise FgnnError("expected int32 indices, got %s" % t.dtype)
+    return t.contiguous()
+
+
+class Schedule:
+    """Degree-binned work list of one pointer array (row_ptr or col_ptr)."""
+
+    def __init__(self, ptr_tensor, seg_len=0):
+        require_cuda(ptr_tensor)
+        self.ptr_tensor = as_i32(ptr_tensor)      # keeps the device memory alive
+        self.n_rows = self.ptr_tensor.numel() - 1
+        handle = c_void_p()
+        with torch.cuda.device(self.ptr_tensor.device):
+            check(lib().fgnn_schedule_create(ptr(self.ptr_tensor), self.n_rows, int(seg_len), stream_ptr(),
+                                             ctypes.byref(handle)), "fgnn_schedule_create")
+        self.handle = handle
+        self.n_items = lib().fgnn_schedule_num_items(handle)
+        self.n_partials = lib().fgnn_schedule_num_partials(handle)
+        self.n_edges = lib().fgnn_schedule_num_edges(handle)
+
+    def __del__(self):
+        h = getattr(self, "handle", None)
+        if h is not None and _lib is not None:
+            _lib.fgnn_schedule_destroy(h)
+            self.handle = None
+
+
+_sched_cache: "collections.OrderedDict" = collections.OrderedDict()
+_SCHED_CACHE_MAX = 32
+
+
+def default_seg_len() -> int:
+    return int(os.environ.get("FGNN_SEG_LEN", "0"))
+
+
+def schedule_for(ptr_tensor, seg_len=None) -> Schedule:
+    """Cached schedule of a pointer array.  The cache entry holds the tensor, so its device
+    address cannot be reused while the entry lives; in-place edits bump `_version`."""
+    if seg_len is None:
+        seg_len = default_seg_len()
+    key = (ptr_tensor.data_ptr(), ptr_tensor.numel(), ptr_tensor.device.index, ptr_tensor._version, int(seg_len))
+    s = _sched_cache.get(key)
+    if s is None:
+        s = Schedule(ptr_tensor, seg_len)
+        _sched_cache[key] = s
+        while len(_sched_cache) > _SCHED_CACHE_MAX:
+            _sched_cache.popitem(last=False)
+    else:
+        _sched_cache.move_to_end(key)
+    return s
+
+
+def clear_schedule_cache():
+    _sched_cache.clear()
+
+
+def workspace(nbytes: int, device):
+    """A float-aligned scratch tensor of at least nbytes (None when nothing is needed)."""
+    if nbytes <= 0:
+        return None, 0
+    t = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=device)
+    return t, t.numel() * 4

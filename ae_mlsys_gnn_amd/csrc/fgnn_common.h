@@ -1,0 +1,287 @@
+// Shared host/device helpers of libfgnn_hip.so (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include "fgnn.h"
+
+#define FGNN_WAVE 64
+#define FGNN_WPB 4      // waves per workgroup: every wave works on its own item
+#define FGNN_TPB 256
+
+// ------------------------------------------------------------------ host side
+void fgnn_set_error(const char *fmt, ...);
+
+#define FGNN_REQUIRE(cond, code, ...)            \
+    do {                                         \
+        if (!(cond)) {                           \
+            fgnn_set_error(__VA_ARGS__);         \
+            return (code);                       \
+        }                                        \
+    } while (0)
+
+#define FGNN_HIP(call)                                                        \
+    do {                                                                      \
+        hipError_t err__ = (call);                                            \
+        if (err__ != hipSuccess) {                                            \
+            fgnn_set_error("%s failed: %s", #call, hipGetErrorString(err__)); \
+            return (int)err__;                                                \
+        }                                                                     \
+    } while (0)
+
+static inline int fgnn_launch_status(const char *what)
+{
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) {
+        fgnn_set_error("launch of %s failed: %s", what, hipGetErrorString(err));
+        return (int)err;
+    }
+    return 0;
+}
+
+static inline bool fgnn_aligned16(const void *p) { return (((uintptr_t)p) & 15u) == 0; }
+static inline size_t fgnn_align256(size_t x) { return (x + 255) & ~(size_t)255; }
+// Fills n floats with v on `st` (a kernel, so it may be captured into a HIP graph).
+int fgnn_fill_f32(float *p, size_t n, float v, hipStream_t st);
+
+// One work item: the edge range [begin, end) of `row`.  slot < 0: the item covers the whole
+// row and writes final results; slot >= 0: a segment of a split row, written as partial `slot`.
+struct fgnn_item { int row, begin, end, slot; };
+// A split row: its partials are slots [first_slot, first_slot + nseg).
+struct fgnn_split { int row, first_slot, nseg, pad; };
+
+struct fgnn_schedule {
+    int n_rows;
+    int64_t n_edges;
+    int seg_len;
+    int n_items;
+    int n_partials;
+    int n_split;
+    fgnn_item *items_dev;
+    fgnn_split *split_dev;
+    const int32_t *ptr_dev;
+    int device;
+};
+
+// Feature-row layout of the gather kernels: a row of `HF` floats is spread over the 64 lanes
+// of a wave in R slabs of 64*VEC floats; VEC = 4 uses 128-bit loads.
+struct fgnn_rowcfg { int vec; int r; bool full; };
+static inline bool fgnn_pick_rowcfg(int HF, int F, bool aligned, fgnn_rowcfg *c)
+{
+    int vec = (aligned && (F % 4 == 0)) ? 4 : 1;
+    int per = 64 * vec;
+    int need = (HF + per - 1) / per;
+    int r = 1;
+    while (r < need) r *= 2;
+    if ((vec == 4 && r > 4) || (vec == 1 && r > 16)) return false;
+    c->vec = vec; c->r = r; c->full = (HF == per * r);
+    return true;
+}
+
+
+// Calls f.template operator()<VEC, R, FULL>() for the row layout chosen at run time.
+template <typename Fn>
+static inline int fgnn_dispatch_rowcfg(const fgnn_rowcfg &c, Fn &&f)
+{
+    if (c.vec == 4) {
+        if (c.r == 1) return c.full ? f.template operator()<4, 1, true>() : f.template operator()<4, 1, false>();
+        if (c.r == 2) return c.full ? f.template operator()<4, 2, true>() : f.template operator()<4, 2, false>();
+        return c.full ? f.template operator()<4, 4, true>() : f.template operator()<4, 4, false>();
+    }
+    switch (c.r) {
+    case 1: return f.template operator()<1, 1, false>();
+    case 2: return f.template operator()<1, 2, false>();
+    case 4: return f.template operator()<1, 4, false>();
+    case 8: return f.template operator()<1, 8, false>();
+    default: return f.template operator()<1, 16, false>();
+    }
+}
+
+// ------------------------------------------------------------------ device side
+#ifdef __HIPCC__
+__device__ __forceinline__ int fg_lane() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
+__device__ __forceinline__ int fg_wave() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+__device__ __forceinline__ int fg_uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ float fg_readlane(float v, int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l)); }
+__device__ __forceinline__ float fg_bperm(float v, int src_lane) { return __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane << 2, __float_as_int(v))); }
+
+template <int CTRL>
+__device__ __forceinline__ float fg_dpp(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+// Butterfly inside each row of 16 lanes (quad xor 1, quad xor 2, half-row mirror, row mirror),
+// then the four row results are combined through scalar registers.  All lanes get the result.
+__device__ __forceinline__ float fg_wave_max(float v)
+{
+    v = fmaxf(v, fg_dpp<0xB1>(v));
+    v = fmaxf(v, fg_dpp<0x4E>(v));
+    v = fmaxf(v, fg_dpp<0x141>(v));
+    v = fmaxf(v, fg_dpp<0x140>(v));
+    float a = fg_readlane(v, 0), b = fg_readlane(v, 16), c = fg_readlane(v, 32), d = fg_readlane(v, 48);
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+__device__ __forceinline__ float fg_wave_sum(float v)
+{
+    v = v + fg_dpp<0xB1>(v);
+    v = v + fg_dpp<0x4E>(v);
+    v = v + fg_dpp<0x141>(v);
+    v = v + fg_dpp<0x140>(v);
+    float a = fg_readlane(v, 0), b = fg_readlane(v, 16), c = fg_readlane(v, 32), d = fg_readlane(v, 48);
+    return (a + b) + (c + d);
+}
+// Orders LDS traffic between the lanes of ONE wave (each wave owns a private LDS region, LDS
+// instructions of a wave execute in order, so only the compiler has to be held back).
+__device__ __forceinline__ void fg_wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+__device__ __forceinline__ float fg_lrelu(float x, float slope) { return x > 0.f ? x : x * slope; }
+
+template <int VEC> struct fg_vec;
+template <> struct fg_vec<4> {
+    float4 v;
+    __device__ __forceinline__ void zero() { v = make_float4(0.f, 0.f, 0.f, 0.f); }
+    __device__ __forceinline__ void load(const float *p) { v = *reinterpret_cast<const float4 *>(p); }
+    __device__ __forceinline__ void store(float *p) const { *reinterpret_cast<float4 *>(p) = v; }
+    __device__ __forceinline__ void fma(float w, const fg_vec &x) { v.x = fmaf(w, x.v.x, v.x); v.y = fmaf(w, x.v.y, v.y); v.z = fmaf(w, x.v.z, v.z); v.w = fmaf(w, x.v.w, v.w); }
+    __device__ __forceinline__ void add(const fg_vec &x) { v.x += x.v.x; v.y += x.v.y; v.z += x.v.z; v.w += x.v.w; }
+    __device__ __forceinline__ void scale(float w) { v.x *= w; v.y *= w; v.z *= w; v.w *= w; }
+    // a*this + b*o
+    __device__ __forceinline__ fg_vec lin(float a, float b, const fg_vec &o) const { fg_vec r; r.v.x = a * v.x + b * o.v.x; r.v.y = a * v.y + b * o.v.y; r.v.z = a * v.z + b * o.v.z; r.v.w = a * v.w + b * o.v.w; return r; }
+    __device__ __forceinline__ float dot(const fg_vec &o) const { return (v.x * o.v.x + v.y * o.v.y) + (v.z * o.v.z + v.w * o.v.w); }
+};
+template <> struct fg_vec<1> {
+    float v;
+    __device__ __forceinline__ void zero() { v = 0.f; }
+    __device__ __forceinline__ void load(const float *p) { v = *p; }
+    __device__ __forceinline__ void store(float *p) const { *p = v; }
+    __device__ __forceinline__ void fma(float w, const fg_vec &x) { v = fmaf(w, x.v, v); }
+    __device__ __forceinline__ void add(const fg_vec &x) { v += x.v; }
+    __device__ __forceinline__ void scale(float w) { v *= w; }
+    __device__ __forceinline__ fg_vec lin(float a, float b, const fg_vec &o) const { fg_vec r; r.v = a * v + b * o.v; return r; }
+    __device__ __forceinline__ float dot(const fg_vec &o) const { return v * o.v; }
+};
+
+// Which floats of a feature row a lane owns: slab r covers floats [eoff[r], eoff[r]+VEC) which
+// all belong to head hd[r]; ok[r] is false past the end of the row.
+template <int VEC, int R>
+struct fg_lanemap {
+    int eoff[R];
+    int hd[R];
+    bool ok[R];
+    __device__ __forceinline__ void init(int lane, int HF, int F)
+    {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            eoff[r] = (lane + 64 * r) * VEC;
+            ok[r] = eoff[r] < HF;
+            hd[r] = ok[r] ? eoff[r] / F : 0;
+        }
+    }
+};
+
+// Decode the work item of this wave.  Returns false when there is none.
+__device__ __forceinline__ bool fg_get_item(const fgnn_item *items, int n_items, const int *ptr,
+                                            int &row, int &b, int &e, int &slot)
+{
+    int item = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (item >= n_items) return false;
+    if (items) {
+        fgnn_item it = items[item];
+        row = fg_uni(it.row); b = fg_uni(it.begin); e = fg_uni(it.end); slot = fg_uni(it.slot);
+    } else {
+        row = item; b = fg_uni(ptr[item]); e = fg_uni(ptr[item + 1]); slot = -1;
+    }
+    return true;
+}
+
+// Weighted accumulation of up to 64 gathered feature rows (the hot loop of every SpMM-shaped
+// kernel here).  Lane t of `idv` holds the node id of edge t of the chunk (lanes >= cnt hold any
+// valid id), wl[h*64 + t] its weight for head h (0 for lanes >= cnt).  Without AUX, T accumulates
+// w * row.  With AUX the weight's sign is a flag: T accumulates |w| * row, P accumulates max(w,0) * row.  Node ids are moved to scalar registers
+// so that every row is fetched by one base-plus-lane-offset 128-bit load per slab.
+template <int VEC, int R, bool AUX, bool SUMS, bool FULL>
+__device__ __forceinline__ void fg_accum_chunk(const float *__restrict__ feat, int HF, int idv, int cnt,
+                                               const float *wl, const fg_lanemap<VEC, R> &lm,
+                                               fg_vec<VEC> (&T)[R], fg_vec<VEC> (&P)[R],
+                                               float (&s)[R], float (&cp)[R])
+{
+    constexpr int U = (R >= 8) ? 1 : 8 / R;
+    for (int t = 0; t < cnt; t += U) {
+        fg_vec<VEC> ld[U][R];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int id = __builtin_amdgcn_readlane(idv, t + u);
+            const float *base = feat + (size_t)id * (size_t)HF;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (FULL || lm.ok[r]) ld[u][r].load(base + lm.eoff[r]);
+                else ld[u][r].zero();
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            float w[U];
+            if constexpr (U % 4 == 0) {
+#pragma unroll
+                for (int u = 0; u < U; u += 4) {
+                    float4 q = *reinterpret_cast<const float4 *>(wl + lm.hd[r] * 64 + t + u);
+                    w[u] = q.x; w[u + 1] = q.y; w[u + 2] = q.z; w[u + 3] = q.w;
+                }
+            } else if constexpr (U == 2) {
+                float2 q = *reinterpret_cast<const float2 *>(wl + lm.hd[r] * 64 + t);
+                w[0] = q.x; w[1] = q.y;
+            } else {
+                w[0] = wl[lm.hd[r] * 64 + t];
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float wa = AUX ? fabsf(w[u]) : w[u];
+                T[r].fma(wa, ld[u][r]);
+                if (AUX) {
+                    float wp = fmaxf(w[u], 0.f);
+                    P[r].fma(wp, ld[u][r]);
+                    if (SUMS) cp[r] += wp;
+                }
+                if (SUMS) s[r] += wa;
+            }
+        }
+    }
+}
+
+// Sum over groups of `lph` consecutive lanes (lph a power of two <= 64, groups aligned); every lane
+// of a group gets the group's sum.  Steps inside a row of 16 lanes are DPP, wider ones go through
+// the LDS crossbar.
+__device__ __forceinline__ float fg_group_sum_pow2(float v, int lph)
+{
+    if (lph >= 2) v += fg_dpp<0xB1>(v);
+    if (lph >= 4) v += fg_dpp<0x4E>(v);
+    if (lph >= 8) v += fg_dpp<0x141>(v);
+    if (lph >= 16) v += fg_dpp<0x140>(v);
+    if (lph >= 32) v += fg_bperm(v, fg_lane() ^ 16);
+    if (lph >= 64) v += fg_bperm(v, fg_lane() ^ 32);
+    return v;
+}
+
+// Per-head sums of per-lane partial values: lane h (< H) returns the sum over the F/VEC
+// lane-slabs of head h.  `scr` is wave-private LDS of at least 64*R floats.
+template <int VEC, int R>
+__device__ __forceinline__ float fg_head_reduce(float *scr, const float (&part)[R], const fg_lanemap<VEC, R> &lm,
+                                                int lane, int H, int F)
+{
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+        if (lm.ok[r]) scr[lane + 64 * r] = part[r];
+    fg_wave_lds_sync();
+    float acc = 0.f;
+    if (lane < H) {
+        int n = F / VEC;
+        for (int k = 0; k < n; ++k) acc += scr[lane * n + k];
+    }
+    fg_wave_lds_sync();
+    return acc;
+}
+#endif  // __HIPCC__

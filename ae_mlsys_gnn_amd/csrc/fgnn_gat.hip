@@ -1,0 +1,545 @@
+// Fused GAT forward / backward for gfx950.
+//
+// Forward (one gather pass over CSR rows): per work item (a row, or a segment of a long row) a
+// wave first finds the per-head maximum of lrelu(attn_row[i] + attn_col[j]) over its edges
+// (reads col_ind and attn_col only), then walks the edges again in chunks of 64: lanes-as-edges
+// compute the softmax numerators into wave-private LDS, lanes-as-features accumulate
+// numerator * in_feat[j] with one 128-bit load per lane and edge.  Next to the plain sum T the
+// wave keeps P, the sum over edges with a positive pre-activation; T and P give both
+//   out  = T / s                         and
+//   out2 = (slope*T + (1-slope)*P) / s   = sum_p alpha_p * lrelu'(e_p) * in_feat[j_p],
+// which turns the gradient of attn_row into node-wise dot products in the backward.
+//
+// Backward (one gather pass over CSC columns): a node-wise pre-kernel forms
+//   delta[i,h] = <g[i,h,:], out[i,h,:]>,  grad_attn_row[i,h] = <g[i,h,:], out2[i,h,:]> - delta*c[i,h]
+// and packs (attn_row, max, 1/sum, delta) per (node, head).  The column pass recomputes alpha
+// from that record, accumulates T = sum alpha*g[i] (= grad_feat) and P likewise, and finishes with
+//   grad_attn_col[j,h] = <in_feat[j,h,:], slope*T + (1-slope)*P> - sum_i alpha*lrelu'(e)*delta[i,h].
+// No atomics anywhere: results are bit-reproducible.
+//
+// Math contract: src/fused_gat/fused_gat_SM.cu:193-286 (forward), :560-607, :656-732, :734-801
+// (backward) of the reference; LeakyReLU derivative at 0 is `slope` as in torch.
+#include "fgnn_common.h"
+
+struct GatFwdP {
+    const fgnn_item *items; int n_items;
+    const int *ptr; const int *idx;
+    const float *ar; const float *ac; const float *x;
+    float *out; float *emax; float *esum; float *out2; float *cc;
+    float *part;
+    int N, H, F, HF; float slope;
+};
+
+// Partial layout (floats): T[HF] | P[HF] (AUX only) | m[H] | s[H] | cp[H]
+__host__ __device__ static inline int gat_fwd_pw(int HF, int H, bool aux) { return ((aux ? 2 : 1) * HF + 3 * H + 3) & ~3; }
+
+template <int VEC, int R, bool AUX, bool FULL>
+__global__ __launch_bounds__(FGNN_TPB) void gat_fwd_kernel(GatFwdP p)
+{
+    extern __shared__ float lds[];
+    int row, b, e, slot;
+    if (!fg_get_item(p.items, p.n_items, p.ptr, row, b, e, slot)) return;
+    const int lane = fg_lane();
+    const int H = p.H;
+    float *wl = lds + fg_wave() * (H * 64);
+    fg_lanemap<VEC, R> lm;
+    lm.init(lane, p.HF, p.F);
+    const float slope = p.slope;
+    const float *arp = p.ar + (size_t)row * H;
+
+    // pass A: per-head maximum; lane h keeps the maximum of head h
+    float mst = -INFINITY;
+    for (int c = b; c < e; c += 64) {
+        int q = c + lane;
+        bool ok = q < e;
+        int id = p.idx[ok ? q : c];
+        const float *acp = p.ac + (size_t)id * H;
+        for (int h = 0; h < H; ++h) {
+            float ev = fg_lrelu(arp[h] + acp[h], slope);
+            ev = ok ? ev : -INFINITY;
+            float r = fg_wave_max(ev);
+            mst = (lane == h) ? fmaxf(mst, r) : mst;
+        }
+    }
+
+    fg_vec<VEC> T[R], P[R];
+    float s[R], cp[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) { T[r].zero(); P[r].zero(); s[r] = 0.f; cp[r] = 0.f; }
+
+    // pass B: numerators into LDS, weighted gather
+    for (int c = b; c < e; c += 64) {
+        int q = c + lane;
+        bool ok = q < e;
+        int cnt = min(64, e - c);
+        int id = p.idx[ok ? q : c];
+        const float *acp = p.ac + (size_t)id * H;
+        for (int h = 0; h < H; ++h) {
+            float mh = fg_readlane(mst, h);
+            float ev = fg_lrelu(arp[h] + acp[h], slope);
+            float w = ok ? __expf(ev - mh) : 0.f;
+            wl[h * 64 + lane] = (!AUX || ev > 0.f) ? w : -w;
+        }
+        fg_wave_lds_sync();
+        fg_accum_chunk<VEC, R, AUX, true, FULL>(p.x, p.HF, id, cnt, wl, lm, T, P, s, cp);
+        fg_wave_lds_sync();
+    }
+
+    // every lane fetches the maximum of its heads while the whole wave is still active
+    float mhr[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) mhr[r] = fg_bperm(mst, lm.hd[r]);
+    if (slot < 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (!(FULL || lm.ok[r])) continue;
+            float inv = s[r] > 0.f ? 1.f / s[r] : 0.f;
+            size_t o = (size_t)row * p.HF + lm.eoff[r];
+            if (AUX) {
+                fg_vec<VEC> o2 = T[r].lin(slope * inv, (1.f - slope) * inv, P[r]);
+                o2.store(p.out2 + o);
+            }
+            T[r].scale(inv);
+            T[r].store(p.out + o);
+            float mh = mhr[r];
+            if (lm.eoff[r] % p.F == 0) {
+                size_t so = (size_t)row * H + lm.hd[r];
+                p.emax[so] = (b < e) ? mh : -1e38f;
+                p.esum[so] = s[r];
+                if (AUX) p.cc[so] = (cp[r] + slope * (s[r] - cp[r])) * inv;
+            }
+        }
+    } else {
+        float *pp = p.part + (size_t)slot * gat_fwd_pw(p.HF, H, AUX);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            float mh = mhr[r];
+            if (!(FULL || lm.ok[r])) continue;
+            T[r].store(pp + lm.eoff[r]);
+            if (AUX) P[r].store(pp + p.HF + lm.eoff[r]);
+            if (lm.eoff[r] % p.F == 0) {
+                float *st = pp + (AUX ? 2 : 1) * p.HF;
+                st[lm.hd[r]] = mh;
+                st[H + lm.hd[r]] = s[r];
+                st[2 * H + lm.hd[r]] = cp[r];
+            }
+        }
+    }
+}
+
+// Merge of the segments of split rows: log-sum-exp combination of (m, s, T, P).
+template <int VEC, int R, bool AUX>
+__global__ __launch_bounds__(FGNN_TPB) void gat_fwd_merge_kernel(GatFwdP p, const fgnn_split *split, int n_split)
+{
+    int w = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (w >= n_split) return;
+    fgnn_split sp = split[w];
+    const int row = fg_uni(sp.row), first = fg_uni(sp.first_slot), nseg = fg_uni(sp.nseg);
+    const int lane = fg_lane();
+    const int H = p.H, HF = p.HF;
+    const int pw = gat_fwd_pw(HF, H, AUX);
+    const float slope = p.slope;
+    fg_lanemap<VEC, R> lm;
+    lm.init(lane, HF, p.F);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (!lm.ok[r]) continue;
+        const int h = lm.hd[r];
+        const float *base = p.part + (size_t)first * pw;
+        const int so = (AUX ? 2 : 1) * HF;
+        float M = -INFINITY;
+        for (int g = 0; g < nseg; ++g) M = fmaxf(M, base[(size_t)g * pw + so + h]);
+        fg_vec<VEC> T, P;
+        T.zero(); P.zero();
+        float s = 0.f, cp = 0.f;
+        for (int g = 0; g < nseg; ++g) {
+            const float *pg = base + (size_t)g * pw;
+            float sc = __expf(pg[so + h] - M);
+            fg_vec<VEC> t; t.load(pg + lm.eoff[r]);
+            T.fma(sc, t);
+            if (AUX) { fg_vec<VEC> q; q.load(pg + HF + lm.eoff[r]); P.fma(sc, q); }
+            s += sc * pg[so + H + h];
+            cp += sc * pg[so + 2 * H + h];
+        }
+        float inv = s > 0.f ? 1.f / s : 0.f;
+        size_t o = (size_t)row * HF + lm.eoff[r];
+        if (AUX) { fg_vec<VEC> o2 = T.lin(slope * inv, (1.f - slope) * inv, P); o2.store(p.out2 + o); }
+        T.scale(inv);
+        T.store(p.out + o);
+        if (lm.eoff[r] % p.F == 0) {
+            size_t q = (size_t)row * H + h;
+            p.emax[q] = M; p.esum[q] = s;
+            if (AUX) p.cc[q] = (cp + slope * (s - cp)) * inv;
+        }
+    }
+}
+
+// Per-edge stash of the stash variants: e_lrelu[p,h] and e_softmax[p,h] from the saved row
+// statistics.  One wave per work item (row or segment); lanes run over (edge, head) pairs.
+__global__ __launch_bounds__(FGNN_TPB) void gat_edge_stash_kernel(GatFwdP p, float *e_lrelu, float *e_softmax)
+{
+    int row, b, e, slot;
+    if (!fg_get_item(p.items, p.n_items, p.ptr, row, b, e, slot)) return;
+    const int lane = fg_lane();
+    const int H = p.H;
+    const int64_t lo = (int64_t)b * H, hi = (int64_t)e * H;
+    for (int64_t k = lo + lane; k < hi; k += 64) {
+        int64_t pos = k / H;
+        int h = (int)(k - pos * H);
+        int j = p.idx[pos];
+        float ev = fg_lrelu(p.ar[(size_t)row * H + h] + p.ac[(size_t)j * H + h], p.slope);
+        float m = p.emax[(size_t)row * H + h], s = p.esum[(size_t)row * H + h];
+        e_lrelu[k] = ev;
+        e_softmax[k] = __expf(ev - m) / s;
+    }
+}
+
+// ------------------------------------------------------------------------------- backward
+struct GatBwdP {
+    const fgnn_item *items; int n_items;
+    const int *ptr; const int *idx; const int *permute;
+    const float4 *rec;
+    const float *ac; const float *x; const float *g;
+    const float *esm; const float *erelu;
+    float *gfeat; float *gac; float *part;
+    int N, H, F, HF; float slope;
+};
+// Partial layout (floats): T[HF] | P[HF] | z[H]
+__host__ __device__ static inline int gat_bwd_pw(int HF, int H) { return (2 * HF + H + 3) & ~3; }
+
+// Node-wise pre-pass: delta, grad_attn_row and the packed per-(node, head) record.
+template <int VEC, int R>
+__global__ __launch_bounds__(FGNN_TPB) void gat_bwd_node_kernel(int N, int H, int F, int HF, const float *g, const float *out,
+                                                                const float *out2, const float *cc, const float *ar,
+                                                                const float *emax, const float *esum, float4 *rec, float *gar)
+{
+    extern __shared__ float lds[];
+    int i = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (i >= N) return;
+    const int lane = fg_lane();
+    float *scr = lds + fg_wave() * (64 * R);
+    fg_lanemap<VEC, R> lm;
+    lm.init(lane, HF, F);
+    float d1[R], d2[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        d1[r] = 0.f; d2[r] = 0.f;
+        if (lm.ok[r]) {
+            size_t o = (size_t)i * HF + lm.eoff[r];
+            fg_vec<VEC> gv, a, c;
+            gv.load(g + o); a.load(out + o); c.load(out2 + o);
+            d1[r] = gv.dot(a); d2[r] = gv.dot(c);
+        }
+    }
+    float delta = fg_head_reduce<VEC, R>(scr, d1, lm, lane, H, F);
+    float dd2 = fg_head_reduce<VEC, R>(scr, d2, lm, lane, H, F);
+    if (lane < H) {
+        size_t q = (size_t)i * H + lane;
+        float s = esum[q];
+        rec[q] = make_float4(ar[q], emax[q], s > 0.f ? 1.f / s : 0.f, delta);
+        gar[q] = dd2 - delta * cc[q];
+    }
+}
+
+template <int VEC, int R>
+__device__ __forceinline__ void gat_bwd_finish(const GatBwdP &p, int col, int lane, float *scr, const fg_lanemap<VEC, R> &lm,
+                                               fg_vec<VEC> (&T)[R], fg_vec<VEC> (&P)[R], float zsum /* lane h: head h */)
+{
+    float d[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        d[r] = 0.f;
+        if (lm.ok[r]) {
+            size_t o = (size_t)col * p.HF + lm.eoff[r];
+            T[r].store(p.gfeat + o);
+            fg_vec<VEC> g2 = T[r].lin(p.slope, 1.f - p.slope, P[r]);
+            fg_vec<VEC> xv; xv.load(p.x + o);
+            d[r] = xv.dot(g2);
+        }
+    }
+    float dot = fg_head_reduce<VEC, R>(scr, d, lm, lane, p.H, p.F);
+    if (lane < p.H) p.gac[(size_t)col * p.H + lane] = dot - zsum;
+}
+
+template <int VEC, int R, bool STASH, bool FULL>
+__global__ __launch_bounds__(FGNN_TPB) void gat_bwd_kernel(GatBwdP p)
+{
+    extern __shared__ float lds[];
+    int col, b, e, slot;
+    if (!fg_get_item(p.items, p.n_items, p.ptr, col, b, e, slot)) return;
+    const int lane = fg_lane();
+    const int H = p.H;
+    const int per_wave = max(2 * H * 64, 64 * R);
+    float *wl = lds + fg_wave() * per_wave;
+    float *zl = wl + H * 64;
+    fg_lanemap<VEC, R> lm;
+    lm.init(lane, p.HF, p.F);
+    const float slope = p.slope;
+    const float *acp = p.ac + (size_t)col * H;
+
+    for (int h = 0; h < H; ++h) zl[h * 64 + lane] = 0.f;
+    fg_vec<VEC> T[R], P[R];
+    float s[R], cp[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) { T[r].zero(); P[r].zero(); s[r] = 0.f; cp[r] = 0.f; }
+
+    for (int c = b; c < e; c += 64) {
+        int q = c + lane;
+        bool ok = q < e;
+        int cnt = min(64, e - c);
+        int id = p.idx[ok ? q : c];
+        const float4 *rp = p.rec + (size_t)id * H;
+        size_t pos = STASH ? (size_t)p.permute[ok ? q : c] * H : 0;
+        for (int h = 0; h < H; ++h) {
+            float4 rc = rp[h];
+            float ev, al;
+            if (STASH) {
+                ev = p.erelu[pos + h];
+                al = p.esm[pos + h];
+            } else {
+                ev = fg_lrelu(rc.x + acp[h], slope);
+                al = __expf(ev - rc.y) * rc.z;
+            }
+            al = ok ? al : 0.f;
+            bool pos_e = ev > 0.f;
+            wl[h * 64 + lane] = pos_e ? al : -al;
+            zl[h * 64 + lane] += (pos_e ? al : al * slope) * rc.w;
+        }
+        fg_wave_lds_sync();
+        fg_accum_chunk<VEC, R, true, false, FULL>(p.g, p.HF, id, cnt, wl, lm, T, P, s, cp);
+        fg_wave_lds_sync();
+    }
+
+    // per-head sum of z over the 64 edge slots; lane h keeps head h
+    float zsum = 0.f;
+    for (int h = 0; h < H; ++h) {
+        float z = fg_wave_sum(zl[h * 64 + lane]);
+        zsum = (lane == h) ? z : zsum;
+    }
+    fg_wave_lds_sync();
+    if (slot < 0) {
+        gat_bwd_finish<VEC, R>(p, col, lane, wl, lm, T, P, zsum);
+    } else {
+        float *pp = p.part + (size_t)slot * gat_bwd_pw(p.HF, H);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (!(FULL || lm.ok[r])) continue;
+            T[r].store(pp + lm.eoff[r]);
+            P[r].store(pp + p.HF + lm.eoff[r]);
+        }
+        if (lane < H) pp[2 * p.HF + lane] = zsum;
+    }
+}
+
+template <int VEC, int R>
+__global__ __launch_bounds__(FGNN_TPB) void gat_bwd_merge_kernel(GatBwdP p, const fgnn_split *split, int n_split)
+{
+    extern __shared__ float lds[];
+    int w = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (w >= n_split) return;
+    fgnn_split sp = split[w];
+    const int col = fg_uni(sp.row), first = fg_uni(sp.first_slot), nseg = fg_uni(sp.nseg);
+    const int lane = fg_lane();
+    const int H = p.H, HF = p.HF;
+    const int pw = gat_bwd_pw(HF, H);
+    float *scr = lds + fg_wave() * (64 * R);
+    fg_lanemap<VEC, R> lm;
+    lm.init(lane, HF, p.F);
+    fg_vec<VEC> T[R], P[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) { T[r].zero(); P[r].zero(); }
+    float zsum = 0.f;
+    const float *base = p.part + (size_t)first * pw;
+    for (int g = 0; g < nseg; ++g) {
+        const float *pg = base + (size_t)g * pw;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (!lm.ok[r]) continue;
+            fg_vec<VEC> t, q;
+            t.load(pg + lm.eoff[r]); q.load(pg + HF + lm.eoff[r]);
+            T[r].add(t); P[r].add(q);
+        }
+        if (lane < H) zsum += pg[2 * HF + lane];
+    }
+    gat_bwd_finish<VEC, R>(p, col, lane, scr, lm, T, P, zsum);
+}
+
+// ------------------------------------------------------------------------------- host
+
+static int check_sched(const fgnn_schedule_t *s, const int32_t *ptr, int n, int64_t E, const char *what)
+{
+    if (!s) return 0;
+    FGNN_REQUIRE(s->ptr_dev == ptr && s->n_rows == n && s->n_edges == E, FGNN_ERR_SCHEDULE,
+                 "%s: schedule was built for another pointer array (n_rows %d vs %d, edges %lld vs %lld)", what,
+                 s->n_rows, n, (long long)s->n_edges, (long long)E);
+    return 0;
+}
+
+static int gat_common_checks(const char *fn, int N, int64_t E, int H, int F)
+{
+    FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1 && F >= 1, FGNN_ERR_SHAPE, "%s: bad sizes N=%d E=%lld H=%d F=%d", fn, N, (long long)E, H, F);
+    FGNN_REQUIRE(E <= 2147483647LL, FGNN_ERR_LIMIT, "%s: E=%lld exceeds int32 positions", fn, (long long)E);
+    FGNN_REQUIRE(H <= 64, FGNN_ERR_LIMIT, "%s: H=%d > 64 heads unsupported", fn, H);
+    FGNN_REQUIRE((int64_t)H * F <= 1024, FGNN_ERR_LIMIT, "%s: H*F=%lld > 1024 unsupported", fn, (long long)H * F);
+    return 0;
+}
+
+extern "C" size_t fgnn_gat_forward_workspace_bytes(const fgnn_schedule_t *sched, int H, int F)
+{
+    if (!sched) return 0;
+    return (size_t)sched->n_partials * gat_fwd_pw(H * F, H, true) * sizeof(float);
+}
+
+static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_row, const float *attn_col,
+                              const int32_t *row_ptr, const int32_t *col_ind, float slope, const float *in_feat,
+                              float *out, float *edge_max, float *edge_sum, float *aux_out2, float *aux_c,
+                              float *e_lrelu, float *e_softmax, const fgnn_schedule_t *sched, void *workspace,
+                              size_t workspace_bytes, hipStream_t st)
+{
+    const int HF = H * F;
+    const bool aux = aux_out2 != nullptr;
+    bool aligned = fgnn_aligned16(in_feat) && fgnn_aligned16(out) && (!aux || fgnn_aligned16(aux_out2)) && fgnn_aligned16(workspace);
+    fgnn_rowcfg cfg;
+    FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, aligned, &cfg), FGNN_ERR_LIMIT, "fgnn_gat_forward: unsupported row width %d", HF);
+    GatFwdP p;
+    p.items = sched ? sched->items_dev : nullptr;
+    p.n_items = sched ? sched->n_items : N;
+    p.ptr = row_ptr; p.idx = col_ind; p.ar = attn_row; p.ac = attn_col; p.x = in_feat;
+    p.out = out; p.emax = edge_max; p.esum = edge_sum; p.out2 = aux_out2; p.cc = aux_c;
+    p.part = (float *)workspace; p.N = N; p.H = H; p.F = F; p.HF = HF; p.slope = slope;
+    if (sched && sched->n_partials > 0) {
+        size_t need = (size_t)sched->n_partials * gat_fwd_pw(HF, H, aux) * sizeof(float);
+        FGNN_REQUIRE(workspace && workspace_bytes >= need, FGNN_ERR_WORKSPACE, "fgnn_gat_forward: workspace %zu < %zu bytes", workspace_bytes, need);
+    }
+    if (p.n_items == 0) return 0;
+    const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
+    const size_t shm = (size_t)FGNN_WPB * H * 64 * sizeof(float);
+    int rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
+        if (aux) hipLaunchKernelGGL((gat_fwd_kernel<VEC, R, true, FULL>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+        else hipLaunchKernelGGL((gat_fwd_kernel<VEC, R, false, FULL>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+        int rc2 = fgnn_launch_status("gat_fwd_kernel");
+        if (rc2) return rc2;
+        if (sched && sched->n_split > 0) {
+            unsigned g2 = (unsigned)((sched->n_split + FGNN_WPB - 1) / FGNN_WPB);
+            if (aux) hipLaunchKernelGGL((gat_fwd_merge_kernel<VEC, R, true>), dim3(g2), dim3(FGNN_TPB), 0, st, p, sched->split_dev, sched->n_split);
+            else hipLaunchKernelGGL((gat_fwd_merge_kernel<VEC, R, false>), dim3(g2), dim3(FGNN_TPB), 0, st, p, sched->split_dev, sched->n_split);
+            return fgnn_launch_status("gat_fwd_merge_kernel");
+        }
+        return 0;
+    });
+    if (rc) return rc;
+    if (e_lrelu) {
+        hipLaunchKernelGGL(gat_edge_stash_kernel, dim3(grid), dim3(FGNN_TPB), 0, st, p, e_lrelu, e_softmax);
+        return fgnn_launch_status("gat_edge_stash_kernel");
+    }
+    return 0;
+}
+
+extern "C" int fgnn_gat_forward(int N, int64_t E, int H, int F, const float *attn_row, const float *attn_col,
+                                const int32_t *row_ptr, const int32_t *col_ind, float negative_slope,
+                                const float *in_feat, float *out, float *edge_max, float *edge_sum,
+                                float *aux_out2, float *aux_c, float *e_lrelu, float *e_softmax,
+                                const fgnn_schedule_t *sched, void *workspace, size_t workspace_bytes, void *stream)
+{
+    int rc = gat_common_checks("fgnn_gat_forward", N, E, H, F);
+    if (rc) return rc;
+    FGNN_REQUIRE(attn_row && attn_col && row_ptr && in_feat && out && edge_max && edge_sum && (col_ind || E == 0),
+                 FGNN_ERR_NULL, "fgnn_gat_forward: NULL argument");
+    FGNN_REQUIRE((aux_out2 == nullptr) == (aux_c == nullptr), FGNN_ERR_NULL, "fgnn_gat_forward: aux_out2 and aux_c go together");
+    FGNN_REQUIRE((e_lrelu == nullptr) == (e_softmax == nullptr), FGNN_ERR_NULL, "fgnn_gat_forward: e_lrelu and e_softmax go together");
+    rc = check_sched(sched, row_ptr, N, E, "fgnn_gat_forward");
+    if (rc) return rc;
+    return gat_forward_launch(N, E, H, F, attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, out, edge_max,
+                              edge_sum, aux_out2, aux_c, e_lrelu, e_softmax, sched, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+// Backward workspace: rec [N*H float4] | recompute area (out, out2 [N*HF each], c [N*H]) | partials
+
+extern "C" size_t fgnn_gat_backward_workspace_bytes(int N, int H, int F, const fgnn_schedule_t *sched_csc,
+                                                    const fgnn_schedule_t *sched_csr, int need_recompute)
+{
+    size_t HF = (size_t)H * F;
+    size_t b = fgnn_align256((size_t)N * H * sizeof(float4));
+    if (need_recompute) {
+        b += 2 * fgnn_align256((size_t)N * HF * sizeof(float)) + fgnn_align256((size_t)N * H * sizeof(float));
+        b += fgnn_align256(fgnn_gat_forward_workspace_bytes(sched_csr, H, F));
+    }
+    if (sched_csc) b += fgnn_align256((size_t)sched_csc->n_partials * gat_bwd_pw((int)HF, H) * sizeof(float));
+    return b;
+}
+
+extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_slope, const int32_t *row_ptr,
+                                 const int32_t *col_ind, const int32_t *col_ptr, const int32_t *row_ind,
+                                 const int32_t *permute, const float *e_lrelu, const float *e_softmax,
+                                 const float *edge_max, const float *edge_sum, const float *in_feat,
+                                 const float *attn_row, const float *attn_col, const float *out_feat,
+                                 const float *aux_out2, const float *aux_c, const float *grad_out, float *grad_feat,
+                                 float *grad_attn_row, float *grad_attn_col, const fgnn_schedule_t *sched_csc,
+                                 const fgnn_schedule_t *sched_csr, void *workspace, size_t workspace_bytes, void *stream)
+{
+    int rc = gat_common_checks("fgnn_gat_backward", N, E, H, F);
+    if (rc) return rc;
+    FGNN_REQUIRE(col_ptr && (row_ind || E == 0) && edge_max && edge_sum && in_feat && attn_row && attn_col && grad_out &&
+                     grad_feat && grad_attn_row && grad_attn_col,
+                 FGNN_ERR_NULL, "fgnn_gat_backward: NULL argument");
+    const bool stash = e_softmax != nullptr;
+    FGNN_REQUIRE(!stash || (permute && e_lrelu), FGNN_ERR_NULL, "fgnn_gat_backward: stashed attention needs permute, e_lrelu and e_softmax");
+    const bool recompute = !(out_feat && aux_out2 && aux_c);
+    FGNN_REQUIRE(!recompute || (row_ptr && (col_ind || E == 0)), FGNN_ERR_NULL, "fgnn_gat_backward: recomputing the forward needs row_ptr/col_ind");
+    rc = check_sched(sched_csc, col_ptr, N, E, "fgnn_gat_backward(csc)");
+    if (rc) return rc;
+    if (recompute) { rc = check_sched(sched_csr, row_ptr, N, E, "fgnn_gat_backward(csr)"); if (rc) return rc; }
+    size_t need = fgnn_gat_backward_workspace_bytes(N, H, F, sched_csc, recompute ? sched_csr : nullptr, recompute);
+    FGNN_REQUIRE(workspace && workspace_bytes >= need, FGNN_ERR_WORKSPACE, "fgnn_gat_backward: workspace %zu < %zu bytes", workspace_bytes, need);
+    FGNN_REQUIRE(fgnn_aligned16(workspace), FGNN_ERR_ALIGN, "fgnn_gat_backward: workspace not 16-byte aligned");
+    if (N == 0) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    const int HF = H * F;
+    char *w = (char *)workspace;
+    float4 *rec = (float4 *)w; w += fgnn_align256((size_t)N * H * sizeof(float4));
+    if (recompute) {
+        float *r_out = (float *)w; w += fgnn_align256((size_t)N * HF * sizeof(float));
+        float *r_out2 = (float *)w; w += fgnn_align256((size_t)N * HF * sizeof(float));
+        float *r_c = (float *)w; w += fgnn_align256((size_t)N * H * sizeof(float));
+        void *fws = w; size_t fwb = fgnn_align256(fgnn_gat_forward_workspace_bytes(sched_csr, H, F)); w += fwb;
+        // edge_max / edge_sum are rewritten with identical values by the recomputation
+        rc = gat_forward_launch(N, E, H, F, attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, r_out,
+                                (float *)edge_max, (float *)edge_sum, r_out2, r_c, nullptr, nullptr, sched_csr, fws, fwb, st);
+        if (rc) return rc;
+        out_feat = r_out; aux_out2 = r_out2; aux_c = r_c;
+    }
+    float *part = (float *)w;
+
+    bool aligned = fgnn_aligned16(in_feat) && fgnn_aligned16(grad_out) && fgnn_aligned16(grad_feat) && fgnn_aligned16(out_feat) && fgnn_aligned16(aux_out2);
+    fgnn_rowcfg cfg;
+    FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, aligned, &cfg), FGNN_ERR_LIMIT, "fgnn_gat_backward: unsupported row width %d", HF);
+
+    GatBwdP p;
+    p.items = sched_csc ? sched_csc->items_dev : nullptr;
+    p.n_items = sched_csc ? sched_csc->n_items : N;
+    p.ptr = col_ptr; p.idx = row_ind; p.permute = permute; p.rec = rec; p.ac = attn_col; p.x = in_feat; p.g = grad_out;
+    p.esm = e_softmax; p.erelu = e_lrelu; p.gfeat = grad_feat; p.gac = grad_attn_col; p.part = part;
+    p.N = N; p.H = H; p.F = F; p.HF = HF; p.slope = negative_slope;
+
+    return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
+        const unsigned gn = (unsigned)((N + FGNN_WPB - 1) / FGNN_WPB);
+        hipLaunchKernelGGL((gat_bwd_node_kernel<VEC, R>), dim3(gn), dim3(FGNN_TPB), (size_t)FGNN_WPB * 64 * R * sizeof(float), st,
+                           N, H, F, HF, grad_out, out_feat, aux_out2, aux_c, attn_row, edge_max, edge_sum, rec, grad_attn_row);
+        int rc2 = fgnn_launch_status("gat_bwd_node_kernel");
+        if (rc2) return rc2;
+        const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
+        const size_t per_wave = (size_t)((2 * H * 64 > 64 * R) ? 2 * H * 64 : 64 * R);
+        const size_t shm = FGNN_WPB * per_wave * sizeof(float);
+        if (stash) hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, true, FULL>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+        else hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, false, FULL>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+        rc2 = fgnn_launch_status("gat_bwd_kernel");
+        if (rc2) return rc2;
+        if (sched_csc && sched_csc->n_split > 0) {
+            unsigned g2 = (unsigned)((sched_csc->n_split + FGNN_WPB - 1) / FGNN_WPB);
+            hipLaunchKernelGGL((gat_bwd_merge_kernel<VEC, R>), dim3(g2), dim3(FGNN_TPB), (size_t)FGNN_WPB * 64 * R * sizeof(float), st,
+                               p, sched_csc->split_dev, sched_csc->n_split);
+            return fgnn_launch_status("gat_bwd_merge_kernel");
+        }
+        return 0;
+    });
+}

@@ -1,0 +1,212 @@
+// The small per-edge operators of the reference's operators/ package: multi-head SDDMM,
+// permuted row gather (mhtranspose), edge softmax and u_add_v, each with its backward.
+// One wave per CSR row, lanes over (edge, head) or (edge, column) pairs.
+#include "fgnn_common.h"
+
+// out[p,h] = <a[row,h,:], b[col_ind[p],h,:]> (src/sddmm/mhsddmm.cu:5-81 of the reference, which
+// finds the row of each edge by binary search; here the row is the work item).
+template <int VEC, int R, bool FULL>
+__global__ __launch_bounds__(FGNN_TPB) void mhsddmm_kernel(int N, int H, int F, int HF, const int *ptr, const int *idx,
+                                                           const float *a, const float *b, float *out, int lph_pow2)
+{
+    extern __shared__ float lds[];
+    int row = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (row >= N) return;
+    const int lane = fg_lane();
+    float *scr = lds + fg_wave() * (64 * R);
+    const int pb = fg_uni(ptr[row]), pe = fg_uni(ptr[row + 1]);
+    fg_lanemap<VEC, R> lm;
+    lm.init(lane, HF, F);
+    fg_vec<VEC> ar[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ar[r].load(a + (size_t)row * HF + lm.eoff[r]); else ar[r].zero(); }
+    for (int c = pb; c < pe; c += 64) {
+        int q = c + lane;
+        int cnt = min(64, pe - c);
+        int id = idx[q < pe ? q : c];
+        for (int t = 0; t < cnt; t += 4) {
+            fg_vec<VEC> ld[4][R];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                int j = __builtin_amdgcn_readlane(id, t + u);
+#pragma unroll
+                for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ld[u][r].load(b + (size_t)j * HF + lm.eoff[r]); else ld[u][r].zero(); }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (t + u >= cnt) break;
+                float d[R];
+#pragma unroll
+                for (int r = 0; r < R; ++r) d[r] = ld[u][r].dot(ar[r]);
+                size_t o = (size_t)(c + t + u) * H;
+                if (lph_pow2 > 0) {
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        float s = fg_group_sum_pow2(d[r], lph_pow2);
+                        if ((FULL || lm.ok[r]) && lm.eoff[r] % F == 0) out[o + lm.hd[r]] = s;
+                    }
+                } else {
+                    float s = fg_head_reduce<VEC, R>(scr, d, lm, lane, H, F);
+                    if (lane < H) out[o + lane] = s;
+                }
+            }
+        }
+    }
+}
+
+extern "C" int fgnn_mhsddmm(int N, int64_t E, int H, int F, const int32_t *row_ptr, const int32_t *col_ind, const float *a,
+                            const float *b, float *out, void *stream)
+{
+    FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1 && F >= 1, FGNN_ERR_SHAPE, "fgnn_mhsddmm: bad sizes");
+    FGNN_REQUIRE(H <= 64 && (int64_t)H * F <= 1024, FGNN_ERR_LIMIT, "fgnn_mhsddmm: H=%d H*F=%lld unsupported", H, (long long)H * F);
+    FGNN_REQUIRE(row_ptr && (col_ind || E == 0) && a && b && (out || E == 0), FGNN_ERR_NULL, "fgnn_mhsddmm: NULL argument");
+    if (N == 0 || E == 0) return 0;
+    const int HF = H * F;
+    fgnn_rowcfg cfg;
+    FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, fgnn_aligned16(a) && fgnn_aligned16(b), &cfg), FGNN_ERR_LIMIT, "fgnn_mhsddmm: unsupported row width %d", HF);
+    int lph = F / cfg.vec;
+    int lph_pow2 = (cfg.vec == 4 && (lph & (lph - 1)) == 0 && lph <= 64) ? lph : 0;
+    const unsigned grid = (unsigned)((N + FGNN_WPB - 1) / FGNN_WPB);
+    hipStream_t st = (hipStream_t)stream;
+    return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
+        hipLaunchKernelGGL((mhsddmm_kernel<VEC, R, FULL>), dim3(grid), dim3(FGNN_TPB), (size_t)FGNN_WPB * 64 * R * sizeof(float), st,
+                           N, H, F, HF, row_ptr, col_ind, a, b, out, lph_pow2);
+        return fgnn_launch_status("mhsddmm_kernel");
+    });
+}
+
+// out[q,:] = in[permute[q],:]  (src/csr2csc/mhtranspose.cu:6-26)
+__global__ __launch_bounds__(256) void gather_rows_kernel(int64_t total, int W, const int *permute, const float *in, float *out)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    int64_t q = i / W;
+    int w = (int)(i - q * W);
+    out[i] = in[(size_t)permute[q] * W + w];
+}
+
+extern "C" int fgnn_gather_rows(int64_t E, int W, const int32_t *permute, const float *in, float *out, void *stream)
+{
+    FGNN_REQUIRE(E >= 0 && W >= 1, FGNN_ERR_SHAPE, "fgnn_gather_rows: bad sizes");
+    FGNN_REQUIRE(E == 0 || (permute && in && out), FGNN_ERR_NULL, "fgnn_gather_rows: NULL argument");
+    if (E == 0) return 0;
+    int64_t total = E * W;
+    FGNN_REQUIRE((total + 255) / 256 <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_gather_rows: too many elements");
+    hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, total, W, permute, in, out);
+    return fgnn_launch_status("gather_rows_kernel");
+}
+
+// Per-row, per-head softmax over [E,H] (src/edge_softmax/edge_softmax.cu:7-61) and its backward
+// s*(g - sum_row s*g) (:63-98).  Lanes stride over the row's edges, one head at a time.
+__global__ __launch_bounds__(FGNN_TPB) void edge_softmax_kernel(int N, int H, const int *ptr, const float *in, float *out)
+{
+    int row = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (row >= N) return;
+    const int lane = fg_lane();
+    const int pb = fg_uni(ptr[row]), pe = fg_uni(ptr[row + 1]);
+    for (int h = 0; h < H; ++h) {
+        float m = -INFINITY;
+        for (int q = pb + lane; q < pe; q += 64) m = fmaxf(m, in[(size_t)q * H + h]);
+        m = fg_wave_max(m);
+        float s = 0.f;
+        for (int q = pb + lane; q < pe; q += 64) s += __expf(in[(size_t)q * H + h] - m);
+        s = fg_wave_sum(s);
+        float inv = 1.f / s;
+        for (int q = pb + lane; q < pe; q += 64) out[(size_t)q * H + h] = __expf(in[(size_t)q * H + h] - m) * inv;
+    }
+}
+
+__global__ __launch_bounds__(FGNN_TPB) void edge_softmax_bwd_kernel(int N, int H, const int *ptr, const float *sm, const float *g, float *gin)
+{
+    int row = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (row >= N) return;
+    const int lane = fg_lane();
+    const int pb = fg_uni(ptr[row]), pe = fg_uni(ptr[row + 1]);
+    for (int h = 0; h < H; ++h) {
+        float acc = 0.f;
+        for (int q = pb + lane; q < pe; q += 64) acc += sm[(size_t)q * H + h] * g[(size_t)q * H + h];
+        acc = fg_wave_sum(acc);
+        for (int q = pb + lane; q < pe; q += 64) {
+            size_t o = (size_t)q * H + h;
+            gin[o] = sm[o] * (g[o] - acc);
+        }
+    }
+}
+
+extern "C" int fgnn_edge_softmax(int N, int64_t E, int H, const int32_t *row_ptr, const float *in, float *out, void *stream)
+{
+    FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1, FGNN_ERR_SHAPE, "fgnn_edge_softmax: bad sizes");
+    FGNN_REQUIRE(row_ptr && (E == 0 || (in && out)), FGNN_ERR_NULL, "fgnn_edge_softmax: NULL argument");
+    if (N == 0 || E == 0) return 0;
+    hipLaunchKernelGGL(edge_softmax_kernel, dim3((unsigned)((N + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, (hipStream_t)stream, N, H, row_ptr, in, out);
+    return fgnn_launch_status("edge_softmax_kernel");
+}
+
+extern "C" int fgnn_edge_softmax_backward(int N, int64_t E, int H, const int32_t *row_ptr, const float *sm, const float *grad_out,
+                                          float *grad_in, void *stream)
+{
+    FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1, FGNN_ERR_SHAPE, "fgnn_edge_softmax_backward: bad sizes");
+    FGNN_REQUIRE(row_ptr && (E == 0 || (sm && grad_out && grad_in)), FGNN_ERR_NULL, "fgnn_edge_softmax_backward: NULL argument");
+    if (N == 0 || E == 0) return 0;
+    hipLaunchKernelGGL(edge_softmax_bwd_kernel, dim3((unsigned)((N + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, (hipStream_t)stream, N, H, row_ptr, sm,
+                       grad_out, grad_in);
+    return fgnn_launch_status("edge_softmax_bwd_kernel");
+}
+
+// out[p,w] = row_val[row(p),w] + col_val[col_ind[p],w]  (src/u_add_v/u_add_v.cu:4-26)
+__global__ __launch_bounds__(FGNN_TPB) void u_add_v_kernel(int N, int W, const int *ptr, const int *idx, const float *rv, const float *cv, float *out)
+{
+    int row = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (row >= N) return;
+    const int lane = fg_lane();
+    const int64_t lo = (int64_t)fg_uni(ptr[row]) * W, hi = (int64_t)fg_uni(ptr[row + 1]) * W;
+    for (int64_t k = lo + lane; k < hi; k += 64) {
+        int64_t p = k / W;
+        int w = (int)(k - p * W);
+        out[k] = rv[(size_t)row * W + w] + cv[(size_t)idx[p] * W + w];
+    }
+}
+
+// grad_row[i,w] = sum over the row's edges; grad_col[j,w] += g[p,w] with float atomics into a
+// zero-filled buffer (the reference adds into uninitialised memory, src/u_add_v/u_add_v.cu:67,87).
+__global__ __launch_bounds__(FGNN_TPB) void u_add_v_bwd_kernel(int N, int W, const int *ptr, const int *idx, const float *g, float *grow, float *gcol)
+{
+    int row = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (row >= N) return;
+    const int lane = fg_lane();
+    const int pb = fg_uni(ptr[row]), pe = fg_uni(ptr[row + 1]);
+    for (int w = 0; w < W; ++w) {
+        float acc = 0.f;
+        for (int q = pb + lane; q < pe; q += 64) {
+            float v = g[(size_t)q * W + w];
+            acc += v;
+            atomicAdd(gcol + (size_t)idx[q] * W + w, v);
+        }
+        acc = fg_wave_sum(acc);
+        if (lane == 0) grow[(size_t)row * W + w] = acc;
+    }
+}
+
+extern "C" int fgnn_u_add_v(int N, int64_t E, int W, const int32_t *row_ptr, const int32_t *col_ind, const float *row_val,
+                            const float *col_val, float *out, void *stream)
+{
+    FGNN_REQUIRE(N >= 0 && E >= 0 && W >= 1, FGNN_ERR_SHAPE, "fgnn_u_add_v: bad sizes");
+    FGNN_REQUIRE(row_ptr && row_val && col_val && (E == 0 || (col_ind && out)), FGNN_ERR_NULL, "fgnn_u_add_v: NULL argument");
+    if (N == 0 || E == 0) return 0;
+    hipLaunchKernelGGL(u_add_v_kernel, dim3((unsigned)((N + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, (hipStream_t)stream, N, W, row_ptr, col_ind,
+                       row_val, col_val, out);
+    return fgnn_launch_status("u_add_v_kernel");
+}
+
+extern "C" int fgnn_u_add_v_backward(int N, int64_t E, int W, const int32_t *row_ptr, const int32_t *col_ind, const float *grad_out,
+                                     float *grad_row, float *grad_col, void *stream)
+{
+    FGNN_REQUIRE(N >= 0 && E >= 0 && W >= 1, FGNN_ERR_SHAPE, "fgnn_u_add_v_backward: bad sizes");
+    FGNN_REQUIRE(row_ptr && grad_row && grad_col && (E == 0 || (col_ind && grad_out)), FGNN_ERR_NULL, "fgnn_u_add_v_backward: NULL argument");
+    hipStream_t st = (hipStream_t)stream;
+    int rc = fgnn_fill_f32(grad_col, (size_t)N * W, 0.f, st);
+    if (rc || N == 0) return rc;
+    hipLaunchKernelGGL(u_add_v_bwd_kernel, dim3((unsigned)((N + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, st, N, W, row_ptr, col_ind, grad_out,
+                       grad_row, grad_col);
+    return fgnn_launch_status("u_add_v_bwd_kernel");
+}

@@ -1,0 +1,468 @@
+// Weighted gather-and-sum kernels that share the row engine of the fused GAT kernels:
+//   multi-head SpMM with stored edge weights (mhspmm / spmm of the reference),
+//   GMMConv forward (Gaussian mixture weights computed on the fly, src/fused_gmmconv/gmmconv.cu:48-80),
+//   GMMConv backward in one pass over the CSC arrays, and the standalone Gaussian kernels.
+#include "fgnn_common.h"
+
+struct SpmmP {
+    const fgnn_item *items; int n_items;
+    const int *ptr; const int *idx; const int *pos_map;
+    const float *feat; float *out; float *part;
+    int N, H, F, HF;
+};
+__host__ __device__ static inline int spmm_pw(int HF) { return (HF + 3) & ~3; }
+
+// Weight sources.  fill() runs with lanes-as-edges: lane t writes wl[h*64 + t] for every head.
+struct WAtt {
+    const float *att;   // [E,H] or NULL (all ones)
+    __device__ __forceinline__ void prepare(float *, int, int) const {}
+    __device__ __forceinline__ void fill(float *wl, const float *, int lane, size_t pos, bool ok, int H) const
+    {
+        for (int h = 0; h < H; ++h) wl[h * 64 + lane] = ok ? (att ? att[pos * H + h] : 1.f) : 0.f;
+    }
+};
+struct WGauss {
+    const float *pseudo; const float *mu; const float *isg; float *gauss_out; int dim;
+    // stage mu / inv_sigma [K,dim] into workgroup LDS
+    __device__ __forceinline__ void prepare(float *shared, int tid, int K) const
+    {
+        for (int i = tid; i < K * dim; i += FGNN_TPB) { shared[i] = mu[i]; shared[K * dim + i] = isg[i]; }
+    }
+    __device__ __forceinline__ void fill(float *wl, const float *shared, int lane, size_t pos, bool ok, int K) const
+    {
+        const float *ps = pseudo + pos * dim;
+        for (int k = 0; k < K; ++k) {
+            float acc = 0.f;
+            for (int d = 0; d < dim; ++d) {
+                float t = (ps[d] - shared[k * dim + d]) * shared[K * dim + k * dim + d];
+                acc = fmaf(t, t, acc);
+            }
+            float w = __expf(-0.5f * acc);
+            wl[k * 64 + lane] = ok ? w : 0.f;
+            if (gauss_out && ok) gauss_out[pos * K + k] = w;
+        }
+    }
+};
+
+template <int VEC, int R, bool FULL, class WF>
+__global__ __launch_bounds__(FGNN_TPB) void spmm_kernel(SpmmP p, WF wf, int shared_floats)
+{
+    extern __shared__ float lds[];
+    float *shared = lds + FGNN_WPB * p.H * 64;
+    if (shared_floats > 0) {
+        wf.prepare(shared, (int)threadIdx.x, p.H);
+        __syncthreads();
+    }
+    int row, b, e, slot;
+    if (!fg_get_item(p.items, p.n_items, p.ptr, row, b, e, slot)) return;
+    const int lane = fg_lane();
+    float *wl = lds + fg_wave() * (p.H * 64);
+    fg_lanemap<VEC, R> lm;
+    lm.init(lane, p.HF, p.F);
+    fg_vec<VEC> T[R], P[R];
+    float s[R], cp[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) { T[r].zero(); P[r].zero(); s[r] = 0.f; cp[r] = 0.f; }
+    for (int c = b; c < e; c += 64) {
+        int q = c + lane;
+        bool ok = q < e;
+        int cnt = min(64, e - c);
+        int qq = ok ? q : c;
+        int id = p.idx[qq];
+        size_t pos = p.pos_map ? (size_t)p.pos_map[qq] : (size_t)qq;
+        wf.fill(wl, shared, lane, pos, ok, p.H);
+        fg_wave_lds_sync();
+        fg_accum_chunk<VEC, R, false, false, FULL>(p.feat, p.HF, id, cnt, wl, lm, T, P, s, cp);
+        fg_wave_lds_sync();
+    }
+    float *dst = slot < 0 ? p.out + (size_t)row * p.HF : p.part + (size_t)slot * spmm_pw(p.HF);
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+        if (FULL || lm.ok[r]) T[r].store(dst + lm.eoff[r]);
+}
+
+template <int VEC, int R>
+__global__ __launch_bounds__(FGNN_TPB) void spmm_merge_kernel(SpmmP p, const fgnn_split *split, int n_split)
+{
+    int w = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (w >= n_split) return;
+    fgnn_split sp = split[w];
+    const int row = fg_uni(sp.row), first = fg_uni(sp.first_slot), nseg = fg_uni(sp.nseg);
+    fg_lanemap<VEC, R> lm;
+    lm.init(fg_lane(), p.HF, p.F);
+    const int pw = spmm_pw(p.HF);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (!lm.ok[r]) continue;
+        fg_vec<VEC> T; T.zero();
+        for (int g = 0; g < nseg; ++g) { fg_vec<VEC> t; t.load(p.part + (size_t)(first + g) * pw + lm.eoff[r]); T.add(t); }
+        T.store(p.out + (size_t)row * p.HF + lm.eoff[r]);
+    }
+}
+
+
+static int spmm_checks(const char *fn, int N, int64_t E, int H, int F, const fgnn_schedule_t *sched, const int32_t *ptr)
+{
+    FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1 && F >= 1, FGNN_ERR_SHAPE, "%s: bad sizes N=%d E=%lld H=%d F=%d", fn, N, (long long)E, H, F);
+    FGNN_REQUIRE(E <= 2147483647LL, FGNN_ERR_LIMIT, "%s: E=%lld exceeds int32 positions", fn, (long long)E);
+    FGNN_REQUIRE(H <= 64 && (int64_t)H * F <= 1024, FGNN_ERR_LIMIT, "%s: H=%d, H*F=%lld unsupported (limits 64, 1024)", fn, H, (long long)H * F);
+    if (sched)
+        FGNN_REQUIRE(sched->ptr_dev == ptr && sched->n_rows == N && sched->n_edges == E, FGNN_ERR_SCHEDULE,
+                     "%s: schedule was built for another pointer array", fn);
+    return 0;
+}
+
+template <class WF>
+static int spmm_launch(const char *name, SpmmP p, WF wf, int shared_floats, const fgnn_schedule_t *sched, bool aligned,
+                       void *workspace, size_t workspace_bytes, hipStream_t st)
+{
+    fgnn_rowcfg cfg;
+    FGNN_REQUIRE(fgnn_pick_rowcfg(p.HF, p.F, aligned && fgnn_aligned16(workspace), &cfg), FGNN_ERR_LIMIT, "%s: unsupported row width %d", name, p.HF);
+    p.items = sched ? sched->items_dev : nullptr;
+    p.n_items = sched ? sched->n_items : p.N;
+    p.part = (float *)workspace;
+    if (sched && sched->n_partials > 0) {
+        size_t need = (size_t)sched->n_partials * spmm_pw(p.HF) * sizeof(float);
+        FGNN_REQUIRE(workspace && workspace_bytes >= need, FGNN_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes", name, workspace_bytes, need);
+    }
+    if (p.n_items == 0) return 0;
+    const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
+    const size_t shm = ((size_t)FGNN_WPB * p.H * 64 + shared_floats) * sizeof(float);
+    return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
+        hipLaunchKernelGGL((spmm_kernel<VEC, R, FULL, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
+        int rc = fgnn_launch_status(name);
+        if (rc) return rc;
+        if (sched && sched->n_split > 0) {
+            unsigned g2 = (unsigned)((sched->n_split + FGNN_WPB - 1) / FGNN_WPB);
+            hipLaunchKernelGGL((spmm_merge_kernel<VEC, R>), dim3(g2), dim3(FGNN_TPB), 0, st, p, sched->split_dev, sched->n_split);
+            return fgnn_launch_status("spmm_merge_kernel");
+        }
+        return 0;
+    });
+}
+
+extern "C" size_t fgnn_mhspmm_workspace_bytes(const fgnn_schedule_t *sched, int H, int F)
+{
+    return sched ? (size_t)sched->n_partials * spmm_pw(H * F) * sizeof(float) : 0;
+}
+
+extern "C" int fgnn_mhspmm(int N, int64_t E, int H, int F, const int32_t *ptr, const int32_t *idx, const int32_t *pos_map,
+                           const float *att, const float *feat, float *out, const fgnn_schedule_t *sched, void *workspace,
+                           size_t workspace_bytes, void *stream)
+{
+    int rc = spmm_checks("fgnn_mhspmm", N, E, H, F, sched, ptr);
+    if (rc) return rc;
+    FGNN_REQUIRE(ptr && (idx || E == 0) && feat && out, FGNN_ERR_NULL, "fgnn_mhspmm: NULL argument");
+    SpmmP p{};
+    p.ptr = ptr; p.idx = idx; p.pos_map = pos_map; p.feat = feat; p.out = out; p.N = N; p.H = H; p.F = F; p.HF = H * F;
+    WAtt wf{att};
+    return spmm_launch("fgnn_mhspmm", p, wf, 0, sched, fgnn_aligned16(feat) && fgnn_aligned16(out), workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" size_t fgnn_gmm_forward_workspace_bytes(const fgnn_schedule_t *sched, int K, int F)
+{
+    return fgnn_mhspmm_workspace_bytes(sched, K, F);
+}
+
+extern "C" int fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F, const int32_t *ptr, const int32_t *idx,
+                                const int32_t *pos_map, const float *node_feat, const float *pseudo, const float *mu,
+                                const float *inv_sigma, float *out, float *gauss_out, const fgnn_schedule_t *sched,
+                                void *workspace, size_t workspace_bytes, void *stream)
+{
+    int rc = spmm_checks("fgnn_gmm_forward", N, E, K, F, sched, ptr);
+    if (rc) return rc;
+    FGNN_REQUIRE(dim >= 1 && dim <= 64 && K * dim <= 1024, FGNN_ERR_LIMIT, "fgnn_gmm_forward: dim=%d K*dim=%d unsupported", dim, K * dim);
+    FGNN_REQUIRE(ptr && (idx || E == 0) && node_feat && (pseudo || E == 0) && mu && inv_sigma && out, FGNN_ERR_NULL, "fgnn_gmm_forward: NULL argument");
+    SpmmP p{};
+    p.ptr = ptr; p.idx = idx; p.pos_map = pos_map; p.feat = node_feat; p.out = out; p.N = N; p.H = K; p.F = F; p.HF = K * F;
+    WGauss wf{pseudo, mu, inv_sigma, gauss_out, dim};
+    return spmm_launch("fgnn_gmm_forward", p, wf, 2 * K * dim, sched, fgnn_aligned16(node_feat) && fgnn_aligned16(out), workspace,
+                       workspace_bytes, (hipStream_t)stream);
+}
+
+// ------------------------------------------------------------------------------- GMM backward
+struct GmmBwdP {
+    const fgnn_item *items; int n_items;
+    const int *ptr; const int *idx; const int *permute;
+    const float *x; const float *g; const float *pseudo; const float *mu; const float *isg;
+    float *gfeat; float *gpseudo; float *part; float *red;   // red: [n_items, 2*K*dim] per-item sums
+    int N, K, dim, F, HF;
+};
+
+// One pass over CSC column j (x[j] stays in registers): per in-edge gather grad_out[i], accumulate
+// w * grad_out[i] into grad_feat[j], form the per-kernel dot products gw = <grad_out[i,k,:], x[j,k,:]>
+// and from them the Gaussian derivatives.  grad_pseudo is written once per edge at its CSR
+// position; the mu / inv_sigma derivatives are summed per work item and reduced afterwards.
+template <int VEC, int R, bool FULL>
+__global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p, int lph_pow2)
+{
+    extern __shared__ float lds[];
+    const int K = p.K, dim = p.dim, KD = K * dim;
+    const int per_wave = 2 * K * 64 + 64 * R;
+    float *shared = lds + FGNN_WPB * per_wave;          // mu | inv_sigma
+    for (int i = (int)threadIdx.x; i < KD; i += FGNN_TPB) { shared[i] = p.mu[i]; shared[KD + i] = p.isg[i]; }
+    __syncthreads();
+    int col, b, e, slot;
+    if (!fg_get_item(p.items, p.n_items, p.ptr, col, b, e, slot)) return;
+    const int item = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    const int lane = fg_lane();
+    float *wl = lds + fg_wave() * per_wave;
+    float *gwl = wl + K * 64;
+    float *scr = gwl + K * 64;
+    fg_lanemap<VEC, R> lm;
+    lm.init(lane, p.HF, p.F);
+    fg_vec<VEC> T[R], xr[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        T[r].zero();
+        if (FULL || lm.ok[r]) xr[r].load(p.x + (size_t)col * p.HF + lm.eoff[r]); else xr[r].zero();
+    }
+    float macc = 0.f, sacc = 0.f;    // lane kd keeps the sums for (k,d)
+
+    for (int c = b; c < e; c += 64) {
+        int q = c + lane;
+        bool ok = q < e;
+        int cnt = min(64, e - c);
+        int qq = ok ? q : c;
+        int id = p.idx[qq];
+        size_t pos = (size_t)p.permute[qq];
+        const float *ps = p.pseudo + pos * dim;
+        for (int k = 0; k < K; ++k) {
+            float acc = 0.f;
+            for (int d = 0; d < dim; ++d) {
+                float t = (ps[d] - shared[k * dim + d]) * shared[KD + k * dim + d];
+                acc = fmaf(t, t, acc);
+            }
+            wl[k * 64 + lane] = ok ? __expf(-0.5f * acc) : 0.f;
+        }
+        fg_wave_lds_sync();
+        // lanes-as-features: weighted sum and per-edge dot products
+        for (int t = 0; t < cnt; t += 2) {
+            fg_vec<VEC> ld[2][R];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                int rid = __builtin_amdgcn_readlane(id, t + u);
+                const float *base = p.g + (size_t)rid * p.HF;
+#pragma unroll
+                for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ld[u][r].load(base + lm.eoff[r]); else ld[u][r].zero(); }
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                float dpart[R];
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    float w = wl[lm.hd[r] * 64 + t + u];
+                    T[r].fma(w, ld[u][r]);
+                    dpart[r] = ld[u][r].dot(xr[r]);
+                }
+                if (lph_pow2 > 0) {
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        float sum = fg_group_sum_pow2(dpart[r], lph_pow2);
+                        if ((FULL || lm.ok[r]) && lm.eoff[r] % p.F == 0) gwl[lm.hd[r] * 64 + t + u] = sum;
+                    }
+                } else {
+                    float sum = fg_head_reduce<VEC, R>(scr, dpart, lm, lane, K, p.F);
+                    if (lane < K) gwl[lane * 64 + t + u] = sum;
+                }
+            }
+        }
+        fg_wave_lds_sync();
+        // lanes-as-edges: Gaussian derivatives
+        for (int d = 0; d < dim; ++d) {
+            float gp = 0.f;
+            float psd = ps[d];
+            for (int k = 0; k < K; ++k) {
+                float gww = ok ? gwl[k * 64 + lane] * wl[k * 64 + lane] : 0.f;
+                float diff = psd - shared[k * dim + d];
+                float sg = shared[KD + k * dim + d];
+                float a = gww * diff * sg;          // gw*w*(p-mu)*isg
+                gp -= a * sg;
+                float sm = fg_wave_sum(a * sg);
+                float ss = fg_wave_sum(-a * diff);
+                if (lane == k * dim + d) { macc += sm; sacc += ss; }
+            }
+            if (ok) p.gpseudo[pos * dim + d] = gp;
+        }
+        fg_wave_lds_sync();
+    }
+    float *dst = slot < 0 ? p.gfeat + (size_t)col * p.HF : p.part + (size_t)slot * spmm_pw(p.HF);
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+        if (FULL || lm.ok[r]) T[r].store(dst + lm.eoff[r]);
+    if (lane < KD) {
+        p.red[(size_t)item * 2 * KD + lane] = macc;
+        p.red[(size_t)item * 2 * KD + KD + lane] = sacc;
+    }
+}
+
+// Column sums of red[rows, width] in two deterministic levels.
+__global__ __launch_bounds__(256) void colsum_level1(const float *red, int rows, int width, float *tmp /*[gridDim.x, width]*/)
+{
+    __shared__ float sh[256];
+    int chunk = (rows + gridDim.x - 1) / gridDim.x;
+    int r0 = blockIdx.x * chunk, r1 = min(rows, r0 + chunk);
+    for (int c = 0; c < width; ++c) {
+        float acc = 0.f;
+        for (int r = r0 + (int)threadIdx.x; r < r1; r += 256) acc += red[(size_t)r * width + c];
+        sh[threadIdx.x] = acc;
+        __syncthreads();
+        for (int s = 128; s > 0; s >>= 1) {
+            if ((int)threadIdx.x < s) sh[threadIdx.x] += sh[threadIdx.x + s];
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) tmp[(size_t)blockIdx.x * width + c] = sh[0];
+        __syncthreads();
+    }
+}
+__global__ __launch_bounds__(64) void colsum_level2(const float *tmp, int nblk, int KD, float *gmu, float *gsig)
+{
+    int c = (int)threadIdx.x;
+    if (c >= 2 * KD) return;
+    float acc = 0.f;
+    for (int b = 0; b < nblk; ++b) acc += tmp[(size_t)b * 2 * KD + c];
+    if (c < KD) gmu[c] = acc; else gsig[c - KD] = acc;
+}
+
+static const int kColsumBlocks = 128;
+
+extern "C" size_t fgnn_gmm_backward_workspace_bytes(const fgnn_schedule_t *sched_csc, int K, int dim, int F)
+{
+    // partials | per-item sums | level-1 sums.  Without a schedule the caller passes N items: the
+    // item count is not known here, so the size is computed by fgnn_gmm_backward_workspace_items.
+    size_t items = sched_csc ? (size_t)sched_csc->n_items : 0;
+    size_t b = sched_csc ? fgnn_align256((size_t)sched_csc->n_partials * spmm_pw(K * F) * sizeof(float)) : 0;
+    b += fgnn_align256(items * 2 * K * dim * sizeof(float));
+    b += fgnn_align256((size_t)kColsumBlocks * 2 * K * dim * sizeof(float));
+    return b;
+}
+
+extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const int32_t *col_ptr, const int32_t *row_ind,
+                                 const int32_t *permute, const float *node_feat, const float *pseudo, const float *mu,
+                                 const float *inv_sigma, const float *grad_out, float *grad_feat, float *grad_pseudo,
+                                 float *grad_mu, float *grad_sigma, const fgnn_schedule_t *sched_csc, void *workspace,
+                                 size_t workspace_bytes, void *stream)
+{
+    int rc = spmm_checks("fgnn_gmm_backward", N, E, K, F, sched_csc, col_ptr);
+    if (rc) return rc;
+    FGNN_REQUIRE(dim >= 1 && K * dim <= 32, FGNN_ERR_LIMIT, "fgnn_gmm_backward: K*dim=%d > 32 unsupported", K * dim);
+    FGNN_REQUIRE(col_ptr && (row_ind || E == 0) && (permute || E == 0) && node_feat && (pseudo || E == 0) && mu && inv_sigma &&
+                     grad_out && grad_feat && (grad_pseudo || E == 0) && grad_mu && grad_sigma,
+                 FGNN_ERR_NULL, "fgnn_gmm_backward: NULL argument");
+    FGNN_REQUIRE(sched_csc, FGNN_ERR_SCHEDULE, "fgnn_gmm_backward: a schedule of col_ptr is required");
+    size_t need = fgnn_gmm_backward_workspace_bytes(sched_csc, K, dim, F);
+    FGNN_REQUIRE(workspace && workspace_bytes >= need && fgnn_aligned16(workspace), FGNN_ERR_WORKSPACE,
+                 "fgnn_gmm_backward: workspace %zu < %zu bytes (or unaligned)", workspace_bytes, need);
+    hipStream_t st = (hipStream_t)stream;
+    const int HF = K * F, KD = K * dim;
+    char *w = (char *)workspace;
+    float *part = (float *)w; w += fgnn_align256((size_t)sched_csc->n_partials * spmm_pw(HF) * sizeof(float));
+    float *red = (float *)w; w += fgnn_align256((size_t)sched_csc->n_items * 2 * KD * sizeof(float));
+    float *tmp = (float *)w;
+    if (sched_csc->n_items == 0) {
+        rc = fgnn_fill_f32(grad_mu, KD, 0.f, st);
+        return rc ? rc : fgnn_fill_f32(grad_sigma, KD, 0.f, st);
+    }
+    bool aligned = fgnn_aligned16(node_feat) && fgnn_aligned16(grad_out) && fgnn_aligned16(grad_feat);
+    fgnn_rowcfg cfg;
+    FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, aligned, &cfg), FGNN_ERR_LIMIT, "fgnn_gmm_backward: unsupported row width %d", HF);
+    GmmBwdP p{};
+    p.items = sched_csc->items_dev; p.n_items = sched_csc->n_items; p.ptr = col_ptr; p.idx = row_ind; p.permute = permute;
+    p.x = node_feat; p.g = grad_out; p.pseudo = pseudo; p.mu = mu; p.isg = inv_sigma; p.gfeat = grad_feat; p.gpseudo = grad_pseudo;
+    p.part = part; p.red = red; p.N = N; p.K = K; p.dim = dim; p.F = F; p.HF = HF;
+    int lph = F / cfg.vec;
+    int lph_pow2 = (cfg.vec == 4 && (lph & (lph - 1)) == 0 && lph <= 64) ? lph : 0;
+    const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
+    rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
+        size_t shm = ((size_t)FGNN_WPB * (2 * K * 64 + 64 * R) + 2 * KD) * sizeof(float);
+        hipLaunchKernelGGL((gmm_bwd_kernel<VEC, R, FULL>), dim3(grid), dim3(FGNN_TPB), shm, st, p, lph_pow2);
+        int rc2 = fgnn_launch_status("gmm_bwd_kernel");
+        if (rc2) return rc2;
+        if (sched_csc->n_split > 0) {
+            SpmmP mp{};
+            mp.part = part; mp.out = grad_feat; mp.N = N; mp.H = K; mp.F = F; mp.HF = HF;
+            unsigned g2 = (unsigned)((sched_csc->n_split + FGNN_WPB - 1) / FGNN_WPB);
+            hipLaunchKernelGGL((spmm_merge_kernel<VEC, R>), dim3(g2), dim3(FGNN_TPB), 0, st, mp, sched_csc->split_dev, sched_csc->n_split);
+            return fgnn_launch_status("spmm_merge_kernel");
+        }
+        return 0;
+    });
+    if (rc) return rc;
+    hipLaunchKernelGGL(colsum_level1, dim3(kColsumBlocks), dim3(256), 0, st, red, p.n_items, 2 * KD, tmp);
+    rc = fgnn_launch_status("colsum_level1");
+    if (rc) return rc;
+    hipLaunchKernelGGL(colsum_level2, dim3(1), dim3(64), 0, st, tmp, kColsumBlocks, KD, grad_mu, grad_sigma);
+    return fgnn_launch_status("colsum_level2");
+}
+
+// ------------------------------------------------------------------------------- standalone Gaussian
+__global__ __launch_bounds__(256) void gaussian_kernel(int64_t E, int K, int dim, const float *pseudo, const float *mu,
+                                                       const float *isg, float *out)
+{
+    int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (tid >= E * K) return;
+    int64_t e = tid / K;
+    int k = (int)(tid - e * K);
+    float acc = 0.f;
+    for (int d = 0; d < dim; ++d) {
+        float t = (pseudo[e * dim + d] - mu[k * dim + d]) * isg[k * dim + d];
+        acc = fmaf(t, t, acc);
+    }
+    out[tid] = __expf(-0.5f * acc);
+}
+
+// Closed-form derivatives of w = exp(-0.5 sum_d ((p-mu)*isg)^2) given dL/dw.  One edge per thread;
+// the mu / inv_sigma sums are reduced per wave and added with one float atomic per wave and (k,d).
+__global__ __launch_bounds__(256) void gaussian_bwd_kernel(int64_t E, int K, int dim, const float *pseudo, const float *mu,
+                                                           const float *isg, const float *gw, float *gp, float *gmu, float *gsig)
+{
+    int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    bool ok = e < E;
+    int64_t ee = ok ? e : 0;
+    for (int d = 0; d < dim; ++d) {
+        float acc_p = 0.f;
+        for (int k = 0; k < K; ++k) {
+            float acc = 0.f;
+            for (int dd = 0; dd < dim; ++dd) {
+                float t = (pseudo[ee * dim + dd] - mu[k * dim + dd]) * isg[k * dim + dd];
+                acc = fmaf(t, t, acc);
+            }
+            float w = __expf(-0.5f * acc);
+            float diff = pseudo[ee * dim + d] - mu[k * dim + d];
+            float sg = isg[k * dim + d];
+            float a = ok ? gw[ee * K + k] * w * diff * sg : 0.f;
+            acc_p -= a * sg;
+            float sm = fg_wave_sum(a * sg);
+            float ss = fg_wave_sum(-a * diff);
+            if (fg_lane() == 0) { atomicAdd(gmu + k * dim + d, sm); atomicAdd(gsig + k * dim + d, ss); }
+        }
+        if (ok) gp[e * dim + d] = acc_p;
+    }
+}
+
+extern "C" int fgnn_gaussian(int64_t E, int K, int dim, const float *pseudo, const float *mu, const float *inv_sigma,
+                             float *out, void *stream)
+{
+    FGNN_REQUIRE(E >= 0 && K >= 1 && dim >= 1, FGNN_ERR_SHAPE, "fgnn_gaussian: bad sizes");
+    FGNN_REQUIRE((pseudo || E == 0) && mu && inv_sigma && (out || E == 0), FGNN_ERR_NULL, "fgnn_gaussian: NULL argument");
+    if (E == 0) return 0;
+    int64_t total = E * K;
+    hipLaunchKernelGGL(gaussian_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, E, K, dim, pseudo, mu, inv_sigma, out);
+    return fgnn_launch_status("gaussian_kernel");
+}
+
+extern "C" int fgnn_gaussian_backward(int64_t E, int K, int dim, const float *pseudo, const float *mu, const float *inv_sigma,
+                                      const float *grad_w, float *grad_pseudo, float *grad_mu, float *grad_sigma, void *stream)
+{
+    FGNN_REQUIRE(E >= 0 && K >= 1 && dim >= 1, FGNN_ERR_SHAPE, "fgnn_gaussian_backward: bad sizes");
+    FGNN_REQUIRE((pseudo || E == 0) && mu && inv_sigma && (grad_w || E == 0) && (grad_pseudo || E == 0) && grad_mu && grad_sigma,
+                 FGNN_ERR_NULL, "fgnn_gaussian_backward: NULL argument");
+    hipStream_t st = (hipStream_t)stream;
+    int rc = fgnn_fill_f32(grad_mu, (size_t)K * dim, 0.f, st);
+    if (rc) return rc;
+    rc = fgnn_fill_f32(grad_sigma, (size_t)K * dim, 0.f, st);
+    if (rc || E == 0) return rc;
+    hipLaunchKernelGGL(gaussian_bwd_kernel, dim3((unsigned)((E + 255) / 256)), dim3(256), 0, st, E, K, dim, pseudo, mu, inv_sigma,
+                       grad_w, grad_pseudo, grad_mu, grad_sigma);
+    return fgnn_launch_status("gaussian_bwd_kernel");
+}

@@ -1,0 +1,147 @@
+"""Fused GAT operators: the reference's operators/fused_gat.py surface on libfgnn_hip.so.
+
+``fused_gat_op`` / ``FusedGATFunction_SM``        recompute variant (operators/fused_gat.py:30-31,52-71)
+``fused_gat_stash_op`` / ``FusedGATFunction_stash``  stash variant  (operators/fused_gat.py:33-34,73-86)
+``fused_gat_fusescatter`` / ``FusedGATFunction``  fuse-scatter variant (operators/fused_gat.py:27-28,36-50)
+
+All three share one forward kernel and one backward kernel; the stash variants additionally
+write / read the per-edge ``[E,H]`` LeakyReLU and softmax tensors.  What the recompute variant
+keeps for the backward is node-sized only: ``out``, ``out2`` ([N,H,F]) and three ``[N,H]`` arrays.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+from .._lib import as_f32, as_i32, check, lib, ptr, require_cuda, schedule_for, stream_ptr, workspace
+
+
+class gat_native:
+    """Native entry points with the argument order of the reference's pybind modules
+    (fused_gat_SM.gat_forward / gat_backward, src/fused_gat/fused_gat_SM.cpp:14-124)."""
+
+    @staticmethod
+    def gat_forward(attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, *, need_aux=True, stash=False,
+                    use_schedule=True):
+        require_cuda(attn_row, attn_col, row_ptr, col_ind, in_feat)
+        attn_row, attn_col, in_feat = as_f32(attn_row), as_f32(attn_col), as_f32(in_feat)
+        row_ptr, col_ind = as_i32(row_ptr), as_i32(col_ind)
+        if in_feat.dim() != 3:
+            raise _lib.FgnnError("in_feat must be [N,H,F], got %s" % (tuple(in_feat.shape),))
+        n, h, f = in_feat.shape
+        e = col_ind.numel()
+        if attn_row.shape != (n, h) or attn_col.shape != (n, h) or row_ptr.numel() != n + 1:
+            raise _lib.FgnnError("shape mismatch: attn_row %s attn_col %s row_ptr %s for N=%d H=%d" % (
+                tuple(attn_row.shape), tuple(attn_col.shape), tuple(row_ptr.shape), n, h))
+        dev = in_feat.device
+        out = torch.empty_like(in_feat)
+        edge_max = torch.empty((n, h), dtype=torch.float32, device=dev)
+        edge_sum = torch.empty((n, h), dtype=torch.float32, device=dev)
+        out2 = torch.empty_like(in_feat) if need_aux else None
+        cc = torch.empty((n, h), dtype=torch.float32, device=dev) if need_aux else None
+        e_lrelu = torch.empty((e, h), dtype=torch.float32, device=dev) if stash else None
+        e_soft = torch.empty((e, h), dtype=torch.float32, device=dev) if stash else None
+        sched = schedule_for(row_ptr) if use_schedule else None
+        sh = sched.handle if sched is not None else None
+        with torch.cuda.device(dev):
+            ws, wsb = workspace(lib().fgnn_gat_forward_workspace_bytes(sh, h, f), dev)
+            check(lib().fgnn_gat_forward(n, e, h, f, ptr(attn_row), ptr(attn_col), ptr(row_ptr), ptr(col_ind),
+                                         float(negative_slope), ptr(in_feat), ptr(out), ptr(edge_max), ptr(edge_sum),
+                                         ptr(out2), ptr(cc), ptr(e_lrelu), ptr(e_soft), sh, ptr(ws), wsb, stream_ptr()),
+                  "fgnn_gat_forward")
+        return out, edge_max, edge_sum, out2, cc, e_lrelu, e_soft
+
+    @staticmethod
+    def gat_backward(negative_slope, row_ptr, col_ind, col_ptr, row_ind, edge_max, edge_sum, in_feat, attn_row, attn_col,
+                     grad, *, out_feat=None, out2=None, cc=None, permute=None, e_lrelu=None, e_soft=None,
+                     use_schedule=True):
+        require_cuda(grad, in_feat, col_ptr, row_ind)
+        grad = as_f32(grad)
+        n, h, f = in_feat.shape
+        e = row_ind.numel()
+        dev = in_feat.device
+        col_ptr, row_ind = as_i32(col_ptr), as_i32(row_ind)
+        grad_feat = torch.empty_like(in_feat)
+        grad_attn_row = torch.empty((n, h), dtype=torch.float32, device=dev)
+        grad_attn_col = torch.empty((n, h), dtype=torch.float32, device=dev)
+        recompute = out_feat is None or out2 is None or cc is None
+        sched_csc = schedule_for(col_ptr) if use_schedule else None
+        sched_csr = schedule_for(row_ptr) if (use_schedule and recompute) else None
+        hc = sched_csc.handle if sched_csc is not None else None
+        hr = sched_csr.handle if sched_csr is not None else None
+        with torch.cuda.device(dev):
+            ws, wsb = workspace(lib().fgnn_gat_backward_workspace_bytes(n, h, f, hc, hr, int(recompute)), dev)
+            check(lib().fgnn_gat_backward(n, e, h, f, float(negative_slope), ptr(row_ptr), ptr(col_ind), ptr(col_ptr),
+                                          ptr(row_ind), ptr(permute), ptr(e_lrelu), ptr(e_soft), ptr(edge_max),
+                                          ptr(edge_sum), ptr(in_feat), ptr(attn_row), ptr(attn_col),
+                                          None if recompute else ptr(out_feat), None if recompute else ptr(out2),
+                                          None if recompute else ptr(cc), ptr(grad), ptr(grad_feat), ptr(grad_attn_row),
+                                          ptr(grad_attn_col), hc, hr, ptr(ws), wsb, stream_ptr()),
+                  "fgnn_gat_backward")
+        return grad_feat, grad_attn_row, grad_attn_col
+
+
+def fused_gat_fusescatter(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute):
+    return FusedGATFunction.apply(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute)
+
+
+def fused_gat_op(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, save_memory=True):
+    return FusedGATFunction_SM.apply(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat)
+
+
+def fused_gat_stash_op(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute):
+    return FusedGATFunction_stash.apply(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute)
+
+
+def _needs_grad(ctx):
+    return any(ctx.needs_input_grad)
+
+
+class FusedGATFunction_SM(torch.autograd.Function):
+    """Recompute ("save memory") variant: nothing edge-sized is kept between forward and backward."""
+
+    @staticmethod
+    def forward(ctx, attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat):
+        need = _needs_grad(ctx)
+        out, edge_max, edge_sum, out2, cc, _, _ = gat_native.gat_forward(
+            attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, need_aux=need)
+        if need:
+            ctx.save_for_backward(row_ptr, col_ind, col_ptr, row_ind, edge_max, edge_sum, in_feat, attn_row, attn_col,
+                                  out, out2, cc)
+        ctx.negative_slope = negative_slope
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        row_ptr, col_ind, col_ptr, row_ind, edge_max, edge_sum, in_feat, attn_row, attn_col, out, out2, cc = ctx.saved_tensors
+        grad_feat, grad_attn_row, grad_attn_col = gat_native.gat_backward(
+            ctx.negative_slope, row_ptr, col_ind, col_ptr, row_ind, edge_max, edge_sum, in_feat, attn_row, attn_col,
+            grad_out.contiguous(), out_feat=out, out2=out2, cc=cc)
+        return grad_attn_row, grad_attn_col, None, None, None, None, None, grad_feat
+
+
+class FusedGATFunction_stash(torch.autograd.Function):
+    """Stash variant: the forward also writes edge LeakyReLU / softmax [E,H]; the backward reads them."""
+
+    @staticmethod
+    def forward(ctx, attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute):
+        out, edge_max, edge_sum, out2, cc, e_lrelu, e_soft = gat_native.gat_forward(
+            attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, need_aux=True, stash=True)
+        ctx.save_for_backward(row_ptr, col_ind, col_ptr, row_ind, permute, e_soft, e_lrelu, in_feat, attn_row, attn_col,
+                              edge_max, edge_sum, out, out2, cc)
+        ctx.negative_slope = negative_slope
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (row_ptr, col_ind, col_ptr, row_ind, permute, e_soft, e_lrelu, in_feat, attn_row, attn_col,
+         edge_max, edge_sum, out, out2, cc) = ctx.saved_tensors
+        grad_feat, grad_attn_row, grad_attn_col = gat_native.gat_backward(
+            ctx.negative_slope, row_ptr, col_ind, col_ptr, row_ind, edge_max, edge_sum, in_feat, attn_row, attn_col,
+            grad_out.contiguous(), out_feat=out, out2=out2, cc=cc, permute=as_i32(permute), e_lrelu=e_lrelu, e_soft=e_soft)
+        return grad_attn_row, grad_attn_col, None, None, None, None, None, grad_feat, None
+
+
+class FusedGATFunction(FusedGATFunction_stash):
+    """Fuse-scatter variant of the reference (edge softmax stashed, separate SpMM).  Here the
+    stashed tensors come out of the same fused forward, so it shares the stash implementation."""

@@ -1,0 +1,186 @@
+/*
+ * fgnn.h -- C ABI of libfgnn_hip.so: fused GNN sparse operators for AMD gfx950 (MI355X).
+ *
+ * Every entry point takes plain device pointers and sizes, launches on the HIP stream handed
+ * in (`stream` is a hipStream_t passed as void*; NULL = the null stream) and returns
+ *      0            success
+ *      < 0          argument error (FGNN_ERR_*), nothing was launched
+ *      > 0          a hipError_t from a launch or runtime call
+ * fgnn_last_error() gives a thread-local message for the last non-zero return.  Nothing in the
+ * library aborts, exits or prints.  The caller owns every buffer (inputs, outputs, workspace);
+ * the library owns only the schedule objects it hands out.  All index arrays are int32, all
+ * value arrays are contiguous float32.  Graphs are CSR indexed by DESTINATION node (row = dst,
+ * col_ind = src); per-edge arrays are in CSR position order; the CSC arrays (col_ptr, row_ind)
+ * are the transpose with `permute[q]` = CSR position of CSC entry q.
+ *
+ * Each declaration cites the interface of the reference (mlsysAE2022/ae_mlsys_gnn) that it
+ * stands in for.
+ */
+#ifndef FGNN_H
+#define FGNN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FGNN_ERR_NULL      (-1)  /* a required pointer is NULL */
+#define FGNN_ERR_SHAPE     (-2)  /* a size is negative or inconsistent */
+#define FGNN_ERR_ALIGN     (-3)  /* a float buffer is not 16-byte aligned */
+#define FGNN_ERR_LIMIT     (-4)  /* a size exceeds what the kernels support */
+#define FGNN_ERR_WORKSPACE (-5)  /* workspace missing or too small */
+#define FGNN_ERR_SCHEDULE  (-6)  /* schedule does not match the arrays it is used with */
+
+int         fgnn_version(void);
+const char *fgnn_last_error(void);
+
+/* ---------------------------------------------------------------- row schedules
+ * A schedule is the degree-binned work list of one pointer array (row_ptr for forward passes,
+ * col_ptr for backward passes): rows longer than `seg_len` edges are cut into segments that are
+ * reduced separately and merged, and the work items are ordered longest first.  The reference
+ * has no counterpart (it launches one block per row: src/fused_gat/fused_gat_SM.cu:518-532);
+ * passing sched == NULL to an operator selects the same one-wave-per-row mapping.
+ * fgnn_schedule_create reads `ptr` back to the host once (it synchronises `stream`). */
+typedef struct fgnn_schedule fgnn_schedule_t;
+int     fgnn_schedule_create(const int32_t *ptr_dev, int n_rows, int seg_len, void *stream,
+                             fgnn_schedule_t **out);
+void    fgnn_schedule_destroy(fgnn_schedule_t *s);
+int     fgnn_schedule_num_items(const fgnn_schedule_t *s);
+int     fgnn_schedule_num_partials(const fgnn_schedule_t *s);   /* segments of split rows */
+int64_t fgnn_schedule_num_edges(const fgnn_schedule_t *s);
+
+/* ---------------------------------------------------------------- fused GAT
+ * Replaces fused_gat_SM.gat_forward (src/fused_gat/fused_gat_SM.cpp:14-38, host launcher
+ * fused_gat_SM.cu:536-558) and, with e_lrelu/e_softmax non-NULL, fused_gat_stash.gat_forward
+ * and fused_gat.gat_forward (src/fused_gat/fused_gat_stash.cu:420-442, fused_gat.cu:365-386).
+ *   out[i,h,:] = sum_p softmax_p(lrelu(attn_row[i,h] + attn_col[col_ind[p],h])) * in_feat[col_ind[p],h,:]
+ * Outputs: out [N,H,F], edge_max, edge_sum [N,H].  Optional (NULL to skip):
+ *   aux_out2 [N,H,F], aux_c [N,H]  -- sum_p alpha*lrelu'(e) * in_feat and sum_p alpha*lrelu'(e);
+ *                                     they let the backward run in a single gather pass
+ *   e_lrelu, e_softmax [E,H]       -- the stashed per-edge tensors of the stash variants
+ * Workspace: fgnn_gat_forward_workspace_bytes(sched, H, F) bytes (0 when sched is NULL). */
+size_t fgnn_gat_forward_workspace_bytes(const fgnn_schedule_t *sched, int H, int F);
+int    fgnn_gat_forward(int N, int64_t E, int H, int F,
+                        const float *attn_row, const float *attn_col,
+                        const int32_t *row_ptr, const int32_t *col_ind, float negative_slope,
+                        const float *in_feat, float *out, float *edge_max, float *edge_sum,
+                        float *aux_out2, float *aux_c, float *e_lrelu, float *e_softmax,
+                        const fgnn_schedule_t *sched, void *workspace, size_t workspace_bytes,
+                        void *stream);
+
+/* Replaces fused_gat_SM.gat_backward (src/fused_gat/fused_gat_SM.cpp:40-124, host launcher
+ * fused_gat_SM.cu:865-893); with permute/e_lrelu/e_softmax non-NULL it reads the stashed
+ * attention instead of recomputing it (fused_gat_stash.gat_backward, fused_gat_stash.cu:776-804;
+ * fused_gat.gat_backward, fused_gat.cu:641-670).
+ * Inputs as the reference's plus out_feat/aux_out2/aux_c from the forward; when those three are
+ * NULL they are recomputed into the workspace from (row_ptr, col_ind) first.
+ * Outputs: grad_feat [N,H,F], grad_attn_row, grad_attn_col [N,H]; all fully overwritten and
+ * bit-reproducible from run to run (no atomics).
+ * sched_csr is only used for the recompute case. */
+size_t fgnn_gat_backward_workspace_bytes(int N, int H, int F, const fgnn_schedule_t *sched_csc,
+                                         const fgnn_schedule_t *sched_csr, int need_recompute);
+int    fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_slope,
+                         const int32_t *row_ptr, const int32_t *col_ind,
+                         const int32_t *col_ptr, const int32_t *row_ind,
+                         const int32_t *permute, const float *e_lrelu, const float *e_softmax,
+                         const float *edge_max, const float *edge_sum,
+                         const float *in_feat, const float *attn_row, const float *attn_col,
+                         const float *out_feat, const float *aux_out2, const float *aux_c,
+                         const float *grad_out,
+                         float *grad_feat, float *grad_attn_row, float *grad_attn_col,
+                         const fgnn_schedule_t *sched_csc, const fgnn_schedule_t *sched_csr,
+                         void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---------------------------------------------------------------- fused EdgeConv
+ * Replaces fused_edgeconv.edgeconv_forward / edgeconv_backward
+ * (src/fused_edgeconv/fused_edgeconv.cpp:12-51; fused_edgeconv.cu:148-200).
+ *   out[i,f] = max_{p in [i*k,(i+1)*k)} (h_dst[i,f] + h_src[src_ind[p],f]);  argmax[i,f] = the
+ *   source node id at the FIRST maximal position (int32; the reference stores a float).
+ * backward: grad_src[n_src,F] = scatter-add of grad_out at argmax (zero-filled first). */
+int fgnn_edgeconv_forward(int N, int n_src, int F, int k, const int32_t *src_ind,
+                          const float *h_src, const float *h_dst, float *out, int32_t *argmax,
+                          void *stream);
+int fgnn_edgeconv_backward(int N, int n_src, int F, const int32_t *argmax, const float *grad_out,
+                           float *grad_src, void *stream);
+
+/* ---------------------------------------------------------------- fused GMMConv (MoNet)
+ * Replaces gmmconv.gmmconv / gmmconveb / gmmconvstash (src/fused_gmmconv/gmmconv.cc:43-78;
+ * gmmconv.cu:201-263):  w[p,k] = exp(-0.5 sum_d ((pseudo[p,d]-mu[k,d])*inv_sigma[k,d])^2),
+ *   out[i,k,:] = sum_p w[p,k] * node_feat[col_ind[p],k,:].
+ * pseudo [E,dim] is in the position order of (ptr, idx); when pos_map is non-NULL the row
+ * pseudo[pos_map[p]] is used instead (lets a CSC pass read CSR-ordered pseudo without the
+ * mhtranspose copy of operators/fused_gmmconv.py:55).  gauss_out [E,K] optional. */
+size_t fgnn_gmm_forward_workspace_bytes(const fgnn_schedule_t *sched, int K, int F);
+int    fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F,
+                        const int32_t *ptr, const int32_t *idx, const int32_t *pos_map,
+                        const float *node_feat, const float *pseudo, const float *mu,
+                        const float *inv_sigma, float *out, float *gauss_out,
+                        const fgnn_schedule_t *sched, void *workspace, size_t workspace_bytes,
+                        void *stream);
+
+/* Replaces the backward sequence of operators/fused_gmmconv.py:51-58 (mhsddmm + mhtranspose +
+ * gmmconv over CSC + GaussianBp, gmmconv.cu:265-285) with one pass over the CSC arrays:
+ * grad_feat [N,K,F], grad_pseudo [E,dim] (CSR order), grad_mu, grad_sigma [K,dim].
+ * grad_mu / grad_sigma are accumulated with float atomics (K*dim values per workgroup). */
+size_t fgnn_gmm_backward_workspace_bytes(const fgnn_schedule_t *sched_csc, int K, int dim, int F);
+int    fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F,
+                         const int32_t *col_ptr, const int32_t *row_ind, const int32_t *permute,
+                         const float *node_feat, const float *pseudo, const float *mu,
+                         const float *inv_sigma, const float *grad_out,
+                         float *grad_feat, float *grad_pseudo, float *grad_mu, float *grad_sigma,
+                         const fgnn_schedule_t *sched_csc, void *workspace, size_t workspace_bytes,
+                         void *stream);
+
+/* gmmconv.Gaussian / gmmconv.GaussianBp (gmmconv.cc:36-41,80-86; gmmconv.cu:187-199,265-285).
+ * The backward implements the closed-form derivatives of the Gaussian weight. */
+int fgnn_gaussian(int64_t E, int K, int dim, const float *pseudo, const float *mu,
+                  const float *inv_sigma, float *out, void *stream);
+int fgnn_gaussian_backward(int64_t E, int K, int dim, const float *pseudo, const float *mu,
+                           const float *inv_sigma, const float *grad_w,
+                           float *grad_pseudo, float *grad_mu, float *grad_sigma, void *stream);
+
+/* ---------------------------------------------------------------- small operators
+ * mhspmm.mhspmm (src/spmm/mhspmm.cc; mhspmm.cu:44-66): out[i,h,:] = sum_p att[p,h]*feat[idx[p],h,:];
+ * att row used is att[pos_map[p]] when pos_map is non-NULL.  With H == 1 and att == NULL it is
+ * the unweighted single-head SpMM of operators/spmm.py:38-41. */
+size_t fgnn_mhspmm_workspace_bytes(const fgnn_schedule_t *sched, int H, int F);
+int    fgnn_mhspmm(int N, int64_t E, int H, int F, const int32_t *ptr, const int32_t *idx,
+                   const int32_t *pos_map, const float *att, const float *feat, float *out,
+                   const fgnn_schedule_t *sched, void *workspace, size_t workspace_bytes,
+                   void *stream);
+/* mhsddmm.mhsddmm (src/sddmm/mhsddmm.cc; mhsddmm.cu:83-99) and, with H == 1, sddmm.csr_sddmm
+ * (src/sddmm/sddmm.cpp): out[p,h] = <a[row(p),h,:], b[col_ind[p],h,:]>. */
+int    fgnn_mhsddmm(int N, int64_t E, int H, int F, const int32_t *row_ptr, const int32_t *col_ind,
+                    const float *a, const float *b, float *out, void *stream);
+/* mhtranspose.mhtranspose (src/csr2csc/mhtranspose.cc; mhtranspose.cu:28-47): out[q,:] = in[permute[q],:]. */
+int    fgnn_gather_rows(int64_t E, int W, const int32_t *permute, const float *in, float *out,
+                        void *stream);
+/* edge_softmax.edge_softmax / edge_softmax_backward (src/edge_softmax/edge_softmax.cc;
+ * edge_softmax.cu:100-128). */
+int    fgnn_edge_softmax(int N, int64_t E, int H, const int32_t *row_ptr, const float *in, float *out,
+                         void *stream);
+int    fgnn_edge_softmax_backward(int N, int64_t E, int H, const int32_t *row_ptr, const float *sm,
+                                  const float *grad_out, float *grad_in, void *stream);
+/* u_add_v.u_add_v_forward / u_add_v_backward (src/u_add_v/u_add_v.cpp; u_add_v.cu:28-90).
+ * The backward needs the CSC arrays to reduce per source node without atomics. */
+int    fgnn_u_add_v(int N, int64_t E, int W, const int32_t *row_ptr, const int32_t *col_ind,
+                    const float *row_val, const float *col_val, float *out, void *stream);
+int    fgnn_u_add_v_backward(int N, int64_t E, int W, const int32_t *row_ptr, const int32_t *col_ind,
+                             const float *grad_out, float *grad_row, float *grad_col, void *stream);
+
+/* ---------------------------------------------------------------- csr2csc
+ * Replaces csrtocsc.csr2csc (src/csr2csc/csr2csc.cc; csr2csc.cu:7-43, a cuSPARSE
+ * cusparseCsr2cscEx2 call).  Stable: entries of a column keep ascending CSR position.
+ * Outputs col_ptr [n_cols+1], row_ind [E], permute [E] (int32 positions; the reference carries
+ * them as float values). */
+size_t fgnn_csr2csc_workspace_bytes(int n_rows, int n_cols, int64_t E);
+int    fgnn_csr2csc(int n_rows, int n_cols, int64_t E, const int32_t *row_ptr, const int32_t *col_ind,
+                    int32_t *col_ptr, int32_t *row_ind, int32_t *permute,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FGNN_H */

@@ -1,0 +1,87 @@
+"""GPU parity of the fused GAT operators against the float64 oracle (through the C ABI)."""
+import pytest
+import torch
+
+from oracle import fgnn_oracle as orc
+from tests.util import assert_close, degree_edge_graph, gat_inputs, custom_graph
+from ae_mlsys_gnn_amd import graphs
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle_fwd_bwd(g, x, ar, ac, go, slope):
+    x = x.clone().requires_grad_(True)
+    ar = ar.clone().requires_grad_(True)
+    ac = ac.clone().requires_grad_(True)
+    out = orc.gat_forward(ar, ac, g.row_ptr, g.col_ind, slope, x)
+    out.backward(go)
+    return out.detach(), x.grad, ar.grad, ac.grad
+
+
+def _run(g, h, f, slope=0.2, seed=0, attn_scale=1.0, variant="sm", seg_len=None, monkeypatch=None):
+    from ae_mlsys_gnn_amd.operators import fused_gat as fg
+    g = graphs.add_csc_torch(g)
+    x, ar, ac, go = gat_inputs(g, h, f, seed, attn_scale)
+    ref = _oracle_fwd_bwd(g, x, ar, ac, go, slope)
+    dev = torch.device("cuda:0")
+    gd = g.to(dev)
+    xd = x.float().to(dev).requires_grad_(True)
+    ard = ar.float().to(dev).requires_grad_(True)
+    acd = ac.float().to(dev).requires_grad_(True)
+    if variant == "sm":
+        out = fg.fused_gat_op(ard, acd, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, slope, xd)
+    elif variant == "stash":
+        out = fg.fused_gat_stash_op(ard, acd, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, slope, xd, gd.permute)
+    else:
+        out = fg.fused_gat_fusescatter(ard, acd, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, slope, xd, gd.permute)
+    out.backward(go.float().to(dev))
+    torch.cuda.synchronize()
+    assert_close(out, ref[0], "out")
+    assert_close(xd.grad, ref[1], "grad_feat")
+    # grad_attn_* are sums of E/N terms of either sign: the absolute part of the bar scales with
+    # the magnitude of the summands
+    scale = float(go.abs().max() * x.abs().max() * f)
+    assert_close(ard.grad, ref[2], "grad_attn_row", atol=1e-5 * max(1.0, scale))
+    assert_close(acd.grad, ref[3], "grad_attn_col", atol=1e-5 * max(1.0, scale))
+
+
+@pytest.mark.parametrize("h,f", [(8, 32), (4, 16), (1, 64), (1, 47), (3, 20), (4, 128), (8, 128), (2, 65), (1, 1)])
+def test_gat_shapes(h, f):
+    g = graphs.rmat_graph(600, 12000, seed=3)
+    _run(g, h, f)
+
+
+@pytest.mark.parametrize("variant", ["sm", "stash", "fusescatter"])
+def test_gat_variants_degree_edges(variant):
+    _run(degree_edge_graph(), 8, 32, variant=variant)
+
+
+def test_gat_split_rows(monkeypatch):
+    monkeypatch.setenv("FGNN_SEG_LEN", "256")
+    from ae_mlsys_gnn_amd import _lib
+    _lib.clear_schedule_cache()
+    _run(degree_edge_graph(seed=5), 8, 32)
+    _run(degree_edge_graph(seed=6), 1, 47)
+    _lib.clear_schedule_cache()
+
+
+def test_gat_large_attention():
+    # wide score range: the softmax must stay stable
+    _run(graphs.rmat_graph(500, 8000, seed=9), 4, 32, attn_scale=30.0)
+
+
+def test_gat_self_loops_only_is_identity():
+    # the 4-node graph of the reference's script/inference/gatconv_test.py:75-76
+    from ae_mlsys_gnn_amd.operators import fused_gat as fg
+    g = custom_graph([[0], [1], [2], [3]])
+    g = graphs.add_csc_torch(g).to("cuda:0")
+    x = torch.randn(4, 2, 8, device="cuda:0")
+    ar = torch.randn(4, 2, device="cuda:0")
+    ac = torch.randn(4, 2, device="cuda:0")
+    out = fg.fused_gat_op(ar, ac, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, 0.2, x)
+    assert torch.equal(out, x)
+
+
+def test_gat_c1_config():
+    # BASELINE config 1: N=4096, 32k uniform edges + self loops, 4 heads x 16
+    _run(graphs.uniform_graph(4096, 32768, seed=0), 4, 16)

@@ -1,0 +1,56 @@
+"""Shared helpers of the test suite: seeded inputs and the parity bar."""
+import numpy as np
+import torch
+
+from ae_mlsys_gnn_amd import graphs
+
+# fp32 parity bar of the fused operators against the float64 oracle
+RTOL = 1e-4
+ATOL = 1e-5
+
+
+def assert_close(got, ref, what, rtol=RTOL, atol=ATOL):
+    got = got.detach().cpu().double()
+    ref = ref.detach().cpu().double()
+    assert got.shape == ref.shape, "%s: shape %s vs %s" % (what, tuple(got.shape), tuple(ref.shape))
+    err = (got - ref).abs()
+    tol = atol + rtol * ref.abs()
+    bad = err > tol
+    if bad.any():
+        i = int(torch.argmax(err - tol))
+        raise AssertionError("%s: %d/%d outside rtol=%g atol=%g; worst |err|=%.3e at flat %d (got %.7g ref %.7g)" % (
+            what, int(bad.sum()), bad.numel(), rtol, atol, float(err.flatten()[i]), i,
+            float(got.flatten()[i]), float(ref.flatten()[i])))
+
+
+def gat_inputs(g, h, f, seed=0, attn_scale=1.0, dtype=torch.float64):
+    gen = torch.Generator().manual_seed(seed)
+    x = torch.randn(g.n, h, f, generator=gen, dtype=dtype)
+    ar = torch.randn(g.n, h, generator=gen, dtype=dtype) * attn_scale
+    ac = torch.randn(g.n, h, generator=gen, dtype=dtype) * attn_scale
+    go = torch.randn(g.n, h, f, generator=gen, dtype=dtype)
+    return x, ar, ac, go
+
+
+def custom_graph(row_lists, n=None):
+    """Graph from per-destination source lists."""
+    n = len(row_lists) if n is None else n
+    rp = [0]
+    ci = []
+    for r in row_lists:
+        ci.extend(r)
+        rp.append(len(ci))
+    while len(rp) < n + 1:
+        rp.append(len(ci))
+    return graphs.Graph(n, torch.tensor(rp, dtype=torch.int32), torch.tensor(ci, dtype=torch.int32))
+
+
+def degree_edge_graph(n=700, seed=0):
+    """Rows with degrees 0, 1, 31..33, 63..65, 511..513 and one hub; sources uniform random."""
+    gen = np.random.default_rng(seed)
+    degs = [0, 1, 2, 7, 8, 9, 31, 32, 33, 63, 64, 65, 127, 128, 129, 511, 512, 513, 0, 3000]
+    rows = []
+    for i in range(n):
+        d = degs[i] if i < len(degs) else int(gen.integers(0, 12))
+        rows.append(list(gen.integers(0, n, size=d)))
+    return custom_graph(rows, n)

@@ -1,0 +1,29 @@
+"""EdgeConv layer on the fused operator (interface of the reference's layers/edgeconv_layer.py:6-43)."""
+from __future__ import annotations
+
+from torch import nn
+
+from ..operators.fused_edgeconv import fused_edgeconv_op
+
+
+class EdgeConv(nn.Module):
+    """out_i = max_j (theta(x_j) + phi(x_i) - theta(x_i)) over the k neighbours j of i, i.e. the
+    operator-reorganised form of max_j (theta(x_j - x_i) + phi(x_i)) with bias-free theta, phi."""
+
+    def __init__(self, in_feat, out_feat, batch_norm=False, allow_zero_in_degree=False):
+        super().__init__()
+        self.batch_norm = batch_norm
+        self._allow_zero_in_degree = allow_zero_in_degree
+        self.theta = nn.Linear(in_feat, out_feat, bias=False)
+        self.phi = nn.Linear(in_feat, out_feat, bias=False)
+        if batch_norm:
+            self.bn = nn.BatchNorm1d(out_feat)
+
+    def set_allow_zero_in_degree(self, set_value):
+        self._allow_zero_in_degree = set_value
+
+    def forward(self, k, src_ind, feat):
+        h_theta = self.theta(feat)
+        h_src = h_theta
+        h_dst = self.phi(feat) - h_theta
+        return fused_edgeconv_op(k, src_ind, h_src, h_dst)

@@ -1,0 +1,60 @@
+"""Fused EdgeConv operator: the reference's operators/fused_edgeconv.py surface on libfgnn_hip.so."""
+from __future__ import annotations
+
+import torch
+
+from .._lib import FgnnError, as_f32, as_i32, check, lib, ptr, require_cuda, stream_ptr
+
+
+class edgeconv_native:
+    """fused_edgeconv.edgeconv_forward / edgeconv_backward (src/fused_edgeconv/fused_edgeconv.cpp:12-51)."""
+
+    @staticmethod
+    def edgeconv_forward(k, src_ind, h_src, h_dst):
+        require_cuda(src_ind, h_src, h_dst)
+        src_ind, h_src, h_dst = as_i32(src_ind), as_f32(h_src), as_f32(h_dst)
+        n, f = h_dst.shape
+        if h_src.shape[1] != f or src_ind.numel() != n * int(k):
+            raise FgnnError("edgeconv: src_ind has %d entries, expected N*k = %d*%d; feature widths %d vs %d" % (
+                src_ind.numel(), n, int(k), h_src.shape[1], f))
+        out = torch.empty_like(h_dst)
+        max_idx = torch.empty((n, f), dtype=torch.int32, device=h_dst.device)
+        with torch.cuda.device(h_dst.device):
+            check(lib().fgnn_edgeconv_forward(n, h_src.shape[0], f, int(k), ptr(src_ind), ptr(h_src), ptr(h_dst), ptr(out),
+                                              ptr(max_idx), stream_ptr()), "fgnn_edgeconv_forward")
+        return out, max_idx
+
+    @staticmethod
+    def edgeconv_backward(grad_out, max_idx, n_src=None):
+        require_cuda(grad_out, max_idx)
+        grad_out, max_idx = as_f32(grad_out), as_i32(max_idx)
+        n, f = grad_out.shape
+        n_src = n if n_src is None else n_src
+        grad_src = torch.empty((n_src, f), dtype=torch.float32, device=grad_out.device)
+        with torch.cuda.device(grad_out.device):
+            check(lib().fgnn_edgeconv_backward(n, n_src, f, ptr(max_idx), ptr(grad_out), ptr(grad_src), stream_ptr()),
+                  "fgnn_edgeconv_backward")
+        return grad_src
+
+
+def fused_edgeconv_op(k, src_ind, h_src, h_dst):
+    return FusedEdgeConvFunction.apply(k, src_ind, h_src, h_dst)
+
+
+class FusedEdgeConvFunction(torch.autograd.Function):
+    """out[i,f] = h_dst[i,f] + max_j h_src[j,f] over the k neighbours of i; the argmax (int32 source
+    node id, first maximum wins) is kept for the backward (operators/fused_edgeconv.py:18-29)."""
+
+    @staticmethod
+    def forward(ctx, k, src_ind, h_src, h_dst):
+        out_feat, max_idx = edgeconv_native.edgeconv_forward(k, src_ind, h_src, h_dst)
+        ctx.save_for_backward(max_idx)
+        ctx.n_src = h_src.shape[0]
+        return out_feat
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        max_idx = ctx.saved_tensors[0]
+        grad_out = grad_out.contiguous()
+        grad_src = edgeconv_native.edgeconv_backward(grad_out, max_idx, ctx.n_src)
+        return None, None, grad_src, grad_out

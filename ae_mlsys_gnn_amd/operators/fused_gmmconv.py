@@ -1,0 +1,150 @@
+"""Fused GMMConv (MoNet) operators: the reference's operators/fused_gmmconv.py surface on
+libfgnn_hip.so.  The backward is one pass over the CSC arrays (the reference runs mhsddmm,
+mhtranspose, a CSC gmmconv and GaussianBp: operators/fused_gmmconv.py:51-58) and implements the
+closed-form Gaussian derivatives."""
+from __future__ import annotations
+
+import torch
+
+from .._lib import FgnnError, as_f32, as_i32, check, lib, ptr, require_cuda, schedule_for, stream_ptr, workspace
+
+
+class gmm_native:
+    """gmmconv.gmmconv / gmmconvstash / Gaussian / GaussianBp (src/fused_gmmconv/gmmconv.cc:36-94)."""
+
+    @staticmethod
+    def gmmconv(rowptr, colind, node_feat, pseudo, mu, sigma, *, pos_map=None, want_gauss=False):
+        require_cuda(rowptr, colind, node_feat, pseudo, mu, sigma)
+        rowptr, colind = as_i32(rowptr), as_i32(colind)
+        node_feat, pseudo, mu, sigma = as_f32(node_feat), as_f32(pseudo), as_f32(mu), as_f32(sigma)
+        if node_feat.dim() != 3:
+            raise FgnnError("node_feat must be [N,K,F], got %s" % (tuple(node_feat.shape),))
+        n, k, f = node_feat.shape
+        e = colind.numel()
+        dim = mu.shape[1]
+        if mu.shape != (k, dim) or sigma.shape != (k, dim) or pseudo.shape != (e, dim) or rowptr.numel() != n + 1:
+            raise FgnnError("gmmconv: shape mismatch mu %s sigma %s pseudo %s for K=%d E=%d" % (
+                tuple(mu.shape), tuple(sigma.shape), tuple(pseudo.shape), k, e))
+        out = torch.empty_like(node_feat)
+        gauss = torch.empty((e, k), dtype=torch.float32, device=node_feat.device) if want_gauss else None
+        sched = schedule_for(rowptr)
+        with torch.cuda.device(node_feat.device):
+            ws, wsb = workspace(lib().fgnn_gmm_forward_workspace_bytes(sched.handle, k, f), node_feat.device)
+            check(lib().fgnn_gmm_forward(n, e, k, dim, f, ptr(rowptr), ptr(colind), ptr(pos_map), ptr(node_feat), ptr(pseudo),
+                                         ptr(mu), ptr(sigma), ptr(out), ptr(gauss), sched.handle, ptr(ws), wsb, stream_ptr()),
+                  "fgnn_gmm_forward")
+        return (out, gauss) if want_gauss else out
+
+    @staticmethod
+    def gmmconv_backward(colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out):
+        require_cuda(colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out)
+        colptr, rowind, permute = as_i32(colptr), as_i32(rowind), as_i32(permute)
+        grad_out = as_f32(grad_out)
+        n, k, f = node_feat.shape
+        e = rowind.numel()
+        dim = mu.shape[1]
+        dev = node_feat.device
+        grad_feat = torch.empty_like(node_feat)
+        grad_pseudo = torch.empty((e, dim), dtype=torch.float32, device=dev)
+        grad_mu = torch.empty_like(mu)
+        grad_sigma = torch.empty_like(sigma)
+        sched = schedule_for(colptr)
+        with torch.cuda.device(dev):
+            ws, wsb = workspace(lib().fgnn_gmm_backward_workspace_bytes(sched.handle, k, dim, f), dev)
+            check(lib().fgnn_gmm_backward(n, e, k, dim, f, ptr(colptr), ptr(rowind), ptr(permute), ptr(node_feat), ptr(pseudo),
+                                          ptr(mu), ptr(sigma), ptr(grad_out), ptr(grad_feat), ptr(grad_pseudo), ptr(grad_mu),
+                                          ptr(grad_sigma), sched.handle, ptr(ws), wsb, stream_ptr()), "fgnn_gmm_backward")
+        return grad_feat, grad_pseudo, grad_mu, grad_sigma
+
+    @staticmethod
+    def Gaussian(pseudo, mu, sigma):
+        require_cuda(pseudo, mu, sigma)
+        pseudo, mu, sigma = as_f32(pseudo), as_f32(mu), as_f32(sigma)
+        e, dim = pseudo.shape
+        k = mu.shape[0]
+        out = torch.empty((e, k), dtype=torch.float32, device=pseudo.device)
+        with torch.cuda.device(pseudo.device):
+            check(lib().fgnn_gaussian(e, k, dim, ptr(pseudo), ptr(mu), ptr(sigma), ptr(out), stream_ptr()), "fgnn_gaussian")
+        return out
+
+    @staticmethod
+    def GaussianBp(pseudo, mu, sigma, grad_out):
+        require_cuda(pseudo, mu, sigma, grad_out)
+        pseudo, mu, sigma, grad_out = as_f32(pseudo), as_f32(mu), as_f32(sigma), as_f32(grad_out)
+        e, dim = pseudo.shape
+        k = mu.shape[0]
+        gp = torch.empty_like(pseudo)
+        gm = torch.empty_like(mu)
+        gs = torch.empty_like(sigma)
+        with torch.cuda.device(pseudo.device):
+            check(lib().fgnn_gaussian_backward(e, k, dim, ptr(pseudo), ptr(mu), ptr(sigma), ptr(grad_out), ptr(gp), ptr(gm),
+                                               ptr(gs), stream_ptr()), "fgnn_gaussian_backward")
+        return gp, gm, gs
+
+
+def GmmConvFuse(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma):
+    return GmmFuseFunction.apply(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma)
+
+
+class GmmFuseFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma):
+        out = gmm_native.gmmconv(rowptr, colind, node_feat, pseudo, mu, sigma)      # [N, K, F]
+        ctx.save_for_backward(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma = ctx.saved_tensors
+        grad_feat, grad_pseudo, grad_mu, grad_sigma = gmm_native.gmmconv_backward(
+            colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out.contiguous())
+        return None, None, None, None, None, grad_feat, grad_pseudo, grad_mu, grad_sigma
+
+
+def GmmConvFuseEb(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma):
+    return GmmFuseEbFunction.apply(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma)
+
+
+class GmmFuseEbFunction(GmmFuseFunction):
+    """The reference's edge-balanced variant (operators/fused_gmmconv.py:61-79).  Load balance is
+    handled by the degree-binned schedule here, so it is the same computation."""
+
+
+def GaussianCp(pseudo, mu, sigma):
+    return GaussianFunction.apply(pseudo, mu, sigma)
+
+
+class GaussianFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, pseudo, mu, sigma):
+        out = gmm_native.Gaussian(pseudo, mu, sigma)
+        ctx.save_for_backward(pseudo, mu, sigma)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        pseudo, mu, sigma = ctx.saved_tensors
+        return gmm_native.GaussianBp(pseudo, mu, sigma, grad_out.contiguous())
+
+
+def GmmConvStash(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma):
+    return GmmStashFunction.apply(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma)
+
+
+class GmmStashFunction(torch.autograd.Function):
+    """Stash variant (operators/fused_gmmconv.py:100-118): the forward also writes the Gaussian
+    weights [E,K].  The backward uses the same single CSC pass as GmmFuseFunction (recomputing
+    the weights is cheaper than reading them back through `permute`)."""
+
+    @staticmethod
+    def forward(ctx, rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma):
+        out, gauss = gmm_native.gmmconv(rowptr, colind, node_feat, pseudo, mu, sigma, want_gauss=True)
+        ctx.save_for_backward(rowptr, colind, colptr, rowind, permute, gauss, node_feat, pseudo, mu, sigma)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        rowptr, colind, colptr, rowind, permute, gauss, node_feat, pseudo, mu, sigma = ctx.saved_tensors
+        grad_feat, grad_pseudo, grad_mu, grad_sigma = gmm_native.gmmconv_backward(
+            colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out.contiguous())
+        return None, None, None, None, None, grad_feat, grad_pseudo, grad_mu, grad_sigma

@@ -1,0 +1,310 @@
+"""GPU parity of EdgeConv, GMMConv, csr2csc and the small operators against the oracle,
+called through the C ABI (ctypes binding of libfgnn_hip.so)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fgnn_oracle as orc
+from oracle import c_oracle
+from tests.util import assert_close, custom_graph, degree_edge_graph
+from ae_mlsys_gnn_amd import graphs
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+# ------------------------------------------------------------------ csr2csc (bit-exact)
+@pytest.mark.parametrize("n,e,seed", [(1, 1, 0), (7, 20, 1), (300, 5000, 2), (5000, 200000, 3), (70000, 300000, 4)])
+def test_csr2csc_bit_exact(n, e, seed):
+    from ae_mlsys_gnn_amd.operators import csr2csc as op
+    g = graphs.rmat_graph(n, e, seed=seed)
+    cp, ri, pm = orc.csr2csc(g.row_ptr.numpy(), g.col_ind.numpy())
+    gd = g.to(DEV)
+    col_ptr, row_ind, permute = op.csr2csc(gd.row_ptr, gd.col_ind)
+    assert np.array_equal(col_ptr.cpu().numpy(), cp)
+    assert np.array_equal(permute.cpu().numpy(), pm)
+    assert np.array_equal(row_ind.cpu().numpy(), ri)
+
+
+def test_csr2csc_duplicates_unsorted_and_empty():
+    from ae_mlsys_gnn_amd.operators import csr2csc as op
+    # duplicate (i,j) entries, columns not sorted inside a row, empty rows and empty columns
+    g = custom_graph([[3, 1, 3, 3], [], [0, 0], [4, 1], [], [1]], n=6)
+    cp, ri, pm = orc.csr2csc_bruteforce(g.row_ptr.numpy(), g.col_ind.numpy())
+    gd = g.to(DEV)
+    col_ptr, row_ind, permute = op.csr2csc(gd.row_ptr, gd.col_ind)
+    assert np.array_equal(col_ptr.cpu().numpy(), cp)
+    assert np.array_equal(permute.cpu().numpy(), pm)
+    assert np.array_equal(row_ind.cpu().numpy(), ri)
+    # no edges at all
+    g0 = custom_graph([[], [], []]).to(DEV)
+    col_ptr, row_ind, permute = op.csr2csc(g0.row_ptr, g0.col_ind)
+    assert col_ptr.tolist() == [0, 0, 0, 0] and row_ind.numel() == 0
+    # sparsetrans carries values along
+    vals = torch.arange(g.n_edges, dtype=torch.float32, device=DEV) * 0.5
+    out = op.sparsetrans(gd.row_ptr, gd.col_ind, vals)
+    assert torch.equal(out.cpu(), torch.from_numpy(pm).float() * 0.5)
+
+
+def test_csr2csc_round_trip_large():
+    # transpose of the transpose is the original (columns sorted inside rows): size-independent property
+    from ae_mlsys_gnn_amd.operators import csr2csc as op
+    g = graphs.rmat_graph(100000, 3000000, seed=11, device=DEV)
+    col_ptr, row_ind, permute = op.csr2csc(g.row_ptr, g.col_ind)
+    rp2, ci2, pm2 = op.csr2csc(col_ptr, row_ind)
+    assert torch.equal(rp2, g.row_ptr) and torch.equal(ci2, g.col_ind)
+    assert torch.equal(permute.long()[pm2.long()], torch.arange(g.n_edges, device=DEV))
+    assert torch.equal(torch.sort(permute).values.long(), torch.arange(g.n_edges, device=DEV))
+
+
+# ------------------------------------------------------------------ EdgeConv (argmax bit-exact)
+def _edgeconv_case(bsz, npts, k, fin, fout, seed, quantize=False):
+    gen = torch.Generator().manual_seed(seed)
+    pts = torch.rand(bsz, npts, 3, generator=gen) * 2 - 1
+    src = graphs.knn_graph(pts, k)
+    n = bsz * npts
+    h_src = torch.randn(n, fout, generator=gen)
+    h_dst = torch.randn(n, fout, generator=gen)
+    if quantize:   # many exact ties
+        h_src = torch.round(h_src * 2) / 2
+        h_dst = torch.round(h_dst * 2) / 2
+    return src, h_src, h_dst
+
+
+@pytest.mark.parametrize("bsz,npts,k,f,quant", [(2, 64, 5, 64, False), (3, 100, 20, 64, False), (2, 64, 7, 3, False),
+                                                (2, 128, 20, 64, True), (1, 50, 33, 130, True), (1, 40, 1, 8, False)])
+def test_edgeconv_forward_bit_exact(bsz, npts, k, f, quant):
+    from ae_mlsys_gnn_amd.operators.fused_edgeconv import edgeconv_native
+    src, h_src, h_dst = _edgeconv_case(bsz, npts, k, 3, f, seed=k + f, quantize=quant)
+    ref_out, ref_arg = orc.edgeconv_forward(k, src, h_src, h_dst)
+    c_out, c_arg = c_oracle.edgeconv_forward(k, src.numpy(), h_src.numpy(), h_dst.numpy())
+    assert np.array_equal(ref_arg.numpy(), c_arg) and np.array_equal(ref_out.numpy(), c_out)
+    out, arg = edgeconv_native.edgeconv_forward(k, src.to(DEV), h_src.to(DEV), h_dst.to(DEV))
+    assert arg.dtype == torch.int32
+    assert torch.equal(arg.cpu(), ref_arg), "argmax indices differ"
+    assert torch.equal(out.cpu(), ref_out), "max values are not bit-identical"
+
+
+def test_edgeconv_backward_and_layer():
+    from ae_mlsys_gnn_amd.layers import EdgeConv
+    torch.manual_seed(0)
+    bsz, npts, k = 2, 96, 20
+    pts = torch.rand(bsz, npts, 3) * 2 - 1
+    src = graphs.knn_graph(pts, k)
+    x = pts.reshape(-1, 3)
+    layer = EdgeConv(3, 64)
+    # oracle: EdgeConv_reorg math in float64 with autograd (maxima are unique for random inputs)
+    th = layer.theta.weight.detach().double().requires_grad_(True)
+    ph = layer.phi.weight.detach().double().requires_grad_(True)
+    xd = x.double()
+    h_src = xd @ th.t()
+    h_dst = xd @ ph.t() - h_src
+    ref = orc.edgeconv_forward_autograd(k, src, h_src, h_dst)
+    go = torch.randn(ref.shape, dtype=torch.float64)
+    ref.backward(go)
+    layer = layer.to(DEV)
+    out = layer(k, src.to(DEV), x.to(DEV))
+    out.backward(go.float().to(DEV))
+    assert_close(out, ref.detach(), "edgeconv out")
+    assert_close(layer.theta.weight.grad, th.grad, "theta grad", atol=1e-4)
+    assert_close(layer.phi.weight.grad, ph.grad, "phi grad", atol=1e-4)
+
+
+def test_edgeconv_backward_scatter_exact_counts():
+    # grad_out = 1 makes the scatter-add an exact histogram of argmax: integer-valued, order independent
+    from ae_mlsys_gnn_amd.operators.fused_edgeconv import edgeconv_native
+    src, h_src, h_dst = _edgeconv_case(4, 256, 20, 3, 64, seed=5)
+    out, arg = edgeconv_native.edgeconv_forward(20, src.to(DEV), h_src.to(DEV), h_dst.to(DEV))
+    gs = edgeconv_native.edgeconv_backward(torch.ones_like(out), arg, h_src.shape[0])
+    ref = c_oracle.edgeconv_backward(arg.cpu().numpy(), np.ones(out.shape), h_src.shape[0])
+    assert np.array_equal(gs.cpu().numpy().astype(np.float64), ref)
+
+
+# ------------------------------------------------------------------ GMMConv
+def _gmm_case(g, k, dim, f, seed):
+    gen = torch.Generator().manual_seed(seed)
+    x = torch.randn(g.n, k, f, generator=gen, dtype=torch.float64)
+    pseudo = torch.rand(g.n_edges, dim, generator=gen, dtype=torch.float64)
+    mu = torch.rand(k, dim, generator=gen, dtype=torch.float64)
+    isg = 0.5 + torch.rand(k, dim, generator=gen, dtype=torch.float64)
+    go = torch.randn(g.n, k, f, generator=gen, dtype=torch.float64)
+    return x, pseudo, mu, isg, go
+
+
+@pytest.mark.parametrize("k,dim,f,variant", [(3, 2, 64, "fuse"), (2, 1, 16, "fuse"), (3, 2, 64, "stash"), (1, 3, 47, "fuse"),
+                                              (4, 2, 33, "eb"), (3, 2, 128, "fuse")])
+def test_gmm_forward_backward(k, dim, f, variant, monkeypatch):
+    from ae_mlsys_gnn_amd.operators import fused_gmmconv as fg
+    from ae_mlsys_gnn_amd import _lib
+    monkeypatch.setenv("FGNN_SEG_LEN", "256")
+    _lib.clear_schedule_cache()
+    g = graphs.add_csc_torch(degree_edge_graph(n=400, seed=k + f))
+    x, pseudo, mu, isg, go = _gmm_case(g, k, dim, f, seed=1)
+    leaves = [t.clone().requires_grad_(True) for t in (x, pseudo, mu, isg)]
+    ref = orc.gmm_forward(g.row_ptr, g.col_ind, *leaves)
+    ref.backward(go)
+    gd = g.to(DEV)
+    dl = [t.float().to(DEV).requires_grad_(True) for t in (x, pseudo, mu, isg)]
+    op = {"fuse": fg.GmmConvFuse, "stash": fg.GmmConvStash, "eb": fg.GmmConvFuseEb}[variant]
+    out = op(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, *dl)
+    out.backward(go.float().to(DEV))
+    _lib.clear_schedule_cache()
+    assert_close(out, ref.detach(), "gmm out")
+    assert_close(dl[0].grad, leaves[0].grad, "grad node_feat")
+    assert_close(dl[1].grad, leaves[1].grad, "grad pseudo", atol=1e-4)
+    # sums over all E edges: absolute bar scales with the number of summands
+    assert_close(dl[2].grad, leaves[2].grad, "grad mu", rtol=1e-3, atol=1e-2)
+    assert_close(dl[3].grad, leaves[3].grad, "grad inv_sigma", rtol=1e-3, atol=1e-2)
+
+
+def test_gaussian_op():
+    from ae_mlsys_gnn_amd.operators import fused_gmmconv as fg
+    gen = torch.Generator().manual_seed(3)
+    pseudo = torch.rand(1000, 2, generator=gen, dtype=torch.float64)
+    mu = torch.rand(3, 2, generator=gen, dtype=torch.float64)
+    isg = 0.5 + torch.rand(3, 2, generator=gen, dtype=torch.float64)
+    go = torch.randn(1000, 3, generator=gen, dtype=torch.float64)
+    leaves = [t.clone().requires_grad_(True) for t in (pseudo, mu, isg)]
+    ref = orc.gaussian(*leaves)
+    ref.backward(go)
+    dl = [t.float().to(DEV).requires_grad_(True) for t in (pseudo, mu, isg)]
+    out = fg.GaussianCp(*dl)
+    out.backward(go.float().to(DEV))
+    assert_close(out, ref.detach(), "gaussian")
+    assert_close(dl[0].grad, leaves[0].grad, "grad pseudo")
+    assert_close(dl[1].grad, leaves[1].grad, "grad mu", rtol=1e-3, atol=1e-3)
+    assert_close(dl[2].grad, leaves[2].grad, "grad sigma", rtol=1e-3, atol=1e-3)
+
+
+def test_gmm_layer_matches_dgl_composed():
+    from ae_mlsys_gnn_amd.layers import GMMConv
+    torch.manual_seed(1)
+    g = graphs.add_csc_torch(graphs.rmat_graph(500, 6000, seed=2))
+    layer = GMMConv(32, 16, dim=2, n_kernels=3, residual=True, bias=True)
+    with torch.no_grad():
+        layer.bias.normal_()
+    feat = torch.randn(g.n, 32)
+    pseudo = torch.rand(g.n_edges, 2)
+    ref = orc.gmm_layer_dgl(layer.fc.weight.double(), layer.mu.double(), layer.inv_sigma.double(), layer.bias.double(),
+                            g.row_ptr, g.col_ind, feat.double(), pseudo.double(), layer.res_fc.weight.double())
+    gd = g.to(DEV)
+    out = layer.to(DEV)(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, feat.to(DEV), pseudo.to(DEV))
+    assert_close(out, ref.detach(), "GMMConv layer", atol=1e-4)
+
+
+# ------------------------------------------------------------------ GAT layer vs the DGL-composed layer
+def test_gat_layer_matches_dgl_composed():
+    from ae_mlsys_gnn_amd.layers import GATConv
+    torch.manual_seed(2)
+    g = graphs.add_csc_torch(graphs.uniform_graph(4096, 32768, seed=0))
+    layer = GATConv(64, 16, 4)
+    feat = torch.randn(g.n, 64)
+    # weight mapping to GATConv_dgl: fc.weight = W^T, attn_l(dgl) = attn_r(ours), attn_r(dgl) = attn_l(ours)
+    ref = orc.gat_layer_dgl(layer.W.t().double(), layer.attn_r.double(), layer.attn_l.double(), g.row_ptr, g.col_ind, 0.2,
+                            feat.double())
+    gd = g.to(DEV)
+    out = layer.to(DEV)(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, feat.to(DEV))
+    assert_close(out, ref.detach(), "GATConv layer")
+
+
+# ------------------------------------------------------------------ small operators
+def _small_graph():
+    return graphs.add_csc_torch(degree_edge_graph(n=300, seed=4))
+
+
+@pytest.mark.parametrize("h,f", [(4, 16), (8, 32), (1, 47), (3, 20), (2, 128)])
+def test_mhspmm_and_mhsddmm(h, f):
+    from ae_mlsys_gnn_amd.operators import mhspmm as op
+    g = _small_graph()
+    gen = torch.Generator().manual_seed(h * f)
+    feat = torch.randn(g.n, h, f, generator=gen, dtype=torch.float64)
+    att = torch.randn(g.n_edges, h, generator=gen, dtype=torch.float64)
+    go = torch.randn(g.n, h, f, generator=gen, dtype=torch.float64)
+    fl, al = feat.clone().requires_grad_(True), att.clone().requires_grad_(True)
+    ref = orc.mhspmm(g.row_ptr, g.col_ind, al, fl)
+    ref.backward(go)
+    gd = g.to(DEV)
+    fd, ad = feat.float().to(DEV).requires_grad_(True), att.float().to(DEV).requires_grad_(True)
+    out = op.csrmhspmm(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, ad)
+    out.backward(go.float().to(DEV))
+    assert_close(out, ref.detach(), "mhspmm", atol=1e-4)
+    assert_close(fd.grad, fl.grad, "mhspmm grad feat", atol=1e-4)
+    assert_close(ad.grad, al.grad, "mhspmm grad att (mhsddmm)", atol=1e-4)
+    tr = op.mhtranspose(gd.permute, ad.detach())
+    assert torch.equal(tr.cpu(), att.float()[g.permute.long()])
+
+
+def test_edge_softmax():
+    from ae_mlsys_gnn_amd.operators import edge_softmax as op
+    g = _small_graph()
+    h = torch.randn(g.n_edges, 4, dtype=torch.float64) * 3
+    go = torch.randn(g.n_edges, 4, dtype=torch.float64)
+    hl = h.clone().requires_grad_(True)
+    ref = orc.edge_softmax(g.row_ptr, hl)
+    ref.backward(go)
+    hd = h.float().to(DEV).requires_grad_(True)
+    out = op.csr_edge_softmax(g.row_ptr.to(DEV), hd)
+    out.backward(go.float().to(DEV))
+    assert_close(out, ref.detach(), "edge_softmax")
+    assert_close(hd.grad, hl.grad, "edge_softmax grad")
+
+
+def test_u_add_v():
+    from ae_mlsys_gnn_amd.operators import u_add_v as op
+    g = _small_graph()
+    rv = torch.randn(g.n, 4, dtype=torch.float64)
+    cv = torch.randn(g.n, 4, dtype=torch.float64)
+    go = torch.randn(g.n_edges, 4, dtype=torch.float64)
+    rl, cl = rv.clone().requires_grad_(True), cv.clone().requires_grad_(True)
+    ref = orc.u_add_v(g.row_ptr, g.col_ind, rl, cl)
+    ref.backward(go)
+    rd, cd = rv.float().to(DEV).requires_grad_(True), cv.float().to(DEV).requires_grad_(True)
+    out = op.u_add_v_op(g.row_ptr.to(DEV), g.col_ind.to(DEV), rd, cd)
+    out.backward(go.float().to(DEV))
+    assert_close(out, ref.detach(), "u_add_v")
+    assert_close(rd.grad, rl.grad, "u_add_v grad row", atol=1e-4)
+    assert_close(cd.grad, cl.grad, "u_add_v grad col", atol=1e-4)
+
+
+@pytest.mark.parametrize("weighted,sym", [(True, False), (False, False), (True, True)])
+def test_csrspmm(weighted, sym):
+    from ae_mlsys_gnn_amd.operators import spmm as op
+    g = _small_graph()
+    if sym:   # symmetric pattern: union of the graph and its transpose
+        dst = orc.row_of_edge(g.row_ptr)
+        src = g.col_ind.long()
+        keys = torch.unique(torch.cat([dst * g.n + src, src * g.n + dst]))
+        g = graphs.csr_from_keys(keys, g.n)
+    x = torch.randn(g.n, 48, dtype=torch.float64)
+    w = torch.rand(g.n_edges, dtype=torch.float64) if weighted else None
+    if sym and weighted:   # symmetric values too
+        dst = orc.row_of_edge(g.row_ptr)
+        src = g.col_ind.long()
+        w = torch.sin((dst + src).double()) + 0.1 * (dst * src % 7).double()
+    go = torch.randn(g.n, 48, dtype=torch.float64)
+    xl = x.clone().requires_grad_(True)
+    wl = None if w is None else w.clone().requires_grad_(True)
+    ref = orc.spmm(g.row_ptr, g.col_ind, xl, wl)
+    ref.backward(go)
+    xd = x.float().to(DEV).requires_grad_(True)
+    wd = None if w is None else w.float().to(DEV).requires_grad_(True)
+    out = op.csrspmm(g.row_ptr.to(DEV), g.col_ind.to(DEV), xd, wd, sym)
+    out.backward(go.float().to(DEV))
+    assert_close(out, ref.detach(), "csrspmm", atol=1e-4)
+    assert_close(xd.grad, xl.grad, "csrspmm grad x", atol=1e-4)
+    if weighted:
+        assert_close(wd.grad, wl.grad, "csrspmm grad w", atol=1e-4)
+
+
+def test_error_paths_return_codes_not_aborts():
+    from ae_mlsys_gnn_amd._lib import FgnnError
+    from ae_mlsys_gnn_amd.operators import fused_gat as fg
+    g = graphs.add_csc_torch(graphs.uniform_graph(64, 256)).to(DEV)
+    x = torch.randn(64, 8, 256, device=DEV)       # H*F = 2048 > limit
+    a = torch.randn(64, 8, device=DEV)
+    with pytest.raises(FgnnError, match="1024"):
+        fg.fused_gat_op(a, a, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, 0.2, x)
+    with pytest.raises(FgnnError, match="GPU only"):
+        fg.fused_gat_op(a.cpu(), a.cpu(), g.row_ptr.cpu(), g.col_ind.cpu(), g.col_ptr.cpu(), g.row_ind.cpu(), 0.2, x.cpu())
+    with pytest.raises(FgnnError, match="int32"):
+        fg.fused_gat_op(a, a, g.row_ptr.long(), g.col_ind, g.col_ptr, g.row_ind, 0.2, torch.randn(64, 8, 4, device=DEV))

@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(HERE, "libfgnn_hip.so")
 OBJ_DIR = os.path.join(HERE, "csrc", "_obj")
 
 HIPCC_FLAGS = [
-    "-std=c++20", "-O3", "--offload-arch=gfx950", "-fPIC",
+    "-std=c++20", "-O3", "--offload-arch=gfx950", "-fPIC", "-fvisibility=hidden",
     "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
     # packed fp32 VALU ops are kept off for every device function of the library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

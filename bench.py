@@ -1,0 +1,320 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused GNN sparse-operator path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gat_c2|gat_c5|edgeconv_c3|gmm_c4]
+
+Default workload = BASELINE config 2: one fused GAT layer forward+backward (dense projection by
+torch.matmul, fused sparse op by libfgnn_hip.so) on a seeded R-MAT power-law graph with 232,965
+nodes and ~114.6 M edges plus self loops, features [N,256], 8 heads x 32, fp32.  A step is one
+layer forward + backward; inputs are resident in HBM before the timed region; graph
+preprocessing (csr2csc, schedules) is reported separately.  One JSON line is printed with the
+metric, the roofline record of the dominant kernel (algorithmic bytes / live HIP-event time) and
+a CPU baseline (the torch-composed DGL-style layer of oracle/ on the host cores, on a bounded
+sample of the same graph).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published peak
+
+# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE,
+# scaled by a copy kernel of known size); see profiles/.  None = not measured for that workload.
+MEASURED_TRAFFIC_BYTES = {
+    "gat_c2": None,
+}
+
+
+def gat_alg_bytes(n, e, h, f):
+    """No-reuse gather model: every edge moves one feature row per gather pass."""
+    fwd = e * (4 * h * f + 4 * h + 4) + n * (4 * h * f + 12 * h + 4)
+    bwd = e * (4 * h * f + 16 * h + 4) + n * (16 * h * f + 24 * h + 4)
+    return fwd, bwd
+
+
+def time_calls(fn, steps, warmup):
+    """Average milliseconds of fn() over `steps` calls, HIP events on torch's current stream (the
+    stream every fgnn_* launch is given)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in ev:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    ts = [a.elapsed_time(b) for a, b in ev]
+    return sum(ts) / len(ts), min(ts), sorted(ts)[len(ts) // 2]
+
+
+def build_gat_graph(n, e, dev, seed=0):
+    import torch
+    from ae_mlsys_gnn_amd import graphs
+    from ae_mlsys_gnn_amd.operators import csr2csc as csc_op
+    t0 = time.time()
+    g = graphs.rmat_graph(n, e, seed=seed, device=dev)
+    torch.cuda.synchronize()
+    t_gen = time.time() - t0
+    t0 = time.time()
+    g.col_ptr, g.row_ind, g.permute = csc_op.csr2csc(g.row_ptr, g.col_ind)
+    torch.cuda.synchronize()
+    t_csc = time.time() - t0
+    return g, t_gen, t_csc
+
+
+def cpu_baseline_gat(g, x_feat, layer, slope, target_edges, go):
+    """The DGL-composed GAT layer (oracle.gat_layer_dgl: u_add_v, LeakyReLU, edge softmax,
+    u_mul_e + sum in plain torch) forward+backward on the host cores, on the sub-graph formed by the
+    first rows of the benchmark graph holding about `target_edges` edges; scaled to the full edge
+    count."""
+    import torch
+    from oracle import fgnn_oracle as orc
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    rp = g.row_ptr.cpu()
+    r = int(torch.searchsorted(rp.long(), torch.tensor([target_edges])).item())
+    r = max(1, min(r, g.n))
+    e_s = int(rp[r])
+    rp_s = torch.cat([rp[: r + 1], torch.full((g.n - r,), e_s, dtype=rp.dtype)])     # rows >= r are empty
+    ci_s = g.col_ind[:e_s].cpu()
+    feat = x_feat.detach().cpu()
+    w_t = layer.W.detach().cpu().t().contiguous().requires_grad_(True)
+    # weight mapping to GATConv_dgl: attn_l(dgl) = attn_r(ours), attn_r(dgl) = attn_l(ours)
+    al = layer.attn_r.detach().cpu().clone().requires_grad_(True)
+    ar = layer.attn_l.detach().cpu().clone().requires_grad_(True)
+    go_c = go.detach().cpu()
+
+    def step():
+        out = orc.gat_layer_dgl(w_t, al, ar, rp_s, ci_s, slope, feat)
+        out.backward(go_c)
+        w_t.grad = None; al.grad = None; ar.grad = None
+
+    step()
+    ts = []
+    t_all = time.time()
+    while len(ts) < 3 or (time.time() - t_all < 10.0 and len(ts) < 20):
+        t0 = time.time()
+        step()
+        ts.append((time.time() - t0) * 1e3)
+    ms = sorted(ts)[len(ts) // 2]
+    return ms, e_s, r, cores, len(ts)
+
+
+def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
+    import torch
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd.layers import GATConv
+    from ae_mlsys_gnn_amd.operators.fused_gat import gat_native
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    g, t_gen, t_csc = build_gat_graph(n, e_target, dev)
+    e = g.n_edges
+    t0 = time.time()
+    s_csr = _lib.schedule_for(g.row_ptr)
+    s_csc = _lib.schedule_for(g.col_ptr)
+    t_sched = time.time() - t0
+    slope = 0.2
+    layer = GATConv(in_feats, out_feats, heads, slope).to(dev)
+    with torch.no_grad():          # config: attn_l / attn_r ~ N(0, 0.1)
+        layer.attn_l.normal_(0, 0.1)
+        layer.attn_r.normal_(0, 0.1)
+    x = torch.randn(n, in_feats, device=dev)
+    go = torch.randn(n, heads, out_feats, device=dev)
+
+    def step():
+        out = layer(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, x)
+        out.backward(go)
+        for p in layer.parameters():
+            p.grad = None
+
+    # timed region: exactly K steps between two synchronisations
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # dominant kernels alone, through the C ABI, HIP events on the launch stream
+    with torch.no_grad():
+        h = torch.matmul(x, layer.W).view(-1, heads, out_feats).contiguous()
+        a_row = (layer.attn_l * h).sum(-1).contiguous()
+        a_col = (layer.attn_r * h).sum(-1).contiguous()
+    fwd_out = gat_native.gat_forward(a_row, a_col, g.row_ptr, g.col_ind, slope, h)
+    ms_fwd, ms_fwd_min, _ = time_calls(lambda: gat_native.gat_forward(a_row, a_col, g.row_ptr, g.col_ind, slope, h), args.steps, 2)
+    o = fwd_out
+    ms_bwd, ms_bwd_min, _ = time_calls(
+        lambda: gat_native.gat_backward(slope, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, o[1], o[2], h, a_row, a_col, go,
+                                        out_feat=o[0], out2=o[3], cc=o[4]), args.steps, 2)
+    b_fwd, b_bwd = gat_alg_bytes(n, e, heads, out_feats)
+    peak_mem = torch.cuda.max_memory_allocated() / 2**30
+
+    cpu_ms, cpu_e, cpu_rows, cores, cpu_iters = cpu_baseline_gat(g, x, layer, slope, args.cpu_sample_edges, go)
+    rec = {
+        "metric": "GAT layer fwd+bwd ms/iter + achieved HBM GB/s (% of peak), 1 MI355X",
+        "value": round(ms_step, 4), "unit": "ms/iter", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": workload, "graph": "R-MAT a=0.57 b=0.19 c=0.19 d=0.05 seed 0, unique edges + self loops",
+                   "nodes": n, "edges": e, "in_feats": in_feats, "heads": heads, "out_feats": out_feats,
+                   "negative_slope": slope, "step": "GATConv forward + backward (torch.matmul projection + fused sparse op)"},
+        "roofline": {"bound": "hbm", "kernel": "gat_fwd_kernel (+merge of split rows)", "achieved": round(b_fwd / ms_fwd / 1e6, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(b_fwd / ms_fwd / 1e6 / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(workload), "alg_bytes": b_fwd, "ms": round(ms_fwd, 4)},
+        "roofline_bwd": {"bound": "hbm", "kernel": "gat_bwd_node_kernel + gat_bwd_kernel (+merge)", "achieved": round(b_bwd / ms_bwd / 1e6, 1),
+                         "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(b_bwd / ms_bwd / 1e6 / HBM_PEAK_GBPS, 4),
+                         "alg_bytes": b_bwd, "ms": round(ms_bwd, 4)},
+        "sparse_fwd_bwd": {"ms": round(ms_fwd + ms_bwd, 4), "alg_bytes": b_fwd + b_bwd,
+                           "achieved_GBps": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6, 1),
+                           "frac_of_peak": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6 / HBM_PEAK_GBPS, 4)},
+        "cpu_baseline": {"value": round(cpu_ms * e / cpu_e, 1), "unit": "ms/iter", "cores": cores, "kind": "port",
+                         "sample": "DGL-composed GAT layer (torch CPU, %d threads) fwd+bwd on the first %d rows = %d edges of the same graph: "
+                                   "median %.1f ms over %d iters, scaled by E/E_sample = %.1f" % (cores, cpu_rows, cpu_e, cpu_ms, cpu_iters, e / cpu_e)},
+        "preprocess_s": {"graph_gen": round(t_gen, 3), "csr2csc_first_call": round(t_csc, 4), "schedules": round(t_sched, 4)},
+        "schedule": {"csr_items": s_csr.n_items, "csr_partials": s_csr.n_partials, "csc_items": s_csc.n_items, "csc_partials": s_csc.n_partials},
+        "peak_hbm_GiB": round(peak_mem, 3),
+    }
+    return rec
+
+
+def run_edgeconv(args):
+    import torch
+    from ae_mlsys_gnn_amd import graphs
+    from ae_mlsys_gnn_amd.operators.fused_edgeconv import edgeconv_native
+    from oracle import fgnn_oracle as orc
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    bsz, npts, k, f = 32, 1024, 20, 64
+    pts = (torch.rand(bsz, npts, 3, device=dev) * 2 - 1)
+    src = graphs.knn_graph(pts, k)
+    n = bsz * npts
+    theta = torch.nn.Linear(3, f, bias=False).to(dev)
+    phi = torch.nn.Linear(3, f, bias=False).to(dev)
+    xin = pts.reshape(-1, 3)
+    with torch.no_grad():
+        h_src = theta(xin).contiguous()
+        h_dst = (phi(xin) - h_src).contiguous()
+    go = torch.randn(n, f, device=dev)
+    out, arg = edgeconv_native.edgeconv_forward(k, src, h_src, h_dst)
+    ms_f, _, _ = time_calls(lambda: edgeconv_native.edgeconv_forward(k, src, h_src, h_dst), args.steps, args.warmup)
+    ms_b, _, _ = time_calls(lambda: edgeconv_native.edgeconv_backward(go, arg, n), args.steps, args.warmup)
+    e = n * k
+    b_f = e * (4 * f + 4) + n * f * 12
+    b_b = n * f * 20
+    # CPU baseline: EdgeConv_reorg composed math on the host, full size (it is small)
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    hs_c, hd_c, src_c = h_src.cpu().requires_grad_(True), h_dst.cpu().requires_grad_(True), src.cpu()
+    go_c = go.cpu()
+    ts = []
+    for _ in range(5):
+        t0 = time.time()
+        o = orc.edgeconv_forward_autograd(k, src_c, hs_c, hd_c)
+        o.backward(go_c)
+        hs_c.grad = None; hd_c.grad = None
+        ts.append((time.time() - t0) * 1e3)
+    ms = ms_f + ms_b
+    return {
+        "metric": "fused EdgeConv fwd+bwd us/iter + achieved GB/s, 1 MI355X", "value": round(ms * 1e3, 2), "unit": "us/iter", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "edgeconv_c3", "clouds": bsz, "points": npts, "k": k, "F": f, "edges": e},
+        "roofline": {"bound": "hbm", "kernel": "edgeconv_fwd_kernel", "achieved": round(b_f / ms_f / 1e6, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(b_f / ms_f / 1e6 / HBM_PEAK_GBPS, 4), "traffic": None, "alg_bytes": b_f, "ms": round(ms_f, 5)},
+        "roofline_bwd": {"bound": "hbm", "kernel": "fill + edgeconv_bwd_kernel", "achieved": round(b_b / ms_b / 1e6, 1), "peak": HBM_PEAK_GBPS,
+                         "unit": "GB/s", "frac": round(b_b / ms_b / 1e6 / HBM_PEAK_GBPS, 4), "alg_bytes": b_b, "ms": round(ms_b, 5)},
+        "cpu_baseline": {"value": round(sorted(ts)[len(ts) // 2] * 1e3, 1), "unit": "us/iter", "cores": cores, "kind": "port",
+                         "sample": "EdgeConv_reorg composed math (torch CPU gather + max over k) fwd+bwd at full size, median of 5"},
+    }
+
+
+def run_gmm(args):
+    import torch
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd.operators.fused_gmmconv import gmm_native
+    from oracle import fgnn_oracle as orc
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    n, e_t, kk, dim, f = 169343, 2_300_000, 3, 2, 64
+    g, t_gen, t_csc = build_gat_graph(n, e_t, dev, seed=1)
+    e = g.n_edges
+    deg = (g.row_ptr[1:] - g.row_ptr[:-1]).float()
+    dst = torch.repeat_interleave(torch.arange(n, device=dev), (g.row_ptr[1:] - g.row_ptr[:-1]).long())
+    src = g.col_ind.long()
+    pseudo = torch.stack([deg[src].rsqrt(), deg[dst].rsqrt()], 1).contiguous()      # CSR position order
+    x = torch.randn(n, kk, f, device=dev)
+    mu = torch.rand(kk, dim, device=dev)
+    isg = torch.ones(kk, dim, device=dev)
+    go = torch.randn(n, kk, f, device=dev)
+    _lib.schedule_for(g.row_ptr); _lib.schedule_for(g.col_ptr)
+    ms_f, _, _ = time_calls(lambda: gmm_native.gmmconv(g.row_ptr, g.col_ind, x, pseudo, mu, isg), args.steps, args.warmup)
+    ms_b, _, _ = time_calls(lambda: gmm_native.gmmconv_backward(g.col_ptr, g.row_ind, g.permute, x, pseudo, mu, isg, go), args.steps, args.warmup)
+    b_f = e * (4 * kk * f + 4 * dim + 4) + n * (4 * kk * f + 4)
+    b_b = e * (4 * kk * f + 8 * dim + 12) + n * (8 * kk * f + 4)
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    leaves = [t.cpu().requires_grad_(True) for t in (x, pseudo, mu, isg)]
+    rp_c, ci_c, go_c = g.row_ptr.cpu(), g.col_ind.cpu(), go.cpu()
+    ts = []
+    for _ in range(3):
+        t0 = time.time()
+        orc.gmm_forward(rp_c, ci_c, *leaves).backward(go_c)
+        for t in leaves:
+            t.grad = None
+        ts.append((time.time() - t0) * 1e3)
+    ms = ms_f + ms_b
+    return {
+        "metric": "fused GMMConv fwd+bwd ms/iter + achieved GB/s, 1 MI355X", "value": round(ms, 4), "unit": "ms/iter", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "gmm_c4", "nodes": n, "edges": e, "K": kk, "dim": dim, "F": f},
+        "roofline": {"bound": "hbm", "kernel": "spmm_kernel<WGauss>", "achieved": round(b_f / ms_f / 1e6, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(b_f / ms_f / 1e6 / HBM_PEAK_GBPS, 4), "traffic": None, "alg_bytes": b_f, "ms": round(ms_f, 4)},
+        "roofline_bwd": {"bound": "hbm", "kernel": "gmm_bwd_kernel (+column sums)", "achieved": round(b_b / ms_b / 1e6, 1), "peak": HBM_PEAK_GBPS,
+                         "unit": "GB/s", "frac": round(b_b / ms_b / 1e6 / HBM_PEAK_GBPS, 4), "alg_bytes": b_b, "ms": round(ms_b, 4)},
+        "cpu_baseline": {"value": round(sorted(ts)[1], 1), "unit": "ms/iter", "cores": cores, "kind": "port",
+                         "sample": "GMMConv_dgl composed math (torch CPU) fwd+bwd at full size, median of 3"},
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="gat_c2", choices=["gat_c2", "gat_c5", "edgeconv_c3", "gmm_c4"])
+    ap.add_argument("--cpu-sample-edges", type=int, default=1_500_000)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures ONE GPU: the fused sparse-operator path is single-GPU (as is the reference); "
+              "run with --gpus 1 (got --gpus %d, WORLD_SIZE=%s)" % (args.gpus, os.environ.get("WORLD_SIZE", "1")), file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (torch.cuda.is_available() is False)", file=sys.stderr)
+        sys.exit(2)
+    if args.workload == "gat_c2":
+        rec = run_gat(args, 232965, 114_600_000, 256, 8, 32, "gat_c2")
+    elif args.workload == "gat_c5":
+        rec = run_gat(args, 2449029, 61_900_000, 100, 8, 32, "gat_c5_layer1")
+    elif args.workload == "edgeconv_c3":
+        rec = run_edgeconv(args)
+    else:
+        rec = run_gmm(args)
+    print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+    main()

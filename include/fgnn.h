@@ -25,6 +25,8 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+/* the library is built with hidden visibility; only the declarations below are exported */
+#pragma GCC visibility push(default)
 
 #define FGNN_ERR_NULL      (-1)  /* a required pointer is NULL */
 #define FGNN_ERR_SHAPE     (-2)  /* a size is negative or inconsistent */
@@ -123,7 +125,8 @@ int    fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F,
 /* Replaces the backward sequence of operators/fused_gmmconv.py:51-58 (mhsddmm + mhtranspose +
  * gmmconv over CSC + GaussianBp, gmmconv.cu:265-285) with one pass over the CSC arrays:
  * grad_feat [N,K,F], grad_pseudo [E,dim] (CSR order), grad_mu, grad_sigma [K,dim].
- * grad_mu / grad_sigma are accumulated with float atomics (K*dim values per workgroup). */
+ * grad_mu / grad_sigma are summed per work item and reduced in two fixed-order levels
+ * (bit-reproducible).  A schedule of col_ptr is required; K*dim <= 32. */
 size_t fgnn_gmm_backward_workspace_bytes(const fgnn_schedule_t *sched_csc, int K, int dim, int F);
 int    fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F,
                          const int32_t *col_ptr, const int32_t *row_ind, const int32_t *permute,
@@ -180,6 +183,7 @@ int    fgnn_csr2csc(int n_rows, int n_cols, int64_t E, const int32_t *row_ptr, c
                     int32_t *col_ptr, int32_t *row_ind, int32_t *permute,
                     void *workspace, size_t workspace_bytes, void *stream);
 
+#pragma GCC visibility pop
 #ifdef __cplusplus
 }
 #endif

@@ -12,8 +12,9 @@ _SO = os.path.join(_HERE, "_build", "libfgnn_oracle.so")
 
 
 def build(force: bool = False) -> str:
-    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(os.path.join(_HERE, "fgnn_oracle.c")):
-        subprocess.check_call(["make", "-s", "-B" if force else "-s", "-C", _HERE])
+    src = os.path.join(_HERE, "fgnn_oracle.c")
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-s", "-C", _HERE] + (["-B"] if force else []))
     return _SO
 
 

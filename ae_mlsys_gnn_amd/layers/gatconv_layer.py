@@ -30,10 +30,16 @@ class _GATBase(nn.Module):
             nn.init.xavier_normal_(p, gain=gain)
 
     def _project(self, feat):
-        h = torch.matmul(feat, self.W).view(-1, self.num_heads, self.out_feats)
-        attn_row = (self.attn_l * h).sum(dim=-1)
-        attn_col = (self.attn_r * h).sum(dim=-1)
-        return h, attn_row, attn_col
+        """h = feat @ W and the two attention scores (attn_l * h).sum(-1), (attn_r * h).sum(-1)
+        (layers/gatconv_layer.py:50-53 of the reference).  The scores are formed as
+        feat @ ((W * attn).sum(-1)): the same sums taken in another order, as one thin GEMM over
+        `feat` instead of two strided reductions over the [N,H,F] projection."""
+        hh, ff = self.num_heads, self.out_feats
+        h = torch.matmul(feat, self.W).view(-1, hh, ff)
+        wv = self.W.view(self.in_feats, hh, ff)
+        w_score = torch.cat([(wv * self.attn_l).sum(-1), (wv * self.attn_r).sum(-1)], dim=1)      # [in, 2H]
+        score = torch.matmul(feat, w_score)
+        return h, score[:, :hh].contiguous(), score[:, hh:].contiguous()
 
 
 class GATConv(_GATBase):

@@ -1,11 +1,11 @@
 // Fused GAT forward / backward for gfx950.
 //
 // Forward (one gather pass over CSR rows): per work item (a row, or a segment of a long row) a
-// wave first finds the per-head maximum of lrelu(attn_row[i] + attn_col[j]) over its edges
-// (reads col_ind and attn_col only), then walks the edges again in chunks of 64: lanes-as-edges
-// compute the softmax numerators into wave-private LDS, lanes-as-features accumulate
-// numerator * in_feat[j] with one 128-bit load per lane and edge.  Next to the plain sum T the
-// wave keeps P, the sum over edges with a positive pre-activation; T and P give both
+// wave streams over the edges 8 at a time.  The 64 lanes own the floats of a feature row (one
+// 128-bit load per lane and edge); every lane also reads attn_col[j, head of its floats] and
+// computes the softmax numerator itself, with an online (running-maximum) softmax, so there is
+// no separate maximum pass, no cross-lane traffic and no LDS.  Next to the plain sum T the wave
+// keeps P, the sum over edges with a positive pre-activation; T and P give both
 //   out  = T / s                         and
 //   out2 = (slope*T + (1-slope)*P) / s   = sum_p alpha_p * lrelu'(e_p) * in_feat[j_p],
 // which turns the gradient of attn_row into node-wise dot products in the backward.
@@ -33,62 +33,99 @@ struct GatFwdP {
 // Partial layout (floats): T[HF] | P[HF] (AUX only) | m[H] | s[H] | cp[H]
 __host__ __device__ static inline int gat_fwd_pw(int HF, int H, bool aux) { return ((aux ? 2 : 1) * HF + 3 * H + 3) & ~3; }
 
+// One batch of UB edges of the forward: UB feature rows and UB x R attention scores are fetched
+// together (every lane reads the score of the head its features belong to), then the running
+// maximum of the online softmax is raised once for the batch and the rows are accumulated.
+template <int VEC, int R, bool AUX, bool FULL, int UB>
+__device__ __forceinline__ void gat_fwd_batch(const GatFwdP &p, const fg_lanemap<VEC, R> &lm, int idv, int t, int cnt,
+                                              const float (&arh)[R], float (&m)[R], float (&s)[R], float (&cp)[R],
+                                              fg_vec<VEC> (&T)[R], fg_vec<VEC> (&P)[R])
+{
+    fg_vec<VEC> ld[UB][R];
+    float ev[UB][R];
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+        int j = __builtin_amdgcn_readlane(idv, t + u);
+        const float *base = p.x + (size_t)j * (size_t)p.HF;
+        const float *acb = p.ac + (size_t)j * (size_t)p.H;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (FULL || lm.ok[r]) { ld[u][r].load(base + lm.eoff[r]); ev[u][r] = acb[lm.hd[r]]; }
+            else { ld[u][r].zero(); ev[u][r] = 0.f; }
+        }
+    }
+    float bm[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) bm[r] = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+        const bool live = (t + u) < cnt;           // wave-uniform: edges past the chunk get weight 0
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            float v = fg_lrelu(arh[r] + ev[u][r], p.slope);
+            v = live ? v : -INFINITY;
+            ev[u][r] = v;
+            bm[r] = fmaxf(bm[r], v);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        float mn = fmaxf(m[r], bm[r]);
+        float sc = __expf(m[r] - mn);              // 1 when the maximum did not move, 0 on the first batch
+        m[r] = mn;
+        T[r].scale(sc);
+        s[r] *= sc;
+        if (AUX) { P[r].scale(sc); cp[r] *= sc; }
+    }
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            float w = __expf(ev[u][r] - m[r]);
+            T[r].fma(w, ld[u][r]);
+            s[r] += w;
+            if (AUX) {
+                float wp = ev[u][r] > 0.f ? w : 0.f;
+                P[r].fma(wp, ld[u][r]);
+                cp[r] += wp;
+            }
+        }
+    }
+}
+
 template <int VEC, int R, bool AUX, bool FULL>
 __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_kernel(GatFwdP p)
 {
-    extern __shared__ float lds[];
     int row, b, e, slot;
     if (!fg_get_item(p.items, p.n_items, p.ptr, row, b, e, slot)) return;
     const int lane = fg_lane();
     const int H = p.H;
-    float *wl = lds + fg_wave() * (H * 64);
     fg_lanemap<VEC, R> lm;
     lm.init(lane, p.HF, p.F);
     const float slope = p.slope;
-    const float *arp = p.ar + (size_t)row * H;
-
-    // pass A: per-head maximum; lane h keeps the maximum of head h
-    float mst = -INFINITY;
-    for (int c = b; c < e; c += 64) {
-        int q = c + lane;
-        bool ok = q < e;
-        int id = p.idx[ok ? q : c];
-        const float *acp = p.ac + (size_t)id * H;
-        for (int h = 0; h < H; ++h) {
-            float ev = fg_lrelu(arp[h] + acp[h], slope);
-            ev = ok ? ev : -INFINITY;
-            float r = fg_wave_max(ev);
-            mst = (lane == h) ? fmaxf(mst, r) : mst;
-        }
-    }
 
     fg_vec<VEC> T[R], P[R];
-    float s[R], cp[R];
+    float arh[R], m[R], s[R], cp[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) { T[r].zero(); P[r].zero(); s[r] = 0.f; cp[r] = 0.f; }
-
-    // pass B: numerators into LDS, weighted gather
+    for (int r = 0; r < R; ++r) {
+        T[r].zero(); P[r].zero(); s[r] = 0.f; cp[r] = 0.f; m[r] = -INFINITY;
+        arh[r] = p.ar[(size_t)row * H + lm.hd[r]];
+    }
+    constexpr int U = (R >= 8) ? 1 : 8 / R;        // feature rows in flight per wave
     for (int c = b; c < e; c += 64) {
         int q = c + lane;
-        bool ok = q < e;
         int cnt = min(64, e - c);
-        int id = p.idx[ok ? q : c];
-        const float *acp = p.ac + (size_t)id * H;
-        for (int h = 0; h < H; ++h) {
-            float mh = fg_readlane(mst, h);
-            float ev = fg_lrelu(arp[h] + acp[h], slope);
-            float w = ok ? __expf(ev - mh) : 0.f;
-            wl[h * 64 + lane] = (!AUX || ev > 0.f) ? w : -w;
+        int idv = p.idx[q < e ? q : c];            // lanes past the end repeat a valid id
+        int t = 0;
+        for (; t + U <= cnt; t += U) gat_fwd_batch<VEC, R, AUX, FULL, U>(p, lm, idv, t, cnt, arh, m, s, cp, T, P);
+        if constexpr (U >= 4) {
+            if (cnt - t > U / 2) { gat_fwd_batch<VEC, R, AUX, FULL, U>(p, lm, idv, t, cnt, arh, m, s, cp, T, P); t = cnt; }
+            else if (cnt - t > 0) { gat_fwd_batch<VEC, R, AUX, FULL, U / 2>(p, lm, idv, t, cnt, arh, m, s, cp, T, P); t = cnt; }
+        } else {
+            if (cnt - t > 0) gat_fwd_batch<VEC, R, AUX, FULL, U>(p, lm, idv, t, cnt, arh, m, s, cp, T, P);
         }
-        fg_wave_lds_sync();
-        fg_accum_chunk<VEC, R, AUX, true, FULL>(p.x, p.HF, id, cnt, wl, lm, T, P, s, cp);
-        fg_wave_lds_sync();
     }
 
-    // every lane fetches the maximum of its heads while the whole wave is still active
-    float mhr[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) mhr[r] = fg_bperm(mst, lm.hd[r]);
     if (slot < 0) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -101,10 +138,9 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_kernel(GatFwdP p)
             }
             T[r].scale(inv);
             T[r].store(p.out + o);
-            float mh = mhr[r];
             if (lm.eoff[r] % p.F == 0) {
                 size_t so = (size_t)row * H + lm.hd[r];
-                p.emax[so] = (b < e) ? mh : -1e38f;
+                p.emax[so] = (b < e) ? m[r] : -1e38f;
                 p.esum[so] = s[r];
                 if (AUX) p.cc[so] = (cp[r] + slope * (s[r] - cp[r])) * inv;
             }
@@ -113,13 +149,12 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_kernel(GatFwdP p)
         float *pp = p.part + (size_t)slot * gat_fwd_pw(p.HF, H, AUX);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            float mh = mhr[r];
             if (!(FULL || lm.ok[r])) continue;
             T[r].store(pp + lm.eoff[r]);
             if (AUX) P[r].store(pp + p.HF + lm.eoff[r]);
             if (lm.eoff[r] % p.F == 0) {
                 float *st = pp + (AUX ? 2 : 1) * p.HF;
-                st[lm.hd[r]] = mh;
+                st[lm.hd[r]] = m[r];
                 st[H + lm.hd[r]] = s[r];
                 st[2 * H + lm.hd[r]] = cp[r];
             }
@@ -241,11 +276,14 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_node_kernel(int N, int H, in
     }
 }
 
+// Writes grad_feat[col] = T and grad_attn_col[col,h] = <x[col,h,:], slope*T + (1-slope)*P> - z[h].
+// z[r] is held by every lane of head hd[r]; scr is wave-private LDS of 64*R + 64 floats.
 template <int VEC, int R>
 __device__ __forceinline__ void gat_bwd_finish(const GatBwdP &p, int col, int lane, float *scr, const fg_lanemap<VEC, R> &lm,
-                                               fg_vec<VEC> (&T)[R], fg_vec<VEC> (&P)[R], float zsum /* lane h: head h */)
+                                               fg_vec<VEC> (&T)[R], fg_vec<VEC> (&P)[R], const float (&z)[R])
 {
     float d[R];
+    float *zs = scr + 64 * R;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         d[r] = 0.f;
@@ -255,10 +293,54 @@ __device__ __forceinline__ void gat_bwd_finish(const GatBwdP &p, int col, int la
             fg_vec<VEC> g2 = T[r].lin(p.slope, 1.f - p.slope, P[r]);
             fg_vec<VEC> xv; xv.load(p.x + o);
             d[r] = xv.dot(g2);
+            if (lm.eoff[r] % p.F == 0) zs[lm.hd[r]] = z[r];
         }
     }
     float dot = fg_head_reduce<VEC, R>(scr, d, lm, lane, p.H, p.F);
-    if (lane < p.H) p.gac[(size_t)col * p.H + lane] = dot - zsum;
+    if (lane < p.H) p.gac[(size_t)col * p.H + lane] = dot - zs[lane];
+}
+
+// One batch of UB edges of the backward column pass.  Every lane reads the 16-byte record
+// (attn_row, max, 1/sum, delta) of the head its features belong to and recomputes alpha itself.
+template <int VEC, int R, bool STASH, bool FULL, int UB>
+__device__ __forceinline__ void gat_bwd_batch(const GatBwdP &p, const fg_lanemap<VEC, R> &lm, int idv, int posv, int t, int cnt,
+                                              const float (&ach)[R], float (&z)[R], fg_vec<VEC> (&T)[R], fg_vec<VEC> (&P)[R])
+{
+    fg_vec<VEC> ld[UB][R];
+    float4 rc[UB][R];
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+        int i = __builtin_amdgcn_readlane(idv, t + u);
+        const float *base = p.g + (size_t)i * (size_t)p.HF;
+        const float4 *rb = p.rec + (size_t)i * (size_t)p.H;
+        size_t pos = STASH ? (size_t)__builtin_amdgcn_readlane(posv, t + u) * (size_t)p.H : 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (FULL || lm.ok[r]) {
+                ld[u][r].load(base + lm.eoff[r]);
+                rc[u][r] = rb[lm.hd[r]];
+                if (STASH) { rc[u][r].x = p.erelu[pos + lm.hd[r]]; rc[u][r].y = p.esm[pos + lm.hd[r]]; }
+            } else {
+                ld[u][r].zero();
+                rc[u][r] = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+        const bool live = (t + u) < cnt;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            float ev, al;
+            if (STASH) { ev = rc[u][r].x; al = rc[u][r].y; }
+            else { ev = fg_lrelu(rc[u][r].x + ach[r], p.slope); al = __expf(ev - rc[u][r].y) * rc[u][r].z; }
+            al = live ? al : 0.f;
+            const bool pos_e = ev > 0.f;
+            T[r].fma(al, ld[u][r]);
+            P[r].fma(pos_e ? al : 0.f, ld[u][r]);
+            z[r] = fmaf(pos_e ? al : al * p.slope, rc[u][r].w, z[r]);
+        }
+    }
 }
 
 template <int VEC, int R, bool STASH, bool FULL>
@@ -269,56 +351,34 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_kernel(GatBwdP p)
     if (!fg_get_item(p.items, p.n_items, p.ptr, col, b, e, slot)) return;
     const int lane = fg_lane();
     const int H = p.H;
-    const int per_wave = max(2 * H * 64, 64 * R);
-    float *wl = lds + fg_wave() * per_wave;
-    float *zl = wl + H * 64;
+    float *scr = lds + fg_wave() * (64 * R + 64);
     fg_lanemap<VEC, R> lm;
     lm.init(lane, p.HF, p.F);
-    const float slope = p.slope;
-    const float *acp = p.ac + (size_t)col * H;
 
-    for (int h = 0; h < H; ++h) zl[h * 64 + lane] = 0.f;
     fg_vec<VEC> T[R], P[R];
-    float s[R], cp[R];
+    float ach[R], z[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) { T[r].zero(); P[r].zero(); s[r] = 0.f; cp[r] = 0.f; }
+    for (int r = 0; r < R; ++r) { T[r].zero(); P[r].zero(); z[r] = 0.f; ach[r] = p.ac[(size_t)col * H + lm.hd[r]]; }
 
+    constexpr int U = (R >= 8) ? 1 : 8 / R;
     for (int c = b; c < e; c += 64) {
         int q = c + lane;
-        bool ok = q < e;
         int cnt = min(64, e - c);
-        int id = p.idx[ok ? q : c];
-        const float4 *rp = p.rec + (size_t)id * H;
-        size_t pos = STASH ? (size_t)p.permute[ok ? q : c] * H : 0;
-        for (int h = 0; h < H; ++h) {
-            float4 rc = rp[h];
-            float ev, al;
-            if (STASH) {
-                ev = p.erelu[pos + h];
-                al = p.esm[pos + h];
-            } else {
-                ev = fg_lrelu(rc.x + acp[h], slope);
-                al = __expf(ev - rc.y) * rc.z;
-            }
-            al = ok ? al : 0.f;
-            bool pos_e = ev > 0.f;
-            wl[h * 64 + lane] = pos_e ? al : -al;
-            zl[h * 64 + lane] += (pos_e ? al : al * slope) * rc.w;
+        int qq = q < e ? q : c;
+        int idv = p.idx[qq];
+        int posv = STASH ? p.permute[qq] : 0;
+        int t = 0;
+        for (; t + U <= cnt; t += U) gat_bwd_batch<VEC, R, STASH, FULL, U>(p, lm, idv, posv, t, cnt, ach, z, T, P);
+        if constexpr (U >= 4) {
+            if (cnt - t > U / 2) gat_bwd_batch<VEC, R, STASH, FULL, U>(p, lm, idv, posv, t, cnt, ach, z, T, P);
+            else if (cnt - t > 0) gat_bwd_batch<VEC, R, STASH, FULL, U / 2>(p, lm, idv, posv, t, cnt, ach, z, T, P);
+        } else {
+            if (cnt - t > 0) gat_bwd_batch<VEC, R, STASH, FULL, U>(p, lm, idv, posv, t, cnt, ach, z, T, P);
         }
-        fg_wave_lds_sync();
-        fg_accum_chunk<VEC, R, true, false, FULL>(p.g, p.HF, id, cnt, wl, lm, T, P, s, cp);
-        fg_wave_lds_sync();
     }
 
-    // per-head sum of z over the 64 edge slots; lane h keeps head h
-    float zsum = 0.f;
-    for (int h = 0; h < H; ++h) {
-        float z = fg_wave_sum(zl[h * 64 + lane]);
-        zsum = (lane == h) ? z : zsum;
-    }
-    fg_wave_lds_sync();
     if (slot < 0) {
-        gat_bwd_finish<VEC, R>(p, col, lane, wl, lm, T, P, zsum);
+        gat_bwd_finish<VEC, R>(p, col, lane, scr, lm, T, P, z);
     } else {
         float *pp = p.part + (size_t)slot * gat_bwd_pw(p.HF, H);
 #pragma unroll
@@ -326,8 +386,8 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_kernel(GatBwdP p)
             if (!(FULL || lm.ok[r])) continue;
             T[r].store(pp + lm.eoff[r]);
             P[r].store(pp + p.HF + lm.eoff[r]);
+            if (lm.eoff[r] % p.F == 0) pp[2 * p.HF + lm.hd[r]] = z[r];
         }
-        if (lane < H) pp[2 * p.HF + lane] = zsum;
     }
 }
 
@@ -342,13 +402,13 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_merge_kernel(GatBwdP p, cons
     const int lane = fg_lane();
     const int H = p.H, HF = p.HF;
     const int pw = gat_bwd_pw(HF, H);
-    float *scr = lds + fg_wave() * (64 * R);
+    float *scr = lds + fg_wave() * (64 * R + 64);
     fg_lanemap<VEC, R> lm;
     lm.init(lane, HF, p.F);
     fg_vec<VEC> T[R], P[R];
+    float z[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) { T[r].zero(); P[r].zero(); }
-    float zsum = 0.f;
+    for (int r = 0; r < R; ++r) { T[r].zero(); P[r].zero(); z[r] = 0.f; }
     const float *base = p.part + (size_t)first * pw;
     for (int g = 0; g < nseg; ++g) {
         const float *pg = base + (size_t)g * pw;
@@ -358,10 +418,10 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_merge_kernel(GatBwdP p, cons
             fg_vec<VEC> t, q;
             t.load(pg + lm.eoff[r]); q.load(pg + HF + lm.eoff[r]);
             T[r].add(t); P[r].add(q);
+            z[r] += pg[2 * HF + lm.hd[r]];
         }
-        if (lane < H) zsum += pg[2 * HF + lane];
     }
-    gat_bwd_finish<VEC, R>(p, col, lane, scr, lm, T, P, zsum);
+    gat_bwd_finish<VEC, R>(p, col, lane, scr, lm, T, P, z);
 }
 
 // ------------------------------------------------------------------------------- host
@@ -413,7 +473,7 @@ static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_
     }
     if (p.n_items == 0) return 0;
     const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
-    const size_t shm = (size_t)FGNN_WPB * H * 64 * sizeof(float);
+    const size_t shm = 0;
     int rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
         if (aux) hipLaunchKernelGGL((gat_fwd_kernel<VEC, R, true, FULL>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
         else hipLaunchKernelGGL((gat_fwd_kernel<VEC, R, false, FULL>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
@@ -528,15 +588,14 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
         int rc2 = fgnn_launch_status("gat_bwd_node_kernel");
         if (rc2) return rc2;
         const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
-        const size_t per_wave = (size_t)((2 * H * 64 > 64 * R) ? 2 * H * 64 : 64 * R);
-        const size_t shm = FGNN_WPB * per_wave * sizeof(float);
+        const size_t shm = (size_t)FGNN_WPB * (64 * R + 64) * sizeof(float);
         if (stash) hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, true, FULL>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
         else hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, false, FULL>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
         rc2 = fgnn_launch_status("gat_bwd_kernel");
         if (rc2) return rc2;
         if (sched_csc && sched_csc->n_split > 0) {
             unsigned g2 = (unsigned)((sched_csc->n_split + FGNN_WPB - 1) / FGNN_WPB);
-            hipLaunchKernelGGL((gat_bwd_merge_kernel<VEC, R>), dim3(g2), dim3(FGNN_TPB), (size_t)FGNN_WPB * 64 * R * sizeof(float), st,
+            hipLaunchKernelGGL((gat_bwd_merge_kernel<VEC, R>), dim3(g2), dim3(FGNN_TPB), shm, st,
                                p, sched_csc->split_dev, sched_csc->n_split);
             return fgnn_launch_status("gat_bwd_merge_kernel");
         }

@@ -1,0 +1,161 @@
+"""Full-size checks at the benchmark configurations.  Where the CPU oracle is too slow (the
+115 M-edge GAT graph) the checks are size-independent properties of the math: attention rows sum
+to one, zero attention is the neighbour mean, linearity in the features, the column-sum checksum
+of grad_feat, the slope == 1 shift invariance, and the transpose round trip of csr2csc.  EdgeConv
+(C3) and GMMConv (C4) are small enough to compare with the oracle at full size."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle
+from oracle import fgnn_oracle as orc
+from tests.util import assert_close
+from ae_mlsys_gnn_amd import graphs
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def c2_graph():
+    from ae_mlsys_gnn_amd.operators import csr2csc as csc_op
+    g = graphs.rmat_graph(232965, 114_600_000, seed=0, device=DEV)
+    g.col_ptr, g.row_ind, g.permute = csc_op.csr2csc(g.row_ptr, g.col_ind)
+    return g
+
+
+def test_c2_csr2csc_properties(c2_graph):
+    from ae_mlsys_gnn_amd.operators import csr2csc as csc_op
+    g = c2_graph
+    e = g.n_edges
+    assert e == 114_600_000 + g.n
+    # permute is a permutation; columns ascending; positions ascending inside a column (stable)
+    pm = g.permute.long()
+    assert torch.equal(torch.sort(pm).values, torch.arange(e, device=DEV))
+    cols = g.col_ind.long()[pm]
+    assert bool((cols[1:] >= cols[:-1]).all())
+    same = cols[1:] == cols[:-1]
+    assert bool((pm[1:][same] > pm[:-1][same]).all())
+    assert torch.equal(g.col_ptr.long(), torch.cat([torch.zeros(1, dtype=torch.long, device=DEV),
+                                                    torch.cumsum(torch.bincount(g.col_ind.long(), minlength=g.n), 0)]))
+    # transpose of the transpose is the original (columns are sorted inside the rows of this graph)
+    rp2, ci2, pm2 = csc_op.csr2csc(g.col_ptr, g.row_ind)
+    assert torch.equal(rp2, g.row_ptr) and torch.equal(ci2, g.col_ind)
+    assert torch.equal(pm[pm2.long()], torch.arange(e, device=DEV))
+
+
+def test_c2_gat_forward_properties(c2_graph):
+    from ae_mlsys_gnn_amd.operators.fused_gat import gat_native
+    g = c2_graph
+    n, h, f = g.n, 8, 32
+    torch.manual_seed(0)
+    ar = torch.randn(n, h, device=DEV)
+    ac = torch.randn(n, h, device=DEV)
+    # (1) constant feature rows come back unchanged: attention rows sum to one
+    c = torch.randn(1, h, f, device=DEV).expand(n, h, f).contiguous()
+    out = gat_native.gat_forward(ar, ac, g.row_ptr, g.col_ind, 0.2, c)[0]
+    assert float((out - c).abs().max()) < 2e-5
+    # (2) linearity in the features for fixed attention
+    x1 = torch.randn(n, h, f, device=DEV)
+    x2 = torch.randn(n, h, f, device=DEV)
+    o1 = gat_native.gat_forward(ar, ac, g.row_ptr, g.col_ind, 0.2, x1)[0]
+    o2 = gat_native.gat_forward(ar, ac, g.row_ptr, g.col_ind, 0.2, x2)[0]
+    o12 = gat_native.gat_forward(ar, ac, g.row_ptr, g.col_ind, 0.2, x1 + 2 * x2)[0]
+    assert float((o12 - (o1 + 2 * o2)).abs().max()) < 5e-5
+    # (3) zero attention is the neighbour mean (reference sum built with index_add_ in edge chunks)
+    z = torch.zeros(n, h, device=DEV)
+    om = gat_native.gat_forward(z, z, g.row_ptr, g.col_ind, 0.2, x1)[0]
+    deg = (g.row_ptr[1:] - g.row_ptr[:-1]).long()
+    dst = torch.repeat_interleave(torch.arange(n, device=DEV), deg)
+    acc = torch.zeros(n, h * f, dtype=torch.float64, device=DEV)
+    xf = x1.view(n, h * f)
+    step = 4_000_000
+    for s in range(0, g.n_edges, step):
+        sl = slice(s, min(s + step, g.n_edges))
+        acc.index_add_(0, dst[sl], xf[g.col_ind[sl].long()].double())
+    mean = (acc / deg.view(n, 1)).view(n, h, f)
+    assert_close(om, mean, "neighbour mean at C2", atol=2e-5)
+    # (4) stored row statistics: with zero attention max = 0 and sum = degree
+    st = gat_native.gat_forward(z, z, g.row_ptr, g.col_ind, 0.2, x1)
+    assert float(st[1].abs().max()) == 0.0
+    assert torch.equal(st[2], deg.float().view(n, 1).expand(n, h))
+
+
+def test_c2_gat_backward_properties(c2_graph):
+    from ae_mlsys_gnn_amd.operators.fused_gat import gat_native
+    g = c2_graph
+    n, h, f = g.n, 8, 32
+    torch.manual_seed(1)
+    ar = torch.randn(n, h, device=DEV) * 0.5
+    ac = torch.randn(n, h, device=DEV) * 0.5
+    x = torch.randn(n, h, f, device=DEV)
+    go = torch.randn(n, h, f, device=DEV)
+
+    def run(slope, feat):
+        o = gat_native.gat_forward(ar, ac, g.row_ptr, g.col_ind, slope, feat)
+        return o, gat_native.gat_backward(slope, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, o[1], o[2], feat, ar, ac, go,
+                                          out_feat=o[0], out2=o[3], cc=o[4])
+    # checksum: every attention row sums to one, so the column sums of grad_feat equal those of grad_out
+    o, (gx, gar, gac) = run(0.2, x)
+    assert_close(gx.double().sum(0), go.double().sum(0), "sum_j grad_feat == sum_i grad_out", rtol=1e-5, atol=1e-2)
+    # total score gradient agrees whichever side it is summed on: sum_i grad_attn_row == sum_j grad_attn_col
+    assert_close(gar.double().sum(0), gac.double().sum(0), "sum grad_attn_row == sum grad_attn_col", rtol=1e-4, atol=5e-2)
+    # slope == 1: a softmax is invariant to a per-row shift, so grad_attn_row vanishes
+    _, (gx1, gar1, gac1) = run(1.0, x)
+    assert float(gar1.abs().max()) < 5e-4
+    # grad_feat is linear in grad_out and does not depend on the features
+    _, (gx2, _, _) = run(0.2, x * 3.0)
+    assert torch.equal(gx2, gx)
+    # constant features: out is constant, grad of the scores vanishes (every edge gives the same dot product)
+    c = torch.randn(1, h, f, device=DEV).expand(n, h, f).contiguous()
+    _, (_, garc, gacc) = run(0.2, c)
+    assert float(garc.abs().max()) < 5e-4 and float(gacc.abs().max()) < 5e-2
+
+
+def test_c3_edgeconv_full_size_vs_oracle():
+    from ae_mlsys_gnn_amd.operators.fused_edgeconv import edgeconv_native
+    torch.manual_seed(0)
+    bsz, npts, k, f = 32, 1024, 20, 64
+    pts = torch.rand(bsz, npts, 3) * 2 - 1
+    src = graphs.knn_graph(pts.to(DEV), k).cpu()
+    theta = torch.randn(f, 3)
+    phi = torch.randn(f, 3)
+    x = pts.reshape(-1, 3)
+    h_src = x @ theta.t()
+    h_dst = x @ phi.t() - h_src
+    ref_out, ref_arg = c_oracle.edgeconv_forward(k, src.numpy(), h_src.numpy(), h_dst.numpy())
+    out, arg = edgeconv_native.edgeconv_forward(k, src.to(DEV), h_src.to(DEV), h_dst.to(DEV))
+    assert np.array_equal(arg.cpu().numpy(), ref_arg), "argmax differs at C3"
+    assert np.array_equal(out.cpu().numpy(), ref_out), "max values differ at C3"
+    go = torch.randn(bsz * npts, f)
+    gs = edgeconv_native.edgeconv_backward(go.to(DEV), arg, bsz * npts)
+    ref_gs = c_oracle.edgeconv_backward(ref_arg, go.numpy(), bsz * npts)
+    assert_close(gs, torch.from_numpy(ref_gs), "grad_src at C3", atol=1e-4)
+
+
+def test_c4_gmm_full_size_vs_oracle():
+    from ae_mlsys_gnn_amd.operators import csr2csc as csc_op
+    from ae_mlsys_gnn_amd.operators.fused_gmmconv import gmm_native
+    n, kk, dim, f = 169343, 3, 2, 64
+    g = graphs.rmat_graph(n, 2_300_000, seed=1, device=DEV)
+    g.col_ptr, g.row_ind, g.permute = csc_op.csr2csc(g.row_ptr, g.col_ind)
+    torch.manual_seed(2)
+    deg = (g.row_ptr[1:] - g.row_ptr[:-1]).float()
+    dst = torch.repeat_interleave(torch.arange(n, device=DEV), (g.row_ptr[1:] - g.row_ptr[:-1]).long())
+    pseudo = torch.stack([deg[g.col_ind.long()].rsqrt(), deg[dst].rsqrt()], 1).contiguous()
+    x = torch.randn(n, kk, f, device=DEV)
+    mu = torch.rand(kk, dim, device=DEV)
+    isg = torch.ones(kk, dim, device=DEV)
+    go = torch.randn(n, kk, f, device=DEV)
+    out = gmm_native.gmmconv(g.row_ptr, g.col_ind, x, pseudo, mu, isg)
+    gx, gp, gm, gs = gmm_native.gmmconv_backward(g.col_ptr, g.row_ind, g.permute, x, pseudo, mu, isg, go)
+    rp, ci = g.row_ptr.cpu().numpy(), g.col_ind.cpu().numpy()
+    args = [t.cpu().numpy() for t in (x, pseudo, mu, isg)]
+    ref = c_oracle.gmm_forward(rp, ci, *args)
+    rgx, rgp, rgm, rgs = c_oracle.gmm_backward(rp, ci, *args, go.cpu().numpy())
+    assert_close(out, torch.from_numpy(ref), "gmm out at C4", atol=1e-4)
+    assert_close(gx, torch.from_numpy(rgx), "gmm grad_feat at C4", atol=1e-4)
+    assert_close(gp, torch.from_numpy(rgp), "gmm grad_pseudo at C4", atol=1e-3)
+    # sums over 2.47 M edges of terms of either sign
+    assert_close(gm, torch.from_numpy(rgm), "gmm grad_mu at C4", rtol=1e-3, atol=1.0)
+    assert_close(gs, torch.from_numpy(rgs), "gmm grad_sigma at C4", rtol=1e-3, atol=1.0)

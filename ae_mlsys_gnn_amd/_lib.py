@@ -43,7 +43,8 @@ _SIGNATURES = {
     "fgnn_gmm_backward": (c_int, [c_int, c_int64, c_int, c_int, c_int] + [c_void_p] * 12
                           + [c_void_p, c_void_p, c_size_t, c_void_p]),
     "fgnn_gaussian": (c_int, [c_int64, c_int, c_int] + [c_void_p] * 4 + [c_void_p]),
-    "fgnn_gaussian_backward": (c_int, [c_int64, c_int, c_int] + [c_void_p] * 7 + [c_void_p]),
+    "fgnn_gaussian_backward_workspace_bytes": (c_size_t, [c_int64, c_int, c_int]),
+    "fgnn_gaussian_backward": (c_int, [c_int64, c_int, c_int] + [c_void_p] * 7 + [c_void_p, c_size_t, c_void_p]),
     "fgnn_mhspmm_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int]),
     "fgnn_mhspmm": (c_int, [c_int, c_int64, c_int, c_int] + [c_void_p] * 6 + [c_void_p, c_void_p, c_size_t, c_void_p]),
     "fgnn_mhsddmm": (c_int, [c_int, c_int64, c_int, c_int] + [c_void_p] * 5 + [c_void_p]),

@@ -252,18 +252,40 @@ __device__ __forceinline__ void fg_accum_chunk(const float *__restrict__ feat, i
     }
 }
 
-// Sum over groups of `lph` consecutive lanes (lph a power of two <= 64, groups aligned); every lane
+// Sum over groups of LPH consecutive lanes (LPH a power of two <= 64, groups aligned); every lane
 // of a group gets the group's sum.  Steps inside a row of 16 lanes are DPP, wider ones go through
 // the LDS crossbar.
-__device__ __forceinline__ float fg_group_sum_pow2(float v, int lph)
+template <int LPH>
+__device__ __forceinline__ float fg_group_sum(float v)
 {
-    if (lph >= 2) v += fg_dpp<0xB1>(v);
-    if (lph >= 4) v += fg_dpp<0x4E>(v);
-    if (lph >= 8) v += fg_dpp<0x141>(v);
-    if (lph >= 16) v += fg_dpp<0x140>(v);
-    if (lph >= 32) v += fg_bperm(v, fg_lane() ^ 16);
-    if (lph >= 64) v += fg_bperm(v, fg_lane() ^ 32);
+    if constexpr (LPH >= 2) v += fg_dpp<0xB1>(v);
+    if constexpr (LPH >= 4) v += fg_dpp<0x4E>(v);
+    if constexpr (LPH >= 8) v += fg_dpp<0x141>(v);
+    if constexpr (LPH >= 16) v += fg_dpp<0x140>(v);
+    if constexpr (LPH >= 32) v += fg_bperm(v, fg_lane() ^ 16);
+    if constexpr (LPH >= 64) v += fg_bperm(v, fg_lane() ^ 32);
     return v;
+}
+// Lanes per head for which the kernels have a DPP reduction; 0 selects the generic LDS path.
+static inline int fgnn_pick_lph(int vec, int F)
+{
+    int lph = F / vec;
+    if (vec == 4 && (lph == 1 || lph == 2 || lph == 4 || lph == 8 || lph == 16 || lph == 32)) return lph;
+    return 0;
+}
+// Calls f.template operator()<LPH>() for a value returned by fgnn_pick_lph.
+template <typename Fn>
+static inline int fgnn_dispatch_lph(int lph, Fn &&f)
+{
+    switch (lph) {
+    case 1: return f.template operator()<1>();
+    case 2: return f.template operator()<2>();
+    case 4: return f.template operator()<4>();
+    case 8: return f.template operator()<8>();
+    case 16: return f.template operator()<16>();
+    case 32: return f.template operator()<32>();
+    default: return f.template operator()<0>();
+    }
 }
 
 // Per-head sums of per-lane partial values: lane h (< H) returns the sum over the F/VEC

@@ -5,9 +5,9 @@
 
 // out[p,h] = <a[row,h,:], b[col_ind[p],h,:]> (src/sddmm/mhsddmm.cu:5-81 of the reference, which
 // finds the row of each edge by binary search; here the row is the work item).
-template <int VEC, int R, bool FULL>
+template <int VEC, int R, bool FULL, int LPH>
 __global__ __launch_bounds__(FGNN_TPB) void mhsddmm_kernel(int N, int H, int F, int HF, const int *ptr, const int *idx,
-                                                           const float *a, const float *b, float *out, int lph_pow2)
+                                                           const float *a, const float *b, float *out)
 {
     extern __shared__ float lds[];
     int row = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
@@ -39,10 +39,10 @@ __global__ __launch_bounds__(FGNN_TPB) void mhsddmm_kernel(int N, int H, int F, 
 #pragma unroll
                 for (int r = 0; r < R; ++r) d[r] = ld[u][r].dot(ar[r]);
                 size_t o = (size_t)(c + t + u) * H;
-                if (lph_pow2 > 0) {
+                if constexpr (LPH > 0) {
 #pragma unroll
                     for (int r = 0; r < R; ++r) {
-                        float s = fg_group_sum_pow2(d[r], lph_pow2);
+                        float s = fg_group_sum<LPH>(d[r]);
                         if ((FULL || lm.ok[r]) && lm.eoff[r] % F == 0) out[o + lm.hd[r]] = s;
                     }
                 } else {
@@ -64,14 +64,15 @@ extern "C" int fgnn_mhsddmm(int N, int64_t E, int H, int F, const int32_t *row_p
     const int HF = H * F;
     fgnn_rowcfg cfg;
     FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, fgnn_aligned16(a) && fgnn_aligned16(b), &cfg), FGNN_ERR_LIMIT, "fgnn_mhsddmm: unsupported row width %d", HF);
-    int lph = F / cfg.vec;
-    int lph_pow2 = (cfg.vec == 4 && (lph & (lph - 1)) == 0 && lph <= 64) ? lph : 0;
+    const int lph = fgnn_pick_lph(cfg.vec, F);
     const unsigned grid = (unsigned)((N + FGNN_WPB - 1) / FGNN_WPB);
     hipStream_t st = (hipStream_t)stream;
     return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
-        hipLaunchKernelGGL((mhsddmm_kernel<VEC, R, FULL>), dim3(grid), dim3(FGNN_TPB), (size_t)FGNN_WPB * 64 * R * sizeof(float), st,
-                           N, H, F, HF, row_ptr, col_ind, a, b, out, lph_pow2);
-        return fgnn_launch_status("mhsddmm_kernel");
+        return fgnn_dispatch_lph(VEC == 4 ? lph : 0, [&]<int LPH>() -> int {
+            hipLaunchKernelGGL((mhsddmm_kernel<VEC, R, FULL, (VEC == 4 ? LPH : 0)>), dim3(grid), dim3(FGNN_TPB),
+                               (size_t)FGNN_WPB * 64 * R * sizeof(float), st, N, H, F, HF, row_ptr, col_ind, a, b, out);
+            return fgnn_launch_status("mhsddmm_kernel");
+        });
     });
 }
 

@@ -185,30 +185,28 @@ struct GmmBwdP {
     const fgnn_item *items; int n_items;
     const int *ptr; const int *idx; const int *permute;
     const float *x; const float *g; const float *pseudo; const float *mu; const float *isg;
-    float *gfeat; float *gpseudo; float *part; float *red;   // red: [n_items, 2*K*dim] per-item sums
+    float *gfeat; float *gww; float *part;      // gww: [E,K] in CSR position order, gw * w per edge and kernel
     int N, K, dim, F, HF;
 };
 
 // One pass over CSC column j (x[j] stays in registers): per in-edge gather grad_out[i], accumulate
-// w * grad_out[i] into grad_feat[j], form the per-kernel dot products gw = <grad_out[i,k,:], x[j,k,:]>
-// and from them the Gaussian derivatives.  grad_pseudo is written once per edge at its CSR
-// position; the mu / inv_sigma derivatives are summed per work item and reduced afterwards.
-template <int VEC, int R, bool FULL>
-__global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p, int lph_pow2)
+// w * grad_out[i] into grad_feat[j] and form gw = <grad_out[i,k,:], x[j,k,:]> per mixture kernel
+// (DPP butterflies inside head groups).  gw*w is written once per edge at its CSR position; the
+// Gaussian derivatives are finished by gauss_grad_kernel below.
+template <int VEC, int R, bool FULL, int LPH>
+__global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p)
 {
     extern __shared__ float lds[];
     const int K = p.K, dim = p.dim, KD = K * dim;
-    const int per_wave = 2 * K * 64 + 64 * R;
+    const int per_wave = K * 64 + 64 * R;
     float *shared = lds + FGNN_WPB * per_wave;          // mu | inv_sigma
     for (int i = (int)threadIdx.x; i < KD; i += FGNN_TPB) { shared[i] = p.mu[i]; shared[KD + i] = p.isg[i]; }
     __syncthreads();
     int col, b, e, slot;
     if (!fg_get_item(p.items, p.n_items, p.ptr, col, b, e, slot)) return;
-    const int item = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
     const int lane = fg_lane();
     float *wl = lds + fg_wave() * per_wave;
-    float *gwl = wl + K * 64;
-    float *scr = gwl + K * 64;
+    float *scr = wl + K * 64;
     fg_lanemap<VEC, R> lm;
     lm.init(lane, p.HF, p.F);
     fg_vec<VEC> T[R], xr[R];
@@ -217,16 +215,14 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p, int lph_po
         T[r].zero();
         if (FULL || lm.ok[r]) xr[r].load(p.x + (size_t)col * p.HF + lm.eoff[r]); else xr[r].zero();
     }
-    float macc = 0.f, sacc = 0.f;    // lane kd keeps the sums for (k,d)
-
     for (int c = b; c < e; c += 64) {
         int q = c + lane;
         bool ok = q < e;
         int cnt = min(64, e - c);
         int qq = ok ? q : c;
         int id = p.idx[qq];
-        size_t pos = (size_t)p.permute[qq];
-        const float *ps = p.pseudo + pos * dim;
+        int posv = p.permute[qq];
+        const float *ps = p.pseudo + (size_t)(unsigned)posv * dim;
         for (int k = 0; k < K; ++k) {
             float acc = 0.f;
             for (int d = 0; d < dim; ++d) {
@@ -236,53 +232,38 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p, int lph_po
             wl[k * 64 + lane] = ok ? __expf(-0.5f * acc) : 0.f;
         }
         fg_wave_lds_sync();
-        // lanes-as-features: weighted sum and per-edge dot products
-        for (int t = 0; t < cnt; t += 2) {
-            fg_vec<VEC> ld[2][R];
+        constexpr int UG = (R >= 8) ? 1 : 8 / R;
+        for (int t = 0; t < cnt; t += UG) {
+            fg_vec<VEC> ld[UG][R];
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
+            for (int u = 0; u < UG; ++u) {
                 int rid = __builtin_amdgcn_readlane(id, t + u);
                 const float *base = p.g + (size_t)rid * p.HF;
 #pragma unroll
                 for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ld[u][r].load(base + lm.eoff[r]); else ld[u][r].zero(); }
             }
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                float dpart[R];
+            for (int u = 0; u < UG; ++u) {
+                if (t + u >= cnt) break;
+                float *gdst = p.gww + (size_t)(unsigned)__builtin_amdgcn_readlane(posv, t + u) * K;
+                float dpart[R], w[R];
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
-                    float w = wl[lm.hd[r] * 64 + t + u];
-                    T[r].fma(w, ld[u][r]);
+                    w[r] = wl[lm.hd[r] * 64 + t + u];
+                    T[r].fma(w[r], ld[u][r]);
                     dpart[r] = ld[u][r].dot(xr[r]);
                 }
-                if (lph_pow2 > 0) {
+                if constexpr (LPH > 0) {
 #pragma unroll
                     for (int r = 0; r < R; ++r) {
-                        float sum = fg_group_sum_pow2(dpart[r], lph_pow2);
-                        if ((FULL || lm.ok[r]) && lm.eoff[r] % p.F == 0) gwl[lm.hd[r] * 64 + t + u] = sum;
+                        float sum = fg_group_sum<LPH>(dpart[r]);
+                        if ((FULL || lm.ok[r]) && lm.eoff[r] % p.F == 0) gdst[lm.hd[r]] = sum * w[r];
                     }
                 } else {
                     float sum = fg_head_reduce<VEC, R>(scr, dpart, lm, lane, K, p.F);
-                    if (lane < K) gwl[lane * 64 + t + u] = sum;
+                    if (lane < K) gdst[lane] = sum * wl[lane * 64 + t + u];
                 }
             }
-        }
-        fg_wave_lds_sync();
-        // lanes-as-edges: Gaussian derivatives
-        for (int d = 0; d < dim; ++d) {
-            float gp = 0.f;
-            float psd = ps[d];
-            for (int k = 0; k < K; ++k) {
-                float gww = ok ? gwl[k * 64 + lane] * wl[k * 64 + lane] : 0.f;
-                float diff = psd - shared[k * dim + d];
-                float sg = shared[KD + k * dim + d];
-                float a = gww * diff * sg;          // gw*w*(p-mu)*isg
-                gp -= a * sg;
-                float sm = fg_wave_sum(a * sg);
-                float ss = fg_wave_sum(-a * diff);
-                if (lane == k * dim + d) { macc += sm; sacc += ss; }
-            }
-            if (ok) p.gpseudo[pos * dim + d] = gp;
         }
         fg_wave_lds_sync();
     }
@@ -290,10 +271,68 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p, int lph_po
 #pragma unroll
     for (int r = 0; r < R; ++r)
         if (FULL || lm.ok[r]) T[r].store(dst + lm.eoff[r]);
-    if (lane < KD) {
-        p.red[(size_t)item * 2 * KD + lane] = macc;
-        p.red[(size_t)item * 2 * KD + KD + lane] = sacc;
+}
+
+// Closed-form derivatives of w[p,k] = exp(-0.5 sum_d ((pseudo[p,d]-mu[k,d])*isg[k,d])^2), one edge per
+// thread.  src[p,k] is either dL/dw (premultiplied == 0: the weight is recomputed here) or dL/dw * w.
+//   d/dpseudo[p,d] = -sum_k gww*diff*isg^2,  d/dmu[k,d] = sum_p gww*diff*isg^2,  d/disg[k,d] = -sum_p gww*diff^2*isg
+// The mu / isg sums are reduced per workgroup in a fixed order into red[block, 2*K*dim].
+__global__ __launch_bounds__(256) void gauss_grad_kernel(int64_t E, int K, int dim, const float *__restrict__ pseudo,
+                                                         const float *__restrict__ mu, const float *__restrict__ isg,
+                                                         const float *__restrict__ src, int premultiplied,
+                                                         float *__restrict__ gp, float *__restrict__ red)
+{
+    extern __shared__ float lds[];
+    const int KD = K * dim;
+    float *shared = lds;                 // mu | isg
+    float *wsum = lds + 2 * KD;          // [4 waves][2*KD]
+    for (int i = (int)threadIdx.x; i < KD; i += 256) { shared[i] = mu[i]; shared[KD + i] = isg[i]; }
+    __syncthreads();
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const bool ok = e < E;
+    const int64_t ee = ok ? e : 0;
+    const int lane = fg_lane(), wave = fg_wave();
+    for (int k = 0; k < K; ++k) {
+        float gww = ok ? src[ee * K + k] : 0.f;
+        if (!premultiplied) {
+            float acc = 0.f;
+            for (int d = 0; d < dim; ++d) {
+                float t = (pseudo[ee * dim + d] - shared[k * dim + d]) * shared[KD + k * dim + d];
+                acc = fmaf(t, t, acc);
+            }
+            gww *= __expf(-0.5f * acc);
+        }
+        for (int d = 0; d < dim; ++d) {
+            float diff = pseudo[ee * dim + d] - shared[k * dim + d];
+            float sg = shared[KD + k * dim + d];
+            float a = gww * diff * sg;
+            float sm = fg_wave_sum(a * sg);
+            float ss = fg_wave_sum(-a * diff);
+            if (lane == 0) { wsum[wave * 2 * KD + k * dim + d] = sm; wsum[wave * 2 * KD + KD + k * dim + d] = ss; }
+        }
     }
+    if (ok) {
+        for (int d = 0; d < dim; ++d) {
+            float acc = 0.f, psd = pseudo[ee * dim + d];
+            for (int k = 0; k < K; ++k) {
+                float gww = src[ee * K + k];
+                if (!premultiplied) {
+                    float a2 = 0.f;
+                    for (int dd = 0; dd < dim; ++dd) {
+                        float t = (pseudo[ee * dim + dd] - shared[k * dim + dd]) * shared[KD + k * dim + dd];
+                        a2 = fmaf(t, t, a2);
+                    }
+                    gww *= __expf(-0.5f * a2);
+                }
+                float sg = shared[KD + k * dim + d];
+                acc = fmaf(-gww * (psd - shared[k * dim + d]), sg * sg, acc);
+            }
+            gp[e * dim + d] = acc;
+        }
+    }
+    __syncthreads();
+    for (int i = (int)threadIdx.x; i < 2 * KD; i += 256)
+        red[(size_t)blockIdx.x * 2 * KD + i] = (wsum[i] + wsum[2 * KD + i]) + (wsum[4 * KD + i] + wsum[6 * KD + i]);
 }
 
 // Column sums of red[rows, width] in two deterministic levels.
@@ -317,23 +356,50 @@ __global__ __launch_bounds__(256) void colsum_level1(const float *red, int rows,
 }
 __global__ __launch_bounds__(64) void colsum_level2(const float *tmp, int nblk, int KD, float *gmu, float *gsig)
 {
-    int c = (int)threadIdx.x;
-    if (c >= 2 * KD) return;
-    float acc = 0.f;
-    for (int b = 0; b < nblk; ++b) acc += tmp[(size_t)b * 2 * KD + c];
-    if (c < KD) gmu[c] = acc; else gsig[c - KD] = acc;
+    for (int c = (int)threadIdx.x; c < 2 * KD; c += 64) {
+        float acc = 0.f;
+        for (int b = 0; b < nblk; ++b) acc += tmp[(size_t)b * 2 * KD + c];
+        if (c < KD) gmu[c] = acc; else gsig[c - KD] = acc;
+    }
 }
 
-static const int kColsumBlocks = 128;
+static const int kColsumBlocks = 64;
+
+// gauss_grad_kernel + column sums on `st`; ws must hold gauss_grad_workspace(E, K, dim) bytes.
+static size_t gauss_grad_workspace(int64_t E, int K, int dim)
+{
+    size_t nblk = (size_t)((E + 255) / 256);
+    return fgnn_align256(nblk * 2 * K * dim * sizeof(float)) + fgnn_align256((size_t)kColsumBlocks * 2 * K * dim * sizeof(float));
+}
+static int gauss_grad_launch(int64_t E, int K, int dim, const float *pseudo, const float *mu, const float *isg, const float *src,
+                             int premultiplied, float *gp, float *gmu, float *gsig, void *ws, hipStream_t st)
+{
+    const int KD = K * dim;
+    if (E == 0) {
+        int rc = fgnn_fill_f32(gmu, KD, 0.f, st);
+        return rc ? rc : fgnn_fill_f32(gsig, KD, 0.f, st);
+    }
+    const int nblk = (int)((E + 255) / 256);
+    float *red = (float *)ws;
+    float *tmp = (float *)((char *)ws + fgnn_align256((size_t)nblk * 2 * KD * sizeof(float)));
+    size_t shm = (size_t)(2 * KD + 4 * 2 * KD) * sizeof(float);
+    hipLaunchKernelGGL(gauss_grad_kernel, dim3(nblk), dim3(256), shm, st, E, K, dim, pseudo, mu, isg, src, premultiplied, gp, red);
+    int rc = fgnn_launch_status("gauss_grad_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(colsum_level1, dim3(kColsumBlocks), dim3(256), 0, st, red, nblk, 2 * KD, tmp);
+    rc = fgnn_launch_status("colsum_level1");
+    if (rc) return rc;
+    hipLaunchKernelGGL(colsum_level2, dim3(1), dim3(64), 0, st, tmp, kColsumBlocks, KD, gmu, gsig);
+    return fgnn_launch_status("colsum_level2");
+}
 
 extern "C" size_t fgnn_gmm_backward_workspace_bytes(const fgnn_schedule_t *sched_csc, int K, int dim, int F)
 {
-    // partials | per-item sums | level-1 sums.  Without a schedule the caller passes N items: the
-    // item count is not known here, so the size is computed by fgnn_gmm_backward_workspace_items.
-    size_t items = sched_csc ? (size_t)sched_csc->n_items : 0;
-    size_t b = sched_csc ? fgnn_align256((size_t)sched_csc->n_partials * spmm_pw(K * F) * sizeof(float)) : 0;
-    b += fgnn_align256(items * 2 * K * dim * sizeof(float));
-    b += fgnn_align256((size_t)kColsumBlocks * 2 * K * dim * sizeof(float));
+    // partials | gw*w [E,K] | reduction scratch
+    if (!sched_csc) return 0;
+    size_t b = fgnn_align256((size_t)sched_csc->n_partials * spmm_pw(K * F) * sizeof(float));
+    b += fgnn_align256((size_t)sched_csc->n_edges * K * sizeof(float));
+    b += gauss_grad_workspace(sched_csc->n_edges, K, dim);
     return b;
 }
 
@@ -345,7 +411,7 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
 {
     int rc = spmm_checks("fgnn_gmm_backward", N, E, K, F, sched_csc, col_ptr);
     if (rc) return rc;
-    FGNN_REQUIRE(dim >= 1 && K * dim <= 32, FGNN_ERR_LIMIT, "fgnn_gmm_backward: K*dim=%d > 32 unsupported", K * dim);
+    FGNN_REQUIRE(dim >= 1 && dim <= 64 && K * dim <= 1024, FGNN_ERR_LIMIT, "fgnn_gmm_backward: dim=%d K*dim=%d unsupported", dim, K * dim);
     FGNN_REQUIRE(col_ptr && (row_ind || E == 0) && (permute || E == 0) && node_feat && (pseudo || E == 0) && mu && inv_sigma &&
                      grad_out && grad_feat && (grad_pseudo || E == 0) && grad_mu && grad_sigma,
                  FGNN_ERR_NULL, "fgnn_gmm_backward: NULL argument");
@@ -357,42 +423,37 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
     const int HF = K * F, KD = K * dim;
     char *w = (char *)workspace;
     float *part = (float *)w; w += fgnn_align256((size_t)sched_csc->n_partials * spmm_pw(HF) * sizeof(float));
-    float *red = (float *)w; w += fgnn_align256((size_t)sched_csc->n_items * 2 * KD * sizeof(float));
-    float *tmp = (float *)w;
-    if (sched_csc->n_items == 0) {
-        rc = fgnn_fill_f32(grad_mu, KD, 0.f, st);
-        return rc ? rc : fgnn_fill_f32(grad_sigma, KD, 0.f, st);
+    float *gww = (float *)w; w += fgnn_align256((size_t)E * K * sizeof(float));
+    void *gws = w;
+    if (sched_csc->n_items > 0) {
+        bool aligned = fgnn_aligned16(node_feat) && fgnn_aligned16(grad_out) && fgnn_aligned16(grad_feat);
+        fgnn_rowcfg cfg;
+        FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, aligned, &cfg), FGNN_ERR_LIMIT, "fgnn_gmm_backward: unsupported row width %d", HF);
+        GmmBwdP p{};
+        p.items = sched_csc->items_dev; p.n_items = sched_csc->n_items; p.ptr = col_ptr; p.idx = row_ind; p.permute = permute;
+        p.x = node_feat; p.g = grad_out; p.pseudo = pseudo; p.mu = mu; p.isg = inv_sigma; p.gfeat = grad_feat; p.gww = gww;
+        p.part = part; p.N = N; p.K = K; p.dim = dim; p.F = F; p.HF = HF;
+        const int lph = fgnn_pick_lph(cfg.vec, F);
+        const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
+        rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
+            size_t shm = ((size_t)FGNN_WPB * (K * 64 + 64 * R) + 2 * KD) * sizeof(float);
+            int rc2 = fgnn_dispatch_lph(VEC == 4 ? lph : 0, [&]<int LPH>() -> int {
+                hipLaunchKernelGGL((gmm_bwd_kernel<VEC, R, FULL, (VEC == 4 ? LPH : 0)>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                return fgnn_launch_status("gmm_bwd_kernel");
+            });
+            if (rc2) return rc2;
+            if (sched_csc->n_split > 0) {
+                SpmmP mp{};
+                mp.part = part; mp.out = grad_feat; mp.N = N; mp.H = K; mp.F = F; mp.HF = HF;
+                unsigned g2 = (unsigned)((sched_csc->n_split + FGNN_WPB - 1) / FGNN_WPB);
+                hipLaunchKernelGGL((spmm_merge_kernel<VEC, R>), dim3(g2), dim3(FGNN_TPB), 0, st, mp, sched_csc->split_dev, sched_csc->n_split);
+                return fgnn_launch_status("spmm_merge_kernel");
+            }
+            return 0;
+        });
+        if (rc) return rc;
     }
-    bool aligned = fgnn_aligned16(node_feat) && fgnn_aligned16(grad_out) && fgnn_aligned16(grad_feat);
-    fgnn_rowcfg cfg;
-    FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, aligned, &cfg), FGNN_ERR_LIMIT, "fgnn_gmm_backward: unsupported row width %d", HF);
-    GmmBwdP p{};
-    p.items = sched_csc->items_dev; p.n_items = sched_csc->n_items; p.ptr = col_ptr; p.idx = row_ind; p.permute = permute;
-    p.x = node_feat; p.g = grad_out; p.pseudo = pseudo; p.mu = mu; p.isg = inv_sigma; p.gfeat = grad_feat; p.gpseudo = grad_pseudo;
-    p.part = part; p.red = red; p.N = N; p.K = K; p.dim = dim; p.F = F; p.HF = HF;
-    int lph = F / cfg.vec;
-    int lph_pow2 = (cfg.vec == 4 && (lph & (lph - 1)) == 0 && lph <= 64) ? lph : 0;
-    const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
-    rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
-        size_t shm = ((size_t)FGNN_WPB * (2 * K * 64 + 64 * R) + 2 * KD) * sizeof(float);
-        hipLaunchKernelGGL((gmm_bwd_kernel<VEC, R, FULL>), dim3(grid), dim3(FGNN_TPB), shm, st, p, lph_pow2);
-        int rc2 = fgnn_launch_status("gmm_bwd_kernel");
-        if (rc2) return rc2;
-        if (sched_csc->n_split > 0) {
-            SpmmP mp{};
-            mp.part = part; mp.out = grad_feat; mp.N = N; mp.H = K; mp.F = F; mp.HF = HF;
-            unsigned g2 = (unsigned)((sched_csc->n_split + FGNN_WPB - 1) / FGNN_WPB);
-            hipLaunchKernelGGL((spmm_merge_kernel<VEC, R>), dim3(g2), dim3(FGNN_TPB), 0, st, mp, sched_csc->split_dev, sched_csc->n_split);
-            return fgnn_launch_status("spmm_merge_kernel");
-        }
-        return 0;
-    });
-    if (rc) return rc;
-    hipLaunchKernelGGL(colsum_level1, dim3(kColsumBlocks), dim3(256), 0, st, red, p.n_items, 2 * KD, tmp);
-    rc = fgnn_launch_status("colsum_level1");
-    if (rc) return rc;
-    hipLaunchKernelGGL(colsum_level2, dim3(1), dim3(64), 0, st, tmp, kColsumBlocks, KD, grad_mu, grad_sigma);
-    return fgnn_launch_status("colsum_level2");
+    return gauss_grad_launch(E, K, dim, pseudo, mu, inv_sigma, gww, 1, grad_pseudo, grad_mu, grad_sigma, gws, st);
 }
 
 // ------------------------------------------------------------------------------- standalone Gaussian
@@ -411,35 +472,6 @@ __global__ __launch_bounds__(256) void gaussian_kernel(int64_t E, int K, int dim
     out[tid] = __expf(-0.5f * acc);
 }
 
-// Closed-form derivatives of w = exp(-0.5 sum_d ((p-mu)*isg)^2) given dL/dw.  One edge per thread;
-// the mu / inv_sigma sums are reduced per wave and added with one float atomic per wave and (k,d).
-__global__ __launch_bounds__(256) void gaussian_bwd_kernel(int64_t E, int K, int dim, const float *pseudo, const float *mu,
-                                                           const float *isg, const float *gw, float *gp, float *gmu, float *gsig)
-{
-    int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    bool ok = e < E;
-    int64_t ee = ok ? e : 0;
-    for (int d = 0; d < dim; ++d) {
-        float acc_p = 0.f;
-        for (int k = 0; k < K; ++k) {
-            float acc = 0.f;
-            for (int dd = 0; dd < dim; ++dd) {
-                float t = (pseudo[ee * dim + dd] - mu[k * dim + dd]) * isg[k * dim + dd];
-                acc = fmaf(t, t, acc);
-            }
-            float w = __expf(-0.5f * acc);
-            float diff = pseudo[ee * dim + d] - mu[k * dim + d];
-            float sg = isg[k * dim + d];
-            float a = ok ? gw[ee * K + k] * w * diff * sg : 0.f;
-            acc_p -= a * sg;
-            float sm = fg_wave_sum(a * sg);
-            float ss = fg_wave_sum(-a * diff);
-            if (fg_lane() == 0) { atomicAdd(gmu + k * dim + d, sm); atomicAdd(gsig + k * dim + d, ss); }
-        }
-        if (ok) gp[e * dim + d] = acc_p;
-    }
-}
-
 extern "C" int fgnn_gaussian(int64_t E, int K, int dim, const float *pseudo, const float *mu, const float *inv_sigma,
                              float *out, void *stream)
 {
@@ -451,18 +483,17 @@ extern "C" int fgnn_gaussian(int64_t E, int K, int dim, const float *pseudo, con
     return fgnn_launch_status("gaussian_kernel");
 }
 
+extern "C" size_t fgnn_gaussian_backward_workspace_bytes(int64_t E, int K, int dim) { return gauss_grad_workspace(E, K, dim); }
+
 extern "C" int fgnn_gaussian_backward(int64_t E, int K, int dim, const float *pseudo, const float *mu, const float *inv_sigma,
-                                      const float *grad_w, float *grad_pseudo, float *grad_mu, float *grad_sigma, void *stream)
+                                      const float *grad_w, float *grad_pseudo, float *grad_mu, float *grad_sigma,
+                                      void *workspace, size_t workspace_bytes, void *stream)
 {
-    FGNN_REQUIRE(E >= 0 && K >= 1 && dim >= 1, FGNN_ERR_SHAPE, "fgnn_gaussian_backward: bad sizes");
+    FGNN_REQUIRE(E >= 0 && K >= 1 && dim >= 1 && K * dim <= 1024, FGNN_ERR_SHAPE, "fgnn_gaussian_backward: bad sizes");
     FGNN_REQUIRE((pseudo || E == 0) && mu && inv_sigma && (grad_w || E == 0) && (grad_pseudo || E == 0) && grad_mu && grad_sigma,
                  FGNN_ERR_NULL, "fgnn_gaussian_backward: NULL argument");
-    hipStream_t st = (hipStream_t)stream;
-    int rc = fgnn_fill_f32(grad_mu, (size_t)K * dim, 0.f, st);
-    if (rc) return rc;
-    rc = fgnn_fill_f32(grad_sigma, (size_t)K * dim, 0.f, st);
-    if (rc || E == 0) return rc;
-    hipLaunchKernelGGL(gaussian_bwd_kernel, dim3((unsigned)((E + 255) / 256)), dim3(256), 0, st, E, K, dim, pseudo, mu, inv_sigma,
-                       grad_w, grad_pseudo, grad_mu, grad_sigma);
-    return fgnn_launch_status("gaussian_bwd_kernel");
+    size_t need = gauss_grad_workspace(E, K, dim);
+    FGNN_REQUIRE(E == 0 || (workspace && workspace_bytes >= need), FGNN_ERR_WORKSPACE, "fgnn_gaussian_backward: workspace %zu < %zu bytes",
+                 workspace_bytes, need);
+    return gauss_grad_launch(E, K, dim, pseudo, mu, inv_sigma, grad_w, 0, grad_pseudo, grad_mu, grad_sigma, workspace, (hipStream_t)stream);
 }

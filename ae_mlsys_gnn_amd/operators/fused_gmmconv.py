@@ -77,8 +77,9 @@ class gmm_native:
         gm = torch.empty_like(mu)
         gs = torch.empty_like(sigma)
         with torch.cuda.device(pseudo.device):
+            ws, wsb = workspace(lib().fgnn_gaussian_backward_workspace_bytes(e, k, dim), pseudo.device)
             check(lib().fgnn_gaussian_backward(e, k, dim, ptr(pseudo), ptr(mu), ptr(sigma), ptr(grad_out), ptr(gp), ptr(gm),
-                                               ptr(gs), stream_ptr()), "fgnn_gaussian_backward")
+                                               ptr(gs), ptr(ws), wsb, stream_ptr()), "fgnn_gaussian_backward")
         return gp, gm, gs
 
 

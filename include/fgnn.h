@@ -125,8 +125,9 @@ int    fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F,
 /* Replaces the backward sequence of operators/fused_gmmconv.py:51-58 (mhsddmm + mhtranspose +
  * gmmconv over CSC + GaussianBp, gmmconv.cu:265-285) with one pass over the CSC arrays:
  * grad_feat [N,K,F], grad_pseudo [E,dim] (CSR order), grad_mu, grad_sigma [K,dim].
- * grad_mu / grad_sigma are summed per work item and reduced in two fixed-order levels
- * (bit-reproducible).  A schedule of col_ptr is required; K*dim <= 32. */
+ * The pass writes gw*w per edge into the workspace; a second edge-parallel kernel finishes the
+ * Gaussian derivatives, grad_mu / grad_sigma reduced in a fixed order (bit-reproducible).
+ * A schedule of col_ptr is required. */
 size_t fgnn_gmm_backward_workspace_bytes(const fgnn_schedule_t *sched_csc, int K, int dim, int F);
 int    fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F,
                          const int32_t *col_ptr, const int32_t *row_ind, const int32_t *permute,
@@ -137,12 +138,15 @@ int    fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F,
                          void *stream);
 
 /* gmmconv.Gaussian / gmmconv.GaussianBp (gmmconv.cc:36-41,80-86; gmmconv.cu:187-199,265-285).
- * The backward implements the closed-form derivatives of the Gaussian weight. */
-int fgnn_gaussian(int64_t E, int K, int dim, const float *pseudo, const float *mu,
-                  const float *inv_sigma, float *out, void *stream);
-int fgnn_gaussian_backward(int64_t E, int K, int dim, const float *pseudo, const float *mu,
-                           const float *inv_sigma, const float *grad_w,
-                           float *grad_pseudo, float *grad_mu, float *grad_sigma, void *stream);
+ * The backward implements the closed-form derivatives of the Gaussian weight; grad_mu and
+ * grad_sigma are reduced in a fixed order (bit-reproducible). */
+int    fgnn_gaussian(int64_t E, int K, int dim, const float *pseudo, const float *mu,
+                     const float *inv_sigma, float *out, void *stream);
+size_t fgnn_gaussian_backward_workspace_bytes(int64_t E, int K, int dim);
+int    fgnn_gaussian_backward(int64_t E, int K, int dim, const float *pseudo, const float *mu,
+                              const float *inv_sigma, const float *grad_w,
+                              float *grad_pseudo, float *grad_mu, float *grad_sigma,
+                              void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---------------------------------------------------------------- small operators
  * mhspmm.mhspmm (src/spmm/mhspmm.cc; mhspmm.cu:44-66): out[i,h,:] = sum_p att[p,h]*feat[idx[p],h,:];

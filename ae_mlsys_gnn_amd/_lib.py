@@ -24,6 +24,7 @@ _SIGNATURES = {
     "fgnn_version": (c_int, []),
     "fgnn_last_error": (ctypes.c_char_p, []),
     "fgnn_schedule_create": (c_int, [c_void_p, c_int, c_int, c_void_p, ctypes.POINTER(c_void_p)]),
+    "fgnn_schedule_create_bucketed": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, ctypes.POINTER(c_void_p)]),
     "fgnn_schedule_destroy": (None, [c_void_p]),
     "fgnn_schedule_num_items": (c_int, [c_void_p]),
     "fgnn_schedule_num_partials": (c_int, [c_void_p]),
@@ -116,16 +117,23 @@ def as_i32(t):
 
 
 class Schedule:
-    """Degree-binned work list of one pointer array (row_ptr or col_ptr)."""
+    """Degree-binned work list of one pointer array (row_ptr or col_ptr).  With `idx_tensor` it is
+    the XCD-aware form: long rows are cut by source bucket and each XCD gets one bucket."""
 
-    def __init__(self, ptr_tensor, seg_len=0):
+    def __init__(self, ptr_tensor, seg_len=0, idx_tensor=None, min_deg=0):
         require_cuda(ptr_tensor)
         self.ptr_tensor = as_i32(ptr_tensor)      # keeps the device memory alive
+        self.idx_tensor = None if idx_tensor is None else as_i32(idx_tensor)
         self.n_rows = self.ptr_tensor.numel() - 1
         handle = c_void_p()
         with torch.cuda.device(self.ptr_tensor.device):
-            check(lib().fgnn_schedule_create(ptr(self.ptr_tensor), self.n_rows, int(seg_len), stream_ptr(),
-                                             ctypes.byref(handle)), "fgnn_schedule_create")
+            if self.idx_tensor is None:
+                check(lib().fgnn_schedule_create(ptr(self.ptr_tensor), self.n_rows, int(seg_len), stream_ptr(),
+                                                 ctypes.byref(handle)), "fgnn_schedule_create")
+            else:
+                check(lib().fgnn_schedule_create_bucketed(ptr(self.ptr_tensor), ptr(self.idx_tensor), self.n_rows, int(seg_len),
+                                                          int(min_deg), stream_ptr(), ctypes.byref(handle)),
+                      "fgnn_schedule_create_bucketed")
         self.handle = handle
         self.n_items = lib().fgnn_schedule_num_items(handle)
         self.n_partials = lib().fgnn_schedule_num_partials(handle)
@@ -146,15 +154,29 @@ def default_seg_len() -> int:
     return int(os.environ.get("FGNN_SEG_LEN", "0"))
 
 
-def schedule_for(ptr_tensor, seg_len=None) -> Schedule:
-    """Cached schedule of a pointer array.  The cache entry holds the tensor, so its device
-    address cannot be reused while the entry lives; in-place edits bump `_version`."""
+def xcd_buckets_enabled(n_rows: int, n_edges: int) -> bool:
+    """XCD-aware schedules pay off when rows are long enough to be cut in eight: on by default for
+    graphs with an average degree of at least 64 (FGNN_XCD_BUCKETS=0/1 overrides)."""
+    env = os.environ.get("FGNN_XCD_BUCKETS")
+    if env is not None:
+        return env not in ("0", "")
+    return n_rows > 0 and n_edges >= 64 * n_rows
+
+
+def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None) -> Schedule:
+    """Cached schedule of a pointer array.  The cache entry holds the tensors, so their device
+    addresses cannot be reused while the entry lives; in-place edits bump `_version`.
+    idx_tensor: the index array, for operators that may use an XCD-aware schedule."""
     if seg_len is None:
         seg_len = default_seg_len()
-    key = (ptr_tensor.data_ptr(), ptr_tensor.numel(), ptr_tensor.device.index, ptr_tensor._version, int(seg_len))
+    if idx_tensor is not None and not xcd_buckets_enabled(ptr_tensor.numel() - 1, idx_tensor.numel()):
+        idx_tensor = None
+    min_deg = int(os.environ.get("FGNN_BUCKET_MIN_DEG", "0"))
+    key = (ptr_tensor.data_ptr(), ptr_tensor.numel(), ptr_tensor.device.index, ptr_tensor._version, int(seg_len),
+           None if idx_tensor is None else (idx_tensor.data_ptr(), idx_tensor._version, min_deg))
     s = _sched_cache.get(key)
     if s is None:
-        s = Schedule(ptr_tensor, seg_len)
+        s = Schedule(ptr_tensor, seg_len, idx_tensor, min_deg)
         _sched_cache[key] = s
         while len(_sched_cache) > _SCHED_CACHE_MAX:
             _sched_cache.popitem(last=False)

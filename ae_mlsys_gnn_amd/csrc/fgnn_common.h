@@ -61,7 +61,16 @@ struct fgnn_schedule {
     fgnn_split *split_dev;
     const int32_t *ptr_dev;
     int device;
+    // XCD-aware schedules only: the index array with every row's entries grouped by source bucket
+    // (a per-row permutation of the caller's index array), else NULL
+    int n_buckets;
+    const int32_t *idx_src_dev;
+    int32_t *bidx_dev;
 };
+
+#define FGNN_NUM_XCD 8      // workgroup w of a dispatch runs on XCD w % 8 (gfx942 / gfx950, SPX mode)
+// Source bucket of a node id: the top 3 bits of a multiplicative hash, so hot ids spread evenly.
+static __host__ __device__ inline int fgnn_bucket_of(int id) { return (int)(((uint32_t)id * 2654435761u) >> 29); }
 
 // Feature-row layout of the gather kernels: a row of `HF` floats is spread over the 64 lanes
 // of a wave in R slabs of 64*VEC floats; VEC = 4 uses 128-bit loads.
@@ -192,6 +201,7 @@ __device__ __forceinline__ bool fg_get_item(const fgnn_item *items, int n_items,
     if (items) {
         fgnn_item it = items[item];
         row = fg_uni(it.row); b = fg_uni(it.begin); e = fg_uni(it.end); slot = fg_uni(it.slot);
+        if (row < 0) return false;         // padding item of an XCD-aware schedule
     } else {
         row = item; b = fg_uni(ptr[item]); e = fg_uni(ptr[item + 1]); slot = -1;
     }

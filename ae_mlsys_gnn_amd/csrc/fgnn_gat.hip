@@ -426,14 +426,21 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_merge_kernel(GatBwdP p, cons
 
 // ------------------------------------------------------------------------------- host
 
-static int check_sched(const fgnn_schedule_t *s, const int32_t *ptr, int n, int64_t E, const char *what)
+// idx: the index array the operator was given; positional: the call reads or writes per-edge arrays
+// in the caller's position order, which a bucket-ordered schedule cannot serve
+static int check_sched(const fgnn_schedule_t *s, const int32_t *ptr, const int32_t *idx, bool positional, int n, int64_t E, const char *what)
 {
     if (!s) return 0;
     FGNN_REQUIRE(s->ptr_dev == ptr && s->n_rows == n && s->n_edges == E, FGNN_ERR_SCHEDULE,
                  "%s: schedule was built for another pointer array (n_rows %d vs %d, edges %lld vs %lld)", what,
                  s->n_rows, n, (long long)s->n_edges, (long long)E);
+    if (s->n_buckets > 0) {
+        FGNN_REQUIRE(s->idx_src_dev == idx, FGNN_ERR_SCHEDULE, "%s: XCD-aware schedule was built from another index array", what);
+        FGNN_REQUIRE(!positional, FGNN_ERR_SCHEDULE, "%s: an XCD-aware schedule cannot be used with per-edge (stashed) arrays", what);
+    }
     return 0;
 }
+static inline const int32_t *sched_idx(const fgnn_schedule_t *s, const int32_t *idx) { return (s && s->n_buckets > 0) ? s->bidx_dev : idx; }
 
 static int gat_common_checks(const char *fn, int N, int64_t E, int H, int F)
 {
@@ -464,7 +471,7 @@ static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_
     GatFwdP p;
     p.items = sched ? sched->items_dev : nullptr;
     p.n_items = sched ? sched->n_items : N;
-    p.ptr = row_ptr; p.idx = col_ind; p.ar = attn_row; p.ac = attn_col; p.x = in_feat;
+    p.ptr = row_ptr; p.idx = sched_idx(sched, col_ind); p.ar = attn_row; p.ac = attn_col; p.x = in_feat;
     p.out = out; p.emax = edge_max; p.esum = edge_sum; p.out2 = aux_out2; p.cc = aux_c;
     p.part = (float *)workspace; p.N = N; p.H = H; p.F = F; p.HF = HF; p.slope = slope;
     if (sched && sched->n_partials > 0) {
@@ -507,7 +514,7 @@ extern "C" int fgnn_gat_forward(int N, int64_t E, int H, int F, const float *att
                  FGNN_ERR_NULL, "fgnn_gat_forward: NULL argument");
     FGNN_REQUIRE((aux_out2 == nullptr) == (aux_c == nullptr), FGNN_ERR_NULL, "fgnn_gat_forward: aux_out2 and aux_c go together");
     FGNN_REQUIRE((e_lrelu == nullptr) == (e_softmax == nullptr), FGNN_ERR_NULL, "fgnn_gat_forward: e_lrelu and e_softmax go together");
-    rc = check_sched(sched, row_ptr, N, E, "fgnn_gat_forward");
+    rc = check_sched(sched, row_ptr, col_ind, e_lrelu != nullptr, N, E, "fgnn_gat_forward");
     if (rc) return rc;
     return gat_forward_launch(N, E, H, F, attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, out, edge_max,
                               edge_sum, aux_out2, aux_c, e_lrelu, e_softmax, sched, workspace, workspace_bytes, (hipStream_t)stream);
@@ -546,9 +553,9 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
     FGNN_REQUIRE(!stash || (permute && e_lrelu), FGNN_ERR_NULL, "fgnn_gat_backward: stashed attention needs permute, e_lrelu and e_softmax");
     const bool recompute = !(out_feat && aux_out2 && aux_c);
     FGNN_REQUIRE(!recompute || (row_ptr && (col_ind || E == 0)), FGNN_ERR_NULL, "fgnn_gat_backward: recomputing the forward needs row_ptr/col_ind");
-    rc = check_sched(sched_csc, col_ptr, N, E, "fgnn_gat_backward(csc)");
+    rc = check_sched(sched_csc, col_ptr, row_ind, stash, N, E, "fgnn_gat_backward(csc)");
     if (rc) return rc;
-    if (recompute) { rc = check_sched(sched_csr, row_ptr, N, E, "fgnn_gat_backward(csr)"); if (rc) return rc; }
+    if (recompute) { rc = check_sched(sched_csr, row_ptr, col_ind, false, N, E, "fgnn_gat_backward(csr)"); if (rc) return rc; }
     size_t need = fgnn_gat_backward_workspace_bytes(N, H, F, sched_csc, recompute ? sched_csr : nullptr, recompute);
     FGNN_REQUIRE(workspace && workspace_bytes >= need, FGNN_ERR_WORKSPACE, "fgnn_gat_backward: workspace %zu < %zu bytes", workspace_bytes, need);
     FGNN_REQUIRE(fgnn_aligned16(workspace), FGNN_ERR_ALIGN, "fgnn_gat_backward: workspace not 16-byte aligned");
@@ -577,7 +584,7 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
     GatBwdP p;
     p.items = sched_csc ? sched_csc->items_dev : nullptr;
     p.n_items = sched_csc ? sched_csc->n_items : N;
-    p.ptr = col_ptr; p.idx = row_ind; p.permute = permute; p.rec = rec; p.ac = attn_col; p.x = in_feat; p.g = grad_out;
+    p.ptr = col_ptr; p.idx = sched_idx(sched_csc, row_ind); p.permute = permute; p.rec = rec; p.ac = attn_col; p.x = in_feat; p.g = grad_out;
     p.esm = e_softmax; p.erelu = e_lrelu; p.gfeat = grad_feat; p.gac = grad_attn_col; p.part = part;
     p.N = N; p.H = H; p.F = F; p.HF = HF; p.slope = negative_slope;
 

@@ -1,4 +1,4 @@
-// Error reporting, version and row schedules of libfgnn_hip.so (host code only).
+// Error reporting, version and row schedules of libfgnn_hip.so.
 #include <algorithm>
 #include <cstdarg>
 #include <cstring>
@@ -18,57 +18,66 @@ void fgnn_set_error(const char *fmt, ...)
 extern "C" const char *fgnn_last_error(void) { return g_err; }
 extern "C" int fgnn_version(void) { return 100; }
 
-extern "C" int fgnn_schedule_create(const int32_t *ptr_dev, int n_rows, int seg_len, void *stream, fgnn_schedule_t **out)
+// Per row: stable partition of the row's index entries by source bucket.  One wave per row; pass 1
+// counts the buckets (ballots), pass 2 places every entry at its bucket's running offset.  Writes
+// the permuted index array and the per-(row, bucket) counts.
+__global__ __launch_bounds__(FGNN_TPB) void bucket_partition_kernel(int n_rows, const int *__restrict__ ptr, const int *__restrict__ idx,
+                                                                    int *__restrict__ bidx, int *__restrict__ bcnt)
 {
-    FGNN_REQUIRE(ptr_dev && out, FGNN_ERR_NULL, "fgnn_schedule_create: NULL argument");
-    FGNN_REQUIRE(n_rows >= 0, FGNN_ERR_SHAPE, "fgnn_schedule_create: n_rows=%d", n_rows);
-    if (seg_len <= 0) seg_len = 2048;
-    seg_len = (seg_len + 63) & ~63;
-    hipStream_t st = (hipStream_t)stream;
-    std::vector<int32_t> ptr((size_t)n_rows + 1);
-    FGNN_HIP(hipMemcpyAsync(ptr.data(), ptr_dev, sizeof(int32_t) * ((size_t)n_rows + 1), hipMemcpyDeviceToHost, st));
-    FGNN_HIP(hipStreamSynchronize(st));
-    FGNN_REQUIRE(ptr[0] == 0, FGNN_ERR_SHAPE, "fgnn_schedule_create: ptr[0]=%d, expected 0", ptr[0]);
-    for (int i = 0; i < n_rows; ++i)
-        FGNN_REQUIRE(ptr[i + 1] >= ptr[i], FGNN_ERR_SHAPE, "fgnn_schedule_create: ptr decreases at row %d", i);
-
-    std::vector<fgnn_item> items;
-    std::vector<fgnn_split> splits;
-    items.reserve((size_t)n_rows + 1024);
-    int n_part = 0;
-    // segments of long rows first (they are the largest items), then whole rows, longest first
-    for (int i = 0; i < n_rows; ++i) {
-        int deg = ptr[i + 1] - ptr[i];
-        if (deg <= seg_len) continue;
-        int nseg = (deg + seg_len - 1) / seg_len;
-        int len = (((deg + nseg - 1) / nseg) + 63) & ~63;
-        nseg = (deg + len - 1) / len;
-        splits.push_back({i, n_part, nseg, 0});
-        for (int g = 0; g < nseg; ++g) {
-            int b = ptr[i] + g * len;
-            int e = std::min(ptr[i + 1], b + len);
-            items.push_back({i, b, e, n_part++});
+    int row = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (row >= n_rows) return;
+    const int lane = fg_lane();
+    const int pb = fg_uni(ptr[row]), pe = fg_uni(ptr[row + 1]);
+    int cnt[FGNN_NUM_XCD];
+#pragma unroll
+    for (int b = 0; b < FGNN_NUM_XCD; ++b) cnt[b] = 0;
+    for (int c = pb; c < pe; c += 64) {
+        int q = c + lane;
+        bool ok = q < pe;
+        int bk = ok ? fgnn_bucket_of(idx[q]) : -1;
+#pragma unroll
+        for (int b = 0; b < FGNN_NUM_XCD; ++b) cnt[b] += __popcll(__builtin_amdgcn_ballot_w64(bk == b));
+    }
+    int off[FGNN_NUM_XCD];
+    int run = pb;
+#pragma unroll
+    for (int b = 0; b < FGNN_NUM_XCD; ++b) { off[b] = run; run += cnt[b]; }
+    if (lane < FGNN_NUM_XCD) {
+        int v = 0;
+#pragma unroll
+        for (int b = 0; b < FGNN_NUM_XCD; ++b) v = (lane == b) ? cnt[b] : v;
+        bcnt[(size_t)row * FGNN_NUM_XCD + lane] = v;
+    }
+    const unsigned long long lt = (1ull << lane) - 1ull;
+    for (int c = pb; c < pe; c += 64) {
+        int q = c + lane;
+        bool ok = q < pe;
+        int id = ok ? idx[q] : 0;
+        int bk = ok ? fgnn_bucket_of(id) : -1;
+        int dst = 0;
+#pragma unroll
+        for (int b = 0; b < FGNN_NUM_XCD; ++b) {
+            unsigned long long m = __builtin_amdgcn_ballot_w64(bk == b);
+            if (bk == b) dst = off[b] + __popcll(m & lt);
+            off[b] += __popcll(m);
         }
+        if (ok) bidx[dst] = id;
     }
-    size_t first_whole = items.size();
-    for (int i = 0; i < n_rows; ++i) {
-        int deg = ptr[i + 1] - ptr[i];
-        if (deg <= seg_len) items.push_back({i, ptr[i], ptr[i + 1], -1});
-    }
-    std::stable_sort(items.begin() + first_whole, items.end(),
-                     [](const fgnn_item &a, const fgnn_item &b) { return (a.end - a.begin) > (b.end - b.begin); });
+}
 
-    fgnn_schedule *s = new fgnn_schedule();
-    s->n_rows = n_rows;
-    s->n_edges = n_rows ? ptr[n_rows] : 0;
-    s->seg_len = seg_len;
-    s->n_items = (int)items.size();
-    s->n_partials = n_part;
-    s->n_split = (int)splits.size();
-    s->items_dev = nullptr;
-    s->split_dev = nullptr;
-    s->ptr_dev = ptr_dev;
-    (void)hipGetDevice(&s->device);
+static void split_range(std::vector<fgnn_item> &out, int row, int b, int e, int seg_len, int &n_part, int &nseg_total)
+{
+    int len = e - b;
+    int nseg = (len + seg_len - 1) / seg_len;
+    int step = (((len + nseg - 1) / nseg) + 63) & ~63;
+    for (int s = b; s < e; s += step) {
+        out.push_back({row, s, std::min(e, s + step), n_part++});
+        ++nseg_total;
+    }
+}
+
+static int upload_schedule(fgnn_schedule *s, const std::vector<fgnn_item> &items, const std::vector<fgnn_split> &splits, hipStream_t st)
+{
     hipError_t err = hipSuccess;
     if (!items.empty()) {
         err = hipMalloc((void **)&s->items_dev, items.size() * sizeof(fgnn_item));
@@ -80,10 +89,165 @@ extern "C" int fgnn_schedule_create(const int32_t *ptr_dev, int n_rows, int seg_
     }
     if (err == hipSuccess) err = hipStreamSynchronize(st);   // the host vectors die at return
     if (err != hipSuccess) {
-        fgnn_set_error("fgnn_schedule_create: %s", hipGetErrorString(err));
-        fgnn_schedule_destroy(s);
+        fgnn_set_error("schedule upload: %s", hipGetErrorString(err));
         return (int)err;
     }
+    return 0;
+}
+
+static int read_ptr(const int32_t *ptr_dev, int n_rows, hipStream_t st, std::vector<int32_t> &ptr)
+{
+    ptr.resize((size_t)n_rows + 1);
+    FGNN_HIP(hipMemcpyAsync(ptr.data(), ptr_dev, sizeof(int32_t) * ((size_t)n_rows + 1), hipMemcpyDeviceToHost, st));
+    FGNN_HIP(hipStreamSynchronize(st));
+    FGNN_REQUIRE(ptr[0] == 0, FGNN_ERR_SHAPE, "schedule: ptr[0]=%d, expected 0", ptr[0]);
+    for (int i = 0; i < n_rows; ++i)
+        FGNN_REQUIRE(ptr[i + 1] >= ptr[i], FGNN_ERR_SHAPE, "schedule: ptr decreases at row %d", i);
+    return 0;
+}
+
+static fgnn_schedule *new_schedule(const int32_t *ptr_dev, int n_rows, int64_t n_edges, int seg_len)
+{
+    fgnn_schedule *s = new fgnn_schedule();
+    s->n_rows = n_rows; s->n_edges = n_edges; s->seg_len = seg_len;
+    s->n_items = s->n_partials = s->n_split = 0;
+    s->items_dev = nullptr; s->split_dev = nullptr; s->ptr_dev = ptr_dev;
+    s->n_buckets = 0; s->idx_src_dev = nullptr; s->bidx_dev = nullptr;
+    (void)hipGetDevice(&s->device);
+    return s;
+}
+
+extern "C" int fgnn_schedule_create(const int32_t *ptr_dev, int n_rows, int seg_len, void *stream, fgnn_schedule_t **out)
+{
+    FGNN_REQUIRE(ptr_dev && out, FGNN_ERR_NULL, "fgnn_schedule_create: NULL argument");
+    FGNN_REQUIRE(n_rows >= 0, FGNN_ERR_SHAPE, "fgnn_schedule_create: n_rows=%d", n_rows);
+    if (seg_len <= 0) seg_len = 2048;
+    seg_len = (seg_len + 63) & ~63;
+    hipStream_t st = (hipStream_t)stream;
+    std::vector<int32_t> ptr;
+    int rc = read_ptr(ptr_dev, n_rows, st, ptr);
+    if (rc) return rc;
+
+    std::vector<fgnn_item> items;
+    std::vector<fgnn_split> splits;
+    items.reserve((size_t)n_rows + 1024);
+    int n_part = 0;
+    // segments of long rows first (they are the largest items), then whole rows, longest first
+    for (int i = 0; i < n_rows; ++i) {
+        int deg = ptr[i + 1] - ptr[i];
+        if (deg <= seg_len) continue;
+        int first = n_part, nseg = 0;
+        split_range(items, i, ptr[i], ptr[i + 1], seg_len, n_part, nseg);
+        splits.push_back({i, first, nseg, 0});
+    }
+    size_t first_whole = items.size();
+    for (int i = 0; i < n_rows; ++i) {
+        int deg = ptr[i + 1] - ptr[i];
+        if (deg <= seg_len) items.push_back({i, ptr[i], ptr[i + 1], -1});
+    }
+    std::stable_sort(items.begin() + first_whole, items.end(),
+                     [](const fgnn_item &a, const fgnn_item &b) { return (a.end - a.begin) > (b.end - b.begin); });
+
+    fgnn_schedule *s = new_schedule(ptr_dev, n_rows, n_rows ? ptr[n_rows] : 0, seg_len);
+    s->n_items = (int)items.size();
+    s->n_partials = n_part;
+    s->n_split = (int)splits.size();
+    rc = upload_schedule(s, items, splits, st);
+    if (rc) { fgnn_schedule_destroy(s); return rc; }
+    *out = s;
+    return 0;
+}
+
+// XCD-aware schedule.  Rows with more than `min_deg` entries are cut by SOURCE BUCKET (8 buckets,
+// fgnn_bucket_of): the library keeps a copy of the index array with every row's entries grouped by
+// bucket, and lays the work items out so that workgroup w only gets segments of bucket w % 8.  Each
+// XCD's L2 then sees one eighth of the gathered rows, which is what lets the hot ones stay resident.
+// Shorter rows stay whole and are dealt round-robin.  Segments are partial results merged by row.
+extern "C" int fgnn_schedule_create_bucketed(const int32_t *ptr_dev, const int32_t *idx_dev, int n_rows, int seg_len, int min_deg,
+                                             void *stream, fgnn_schedule_t **out)
+{
+    FGNN_REQUIRE(ptr_dev && out, FGNN_ERR_NULL, "fgnn_schedule_create_bucketed: NULL argument");
+    FGNN_REQUIRE(n_rows >= 0, FGNN_ERR_SHAPE, "fgnn_schedule_create_bucketed: n_rows=%d", n_rows);
+    if (seg_len <= 0) seg_len = 2048;
+    seg_len = (seg_len + 63) & ~63;
+    if (min_deg <= 0) min_deg = 64;
+    hipStream_t st = (hipStream_t)stream;
+    std::vector<int32_t> ptr;
+    int rc = read_ptr(ptr_dev, n_rows, st, ptr);
+    if (rc) return rc;
+    const int64_t n_edges = n_rows ? ptr[n_rows] : 0;
+    FGNN_REQUIRE(idx_dev || n_edges == 0, FGNN_ERR_NULL, "fgnn_schedule_create_bucketed: idx is NULL");
+
+    fgnn_schedule *s = new_schedule(ptr_dev, n_rows, n_edges, seg_len);
+    s->n_buckets = FGNN_NUM_XCD;
+    s->idx_src_dev = idx_dev;
+    std::vector<int32_t> bcnt((size_t)n_rows * FGNN_NUM_XCD);
+    if (n_rows > 0) {
+        int32_t *bcnt_dev = nullptr;
+        hipError_t err = hipMalloc((void **)&bcnt_dev, bcnt.size() * sizeof(int32_t));
+        if (err == hipSuccess && n_edges > 0) err = hipMalloc((void **)&s->bidx_dev, (size_t)n_edges * sizeof(int32_t));
+        if (err == hipSuccess) {
+            hipLaunchKernelGGL(bucket_partition_kernel, dim3((unsigned)((n_rows + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, st,
+                               n_rows, ptr_dev, idx_dev, s->bidx_dev, bcnt_dev);
+            err = hipGetLastError();
+        }
+        if (err == hipSuccess) err = hipMemcpyAsync(bcnt.data(), bcnt_dev, bcnt.size() * sizeof(int32_t), hipMemcpyDeviceToHost, st);
+        if (err == hipSuccess) err = hipStreamSynchronize(st);
+        if (bcnt_dev) (void)hipFree(bcnt_dev);
+        if (err != hipSuccess) {
+            fgnn_set_error("fgnn_schedule_create_bucketed: %s", hipGetErrorString(err));
+            fgnn_schedule_destroy(s);
+            return (int)err;
+        }
+    }
+
+    std::vector<fgnn_item> lists[FGNN_NUM_XCD];
+    std::vector<fgnn_split> splits;
+    int n_part = 0;
+    for (int i = 0; i < n_rows; ++i) {
+        int deg = ptr[i + 1] - ptr[i];
+        if (deg <= min_deg) continue;
+        int first = n_part, nseg = 0, b0 = ptr[i];
+        for (int b = 0; b < FGNN_NUM_XCD; ++b) {
+            int c = bcnt[(size_t)i * FGNN_NUM_XCD + b];
+            if (c > 0) split_range(lists[b], i, b0, b0 + c, seg_len, n_part, nseg);
+            b0 += c;
+        }
+        splits.push_back({i, first, nseg, 0});
+    }
+    for (int b = 0; b < FGNN_NUM_XCD; ++b)
+        std::stable_sort(lists[b].begin(), lists[b].end(),
+                         [](const fgnn_item &a, const fgnn_item &c) { return (a.end - a.begin) > (c.end - c.begin); });
+    // whole rows, longest first, dealt to the currently shortest list (by item count)
+    std::vector<fgnn_item> whole;
+    for (int i = 0; i < n_rows; ++i) {
+        int deg = ptr[i + 1] - ptr[i];
+        if (deg <= min_deg) whole.push_back({i, ptr[i], ptr[i + 1], -1});
+    }
+    std::stable_sort(whole.begin(), whole.end(), [](const fgnn_item &a, const fgnn_item &c) { return (a.end - a.begin) > (c.end - c.begin); });
+    {
+        size_t target = 0;
+        for (int b = 0; b < FGNN_NUM_XCD; ++b) target += lists[b].size();
+        target = (target + whole.size() + FGNN_NUM_XCD - 1) / FGNN_NUM_XCD;
+        size_t w = 0;
+        // first level the lists, then deal the rest round-robin
+        for (int b = 0; b < FGNN_NUM_XCD && w < whole.size(); ++b)
+            while (lists[b].size() < target && w < whole.size()) lists[b].push_back(whole[w++]);
+        for (int b = 0; w < whole.size(); b = (b + 1) % FGNN_NUM_XCD) lists[b].push_back(whole[w++]);
+    }
+    size_t longest = 0;
+    for (int b = 0; b < FGNN_NUM_XCD; ++b) longest = std::max(longest, lists[b].size());
+    size_t groups = (longest + FGNN_WPB - 1) / FGNN_WPB;
+    std::vector<fgnn_item> items(groups * FGNN_NUM_XCD * FGNN_WPB, fgnn_item{-1, 0, 0, -1});
+    for (int b = 0; b < FGNN_NUM_XCD; ++b)
+        for (size_t k = 0; k < lists[b].size(); ++k)
+            items[((k / FGNN_WPB) * FGNN_NUM_XCD + b) * FGNN_WPB + (k % FGNN_WPB)] = lists[b][k];   // workgroup = group*8 + bucket
+
+    s->n_items = (int)items.size();
+    s->n_partials = n_part;
+    s->n_split = (int)splits.size();
+    rc = upload_schedule(s, items, splits, st);
+    if (rc) { fgnn_schedule_destroy(s); return rc; }
     *out = s;
     return 0;
 }
@@ -93,6 +257,7 @@ extern "C" void fgnn_schedule_destroy(fgnn_schedule_t *s)
     if (!s) return;
     if (s->items_dev) (void)hipFree(s->items_dev);
     if (s->split_dev) (void)hipFree(s->split_dev);
+    if (s->bidx_dev) (void)hipFree(s->bidx_dev);
     delete s;
 }
 

@@ -106,9 +106,11 @@ static int spmm_checks(const char *fn, int N, int64_t E, int H, int F, const fgn
     FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1 && F >= 1, FGNN_ERR_SHAPE, "%s: bad sizes N=%d E=%lld H=%d F=%d", fn, N, (long long)E, H, F);
     FGNN_REQUIRE(E <= 2147483647LL, FGNN_ERR_LIMIT, "%s: E=%lld exceeds int32 positions", fn, (long long)E);
     FGNN_REQUIRE(H <= 64 && (int64_t)H * F <= 1024, FGNN_ERR_LIMIT, "%s: H=%d, H*F=%lld unsupported (limits 64, 1024)", fn, H, (long long)H * F);
-    if (sched)
+    if (sched) {
         FGNN_REQUIRE(sched->ptr_dev == ptr && sched->n_rows == N && sched->n_edges == E, FGNN_ERR_SCHEDULE,
                      "%s: schedule was built for another pointer array", fn);
+        FGNN_REQUIRE(sched->n_buckets == 0, FGNN_ERR_SCHEDULE, "%s: an XCD-aware schedule cannot be used with per-edge arrays", fn);
+    }
     return 0;
 }
 

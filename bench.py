@@ -120,8 +120,9 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
     g, t_gen, t_csc = build_gat_graph(n, e_target, dev)
     e = g.n_edges
     t0 = time.time()
-    s_csr = _lib.schedule_for(g.row_ptr)
-    s_csc = _lib.schedule_for(g.col_ptr)
+    s_csr = _lib.schedule_for(g.row_ptr, idx_tensor=g.col_ind)
+    s_csc = _lib.schedule_for(g.col_ptr, idx_tensor=g.row_ind)
+    torch.cuda.synchronize()
     t_sched = time.time() - t0
     slope = 0.2
     layer = GATConv(in_feats, out_feats, heads, slope).to(dev)
@@ -186,7 +187,8 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
                          "sample": "DGL-composed GAT layer (torch CPU, %d threads) fwd+bwd on the first %d rows = %d edges of the same graph: "
                                    "median %.1f ms over %d iters, scaled by E/E_sample = %.1f" % (cores, cpu_rows, cpu_e, cpu_ms, cpu_iters, e / cpu_e)},
         "preprocess_s": {"graph_gen": round(t_gen, 3), "csr2csc_first_call": round(t_csc, 4), "schedules": round(t_sched, 4)},
-        "schedule": {"csr_items": s_csr.n_items, "csr_partials": s_csr.n_partials, "csc_items": s_csc.n_items, "csc_partials": s_csc.n_partials},
+        "schedule": {"xcd_aware": s_csr.idx_tensor is not None, "csr_items": s_csr.n_items, "csr_partials": s_csr.n_partials,
+                     "csc_items": s_csc.n_items, "csc_partials": s_csc.n_partials},
         "peak_hbm_GiB": round(peak_mem, 3),
     }
     return rec

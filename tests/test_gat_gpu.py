@@ -85,3 +85,31 @@ def test_gat_self_loops_only_is_identity():
 def test_gat_c1_config():
     # BASELINE config 1: N=4096, 32k uniform edges + self loops, 4 heads x 16
     _run(graphs.uniform_graph(4096, 32768, seed=0), 4, 16)
+
+
+@pytest.mark.parametrize("h,f", [(8, 32), (1, 47), (4, 128)])
+def test_gat_xcd_bucketed_schedule(h, f, monkeypatch):
+    # force the XCD-aware schedule on a small graph: rows above 16 entries are cut by source bucket
+    from ae_mlsys_gnn_amd import _lib
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
+    monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+    monkeypatch.setenv("FGNN_SEG_LEN", "128")
+    _lib.clear_schedule_cache()
+    _run(degree_edge_graph(seed=7), h, f)
+    _run(graphs.rmat_graph(3000, 200000, seed=8), h, f)
+    _lib.clear_schedule_cache()
+
+
+def test_gat_xcd_bucketed_rejects_stash(monkeypatch):
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd._lib import FgnnError, lib, ptr, stream_ptr
+    g = graphs.add_csc_torch(graphs.rmat_graph(500, 20000, seed=1)).to("cuda:0")
+    s = _lib.Schedule(g.row_ptr, 0, g.col_ind, 16)
+    n, h, f = g.n, 2, 8
+    x = torch.randn(n, h, f, device="cuda:0"); a = torch.randn(n, h, device="cuda:0")
+    out = torch.empty_like(x); m = torch.empty(n, h, device="cuda:0"); sm = torch.empty_like(m)
+    el = torch.empty(g.n_edges, h, device="cuda:0"); es = torch.empty_like(el)
+    ws = torch.empty(lib().fgnn_gat_forward_workspace_bytes(s.handle, h, f) // 4 + 4, device="cuda:0")
+    rc = lib().fgnn_gat_forward(n, g.n_edges, h, f, ptr(a), ptr(a), ptr(g.row_ptr), ptr(g.col_ind), 0.2, ptr(x), ptr(out), ptr(m),
+                                ptr(sm), None, None, ptr(el), ptr(es), s.handle, ptr(ws), ws.numel() * 4, stream_ptr())
+    assert rc == -6 and b"XCD-aware" in lib().fgnn_last_error()

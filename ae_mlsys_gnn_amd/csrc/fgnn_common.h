@@ -148,12 +148,19 @@ __device__ __forceinline__ void fg_wave_lds_sync()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 __device__ __forceinline__ float fg_lrelu(float x, float slope) { return x > 0.f ? x : x * slope; }
+// SLE1: the slope is known to lie in [0, 1], where LeakyReLU(x) == max(x, slope*x)
+template <bool SLE1>
+__device__ __forceinline__ float fg_lrelu_t(float x, float slope) { return SLE1 ? fmaxf(x, x * slope) : (x > 0.f ? x : x * slope); }
+#define FGNN_LOG2E 1.4426950408889634f
+#define FGNN_LN2 0.6931471805599453f
 
 template <int VEC> struct fg_vec;
 template <> struct fg_vec<4> {
     float4 v;
     __device__ __forceinline__ void zero() { v = make_float4(0.f, 0.f, 0.f, 0.f); }
     __device__ __forceinline__ void load(const float *p) { v = *reinterpret_cast<const float4 *>(p); }
+    // wave-uniform base + unsigned 32-bit byte offset: lets the load use a scalar base register
+    __device__ __forceinline__ void load_off(const char *base, uint32_t off) { v = *reinterpret_cast<const float4 *>(base + off); }
     __device__ __forceinline__ void store(float *p) const { *reinterpret_cast<float4 *>(p) = v; }
     __device__ __forceinline__ void fma(float w, const fg_vec &x) { v.x = fmaf(w, x.v.x, v.x); v.y = fmaf(w, x.v.y, v.y); v.z = fmaf(w, x.v.z, v.z); v.w = fmaf(w, x.v.w, v.w); }
     __device__ __forceinline__ void add(const fg_vec &x) { v.x += x.v.x; v.y += x.v.y; v.z += x.v.z; v.w += x.v.w; }
@@ -166,6 +173,7 @@ template <> struct fg_vec<1> {
     float v;
     __device__ __forceinline__ void zero() { v = 0.f; }
     __device__ __forceinline__ void load(const float *p) { v = *p; }
+    __device__ __forceinline__ void load_off(const char *base, uint32_t off) { v = *reinterpret_cast<const float *>(base + off); }
     __device__ __forceinline__ void store(float *p) const { *p = v; }
     __device__ __forceinline__ void fma(float w, const fg_vec &x) { v = fmaf(w, x.v, v); }
     __device__ __forceinline__ void add(const fg_vec &x) { v += x.v; }

@@ -36,21 +36,24 @@ __host__ __device__ static inline int gat_fwd_pw(int HF, int H, bool aux) { retu
 // One batch of UB edges of the forward: UB feature rows and UB x R attention scores are fetched
 // together (every lane reads the score of the head its features belong to), then the running
 // maximum of the online softmax is raised once for the batch and the rows are accumulated.
-template <int VEC, int R, bool AUX, bool FULL, int UB>
-__device__ __forceinline__ void gat_fwd_batch(const GatFwdP &p, const fg_lanemap<VEC, R> &lm, int idv, int t, int cnt,
-                                              const float (&arh)[R], float (&m)[R], float (&s)[R], float (&cp)[R],
-                                              fg_vec<VEC> (&T)[R], fg_vec<VEC> (&P)[R])
+// Scores are kept in log2 units (LeakyReLU commutes with the positive factor log2(e)), so the
+// numerator is one v_exp_f32.  TAIL: the batch may reach past the end of the chunk.
+template <int VEC, int R, bool AUX, bool FULL, int UB, bool TAIL, bool SLE1>
+__device__ __forceinline__ void gat_fwd_batch(const GatFwdP &p, const fg_lanemap<VEC, R> &lm, const uint32_t (&boff)[R],
+                                              const uint32_t (&hoff)[R], int idv, int t, int cnt, const float (&arh)[R],
+                                              float (&m)[R], float (&s)[R], float (&cp)[R], fg_vec<VEC> (&T)[R], fg_vec<VEC> (&P)[R])
 {
     fg_vec<VEC> ld[UB][R];
     float ev[UB][R];
+    const size_t row_bytes = (size_t)p.HF * sizeof(float), sc_bytes = (size_t)p.H * sizeof(float);
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
-        int j = __builtin_amdgcn_readlane(idv, t + u);
-        const float *base = p.x + (size_t)j * (size_t)p.HF;
-        const float *acb = p.ac + (size_t)j * (size_t)p.H;
+        size_t j = (size_t)(unsigned)__builtin_amdgcn_readlane(idv, t + u);
+        const char *base = (const char *)p.x + j * row_bytes;
+        const char *acb = (const char *)p.ac + j * sc_bytes;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            if (FULL || lm.ok[r]) { ld[u][r].load(base + lm.eoff[r]); ev[u][r] = acb[lm.hd[r]]; }
+            if (FULL || lm.ok[r]) { ld[u][r].load_off(base, boff[r]); ev[u][r] = *(const float *)(acb + hoff[r]); }
             else { ld[u][r].zero(); ev[u][r] = 0.f; }
         }
     }
@@ -59,29 +62,33 @@ __device__ __forceinline__ void gat_fwd_batch(const GatFwdP &p, const fg_lanemap
     for (int r = 0; r < R; ++r) bm[r] = -INFINITY;
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
-        const bool live = (t + u) < cnt;           // wave-uniform: edges past the chunk get weight 0
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            float v = fg_lrelu(arh[r] + ev[u][r], p.slope);
-            v = live ? v : -INFINITY;
+            float v = fg_lrelu_t<SLE1>(fmaf(ev[u][r], FGNN_LOG2E, arh[r]), p.slope);
+            if (TAIL) v = ((t + u) < cnt) ? v : -INFINITY;      // wave-uniform: edges past the chunk get weight 0
             ev[u][r] = v;
             bm[r] = fmaxf(bm[r], v);
         }
     }
+    bool raised = false;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        float mn = fmaxf(m[r], bm[r]);
-        float sc = __expf(m[r] - mn);              // 1 when the maximum did not move, 0 on the first batch
-        m[r] = mn;
-        T[r].scale(sc);
-        s[r] *= sc;
-        if (AUX) { P[r].scale(sc); cp[r] *= sc; }
+    for (int r = 0; r < R; ++r) raised |= bm[r] > m[r];
+    if (__builtin_amdgcn_ballot_w64(raised) != 0ull) {          // the running maximum rarely moves after the first batches
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            float mn = fmaxf(m[r], bm[r]);
+            float sc = __builtin_amdgcn_exp2f(m[r] - mn);        // 1 when this head's maximum did not move, 0 on the first batch
+            m[r] = mn;
+            T[r].scale(sc);
+            s[r] *= sc;
+            if (AUX) { P[r].scale(sc); cp[r] *= sc; }
+        }
     }
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            float w = __expf(ev[u][r] - m[r]);
+            float w = __builtin_amdgcn_exp2f(ev[u][r] - m[r]);
             T[r].fma(w, ld[u][r]);
             s[r] += w;
             if (AUX) {
@@ -93,7 +100,7 @@ __device__ __forceinline__ void gat_fwd_batch(const GatFwdP &p, const fg_lanemap
     }
 }
 
-template <int VEC, int R, bool AUX, bool FULL>
+template <int VEC, int R, bool AUX, bool FULL, bool SLE1>
 __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_kernel(GatFwdP p)
 {
     int row, b, e, slot;
@@ -106,10 +113,13 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_kernel(GatFwdP p)
 
     fg_vec<VEC> T[R], P[R];
     float arh[R], m[R], s[R], cp[R];
+    uint32_t boff[R], hoff[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         T[r].zero(); P[r].zero(); s[r] = 0.f; cp[r] = 0.f; m[r] = -INFINITY;
-        arh[r] = p.ar[(size_t)row * H + lm.hd[r]];
+        arh[r] = p.ar[(size_t)row * H + lm.hd[r]] * FGNN_LOG2E;
+        boff[r] = (uint32_t)lm.eoff[r] * 4u;
+        hoff[r] = (uint32_t)lm.hd[r] * 4u;
     }
     constexpr int U = (R >= 8) ? 1 : 8 / R;        // feature rows in flight per wave
     for (int c = b; c < e; c += 64) {
@@ -117,15 +127,24 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_kernel(GatFwdP p)
         int cnt = min(64, e - c);
         int idv = p.idx[q < e ? q : c];            // lanes past the end repeat a valid id
         int t = 0;
-        for (; t + U <= cnt; t += U) gat_fwd_batch<VEC, R, AUX, FULL, U>(p, lm, idv, t, cnt, arh, m, s, cp, T, P);
+        for (; t + U <= cnt; t += U) gat_fwd_batch<VEC, R, AUX, FULL, U, false, SLE1>(p, lm, boff, hoff, idv, t, cnt, arh, m, s, cp, T, P);
         if constexpr (U >= 4) {
-            if (cnt - t > U / 2) { gat_fwd_batch<VEC, R, AUX, FULL, U>(p, lm, idv, t, cnt, arh, m, s, cp, T, P); t = cnt; }
-            else if (cnt - t > 0) { gat_fwd_batch<VEC, R, AUX, FULL, U / 2>(p, lm, idv, t, cnt, arh, m, s, cp, T, P); t = cnt; }
+            if (cnt - t > U / 2) gat_fwd_batch<VEC, R, AUX, FULL, U, true, SLE1>(p, lm, boff, hoff, idv, t, cnt, arh, m, s, cp, T, P);
+            else if (cnt - t > 0) gat_fwd_batch<VEC, R, AUX, FULL, U / 2, true, SLE1>(p, lm, boff, hoff, idv, t, cnt, arh, m, s, cp, T, P);
         } else {
-            if (cnt - t > 0) gat_fwd_batch<VEC, R, AUX, FULL, U>(p, lm, idv, t, cnt, arh, m, s, cp, T, P);
+            if (cnt - t > 0) gat_fwd_batch<VEC, R, AUX, FULL, U, true, SLE1>(p, lm, boff, hoff, idv, t, cnt, arh, m, s, cp, T, P);
         }
     }
 
+    // The maximum leaves the kernel in natural units.  Its rounding is absorbed into the sums, so
+    // that (max, sum) stay an exact pair for whoever rebuilds alpha = exp(e - max) / sum from them
+    // with max * log2(e) as the exponent offset (the backward does).
+    float mnat[R], fix[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        mnat[r] = m[r] * FGNN_LN2;
+        fix[r] = (b < e) ? __builtin_amdgcn_exp2f(m[r] - mnat[r] * FGNN_LOG2E) : 1.f;
+    }
     if (slot < 0) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -140,8 +159,8 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_kernel(GatFwdP p)
             T[r].store(p.out + o);
             if (lm.eoff[r] % p.F == 0) {
                 size_t so = (size_t)row * H + lm.hd[r];
-                p.emax[so] = (b < e) ? m[r] : -1e38f;
-                p.esum[so] = s[r];
+                p.emax[so] = (b < e) ? mnat[r] : -1e38f;
+                p.esum[so] = s[r] * fix[r];
                 if (AUX) p.cc[so] = (cp[r] + slope * (s[r] - cp[r])) * inv;
             }
         }
@@ -150,13 +169,14 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_kernel(GatFwdP p)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if (!(FULL || lm.ok[r])) continue;
+            T[r].scale(fix[r]);
             T[r].store(pp + lm.eoff[r]);
-            if (AUX) P[r].store(pp + p.HF + lm.eoff[r]);
+            if (AUX) { P[r].scale(fix[r]); P[r].store(pp + p.HF + lm.eoff[r]); }
             if (lm.eoff[r] % p.F == 0) {
                 float *st = pp + (AUX ? 2 : 1) * p.HF;
-                st[lm.hd[r]] = m[r];
-                st[H + lm.hd[r]] = s[r];
-                st[2 * H + lm.hd[r]] = cp[r];
+                st[lm.hd[r]] = mnat[r];
+                st[H + lm.hd[r]] = s[r] * fix[r];
+                st[2 * H + lm.hd[r]] = cp[r] * fix[r];
             }
         }
     }
@@ -271,7 +291,8 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_node_kernel(int N, int H, in
     if (lane < H) {
         size_t q = (size_t)i * H + lane;
         float s = esum[q];
-        rec[q] = make_float4(ar[q], emax[q], s > 0.f ? 1.f / s : 0.f, delta);
+        // attn_row and the maximum are stored in log2 units for the column pass
+        rec[q] = make_float4(ar[q] * FGNN_LOG2E, emax[q] * FGNN_LOG2E, s > 0.f ? 1.f / s : 0.f, delta);
         gar[q] = dd2 - delta * cc[q];
     }
 }
@@ -301,25 +322,31 @@ __device__ __forceinline__ void gat_bwd_finish(const GatBwdP &p, int col, int la
 }
 
 // One batch of UB edges of the backward column pass.  Every lane reads the 16-byte record
-// (attn_row, max, 1/sum, delta) of the head its features belong to and recomputes alpha itself.
-template <int VEC, int R, bool STASH, bool FULL, int UB>
-__device__ __forceinline__ void gat_bwd_batch(const GatBwdP &p, const fg_lanemap<VEC, R> &lm, int idv, int posv, int t, int cnt,
+// (attn_row, max, 1/sum, delta) of the head its features belong to (the first two in log2 units)
+// and recomputes alpha itself.
+template <int VEC, int R, bool STASH, bool FULL, int UB, bool TAIL, bool SLE1>
+__device__ __forceinline__ void gat_bwd_batch(const GatBwdP &p, const fg_lanemap<VEC, R> &lm, const uint32_t (&boff)[R],
+                                              const uint32_t (&roff)[R], const uint32_t (&hoff)[R], int idv, int posv, int t, int cnt,
                                               const float (&ach)[R], float (&z)[R], fg_vec<VEC> (&T)[R], fg_vec<VEC> (&P)[R])
 {
     fg_vec<VEC> ld[UB][R];
     float4 rc[UB][R];
+    const size_t row_bytes = (size_t)p.HF * sizeof(float), rec_bytes = (size_t)p.H * sizeof(float4), sc_bytes = (size_t)p.H * sizeof(float);
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
-        int i = __builtin_amdgcn_readlane(idv, t + u);
-        const float *base = p.g + (size_t)i * (size_t)p.HF;
-        const float4 *rb = p.rec + (size_t)i * (size_t)p.H;
-        size_t pos = STASH ? (size_t)__builtin_amdgcn_readlane(posv, t + u) * (size_t)p.H : 0;
+        size_t i = (size_t)(unsigned)__builtin_amdgcn_readlane(idv, t + u);
+        const char *base = (const char *)p.g + i * row_bytes;
+        const char *rb = (const char *)p.rec + i * rec_bytes;
+        size_t pos = STASH ? (size_t)(unsigned)__builtin_amdgcn_readlane(posv, t + u) * sc_bytes : 0;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if (FULL || lm.ok[r]) {
-                ld[u][r].load(base + lm.eoff[r]);
-                rc[u][r] = rb[lm.hd[r]];
-                if (STASH) { rc[u][r].x = p.erelu[pos + lm.hd[r]]; rc[u][r].y = p.esm[pos + lm.hd[r]]; }
+                ld[u][r].load_off(base, boff[r]);
+                rc[u][r] = *(const float4 *)(rb + roff[r]);
+                if (STASH) {
+                    rc[u][r].x = *(const float *)((const char *)p.erelu + pos + hoff[r]);
+                    rc[u][r].y = *(const float *)((const char *)p.esm + pos + hoff[r]);
+                }
             } else {
                 ld[u][r].zero();
                 rc[u][r] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -328,13 +355,12 @@ __device__ __forceinline__ void gat_bwd_batch(const GatBwdP &p, const fg_lanemap
     }
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
-        const bool live = (t + u) < cnt;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             float ev, al;
             if (STASH) { ev = rc[u][r].x; al = rc[u][r].y; }
-            else { ev = fg_lrelu(rc[u][r].x + ach[r], p.slope); al = __expf(ev - rc[u][r].y) * rc[u][r].z; }
-            al = live ? al : 0.f;
+            else { ev = fg_lrelu_t<SLE1>(fmaf(ach[r], FGNN_LOG2E, rc[u][r].x), p.slope); al = __builtin_amdgcn_exp2f(ev - rc[u][r].y) * rc[u][r].z; }
+            if (TAIL) al = ((t + u) < cnt) ? al : 0.f;
             const bool pos_e = ev > 0.f;
             T[r].fma(al, ld[u][r]);
             P[r].fma(pos_e ? al : 0.f, ld[u][r]);
@@ -343,7 +369,7 @@ __device__ __forceinline__ void gat_bwd_batch(const GatBwdP &p, const fg_lanemap
     }
 }
 
-template <int VEC, int R, bool STASH, bool FULL>
+template <int VEC, int R, bool STASH, bool FULL, bool SLE1>
 __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_kernel(GatBwdP p)
 {
     extern __shared__ float lds[];
@@ -357,8 +383,15 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_kernel(GatBwdP p)
 
     fg_vec<VEC> T[R], P[R];
     float ach[R], z[R];
+    uint32_t boff[R], roff[R], hoff[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) { T[r].zero(); P[r].zero(); z[r] = 0.f; ach[r] = p.ac[(size_t)col * H + lm.hd[r]]; }
+    for (int r = 0; r < R; ++r) {
+        T[r].zero(); P[r].zero(); z[r] = 0.f;
+        ach[r] = p.ac[(size_t)col * H + lm.hd[r]];
+        boff[r] = (uint32_t)lm.eoff[r] * 4u;
+        roff[r] = (uint32_t)lm.hd[r] * 16u;
+        hoff[r] = (uint32_t)lm.hd[r] * 4u;
+    }
 
     constexpr int U = (R >= 8) ? 1 : 8 / R;
     for (int c = b; c < e; c += 64) {
@@ -368,12 +401,12 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_kernel(GatBwdP p)
         int idv = p.idx[qq];
         int posv = STASH ? p.permute[qq] : 0;
         int t = 0;
-        for (; t + U <= cnt; t += U) gat_bwd_batch<VEC, R, STASH, FULL, U>(p, lm, idv, posv, t, cnt, ach, z, T, P);
+        for (; t + U <= cnt; t += U) gat_bwd_batch<VEC, R, STASH, FULL, U, false, SLE1>(p, lm, boff, roff, hoff, idv, posv, t, cnt, ach, z, T, P);
         if constexpr (U >= 4) {
-            if (cnt - t > U / 2) gat_bwd_batch<VEC, R, STASH, FULL, U>(p, lm, idv, posv, t, cnt, ach, z, T, P);
-            else if (cnt - t > 0) gat_bwd_batch<VEC, R, STASH, FULL, U / 2>(p, lm, idv, posv, t, cnt, ach, z, T, P);
+            if (cnt - t > U / 2) gat_bwd_batch<VEC, R, STASH, FULL, U, true, SLE1>(p, lm, boff, roff, hoff, idv, posv, t, cnt, ach, z, T, P);
+            else if (cnt - t > 0) gat_bwd_batch<VEC, R, STASH, FULL, U / 2, true, SLE1>(p, lm, boff, roff, hoff, idv, posv, t, cnt, ach, z, T, P);
         } else {
-            if (cnt - t > 0) gat_bwd_batch<VEC, R, STASH, FULL, U>(p, lm, idv, posv, t, cnt, ach, z, T, P);
+            if (cnt - t > 0) gat_bwd_batch<VEC, R, STASH, FULL, U, true, SLE1>(p, lm, boff, roff, hoff, idv, posv, t, cnt, ach, z, T, P);
         }
     }
 
@@ -482,8 +515,11 @@ static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_
     const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
     const size_t shm = 0;
     int rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
-        if (aux) hipLaunchKernelGGL((gat_fwd_kernel<VEC, R, true, FULL>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
-        else hipLaunchKernelGGL((gat_fwd_kernel<VEC, R, false, FULL>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+        const bool sle1 = slope >= 0.f && slope <= 1.f;
+        if (aux && sle1) hipLaunchKernelGGL((gat_fwd_kernel<VEC, R, true, FULL, true>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+        else if (aux) hipLaunchKernelGGL((gat_fwd_kernel<VEC, R, true, FULL, false>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+        else if (sle1) hipLaunchKernelGGL((gat_fwd_kernel<VEC, R, false, FULL, true>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+        else hipLaunchKernelGGL((gat_fwd_kernel<VEC, R, false, FULL, false>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
         int rc2 = fgnn_launch_status("gat_fwd_kernel");
         if (rc2) return rc2;
         if (sched && sched->n_split > 0) {
@@ -596,8 +632,10 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
         if (rc2) return rc2;
         const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
         const size_t shm = (size_t)FGNN_WPB * (64 * R + 64) * sizeof(float);
-        if (stash) hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, true, FULL>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
-        else hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, false, FULL>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+        const bool sle1 = negative_slope >= 0.f && negative_slope <= 1.f;
+        if (stash) hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, true, FULL, true>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+        else if (sle1) hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, false, FULL, true>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+        else hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, false, FULL, false>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
         rc2 = fgnn_launch_status("gat_bwd_kernel");
         if (rc2) return rc2;
         if (sched_csc && sched_csc->n_split > 0) {

@@ -18,7 +18,7 @@ def _oracle_fwd_bwd(g, x, ar, ac, go, slope):
     return out.detach(), x.grad, ar.grad, ac.grad
 
 
-def _run(g, h, f, slope=0.2, seed=0, attn_scale=1.0, variant="sm", seg_len=None, monkeypatch=None):
+def _run(g, h, f, slope=0.2, seed=0, attn_scale=1.0, variant="sm", seg_len=None, monkeypatch=None, atol=None):
     from ae_mlsys_gnn_amd.operators import fused_gat as fg
     g = graphs.add_csc_torch(g)
     x, ar, ac, go = gat_inputs(g, h, f, seed, attn_scale)
@@ -36,13 +36,14 @@ def _run(g, h, f, slope=0.2, seed=0, attn_scale=1.0, variant="sm", seg_len=None,
         out = fg.fused_gat_fusescatter(ard, acd, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, slope, xd, gd.permute)
     out.backward(go.float().to(dev))
     torch.cuda.synchronize()
-    assert_close(out, ref[0], "out")
-    assert_close(xd.grad, ref[1], "grad_feat")
+    base_atol = 1e-5 if atol is None else atol
+    assert_close(out, ref[0], "out", atol=base_atol)
+    assert_close(xd.grad, ref[1], "grad_feat", atol=base_atol)
     # grad_attn_* are sums of E/N terms of either sign: the absolute part of the bar scales with
     # the magnitude of the summands
     scale = float(go.abs().max() * x.abs().max() * f)
-    assert_close(ard.grad, ref[2], "grad_attn_row", atol=1e-5 * max(1.0, scale))
-    assert_close(acd.grad, ref[3], "grad_attn_col", atol=1e-5 * max(1.0, scale))
+    assert_close(ard.grad, ref[2], "grad_attn_row", atol=base_atol * max(1.0, scale))
+    assert_close(acd.grad, ref[3], "grad_attn_col", atol=base_atol * max(1.0, scale))
 
 
 @pytest.mark.parametrize("h,f", [(8, 32), (4, 16), (1, 64), (1, 47), (3, 20), (4, 128), (8, 128), (2, 65), (1, 1)])
@@ -66,8 +67,10 @@ def test_gat_split_rows(monkeypatch):
 
 
 def test_gat_large_attention():
-    # wide score range: the softmax must stay stable
-    _run(graphs.rmat_graph(500, 8000, seed=9), 4, 32, attn_scale=30.0)
+    # wide score range: the softmax must stay stable (no overflow, no NaN).  Scores of magnitude ~150
+    # carry an fp32 rounding error of 150 * 2^-24 ~ 1e-5 before the exponential, i.e. a relative error
+    # of that size in every attention weight, so the absolute bar is 1e-4 here instead of 1e-5.
+    _run(graphs.rmat_graph(500, 8000, seed=9), 4, 32, attn_scale=30.0, atol=1e-4)
 
 
 def test_gat_self_loops_only_is_identity():

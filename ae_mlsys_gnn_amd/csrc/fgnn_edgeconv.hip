@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256) void edgeconv_bwd_kernel(long long total, int 
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;
     int f = (int)(i % F);
-    atomicAdd(grad_src + (size_t)argmax[i] * F + f, grad_out[i]);
+    unsafeAtomicAdd(grad_src + (size_t)argmax[i] * F + f, grad_out[i]);     // hardware float add (device memory), no CAS loop
 }
 
 int fgnn_fill_f32(float *p, size_t n, float v, hipStream_t st)

@@ -181,7 +181,7 @@ __global__ __launch_bounds__(FGNN_TPB) void u_add_v_bwd_kernel(int N, int W, con
         for (int q = pb + lane; q < pe; q += 64) {
             float v = g[(size_t)q * W + w];
             acc += v;
-            atomicAdd(gcol + (size_t)idx[q] * W + w, v);
+            unsafeAtomicAdd(gcol + (size_t)idx[q] * W + w, v);
         }
         acc = fg_wave_sum(acc);
         if (lane == 0) grow[(size_t)row * W + w] = acc;

@@ -26,11 +26,24 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published peak
 
-# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE,
-# scaled by a copy kernel of known size); see profiles/.  None = not measured for that workload.
+# L2<->fabric bytes per launch of the dominant kernels measured with rocprofv3 --pmc (FETCH_SIZE scaled
+# x2.000 and WRITE_SIZE x1.000 by the 1 GiB copy of --calibrate-copy; profiles/gat_kernels_gat_c2.md).
+# They bound the HBM traffic from above.  None = not measured for that workload.
 MEASURED_TRAFFIC_BYTES = {
-    "gat_c2": None,
+    "gat_c2": {"fwd": 37_626_766_336, "bwd": 34_242_960_384},
 }
+
+
+def roofline_record(kernel, alg_bytes, ms, traffic):
+    """`achieved` is the algorithmic (no-reuse gather model) rate.  It can exceed the HBM peak when
+    gathered rows are served from the per-XCD L2; `traffic` / `traffic_frac` give the measured
+    L2<->fabric bytes and their share of the HBM peak next to it."""
+    rec = {"bound": "hbm", "kernel": kernel, "achieved": round(alg_bytes / ms / 1e6, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+           "frac": round(alg_bytes / ms / 1e6 / HBM_PEAK_GBPS, 4), "traffic": traffic, "alg_bytes": alg_bytes, "ms": round(ms, 4)}
+    if traffic:
+        rec["traffic_GBps"] = round(traffic / ms / 1e6, 1)
+        rec["traffic_frac"] = round(traffic / ms / 1e6 / HBM_PEAK_GBPS, 4)
+    return rec
 
 
 def gat_alg_bytes(n, e, h, f):
@@ -174,12 +187,9 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
         "config": {"workload": workload, "graph": "R-MAT a=0.57 b=0.19 c=0.19 d=0.05 seed 0, unique edges + self loops",
                    "nodes": n, "edges": e, "in_feats": in_feats, "heads": heads, "out_feats": out_feats,
                    "negative_slope": slope, "step": "GATConv forward + backward (torch.matmul projection + fused sparse op)"},
-        "roofline": {"bound": "hbm", "kernel": "gat_fwd_kernel (+merge of split rows)", "achieved": round(b_fwd / ms_fwd / 1e6, 1),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(b_fwd / ms_fwd / 1e6 / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(workload), "alg_bytes": b_fwd, "ms": round(ms_fwd, 4)},
-        "roofline_bwd": {"bound": "hbm", "kernel": "gat_bwd_node_kernel + gat_bwd_kernel (+merge)", "achieved": round(b_bwd / ms_bwd / 1e6, 1),
-                         "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(b_bwd / ms_bwd / 1e6 / HBM_PEAK_GBPS, 4),
-                         "alg_bytes": b_bwd, "ms": round(ms_bwd, 4)},
+        "roofline": roofline_record("gat_fwd_kernel (+gat_fwd_merge_kernel)", b_fwd, ms_fwd, (MEASURED_TRAFFIC_BYTES.get(workload) or {}).get("fwd")),
+        "roofline_bwd": roofline_record("gat_bwd_node_kernel + gat_bwd_kernel (+gat_bwd_merge_kernel)", b_bwd, ms_bwd,
+                                        (MEASURED_TRAFFIC_BYTES.get(workload) or {}).get("bwd")),
         "sparse_fwd_bwd": {"ms": round(ms_fwd + ms_bwd, 4), "alg_bytes": b_fwd + b_bwd,
                            "achieved_GBps": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6, 1),
                            "frac_of_peak": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6 / HBM_PEAK_GBPS, 4)},

@@ -123,6 +123,36 @@ def cpu_baseline_gat(g, x_feat, layer, slope, target_edges, go):
     return ms, e_s, r, cores, len(ts)
 
 
+def cpu_baseline_c1():
+    """BASELINE config 1 at its real size on the host: the DGL-composed GAT layer forward+backward,
+    N=4096, 32,768 uniform random edges + self loops, X [4096,64], 4 heads x 16, slope 0.2, loss = sum."""
+    import torch
+    from ae_mlsys_gnn_amd import graphs
+    from oracle import fgnn_oracle as orc
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    torch.manual_seed(0)
+    g = graphs.uniform_graph(4096, 32768, seed=0)
+    x = torch.randn(4096, 64)
+    w = torch.nn.init.xavier_normal_(torch.empty(64, 64)).requires_grad_(True)
+    al = (torch.randn(1, 4, 16) * 0.1).requires_grad_(True)
+    ar = (torch.randn(1, 4, 16) * 0.1).requires_grad_(True)
+
+    def step():
+        orc.gat_layer_dgl(w, al, ar, g.row_ptr, g.col_ind, 0.2, x).sum().backward()
+        w.grad = None; al.grad = None; ar.grad = None
+
+    for _ in range(5):
+        step()
+    ts = []
+    for _ in range(20):
+        t0 = time.time()
+        step()
+        ts.append((time.time() - t0) * 1e3)
+    return {"value": round(sorted(ts)[len(ts) // 2], 3), "min": round(min(ts), 3), "unit": "ms/iter", "cores": cores, "kind": "port",
+            "sample": "config C1 at full size (N=4096, E=%d), DGL-composed GAT layer in torch CPU, 5 warm-up + 20 timed, median" % g.n_edges}
+
+
 def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
     import torch
     from ae_mlsys_gnn_amd import _lib
@@ -179,6 +209,7 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
         cpu_ms, cpu_e, cpu_rows, cores, cpu_iters = float("nan"), e, 0, 0, 0
     else:
         cpu_ms, cpu_e, cpu_rows, cores, cpu_iters = cpu_baseline_gat(g, x, layer, slope, args.cpu_sample_edges, go)
+    c1 = None if args.no_cpu_baseline else cpu_baseline_c1()
     rec = {
         "metric": "GAT layer fwd+bwd ms/iter + achieved HBM GB/s (% of peak), 1 MI355X",
         "value": round(ms_step, 4), "unit": "ms/iter", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -196,6 +227,7 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
         "cpu_baseline": {"value": round(cpu_ms * e / cpu_e, 1), "unit": "ms/iter", "cores": cores, "kind": "port",
                          "sample": "DGL-composed GAT layer (torch CPU, %d threads) fwd+bwd on the first %d rows = %d edges of the same graph: "
                                    "median %.1f ms over %d iters, scaled by E/E_sample = %.1f" % (cores, cpu_rows, cpu_e, cpu_ms, cpu_iters, e / cpu_e)},
+        "cpu_baseline_c1": c1,
         "preprocess_s": {"graph_gen": round(t_gen, 3), "csr2csc_first_call": round(t_csc, 4), "schedules": round(t_sched, 4)},
         "schedule": {"xcd_aware": s_csr.idx_tensor is not None, "csr_items": s_csr.n_items, "csr_partials": s_csr.n_partials,
                      "csc_items": s_csc.n_items, "csc_partials": s_csc.n_partials},

@@ -116,3 +116,44 @@ def test_gat_xcd_bucketed_rejects_stash(monkeypatch):
     rc = lib().fgnn_gat_forward(n, g.n_edges, h, f, ptr(a), ptr(a), ptr(g.row_ptr), ptr(g.col_ind), 0.2, ptr(x), ptr(out), ptr(m),
                                 ptr(sm), None, None, ptr(el), ptr(es), s.handle, ptr(ws), ws.numel() * 4, stream_ptr())
     assert rc == -6 and b"XCD-aware" in lib().fgnn_last_error()
+
+
+def test_gat_degenerate_graphs():
+    """No edges at all, isolated nodes between connected ones, a single node with a self loop."""
+    from ae_mlsys_gnn_amd.operators import fused_gat as fg
+    dev = "cuda:0"
+    # (a) 5 nodes, no edges: outputs and every gradient are zero
+    g = graphs.add_csc_torch(custom_graph([[], [], [], [], []])).to(dev)
+    x = torch.randn(5, 2, 8, device=dev, requires_grad=True)
+    a = torch.randn(5, 2, device=dev, requires_grad=True)
+    b = torch.randn(5, 2, device=dev, requires_grad=True)
+    out = fg.fused_gat_op(a, b, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, 0.2, x)
+    out.backward(torch.ones_like(out))
+    for t in (out, x.grad, a.grad, b.grad):
+        assert bool(torch.isfinite(t).all()) and float(t.abs().max()) == 0.0
+    # (b) isolated nodes among connected ones, duplicate edges
+    _run(custom_graph([[1, 1, 2], [], [0], [], [4, 0, 0, 3], []]), 2, 8)
+    # (c) one node, one self loop: identity, gradients of the scores vanish
+    g = graphs.add_csc_torch(custom_graph([[0]])).to(dev)
+    x = torch.randn(1, 4, 16, device=dev, requires_grad=True)
+    a = torch.randn(1, 4, device=dev, requires_grad=True)
+    out = fg.fused_gat_op(a, a, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, 0.2, x)
+    go = torch.randn_like(out)
+    out.backward(go)
+    assert torch.equal(out, x) and torch.equal(x.grad, go) and float(a.grad.abs().max()) < 1e-6
+
+
+def test_gat_widest_supported_row_and_hub():
+    # H*F = 1024 (the documented limit) and one destination that every node points to
+    n = 3000
+    rows = [[(i * 7 + 1) % n, (i * 13 + 5) % n] for i in range(n)]
+    rows[17] = list(range(n))
+    _run(custom_graph(rows), 8, 128)
+    _run(custom_graph(rows), 16, 64)
+
+
+def test_gat_negative_slope_outside_unit_interval():
+    g = graphs.rmat_graph(400, 5000, seed=4)
+    _run(g, 4, 16, slope=1.5)
+    _run(g, 4, 16, slope=0.0)
+    _run(g, 4, 16, slope=1.0)

@@ -7,6 +7,7 @@ from .fused_gat import (FusedGATFunction, FusedGATFunction_SM, FusedGATFunction_
                         fused_gat_fusescatter, fused_gat_op, fused_gat_stash_op)
 from .fused_gmmconv import (GaussianCp, GaussianFunction, GmmConvFuse, GmmConvFuseEb, GmmConvStash,  # noqa: F401
                             GmmFuseEbFunction, GmmFuseFunction, GmmStashFunction)
+from .knn import knn_graph  # noqa: F401
 from .mhspmm import MHSPMMFunction, csrmhspmm, mhsddmm, mhtranspose  # noqa: F401
 from .spmm import SPMMFunction, csrspmm  # noqa: F401
 from .u_add_v import u_add_v_Function, u_add_v_op  # noqa: F401

@@ -114,6 +114,13 @@ int fgnn_edgeconv_forward(int N, int n_src, int F, int k, const int32_t *src_ind
 int fgnn_edgeconv_backward(int N, int n_src, int F, const int32_t *argmax, const float *grad_out,
                            float *grad_src, void *stream);
 
+/* k-nearest-neighbour graph of batched point clouds, the input of fgnn_edgeconv_forward: points
+ * [n_clouds*P, D]; src_ind [n_clouds*P*k] gets, for every point, the global ids of the k nearest
+ * points of its own cloud (itself included), nearest first, ties to the smaller id.  Stands in for
+ * the DGL KNNGraph call of the reference's DGCNN loop (script/train/train_edgeconv_our.py:51-55). */
+int fgnn_knn_graph(int n_clouds, int P, int D, int k, const float *points, int32_t *src_ind,
+                   void *stream);
+
 /* ---------------------------------------------------------------- fused GMMConv (MoNet)
  * Replaces gmmconv.gmmconv / gmmconveb / gmmconvstash (src/fused_gmmconv/gmmconv.cc:43-78;
  * gmmconv.cu:201-263):  w[p,k] = exp(-0.5 sum_d ((pseudo[p,d]-mu[k,d])*inv_sigma[k,d])^2),

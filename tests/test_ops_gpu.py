@@ -308,3 +308,38 @@ def test_error_paths_return_codes_not_aborts():
         fg.fused_gat_op(a.cpu(), a.cpu(), g.row_ptr.cpu(), g.col_ind.cpu(), g.col_ptr.cpu(), g.row_ind.cpu(), 0.2, x.cpu())
     with pytest.raises(FgnnError, match="int32"):
         fg.fused_gat_op(a, a, g.row_ptr.long(), g.col_ind, g.col_ptr, g.row_ind, 0.2, torch.randn(64, 8, 4, device=DEV))
+
+
+# ------------------------------------------------------------------ kNN graph builder
+@pytest.mark.parametrize("b,p,d,k", [(3, 100, 3, 5), (2, 1024, 3, 20), (2, 300, 64, 20), (1, 64, 7, 64), (4, 65, 2, 1)])
+def test_knn_graph(b, p, d, k):
+    from ae_mlsys_gnn_amd.operators.knn import knn_graph
+    gen = torch.Generator().manual_seed(b * p + d)
+    pts = torch.rand(b, p, d, generator=gen) * 2 - 1
+    src = knn_graph(pts.to(DEV), k).cpu().long().view(b, p, k)
+    # brute force in float64: exact squared distances
+    dist = ((pts.double().unsqueeze(2) - pts.double().unsqueeze(1)) ** 2).sum(-1)          # [b,p,p]
+    off = (torch.arange(b) * p).view(b, 1, 1)
+    local = src - off
+    assert bool(((local >= 0) & (local < p)).all()), "neighbours must stay inside their cloud"
+    assert bool((local[:, :, 0] == torch.arange(p).view(1, p)).all()), "the nearest point is the point itself"
+    got = torch.gather(dist, 2, local)
+    want = torch.topk(dist, k, dim=2, largest=False).values
+    # same k smallest distances, in ascending order (fp32 accumulation: tiny slack; ties may swap ids)
+    assert bool((got[:, :, 1:] >= got[:, :, :-1] - 1e-6).all())
+    assert float((got - want).abs().max()) < 1e-5
+    assert all(torch.unique(local[i, j]).numel() == k for i in range(b) for j in range(0, p, 7)), "neighbours of a point are distinct"
+
+
+def test_knn_graph_feeds_edgeconv():
+    from ae_mlsys_gnn_amd.layers import EdgeConv
+    from ae_mlsys_gnn_amd.operators.knn import knn_graph
+    torch.manual_seed(0)
+    pts = (torch.rand(4, 256, 3) * 2 - 1).to(DEV)
+    src = knn_graph(pts, 20)
+    layer = EdgeConv(3, 64).to(DEV)
+    h = layer(20, src, pts.reshape(-1, 3))
+    src2 = knn_graph(h.detach().view(4, 256, 64), 20)          # dynamic graph in feature space, as DGCNN does
+    out = EdgeConv(64, 64).to(DEV)(20, src2, h)
+    out.sum().backward()
+    assert out.shape == (1024, 64) and bool(torch.isfinite(out).all())

@@ -160,11 +160,60 @@ static int rs_num_passes(int n_cols)
     return (bits + 7) / 8;
 }
 
+// Scratch of one radix sort of n (key, payload) pairs: two key buffers, one payload buffer,
+// per-block digit counts and two 256-entry tables.
+static size_t rs_sort_workspace(int64_t n)
+{
+    size_t nblocks = (size_t)((n + RS_TILE - 1) / RS_TILE);
+    return 3 * fgnn_align256((size_t)n * sizeof(int)) + fgnn_align256(256 * nblocks * sizeof(int)) + 2 * fgnn_align256(256 * sizeof(int));
+}
+
+// Stable LSD radix sort of n pairs by the low 8*passes key bits.  keys_in is not modified; pay_in ==
+// NULL sorts the element indices.  The sorted payload lands in pay_out; *sorted_keys points at the
+// sorted keys (inside the workspace).
+static int rs_sort_pairs(const int *keys_in, const int *pay_in, int64_t n, int passes, int *pay_out, const int **sorted_keys, void *workspace,
+                         hipStream_t st)
+{
+    const int nblocks = (int)((n + RS_TILE - 1) / RS_TILE);
+    char *w = (char *)workspace;
+    int *keys[2];
+    keys[0] = (int *)w; w += fgnn_align256((size_t)n * sizeof(int));
+    keys[1] = (int *)w; w += fgnn_align256((size_t)n * sizeof(int));
+    int *pay[2];
+    pay[0] = pay_out;
+    pay[1] = (int *)w; w += fgnn_align256((size_t)n * sizeof(int));
+    int *hist = (int *)w; w += fgnn_align256(256 * (size_t)nblocks * sizeof(int));
+    int *digit_total = (int *)w; w += fgnn_align256(256 * sizeof(int));
+    int *digit_base = (int *)w;
+    const int *kin = keys_in;
+    const int *pin = pay_in;
+    for (int i = 0; i < passes; ++i) {
+        int shift = 8 * i;
+        int *kout = keys[i & 1];
+        int *pout = pay[(passes - 1 - i) & 1];      // the last pass lands in pay_out
+        hipLaunchKernelGGL(rs_hist_kernel, dim3(nblocks), dim3(RS_TPB), 0, st, kin, n, shift, nblocks, hist);
+        int rc = fgnn_launch_status("rs_hist_kernel");
+        if (rc) return rc;
+        hipLaunchKernelGGL(rs_scan_kernel, dim3(256), dim3(RS_TPB), 0, st, hist, nblocks, digit_total);
+        rc = fgnn_launch_status("rs_scan_kernel");
+        if (rc) return rc;
+        hipLaunchKernelGGL(rs_digit_base_kernel, dim3(1), dim3(256), 0, st, digit_total, digit_base);
+        rc = fgnn_launch_status("rs_digit_base_kernel");
+        if (rc) return rc;
+        hipLaunchKernelGGL(rs_scatter_kernel, dim3(nblocks), dim3(RS_TPB), 0, st, kin, pin, n, shift, nblocks, hist, digit_base, kout, pout);
+        rc = fgnn_launch_status("rs_scatter_kernel");
+        if (rc) return rc;
+        kin = kout;
+        pin = pout;
+    }
+    *sorted_keys = kin;
+    return 0;
+}
+
 extern "C" size_t fgnn_csr2csc_workspace_bytes(int n_rows, int n_cols, int64_t E)
 {
     (void)n_rows; (void)n_cols;
-    size_t nblocks = (size_t)((E + RS_TILE - 1) / RS_TILE);
-    return 3 * fgnn_align256((size_t)E * sizeof(int)) + fgnn_align256(256 * nblocks * sizeof(int)) + 2 * fgnn_align256(256 * sizeof(int));
+    return rs_sort_workspace(E);
 }
 
 extern "C" int fgnn_csr2csc(int n_rows, int n_cols, int64_t E, const int32_t *row_ptr, const int32_t *col_ind, int32_t *col_ptr,
@@ -181,40 +230,195 @@ extern "C" int fgnn_csr2csc(int n_rows, int n_cols, int64_t E, const int32_t *ro
     FGNN_REQUIRE(n_cols >= 1 && n_rows >= 1, FGNN_ERR_SHAPE, "fgnn_csr2csc: edges without rows or columns");
     size_t need = fgnn_csr2csc_workspace_bytes(n_rows, n_cols, E);
     FGNN_REQUIRE(workspace && workspace_bytes >= need, FGNN_ERR_WORKSPACE, "fgnn_csr2csc: workspace %zu < %zu bytes", workspace_bytes, need);
-    const int nblocks = (int)((E + RS_TILE - 1) / RS_TILE);
-    char *w = (char *)workspace;
-    int *keys[2];
-    keys[0] = (int *)w; w += fgnn_align256((size_t)E * sizeof(int));
-    keys[1] = (int *)w; w += fgnn_align256((size_t)E * sizeof(int));
-    int *pay[2];
-    pay[0] = permute;
-    pay[1] = (int *)w; w += fgnn_align256((size_t)E * sizeof(int));
-    int *hist = (int *)w; w += fgnn_align256(256 * (size_t)nblocks * sizeof(int));
-    int *digit_total = (int *)w; w += fgnn_align256(256 * sizeof(int));
-    int *digit_base = (int *)w;
-
-    const int passes = rs_num_passes(n_cols);
-    const int *kin = col_ind;
-    const int *pin = nullptr;
-    for (int i = 0; i < passes; ++i) {
-        int shift = 8 * i;
-        int *kout = keys[i & 1];
-        int *pout = pay[(passes - 1 - i) & 1];      // the last pass lands in `permute`
-        hipLaunchKernelGGL(rs_hist_kernel, dim3(nblocks), dim3(RS_TPB), 0, st, kin, E, shift, nblocks, hist);
-        int rc = fgnn_launch_status("rs_hist_kernel");
-        if (rc) return rc;
-        hipLaunchKernelGGL(rs_scan_kernel, dim3(256), dim3(RS_TPB), 0, st, hist, nblocks, digit_total);
-        rc = fgnn_launch_status("rs_scan_kernel");
-        if (rc) return rc;
-        hipLaunchKernelGGL(rs_digit_base_kernel, dim3(1), dim3(256), 0, st, digit_total, digit_base);
-        rc = fgnn_launch_status("rs_digit_base_kernel");
-        if (rc) return rc;
-        hipLaunchKernelGGL(rs_scatter_kernel, dim3(nblocks), dim3(RS_TPB), 0, st, kin, pin, E, shift, nblocks, hist, digit_base, kout, pout);
-        rc = fgnn_launch_status("rs_scatter_kernel");
-        if (rc) return rc;
-        kin = kout;
-        pin = pout;
-    }
-    hipLaunchKernelGGL(csc_finalize_kernel, dim3((unsigned)((E + 255) / 256)), dim3(256), 0, st, E, n_rows, n_cols, kin, permute, row_ptr, col_ptr, row_ind);
+    const int *sorted = nullptr;
+    int rc = rs_sort_pairs(col_ind, nullptr, E, rs_num_passes(n_cols), permute, &sorted, workspace, st);
+    if (rc) return rc;
+    hipLaunchKernelGGL(csc_finalize_kernel, dim3((unsigned)((E + 255) / 256)), dim3(256), 0, st, E, n_rows, n_cols, sorted, permute, row_ptr, col_ptr, row_ind);
     return fgnn_launch_status("csc_finalize_kernel");
+}
+
+// ------------------------------------------------------------------------------- COO -> CSR
+// Edge list (dst[e], src[e]) -> CSR by destination with sources ascending inside a row, optionally
+// merging duplicate edges: what the reference does on the host with scipy's csr_matrix
+// (script/train/train_gatconv_our.py:87-91).  Two stable radix sorts (by src, then by dst), a
+// first-of-its-group flag, an inclusive scan of the flags, and a compaction.
+
+__global__ __launch_bounds__(256) void gather_i32_kernel(int64_t n, const int *__restrict__ idx, const int *__restrict__ in, int *__restrict__ out)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = in[idx[i]];
+}
+
+// flag[q] = 1 when sorted entry q starts a new (dst, src) group (always 1 without dedupe)
+__global__ __launch_bounds__(256) void coo_flag_kernel(int64_t n, const int *__restrict__ dsts, const int *__restrict__ srcs, int dedupe, int *__restrict__ flag)
+{
+    int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (q >= n) return;
+    flag[q] = (!dedupe || q == 0 || dsts[q] != dsts[q - 1] || srcs[q] != srcs[q - 1]) ? 1 : 0;
+}
+
+#define SC_ITEMS 16
+#define SC_TILE (256 * SC_ITEMS)
+// Inclusive scan in three steps: per-tile totals, scan of the totals (one workgroup), per-tile scan + offset.
+__global__ __launch_bounds__(256) void scan_tile_sums_kernel(int64_t n, const int *__restrict__ in, int *__restrict__ sums)
+{
+    __shared__ int sh[256];
+    int64_t base = (int64_t)blockIdx.x * SC_TILE + (int64_t)threadIdx.x * SC_ITEMS;
+    int acc = 0;
+#pragma unroll
+    for (int k = 0; k < SC_ITEMS; ++k) acc += (base + k < n) ? in[base + k] : 0;
+    sh[threadIdx.x] = acc;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) sh[threadIdx.x] += sh[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) sums[blockIdx.x] = sh[0];
+}
+__global__ __launch_bounds__(256) void scan_sums_kernel(int nt, int *__restrict__ sums, int *__restrict__ total)
+{
+    __shared__ int sh[256];
+    __shared__ int carry;
+    if (threadIdx.x == 0) carry = 0;
+    __syncthreads();
+    for (int base = 0; base < nt; base += 256) {
+        int i = base + (int)threadIdx.x;
+        int v = i < nt ? sums[i] : 0;
+        sh[threadIdx.x] = v;
+        __syncthreads();
+        for (int off = 1; off < 256; off <<= 1) {
+            int t = (int)threadIdx.x >= off ? sh[threadIdx.x - off] : 0;
+            __syncthreads();
+            sh[threadIdx.x] += t;
+            __syncthreads();
+        }
+        int incl = sh[threadIdx.x];
+        int c = carry;
+        if (i < nt) sums[i] = c + incl - v;          // exclusive offset of tile i
+        __syncthreads();
+        if (threadIdx.x == 255) carry = c + incl;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *total = carry;
+}
+__global__ __launch_bounds__(256) void scan_apply_kernel(int64_t n, const int *__restrict__ in, const int *__restrict__ sums, int *__restrict__ out)
+{
+    __shared__ int sh[256];
+    int64_t base = (int64_t)blockIdx.x * SC_TILE + (int64_t)threadIdx.x * SC_ITEMS;
+    int v[SC_ITEMS];
+    int acc = 0;
+#pragma unroll
+    for (int k = 0; k < SC_ITEMS; ++k) { v[k] = (base + k < n) ? in[base + k] : 0; acc += v[k]; }
+    sh[threadIdx.x] = acc;
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {
+        int t = (int)threadIdx.x >= off ? sh[threadIdx.x - off] : 0;
+        __syncthreads();
+        sh[threadIdx.x] += t;
+        __syncthreads();
+    }
+    int run = sums[blockIdx.x] + sh[threadIdx.x] - acc;
+#pragma unroll
+    for (int k = 0; k < SC_ITEMS; ++k) {
+        run += v[k];
+        if (base + k < n) out[base + k] = run;
+    }
+}
+
+// Compaction: the first entry of every group writes its source and destination at the group's
+// position; every input edge learns the position of its group.
+__global__ __launch_bounds__(256) void coo_compact_kernel(int64_t n, const int *__restrict__ dsts, const int *__restrict__ srcs,
+                                                          const int *__restrict__ perm, const int *__restrict__ flag, const int *__restrict__ incl,
+                                                          int *__restrict__ col_ind, int *__restrict__ dstc, int *__restrict__ edge_pos)
+{
+    int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (q >= n) return;
+    int pos = incl[q] - 1;
+    if (flag[q]) { col_ind[pos] = srcs[q]; dstc[pos] = dsts[q]; }
+    if (edge_pos) edge_pos[perm[q]] = pos;
+}
+
+// row_ptr from the compacted destinations (ascending); *n_out entries are valid.
+__global__ __launch_bounds__(256) void coo_rowptr_kernel(int64_t n, int n_rows, const int *__restrict__ dstc, const int *__restrict__ n_out_dev,
+                                                         int *__restrict__ row_ptr, int64_t *__restrict__ n_out)
+{
+    int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int m = *n_out_dev;
+    if (q == 0 && n_out) *n_out = m;
+    if (q >= m) return;
+    int key = dstc[q];
+    int prev = q > 0 ? dstc[q - 1] : -1;
+    for (int r = prev + 1; r <= key; ++r) row_ptr[r] = (int)q;
+    if (q == m - 1)
+        for (int r = key + 1; r <= n_rows; ++r) row_ptr[r] = m;
+}
+
+extern "C" size_t fgnn_coo2csr_workspace_bytes(int n_rows, int n_cols, int64_t E)
+{
+    (void)n_rows; (void)n_cols;
+    size_t nt = (size_t)((E + SC_TILE - 1) / SC_TILE);
+    // sort scratch | perm1 | keys2 / srcs | perm2 | flag | incl | dstc | tile sums | total
+    return rs_sort_workspace(E) + 6 * fgnn_align256((size_t)E * sizeof(int)) + fgnn_align256((nt + 1) * sizeof(int)) + 256;
+}
+
+extern "C" int fgnn_coo2csr(int n_rows, int n_cols, int64_t E, const int32_t *dst, const int32_t *src, int dedupe, int32_t *row_ptr,
+                            int32_t *col_ind, int64_t *n_out, int32_t *edge_pos, void *workspace, size_t workspace_bytes, void *stream)
+{
+    FGNN_REQUIRE(n_rows >= 0 && n_cols >= 0 && E >= 0, FGNN_ERR_SHAPE, "fgnn_coo2csr: bad sizes");
+    FGNN_REQUIRE(E <= 2147483647LL - RS_TILE, FGNN_ERR_LIMIT, "fgnn_coo2csr: E=%lld exceeds int32 positions", (long long)E);
+    FGNN_REQUIRE(row_ptr && n_out && (E == 0 || (dst && src && col_ind)), FGNN_ERR_NULL, "fgnn_coo2csr: NULL argument");
+    hipStream_t st = (hipStream_t)stream;
+    if (E == 0) {
+        hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((n_rows + 1 + 255) / 256)), dim3(256), 0, st, row_ptr, (size_t)n_rows + 1, 0);
+        int rc = fgnn_launch_status("fill_i32_kernel");
+        if (rc) return rc;
+        hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(256), 0, st, (int *)n_out, (size_t)2, 0);    // int64 zero, as a kernel
+        return fgnn_launch_status("fill_i32_kernel");
+    }
+    FGNN_REQUIRE(n_cols >= 1 && n_rows >= 1, FGNN_ERR_SHAPE, "fgnn_coo2csr: edges without rows or columns");
+    size_t need = fgnn_coo2csr_workspace_bytes(n_rows, n_cols, E);
+    FGNN_REQUIRE(workspace && workspace_bytes >= need, FGNN_ERR_WORKSPACE, "fgnn_coo2csr: workspace %zu < %zu bytes", workspace_bytes, need);
+    char *w = (char *)workspace;
+    void *sort_ws = w; w += rs_sort_workspace(E);
+    size_t eb = fgnn_align256((size_t)E * sizeof(int));
+    int *perm1 = (int *)w; w += eb;
+    int *tmp = (int *)w; w += eb;          // dst gathered by perm1, later the sorted sources
+    int *perm2 = (int *)w; w += eb;
+    int *flag = (int *)w; w += eb;
+    int *incl = (int *)w; w += eb;
+    int *dstc = (int *)w; w += eb;
+    const int nt = (int)((E + SC_TILE - 1) / SC_TILE);
+    int *sums = (int *)w; w += fgnn_align256(((size_t)nt + 1) * sizeof(int));
+    int *total = (int *)w;
+    const unsigned ge = (unsigned)((E + 255) / 256);
+
+    const int *sorted = nullptr;
+    int rc = rs_sort_pairs(src, nullptr, E, rs_num_passes(n_cols), perm1, &sorted, sort_ws, st);
+    if (rc) return rc;
+    hipLaunchKernelGGL(gather_i32_kernel, dim3(ge), dim3(256), 0, st, E, perm1, dst, tmp);
+    rc = fgnn_launch_status("gather_i32_kernel");
+    if (rc) return rc;
+    const int *dsts = nullptr;
+    rc = rs_sort_pairs(tmp, perm1, E, rs_num_passes(n_rows), perm2, &dsts, sort_ws, st);
+    if (rc) return rc;
+    hipLaunchKernelGGL(gather_i32_kernel, dim3(ge), dim3(256), 0, st, E, perm2, src, tmp);       // sources in (dst, src) order
+    rc = fgnn_launch_status("gather_i32_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(coo_flag_kernel, dim3(ge), dim3(256), 0, st, E, dsts, tmp, dedupe, flag);
+    rc = fgnn_launch_status("coo_flag_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(scan_tile_sums_kernel, dim3(nt), dim3(256), 0, st, E, flag, sums);
+    rc = fgnn_launch_status("scan_tile_sums_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, st, nt, sums, total);
+    rc = fgnn_launch_status("scan_sums_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(scan_apply_kernel, dim3(nt), dim3(256), 0, st, E, flag, sums, incl);
+    rc = fgnn_launch_status("scan_apply_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(coo_compact_kernel, dim3(ge), dim3(256), 0, st, E, dsts, tmp, perm2, flag, incl, col_ind, dstc, edge_pos);
+    rc = fgnn_launch_status("coo_compact_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(coo_rowptr_kernel, dim3(ge), dim3(256), 0, st, E, n_rows, dstc, total, row_ptr, n_out);
+    return fgnn_launch_status("coo_rowptr_kernel");
 }

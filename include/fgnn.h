@@ -201,6 +201,17 @@ int    fgnn_csr2csc(int n_rows, int n_cols, int64_t E, const int32_t *row_ptr, c
                     int32_t *col_ptr, int32_t *row_ind, int32_t *permute,
                     void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---------------------------------------------------------------- coo2csr
+ * Edge list (dst[e], src[e]) -> CSR by destination with ascending sources inside a row; with
+ * dedupe != 0 duplicate (dst, src) pairs are merged.  Replaces the host-side scipy csr_matrix call of
+ * the reference's drivers (script/train/train_gatconv_our.py:87-91).  Outputs: row_ptr [n_rows+1],
+ * col_ind (first *n_out entries valid; capacity E), n_out (device int64: number of CSR entries),
+ * edge_pos [E] optional: CSR position of every input edge (to carry per-edge data along). */
+size_t fgnn_coo2csr_workspace_bytes(int n_rows, int n_cols, int64_t E);
+int    fgnn_coo2csr(int n_rows, int n_cols, int64_t E, const int32_t *dst, const int32_t *src, int dedupe,
+                    int32_t *row_ptr, int32_t *col_ind, int64_t *n_out, int32_t *edge_pos,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
 #pragma GCC visibility pop
 #ifdef __cplusplus
 }

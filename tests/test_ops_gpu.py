@@ -343,3 +343,39 @@ def test_knn_graph_feeds_edgeconv():
     out = EdgeConv(64, 64).to(DEV)(20, src2, h)
     out.sum().backward()
     assert out.shape == (1024, 64) and bool(torch.isfinite(out).all())
+
+
+# ------------------------------------------------------------------ coo2csr (bit-exact)
+@pytest.mark.parametrize("n,e,dedupe", [(1, 1, True), (50, 400, True), (50, 400, False), (3000, 200000, True), (70000, 500000, True), (300, 0, True)])
+def test_coo2csr_bit_exact(n, e, dedupe):
+    import scipy.sparse as sp
+    from ae_mlsys_gnn_amd.operators import csr2csc as op
+    gen = torch.Generator().manual_seed(n + e)
+    # skewed endpoints so that duplicates are common
+    dst = (torch.rand(e, generator=gen) ** 2 * n).long().clamp(max=n - 1).int()
+    src = (torch.rand(e, generator=gen) ** 3 * n).long().clamp(max=n - 1).int()
+    row_ptr, col_ind, edge_pos = op.coo2csr(dst.to(DEV), src.to(DEV), n, dedupe=dedupe, return_edge_pos=True)
+    if dedupe:       # scipy merges duplicates (script/train/train_gatconv_our.py:87-91 relies on that)
+        m = sp.csr_matrix((np.ones(e), (dst.numpy(), src.numpy())), shape=(n, n))
+        m.sum_duplicates(); m.sort_indices()
+        assert np.array_equal(row_ptr.cpu().numpy(), m.indptr) and np.array_equal(col_ind.cpu().numpy(), m.indices)
+    else:
+        order = np.lexsort((src.numpy(), dst.numpy()))
+        assert np.array_equal(col_ind.cpu().numpy(), src.numpy()[order])
+        assert np.array_equal(row_ptr.cpu().numpy(), np.concatenate([[0], np.cumsum(np.bincount(dst.numpy(), minlength=n))]))
+    if e:
+        # every input edge sits at its CSR position
+        ep = edge_pos.cpu().long()
+        rows = orc.row_of_edge(row_ptr.cpu())
+        assert torch.equal(rows[ep], dst.long()) and torch.equal(col_ind.cpu().long()[ep], src.long())
+
+
+def test_coo2csr_matches_graph_builder_at_scale():
+    from ae_mlsys_gnn_amd.operators import csr2csc as op
+    g = graphs.rmat_graph(100000, 4000000, seed=5, device=DEV)
+    dst = torch.repeat_interleave(torch.arange(g.n, device=DEV, dtype=torch.int32), (g.row_ptr[1:] - g.row_ptr[:-1]).long())
+    perm = torch.randperm(g.n_edges, device=DEV)
+    d2 = torch.cat([dst[perm], dst[perm][:1000]])          # shuffled, with 1000 duplicated edges
+    s2 = torch.cat([g.col_ind[perm], g.col_ind[perm][:1000]])
+    row_ptr, col_ind = op.coo2csr(d2, s2, g.n)
+    assert torch.equal(row_ptr, g.row_ptr) and torch.equal(col_ind, g.col_ind)

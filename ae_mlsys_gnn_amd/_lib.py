@@ -39,10 +39,10 @@ _SIGNATURES = {
     "fgnn_edgeconv_backward": (c_int, [c_int, c_int, c_int] + [c_void_p] * 3 + [c_void_p]),
     "fgnn_knn_graph": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "fgnn_gmm_forward_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int]),
-    "fgnn_gmm_forward": (c_int, [c_int, c_int64, c_int, c_int, c_int] + [c_void_p] * 9
+    "fgnn_gmm_forward": (c_int, [c_int, c_int64, c_int, c_int, c_int] + [c_void_p] * 9 + [c_int]
                          + [c_void_p, c_void_p, c_size_t, c_void_p]),
     "fgnn_gmm_backward_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int, c_int]),
-    "fgnn_gmm_backward": (c_int, [c_int, c_int64, c_int, c_int, c_int] + [c_void_p] * 12
+    "fgnn_gmm_backward": (c_int, [c_int, c_int64, c_int, c_int, c_int] + [c_void_p] * 8 + [c_int] + [c_void_p] * 4
                           + [c_void_p, c_void_p, c_size_t, c_void_p]),
     "fgnn_gaussian": (c_int, [c_int64, c_int, c_int] + [c_void_p] * 4 + [c_void_p]),
     "fgnn_gaussian_backward_workspace_bytes": (c_size_t, [c_int64, c_int, c_int]),

@@ -5,7 +5,6 @@
 #include <stdio.h>
 #include "fgnn.h"
 
-#define FGNN_WAVE 64
 #define FGNN_WPB 4      // waves per workgroup: every wave works on its own item
 #define FGNN_TPB 256
 
@@ -216,16 +215,14 @@ __device__ __forceinline__ bool fg_get_item(const fgnn_item *items, int n_items,
     return true;
 }
 
-// Weighted accumulation of up to 64 gathered feature rows (the hot loop of every SpMM-shaped
-// kernel here).  Lane t of `idv` holds the node id of edge t of the chunk (lanes >= cnt hold any
-// valid id), wl[h*64 + t] its weight for head h (0 for lanes >= cnt).  Without AUX, T accumulates
-// w * row.  With AUX the weight's sign is a flag: T accumulates |w| * row, P accumulates max(w,0) * row.  Node ids are moved to scalar registers
-// so that every row is fetched by one base-plus-lane-offset 128-bit load per slab.
-template <int VEC, int R, bool AUX, bool SUMS, bool FULL>
+// Weighted accumulation of up to 64 gathered feature rows with the weights staged in LDS (the
+// stored-weight SpMM and the GMMConv forward; the fused GAT kernels stream instead).  Lane t of
+// `idv` holds the node id of edge t of the chunk (lanes >= cnt hold any valid id), wl[h*64 + t] its
+// weight for head h (0 for lanes >= cnt).  Node ids are moved to scalar registers so that every row
+// is fetched by one base-plus-lane-offset 128-bit load per slab, 8 rows in flight.
+template <int VEC, int R, bool FULL>
 __device__ __forceinline__ void fg_accum_chunk(const float *__restrict__ feat, int HF, int idv, int cnt,
-                                               const float *wl, const fg_lanemap<VEC, R> &lm,
-                                               fg_vec<VEC> (&T)[R], fg_vec<VEC> (&P)[R],
-                                               float (&s)[R], float (&cp)[R])
+                                               const float *wl, const fg_lanemap<VEC, R> &lm, fg_vec<VEC> (&T)[R])
 {
     constexpr int U = (R >= 8) ? 1 : 8 / R;
     for (int t = 0; t < cnt; t += U) {
@@ -256,16 +253,7 @@ __device__ __forceinline__ void fg_accum_chunk(const float *__restrict__ feat, i
                 w[0] = wl[lm.hd[r] * 64 + t];
             }
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                float wa = AUX ? fabsf(w[u]) : w[u];
-                T[r].fma(wa, ld[u][r]);
-                if (AUX) {
-                    float wp = fmaxf(w[u], 0.f);
-                    P[r].fma(wp, ld[u][r]);
-                    if (SUMS) cp[r] += wp;
-                }
-                if (SUMS) s[r] += wa;
-            }
+            for (int u = 0; u < U; ++u) T[r].fma(w[u], ld[u][r]);
         }
     }
 }

@@ -15,8 +15,6 @@
 #define RS_TILE (RS_TPB * RS_ITEMS)    // 4096 elements per workgroup
 #define RS_SUB (64 * RS_ITEMS)         // 1024 per wave
 
-__device__ __forceinline__ int rs_index(int block, int wave, int it, int lane) { return block * RS_TILE + wave * RS_SUB + it * 64 + lane; }
-
 __global__ __launch_bounds__(RS_TPB) void rs_hist_kernel(const int *__restrict__ keys, int64_t n, int shift, int nblocks, int *__restrict__ hist)
 {
     __shared__ int cnt[256];

@@ -9,8 +9,35 @@ struct SpmmP {
     const int *ptr; const int *idx; const int *pos_map;
     const float *feat; float *out; float *part;
     int N, H, F, HF;
+    int sum_h;      // != 0: out is [N,F], the sum over the H heads (GMMConv's .sum(1) fused into the store)
 };
 __host__ __device__ static inline int spmm_pw(int HF) { return (HF + 3) & ~3; }
+
+// Final store of an accumulated row: either the [H,F] row itself or, with sum_h, its sum over heads.
+// scr: wave-private LDS of HF floats (only touched with sum_h).
+template <int VEC, int R, bool FULL>
+__device__ __forceinline__ void spmm_store_row(const SpmmP &p, int row, const fg_lanemap<VEC, R> &lm, fg_vec<VEC> (&T)[R], float *scr)
+{
+    if (!p.sum_h) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            if (FULL || lm.ok[r]) T[r].store(p.out + (size_t)row * p.HF + lm.eoff[r]);
+        return;
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+        if (FULL || lm.ok[r]) T[r].store(scr + lm.eoff[r]);
+    fg_wave_lds_sync();
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if ((FULL || lm.ok[r]) && lm.eoff[r] < p.F) {
+            fg_vec<VEC> acc; acc.zero();
+            for (int h = 0; h < p.H; ++h) { fg_vec<VEC> t; t.load(scr + h * p.F + lm.eoff[r]); acc.add(t); }
+            acc.store(p.out + (size_t)row * p.F + lm.eoff[r]);
+        }
+    }
+    fg_wave_lds_sync();
+}
 
 // Weight sources.  fill() runs with lanes-as-edges: lane t writes wl[h*64 + t] for every head.
 struct WAtt {
@@ -48,7 +75,7 @@ template <int VEC, int R, bool FULL, class WF>
 __global__ __launch_bounds__(FGNN_TPB) void spmm_kernel(SpmmP p, WF wf, int shared_floats)
 {
     extern __shared__ float lds[];
-    float *shared = lds + FGNN_WPB * p.H * 64;
+    float *shared = lds + FGNN_WPB * (p.H * 64 + (p.sum_h ? spmm_pw(p.HF) : 0));
     if (shared_floats > 0) {
         wf.prepare(shared, (int)threadIdx.x, p.H);
         __syncthreads();
@@ -56,13 +83,13 @@ __global__ __launch_bounds__(FGNN_TPB) void spmm_kernel(SpmmP p, WF wf, int shar
     int row, b, e, slot;
     if (!fg_get_item(p.items, p.n_items, p.ptr, row, b, e, slot)) return;
     const int lane = fg_lane();
-    float *wl = lds + fg_wave() * (p.H * 64);
+    float *wl = lds + fg_wave() * (p.H * 64 + (p.sum_h ? spmm_pw(p.HF) : 0));
+    float *scr = wl + p.H * 64;
     fg_lanemap<VEC, R> lm;
     lm.init(lane, p.HF, p.F);
-    fg_vec<VEC> T[R], P[R];
-    float s[R], cp[R];
+    fg_vec<VEC> T[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) { T[r].zero(); P[r].zero(); s[r] = 0.f; cp[r] = 0.f; }
+    for (int r = 0; r < R; ++r) T[r].zero();
     for (int c = b; c < e; c += 64) {
         int q = c + lane;
         bool ok = q < e;
@@ -72,18 +99,23 @@ __global__ __launch_bounds__(FGNN_TPB) void spmm_kernel(SpmmP p, WF wf, int shar
         size_t pos = p.pos_map ? (size_t)p.pos_map[qq] : (size_t)qq;
         wf.fill(wl, shared, lane, pos, ok, p.H);
         fg_wave_lds_sync();
-        fg_accum_chunk<VEC, R, false, false, FULL>(p.feat, p.HF, id, cnt, wl, lm, T, P, s, cp);
+        fg_accum_chunk<VEC, R, FULL>(p.feat, p.HF, id, cnt, wl, lm, T);
         fg_wave_lds_sync();
     }
-    float *dst = slot < 0 ? p.out + (size_t)row * p.HF : p.part + (size_t)slot * spmm_pw(p.HF);
+    if (slot < 0) {
+        spmm_store_row<VEC, R, FULL>(p, row, lm, T, scr);
+    } else {
+        float *dst = p.part + (size_t)slot * spmm_pw(p.HF);
 #pragma unroll
-    for (int r = 0; r < R; ++r)
-        if (FULL || lm.ok[r]) T[r].store(dst + lm.eoff[r]);
+        for (int r = 0; r < R; ++r)
+            if (FULL || lm.ok[r]) T[r].store(dst + lm.eoff[r]);
+    }
 }
 
 template <int VEC, int R>
 __global__ __launch_bounds__(FGNN_TPB) void spmm_merge_kernel(SpmmP p, const fgnn_split *split, int n_split)
 {
+    extern __shared__ float lds[];
     int w = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
     if (w >= n_split) return;
     fgnn_split sp = split[w];
@@ -91,13 +123,14 @@ __global__ __launch_bounds__(FGNN_TPB) void spmm_merge_kernel(SpmmP p, const fgn
     fg_lanemap<VEC, R> lm;
     lm.init(fg_lane(), p.HF, p.F);
     const int pw = spmm_pw(p.HF);
+    fg_vec<VEC> T[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
+        T[r].zero();
         if (!lm.ok[r]) continue;
-        fg_vec<VEC> T; T.zero();
-        for (int g = 0; g < nseg; ++g) { fg_vec<VEC> t; t.load(p.part + (size_t)(first + g) * pw + lm.eoff[r]); T.add(t); }
-        T.store(p.out + (size_t)row * p.HF + lm.eoff[r]);
+        for (int g = 0; g < nseg; ++g) { fg_vec<VEC> t; t.load(p.part + (size_t)(first + g) * pw + lm.eoff[r]); T[r].add(t); }
     }
+    spmm_store_row<VEC, R, false>(p, row, lm, T, lds + fg_wave() * pw);
 }
 
 
@@ -129,14 +162,15 @@ static int spmm_launch(const char *name, SpmmP p, WF wf, int shared_floats, cons
     }
     if (p.n_items == 0) return 0;
     const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
-    const size_t shm = ((size_t)FGNN_WPB * p.H * 64 + shared_floats) * sizeof(float);
+    const size_t shm = ((size_t)FGNN_WPB * (p.H * 64 + (p.sum_h ? spmm_pw(p.HF) : 0)) + shared_floats) * sizeof(float);
+    const size_t shm_merge = p.sum_h ? (size_t)FGNN_WPB * spmm_pw(p.HF) * sizeof(float) : 0;
     return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
         hipLaunchKernelGGL((spmm_kernel<VEC, R, FULL, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
         int rc = fgnn_launch_status(name);
         if (rc) return rc;
         if (sched && sched->n_split > 0) {
             unsigned g2 = (unsigned)((sched->n_split + FGNN_WPB - 1) / FGNN_WPB);
-            hipLaunchKernelGGL((spmm_merge_kernel<VEC, R>), dim3(g2), dim3(FGNN_TPB), 0, st, p, sched->split_dev, sched->n_split);
+            hipLaunchKernelGGL((spmm_merge_kernel<VEC, R>), dim3(g2), dim3(FGNN_TPB), shm_merge, st, p, sched->split_dev, sched->n_split);
             return fgnn_launch_status("spmm_merge_kernel");
         }
         return 0;
@@ -168,8 +202,8 @@ extern "C" size_t fgnn_gmm_forward_workspace_bytes(const fgnn_schedule_t *sched,
 
 extern "C" int fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F, const int32_t *ptr, const int32_t *idx,
                                 const int32_t *pos_map, const float *node_feat, const float *pseudo, const float *mu,
-                                const float *inv_sigma, float *out, float *gauss_out, const fgnn_schedule_t *sched,
-                                void *workspace, size_t workspace_bytes, void *stream)
+                                const float *inv_sigma, float *out, float *gauss_out, int sum_kernels,
+                                const fgnn_schedule_t *sched, void *workspace, size_t workspace_bytes, void *stream)
 {
     int rc = spmm_checks("fgnn_gmm_forward", N, E, K, F, sched, ptr);
     if (rc) return rc;
@@ -177,6 +211,7 @@ extern "C" int fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F, const i
     FGNN_REQUIRE(ptr && (idx || E == 0) && node_feat && (pseudo || E == 0) && mu && inv_sigma && out, FGNN_ERR_NULL, "fgnn_gmm_forward: NULL argument");
     SpmmP p{};
     p.ptr = ptr; p.idx = idx; p.pos_map = pos_map; p.feat = node_feat; p.out = out; p.N = N; p.H = K; p.F = F; p.HF = K * F;
+    p.sum_h = sum_kernels;
     WGauss wf{pseudo, mu, inv_sigma, gauss_out, dim};
     return spmm_launch("fgnn_gmm_forward", p, wf, 2 * K * dim, sched, fgnn_aligned16(node_feat) && fgnn_aligned16(out), workspace,
                        workspace_bytes, (hipStream_t)stream);
@@ -189,6 +224,7 @@ struct GmmBwdP {
     const float *x; const float *g; const float *pseudo; const float *mu; const float *isg;
     float *gfeat; float *gww; float *part;      // gww: [E,K] in CSR position order, gw * w per edge and kernel
     int N, K, dim, F, HF;
+    int g_stride;   // floats per grad_out row: HF, or F when grad_out is the gradient of the sum over kernels
 };
 
 // One pass over CSC column j (x[j] stays in registers): per in-edge gather grad_out[i], accumulate
@@ -212,10 +248,12 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p)
     fg_lanemap<VEC, R> lm;
     lm.init(lane, p.HF, p.F);
     fg_vec<VEC> T[R], xr[R];
+    int goff[R];        // float offset of the lane's slab inside a grad_out row
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         T[r].zero();
         if (FULL || lm.ok[r]) xr[r].load(p.x + (size_t)col * p.HF + lm.eoff[r]); else xr[r].zero();
+        goff[r] = (p.g_stride == p.HF) ? lm.eoff[r] : lm.eoff[r] % p.F;
     }
     for (int c = b; c < e; c += 64) {
         int q = c + lane;
@@ -240,9 +278,9 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p)
 #pragma unroll
             for (int u = 0; u < UG; ++u) {
                 int rid = __builtin_amdgcn_readlane(id, t + u);
-                const float *base = p.g + (size_t)rid * p.HF;
+                const float *base = p.g + (size_t)rid * p.g_stride;
 #pragma unroll
-                for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ld[u][r].load(base + lm.eoff[r]); else ld[u][r].zero(); }
+                for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ld[u][r].load(base + goff[r]); else ld[u][r].zero(); }
             }
 #pragma unroll
             for (int u = 0; u < UG; ++u) {
@@ -407,7 +445,7 @@ extern "C" size_t fgnn_gmm_backward_workspace_bytes(const fgnn_schedule_t *sched
 
 extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const int32_t *col_ptr, const int32_t *row_ind,
                                  const int32_t *permute, const float *node_feat, const float *pseudo, const float *mu,
-                                 const float *inv_sigma, const float *grad_out, float *grad_feat, float *grad_pseudo,
+                                 const float *inv_sigma, const float *grad_out, int sum_kernels, float *grad_feat, float *grad_pseudo,
                                  float *grad_mu, float *grad_sigma, const fgnn_schedule_t *sched_csc, void *workspace,
                                  size_t workspace_bytes, void *stream)
 {
@@ -434,7 +472,7 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
         GmmBwdP p{};
         p.items = sched_csc->items_dev; p.n_items = sched_csc->n_items; p.ptr = col_ptr; p.idx = row_ind; p.permute = permute;
         p.x = node_feat; p.g = grad_out; p.pseudo = pseudo; p.mu = mu; p.isg = inv_sigma; p.gfeat = grad_feat; p.gww = gww;
-        p.part = part; p.N = N; p.K = K; p.dim = dim; p.F = F; p.HF = HF;
+        p.part = part; p.N = N; p.K = K; p.dim = dim; p.F = F; p.HF = HF; p.g_stride = sum_kernels ? F : HF;
         const int lph = fgnn_pick_lph(cfg.vec, F);
         const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
         rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {

@@ -6,11 +6,11 @@ import torch as th
 from torch import nn
 from torch.nn import init
 
-from ..operators.fused_gmmconv import GmmConvFuse, GmmConvStash
+from ..operators.fused_gmmconv import GmmConvFuseSum, GmmConvStash
 
 
 class _GMMBase(nn.Module):
-    _op = None
+    _op = None          # callable(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, inv_sigma) -> [N, F]
 
     def __init__(self, in_feats, out_feats, dim, n_kernels, aggregator_type="sum", residual=False, bias=True,
                  allow_zero_in_degree=False):
@@ -50,7 +50,7 @@ class _GMMBase(nn.Module):
 
     def forward(self, rowptr, colind, colptr, rowind, permute, feat, pseudo):
         node_feat = self.fc(feat).view(-1, self._n_kernels, self._out_feats)
-        rst = type(self)._op(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, self.mu, self.inv_sigma).sum(1)
+        rst = type(self)._op(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, self.mu, self.inv_sigma)
         if self.res_fc is not None:
             rst = rst + self.res_fc(feat)
         if self.bias is not None:
@@ -59,8 +59,14 @@ class _GMMBase(nn.Module):
 
 
 class GMMConv(_GMMBase):
-    _op = staticmethod(GmmConvFuse)
+    """The `.sum(1)` over the mixture kernels of the reference layer (layers/gmmconv_layer.py:69) is
+    fused into the operator."""
+    _op = staticmethod(GmmConvFuseSum)
+
+
+def _stash_sum(*args):
+    return GmmConvStash(*args).sum(1)
 
 
 class GMMConv_stash(_GMMBase):
-    _op = staticmethod(GmmConvStash)
+    _op = staticmethod(_stash_sum)

@@ -5,7 +5,7 @@ from .edge_softmax import EdgeSoftmaxFunction, csr_edge_softmax  # noqa: F401
 from .fused_edgeconv import FusedEdgeConvFunction, fused_edgeconv_op  # noqa: F401
 from .fused_gat import (FusedGATFunction, FusedGATFunction_SM, FusedGATFunction_stash,  # noqa: F401
                         fused_gat_fusescatter, fused_gat_op, fused_gat_stash_op)
-from .fused_gmmconv import (GaussianCp, GaussianFunction, GmmConvFuse, GmmConvFuseEb, GmmConvStash,  # noqa: F401
+from .fused_gmmconv import (GaussianCp, GaussianFunction, GmmConvFuse, GmmConvFuseEb, GmmConvFuseSum, GmmConvStash,  # noqa: F401
                             GmmFuseEbFunction, GmmFuseFunction, GmmStashFunction)
 from .knn import knn_graph  # noqa: F401
 from .mhspmm import MHSPMMFunction, csrmhspmm, mhsddmm, mhtranspose  # noqa: F401

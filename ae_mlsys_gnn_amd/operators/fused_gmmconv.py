@@ -13,7 +13,7 @@ class gmm_native:
     """gmmconv.gmmconv / gmmconvstash / Gaussian / GaussianBp (src/fused_gmmconv/gmmconv.cc:36-94)."""
 
     @staticmethod
-    def gmmconv(rowptr, colind, node_feat, pseudo, mu, sigma, *, pos_map=None, want_gauss=False):
+    def gmmconv(rowptr, colind, node_feat, pseudo, mu, sigma, *, pos_map=None, want_gauss=False, sum_kernels=False):
         require_cuda(rowptr, colind, node_feat, pseudo, mu, sigma)
         rowptr, colind = as_i32(rowptr), as_i32(colind)
         node_feat, pseudo, mu, sigma = as_f32(node_feat), as_f32(pseudo), as_f32(mu), as_f32(sigma)
@@ -25,18 +25,18 @@ class gmm_native:
         if mu.shape != (k, dim) or sigma.shape != (k, dim) or pseudo.shape != (e, dim) or rowptr.numel() != n + 1:
             raise FgnnError("gmmconv: shape mismatch mu %s sigma %s pseudo %s for K=%d E=%d" % (
                 tuple(mu.shape), tuple(sigma.shape), tuple(pseudo.shape), k, e))
-        out = torch.empty_like(node_feat)
+        out = torch.empty((n, f), dtype=torch.float32, device=node_feat.device) if sum_kernels else torch.empty_like(node_feat)
         gauss = torch.empty((e, k), dtype=torch.float32, device=node_feat.device) if want_gauss else None
         sched = schedule_for(rowptr)
         with torch.cuda.device(node_feat.device):
             ws, wsb = workspace(lib().fgnn_gmm_forward_workspace_bytes(sched.handle, k, f), node_feat.device)
             check(lib().fgnn_gmm_forward(n, e, k, dim, f, ptr(rowptr), ptr(colind), ptr(pos_map), ptr(node_feat), ptr(pseudo),
-                                         ptr(mu), ptr(sigma), ptr(out), ptr(gauss), sched.handle, ptr(ws), wsb, stream_ptr()),
+                                         ptr(mu), ptr(sigma), ptr(out), ptr(gauss), int(sum_kernels), sched.handle, ptr(ws), wsb, stream_ptr()),
                   "fgnn_gmm_forward")
         return (out, gauss) if want_gauss else out
 
     @staticmethod
-    def gmmconv_backward(colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out):
+    def gmmconv_backward(colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out, sum_kernels=False):
         require_cuda(colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out)
         colptr, rowind, permute = as_i32(colptr), as_i32(rowind), as_i32(permute)
         grad_out = as_f32(grad_out)
@@ -52,7 +52,7 @@ class gmm_native:
         with torch.cuda.device(dev):
             ws, wsb = workspace(lib().fgnn_gmm_backward_workspace_bytes(sched.handle, k, dim, f), dev)
             check(lib().fgnn_gmm_backward(n, e, k, dim, f, ptr(colptr), ptr(rowind), ptr(permute), ptr(node_feat), ptr(pseudo),
-                                          ptr(mu), ptr(sigma), ptr(grad_out), ptr(grad_feat), ptr(grad_pseudo), ptr(grad_mu),
+                                          ptr(mu), ptr(sigma), ptr(grad_out), int(sum_kernels), ptr(grad_feat), ptr(grad_pseudo), ptr(grad_mu),
                                           ptr(grad_sigma), sched.handle, ptr(ws), wsb, stream_ptr()), "fgnn_gmm_backward")
         return grad_feat, grad_pseudo, grad_mu, grad_sigma
 
@@ -99,6 +99,27 @@ class GmmFuseFunction(torch.autograd.Function):
         rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma = ctx.saved_tensors
         grad_feat, grad_pseudo, grad_mu, grad_sigma = gmm_native.gmmconv_backward(
             colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out.contiguous())
+        return None, None, None, None, None, grad_feat, grad_pseudo, grad_mu, grad_sigma
+
+
+def GmmConvFuseSum(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma):
+    """GmmConvFuse(...).sum(1) as one operator: the sum over the K mixture kernels is fused into the
+    forward's store and the backward gathers [N,F] gradient rows.  Returns [N,F]."""
+    return GmmFuseSumFunction.apply(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma)
+
+
+class GmmFuseSumFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma):
+        out = gmm_native.gmmconv(rowptr, colind, node_feat, pseudo, mu, sigma, sum_kernels=True)      # [N, F]
+        ctx.save_for_backward(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma = ctx.saved_tensors
+        grad_feat, grad_pseudo, grad_mu, grad_sigma = gmm_native.gmmconv_backward(
+            colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out.contiguous(), sum_kernels=True)
         return None, None, None, None, None, grad_feat, grad_pseudo, grad_mu, grad_sigma
 
 

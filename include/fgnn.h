@@ -127,12 +127,14 @@ int fgnn_knn_graph(int n_clouds, int P, int D, int k, const float *points, int32
  *   out[i,k,:] = sum_p w[p,k] * node_feat[col_ind[p],k,:].
  * pseudo [E,dim] is in the position order of (ptr, idx); when pos_map is non-NULL the row
  * pseudo[pos_map[p]] is used instead (lets a CSC pass read CSR-ordered pseudo without the
- * mhtranspose copy of operators/fused_gmmconv.py:55).  gauss_out [E,K] optional. */
+ * mhtranspose copy of operators/fused_gmmconv.py:55).  gauss_out [E,K] optional.
+ * sum_kernels != 0 fuses the layer's `.sum(1)` (layers/gmmconv_layer.py:69) into the store:
+ * out is then [N,F] = sum_k out[i,k,:]. */
 size_t fgnn_gmm_forward_workspace_bytes(const fgnn_schedule_t *sched, int K, int F);
 int    fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F,
                         const int32_t *ptr, const int32_t *idx, const int32_t *pos_map,
                         const float *node_feat, const float *pseudo, const float *mu,
-                        const float *inv_sigma, float *out, float *gauss_out,
+                        const float *inv_sigma, float *out, float *gauss_out, int sum_kernels,
                         const fgnn_schedule_t *sched, void *workspace, size_t workspace_bytes,
                         void *stream);
 
@@ -143,10 +145,12 @@ int    fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F,
  * Gaussian derivatives, grad_mu / grad_sigma reduced in a fixed order (bit-reproducible).
  * A schedule of col_ptr is required. */
 size_t fgnn_gmm_backward_workspace_bytes(const fgnn_schedule_t *sched_csc, int K, int dim, int F);
+/* sum_kernels != 0: grad_out is [N,F], the gradient of the fused sum over kernels (every kernel of a
+ * node sees the same row, so the pass gathers F instead of K*F floats per edge). */
 int    fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F,
                          const int32_t *col_ptr, const int32_t *row_ind, const int32_t *permute,
                          const float *node_feat, const float *pseudo, const float *mu,
-                         const float *inv_sigma, const float *grad_out,
+                         const float *inv_sigma, const float *grad_out, int sum_kernels,
                          float *grad_feat, float *grad_pseudo, float *grad_mu, float *grad_sigma,
                          const fgnn_schedule_t *sched_csc, void *workspace, size_t workspace_bytes,
                          void *stream);

@@ -132,7 +132,8 @@ def _gmm_case(g, k, dim, f, seed):
 
 
 @pytest.mark.parametrize("k,dim,f,variant", [(3, 2, 64, "fuse"), (2, 1, 16, "fuse"), (3, 2, 64, "stash"), (1, 3, 47, "fuse"),
-                                              (4, 2, 33, "eb"), (3, 2, 128, "fuse")])
+                                              (4, 2, 33, "eb"), (3, 2, 128, "fuse"), (3, 2, 64, "sum"), (2, 3, 20, "sum"),
+                                              (5, 2, 33, "sum")])
 def test_gmm_forward_backward(k, dim, f, variant, monkeypatch):
     from ae_mlsys_gnn_amd.operators import fused_gmmconv as fg
     from ae_mlsys_gnn_amd import _lib
@@ -145,11 +146,17 @@ def test_gmm_forward_backward(k, dim, f, variant, monkeypatch):
     ref.backward(go)
     gd = g.to(DEV)
     dl = [t.float().to(DEV).requires_grad_(True) for t in (x, pseudo, mu, isg)]
-    op = {"fuse": fg.GmmConvFuse, "stash": fg.GmmConvStash, "eb": fg.GmmConvFuseEb}[variant]
+    op = {"fuse": fg.GmmConvFuse, "stash": fg.GmmConvStash, "eb": fg.GmmConvFuseEb, "sum": fg.GmmConvFuseSum}[variant]
     out = op(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, *dl)
+    if variant == "sum":      # the sum over kernels fused into the operator: same gradients as summing outside
+        for t in leaves:
+            t.grad = None
+        ref = orc.gmm_forward(g.row_ptr, g.col_ind, *leaves).sum(1)
+        go = go[:, 0, :].contiguous()
+        ref.backward(go)
     out.backward(go.float().to(DEV))
     _lib.clear_schedule_cache()
-    assert_close(out, ref.detach(), "gmm out")
+    assert_close(out, ref.detach(), "gmm out", atol=1e-4 if variant == "sum" else 1e-5)
     assert_close(dl[0].grad, leaves[0].grad, "grad node_feat")
     assert_close(dl[1].grad, leaves[1].grad, "grad pseudo", atol=1e-4)
     # sums over all E edges: absolute bar scales with the number of summands

@@ -65,7 +65,12 @@ struct fgnn_schedule {
     int n_buckets;
     const int32_t *idx_src_dev;
     int32_t *bidx_dev;
+    int32_t *bpos_dev;      // original position of every bucket-ordered entry (for per-edge arrays)
 };
+// The index array a kernel walks under schedule `s`, and the map from its positions back to the
+// caller's edge positions (NULL = identity).
+static inline const int32_t *fgnn_sched_idx(const fgnn_schedule *s, const int32_t *idx) { return (s && s->n_buckets > 0) ? s->bidx_dev : idx; }
+static inline const int32_t *fgnn_sched_pos(const fgnn_schedule *s) { return (s && s->n_buckets > 0) ? s->bpos_dev : nullptr; }
 
 #define FGNN_NUM_XCD 8      // workgroup w of a dispatch runs on XCD w % 8 (gfx942 / gfx950, SPX mode)
 // Source bucket of a node id: the top 3 bits of a multiplicative hash, so hot ids spread evenly.

@@ -23,7 +23,7 @@
 
 struct GatFwdP {
     const fgnn_item *items; int n_items;
-    const int *ptr; const int *idx;
+    const int *ptr; const int *idx; const int *pos;     // pos: caller's edge position of entry q of idx (NULL = q)
     const float *ar; const float *ac; const float *x;
     float *out; float *emax; float *esum; float *out2; float *cc;
     float *part;
@@ -239,20 +239,21 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_edge_stash_kernel(GatFwdP p, flo
     const int H = p.H;
     const int64_t lo = (int64_t)b * H, hi = (int64_t)e * H;
     for (int64_t k = lo + lane; k < hi; k += 64) {
-        int64_t pos = k / H;
-        int h = (int)(k - pos * H);
-        int j = p.idx[pos];
+        int64_t q = k / H;
+        int h = (int)(k - q * H);
+        int j = p.idx[q];
+        int64_t o = (p.pos ? (int64_t)p.pos[q] : q) * H + h;      // the caller's edge position
         float ev = fg_lrelu(p.ar[(size_t)row * H + h] + p.ac[(size_t)j * H + h], p.slope);
         float m = p.emax[(size_t)row * H + h], s = p.esum[(size_t)row * H + h];
-        e_lrelu[k] = ev;
-        e_softmax[k] = __expf(ev - m) / s;
+        e_lrelu[o] = ev;
+        e_softmax[o] = __expf(ev - m) / s;
     }
 }
 
 // ------------------------------------------------------------------------------- backward
 struct GatBwdP {
     const fgnn_item *items; int n_items;
-    const int *ptr; const int *idx; const int *permute;
+    const int *ptr; const int *idx; const int *pos; const int *permute;
     const float4 *rec;
     const float *ac; const float *x; const float *g;
     const float *esm; const float *erelu;
@@ -399,7 +400,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_kernel(GatBwdP p)
         int cnt = min(64, e - c);
         int qq = q < e ? q : c;
         int idv = p.idx[qq];
-        int posv = STASH ? p.permute[qq] : 0;
+        int posv = STASH ? p.permute[p.pos ? p.pos[qq] : qq] : 0;
         int t = 0;
         for (; t + U <= cnt; t += U) gat_bwd_batch<VEC, R, STASH, FULL, U, false, SLE1>(p, lm, boff, roff, hoff, idv, posv, t, cnt, ach, z, T, P);
         if constexpr (U >= 4) {
@@ -459,21 +460,17 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_merge_kernel(GatBwdP p, cons
 
 // ------------------------------------------------------------------------------- host
 
-// idx: the index array the operator was given; positional: the call reads or writes per-edge arrays
-// in the caller's position order, which a bucket-ordered schedule cannot serve
-static int check_sched(const fgnn_schedule_t *s, const int32_t *ptr, const int32_t *idx, bool positional, int n, int64_t E, const char *what)
+// idx: the index array the operator was given (an XCD-aware schedule must have been built from it)
+static int check_sched(const fgnn_schedule_t *s, const int32_t *ptr, const int32_t *idx, int n, int64_t E, const char *what)
 {
     if (!s) return 0;
     FGNN_REQUIRE(s->ptr_dev == ptr && s->n_rows == n && s->n_edges == E, FGNN_ERR_SCHEDULE,
                  "%s: schedule was built for another pointer array (n_rows %d vs %d, edges %lld vs %lld)", what,
                  s->n_rows, n, (long long)s->n_edges, (long long)E);
-    if (s->n_buckets > 0) {
+    if (s->n_buckets > 0)
         FGNN_REQUIRE(s->idx_src_dev == idx, FGNN_ERR_SCHEDULE, "%s: XCD-aware schedule was built from another index array", what);
-        FGNN_REQUIRE(!positional, FGNN_ERR_SCHEDULE, "%s: an XCD-aware schedule cannot be used with per-edge (stashed) arrays", what);
-    }
     return 0;
 }
-static inline const int32_t *sched_idx(const fgnn_schedule_t *s, const int32_t *idx) { return (s && s->n_buckets > 0) ? s->bidx_dev : idx; }
 
 static int gat_common_checks(const char *fn, int N, int64_t E, int H, int F)
 {
@@ -504,7 +501,7 @@ static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_
     GatFwdP p;
     p.items = sched ? sched->items_dev : nullptr;
     p.n_items = sched ? sched->n_items : N;
-    p.ptr = row_ptr; p.idx = sched_idx(sched, col_ind); p.ar = attn_row; p.ac = attn_col; p.x = in_feat;
+    p.ptr = row_ptr; p.idx = fgnn_sched_idx(sched, col_ind); p.pos = fgnn_sched_pos(sched); p.ar = attn_row; p.ac = attn_col; p.x = in_feat;
     p.out = out; p.emax = edge_max; p.esum = edge_sum; p.out2 = aux_out2; p.cc = aux_c;
     p.part = (float *)workspace; p.N = N; p.H = H; p.F = F; p.HF = HF; p.slope = slope;
     if (sched && sched->n_partials > 0) {
@@ -550,7 +547,7 @@ extern "C" int fgnn_gat_forward(int N, int64_t E, int H, int F, const float *att
                  FGNN_ERR_NULL, "fgnn_gat_forward: NULL argument");
     FGNN_REQUIRE((aux_out2 == nullptr) == (aux_c == nullptr), FGNN_ERR_NULL, "fgnn_gat_forward: aux_out2 and aux_c go together");
     FGNN_REQUIRE((e_lrelu == nullptr) == (e_softmax == nullptr), FGNN_ERR_NULL, "fgnn_gat_forward: e_lrelu and e_softmax go together");
-    rc = check_sched(sched, row_ptr, col_ind, e_lrelu != nullptr, N, E, "fgnn_gat_forward");
+    rc = check_sched(sched, row_ptr, col_ind, N, E, "fgnn_gat_forward");
     if (rc) return rc;
     return gat_forward_launch(N, E, H, F, attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, out, edge_max,
                               edge_sum, aux_out2, aux_c, e_lrelu, e_softmax, sched, workspace, workspace_bytes, (hipStream_t)stream);
@@ -589,9 +586,9 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
     FGNN_REQUIRE(!stash || (permute && e_lrelu), FGNN_ERR_NULL, "fgnn_gat_backward: stashed attention needs permute, e_lrelu and e_softmax");
     const bool recompute = !(out_feat && aux_out2 && aux_c);
     FGNN_REQUIRE(!recompute || (row_ptr && (col_ind || E == 0)), FGNN_ERR_NULL, "fgnn_gat_backward: recomputing the forward needs row_ptr/col_ind");
-    rc = check_sched(sched_csc, col_ptr, row_ind, stash, N, E, "fgnn_gat_backward(csc)");
+    rc = check_sched(sched_csc, col_ptr, row_ind, N, E, "fgnn_gat_backward(csc)");
     if (rc) return rc;
-    if (recompute) { rc = check_sched(sched_csr, row_ptr, col_ind, false, N, E, "fgnn_gat_backward(csr)"); if (rc) return rc; }
+    if (recompute) { rc = check_sched(sched_csr, row_ptr, col_ind, N, E, "fgnn_gat_backward(csr)"); if (rc) return rc; }
     size_t need = fgnn_gat_backward_workspace_bytes(N, H, F, sched_csc, recompute ? sched_csr : nullptr, recompute);
     FGNN_REQUIRE(workspace && workspace_bytes >= need, FGNN_ERR_WORKSPACE, "fgnn_gat_backward: workspace %zu < %zu bytes", workspace_bytes, need);
     FGNN_REQUIRE(fgnn_aligned16(workspace), FGNN_ERR_ALIGN, "fgnn_gat_backward: workspace not 16-byte aligned");
@@ -620,7 +617,7 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
     GatBwdP p;
     p.items = sched_csc ? sched_csc->items_dev : nullptr;
     p.n_items = sched_csc ? sched_csc->n_items : N;
-    p.ptr = col_ptr; p.idx = sched_idx(sched_csc, row_ind); p.permute = permute; p.rec = rec; p.ac = attn_col; p.x = in_feat; p.g = grad_out;
+    p.ptr = col_ptr; p.idx = fgnn_sched_idx(sched_csc, row_ind); p.pos = fgnn_sched_pos(sched_csc); p.permute = permute; p.rec = rec; p.ac = attn_col; p.x = in_feat; p.g = grad_out;
     p.esm = e_softmax; p.erelu = e_lrelu; p.gfeat = grad_feat; p.gac = grad_attn_col; p.part = part;
     p.N = N; p.H = H; p.F = F; p.HF = HF; p.slope = negative_slope;
 

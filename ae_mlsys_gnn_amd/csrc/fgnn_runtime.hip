@@ -20,9 +20,9 @@ extern "C" int fgnn_version(void) { return 100; }
 
 // Per row: stable partition of the row's index entries by source bucket.  One wave per row; pass 1
 // counts the buckets (ballots), pass 2 places every entry at its bucket's running offset.  Writes
-// the permuted index array and the per-(row, bucket) counts.
+// the permuted index array, the original position of every entry and the per-(row, bucket) counts.
 __global__ __launch_bounds__(FGNN_TPB) void bucket_partition_kernel(int n_rows, const int *__restrict__ ptr, const int *__restrict__ idx,
-                                                                    int *__restrict__ bidx, int *__restrict__ bcnt)
+                                                                    int *__restrict__ bidx, int *__restrict__ bpos, int *__restrict__ bcnt)
 {
     int row = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
     if (row >= n_rows) return;
@@ -61,7 +61,7 @@ __global__ __launch_bounds__(FGNN_TPB) void bucket_partition_kernel(int n_rows, 
             if (bk == b) dst = off[b] + __popcll(m & lt);
             off[b] += __popcll(m);
         }
-        if (ok) bidx[dst] = id;
+        if (ok) { bidx[dst] = id; bpos[dst] = q; }
     }
 }
 
@@ -112,7 +112,7 @@ static fgnn_schedule *new_schedule(const int32_t *ptr_dev, int n_rows, int64_t n
     s->n_rows = n_rows; s->n_edges = n_edges; s->seg_len = seg_len;
     s->n_items = s->n_partials = s->n_split = 0;
     s->items_dev = nullptr; s->split_dev = nullptr; s->ptr_dev = ptr_dev;
-    s->n_buckets = 0; s->idx_src_dev = nullptr; s->bidx_dev = nullptr;
+    s->n_buckets = 0; s->idx_src_dev = nullptr; s->bidx_dev = nullptr; s->bpos_dev = nullptr;
     (void)hipGetDevice(&s->device);
     return s;
 }
@@ -186,9 +186,10 @@ extern "C" int fgnn_schedule_create_bucketed(const int32_t *ptr_dev, const int32
         int32_t *bcnt_dev = nullptr;
         hipError_t err = hipMalloc((void **)&bcnt_dev, bcnt.size() * sizeof(int32_t));
         if (err == hipSuccess && n_edges > 0) err = hipMalloc((void **)&s->bidx_dev, (size_t)n_edges * sizeof(int32_t));
+        if (err == hipSuccess && n_edges > 0) err = hipMalloc((void **)&s->bpos_dev, (size_t)n_edges * sizeof(int32_t));
         if (err == hipSuccess) {
             hipLaunchKernelGGL(bucket_partition_kernel, dim3((unsigned)((n_rows + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, st,
-                               n_rows, ptr_dev, idx_dev, s->bidx_dev, bcnt_dev);
+                               n_rows, ptr_dev, idx_dev, s->bidx_dev, s->bpos_dev, bcnt_dev);
             err = hipGetLastError();
         }
         if (err == hipSuccess) err = hipMemcpyAsync(bcnt.data(), bcnt_dev, bcnt.size() * sizeof(int32_t), hipMemcpyDeviceToHost, st);
@@ -258,6 +259,7 @@ extern "C" void fgnn_schedule_destroy(fgnn_schedule_t *s)
     if (s->items_dev) (void)hipFree(s->items_dev);
     if (s->split_dev) (void)hipFree(s->split_dev);
     if (s->bidx_dev) (void)hipFree(s->bidx_dev);
+    if (s->bpos_dev) (void)hipFree(s->bpos_dev);
     delete s;
 }
 

@@ -6,7 +6,8 @@
 
 struct SpmmP {
     const fgnn_item *items; int n_items;
-    const int *ptr; const int *idx; const int *pos_map;
+    const int *ptr; const int *idx; const int *pos;      // pos: caller's edge position of entry q of idx (NULL = q)
+    const int *pos_map;
     const float *feat; float *out; float *part;
     int N, H, F, HF;
     int sum_h;      // != 0: out is [N,F], the sum over the H heads (GMMConv's .sum(1) fused into the store)
@@ -96,7 +97,8 @@ __global__ __launch_bounds__(FGNN_TPB) void spmm_kernel(SpmmP p, WF wf, int shar
         int cnt = min(64, e - c);
         int qq = ok ? q : c;
         int id = p.idx[qq];
-        size_t pos = p.pos_map ? (size_t)p.pos_map[qq] : (size_t)qq;
+        int orig = p.pos ? p.pos[qq] : qq;
+        size_t pos = p.pos_map ? (size_t)p.pos_map[orig] : (size_t)orig;
         wf.fill(wl, shared, lane, pos, ok, p.H);
         fg_wave_lds_sync();
         fg_accum_chunk<VEC, R, FULL>(p.feat, p.HF, id, cnt, wl, lm, T);
@@ -134,7 +136,7 @@ __global__ __launch_bounds__(FGNN_TPB) void spmm_merge_kernel(SpmmP p, const fgn
 }
 
 
-static int spmm_checks(const char *fn, int N, int64_t E, int H, int F, const fgnn_schedule_t *sched, const int32_t *ptr)
+static int spmm_checks(const char *fn, int N, int64_t E, int H, int F, const fgnn_schedule_t *sched, const int32_t *ptr, const int32_t *idx)
 {
     FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1 && F >= 1, FGNN_ERR_SHAPE, "%s: bad sizes N=%d E=%lld H=%d F=%d", fn, N, (long long)E, H, F);
     FGNN_REQUIRE(E <= 2147483647LL, FGNN_ERR_LIMIT, "%s: E=%lld exceeds int32 positions", fn, (long long)E);
@@ -142,7 +144,8 @@ static int spmm_checks(const char *fn, int N, int64_t E, int H, int F, const fgn
     if (sched) {
         FGNN_REQUIRE(sched->ptr_dev == ptr && sched->n_rows == N && sched->n_edges == E, FGNN_ERR_SCHEDULE,
                      "%s: schedule was built for another pointer array", fn);
-        FGNN_REQUIRE(sched->n_buckets == 0, FGNN_ERR_SCHEDULE, "%s: an XCD-aware schedule cannot be used with per-edge arrays", fn);
+        FGNN_REQUIRE(sched->n_buckets == 0 || sched->idx_src_dev == idx, FGNN_ERR_SCHEDULE,
+                     "%s: XCD-aware schedule was built from another index array", fn);
     }
     return 0;
 }
@@ -155,6 +158,8 @@ static int spmm_launch(const char *name, SpmmP p, WF wf, int shared_floats, cons
     FGNN_REQUIRE(fgnn_pick_rowcfg(p.HF, p.F, aligned && fgnn_aligned16(workspace), &cfg), FGNN_ERR_LIMIT, "%s: unsupported row width %d", name, p.HF);
     p.items = sched ? sched->items_dev : nullptr;
     p.n_items = sched ? sched->n_items : p.N;
+    p.idx = fgnn_sched_idx(sched, p.idx);
+    p.pos = fgnn_sched_pos(sched);
     p.part = (float *)workspace;
     if (sched && sched->n_partials > 0) {
         size_t need = (size_t)sched->n_partials * spmm_pw(p.HF) * sizeof(float);
@@ -186,7 +191,7 @@ extern "C" int fgnn_mhspmm(int N, int64_t E, int H, int F, const int32_t *ptr, c
                            const float *att, const float *feat, float *out, const fgnn_schedule_t *sched, void *workspace,
                            size_t workspace_bytes, void *stream)
 {
-    int rc = spmm_checks("fgnn_mhspmm", N, E, H, F, sched, ptr);
+    int rc = spmm_checks("fgnn_mhspmm", N, E, H, F, sched, ptr, idx);
     if (rc) return rc;
     FGNN_REQUIRE(ptr && (idx || E == 0) && feat && out, FGNN_ERR_NULL, "fgnn_mhspmm: NULL argument");
     SpmmP p{};
@@ -205,7 +210,7 @@ extern "C" int fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F, const i
                                 const float *inv_sigma, float *out, float *gauss_out, int sum_kernels,
                                 const fgnn_schedule_t *sched, void *workspace, size_t workspace_bytes, void *stream)
 {
-    int rc = spmm_checks("fgnn_gmm_forward", N, E, K, F, sched, ptr);
+    int rc = spmm_checks("fgnn_gmm_forward", N, E, K, F, sched, ptr, idx);
     if (rc) return rc;
     FGNN_REQUIRE(dim >= 1 && dim <= 64 && K * dim <= 1024, FGNN_ERR_LIMIT, "fgnn_gmm_forward: dim=%d K*dim=%d unsupported", dim, K * dim);
     FGNN_REQUIRE(ptr && (idx || E == 0) && node_feat && (pseudo || E == 0) && mu && inv_sigma && out, FGNN_ERR_NULL, "fgnn_gmm_forward: NULL argument");
@@ -220,7 +225,7 @@ extern "C" int fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F, const i
 // ------------------------------------------------------------------------------- GMM backward
 struct GmmBwdP {
     const fgnn_item *items; int n_items;
-    const int *ptr; const int *idx; const int *permute;
+    const int *ptr; const int *idx; const int *pos; const int *permute;
     const float *x; const float *g; const float *pseudo; const float *mu; const float *isg;
     float *gfeat; float *gww; float *part;      // gww: [E,K] in CSR position order, gw * w per edge and kernel
     int N, K, dim, F, HF;
@@ -261,7 +266,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p)
         int cnt = min(64, e - c);
         int qq = ok ? q : c;
         int id = p.idx[qq];
-        int posv = p.permute[qq];
+        int posv = p.permute[p.pos ? p.pos[qq] : qq];
         const float *ps = p.pseudo + (size_t)(unsigned)posv * dim;
         for (int k = 0; k < K; ++k) {
             float acc = 0.f;
@@ -449,7 +454,7 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
                                  float *grad_mu, float *grad_sigma, const fgnn_schedule_t *sched_csc, void *workspace,
                                  size_t workspace_bytes, void *stream)
 {
-    int rc = spmm_checks("fgnn_gmm_backward", N, E, K, F, sched_csc, col_ptr);
+    int rc = spmm_checks("fgnn_gmm_backward", N, E, K, F, sched_csc, col_ptr, row_ind);
     if (rc) return rc;
     FGNN_REQUIRE(dim >= 1 && dim <= 64 && K * dim <= 1024, FGNN_ERR_LIMIT, "fgnn_gmm_backward: dim=%d K*dim=%d unsupported", dim, K * dim);
     FGNN_REQUIRE(col_ptr && (row_ind || E == 0) && (permute || E == 0) && node_feat && (pseudo || E == 0) && mu && inv_sigma &&
@@ -470,7 +475,8 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
         fgnn_rowcfg cfg;
         FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, aligned, &cfg), FGNN_ERR_LIMIT, "fgnn_gmm_backward: unsupported row width %d", HF);
         GmmBwdP p{};
-        p.items = sched_csc->items_dev; p.n_items = sched_csc->n_items; p.ptr = col_ptr; p.idx = row_ind; p.permute = permute;
+        p.items = sched_csc->items_dev; p.n_items = sched_csc->n_items; p.ptr = col_ptr; p.idx = fgnn_sched_idx(sched_csc, row_ind);
+        p.pos = fgnn_sched_pos(sched_csc); p.permute = permute;
         p.x = node_feat; p.g = grad_out; p.pseudo = pseudo; p.mu = mu; p.isg = inv_sigma; p.gfeat = grad_feat; p.gww = gww;
         p.part = part; p.N = N; p.K = K; p.dim = dim; p.F = F; p.HF = HF; p.g_stride = sum_kernels ? F : HF;
         const int lph = fgnn_pick_lph(cfg.vec, F);

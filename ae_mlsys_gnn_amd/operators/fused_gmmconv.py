@@ -27,7 +27,7 @@ class gmm_native:
                 tuple(mu.shape), tuple(sigma.shape), tuple(pseudo.shape), k, e))
         out = torch.empty((n, f), dtype=torch.float32, device=node_feat.device) if sum_kernels else torch.empty_like(node_feat)
         gauss = torch.empty((e, k), dtype=torch.float32, device=node_feat.device) if want_gauss else None
-        sched = schedule_for(rowptr)
+        sched = schedule_for(rowptr, idx_tensor=colind)
         with torch.cuda.device(node_feat.device):
             ws, wsb = workspace(lib().fgnn_gmm_forward_workspace_bytes(sched.handle, k, f), node_feat.device)
             check(lib().fgnn_gmm_forward(n, e, k, dim, f, ptr(rowptr), ptr(colind), ptr(pos_map), ptr(node_feat), ptr(pseudo),
@@ -48,7 +48,7 @@ class gmm_native:
         grad_pseudo = torch.empty((e, dim), dtype=torch.float32, device=dev)
         grad_mu = torch.empty_like(mu)
         grad_sigma = torch.empty_like(sigma)
-        sched = schedule_for(colptr)
+        sched = schedule_for(colptr, idx_tensor=rowind)
         with torch.cuda.device(dev):
             ws, wsb = workspace(lib().fgnn_gmm_backward_workspace_bytes(sched.handle, k, dim, f), dev)
             check(lib().fgnn_gmm_backward(n, e, k, dim, f, ptr(colptr), ptr(rowind), ptr(permute), ptr(node_feat), ptr(pseudo),

@@ -16,7 +16,7 @@ def mhspmm(ptr_arr, idx, attention, feat, pos_map=None):
     if attention is not None and attention.shape != (e, h):
         raise FgnnError("mhspmm: attention is %s, expected (%d, %d)" % (tuple(attention.shape), e, h))
     out = torch.empty((ptr_arr.numel() - 1, h, f), dtype=torch.float32, device=feat.device)
-    sched = schedule_for(ptr_arr)
+    sched = schedule_for(ptr_arr, idx_tensor=idx)
     with torch.cuda.device(feat.device):
         ws, wsb = workspace(lib().fgnn_mhspmm_workspace_bytes(sched.handle, h, f), feat.device)
         check(lib().fgnn_mhspmm(ptr_arr.numel() - 1, e, h, f, ptr(ptr_arr), ptr(idx), ptr(pos_map), ptr(attention), ptr(feat),

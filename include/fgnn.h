@@ -48,11 +48,11 @@ const char *fgnn_last_error(void);
 typedef struct fgnn_schedule fgnn_schedule_t;
 int     fgnn_schedule_create(const int32_t *ptr_dev, int n_rows, int seg_len, void *stream,
                              fgnn_schedule_t **out);
-/* XCD-aware variant for the gather kernels that need no per-edge arrays (fused GAT forward and
- * backward without stashed attention): rows longer than min_deg (<= 0: 64) entries are cut by source
- * bucket (8 buckets, one per XCD) and workgroup w only gets segments of bucket w % 8, so each XCD's
- * L2 sees one eighth of the gathered feature rows.  The schedule keeps its own bucket-ordered copy
- * of `idx` (4*E bytes of device memory); `idx` must be the array later passed to the operator. */
+/* XCD-aware variant for the gather kernels (fused GAT, mhspmm, GMMConv): rows longer than min_deg
+ * (<= 0: 64) entries are cut by source bucket (8 buckets, one per XCD) and workgroup w only gets
+ * segments of bucket w % 8, so each XCD's L2 sees one eighth of the gathered feature rows.  The
+ * schedule keeps its own bucket-ordered copy of `idx` and the original position of every entry
+ * (8*E bytes of device memory); `idx` must be the array later passed to the operator. */
 int     fgnn_schedule_create_bucketed(const int32_t *ptr_dev, const int32_t *idx_dev, int n_rows,
                                       int seg_len, int min_deg, void *stream, fgnn_schedule_t **out);
 void    fgnn_schedule_destroy(fgnn_schedule_t *s);

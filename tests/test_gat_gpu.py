@@ -103,25 +103,39 @@ def test_gat_xcd_bucketed_schedule(h, f, monkeypatch):
     _lib.clear_schedule_cache()
 
 
-def test_gat_xcd_bucketed_rejects_stash(monkeypatch):
+@pytest.mark.parametrize("variant", ["stash", "fusescatter"])
+def test_gat_xcd_bucketed_stash_variants(variant, monkeypatch):
+    # the stashed [E,H] tensors stay in the caller's edge order under a bucket-ordered schedule
     from ae_mlsys_gnn_amd import _lib
-    from ae_mlsys_gnn_amd._lib import FgnnError, lib, ptr, stream_ptr
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
+    monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+    monkeypatch.setenv("FGNN_SEG_LEN", "128")
+    _lib.clear_schedule_cache()
+    _run(degree_edge_graph(seed=9), 8, 32, variant=variant)
+    _run(graphs.rmat_graph(2000, 150000, seed=10), 4, 16, variant=variant)
+    _lib.clear_schedule_cache()
+
+
+def test_xcd_schedule_must_match_index_array():
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd._lib import lib, ptr, stream_ptr
     g = graphs.add_csc_torch(graphs.rmat_graph(500, 20000, seed=1)).to("cuda:0")
     s = _lib.Schedule(g.row_ptr, 0, g.col_ind, 16)
+    other = g.col_ind.clone()
     n, h, f = g.n, 2, 8
     x = torch.randn(n, h, f, device="cuda:0"); a = torch.randn(n, h, device="cuda:0")
     out = torch.empty_like(x); m = torch.empty(n, h, device="cuda:0"); sm = torch.empty_like(m)
-    el = torch.empty(g.n_edges, h, device="cuda:0"); es = torch.empty_like(el)
     ws = torch.empty(lib().fgnn_gat_forward_workspace_bytes(s.handle, h, f) // 4 + 4, device="cuda:0")
-    rc = lib().fgnn_gat_forward(n, g.n_edges, h, f, ptr(a), ptr(a), ptr(g.row_ptr), ptr(g.col_ind), 0.2, ptr(x), ptr(out), ptr(m),
-                                ptr(sm), None, None, ptr(el), ptr(es), s.handle, ptr(ws), ws.numel() * 4, stream_ptr())
-    assert rc == -6 and b"XCD-aware" in lib().fgnn_last_error()
+    rc = lib().fgnn_gat_forward(n, g.n_edges, h, f, ptr(a), ptr(a), ptr(g.row_ptr), ptr(other), 0.2, ptr(x), ptr(out), ptr(m),
+                                ptr(sm), None, None, None, None, s.handle, ptr(ws), ws.numel() * 4, stream_ptr())
+    assert rc == -6 and b"another index array" in lib().fgnn_last_error()
 
 
 def test_gat_degenerate_graphs():
     """No edges at all, isolated nodes between connected ones, a single node with a self loop."""
     from ae_mlsys_gnn_amd.operators import fused_gat as fg
     dev = "cuda:0"
+    torch.manual_seed(0)
     # (a) 5 nodes, no edges: outputs and every gradient are zero
     g = graphs.add_csc_torch(custom_graph([[], [], [], [], []])).to(dev)
     x = torch.randn(5, 2, 8, device=dev, requires_grad=True)
@@ -130,7 +144,7 @@ def test_gat_degenerate_graphs():
     out = fg.fused_gat_op(a, b, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, 0.2, x)
     out.backward(torch.ones_like(out))
     for t in (out, x.grad, a.grad, b.grad):
-        assert bool(torch.isfinite(t).all()) and float(t.abs().max()) == 0.0
+        assert bool(torch.isfinite(t).all()) and float(t.detach().abs().max()) == 0.0
     # (b) isolated nodes among connected ones, duplicate edges
     _run(custom_graph([[1, 1, 2], [], [0], [], [4, 0, 0, 3], []]), 2, 8)
     # (c) one node, one self loop: identity, gradients of the scores vanish
@@ -140,7 +154,8 @@ def test_gat_degenerate_graphs():
     out = fg.fused_gat_op(a, a, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, 0.2, x)
     go = torch.randn_like(out)
     out.backward(go)
-    assert torch.equal(out, x) and torch.equal(x.grad, go) and float(a.grad.abs().max()) < 1e-6
+    # score gradients cancel up to rounding of <g, x> (magnitude ~10)
+    assert torch.equal(out, x) and torch.equal(x.grad, go) and float(a.grad.abs().max()) < 1e-5
 
 
 def test_gat_widest_supported_row_and_hub():

@@ -386,3 +386,42 @@ def test_coo2csr_matches_graph_builder_at_scale():
     s2 = torch.cat([g.col_ind[perm], g.col_ind[perm][:1000]])
     row_ptr, col_ind = op.coo2csr(d2, s2, g.n)
     assert torch.equal(row_ptr, g.row_ptr) and torch.equal(col_ind, g.col_ind)
+
+
+# ------------------------------------------------------------------ per-edge-array operators under XCD-aware schedules
+def test_mhspmm_and_gmm_with_xcd_buckets(monkeypatch):
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd.operators import fused_gmmconv as fg
+    from ae_mlsys_gnn_amd.operators import mhspmm as op
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
+    monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+    monkeypatch.setenv("FGNN_SEG_LEN", "128")
+    _lib.clear_schedule_cache()
+    g = graphs.add_csc_torch(graphs.rmat_graph(1500, 120000, seed=12))
+    gd = g.to(DEV)
+    gen = torch.Generator().manual_seed(5)
+    feat = torch.randn(g.n, 4, 16, generator=gen, dtype=torch.float64)
+    att = torch.randn(g.n_edges, 4, generator=gen, dtype=torch.float64)
+    go = torch.randn(g.n, 4, 16, generator=gen, dtype=torch.float64)
+    fl, al = feat.clone().requires_grad_(True), att.clone().requires_grad_(True)
+    ref = orc.mhspmm(g.row_ptr, g.col_ind, al, fl)
+    ref.backward(go)
+    fd, ad = feat.float().to(DEV).requires_grad_(True), att.float().to(DEV).requires_grad_(True)
+    out = op.csrmhspmm(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, ad)
+    out.backward(go.float().to(DEV))
+    assert_close(out, ref.detach(), "mhspmm (buckets)", atol=2e-4)
+    assert_close(fd.grad, fl.grad, "mhspmm grad feat (buckets)", atol=2e-4)
+    assert_close(ad.grad, al.grad, "mhspmm grad att (buckets)", atol=2e-4)
+    x, pseudo, mu, isg, go = _gmm_case(g, 3, 2, 64, seed=2)
+    leaves = [t.clone().requires_grad_(True) for t in (x, pseudo, mu, isg)]
+    ref = orc.gmm_forward(g.row_ptr, g.col_ind, *leaves)
+    ref.backward(go)
+    dl = [t.float().to(DEV).requires_grad_(True) for t in (x, pseudo, mu, isg)]
+    out = fg.GmmConvStash(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, *dl)
+    out.backward(go.float().to(DEV))
+    _lib.clear_schedule_cache()
+    assert_close(out, ref.detach(), "gmm out (buckets)", atol=1e-4)
+    assert_close(dl[0].grad, leaves[0].grad, "gmm grad node_feat (buckets)", atol=1e-4)
+    assert_close(dl[1].grad, leaves[1].grad, "gmm grad pseudo (buckets)", atol=1e-3)
+    assert_close(dl[2].grad, leaves[2].grad, "gmm grad mu (buckets)", rtol=1e-3, atol=5e-2)
+    assert_close(dl[3].grad, leaves[3].grad, "gmm grad inv_sigma (buckets)", rtol=1e-3, atol=5e-2)

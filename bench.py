@@ -227,6 +227,15 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
                                         out_feat=o[0], out2=o[3], cc=o[4]), args.steps, 2)
     b_fwd, b_bwd = gat_alg_bytes(n, e, heads, out_feats)
     peak_mem = torch.cuda.max_memory_allocated() / 2**30
+    # stash variant of the same operator (per-edge LeakyReLU / softmax [E,H] written by the forward, read by the backward)
+    so = gat_native.gat_forward(a_row, a_col, g.row_ptr, g.col_ind, slope, h, stash=True)
+    ms_sf, _, _ = time_calls(lambda: gat_native.gat_forward(a_row, a_col, g.row_ptr, g.col_ind, slope, h, stash=True), max(3, args.steps // 4), 1)
+    ms_sb, _, _ = time_calls(
+        lambda: gat_native.gat_backward(slope, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, so[1], so[2], h, a_row, a_col, go,
+                                        out_feat=so[0], out2=so[3], cc=so[4], permute=g.permute, e_lrelu=so[5], e_soft=so[6]),
+        max(3, args.steps // 4), 1)
+    stash_bytes = 2 * e * heads * 4
+    del so
     prep = time_device_preprocessing(g)
 
     if args.no_cpu_baseline:
@@ -245,6 +254,7 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
         "roofline": roofline_record("gat_fwd_kernel (+gat_fwd_merge_kernel)", b_fwd, ms_fwd, (MEASURED_TRAFFIC_BYTES.get(workload) or {}).get("fwd")),
         "roofline_bwd": roofline_record("gat_bwd_node_kernel + gat_bwd_kernel (+gat_bwd_merge_kernel)", b_bwd, ms_bwd,
                                         (MEASURED_TRAFFIC_BYTES.get(workload) or {}).get("bwd")),
+        "stash_variant": {"fwd_ms": round(ms_sf, 4), "bwd_ms": round(ms_sb, 4), "stashed_GiB": round(stash_bytes / 2**30, 3)},
         "sparse_fwd_bwd": {"ms": round(ms_fwd + ms_bwd, 4), "alg_bytes": b_fwd + b_bwd,
                            "achieved_GBps": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6, 1),
                            "frac_of_peak": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6 / HBM_PEAK_GBPS, 4)},

@@ -83,3 +83,74 @@ def test_graph_builders():
     src = graphs.knn_graph(pts, 7).view(3, 50, 7)
     assert bool((src[:, :, 0] == torch.arange(150).view(3, 50)).all()), "nearest neighbour of a point is itself"
     assert bool(((src // 50) == torch.arange(3).view(3, 1, 1)).all()), "neighbours stay inside the cloud"
+
+
+def test_reference_import_recipe_resolves_to_this_package(tmp_path, monkeypatch):
+    """The aliasing recipe documented for the reference tree: `operators` resolves to this package's
+    mirror, so a layer file written against the reference's module names imports unchanged."""
+    import importlib
+    import sys
+    import ae_mlsys_gnn_amd.operators as ops
+    for name in ("operators", "operators.fused_gat", "operators.fused_edgeconv", "operators.fused_gmmconv", "operators.mhspmm",
+                 "operators.edge_softmax", "operators.u_add_v", "operators.spmm", "operators.csr2csc"):
+        monkeypatch.delitem(sys.modules, name, raising=False)
+    monkeypatch.setitem(sys.modules, "operators", ops)
+    for m in ("fused_gat", "fused_edgeconv", "fused_gmmconv", "mhspmm", "edge_softmax", "u_add_v", "spmm", "csr2csc"):
+        monkeypatch.setitem(sys.modules, "operators." + m, getattr(ops, m))
+    # a stand-in layer file using the reference's import lines (layers/gatconv_layer.py:7, edgeconv_layer.py:4,
+    # gmmconv_layer.py:9-12)
+    (tmp_path / "ref_style_layer.py").write_text(
+        "from operators.fused_gat import fused_gat_op, fused_gat_stash_op, fused_gat_fusescatter\n"
+        "from operators.fused_edgeconv import fused_edgeconv_op\n"
+        "from operators.fused_gmmconv import GmmConvFuse, GmmConvStash, GaussianCp\n"
+        "from operators.mhspmm import csrmhspmm\n"
+        "from operators.edge_softmax import csr_edge_softmax\n"
+        "from operators.u_add_v import u_add_v_op\n"
+        "from operators.spmm import csrspmm\n"
+        "from operators.csr2csc import sparsetrans\n")
+    monkeypatch.syspath_prepend(str(tmp_path))
+    mod = importlib.import_module("ref_style_layer")
+    assert mod.fused_gat_op is ops.fused_gat.fused_gat_op and mod.sparsetrans is ops.csr2csc.sparsetrans
+
+
+def test_reference_signatures_are_kept():
+    """Argument names and order of the public callables equal the reference's (operators/*.py)."""
+    import inspect
+    from ae_mlsys_gnn_amd import layers, operators as ops
+    want = {
+        ops.fused_gat.fused_gat_op: "attn_row attn_col row_ptr col_ind col_ptr row_ind negative_slope in_feat save_memory",
+        ops.fused_gat.fused_gat_stash_op: "attn_row attn_col row_ptr col_ind col_ptr row_ind negative_slope in_feat permute",
+        ops.fused_gat.fused_gat_fusescatter: "attn_row attn_col row_ptr col_ind col_ptr row_ind negative_slope in_feat permute",
+        ops.fused_edgeconv.fused_edgeconv_op: "k src_ind h_src h_dst",
+        ops.fused_gmmconv.GmmConvFuse: "rowptr colind colptr rowind permute node_feat pseudo mu sigma",
+        ops.fused_gmmconv.GmmConvStash: "rowptr colind colptr rowind permute node_feat pseudo mu sigma",
+        ops.fused_gmmconv.GmmConvFuseEb: "rowptr colind colptr rowind permute node_feat pseudo mu sigma",
+        ops.fused_gmmconv.GaussianCp: "pseudo mu sigma",
+        ops.mhspmm.csrmhspmm: "rowptr colind colptr rowind permute feat attention",
+        ops.edge_softmax.csr_edge_softmax: "rowptr h",
+        ops.u_add_v.u_add_v_op: "row_ptr col_ind row_val col_val",
+        ops.spmm.csrspmm: "rowptr colind x csr_data sym actnn",
+        ops.csr2csc.sparsetrans: "rowptr colind numlist",
+        layers.GATConv.forward: "self row_ptr col_ind col_ptr row_ind feat save_memory",
+        layers.GATConv_stash.forward: "self row_ptr col_ind col_ptr row_ind feat permute",
+        layers.EdgeConv.forward: "self k src_ind feat",
+        layers.GMMConv.forward: "self rowptr colind colptr rowind permute feat pseudo",
+        layers.GATConv.__init__: "self in_feats out_feats num_heads negative_slope",
+        layers.EdgeConv.__init__: "self in_feat out_feat batch_norm allow_zero_in_degree",
+        layers.GMMConv.__init__: "self in_feats out_feats dim n_kernels aggregator_type residual bias allow_zero_in_degree",
+    }
+    for fn, names in want.items():
+        assert list(inspect.signature(fn).parameters) == names.split(), fn
+
+
+def test_more_argument_errors_without_gpu():
+    l = _lib.lib()
+    assert l.fgnn_knn_graph(1, 10, 3, 11, None, None, None) == -2                 # k > P
+    assert l.fgnn_gather_rows(5, 0, None, None, None, None) == -2                 # W < 1
+    assert l.fgnn_edge_softmax(-1, 0, 1, None, None, None, None) == -2
+    assert l.fgnn_gaussian(4, 1, 2, None, None, None, None, None) == -1
+    assert l.fgnn_coo2csr(4, 4, 3, None, None, 1, None, None, None, None, None, 0, None) == -1
+    out = ctypes.c_void_p()
+    assert l.fgnn_schedule_create(None, 4, 0, None, ctypes.byref(out)) == -1
+    assert l.fgnn_schedule_create_bucketed(None, None, 4, 0, 0, None, ctypes.byref(out)) == -1
+    l.fgnn_schedule_destroy(None)                                                  # no-op on NULL

@@ -425,3 +425,42 @@ def test_mhspmm_and_gmm_with_xcd_buckets(monkeypatch):
     assert_close(dl[1].grad, leaves[1].grad, "gmm grad pseudo (buckets)", atol=1e-3)
     assert_close(dl[2].grad, leaves[2].grad, "gmm grad mu (buckets)", rtol=1e-3, atol=5e-2)
     assert_close(dl[3].grad, leaves[3].grad, "gmm grad inv_sigma (buckets)", rtol=1e-3, atol=5e-2)
+
+
+# ------------------------------------------------------------------ HIP graph capture of a launch-bound step
+def test_edgeconv_step_replays_from_a_hip_graph():
+    """EdgeConv forward + backward captured into a HIP graph (the library clears memory with fill
+    kernels, never with memset nodes).  Every replay is checked against an eager run on fresh inputs,
+    with eager work and synchronisations between the replays."""
+    from ae_mlsys_gnn_amd.operators.fused_edgeconv import edgeconv_native
+    from ae_mlsys_gnn_amd.operators.knn import knn_graph
+    torch.manual_seed(3)
+    n, f, k = 4 * 256, 64, 20
+    pts = (torch.rand(4, 256, 3) * 2 - 1).to(DEV)
+    src = knn_graph(pts, k)
+    h_src = torch.randn(n, f, device=DEV)
+    h_dst = torch.randn(n, f, device=DEV)
+    go = torch.randn(n, f, device=DEV)
+    # warm up on a side stream, then capture
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for _ in range(2):
+            out, arg = edgeconv_native.edgeconv_forward(k, src, h_src, h_dst)
+            gs = edgeconv_native.edgeconv_backward(go, arg, n)
+    torch.cuda.current_stream().wait_stream(s)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out, arg = edgeconv_native.edgeconv_forward(k, src, h_src, h_dst)
+        gs = edgeconv_native.edgeconv_backward(go, arg, n)
+    for rep in range(4):
+        h_src.copy_(torch.randn(n, f, device=DEV))           # new inputs in the captured buffers
+        h_dst.copy_(torch.randn(n, f, device=DEV))
+        go.copy_(torch.round(torch.randn(n, f, device=DEV) * 8) / 8)     # dyadic values: the scatter sum is order independent
+        graph.replay()
+        torch.cuda.synchronize()
+        e_out, e_arg = edgeconv_native.edgeconv_forward(k, src, h_src, h_dst)
+        e_gs = edgeconv_native.edgeconv_backward(go, e_arg, n)
+        torch.cuda.synchronize()
+        assert torch.equal(out, e_out) and torch.equal(arg, e_arg), "replay %d: forward differs from eager" % rep
+        assert torch.equal(gs, e_gs), "replay %d: backward differs from eager" % rep

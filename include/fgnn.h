@@ -116,7 +116,8 @@ int fgnn_edgeconv_backward(int N, int n_src, int F, const int32_t *argmax, const
 
 /* k-nearest-neighbour graph of batched point clouds, the input of fgnn_edgeconv_forward: points
  * [n_clouds*P, D]; src_ind [n_clouds*P*k] gets, for every point, the global ids of the k nearest
- * points of its own cloud (itself included), nearest first, ties to the smaller id.  Stands in for
+ * points of its own cloud (itself included), nearest first, ties to the smaller id; 1 <= k <= min(P,
+ * 128).  Stands in for
  * the DGL KNNGraph call of the reference's DGCNN loop (script/train/train_edgeconv_our.py:51-55). */
 int fgnn_knn_graph(int n_clouds, int P, int D, int k, const float *points, int32_t *src_ind,
                    void *stream);

@@ -318,7 +318,8 @@ def test_error_paths_return_codes_not_aborts():
 
 
 # ------------------------------------------------------------------ kNN graph builder
-@pytest.mark.parametrize("b,p,d,k", [(3, 100, 3, 5), (2, 1024, 3, 20), (2, 300, 64, 20), (1, 64, 7, 64), (4, 65, 2, 1)])
+@pytest.mark.parametrize("b,p,d,k", [(3, 100, 3, 5), (2, 1024, 3, 20), (2, 300, 64, 20), (1, 64, 7, 64), (4, 65, 2, 1),
+                                     (2, 2500, 5, 70), (1, 1025, 9, 128), (2, 257, 11, 65), (3, 513, 1, 8)])
 def test_knn_graph(b, p, d, k):
     from ae_mlsys_gnn_amd.operators.knn import knn_graph
     gen = torch.Generator().manual_seed(b * p + d)
@@ -336,6 +337,23 @@ def test_knn_graph(b, p, d, k):
     assert bool((got[:, :, 1:] >= got[:, :, :-1] - 1e-6).all())
     assert float((got - want).abs().max()) < 1e-5
     assert all(torch.unique(local[i, j]).numel() == k for i in range(b) for j in range(0, p, 7)), "neighbours of a point are distinct"
+
+
+def test_knn_graph_ties_are_ordered_by_id():
+    """Integer grid coordinates: every squared distance is exact in fp32 and many are equal, so the
+    neighbour ids themselves are fixed by the (distance, id) order."""
+    from ae_mlsys_gnn_amd.operators.knn import knn_graph
+    from ae_mlsys_gnn_amd._lib import FgnnError
+    gen = torch.Generator().manual_seed(5)
+    for (b, p, d, k) in [(2, 1500, 2, 40), (1, 300, 3, 100), (2, 64, 1, 64)]:
+        pts = torch.randint(0, 12, (b, p, d), generator=gen).float()           # duplicates included
+        src = knn_graph(pts.to(DEV), k).cpu().long().view(b, p, k)
+        dist = ((pts.double().unsqueeze(2) - pts.double().unsqueeze(1)) ** 2).sum(-1)
+        key = dist * p + torch.arange(p, dtype=torch.float64).view(1, 1, p)     # exact: dist < 2^10, p < 2^11
+        want = torch.argsort(key, dim=2)[:, :, :k] + (torch.arange(b) * p).view(b, 1, 1)
+        assert torch.equal(src, want), (b, p, d, k)
+    with pytest.raises(FgnnError, match="128"):
+        knn_graph(torch.zeros(1, 200, 3, device=DEV), 129)
 
 
 def test_knn_graph_feeds_edgeconv():

@@ -317,4 +317,19 @@ __device__ __forceinline__ float fg_head_reduce(float *scr, const float (&part)[
     fg_wave_lds_sync();
     return acc;
 }
+// The same sums for a handful of heads without LDS: one masked wave sum per head.
+#define FGNN_FEW_HEADS 8
+template <int VEC, int R>
+__device__ __forceinline__ float fg_head_reduce_few(const float (&part)[R], const fg_lanemap<VEC, R> &lm, int lane, int H)
+{
+    float res = 0.f;
+    for (int h = 0; h < H; ++h) {
+        float v = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) v += (lm.ok[r] && lm.hd[r] == h) ? part[r] : 0.f;
+        float s = fg_wave_sum(v);
+        if (lane == h) res = s;
+    }
+    return res;
+}
 #endif  // __HIPCC__

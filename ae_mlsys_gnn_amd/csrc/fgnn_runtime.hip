@@ -76,6 +76,21 @@ static void split_range(std::vector<fgnn_item> &out, int row, int b, int e, int 
     }
 }
 
+// Stable sort of work items by length, longest first.  Lengths are bounded by the segment length
+// (or the row-length cap of whole rows), so a counting sort does it in one pass.
+static void sort_longest_first(std::vector<fgnn_item> &v, size_t first = 0)
+{
+    if (v.size() - first < 2) return;
+    int max_len = 0;
+    for (size_t i = first; i < v.size(); ++i) max_len = std::max(max_len, v[i].end - v[i].begin);
+    std::vector<size_t> start((size_t)max_len + 2, 0);
+    for (size_t i = first; i < v.size(); ++i) ++start[(size_t)(max_len - (v[i].end - v[i].begin)) + 1];
+    for (size_t l = 1; l < start.size(); ++l) start[l] += start[l - 1];
+    std::vector<fgnn_item> sorted(v.size() - first);
+    for (size_t i = first; i < v.size(); ++i) sorted[start[(size_t)(max_len - (v[i].end - v[i].begin))]++] = v[i];
+    std::copy(sorted.begin(), sorted.end(), v.begin() + first);
+}
+
 static int upload_schedule(fgnn_schedule *s, const std::vector<fgnn_item> &items, const std::vector<fgnn_split> &splits, hipStream_t st)
 {
     hipError_t err = hipSuccess;
@@ -145,8 +160,7 @@ extern "C" int fgnn_schedule_create(const int32_t *ptr_dev, int n_rows, int seg_
         int deg = ptr[i + 1] - ptr[i];
         if (deg <= seg_len) items.push_back({i, ptr[i], ptr[i + 1], -1});
     }
-    std::stable_sort(items.begin() + first_whole, items.end(),
-                     [](const fgnn_item &a, const fgnn_item &b) { return (a.end - a.begin) > (b.end - b.begin); });
+    sort_longest_first(items, first_whole);
 
     fgnn_schedule *s = new_schedule(ptr_dev, n_rows, n_rows ? ptr[n_rows] : 0, seg_len);
     s->n_items = (int)items.size();
@@ -216,16 +230,14 @@ extern "C" int fgnn_schedule_create_bucketed(const int32_t *ptr_dev, const int32
         }
         splits.push_back({i, first, nseg, 0});
     }
-    for (int b = 0; b < FGNN_NUM_XCD; ++b)
-        std::stable_sort(lists[b].begin(), lists[b].end(),
-                         [](const fgnn_item &a, const fgnn_item &c) { return (a.end - a.begin) > (c.end - c.begin); });
+    for (int b = 0; b < FGNN_NUM_XCD; ++b) sort_longest_first(lists[b]);
     // whole rows, longest first, dealt to the currently shortest list (by item count)
     std::vector<fgnn_item> whole;
     for (int i = 0; i < n_rows; ++i) {
         int deg = ptr[i + 1] - ptr[i];
         if (deg <= min_deg) whole.push_back({i, ptr[i], ptr[i + 1], -1});
     }
-    std::stable_sort(whole.begin(), whole.end(), [](const fgnn_item &a, const fgnn_item &c) { return (a.end - a.begin) > (c.end - c.begin); });
+    sort_longest_first(whole);
     {
         size_t target = 0;
         for (int b = 0; b < FGNN_NUM_XCD; ++b) target += lists[b].size();

@@ -46,7 +46,7 @@ __global__ __launch_bounds__(FGNN_TPB) void mhsddmm_kernel(int N, int H, int F, 
                         if ((FULL || lm.ok[r]) && lm.eoff[r] % F == 0) out[o + lm.hd[r]] = s;
                     }
                 } else {
-                    float s = fg_head_reduce<VEC, R>(scr, d, lm, lane, H, F);
+                    float s = H <= FGNN_FEW_HEADS ? fg_head_reduce_few<VEC, R>(d, lm, lane, H) : fg_head_reduce<VEC, R>(scr, d, lm, lane, H, F);
                     if (lane < H) out[o + lane] = s;
                 }
             }

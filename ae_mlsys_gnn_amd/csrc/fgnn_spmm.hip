@@ -305,7 +305,8 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p)
                         if ((FULL || lm.ok[r]) && lm.eoff[r] % p.F == 0) gdst[lm.hd[r]] = sum * w[r];
                     }
                 } else {
-                    float sum = fg_head_reduce<VEC, R>(scr, dpart, lm, lane, K, p.F);
+                    float sum = K <= FGNN_FEW_HEADS ? fg_head_reduce_few<VEC, R>(dpart, lm, lane, K)
+                                                    : fg_head_reduce<VEC, R>(scr, dpart, lm, lane, K, p.F);
                     if (lane < K) gdst[lane] = sum * wl[lane * 64 + t + u];
                 }
             }

@@ -1,0 +1,37 @@
+"""Shared pieces of the training drivers: the timing protocol of the reference's scripts (untimed
+warm-up steps, then N steps between two device synchronisations, script/train/train_gatconv_our.py:
+158-200), peak-memory accounting and the result row appended to the output CSV."""
+from __future__ import annotations
+
+import time
+
+import torch
+
+
+def accuracy(logits, labels):
+    if labels.numel() == 0:
+        return float("nan")
+    return float((logits.argmax(dim=1) == labels).float().mean())
+
+
+def timed_steps(step, warmup, steps, device):
+    """Runs `step` warmup + steps times; returns (seconds per timed step, peak MB of HBM allocated by
+    torch on `device` over all of them, value returned by the last step)."""
+    torch.cuda.reset_peak_memory_stats(device)
+    last = None
+    for _ in range(warmup):
+        last = step()
+    torch.cuda.synchronize(device)
+    t0 = time.time()
+    for _ in range(steps):
+        last = step()
+    torch.cuda.synchronize(device)
+    sec = (time.time() - t0) / max(1, steps)
+    return sec, torch.cuda.max_memory_allocated(device) / 2**20, last
+
+
+def append_row(path, row):
+    print(row)
+    if path:
+        with open(path, "a") as f:
+            print(row, file=f)

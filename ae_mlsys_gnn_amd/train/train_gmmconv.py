@@ -1,0 +1,124 @@
+"""MoNet (GMMConv) node-classification training on the fused GMMConv operators.
+
+Command line, model and protocol of the reference's script/train/train_gmmconv_our.py and
+train_gmmconv_stash.py: `n-layers` + 2 GMMConv layers, each with its own Linear(2, pseudo-dim) + Tanh
+projection of the degree pseudo-coordinates, dropout between layers; cross-entropy on the training
+nodes, Adam; 5 warm-up steps, then `n-epochs` timed steps (each followed by a validation pass, as in
+the reference); row "train_monet_<variant>,dataset=..,k=..,d=..,latency=..s,memory=..MB".
+
+    python -m ae_mlsys_gnn_amd.train.train_gmmconv --dataset reddit --n-kernels 2 --pseudo-dim 1
+"""
+from __future__ import annotations
+
+import argparse
+
+import torch
+from torch import nn
+
+from ..layers import GMMConv, GMMConv_stash
+from . import common, datasets
+
+VARIANTS = {"our": GMMConv, "stash": GMMConv_stash}
+
+
+class PseudoProj(nn.Linear):
+    """Linear(2, dim) + Tanh over the per-edge pseudo-coordinates (train_gmmconv_our.py:46-57), same
+    parameters as nn.Linear.  With only two input columns and one row per edge the product is written
+    as two broadcast multiplies: its weight gradient is then a column reduction over the edges rather
+    than a 2 x dim GEMM with a reduction length of E, which GEMM libraries run on a single workgroup."""
+
+    def forward(self, pseudo):
+        out = pseudo[:, 0:1] * self.weight[:, 0] + pseudo[:, 1:2] * self.weight[:, 1]
+        return torch.tanh(out + self.bias)
+
+
+class MoNet(nn.Module):
+    def __init__(self, conv, in_feats, n_hidden, out_feats, n_layers, dim, n_kernels, dropout):
+        super().__init__()
+        sizes = [in_feats] + [n_hidden] * (n_layers + 1) + [out_feats]
+        self.layers = nn.ModuleList(conv(sizes[i], sizes[i + 1], dim, n_kernels) for i in range(len(sizes) - 1))
+        self.pseudo_proj = nn.ModuleList(PseudoProj(2, dim) for _ in self.layers)
+        self.dropout = nn.Dropout(dropout)
+
+    def forward(self, g, feat, pseudo):
+        h = feat
+        for i, (layer, proj) in enumerate(zip(self.layers, self.pseudo_proj)):
+            if i:
+                h = self.dropout(h)
+            h = layer(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, g.permute, h, proj(pseudo))
+        return h
+
+
+def build_parser():
+    p = argparse.ArgumentParser(description="MoNet")
+    p.add_argument("--dataset", type=str, default="cora")
+    p.add_argument("--dropout", type=float, default=0.5)
+    p.add_argument("--gpu", type=int, default=0)
+    p.add_argument("--lr", type=float, default=1e-2)
+    p.add_argument("--n-epochs", type=int, default=2, help="number of timed training steps")
+    p.add_argument("--n-hidden", type=int, default=16)
+    p.add_argument("--n-layers", type=int, default=0, help="number of extra hidden layers")
+    p.add_argument("--pseudo-dim", type=int, default=2)
+    p.add_argument("--n-kernels", type=int, default=3)
+    p.add_argument("--weight-decay", type=float, default=5e-4)
+    p.add_argument("--output", type=str, default="figure7.csv")
+    p.add_argument("--variant", choices=sorted(VARIANTS), default="our")
+    p.add_argument("--data-root", type=str, default=None)
+    p.add_argument("--cache-dir", type=str, default=None)
+    p.add_argument("--scale", type=float, default=1.0)
+    p.add_argument("--warmup", type=int, default=5)
+    p.add_argument("--seed", type=int, default=0)
+    return p
+
+
+def main(argv=None):
+    args = build_parser().parse_args(argv)
+    dev = torch.device("cuda", args.gpu)
+    torch.cuda.set_device(dev)
+    data = datasets.load_node_dataset(args.dataset, dev, root=args.data_root, seed=args.seed, scale=args.scale, cache_dir=args.cache_dir)
+    g = data.graph
+    print("----Data statistics------ (%s)\n  #Nodes %d\n  #Edges %d\n  #Classes %d\n  #Train samples %d\n  #Val samples %d\n  #Test samples %d"
+          % (data.source, g.n, g.n_edges, data.n_classes, int(data.train_mask.sum()), int(data.val_mask.sum()), int(data.test_mask.sum())))
+    pseudo = datasets.degree_pseudo(g)
+    torch.manual_seed(args.seed)
+    model = MoNet(VARIANTS[args.variant], data.feat.shape[1], args.n_hidden, data.n_classes, args.n_layers, args.pseudo_dim, args.n_kernels,
+                  args.dropout).to(dev)
+    loss_fcn = nn.CrossEntropyLoss()
+    opt = torch.optim.Adam(model.parameters(), lr=args.lr, weight_decay=args.weight_decay)
+    train_idx = data.train_mask.nonzero().squeeze(1)
+    train_labels = data.label[train_idx]
+
+    def evaluate(mask):
+        model.eval()
+        with torch.no_grad():
+            return common.accuracy(model(g, data.feat, pseudo)[mask], data.label[mask])
+
+    def train_step():
+        model.train()
+        loss = loss_fcn(model(g, data.feat, pseudo)[train_idx], train_labels)
+        opt.zero_grad()
+        loss.backward()
+        opt.step()
+        return loss.detach()
+
+    def epoch():
+        loss = train_step()
+        evaluate(data.val_mask)
+        return loss
+
+    first = float(train_step())
+    for _ in range(args.warmup):
+        train_step()
+    sec, mem, loss = common.timed_steps(epoch, 0, args.n_epochs, dev)
+    acc = evaluate(data.test_mask)
+    print("loss {:.4f} -> {:.4f}".format(first, float(loss)))
+    print("one epoch time: {:.4f} s".format(sec))
+    print("Test Accuracy {:.4f}".format(acc))
+    common.append_row(args.output, "train_monet_{},dataset={},k={},d={},latency={}s,memory={:.1f}MB".format(
+        args.variant, args.dataset, args.n_kernels, args.pseudo_dim, sec, mem))
+    return {"latency_s": sec, "memory_MB": mem, "first_loss": first, "last_loss": float(loss), "test_acc": acc, "source": data.source,
+            "nodes": g.n, "edges": g.n_edges}
+
+
+if __name__ == "__main__":
+    main()

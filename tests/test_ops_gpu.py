@@ -133,7 +133,7 @@ def _gmm_case(g, k, dim, f, seed):
 
 @pytest.mark.parametrize("k,dim,f,variant", [(3, 2, 64, "fuse"), (2, 1, 16, "fuse"), (3, 2, 64, "stash"), (1, 3, 47, "fuse"),
                                               (4, 2, 33, "eb"), (3, 2, 128, "fuse"), (3, 2, 64, "sum"), (2, 3, 20, "sum"),
-                                              (5, 2, 33, "sum")])
+                                              (5, 2, 33, "sum"), (2, 1, 41, "fuse"), (9, 2, 5, "fuse"), (12, 1, 12, "sum")])
 def test_gmm_forward_backward(k, dim, f, variant, monkeypatch):
     from ae_mlsys_gnn_amd.operators import fused_gmmconv as fg
     from ae_mlsys_gnn_amd import _lib
@@ -219,7 +219,7 @@ def _small_graph():
     return graphs.add_csc_torch(degree_edge_graph(n=300, seed=4))
 
 
-@pytest.mark.parametrize("h,f", [(4, 16), (8, 32), (1, 47), (3, 20), (2, 128)])
+@pytest.mark.parametrize("h,f", [(4, 16), (8, 32), (1, 47), (3, 20), (2, 128), (2, 41), (9, 5), (12, 12)])
 def test_mhspmm_and_mhsddmm(h, f):
     from ae_mlsys_gnn_amd.operators import mhspmm as op
     g = _small_graph()

@@ -114,6 +114,95 @@ __global__ __launch_bounds__(FGNN_TPB) void spmm_kernel(SpmmP p, WF wf, int shar
     }
 }
 
+// Rows narrower than a wave (H*F <= 128 floats): G = 2, 4 or 8 entries of the row are gathered by
+// one load instruction.  The wave is cut into G groups of LPR = 64/G lanes; group g takes entries
+// g, g+G, ... of a chunk, lane `sub` of a group owns floats [4*sub, 4*sub+4) of the feature row.  Each
+// group keeps its own partial sums; a butterfly over the groups adds them up at the end.
+template <int G>
+struct fg_packmap {
+    static constexpr int LPR = 64 / G;
+    int grp, eoff, hd;
+    bool ok;
+    __device__ __forceinline__ void init(int lane, int HF, int F)
+    {
+        grp = lane / LPR;
+        eoff = (lane % LPR) * 4;
+        ok = eoff < HF;
+        hd = ok ? eoff / F : 0;
+    }
+};
+// Sum over the G groups; every group ends with the total.
+template <int G>
+__device__ __forceinline__ void fg_pack_reduce(fg_vec<4> &T, int lane)
+{
+#pragma unroll
+    for (int step = 64 / G; step < 64; step <<= 1) {
+        T.v.x += fg_bperm(T.v.x, lane ^ step); T.v.y += fg_bperm(T.v.y, lane ^ step);
+        T.v.z += fg_bperm(T.v.z, lane ^ step); T.v.w += fg_bperm(T.v.w, lane ^ step);
+    }
+}
+static inline int fgnn_pick_pack(int vec, int HF)
+{
+    if (vec != 4) return 1;
+    return HF <= 32 ? 8 : HF <= 64 ? 4 : HF <= 128 ? 2 : 1;
+}
+
+template <int G, class WF>
+__global__ __launch_bounds__(FGNN_TPB) void spmm_packed_kernel(SpmmP p, WF wf, int shared_floats)
+{
+    extern __shared__ float lds[];
+    float *shared = lds + FGNN_WPB * (p.H * 64 + (p.sum_h ? spmm_pw(p.HF) : 0));
+    if (shared_floats > 0) {
+        wf.prepare(shared, (int)threadIdx.x, p.H);
+        __syncthreads();
+    }
+    int row, b, e, slot;
+    if (!fg_get_item(p.items, p.n_items, p.ptr, row, b, e, slot)) return;
+    const int lane = fg_lane();
+    float *wl = lds + fg_wave() * (p.H * 64 + (p.sum_h ? spmm_pw(p.HF) : 0));
+    float *scr = wl + p.H * 64;
+    fg_packmap<G> pm;
+    pm.init(lane, p.HF, p.F);
+    fg_vec<4> T;
+    T.zero();
+    constexpr int U = 8;
+    for (int c = b; c < e; c += 64) {
+        int q = c + lane;
+        bool ok = q < e;
+        int cnt = min(64, e - c);
+        int qq = ok ? q : c;
+        int id = p.idx[qq];
+        int orig = p.pos ? p.pos[qq] : qq;
+        size_t pos = p.pos_map ? (size_t)p.pos_map[orig] : (size_t)orig;
+        wf.fill(wl, shared, lane, pos, ok, p.H);
+        fg_wave_lds_sync();
+        for (int t = 0; t < cnt; t += U * G) {
+            fg_vec<4> ld[U];
+            float w[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u * G + pm.grp;
+                const bool live = ei < cnt && pm.ok;
+                const int rid = __builtin_amdgcn_ds_bpermute((ei & 63) << 2, id);
+                w[u] = live ? wl[pm.hd * 64 + ei] : 0.f;
+                if (live) ld[u].load(p.feat + (size_t)rid * (size_t)p.HF + pm.eoff); else ld[u].zero();
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) T.fma(w[u], ld[u]);
+        }
+        fg_wave_lds_sync();
+    }
+    fg_pack_reduce<G>(T, lane);
+    fg_lanemap<4, 1> lm;
+    lm.eoff[0] = pm.eoff; lm.hd[0] = pm.hd; lm.ok[0] = pm.ok && pm.grp == 0;
+    fg_vec<4> Ts[1] = {T};
+    if (slot < 0) {
+        spmm_store_row<4, 1, false>(p, row, lm, Ts, scr);
+    } else if (lm.ok[0]) {
+        T.store(p.part + (size_t)slot * spmm_pw(p.HF) + pm.eoff);
+    }
+}
+
 template <int VEC, int R>
 __global__ __launch_bounds__(FGNN_TPB) void spmm_merge_kernel(SpmmP p, const fgnn_split *split, int n_split)
 {
@@ -169,8 +258,12 @@ static int spmm_launch(const char *name, SpmmP p, WF wf, int shared_floats, cons
     const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
     const size_t shm = ((size_t)FGNN_WPB * (p.H * 64 + (p.sum_h ? spmm_pw(p.HF) : 0)) + shared_floats) * sizeof(float);
     const size_t shm_merge = p.sum_h ? (size_t)FGNN_WPB * spmm_pw(p.HF) * sizeof(float) : 0;
+    const int pack = fgnn_pick_pack(cfg.vec, p.HF);
     return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
-        hipLaunchKernelGGL((spmm_kernel<VEC, R, FULL, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
+        if (pack == 8) hipLaunchKernelGGL((spmm_packed_kernel<8, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
+        else if (pack == 4) hipLaunchKernelGGL((spmm_packed_kernel<4, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
+        else if (pack == 2) hipLaunchKernelGGL((spmm_packed_kernel<2, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
+        else hipLaunchKernelGGL((spmm_kernel<VEC, R, FULL, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
         int rc = fgnn_launch_status(name);
         if (rc) return rc;
         if (sched && sched->n_split > 0) {
@@ -317,6 +410,74 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p)
 #pragma unroll
     for (int r = 0; r < R; ++r)
         if (FULL || lm.ok[r]) T[r].store(dst + lm.eoff[r]);
+}
+
+// The same pass for rows narrower than a wave, G column entries per load instruction (see
+// spmm_packed_kernel).  Needs F/4 lanes per mixture kernel to be a power of two (LPH > 0).
+template <int G, int LPH>
+__global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_packed_kernel(GmmBwdP p)
+{
+    extern __shared__ float lds[];
+    const int K = p.K, dim = p.dim, KD = K * dim;
+    const int per_wave = K * 64 + 64;
+    float *shared = lds + FGNN_WPB * per_wave;          // mu | inv_sigma
+    for (int i = (int)threadIdx.x; i < KD; i += FGNN_TPB) { shared[i] = p.mu[i]; shared[KD + i] = p.isg[i]; }
+    __syncthreads();
+    int col, b, e, slot;
+    if (!fg_get_item(p.items, p.n_items, p.ptr, col, b, e, slot)) return;
+    const int lane = fg_lane();
+    float *wl = lds + fg_wave() * per_wave;
+    fg_packmap<G> pm;
+    pm.init(lane, p.HF, p.F);
+    fg_vec<4> T, xr;
+    T.zero();
+    if (pm.ok) xr.load(p.x + (size_t)col * p.HF + pm.eoff); else xr.zero();
+    const int goff = (p.g_stride == p.HF) ? pm.eoff : pm.eoff % p.F;
+    const bool writer = pm.ok && pm.eoff % p.F == 0;
+    constexpr int U = 8;
+    for (int c = b; c < e; c += 64) {
+        int q = c + lane;
+        bool ok = q < e;
+        int cnt = min(64, e - c);
+        int qq = ok ? q : c;
+        int id = p.idx[qq];
+        int posv = p.permute[p.pos ? p.pos[qq] : qq];
+        const float *ps = p.pseudo + (size_t)(unsigned)posv * dim;
+        for (int k = 0; k < K; ++k) {
+            float acc = 0.f;
+            for (int d = 0; d < dim; ++d) {
+                float t = (ps[d] - shared[k * dim + d]) * shared[KD + k * dim + d];
+                acc = fmaf(t, t, acc);
+            }
+            wl[k * 64 + lane] = ok ? __expf(-0.5f * acc) : 0.f;
+        }
+        fg_wave_lds_sync();
+        for (int t = 0; t < cnt; t += U * G) {
+            fg_vec<4> ld[U];
+            int pv[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u * G + pm.grp;
+                const bool live = ei < cnt && pm.ok;
+                const int rid = __builtin_amdgcn_ds_bpermute((ei & 63) << 2, id);
+                pv[u] = __builtin_amdgcn_ds_bpermute((ei & 63) << 2, posv);
+                if (live) ld[u].load(p.g + (size_t)rid * p.g_stride + goff); else ld[u].zero();
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u * G + pm.grp;
+                const bool live = ei < cnt && pm.ok;
+                const float w = live ? wl[pm.hd * 64 + ei] : 0.f;
+                T.fma(w, ld[u]);
+                const float sum = fg_group_sum<LPH>(ld[u].dot(xr));
+                if (live && writer) p.gww[(size_t)(unsigned)pv[u] * K + pm.hd] = sum * w;
+            }
+        }
+        fg_wave_lds_sync();
+    }
+    fg_pack_reduce<G>(T, lane);
+    float *dst = slot < 0 ? p.gfeat + (size_t)col * p.HF : p.part + (size_t)slot * spmm_pw(p.HF);
+    if (pm.ok && pm.grp == 0) T.store(dst + pm.eoff);
 }
 
 // Closed-form derivatives of w[p,k] = exp(-0.5 sum_d ((pseudo[p,d]-mu[k,d])*isg[k,d])^2), one edge per
@@ -484,7 +645,14 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
         const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
         rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
             size_t shm = ((size_t)FGNN_WPB * (K * 64 + 64 * R) + 2 * KD) * sizeof(float);
+            const int pack = lph > 0 ? fgnn_pick_pack(cfg.vec, HF) : 1;
             int rc2 = fgnn_dispatch_lph(VEC == 4 ? lph : 0, [&]<int LPH>() -> int {
+                if constexpr (VEC == 4 && R == 1 && LPH > 0 && LPH <= 32) {
+                    // a mixture kernel's LPH lanes must fit inside one group of 64/pack lanes
+                    if (pack == 8 && LPH <= 8) { hipLaunchKernelGGL((gmm_bwd_packed_kernel<8, (LPH <= 8 ? LPH : 1)>), dim3(grid), dim3(FGNN_TPB), shm, st, p); return fgnn_launch_status("gmm_bwd_packed_kernel"); }
+                    if (pack == 4 && LPH <= 16) { hipLaunchKernelGGL((gmm_bwd_packed_kernel<4, (LPH <= 16 ? LPH : 1)>), dim3(grid), dim3(FGNN_TPB), shm, st, p); return fgnn_launch_status("gmm_bwd_packed_kernel"); }
+                    if (pack == 2 && LPH <= 32) { hipLaunchKernelGGL((gmm_bwd_packed_kernel<2, LPH>), dim3(grid), dim3(FGNN_TPB), shm, st, p); return fgnn_launch_status("gmm_bwd_packed_kernel"); }
+                }
                 hipLaunchKernelGGL((gmm_bwd_kernel<VEC, R, FULL, (VEC == 4 ? LPH : 0)>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
                 return fgnn_launch_status("gmm_bwd_kernel");
             });

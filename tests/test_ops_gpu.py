@@ -133,7 +133,10 @@ def _gmm_case(g, k, dim, f, seed):
 
 @pytest.mark.parametrize("k,dim,f,variant", [(3, 2, 64, "fuse"), (2, 1, 16, "fuse"), (3, 2, 64, "stash"), (1, 3, 47, "fuse"),
                                               (4, 2, 33, "eb"), (3, 2, 128, "fuse"), (3, 2, 64, "sum"), (2, 3, 20, "sum"),
-                                              (5, 2, 33, "sum"), (2, 1, 41, "fuse"), (9, 2, 5, "fuse"), (12, 1, 12, "sum")])
+                                              (5, 2, 33, "sum"), (2, 1, 41, "fuse"), (9, 2, 5, "fuse"), (12, 1, 12, "sum"),
+                                              # rows narrower than a wave: several edges per load instruction
+                                              (1, 2, 8, "fuse"), (4, 2, 32, "fuse"), (1, 1, 128, "sum"), (2, 2, 32, "stash"), (2, 1, 16, "sum"),
+                                              (3, 1, 4, "fuse")])
 def test_gmm_forward_backward(k, dim, f, variant, monkeypatch):
     from ae_mlsys_gnn_amd.operators import fused_gmmconv as fg
     from ae_mlsys_gnn_amd import _lib
@@ -219,7 +222,7 @@ def _small_graph():
     return graphs.add_csc_torch(degree_edge_graph(n=300, seed=4))
 
 
-@pytest.mark.parametrize("h,f", [(4, 16), (8, 32), (1, 47), (3, 20), (2, 128), (2, 41), (9, 5), (12, 12)])
+@pytest.mark.parametrize("h,f", [(4, 16), (8, 32), (1, 47), (3, 20), (2, 128), (2, 41), (9, 5), (12, 12), (1, 4), (2, 8), (1, 128)])
 def test_mhspmm_and_mhsddmm(h, f):
     from ae_mlsys_gnn_amd.operators import mhspmm as op
     g = _small_graph()
@@ -430,19 +433,20 @@ def test_mhspmm_and_gmm_with_xcd_buckets(monkeypatch):
     assert_close(out, ref.detach(), "mhspmm (buckets)", atol=2e-4)
     assert_close(fd.grad, fl.grad, "mhspmm grad feat (buckets)", atol=2e-4)
     assert_close(ad.grad, al.grad, "mhspmm grad att (buckets)", atol=2e-4)
-    x, pseudo, mu, isg, go = _gmm_case(g, 3, 2, 64, seed=2)
-    leaves = [t.clone().requires_grad_(True) for t in (x, pseudo, mu, isg)]
-    ref = orc.gmm_forward(g.row_ptr, g.col_ind, *leaves)
-    ref.backward(go)
-    dl = [t.float().to(DEV).requires_grad_(True) for t in (x, pseudo, mu, isg)]
-    out = fg.GmmConvStash(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, *dl)
-    out.backward(go.float().to(DEV))
+    for (k, dim, f) in [(3, 2, 64), (2, 1, 16)]:            # a full-width row and one narrower than a wave
+        x, pseudo, mu, isg, go = _gmm_case(g, k, dim, f, seed=2)
+        leaves = [t.clone().requires_grad_(True) for t in (x, pseudo, mu, isg)]
+        ref = orc.gmm_forward(g.row_ptr, g.col_ind, *leaves)
+        ref.backward(go)
+        dl = [t.float().to(DEV).requires_grad_(True) for t in (x, pseudo, mu, isg)]
+        out = fg.GmmConvStash(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, *dl)
+        out.backward(go.float().to(DEV))
+        assert_close(out, ref.detach(), "gmm out (buckets)", atol=1e-4)
+        assert_close(dl[0].grad, leaves[0].grad, "gmm grad node_feat (buckets)", atol=1e-4)
+        assert_close(dl[1].grad, leaves[1].grad, "gmm grad pseudo (buckets)", atol=1e-3)
+        assert_close(dl[2].grad, leaves[2].grad, "gmm grad mu (buckets)", rtol=1e-3, atol=5e-2)
+        assert_close(dl[3].grad, leaves[3].grad, "gmm grad inv_sigma (buckets)", rtol=1e-3, atol=5e-2)
     _lib.clear_schedule_cache()
-    assert_close(out, ref.detach(), "gmm out (buckets)", atol=1e-4)
-    assert_close(dl[0].grad, leaves[0].grad, "gmm grad node_feat (buckets)", atol=1e-4)
-    assert_close(dl[1].grad, leaves[1].grad, "gmm grad pseudo (buckets)", atol=1e-3)
-    assert_close(dl[2].grad, leaves[2].grad, "gmm grad mu (buckets)", rtol=1e-3, atol=5e-2)
-    assert_close(dl[3].grad, leaves[3].grad, "gmm grad inv_sigma (buckets)", rtol=1e-3, atol=5e-2)
 
 
 # ------------------------------------------------------------------ HIP graph capture of a launch-bound step

@@ -230,23 +230,54 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_merge_kernel(GatFwdP p, cons
 }
 
 // Per-edge stash of the stash variants: e_lrelu[p,h] and e_softmax[p,h] from the saved row
-// statistics.  One wave per work item (row or segment); lanes run over (edge, head) pairs.
-__global__ __launch_bounds__(FGNN_TPB) void gat_edge_stash_kernel(GatFwdP p, float *e_lrelu, float *e_softmax)
+// statistics, in the caller's CSR order whatever schedule the gather pass used: one thread per
+// (edge, head), so both arrays are written as one sequential stream.  The row of an edge is found
+// by bisection of row_ptr, first for the wave's first and last edge (wave-uniform), then per lane
+// inside that usually one- or two-row window.
+__device__ __forceinline__ int gat_row_of(const int *__restrict__ ptr, int lo, int hi, int q)
 {
-    int row, b, e, slot;
-    if (!fg_get_item(p.items, p.n_items, p.ptr, row, b, e, slot)) return;
+    while (lo < hi) {                       // largest r in [lo, hi] with ptr[r] <= q
+        int mid = (lo + hi + 1) >> 1;
+        if (ptr[mid] <= q) lo = mid; else hi = mid - 1;
+    }
+    return lo;
+}
+#define GAT_STASH_CHUNKS 32     // 64-element chunks per wave: the two wave-wide bisections are paid once per 2048 elements
+__global__ __launch_bounds__(FGNN_TPB) void gat_edge_stash_kernel(int N, int64_t E, int H, const int *__restrict__ ptr,
+                                                                  const int *__restrict__ idx, const float *__restrict__ ar,
+                                                                  const float *__restrict__ ac, const float *__restrict__ emax,
+                                                                  const float *__restrict__ esum, float slope,
+                                                                  float *__restrict__ e_lrelu, float *__restrict__ e_softmax)
+{
+    const int64_t total = E * H;
+    const int64_t k0 = ((int64_t)blockIdx.x * FGNN_WPB + fg_wave()) * (64 * GAT_STASH_CHUNKS);
+    if (k0 >= total) return;
+    const int64_t k1 = min(k0 + 64 * GAT_STASH_CHUNKS, total);
     const int lane = fg_lane();
-    const int H = p.H;
-    const int64_t lo = (int64_t)b * H, hi = (int64_t)e * H;
-    for (int64_t k = lo + lane; k < hi; k += 64) {
-        int64_t q = k / H;
-        int h = (int)(k - q * H);
-        int j = p.idx[q];
-        int64_t o = (p.pos ? (int64_t)p.pos[q] : q) * H + h;      // the caller's edge position
-        float ev = fg_lrelu(p.ar[(size_t)row * H + h] + p.ac[(size_t)j * H + h], p.slope);
-        float m = p.emax[(size_t)row * H + h], s = p.esum[(size_t)row * H + h];
-        e_lrelu[o] = ev;
-        e_softmax[o] = __expf(ev - m) / s;
+    const unsigned uh = (unsigned)H;
+    int qbase = fg_uni((int)(k0 / H));                       // edge of the chunk's first element
+    unsigned rem = (unsigned)fg_uni((int)(k0 - (int64_t)qbase * H));
+    const int qlast = fg_uni((int)((k1 - 1) / H));
+    int rlo = gat_row_of(ptr, 0, N - 1, qbase);
+    const int rhi = gat_row_of(ptr, rlo, N - 1, qlast);
+    for (int64_t kk = k0; kk < k1; kk += 64) {
+        const unsigned x = rem + (unsigned)lane;
+        const unsigned dq = x / uh;
+        const int h = (int)(x - dq * uh);
+        const int q = min(qbase + (int)dq, qlast);
+        const int row = gat_row_of(ptr, rlo, rhi, q);
+        const int64_t k = kk + lane;
+        if (k < k1) {
+            const size_t rh = (size_t)row * H + h;
+            const float ev = fg_lrelu(ar[rh] + ac[(size_t)idx[q] * H + h], slope);
+            e_lrelu[k] = ev;
+            e_softmax[k] = __expf(ev - emax[rh]) / esum[rh];
+        }
+        rem += 64u;
+        const unsigned adv = rem / uh;
+        qbase += (int)adv;
+        rem -= adv * uh;
+        rlo = __builtin_amdgcn_readlane(row, 63);           // rows only grow along the chunk
     }
 }
 
@@ -528,8 +559,10 @@ static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_
         return 0;
     });
     if (rc) return rc;
-    if (e_lrelu) {
-        hipLaunchKernelGGL(gat_edge_stash_kernel, dim3(grid), dim3(FGNN_TPB), 0, st, p, e_lrelu, e_softmax);
+    if (e_lrelu && E > 0) {
+        const int64_t waves = (E * H + 64 * GAT_STASH_CHUNKS - 1) / (64 * GAT_STASH_CHUNKS);
+        hipLaunchKernelGGL(gat_edge_stash_kernel, dim3((unsigned)((waves + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, st, N, E, H, row_ptr,
+                           col_ind, attn_row, attn_col, edge_max, edge_sum, slope, e_lrelu, e_softmax);
         return fgnn_launch_status("gat_edge_stash_kernel");
     }
     return 0;

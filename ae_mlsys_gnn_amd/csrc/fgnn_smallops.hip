@@ -76,6 +76,79 @@ extern "C" int fgnn_mhsddmm(int N, int64_t E, int H, int F, const int32_t *row_p
     });
 }
 
+// out[e,h] = <a[row_ind[e],h,:], b[col_ind[e],h,:]> for an edge list (sddmm.coo_sddmm of the
+// reference, src/sddmm/sddmm.cpp:12-27, with H heads).  One wave per 64 edges; both rows of an edge
+// are fetched by base-plus-lane-offset loads, four edges in flight.
+template <int VEC, int R, bool FULL, int LPH>
+__global__ __launch_bounds__(FGNN_TPB) void sddmm_coo_kernel(int64_t E, int H, int F, int HF, const int *rows, const int *cols,
+                                                             const float *a, const float *b, float *out)
+{
+    extern __shared__ float lds[];
+    const int64_t c = ((int64_t)blockIdx.x * FGNN_WPB + fg_wave()) * 64;
+    if (c >= E) return;
+    const int lane = fg_lane();
+    float *scr = lds + fg_wave() * (64 * R);
+    fg_lanemap<VEC, R> lm;
+    lm.init(lane, HF, F);
+    const int cnt = (int)min((int64_t)64, E - c);
+    const int64_t q = c + (lane < cnt ? lane : 0);
+    const int ri = rows[q], ci = cols[q];
+    for (int t = 0; t < cnt; t += 4) {
+        fg_vec<VEC> la[4][R], lb[4][R];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            int i = __builtin_amdgcn_readlane(ri, (t + u) & 63), j = __builtin_amdgcn_readlane(ci, (t + u) & 63);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (FULL || lm.ok[r]) { la[u][r].load(a + (size_t)i * HF + lm.eoff[r]); lb[u][r].load(b + (size_t)j * HF + lm.eoff[r]); }
+                else { la[u][r].zero(); lb[u][r].zero(); }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (t + u >= cnt) break;
+            float d[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) d[r] = la[u][r].dot(lb[u][r]);
+            size_t o = (size_t)(c + t + u) * H;
+            if constexpr (LPH > 0) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    float s = fg_group_sum<LPH>(d[r]);
+                    if ((FULL || lm.ok[r]) && lm.eoff[r] % F == 0) out[o + lm.hd[r]] = s;
+                }
+            } else {
+                float s = H <= FGNN_FEW_HEADS ? fg_head_reduce_few<VEC, R>(d, lm, lane, H) : fg_head_reduce<VEC, R>(scr, d, lm, lane, H, F);
+                if (lane < H) out[o + lane] = s;
+            }
+        }
+    }
+}
+
+extern "C" int fgnn_sddmm_coo(int64_t E, int n_rows, int n_cols, int H, int F, const int32_t *row_ind, const int32_t *col_ind,
+                              const float *a, const float *b, float *out, void *stream)
+{
+    FGNN_REQUIRE(E >= 0 && n_rows >= 0 && n_cols >= 0 && H >= 1 && F >= 1, FGNN_ERR_SHAPE, "fgnn_sddmm_coo: bad sizes");
+    FGNN_REQUIRE(H <= 64 && (int64_t)H * F <= 1024, FGNN_ERR_LIMIT, "fgnn_sddmm_coo: H=%d H*F=%lld unsupported", H, (long long)H * F);
+    FGNN_REQUIRE(E == 0 || (row_ind && col_ind && a && b && out), FGNN_ERR_NULL, "fgnn_sddmm_coo: NULL argument");
+    FGNN_REQUIRE(E == 0 || (n_rows > 0 && n_cols > 0), FGNN_ERR_SHAPE, "fgnn_sddmm_coo: edges without nodes");
+    if (E == 0) return 0;
+    const int HF = H * F;
+    fgnn_rowcfg cfg;
+    FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, fgnn_aligned16(a) && fgnn_aligned16(b), &cfg), FGNN_ERR_LIMIT, "fgnn_sddmm_coo: unsupported row width %d", HF);
+    const int lph = fgnn_pick_lph(cfg.vec, F);
+    const int64_t waves = (E + 63) / 64;
+    const unsigned grid = (unsigned)((waves + FGNN_WPB - 1) / FGNN_WPB);
+    hipStream_t st = (hipStream_t)stream;
+    return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
+        return fgnn_dispatch_lph(VEC == 4 ? lph : 0, [&]<int LPH>() -> int {
+            hipLaunchKernelGGL((sddmm_coo_kernel<VEC, R, FULL, (VEC == 4 ? LPH : 0)>), dim3(grid), dim3(FGNN_TPB),
+                               (size_t)FGNN_WPB * 64 * R * sizeof(float), st, E, H, F, HF, row_ind, col_ind, a, b, out);
+            return fgnn_launch_status("sddmm_coo_kernel");
+        });
+    });
+}
+
 // out[q,:] = in[permute[q],:]  (src/csr2csc/mhtranspose.cu:6-26)
 __global__ __launch_bounds__(256) void gather_rows_kernel(int64_t total, int W, const int *permute, const float *in, float *out)
 {

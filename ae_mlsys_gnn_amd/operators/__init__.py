@@ -9,5 +9,6 @@ from .fused_gmmconv import (GaussianCp, GaussianFunction, GmmConvFuse, GmmConvFu
                             GmmFuseEbFunction, GmmFuseFunction, GmmStashFunction)
 from .knn import knn_graph  # noqa: F401
 from .mhspmm import MHSPMMFunction, csrmhspmm, mhsddmm, mhtranspose  # noqa: F401
+from .sddmm import coo_sddmm, csr_sddmm  # noqa: F401
 from .spmm import SPMMFunction, csrspmm  # noqa: F401
 from .u_add_v import u_add_v_Function, u_add_v_op  # noqa: F401

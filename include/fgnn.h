@@ -180,6 +180,12 @@ int    fgnn_mhspmm(int N, int64_t E, int H, int F, const int32_t *ptr, const int
  * (src/sddmm/sddmm.cpp): out[p,h] = <a[row(p),h,:], b[col_ind[p],h,:]>. */
 int    fgnn_mhsddmm(int N, int64_t E, int H, int F, const int32_t *row_ptr, const int32_t *col_ind,
                     const float *a, const float *b, float *out, void *stream);
+/* sddmm.coo_sddmm (src/sddmm/sddmm.cpp:12-27), with heads: out[e,h] = <a[row_ind[e],h,:],
+ * b[col_ind[e],h,:]> for an edge list; a is [n_rows,H,F], b is [n_cols,H,F].  Indices are not
+ * range-checked on the device. */
+int    fgnn_sddmm_coo(int64_t E, int n_rows, int n_cols, int H, int F, const int32_t *row_ind,
+                      const int32_t *col_ind, const float *a, const float *b, float *out,
+                      void *stream);
 /* mhtranspose.mhtranspose (src/csr2csc/mhtranspose.cc; mhtranspose.cu:28-47): out[q,:] = in[permute[q],:]. */
 int    fgnn_gather_rows(int64_t E, int W, const int32_t *permute, const float *in, float *out,
                         void *stream);

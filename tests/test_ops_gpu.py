@@ -320,6 +320,30 @@ def test_error_paths_return_codes_not_aborts():
         fg.fused_gat_op(a, a, g.row_ptr.long(), g.col_ind, g.col_ptr, g.row_ind, 0.2, torch.randn(64, 8, 4, device=DEV))
 
 
+@pytest.mark.parametrize("h,f", [(1, 64), (1, 47), (4, 16), (3, 20), (9, 5), (2, 256)])
+def test_coo_and_csr_sddmm(h, f):
+    """sddmm.coo_sddmm / csr_sddmm: per-edge dot products, against float64 gathers."""
+    from ae_mlsys_gnn_amd.operators import sddmm
+    g = _small_graph()
+    gen = torch.Generator().manual_seed(h * 100 + f)
+    e = 777                                                    # not a multiple of 64
+    rows = torch.randint(0, g.n, (e,), generator=gen, dtype=torch.int32)
+    cols = torch.randint(0, g.n, (e,), generator=gen, dtype=torch.int32)
+    a = torch.randn(g.n, h, f, generator=gen, dtype=torch.float64)
+    b = torch.randn(g.n, h, f, generator=gen, dtype=torch.float64)
+    want = (a[rows.long()] * b[cols.long()]).sum(-1)
+    got = sddmm.coo_sddmm(rows.to(DEV), cols.to(DEV), a.float().to(DEV), b.float().to(DEV))
+    assert_close(got, want, "coo_sddmm", atol=2e-5 * f ** 0.5)
+    if h == 1:
+        got1 = sddmm.coo_sddmm(rows.to(DEV), cols.to(DEV), a[:, 0].float().to(DEV), b[:, 0].float().to(DEV))
+        assert torch.equal(got1, got[:, 0])
+        dst = torch.repeat_interleave(torch.arange(g.n), (g.row_ptr[1:] - g.row_ptr[:-1]).long())
+        want_csr = (a[dst, 0] * b[g.col_ind.long(), 0]).sum(-1)
+        got_csr = sddmm.csr_sddmm(g.row_ptr.to(DEV), g.col_ind.to(DEV), a[:, 0].float().to(DEV), b[:, 0].float().to(DEV))
+        assert_close(got_csr, want_csr, "csr_sddmm", atol=2e-5 * f ** 0.5)
+    assert sddmm.coo_sddmm(rows[:0].to(DEV), cols[:0].to(DEV), a.float().to(DEV), b.float().to(DEV)).shape == (0, h)
+
+
 # ------------------------------------------------------------------ kNN graph builder
 @pytest.mark.parametrize("b,p,d,k", [(3, 100, 3, 5), (2, 1024, 3, 20), (2, 300, 64, 20), (1, 64, 7, 64), (4, 65, 2, 1),
                                      (2, 2500, 5, 70), (1, 1025, 9, 128), (2, 257, 11, 65), (3, 513, 1, 8)])

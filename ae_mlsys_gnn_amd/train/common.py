@@ -14,6 +14,13 @@ def accuracy(logits, labels):
     return float((logits.argmax(dim=1) == labels).float().mean())
 
 
+def cross_entropy(logits, labels):
+    """Mean cross-entropy, the value of torch.nn.CrossEntropyLoss()(logits, labels), written as
+    logsumexp minus the true-class logit: with millions of rows torch's nll_loss kernels reduce on
+    very few workgroups (9 ms of a 70 ms step at 2.4 M nodes), a gather does not."""
+    return (torch.logsumexp(logits, dim=1) - logits.gather(1, labels.unsqueeze(1)).squeeze(1)).mean()
+
+
 def timed_steps(step, warmup, steps, device):
     """Runs `step` warmup + steps times; returns (seconds per timed step, peak MB of HBM allocated by
     torch on `device` over all of them, value returned by the last step)."""

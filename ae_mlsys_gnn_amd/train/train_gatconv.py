@@ -69,7 +69,7 @@ def main(argv=None):
     heads = [args.num_heads] * args.num_layers + [args.num_out_heads]
     model = GAT(VARIANTS[args.variant], args.num_layers, data.feat.shape[1], args.num_hidden, data.n_classes, heads, args.negative_slope).to(dev)
     extra = True if args.variant == "our" else g.permute
-    loss_fcn = nn.CrossEntropyLoss()
+    loss_fcn = common.cross_entropy
     opt = torch.optim.Adam(model.parameters(), lr=args.lr, weight_decay=args.weight_decay)
     train_idx = data.train_mask.nonzero().squeeze(1)
     train_labels = data.label[train_idx]

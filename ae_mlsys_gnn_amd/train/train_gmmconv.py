@@ -83,7 +83,7 @@ def main(argv=None):
     torch.manual_seed(args.seed)
     model = MoNet(VARIANTS[args.variant], data.feat.shape[1], args.n_hidden, data.n_classes, args.n_layers, args.pseudo_dim, args.n_kernels,
                   args.dropout).to(dev)
-    loss_fcn = nn.CrossEntropyLoss()
+    loss_fcn = common.cross_entropy
     opt = torch.optim.Adam(model.parameters(), lr=args.lr, weight_decay=args.weight_decay)
     train_idx = data.train_mask.nonzero().squeeze(1)
     train_labels = data.label[train_idx]

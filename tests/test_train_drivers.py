@@ -182,3 +182,16 @@ def test_pseudo_projection_equals_linear_tanh():
     gw = torch.autograd.grad(got.sum(), [proj.weight, proj.bias, x])
     ww = torch.autograd.grad(want.sum(), [proj.weight, proj.bias, x])
     assert all(torch.allclose(a, b, atol=1e-12) for a, b in zip(gw, ww))
+
+
+def test_cross_entropy_helper_equals_torch():
+    from ae_mlsys_gnn_amd.train.common import cross_entropy
+    torch.manual_seed(0)
+    logits = (5 * torch.randn(200, 47, dtype=torch.float64)).requires_grad_(True)
+    y = torch.randint(0, 47, (200,))
+    want = torch.nn.CrossEntropyLoss()(logits, y)
+    got = cross_entropy(logits, y)
+    assert abs(float(got) - float(want)) < 1e-12
+    gw, = torch.autograd.grad(want, logits)
+    gg, = torch.autograd.grad(got, logits)
+    assert torch.allclose(gw, gg, atol=1e-14)

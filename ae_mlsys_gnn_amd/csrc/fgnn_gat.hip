@@ -182,6 +182,121 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_kernel(GatFwdP p)
     }
 }
 
+// The forward for rows narrower than a wave (H*F <= 128 floats, 16-byte aligned): the wave is
+// cut into G lane groups (fg_packmap) that take different edges of the row with the same load
+// instruction, each with its own online softmax state; the groups are combined by a log-sum-exp
+// butterfly before the row is written.
+template <int G, bool AUX, bool SLE1>
+__global__ __launch_bounds__(FGNN_TPB) void gat_fwd_packed_kernel(GatFwdP p)
+{
+    int row, b, e, slot;
+    if (!fg_get_item(p.items, p.n_items, p.ptr, row, b, e, slot)) return;
+    const int lane = fg_lane();
+    const int H = p.H;
+    fg_packmap<G> pm;
+    pm.init(lane, p.HF, p.F);
+    const float slope = p.slope;
+    fg_vec<4> T, P;
+    T.zero(); P.zero();
+    float s = 0.f, cp = 0.f, m = -INFINITY;
+    const float arh = p.ar[(size_t)row * H + pm.hd] * FGNN_LOG2E;
+    constexpr int U = 8;
+    for (int c = b; c < e; c += 64) {
+        int q = c + lane;
+        int cnt = min(64, e - c);
+        int idv = p.idx[q < e ? q : c];
+        for (int t = 0; t < cnt; t += U * G) {
+            fg_vec<4> ld[U];
+            float ev[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u * G + pm.grp;
+                const size_t j = (size_t)(unsigned)__builtin_amdgcn_ds_bpermute((ei & 63) << 2, idv);
+                if (ei < cnt && pm.ok) { ld[u].load(p.x + j * p.HF + pm.eoff); ev[u] = p.ac[j * H + pm.hd]; }
+                else { ld[u].zero(); ev[u] = 0.f; }
+            }
+            float bm = -INFINITY;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float v = fg_lrelu_t<SLE1>(fmaf(ev[u], FGNN_LOG2E, arh), slope);
+                v = ((t + u * G + pm.grp) < cnt && pm.ok) ? v : -INFINITY;      // no edge for this lane: weight 0
+                ev[u] = v;
+                bm = fmaxf(bm, v);
+            }
+            if (__builtin_amdgcn_ballot_w64(bm > m) != 0ull) {
+                float mn = fmaxf(m, bm);
+                float sc = (mn == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m - mn);
+                m = mn;
+                T.scale(sc);
+                s *= sc;
+                if (AUX) { P.scale(sc); cp *= sc; }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float w = (ev[u] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ev[u] - m);
+                T.fma(w, ld[u]);
+                s += w;
+                if (AUX) {
+                    float wp = ev[u] > 0.f ? w : 0.f;
+                    P.fma(wp, ld[u]);
+                    cp += wp;
+                }
+            }
+        }
+    }
+    // combine the lane groups: (m, s, cp, T, P) of the partner group, rescaled to the common maximum
+#pragma unroll
+    for (int step = 64 / G; step < 64; step <<= 1) {
+        const int o = lane ^ step;
+        float mo = fg_bperm(m, o);
+        float mn = fmaxf(m, mo);
+        float a = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - mn);
+        float bb = (mo == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mo - mn);
+        fg_vec<4> To;
+        To.v = make_float4(fg_bperm(T.v.x, o), fg_bperm(T.v.y, o), fg_bperm(T.v.z, o), fg_bperm(T.v.w, o));
+        T = T.lin(a, bb, To);
+        s = a * s + bb * fg_bperm(s, o);
+        if (AUX) {
+            fg_vec<4> Po;
+            Po.v = make_float4(fg_bperm(P.v.x, o), fg_bperm(P.v.y, o), fg_bperm(P.v.z, o), fg_bperm(P.v.w, o));
+            P = P.lin(a, bb, Po);
+            cp = a * cp + bb * fg_bperm(cp, o);
+        }
+        m = mn;
+    }
+    if (!(pm.ok && pm.grp == 0)) return;
+    // same epilogue as gat_fwd_kernel: the maximum leaves in natural units, its rounding goes into the sums
+    const float mnat = m * FGNN_LN2;
+    const float fix = (b < e) ? __builtin_amdgcn_exp2f(m - mnat * FGNN_LOG2E) : 1.f;
+    if (slot < 0) {
+        float inv = s > 0.f ? 1.f / s : 0.f;
+        size_t o = (size_t)row * p.HF + pm.eoff;
+        if (AUX) {
+            fg_vec<4> o2 = T.lin(slope * inv, (1.f - slope) * inv, P);
+            o2.store(p.out2 + o);
+        }
+        T.scale(inv);
+        T.store(p.out + o);
+        if (pm.eoff % p.F == 0) {
+            size_t so = (size_t)row * H + pm.hd;
+            p.emax[so] = (b < e) ? mnat : -1e38f;
+            p.esum[so] = s * fix;
+            if (AUX) p.cc[so] = (cp + slope * (s - cp)) * inv;
+        }
+    } else {
+        float *pp = p.part + (size_t)slot * gat_fwd_pw(p.HF, H, AUX);
+        T.scale(fix);
+        T.store(pp + pm.eoff);
+        if (AUX) { P.scale(fix); P.store(pp + p.HF + pm.eoff); }
+        if (pm.eoff % p.F == 0) {
+            float *st = pp + (AUX ? 2 : 1) * p.HF;
+            st[pm.hd] = mnat;
+            st[H + pm.hd] = s * fix;
+            st[2 * H + pm.hd] = cp * fix;
+        }
+    }
+}
+
 // Merge of the segments of split rows: log-sum-exp combination of (m, s, T, P).
 template <int VEC, int R, bool AUX>
 __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_merge_kernel(GatFwdP p, const fgnn_split *split, int n_split)
@@ -456,6 +571,78 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_kernel(GatBwdP p)
     }
 }
 
+// The column pass for rows narrower than a wave: G entries of the column per load instruction
+// (see gat_fwd_packed_kernel); T, P and z are plain sums, so the groups are added by a butterfly.
+template <int G, bool STASH, bool SLE1>
+__global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
+{
+    extern __shared__ float lds[];
+    int col, b, e, slot;
+    if (!fg_get_item(p.items, p.n_items, p.ptr, col, b, e, slot)) return;
+    const int lane = fg_lane();
+    const int H = p.H;
+    float *scr = lds + fg_wave() * (64 + 64);
+    fg_packmap<G> pm;
+    pm.init(lane, p.HF, p.F);
+    fg_vec<4> T, P;
+    T.zero(); P.zero();
+    float z = 0.f;
+    const float ach = p.ac[(size_t)col * H + pm.hd];
+    constexpr int U = 8;
+    for (int c = b; c < e; c += 64) {
+        int q = c + lane;
+        int cnt = min(64, e - c);
+        int qq = q < e ? q : c;
+        int idv = p.idx[qq];
+        int posv = STASH ? p.permute[p.pos ? p.pos[qq] : qq] : 0;
+        for (int t = 0; t < cnt; t += U * G) {
+            fg_vec<4> ld[U];
+            float4 rc[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u * G + pm.grp;
+                const size_t i = (size_t)(unsigned)__builtin_amdgcn_ds_bpermute((ei & 63) << 2, idv);
+                const size_t pos = STASH ? (size_t)(unsigned)__builtin_amdgcn_ds_bpermute((ei & 63) << 2, posv) : 0;
+                if (ei < cnt && pm.ok) {
+                    ld[u].load(p.g + i * p.HF + pm.eoff);
+                    rc[u] = p.rec[i * H + pm.hd];
+                    if (STASH) { rc[u].x = p.erelu[pos * H + pm.hd]; rc[u].y = p.esm[pos * H + pm.hd]; }
+                } else {
+                    ld[u].zero();
+                    rc[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float ev, al;
+                if (STASH) { ev = rc[u].x; al = rc[u].y; }
+                else { ev = fg_lrelu_t<SLE1>(fmaf(ach, FGNN_LOG2E, rc[u].x), p.slope); al = __builtin_amdgcn_exp2f(ev - rc[u].y) * rc[u].z; }
+                al = ((t + u * G + pm.grp) < cnt && pm.ok) ? al : 0.f;
+                const bool pos_e = ev > 0.f;
+                T.fma(al, ld[u]);
+                P.fma(pos_e ? al : 0.f, ld[u]);
+                z = fmaf(pos_e ? al : al * p.slope, rc[u].w, z);
+            }
+        }
+    }
+    fg_pack_reduce<G>(T, lane);
+    fg_pack_reduce<G>(P, lane);
+#pragma unroll
+    for (int step = 64 / G; step < 64; step <<= 1) z += fg_bperm(z, lane ^ step);
+    fg_lanemap<4, 1> lm;
+    lm.eoff[0] = pm.eoff; lm.hd[0] = pm.hd; lm.ok[0] = pm.ok && pm.grp == 0;
+    if (slot < 0) {
+        fg_vec<4> Ts[1] = {T}, Ps[1] = {P};
+        const float zs[1] = {z};
+        gat_bwd_finish<4, 1>(p, col, lane, scr, lm, Ts, Ps, zs);
+    } else if (lm.ok[0]) {
+        float *pp = p.part + (size_t)slot * gat_bwd_pw(p.HF, H);
+        T.store(pp + pm.eoff);
+        P.store(pp + p.HF + pm.eoff);
+        if (pm.eoff % p.F == 0) pp[2 * p.HF + pm.hd] = z;
+    }
+}
+
 template <int VEC, int R>
 __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_merge_kernel(GatBwdP p, const fgnn_split *split, int n_split)
 {
@@ -544,7 +731,19 @@ static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_
     const size_t shm = 0;
     int rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
         const bool sle1 = slope >= 0.f && slope <= 1.f;
-        if (aux && sle1) hipLaunchKernelGGL((gat_fwd_kernel<VEC, R, true, FULL, true>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+        const int pack = fgnn_pick_pack(cfg.vec, HF);
+        if (pack > 1) {
+            auto launch = [&]<int G>() {
+                if (aux && sle1) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, true>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
+                else if (aux) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, false>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
+                else if (sle1) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, false, true>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
+                else hipLaunchKernelGGL((gat_fwd_packed_kernel<G, false, false>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
+            };
+            if (pack == 8) launch.template operator()<8>();
+            else if (pack == 4) launch.template operator()<4>();
+            else launch.template operator()<2>();
+        }
+        else if (aux && sle1) hipLaunchKernelGGL((gat_fwd_kernel<VEC, R, true, FULL, true>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
         else if (aux) hipLaunchKernelGGL((gat_fwd_kernel<VEC, R, true, FULL, false>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
         else if (sle1) hipLaunchKernelGGL((gat_fwd_kernel<VEC, R, false, FULL, true>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
         else hipLaunchKernelGGL((gat_fwd_kernel<VEC, R, false, FULL, false>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
@@ -663,7 +862,18 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
         const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
         const size_t shm = (size_t)FGNN_WPB * (64 * R + 64) * sizeof(float);
         const bool sle1 = negative_slope >= 0.f && negative_slope <= 1.f;
-        if (stash) hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, true, FULL, true>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+        const int pack = fgnn_pick_pack(cfg.vec, HF);
+        if (pack > 1) {
+            auto launch = [&]<int G>() {
+                if (stash) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, true, true>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                else if (sle1) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, false, true>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                else hipLaunchKernelGGL((gat_bwd_packed_kernel<G, false, false>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+            };
+            if (pack == 8) launch.template operator()<8>();
+            else if (pack == 4) launch.template operator()<4>();
+            else launch.template operator()<2>();
+        }
+        else if (stash) hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, true, FULL, true>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
         else if (sle1) hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, false, FULL, true>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
         else hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, false, FULL, false>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
         rc2 = fgnn_launch_status("gat_bwd_kernel");

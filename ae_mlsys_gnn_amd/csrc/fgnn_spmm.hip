@@ -114,39 +114,8 @@ __global__ __launch_bounds__(FGNN_TPB) void spmm_kernel(SpmmP p, WF wf, int shar
     }
 }
 
-// Rows narrower than a wave (H*F <= 128 floats): G = 2, 4 or 8 entries of the row are gathered by
-// one load instruction.  The wave is cut into G groups of LPR = 64/G lanes; group g takes entries
-// g, g+G, ... of a chunk, lane `sub` of a group owns floats [4*sub, 4*sub+4) of the feature row.  Each
-// group keeps its own partial sums; a butterfly over the groups adds them up at the end.
-template <int G>
-struct fg_packmap {
-    static constexpr int LPR = 64 / G;
-    int grp, eoff, hd;
-    bool ok;
-    __device__ __forceinline__ void init(int lane, int HF, int F)
-    {
-        grp = lane / LPR;
-        eoff = (lane % LPR) * 4;
-        ok = eoff < HF;
-        hd = ok ? eoff / F : 0;
-    }
-};
-// Sum over the G groups; every group ends with the total.
-template <int G>
-__device__ __forceinline__ void fg_pack_reduce(fg_vec<4> &T, int lane)
-{
-#pragma unroll
-    for (int step = 64 / G; step < 64; step <<= 1) {
-        T.v.x += fg_bperm(T.v.x, lane ^ step); T.v.y += fg_bperm(T.v.y, lane ^ step);
-        T.v.z += fg_bperm(T.v.z, lane ^ step); T.v.w += fg_bperm(T.v.w, lane ^ step);
-    }
-}
-static inline int fgnn_pick_pack(int vec, int HF)
-{
-    if (vec != 4) return 1;
-    return HF <= 32 ? 8 : HF <= 64 ? 4 : HF <= 128 ? 2 : 1;
-}
-
+// Rows narrower than a wave take the packed lane layout (fg_packmap): G entries of the row per load
+// instruction, one partial sum per lane group, a butterfly over the groups at the end.
 template <int G, class WF>
 __global__ __launch_bounds__(FGNN_TPB) void spmm_packed_kernel(SpmmP p, WF wf, int shared_floats)
 {

@@ -31,8 +31,13 @@ class _GATBase(nn.Module):
 
     def _project(self, feat):
         """h = feat @ W and the two attention scores (attn_l * h).sum(-1), (attn_r * h).sum(-1)
-        (layers/gatconv_layer.py:50-53 of the reference)."""
-        return _ProjectScores.apply(feat, self.W, self.attn_l, self.attn_r)
+        (layers/gatconv_layer.py:50-53 of the reference).  When out_feats is not a multiple of 4
+        (output layers: one head x number of classes) h gets zero columns up to the next multiple,
+        so that the operator takes its 128-bit row layout; `_crop` drops them again."""
+        return _ProjectScores.apply(feat, self.W, self.attn_l, self.attn_r, (-self.out_feats) % 4)
+
+    def _crop(self, out):
+        return out if out.shape[-1] == self.out_feats else out[..., :self.out_feats]
 
 
 class _ProjectScores(torch.autograd.Function):
@@ -43,29 +48,31 @@ class _ProjectScores(torch.autograd.Function):
     product costs the same for 16 columns as for 272) and the input gradient is one GEMM."""
 
     @staticmethod
-    def forward(ctx, feat, W, attn_l, attn_r):
+    def forward(ctx, feat, W, attn_l, attn_r, pad):
         _, hh, ff = attn_l.shape
         wv = W.view(W.shape[0], hh, ff)
         w_score = torch.cat([(wv * attn_l).sum(-1), (wv * attn_r).sum(-1)], dim=1)       # [in, 2H]
-        h = torch.matmul(feat, W)
+        w_proj = W if pad == 0 else torch.cat([wv, wv.new_zeros(W.shape[0], hh, pad)], dim=2).reshape(W.shape[0], -1)
+        h = torch.matmul(feat, w_proj)
         score = torch.matmul(feat, w_score)
-        ctx.save_for_backward(feat, W, attn_l, attn_r, w_score)
-        return h.view(-1, hh, ff), score[:, :hh].contiguous(), score[:, hh:].contiguous()
+        ctx.save_for_backward(feat, W, attn_l, attn_r, torch.cat([w_proj, w_score], dim=1))
+        ctx.pad = pad
+        return h.view(-1, hh, ff + pad), score[:, :hh].contiguous(), score[:, hh:].contiguous()
 
     @staticmethod
     def backward(ctx, dh, drow, dcol):
-        feat, W, attn_l, attn_r, w_score = ctx.saved_tensors
+        feat, W, attn_l, attn_r, w_all = ctx.saved_tensors
         _, hh, ff = attn_l.shape
-        n, hf = feat.shape[0], hh * ff
+        n, hfp = feat.shape[0], hh * (ff + ctx.pad)
         zeros = lambda cols: feat.new_zeros(n, cols)
-        g = torch.cat([zeros(hf) if dh is None else dh.reshape(n, hf), zeros(hh) if drow is None else drow,
-                       zeros(hh) if dcol is None else dcol], dim=1)                        # [N, HF + 2H]
-        dfeat = torch.matmul(g, torch.cat([W, w_score], dim=1).t()) if ctx.needs_input_grad[0] else None
-        dw_ext = torch.matmul(feat.t(), g)                                                # [in, HF + 2H]
-        dwl, dwr = dw_ext[:, hf:hf + hh].unsqueeze(-1), dw_ext[:, hf + hh:].unsqueeze(-1)  # [in, H, 1]
+        g = torch.cat([zeros(hfp) if dh is None else dh.reshape(n, hfp), zeros(hh) if drow is None else drow,
+                       zeros(hh) if dcol is None else dcol], dim=1)                        # [N, H*Fp + 2H]
+        dfeat = torch.matmul(g, w_all.t()) if ctx.needs_input_grad[0] else None
+        dw_ext = torch.matmul(feat.t(), g)                                                # [in, H*Fp + 2H]
+        dwl, dwr = dw_ext[:, hfp:hfp + hh].unsqueeze(-1), dw_ext[:, hfp + hh:].unsqueeze(-1)   # [in, H, 1]
         wv = W.view(W.shape[0], hh, ff)
-        dW = dw_ext[:, :hf] + (dwl * attn_l + dwr * attn_r).reshape(W.shape[0], hf)
-        return dfeat, dW, (wv * dwl).sum(0, keepdim=True), (wv * dwr).sum(0, keepdim=True)
+        dW = dw_ext[:, :hfp].view(W.shape[0], hh, ff + ctx.pad)[:, :, :ff] + dwl * attn_l + dwr * attn_r
+        return dfeat, dW.reshape(W.shape), (wv * dwl).sum(0, keepdim=True), (wv * dwr).sum(0, keepdim=True), None
 
 
 class GATConv(_GATBase):
@@ -73,7 +80,7 @@ class GATConv(_GATBase):
 
     def forward(self, row_ptr, col_ind, col_ptr, row_ind, feat, save_memory=True):
         h, attn_row, attn_col = self._project(feat)
-        return fused_gat_op(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, self.negative_slope, h, save_memory)
+        return self._crop(fused_gat_op(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, self.negative_slope, h, save_memory))
 
 
 class GATConv_stash(_GATBase):
@@ -81,10 +88,10 @@ class GATConv_stash(_GATBase):
 
     def forward(self, row_ptr, col_ind, col_ptr, row_ind, feat, permute):
         h, attn_row, attn_col = self._project(feat)
-        return fused_gat_stash_op(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, self.negative_slope, h, permute)
+        return self._crop(fused_gat_stash_op(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, self.negative_slope, h, permute))
 
 
 class GATConv_fusescatter(_GATBase):
     def forward(self, row_ptr, col_ind, col_ptr, row_ind, feat, permute):
         h, attn_row, attn_col = self._project(feat)
-        return fused_gat_fusescatter(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, self.negative_slope, h, permute)
+        return self._crop(fused_gat_fusescatter(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, self.negative_slope, h, permute))

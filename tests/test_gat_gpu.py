@@ -46,7 +46,8 @@ def _run(g, h, f, slope=0.2, seed=0, attn_scale=1.0, variant="sm", seg_len=None,
     assert_close(acd.grad, ref[3], "grad_attn_col", atol=base_atol * max(1.0, scale))
 
 
-@pytest.mark.parametrize("h,f", [(8, 32), (4, 16), (1, 64), (1, 47), (3, 20), (4, 128), (8, 128), (2, 65), (1, 1)])
+@pytest.mark.parametrize("h,f", [(8, 32), (4, 16), (1, 64), (1, 47), (3, 20), (4, 128), (8, 128), (2, 65), (1, 1),
+                                 (1, 128), (2, 16), (1, 4), (8, 4), (1, 12), (5, 24)])
 def test_gat_shapes(h, f):
     g = graphs.rmat_graph(600, 12000, seed=3)
     _run(g, h, f)
@@ -55,6 +56,23 @@ def test_gat_shapes(h, f):
 @pytest.mark.parametrize("variant", ["sm", "stash", "fusescatter"])
 def test_gat_variants_degree_edges(variant):
     _run(degree_edge_graph(), 8, 32, variant=variant)
+
+
+@pytest.mark.parametrize("variant", ["sm", "stash", "fusescatter"])
+@pytest.mark.parametrize("h,f", [(1, 128), (4, 16), (2, 8)])
+def test_gat_rows_narrower_than_a_wave(h, f, variant, monkeypatch):
+    """H*F <= 128: 2, 4 or 8 edges share a load instruction; degrees 0..3000, split rows and an
+    XCD-aware schedule included."""
+    from ae_mlsys_gnn_amd import _lib
+    _run(degree_edge_graph(seed=11), h, f, variant=variant)
+    monkeypatch.setenv("FGNN_SEG_LEN", "256")
+    _lib.clear_schedule_cache()
+    _run(degree_edge_graph(seed=12), h, f, variant=variant)
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
+    monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+    _lib.clear_schedule_cache()
+    _run(graphs.rmat_graph(2000, 150000, seed=13), h, f, variant=variant)
+    _lib.clear_schedule_cache()
 
 
 def test_gat_split_rows(monkeypatch):

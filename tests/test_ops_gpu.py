@@ -203,18 +203,33 @@ def test_gmm_layer_matches_dgl_composed():
 
 
 # ------------------------------------------------------------------ GAT layer vs the DGL-composed layer
-def test_gat_layer_matches_dgl_composed():
-    from ae_mlsys_gnn_amd.layers import GATConv
+@pytest.mark.parametrize("fin,f,h,variant", [(64, 16, 4, "our"), (30, 47, 1, "our"), (30, 47, 1, "stash"), (20, 6, 3, "fusescatter"),
+                                             (12, 128, 1, "our")])
+def test_gat_layer_matches_dgl_composed(fin, f, h, variant):
+    """Output and the gradients of the input and of all three parameters against autograd through the
+    float64 DGL-composed layer (config C1 graph); odd widths go through the layer's zero padding."""
+    from ae_mlsys_gnn_amd.layers import GATConv, GATConv_fusescatter, GATConv_stash
     torch.manual_seed(2)
     g = graphs.add_csc_torch(graphs.uniform_graph(4096, 32768, seed=0))
-    layer = GATConv(64, 16, 4)
-    feat = torch.randn(g.n, 64)
+    layer = {"our": GATConv, "stash": GATConv_stash, "fusescatter": GATConv_fusescatter}[variant](fin, f, h)
+    feat = torch.randn(g.n, fin)
+    go = torch.randn(g.n, h, f)
     # weight mapping to GATConv_dgl: fc.weight = W^T, attn_l(dgl) = attn_r(ours), attn_r(dgl) = attn_l(ours)
-    ref = orc.gat_layer_dgl(layer.W.t().double(), layer.attn_r.double(), layer.attn_l.double(), g.row_ptr, g.col_ind, 0.2,
-                            feat.double())
+    leaves = [t.detach().double().requires_grad_(True) for t in (layer.W, layer.attn_l, layer.attn_r, feat)]
+    ref = orc.gat_layer_dgl(leaves[0].t(), leaves[2], leaves[1], g.row_ptr, g.col_ind, 0.2, leaves[3])
+    ref.backward(go.double())
     gd = g.to(DEV)
-    out = layer.to(DEV)(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, feat.to(DEV))
+    layer = layer.to(DEV)
+    fd = feat.to(DEV).requires_grad_(True)
+    out = layer(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, fd, True if variant == "our" else gd.permute)
+    assert out.shape == (g.n, h, f)
+    out.backward(go.to(DEV))
     assert_close(out, ref.detach(), "GATConv layer")
+    assert_close(fd.grad, leaves[3].grad, "GATConv grad feat", atol=1e-4)
+    # parameter gradients are sums over 4096 nodes (and their edges) of terms of either sign
+    assert_close(layer.W.grad, leaves[0].grad, "GATConv grad W", rtol=1e-4, atol=2e-3)
+    assert_close(layer.attn_l.grad, leaves[1].grad, "GATConv grad attn_l", rtol=1e-4, atol=2e-3)
+    assert_close(layer.attn_r.grad, leaves[2].grad, "GATConv grad attn_r", rtol=1e-4, atol=2e-3)
 
 
 # ------------------------------------------------------------------ small operators

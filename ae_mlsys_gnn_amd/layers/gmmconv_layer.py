@@ -50,7 +50,12 @@ class _GMMBase(nn.Module):
 
     def forward(self, rowptr, colind, colptr, rowind, permute, feat, pseudo):
         node_feat = self.fc(feat).view(-1, self._n_kernels, self._out_feats)
+        pad = (-self._out_feats) % 4
+        if pad:         # zero columns up to a multiple of 4: the operator then takes its 128-bit row layout
+            node_feat = th.nn.functional.pad(node_feat, (0, pad))
         rst = type(self)._op(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, self.mu, self.inv_sigma)
+        if pad:
+            rst = rst[..., :self._out_feats]
         if self.res_fc is not None:
             rst = rst + self.res_fc(feat)
         if self.bias is not None:

@@ -186,20 +186,37 @@ def test_gaussian_op():
     assert_close(dl[2].grad, leaves[2].grad, "grad sigma", rtol=1e-3, atol=1e-3)
 
 
-def test_gmm_layer_matches_dgl_composed():
-    from ae_mlsys_gnn_amd.layers import GMMConv
+@pytest.mark.parametrize("fout,k,dim,variant", [(16, 3, 2, "our"), (41, 2, 1, "our"), (7, 3, 2, "stash"), (16, 2, 3, "stash")])
+def test_gmm_layer_matches_dgl_composed(fout, k, dim, variant):
+    """Output and the gradients of the input, the pseudo-coordinates and every parameter against
+    autograd through the float64 DGL-composed layer; odd widths go through the layer's zero padding."""
+    from ae_mlsys_gnn_amd.layers import GMMConv, GMMConv_stash
     torch.manual_seed(1)
     g = graphs.add_csc_torch(graphs.rmat_graph(500, 6000, seed=2))
-    layer = GMMConv(32, 16, dim=2, n_kernels=3, residual=True, bias=True)
+    layer = (GMMConv if variant == "our" else GMMConv_stash)(32, fout, dim=dim, n_kernels=k, residual=True, bias=True)
     with torch.no_grad():
         layer.bias.normal_()
     feat = torch.randn(g.n, 32)
-    pseudo = torch.rand(g.n_edges, 2)
-    ref = orc.gmm_layer_dgl(layer.fc.weight.double(), layer.mu.double(), layer.inv_sigma.double(), layer.bias.double(),
-                            g.row_ptr, g.col_ind, feat.double(), pseudo.double(), layer.res_fc.weight.double())
+    pseudo = torch.rand(g.n_edges, dim)
+    go = torch.randn(g.n, fout)
+    params = [layer.fc.weight, layer.mu, layer.inv_sigma, layer.bias, layer.res_fc.weight]
+    leaves = [t.detach().double().requires_grad_(True) for t in params + [feat, pseudo]]
+    ref = orc.gmm_layer_dgl(leaves[0], leaves[1], leaves[2], leaves[3], g.row_ptr, g.col_ind, leaves[5], leaves[6], leaves[4])
+    ref.backward(go.double())
     gd = g.to(DEV)
-    out = layer.to(DEV)(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, feat.to(DEV), pseudo.to(DEV))
+    layer = layer.to(DEV)
+    fd, pd = feat.to(DEV).requires_grad_(True), pseudo.to(DEV).requires_grad_(True)
+    out = layer(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, pd)
+    assert out.shape == (g.n, fout)
+    out.backward(go.to(DEV))
     assert_close(out, ref.detach(), "GMMConv layer", atol=1e-4)
+    assert_close(fd.grad, leaves[5].grad, "GMMConv grad feat", atol=1e-4)
+    assert_close(pd.grad, leaves[6].grad, "GMMConv grad pseudo", atol=1e-3)
+    # parameter gradients are sums over all nodes / edges of terms of either sign
+    for name, got, want in zip(("fc.weight", "mu", "inv_sigma", "bias", "res_fc.weight"),
+                               (layer.fc.weight.grad, layer.mu.grad, layer.inv_sigma.grad, layer.bias.grad, layer.res_fc.weight.grad),
+                               (l.grad for l in leaves[:5])):
+        assert_close(got, want, "GMMConv grad " + name, rtol=1e-3, atol=5e-2)
 
 
 # ------------------------------------------------------------------ GAT layer vs the DGL-composed layer

@@ -227,6 +227,7 @@ static int spmm_launch(const char *name, SpmmP p, WF wf, int shared_floats, cons
     const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
     const size_t shm = ((size_t)FGNN_WPB * (p.H * 64 + (p.sum_h ? spmm_pw(p.HF) : 0)) + shared_floats) * sizeof(float);
     const size_t shm_merge = p.sum_h ? (size_t)FGNN_WPB * spmm_pw(p.HF) * sizeof(float) : 0;
+    FGNN_REQUIRE(shm <= 64 * 1024, FGNN_ERR_LIMIT, "%s: H=%d needs %zu bytes of LDS per workgroup (limit 64 KiB)", name, p.H, shm);
     const int pack = fgnn_pick_pack(cfg.vec, p.HF);
     return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
         if (pack == 8) hipLaunchKernelGGL((spmm_packed_kernel<8, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
@@ -329,6 +330,20 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p)
         int qq = ok ? q : c;
         int id = p.idx[qq];
         int posv = p.permute[p.pos ? p.pos[qq] : qq];
+        // the first rows are requested before the weights are formed: the pseudo-coordinate fetch
+        // (itself behind the permute fetch) then overlaps with the row fetches
+        constexpr int UG = (R >= 8) ? 1 : 8 / R;
+        fg_vec<VEC> ld[UG][R];
+        auto request = [&](int t) {
+#pragma unroll
+            for (int u = 0; u < UG; ++u) {
+                int rid = __builtin_amdgcn_readlane(id, (t + u) & 63);
+                const float *base = p.g + (size_t)rid * p.g_stride;
+#pragma unroll
+                for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ld[u][r].load(base + goff[r]); else ld[u][r].zero(); }
+            }
+        };
+        request(0);
         const float *ps = p.pseudo + (size_t)(unsigned)posv * dim;
         for (int k = 0; k < K; ++k) {
             float acc = 0.f;
@@ -339,16 +354,8 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p)
             wl[k * 64 + lane] = ok ? __expf(-0.5f * acc) : 0.f;
         }
         fg_wave_lds_sync();
-        constexpr int UG = (R >= 8) ? 1 : 8 / R;
         for (int t = 0; t < cnt; t += UG) {
-            fg_vec<VEC> ld[UG][R];
-#pragma unroll
-            for (int u = 0; u < UG; ++u) {
-                int rid = __builtin_amdgcn_readlane(id, t + u);
-                const float *base = p.g + (size_t)rid * p.g_stride;
-#pragma unroll
-                for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ld[u][r].load(base + goff[r]); else ld[u][r].zero(); }
-            }
+            if (t > 0) request(t);
 #pragma unroll
             for (int u = 0; u < UG; ++u) {
                 if (t + u >= cnt) break;
@@ -614,6 +621,7 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
         const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
         rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
             size_t shm = ((size_t)FGNN_WPB * (K * 64 + 64 * R) + 2 * KD) * sizeof(float);
+            FGNN_REQUIRE(shm <= 64 * 1024, FGNN_ERR_LIMIT, "fgnn_gmm_backward: K=%d, dim=%d need %zu bytes of LDS per workgroup (limit 64 KiB)", K, dim, shm);
             const int pack = lph > 0 ? fgnn_pick_pack(cfg.vec, HF) : 1;
             int rc2 = fgnn_dispatch_lph(VEC == 4 ? lph : 0, [&]<int LPH>() -> int {
                 if constexpr (VEC == 4 && R == 1 && LPH > 0 && LPH <= 32) {

@@ -159,3 +159,51 @@ def test_c4_gmm_full_size_vs_oracle():
     # sums over 2.47 M edges of terms of either sign
     assert_close(gm, torch.from_numpy(rgm), "gmm grad_mu at C4", rtol=1e-3, atol=1.0)
     assert_close(gs, torch.from_numpy(rgs), "gmm grad_sigma at C4", rtol=1e-3, atol=1.0)
+
+
+@pytest.fixture(scope="module")
+def c5_graph():
+    from ae_mlsys_gnn_amd.operators import csr2csc as csc_op
+    g = graphs.rmat_graph(2449029, 61_900_000, seed=0, device=DEV)
+    g.col_ptr, g.row_ind, g.permute = csc_op.csr2csc(g.row_ptr, g.col_ind)
+    return g
+
+
+@pytest.mark.parametrize("h,f", [(1, 47), (1, 48), (8, 32)])
+def test_c5_gat_properties(c5_graph, h, f):
+    """Config C5 (2,449,029 nodes, 61.9 M edges + self loops; features larger than every cache):
+    layer 2 in its scalar layout (1 x 47), in the zero-padded packed layout the GAT layer uses
+    (1 x 48) and layer 1 (8 x 32).  Same size-independent properties as at C2."""
+    from ae_mlsys_gnn_amd.operators.fused_gat import gat_native
+    g = c5_graph
+    n = g.n
+    torch.manual_seed(h * 100 + f)
+    ar = torch.randn(n, h, device=DEV) * 0.5
+    ac = torch.randn(n, h, device=DEV) * 0.5
+    x = torch.randn(n, h, f, device=DEV)
+    go = torch.randn(n, h, f, device=DEV)
+    # forward: constant rows come back unchanged; zero attention is the neighbour mean
+    c = torch.randn(1, h, f, device=DEV).expand(n, h, f).contiguous()
+    assert float((gat_native.gat_forward(ar, ac, g.row_ptr, g.col_ind, 0.2, c)[0] - c).abs().max()) < 2e-5
+    z = torch.zeros(n, h, device=DEV)
+    om = gat_native.gat_forward(z, z, g.row_ptr, g.col_ind, 0.2, x)
+    deg = (g.row_ptr[1:] - g.row_ptr[:-1]).long()
+    dst = torch.repeat_interleave(torch.arange(n, device=DEV), deg)
+    acc = torch.zeros(n, h * f, dtype=torch.float64, device=DEV)
+    xf = x.view(n, h * f)
+    for s in range(0, g.n_edges, 4_000_000):
+        sl = slice(s, min(s + 4_000_000, g.n_edges))
+        acc.index_add_(0, dst[sl], xf[g.col_ind[sl].long()].double())
+    assert_close(om[0], (acc / deg.view(n, 1)).view(n, h, f), "neighbour mean at C5", atol=2e-5)
+    assert torch.equal(om[2], deg.float().view(n, 1).expand(n, h))
+    del acc, dst
+    # backward: column-sum checksum, both sides of the score gradient, independence of the features
+    o = gat_native.gat_forward(ar, ac, g.row_ptr, g.col_ind, 0.2, x)
+    gx, gar, gac = gat_native.gat_backward(0.2, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, o[1], o[2], x, ar, ac, go,
+                                           out_feat=o[0], out2=o[3], cc=o[4])
+    assert_close(gx.double().sum(0), go.double().sum(0), "sum_j grad_feat == sum_i grad_out", rtol=1e-5, atol=2e-2)
+    assert_close(gar.double().sum(0), gac.double().sum(0), "sum grad_attn_row == sum grad_attn_col", rtol=1e-4, atol=5e-2)
+    o3 = gat_native.gat_forward(ar, ac, g.row_ptr, g.col_ind, 0.2, x * 3.0)
+    gx3 = gat_native.gat_backward(0.2, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, o3[1], o3[2], x * 3.0, ar, ac, go,
+                                  out_feat=o3[0], out2=o3[3], cc=o3[4])[0]
+    assert torch.equal(gx3, gx)

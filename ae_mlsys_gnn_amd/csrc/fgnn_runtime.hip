@@ -231,30 +231,28 @@ extern "C" int fgnn_schedule_create_bucketed(const int32_t *ptr_dev, const int32
         splits.push_back({i, first, nseg, 0});
     }
     for (int b = 0; b < FGNN_NUM_XCD; ++b) sort_longest_first(lists[b]);
-    // whole rows, longest first, dealt to the currently shortest list (by item count)
-    std::vector<fgnn_item> whole;
-    for (int i = 0; i < n_rows; ++i) {
-        int deg = ptr[i + 1] - ptr[i];
-        if (deg <= min_deg) whole.push_back({i, ptr[i], ptr[i + 1], -1});
-    }
-    sort_longest_first(whole);
+    // whole (short) rows, longest first, dealt round-robin; they run after the bucketed segments, so
+    // their gathers from arbitrary buckets do not disturb the per-XCD working sets
+    std::vector<fgnn_item> tails[FGNN_NUM_XCD];
     {
-        size_t target = 0;
-        for (int b = 0; b < FGNN_NUM_XCD; ++b) target += lists[b].size();
-        target = (target + whole.size() + FGNN_NUM_XCD - 1) / FGNN_NUM_XCD;
-        size_t w = 0;
-        // first level the lists, then deal the rest round-robin
-        for (int b = 0; b < FGNN_NUM_XCD && w < whole.size(); ++b)
-            while (lists[b].size() < target && w < whole.size()) lists[b].push_back(whole[w++]);
-        for (int b = 0; w < whole.size(); b = (b + 1) % FGNN_NUM_XCD) lists[b].push_back(whole[w++]);
+        std::vector<fgnn_item> whole;
+        for (int i = 0; i < n_rows; ++i) {
+            int deg = ptr[i + 1] - ptr[i];
+            if (deg <= min_deg) whole.push_back({i, ptr[i], ptr[i + 1], -1});
+        }
+        sort_longest_first(whole);
+        for (size_t w = 0; w < whole.size(); ++w) tails[w % FGNN_NUM_XCD].push_back(whole[w]);
     }
-    size_t longest = 0;
-    for (int b = 0; b < FGNN_NUM_XCD; ++b) longest = std::max(longest, lists[b].size());
-    size_t groups = (longest + FGNN_WPB - 1) / FGNN_WPB;
-    std::vector<fgnn_item> items(groups * FGNN_NUM_XCD * FGNN_WPB, fgnn_item{-1, 0, 0, -1});
-    for (int b = 0; b < FGNN_NUM_XCD; ++b)
-        for (size_t k = 0; k < lists[b].size(); ++k)
-            items[((k / FGNN_WPB) * FGNN_NUM_XCD + b) * FGNN_WPB + (k % FGNN_WPB)] = lists[b][k];   // workgroup = group*8 + bucket
+    std::vector<fgnn_item> items;
+    for (const std::vector<fgnn_item> *part : {lists, tails}) {
+        size_t longest = 0;
+        for (int b = 0; b < FGNN_NUM_XCD; ++b) longest = std::max(longest, part[b].size());
+        size_t groups = (longest + FGNN_WPB - 1) / FGNN_WPB, base = items.size();
+        items.resize(base + groups * FGNN_NUM_XCD * FGNN_WPB, fgnn_item{-1, 0, 0, -1});
+        for (int b = 0; b < FGNN_NUM_XCD; ++b)
+            for (size_t k = 0; k < part[b].size(); ++k)
+                items[base + ((k / FGNN_WPB) * FGNN_NUM_XCD + b) * FGNN_WPB + (k % FGNN_WPB)] = part[b][k];   // workgroup = group*8 + bucket
+    }
 
     s->n_items = (int)items.size();
     s->n_partials = n_part;

@@ -30,7 +30,7 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published peak
 # x2.000 and WRITE_SIZE x1.000 by the 1 GiB copy of --calibrate-copy; profiles/gat_kernels_gat_c2.md).
 # They bound the HBM traffic from above.  None = not measured for that workload.
 MEASURED_TRAFFIC_BYTES = {
-    "gat_c2": {"fwd": 37_626_766_336, "bwd": 34_242_960_384},
+    "gat_c2": {"fwd": 37_940_294_041, "bwd": 34_175_510_118},
 }
 
 

@@ -402,7 +402,7 @@ struct GatBwdP {
     const int *ptr; const int *idx; const int *pos; const int *permute;
     const float4 *rec;
     const float *ac; const float *x; const float *g;
-    const float *esm; const float *erelu;
+    const float *esm;
     float *gfeat; float *gac; float *part;
     int N, H, F, HF; float slope;
 };
@@ -490,10 +490,7 @@ __device__ __forceinline__ void gat_bwd_batch(const GatBwdP &p, const fg_lanemap
             if (FULL || lm.ok[r]) {
                 ld[u][r].load_off(base, boff[r]);
                 rc[u][r] = *(const float4 *)(rb + roff[r]);
-                if (STASH) {
-                    rc[u][r].x = *(const float *)((const char *)p.erelu + pos + hoff[r]);
-                    rc[u][r].y = *(const float *)((const char *)p.esm + pos + hoff[r]);
-                }
+                if (STASH) rc[u][r].y = *(const float *)((const char *)p.esm + pos + hoff[r]);
             } else {
                 ld[u][r].zero();
                 rc[u][r] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -505,7 +502,9 @@ __device__ __forceinline__ void gat_bwd_batch(const GatBwdP &p, const fg_lanemap
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             float ev, al;
-            if (STASH) { ev = rc[u][r].x; al = rc[u][r].y; }
+            // stash variants: alpha comes from the stash; only the sign of the pre-activation is still
+            // needed, and that is the sign of attn_row + attn_col (no second per-edge gather)
+            if (STASH) { ev = fmaf(ach[r], FGNN_LOG2E, rc[u][r].x); al = rc[u][r].y; }
             else { ev = fg_lrelu_t<SLE1>(fmaf(ach[r], FGNN_LOG2E, rc[u][r].x), p.slope); al = __builtin_amdgcn_exp2f(ev - rc[u][r].y) * rc[u][r].z; }
             if (TAIL) al = ((t + u) < cnt) ? al : 0.f;
             const bool pos_e = ev > 0.f;
@@ -606,7 +605,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
                 if (ei < cnt && pm.ok) {
                     ld[u].load(p.g + i * p.HF + pm.eoff);
                     rc[u] = p.rec[i * H + pm.hd];
-                    if (STASH) { rc[u].x = p.erelu[pos * H + pm.hd]; rc[u].y = p.esm[pos * H + pm.hd]; }
+                    if (STASH) rc[u].y = p.esm[pos * H + pm.hd];
                 } else {
                     ld[u].zero();
                     rc[u] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -615,7 +614,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 float ev, al;
-                if (STASH) { ev = rc[u].x; al = rc[u].y; }
+                if (STASH) { ev = fmaf(ach, FGNN_LOG2E, rc[u].x); al = rc[u].y; }
                 else { ev = fg_lrelu_t<SLE1>(fmaf(ach, FGNN_LOG2E, rc[u].x), p.slope); al = __builtin_amdgcn_exp2f(ev - rc[u].y) * rc[u].z; }
                 al = ((t + u * G + pm.grp) < cnt && pm.ok) ? al : 0.f;
                 const bool pos_e = ev > 0.f;
@@ -815,7 +814,8 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
                      grad_feat && grad_attn_row && grad_attn_col,
                  FGNN_ERR_NULL, "fgnn_gat_backward: NULL argument");
     const bool stash = e_softmax != nullptr;
-    FGNN_REQUIRE(!stash || (permute && e_lrelu), FGNN_ERR_NULL, "fgnn_gat_backward: stashed attention needs permute, e_lrelu and e_softmax");
+    FGNN_REQUIRE(!stash || permute, FGNN_ERR_NULL, "fgnn_gat_backward: stashed attention needs permute");
+    (void)e_lrelu;      // the sign of the pre-activation is taken from attn_row + attn_col
     const bool recompute = !(out_feat && aux_out2 && aux_c);
     FGNN_REQUIRE(!recompute || (row_ptr && (col_ind || E == 0)), FGNN_ERR_NULL, "fgnn_gat_backward: recomputing the forward needs row_ptr/col_ind");
     rc = check_sched(sched_csc, col_ptr, row_ind, N, E, "fgnn_gat_backward(csc)");
@@ -850,7 +850,7 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
     p.items = sched_csc ? sched_csc->items_dev : nullptr;
     p.n_items = sched_csc ? sched_csc->n_items : N;
     p.ptr = col_ptr; p.idx = fgnn_sched_idx(sched_csc, row_ind); p.pos = fgnn_sched_pos(sched_csc); p.permute = permute; p.rec = rec; p.ac = attn_col; p.x = in_feat; p.g = grad_out;
-    p.esm = e_softmax; p.erelu = e_lrelu; p.gfeat = grad_feat; p.gac = grad_attn_col; p.part = part;
+    p.esm = e_softmax; p.gfeat = grad_feat; p.gac = grad_attn_col; p.part = part;
     p.N = N; p.H = H; p.F = F; p.HF = HF; p.slope = negative_slope;
 
     return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {

@@ -80,9 +80,10 @@ int    fgnn_gat_forward(int N, int64_t E, int H, int F,
                         void *stream);
 
 /* Replaces fused_gat_SM.gat_backward (src/fused_gat/fused_gat_SM.cpp:40-124, host launcher
- * fused_gat_SM.cu:865-893); with permute/e_lrelu/e_softmax non-NULL it reads the stashed
- * attention instead of recomputing it (fused_gat_stash.gat_backward, fused_gat_stash.cu:776-804;
- * fused_gat.gat_backward, fused_gat.cu:641-670).
+ * fused_gat_SM.cu:865-893); with permute/e_softmax non-NULL it reads the stashed attention
+ * instead of recomputing it (fused_gat_stash.gat_backward, fused_gat_stash.cu:776-804;
+ * fused_gat.gat_backward, fused_gat.cu:641-670).  e_lrelu is accepted for the reference's argument
+ * list and not read: the sign of the pre-activation is that of attn_row + attn_col.
  * Inputs as the reference's plus out_feat/aux_out2/aux_c from the forward; when those three are
  * NULL they are recomputed into the workspace from (row_ptr, col_ind) first.
  * Outputs: grad_feat [N,H,F], grad_attn_row, grad_attn_col [N,H]; all fully overwritten and

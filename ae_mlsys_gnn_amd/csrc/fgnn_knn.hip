@@ -193,7 +193,6 @@ extern "C" int fgnn_knn_graph(int n_clouds, int P, int D, int k, const float *po
     FGNN_REQUIRE(k <= P, FGNN_ERR_SHAPE, "fgnn_knn_graph: k=%d exceeds the %d points of a cloud", k, P);
     FGNN_REQUIRE(k <= KNN_MAX_K, FGNN_ERR_LIMIT, "fgnn_knn_graph: k=%d exceeds the limit of %d neighbours", k, KNN_MAX_K);
     FGNN_REQUIRE((int64_t)n_clouds * P * k <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_knn_graph: more than 2^31 edges");
-    FGNN_REQUIRE((int64_t)n_clouds * P * D <= 2147483647LL * 4, FGNN_ERR_LIMIT, "fgnn_knn_graph: point array too large");
     FGNN_REQUIRE(points && src_ind, FGNN_ERR_NULL, "fgnn_knn_graph: NULL argument");
     FGNN_REQUIRE(n_clouds <= 65535, FGNN_ERR_LIMIT, "fgnn_knn_graph: more than 65535 clouds");
     if (n_clouds == 0) return 0;

@@ -191,7 +191,7 @@ def test_cross_entropy_helper_equals_torch():
     y = torch.randint(0, 47, (200,))
     want = torch.nn.CrossEntropyLoss()(logits, y)
     got = cross_entropy(logits, y)
-    assert abs(float(got) - float(want)) < 1e-12
+    assert abs(float(got.detach()) - float(want.detach())) < 1e-12
     gw, = torch.autograd.grad(want, logits)
     gg, = torch.autograd.grad(got, logits)
     assert torch.allclose(gw, gg, atol=1e-14)

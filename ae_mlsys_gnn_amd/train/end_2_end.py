@@ -14,7 +14,7 @@ import gc
 
 import torch
 
-from . import train_edgeconv, train_gatconv, train_gmmconv
+from . import forward_latency, train_edgeconv, train_gatconv, train_gmmconv
 
 # (seconds, MB) the reference's example_data holds for its fused ("our") rows; figure10 for stash
 PUBLISHED = {
@@ -24,6 +24,9 @@ PUBLISHED = {
     ("monet", "reddit", "our"): (0.7364, 7202), ("monet", "reddit", "stash"): (0.7447, 9396),
     ("edgeconv", (20, 32), "our"): (0.0947, 2376), ("edgeconv", (20, 64), "our"): (0.1774, 2762),
     ("edgeconv", (40, 32), "our"): (0.1036, 2376), ("edgeconv", (40, 64), "our"): (0.1883, 2762),
+    # figure9.csv: single-layer forward
+    ("forward", "gat 64->4x64", "our"): (0.1021, 2774), ("forward", "edgeconv b=64 k=40", "our"): (0.004418, 1470),
+    ("forward", "monet 16->16 K=2 d=1", "our"): (0.02439, 3212),
 }
 
 
@@ -36,7 +39,7 @@ def _free():
 
 def main(argv=None):
     p = argparse.ArgumentParser(description="end-to-end sweeps")
-    p.add_argument("--sets", nargs="+", default=["gat", "monet", "edgeconv", "stash"], choices=["gat", "monet", "edgeconv", "stash"])
+    p.add_argument("--sets", nargs="+", default=["gat", "monet", "edgeconv", "stash", "forward"], choices=["gat", "monet", "edgeconv", "stash", "forward"])
     p.add_argument("--datasets", nargs="+", default=["cora", "pubmed", "citeseer", "reddit"])
     p.add_argument("--epochs", type=int, default=20)
     p.add_argument("--edgeconv-iters", type=int, default=20, help="training iterations per timed epoch of the DGCNN runs")
@@ -73,6 +76,13 @@ def main(argv=None):
                                                                      "--variant", variant] + common))
             record("monet", "reddit", variant, train_gmmconv.main(["--dataset", "reddit", "--n-epochs", str(args.epochs), "--n-hidden", "16", "--n-kernels", "2",
                                                                    "--pseudo-dim", "1", "--variant", variant] + common))
+    if "forward" in args.sets:                  # figure9.sh
+        fwd = ["--output", args.output, "--epochs", str(max(20, args.epochs))]
+        ds = ["--dataset", "reddit", "--scale", str(args.scale)] + (["--data-root", args.data_root] if args.data_root else [])
+        record("forward", "gat 64->4x64", "our", forward_latency.main(["gat", "--in_feats", "64", "--out_feats", "64", "--num-heads", "4"] + ds + fwd))
+        record("forward", "edgeconv b=64 k=40", "our", forward_latency.main(["edgeconv", "--batch-size", "64", "--k", "40"] + fwd))
+        record("forward", "monet 16->16 K=2 d=1", "our", forward_latency.main(["monet", "--in-feat", "16", "--out-feat", "16", "--n-kernels", "2", "--pseudo-dim", "1"]
+                                                                             + ds + ["--output", args.output, "--n-epochs", str(max(20, args.epochs))]))
     print("\n| run | config | variant | s/step | peak MB | recorded by the reference (RTX 3090) |")
     print("|---|---|---|---|---|---|")
     for kind, key, variant, sec, mem, pub in rows:

@@ -195,3 +195,15 @@ def test_cross_entropy_helper_equals_torch():
     gw, = torch.autograd.grad(want, logits)
     gg, = torch.autograd.grad(got, logits)
     assert torch.allclose(gw, gg, atol=1e-14)
+
+
+@pytest.mark.gpu
+def test_forward_latency_driver(tmp_path):
+    from ae_mlsys_gnn_amd.train import forward_latency
+    out = tmp_path / "figure9.csv"
+    forward_latency.main(["gat", "--dataset", "cora", "--in_feats", "16", "--out_feats", "6", "--num-heads", "2", "--epochs", "5", "--output", str(out)])
+    forward_latency.main(["edgeconv", "--batch-size", "2", "--k", "10", "--epochs", "5", "--output", str(out)])
+    forward_latency.main(["monet", "--dataset", "cora", "--n-epochs", "5", "--output", str(out)])
+    rows = out.read_text().splitlines()
+    assert [r.split(",")[0] for r in rows] == ["gat_with_fusion", "edgeconv_with_fusion", "monet_with_fusion"]
+    assert all("latency=" in r and r.endswith("MB") for r in rows)

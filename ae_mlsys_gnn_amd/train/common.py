@@ -37,6 +37,31 @@ def timed_steps(step, warmup, steps, device):
     return sec, torch.cuda.max_memory_allocated(device) / 2**20, last
 
 
+def capture_step(step, device, warmup=3):
+    """Captures `step` (forward, loss, backward, optimizer step; it must return the loss tensor) into
+    a HIP graph after `warmup` eager calls on a side stream, and returns a callable that replays it
+    and hands back the graph's loss tensor.  For small graphs a training step is a few dozen short
+    kernels and launch-bound; the replay submits them as one unit.  The library's operators enqueue
+    kernels only (buffers are cleared with fill kernels, never memset nodes, and nothing
+    synchronises once the schedules exist), so they can be captured; the optimizer must be built
+    with capturable=True."""
+    side = torch.cuda.Stream(device)
+    side.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(side):
+        for _ in range(warmup):
+            step()
+    torch.cuda.current_stream(device).wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        loss = step()
+
+    def replay():
+        graph.replay()
+        return loss
+    replay.graph = graph
+    return replay
+
+
 def append_row(path, row):
     print(row)
     if path:

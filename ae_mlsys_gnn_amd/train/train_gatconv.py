@@ -53,6 +53,7 @@ def build_parser():
     p.add_argument("--scale", type=float, default=1.0, help="shrink a synthetic dataset (nodes and edges) by this factor")
     p.add_argument("--warmup", type=int, default=10)
     p.add_argument("--seed", type=int, default=0)
+    p.add_argument("--hip-graph", action="store_true", help="capture the training step into a HIP graph and replay it (pays off on small graphs)")
     return p
 
 
@@ -70,7 +71,7 @@ def main(argv=None):
     model = GAT(VARIANTS[args.variant], args.num_layers, data.feat.shape[1], args.num_hidden, data.n_classes, heads, args.negative_slope).to(dev)
     extra = True if args.variant == "our" else g.permute
     loss_fcn = common.cross_entropy
-    opt = torch.optim.Adam(model.parameters(), lr=args.lr, weight_decay=args.weight_decay)
+    opt = torch.optim.Adam(model.parameters(), lr=args.lr, weight_decay=args.weight_decay, capturable=args.hip_graph)
     train_idx = data.train_mask.nonzero().squeeze(1)
     train_labels = data.label[train_idx]
 
@@ -78,12 +79,14 @@ def main(argv=None):
         model.train()
         logits = model(g, data.feat, extra)
         loss = loss_fcn(logits[train_idx], train_labels)
-        opt.zero_grad()
+        opt.zero_grad(set_to_none=False)
         loss.backward()
         opt.step()
         return loss.detach()
 
     first = float(step())
+    if args.hip_graph:
+        step = common.capture_step(step, dev)
     sec, mem, loss = common.timed_steps(step, args.warmup, args.epochs, dev)
     model.eval()
     with torch.no_grad():

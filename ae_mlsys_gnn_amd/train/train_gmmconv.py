@@ -68,6 +68,7 @@ def build_parser():
     p.add_argument("--scale", type=float, default=1.0)
     p.add_argument("--warmup", type=int, default=5)
     p.add_argument("--seed", type=int, default=0)
+    p.add_argument("--hip-graph", action="store_true", help="capture the training step into a HIP graph and replay it (pays off on small graphs)")
     return p
 
 
@@ -84,7 +85,7 @@ def main(argv=None):
     model = MoNet(VARIANTS[args.variant], data.feat.shape[1], args.n_hidden, data.n_classes, args.n_layers, args.pseudo_dim, args.n_kernels,
                   args.dropout).to(dev)
     loss_fcn = common.cross_entropy
-    opt = torch.optim.Adam(model.parameters(), lr=args.lr, weight_decay=args.weight_decay)
+    opt = torch.optim.Adam(model.parameters(), lr=args.lr, weight_decay=args.weight_decay, capturable=args.hip_graph)
     train_idx = data.train_mask.nonzero().squeeze(1)
     train_labels = data.label[train_idx]
 
@@ -96,7 +97,7 @@ def main(argv=None):
     def train_step():
         model.train()
         loss = loss_fcn(model(g, data.feat, pseudo)[train_idx], train_labels)
-        opt.zero_grad()
+        opt.zero_grad(set_to_none=False)
         loss.backward()
         opt.step()
         return loss.detach()
@@ -107,6 +108,8 @@ def main(argv=None):
         return loss
 
     first = float(train_step())
+    if args.hip_graph:
+        train_step = common.capture_step(train_step, dev)
     for _ in range(args.warmup):
         train_step()
     sec, mem, loss = common.timed_steps(epoch, 0, args.n_epochs, dev)

@@ -207,3 +207,23 @@ def test_forward_latency_driver(tmp_path):
     rows = out.read_text().splitlines()
     assert [r.split(",")[0] for r in rows] == ["gat_with_fusion", "edgeconv_with_fusion", "monet_with_fusion"]
     assert all("latency=" in r and r.endswith("MB") for r in rows)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("model", ["gat", "monet"])
+def test_training_step_replays_from_a_hip_graph(model):
+    """--hip-graph: the captured step, replayed 12 times with eager work (validation passes, the
+    driver's own synchronisations) in between, follows the eager loss trajectory.  The capture is
+    preceded by 3 eager steps on a side stream, so 12 replays end where 15 eager steps end."""
+    from ae_mlsys_gnn_amd.train import train_gatconv, train_gmmconv
+    if model == "gat":
+        argv = ["--dataset", "cora", "--num-heads", "2", "--num-hidden", "16", "--warmup", "0", "--output", ""]
+        eager, graphed = train_gatconv.main(argv + ["--epochs", "15"]), train_gatconv.main(argv + ["--epochs", "12", "--hip-graph"])
+    else:
+        argv = ["--dataset", "cora", "--warmup", "0", "--dropout", "0", "--output", ""]
+        eager, graphed = train_gmmconv.main(argv + ["--n-epochs", "15"]), train_gmmconv.main(argv + ["--n-epochs", "12", "--hip-graph"])
+    assert eager["first_loss"] == graphed["first_loss"]
+    # torch's backward of logits[train_idx] adds with atomics, so two eager runs already differ in the
+    # last bits and 16 optimizer steps amplify that; a wrong replay would be off by far more
+    assert abs(eager["last_loss"] - graphed["last_loss"]) <= 5e-4 * abs(eager["last_loss"]), (eager, graphed)
+    assert abs(eager["test_acc"] - graphed["test_acc"]) < 0.02

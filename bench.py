@@ -27,10 +27,14 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published peak
 
 # L2<->fabric bytes per launch of the dominant kernels measured with rocprofv3 --pmc (FETCH_SIZE scaled
-# x2.000 and WRITE_SIZE x1.000 by the 1 GiB copy of --calibrate-copy; profiles/gat_kernels_gat_c2.md).
+# x2.000 and WRITE_SIZE x1.000 by the 1 GiB copy of --calibrate-copy; profiles/gat_kernels_gat_c2.md and
+# profiles/other_workloads.md); all kernels of the entry point summed.
 # They bound the HBM traffic from above.  None = not measured for that workload.
 MEASURED_TRAFFIC_BYTES = {
     "gat_c2": {"fwd": 37_940_294_041, "bwd": 34_175_510_118},
+    "gat_c5_layer1": {"fwd": 72_099_949_465, "bwd": 81_156_805_427},
+    "gmm_c4": {"fwd": 1_154_166_988, "bwd": 1_514_758_144},
+    "edgeconv_c3": {"fwd": 123_305_574, "bwd": 73_504_972},
 }
 
 
@@ -329,10 +333,8 @@ def run_edgeconv(args):
         "config": {"workload": "edgeconv_c3", "clouds": bsz, "points": npts, "k": k, "F": f, "edges": e},
         "hip_graph_replay": {"fwd_bwd_us": round(ms_graph * 1e3, 2), "matches_eager": graph_ok},
         "knn_graph_ms": round(ms_knn, 3),
-        "roofline": {"bound": "hbm", "kernel": "edgeconv_fwd_kernel", "achieved": round(b_f / ms_f / 1e6, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(b_f / ms_f / 1e6 / HBM_PEAK_GBPS, 4), "traffic": None, "alg_bytes": b_f, "ms": round(ms_f, 5)},
-        "roofline_bwd": {"bound": "hbm", "kernel": "fill + edgeconv_bwd_kernel", "achieved": round(b_b / ms_b / 1e6, 1), "peak": HBM_PEAK_GBPS,
-                         "unit": "GB/s", "frac": round(b_b / ms_b / 1e6 / HBM_PEAK_GBPS, 4), "alg_bytes": b_b, "ms": round(ms_b, 5)},
+        "roofline": roofline_record("edgeconv_fwd_kernel", b_f, ms_f, MEASURED_TRAFFIC_BYTES["edgeconv_c3"]["fwd"]),
+        "roofline_bwd": roofline_record("fill + edgeconv_bwd_kernel", b_b, ms_b, MEASURED_TRAFFIC_BYTES["edgeconv_c3"]["bwd"]),
         "cpu_baseline": {"value": round(sorted(ts)[len(ts) // 2] * 1e3, 1), "unit": "us/iter", "cores": cores, "kind": "port",
                          "sample": "EdgeConv_reorg composed math (torch CPU gather + max over k) fwd+bwd at full size, median of 5"},
     }
@@ -383,10 +385,8 @@ def run_gmm(args):
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "gmm_c4", "nodes": n, "edges": e, "K": kk, "dim": dim, "F": f},
-        "roofline": {"bound": "hbm", "kernel": "spmm_kernel<WGauss>", "achieved": round(b_f / ms_f / 1e6, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(b_f / ms_f / 1e6 / HBM_PEAK_GBPS, 4), "traffic": None, "alg_bytes": b_f, "ms": round(ms_f, 4)},
-        "roofline_bwd": {"bound": "hbm", "kernel": "gmm_bwd_kernel (+column sums)", "achieved": round(b_b / ms_b / 1e6, 1), "peak": HBM_PEAK_GBPS,
-                         "unit": "GB/s", "frac": round(b_b / ms_b / 1e6 / HBM_PEAK_GBPS, 4), "alg_bytes": b_b, "ms": round(ms_b, 4)},
+        "roofline": roofline_record("spmm_kernel<WGauss>", b_f, ms_f, MEASURED_TRAFFIC_BYTES["gmm_c4"]["fwd"]),
+        "roofline_bwd": roofline_record("gmm_bwd_kernel + gauss_grad_kernel + column sums", b_b, ms_b, MEASURED_TRAFFIC_BYTES["gmm_c4"]["bwd"]),
         "fused_sum_over_kernels": {"fwd_ms": round(ms_fs, 4), "bwd_ms": round(ms_bs, 4)},
         "cpu_baseline": {"value": round(sorted(ts)[1], 1), "unit": "ms/iter", "cores": cores, "kind": "port",
                          "sample": "GMMConv_dgl composed math (torch CPU) fwd+bwd at full size, median of 3"},

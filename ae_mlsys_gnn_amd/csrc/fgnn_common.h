@@ -166,6 +166,8 @@ template <> struct fg_vec<4> {
     // wave-uniform base + unsigned 32-bit byte offset: lets the load use a scalar base register
     __device__ __forceinline__ void load_off(const char *base, uint32_t off) { v = *reinterpret_cast<const float4 *>(base + off); }
     __device__ __forceinline__ void store(float *p) const { *reinterpret_cast<float4 *>(p) = v; }
+    // streaming store: the line is not kept in L2 (results nobody gathers again in this kernel)
+    __device__ __forceinline__ void store_nt(float *p) const { __builtin_nontemporal_store(v.x, p); __builtin_nontemporal_store(v.y, p + 1); __builtin_nontemporal_store(v.z, p + 2); __builtin_nontemporal_store(v.w, p + 3); }
     __device__ __forceinline__ void fma(float w, const fg_vec &x) { v.x = fmaf(w, x.v.x, v.x); v.y = fmaf(w, x.v.y, v.y); v.z = fmaf(w, x.v.z, v.z); v.w = fmaf(w, x.v.w, v.w); }
     __device__ __forceinline__ void add(const fg_vec &x) { v.x += x.v.x; v.y += x.v.y; v.z += x.v.z; v.w += x.v.w; }
     __device__ __forceinline__ void scale(float w) { v.x *= w; v.y *= w; v.z *= w; v.w *= w; }
@@ -179,6 +181,7 @@ template <> struct fg_vec<1> {
     __device__ __forceinline__ void load(const float *p) { v = *p; }
     __device__ __forceinline__ void load_off(const char *base, uint32_t off) { v = *reinterpret_cast<const float *>(base + off); }
     __device__ __forceinline__ void store(float *p) const { *p = v; }
+    __device__ __forceinline__ void store_nt(float *p) const { __builtin_nontemporal_store(v, p); }
     __device__ __forceinline__ void fma(float w, const fg_vec &x) { v = fmaf(w, x.v, v); }
     __device__ __forceinline__ void add(const fg_vec &x) { v += x.v; }
     __device__ __forceinline__ void scale(float w) { v *= w; }

@@ -153,10 +153,10 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_kernel(GatFwdP p)
             size_t o = (size_t)row * p.HF + lm.eoff[r];
             if (AUX) {
                 fg_vec<VEC> o2 = T[r].lin(slope * inv, (1.f - slope) * inv, P[r]);
-                o2.store(p.out2 + o);
+                o2.store_nt(p.out2 + o);
             }
             T[r].scale(inv);
-            T[r].store(p.out + o);
+            T[r].store_nt(p.out + o);
             if (lm.eoff[r] % p.F == 0) {
                 size_t so = (size_t)row * H + lm.hd[r];
                 p.emax[so] = (b < e) ? mnat[r] : -1e38f;
@@ -170,8 +170,8 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_kernel(GatFwdP p)
         for (int r = 0; r < R; ++r) {
             if (!(FULL || lm.ok[r])) continue;
             T[r].scale(fix[r]);
-            T[r].store(pp + lm.eoff[r]);
-            if (AUX) { P[r].scale(fix[r]); P[r].store(pp + p.HF + lm.eoff[r]); }
+            T[r].store_nt(pp + lm.eoff[r]);
+            if (AUX) { P[r].scale(fix[r]); P[r].store_nt(pp + p.HF + lm.eoff[r]); }
             if (lm.eoff[r] % p.F == 0) {
                 float *st = pp + (AUX ? 2 : 1) * p.HF;
                 st[lm.hd[r]] = mnat[r];
@@ -273,10 +273,10 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_packed_kernel(GatFwdP p)
         size_t o = (size_t)row * p.HF + pm.eoff;
         if (AUX) {
             fg_vec<4> o2 = T.lin(slope * inv, (1.f - slope) * inv, P);
-            o2.store(p.out2 + o);
+            o2.store_nt(p.out2 + o);
         }
         T.scale(inv);
-        T.store(p.out + o);
+        T.store_nt(p.out + o);
         if (pm.eoff % p.F == 0) {
             size_t so = (size_t)row * H + pm.hd;
             p.emax[so] = (b < e) ? mnat : -1e38f;
@@ -286,8 +286,8 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_packed_kernel(GatFwdP p)
     } else {
         float *pp = p.part + (size_t)slot * gat_fwd_pw(p.HF, H, AUX);
         T.scale(fix);
-        T.store(pp + pm.eoff);
-        if (AUX) { P.scale(fix); P.store(pp + p.HF + pm.eoff); }
+        T.store_nt(pp + pm.eoff);
+        if (AUX) { P.scale(fix); P.store_nt(pp + p.HF + pm.eoff); }
         if (pm.eoff % p.F == 0) {
             float *st = pp + (AUX ? 2 : 1) * p.HF;
             st[pm.hd] = mnat;
@@ -385,8 +385,8 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_edge_stash_kernel(int N, int64_t
         if (k < k1) {
             const size_t rh = (size_t)row * H + h;
             const float ev = fg_lrelu(ar[rh] + ac[(size_t)idx[q] * H + h], slope);
-            e_lrelu[k] = ev;
-            e_softmax[k] = __expf(ev - emax[rh]) / esum[rh];
+            __builtin_nontemporal_store(ev, e_lrelu + k);
+            __builtin_nontemporal_store(__expf(ev - emax[rh]) / esum[rh], e_softmax + k);
         }
         rem += 64u;
         const unsigned adv = rem / uh;
@@ -457,7 +457,7 @@ __device__ __forceinline__ void gat_bwd_finish(const GatBwdP &p, int col, int la
         d[r] = 0.f;
         if (lm.ok[r]) {
             size_t o = (size_t)col * p.HF + lm.eoff[r];
-            T[r].store(p.gfeat + o);
+            T[r].store_nt(p.gfeat + o);
             fg_vec<VEC> g2 = T[r].lin(p.slope, 1.f - p.slope, P[r]);
             fg_vec<VEC> xv; xv.load(p.x + o);
             d[r] = xv.dot(g2);
@@ -563,8 +563,8 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_kernel(GatBwdP p)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if (!(FULL || lm.ok[r])) continue;
-            T[r].store(pp + lm.eoff[r]);
-            P[r].store(pp + p.HF + lm.eoff[r]);
+            T[r].store_nt(pp + lm.eoff[r]);
+            P[r].store_nt(pp + p.HF + lm.eoff[r]);
             if (lm.eoff[r] % p.F == 0) pp[2 * p.HF + lm.hd[r]] = z[r];
         }
     }
@@ -636,8 +636,8 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
         gat_bwd_finish<4, 1>(p, col, lane, scr, lm, Ts, Ps, zs);
     } else if (lm.ok[0]) {
         float *pp = p.part + (size_t)slot * gat_bwd_pw(p.HF, H);
-        T.store(pp + pm.eoff);
-        P.store(pp + p.HF + pm.eoff);
+        T.store_nt(pp + pm.eoff);
+        P.store_nt(pp + p.HF + pm.eoff);
         if (pm.eoff % p.F == 0) pp[2 * p.HF + pm.hd] = z;
     }
 }

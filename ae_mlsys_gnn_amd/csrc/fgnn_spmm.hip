@@ -22,7 +22,7 @@ __device__ __forceinline__ void spmm_store_row(const SpmmP &p, int row, const fg
     if (!p.sum_h) {
 #pragma unroll
         for (int r = 0; r < R; ++r)
-            if (FULL || lm.ok[r]) T[r].store(p.out + (size_t)row * p.HF + lm.eoff[r]);
+            if (FULL || lm.ok[r]) T[r].store_nt(p.out + (size_t)row * p.HF + lm.eoff[r]);
         return;
     }
 #pragma unroll
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(FGNN_TPB) void spmm_kernel(SpmmP p, WF wf, int shar
         float *dst = p.part + (size_t)slot * spmm_pw(p.HF);
 #pragma unroll
         for (int r = 0; r < R; ++r)
-            if (FULL || lm.ok[r]) T[r].store(dst + lm.eoff[r]);
+            if (FULL || lm.ok[r]) T[r].store_nt(dst + lm.eoff[r]);
     }
 }
 
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(FGNN_TPB) void spmm_packed_kernel(SpmmP p, WF wf, i
     if (slot < 0) {
         spmm_store_row<4, 1, false>(p, row, lm, Ts, scr);
     } else if (lm.ok[0]) {
-        T.store(p.part + (size_t)slot * spmm_pw(p.HF) + pm.eoff);
+        T.store_nt(p.part + (size_t)slot * spmm_pw(p.HF) + pm.eoff);
     }
 }
 
@@ -385,7 +385,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p)
     float *dst = slot < 0 ? p.gfeat + (size_t)col * p.HF : p.part + (size_t)slot * spmm_pw(p.HF);
 #pragma unroll
     for (int r = 0; r < R; ++r)
-        if (FULL || lm.ok[r]) T[r].store(dst + lm.eoff[r]);
+        if (FULL || lm.ok[r]) T[r].store_nt(dst + lm.eoff[r]);
 }
 
 // The same pass for rows narrower than a wave, G column entries per load instruction (see
@@ -453,7 +453,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_packed_kernel(GmmBwdP p)
     }
     fg_pack_reduce<G>(T, lane);
     float *dst = slot < 0 ? p.gfeat + (size_t)col * p.HF : p.part + (size_t)slot * spmm_pw(p.HF);
-    if (pm.ok && pm.grp == 0) T.store(dst + pm.eoff);
+    if (pm.ok && pm.grp == 0) T.store_nt(dst + pm.eoff);
 }
 
 // Closed-form derivatives of w[p,k] = exp(-0.5 sum_d ((pseudo[p,d]-mu[k,d])*isg[k,d])^2), one edge per

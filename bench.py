@@ -31,7 +31,7 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published peak
 # profiles/other_workloads.md); all kernels of the entry point summed.
 # They bound the HBM traffic from above.  None = not measured for that workload.
 MEASURED_TRAFFIC_BYTES = {
-    "gat_c2": {"fwd": 37_940_294_041, "bwd": 34_175_510_118},
+    "gat_c2": {"fwd": 37136911667, "bwd": 33567448883},
     "gat_c5_layer1": {"fwd": 72_099_949_465, "bwd": 81_156_805_427},
     "gmm_c4": {"fwd": 1_154_166_988, "bwd": 1_514_758_144},
     "edgeconv_c3": {"fwd": 123_305_574, "bwd": 73_504_972},

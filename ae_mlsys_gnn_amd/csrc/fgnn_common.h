@@ -326,6 +326,21 @@ __device__ __forceinline__ float fg_head_reduce(float *scr, const float (&part)[
     fg_wave_lds_sync();
     return acc;
 }
+// The same sums for a handful of heads without LDS: one masked wave sum per head.
+#define FGNN_FEW_HEADS 8
+template <int VEC, int R>
+__device__ __forceinline__ float fg_head_reduce_few(const float (&part)[R], const fg_lanemap<VEC, R> &lm, int lane, int H)
+{
+    float res = 0.f;
+    for (int h = 0; h < H; ++h) {
+        float v = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) v += (lm.ok[r] && lm.hd[r] == h) ? part[r] : 0.f;
+        float s = fg_wave_sum(v);
+        if (lane == h) res = s;
+    }
+    return res;
+}
 // Rows narrower than a wave (H*F <= 128 floats): G = 2, 4 or 8 entries of the row are gathered by
 // one load instruction.  The wave is cut into G groups of LPR = 64/G lanes; group g takes entries
 // g, g+G, ... of a chunk, lane `sub` of a group owns floats [4*sub, 4*sub+4) of the feature row.  Each
@@ -352,20 +367,5 @@ __device__ __forceinline__ void fg_pack_reduce(fg_vec<4> &T, int lane)
         T.v.x += fg_bperm(T.v.x, lane ^ step); T.v.y += fg_bperm(T.v.y, lane ^ step);
         T.v.z += fg_bperm(T.v.z, lane ^ step); T.v.w += fg_bperm(T.v.w, lane ^ step);
     }
-}
-// The same sums for a handful of heads without LDS: one masked wave sum per head.
-#define FGNN_FEW_HEADS 8
-template <int VEC, int R>
-__device__ __forceinline__ float fg_head_reduce_few(const float (&part)[R], const fg_lanemap<VEC, R> &lm, int lane, int H)
-{
-    float res = 0.f;
-    for (int h = 0; h < H; ++h) {
-        float v = 0.f;
-#pragma unroll
-        for (int r = 0; r < R; ++r) v += (lm.ok[r] && lm.hd[r] == h) ? part[r] : 0.f;
-        float s = fg_wave_sum(v);
-        if (lane == h) res = s;
-    }
-    return res;
 }
 #endif  // __HIPCC__

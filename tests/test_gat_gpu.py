@@ -190,3 +190,25 @@ def test_gat_negative_slope_outside_unit_interval():
     _run(g, 4, 16, slope=1.5)
     _run(g, 4, 16, slope=0.0)
     _run(g, 4, 16, slope=1.0)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_gat_random_shapes_and_graphs(seed):
+    """Seeded sweep over head counts, widths (all lane layouts: 128-bit, packed, scalar, multi-slab),
+    slopes, variants and graph kinds."""
+    import random
+    rnd = random.Random(1000 + seed)
+    h = rnd.choice([1, 1, 2, 3, 4, 5, 8, 12])
+    f = rnd.choice([1, 2, 4, 7, 8, 12, 16, 20, 31, 32, 47, 64, 100, 128])
+    while h * f > 1024:
+        f //= 2
+    slope = rnd.choice([0.2, 0.2, 0.01, 0.5, 1.0])
+    variant = rnd.choice(["sm", "sm", "stash", "fusescatter"])
+    kind = rnd.choice(["rmat", "uniform", "degrees"])
+    if kind == "rmat":
+        g = graphs.rmat_graph(rnd.randrange(50, 1500), rnd.randrange(500, 40000), seed=seed)
+    elif kind == "uniform":
+        g = graphs.uniform_graph(rnd.randrange(10, 3000), rnd.randrange(10, 20000), seed=seed, self_loops=rnd.random() < 0.7)
+    else:
+        g = degree_edge_graph(seed=100 + seed)
+    _run(g, h, f, slope=slope, seed=seed, variant=variant)

@@ -1,7 +1,8 @@
 """Full-size checks at the benchmark configurations.  Where the CPU oracle is too slow (the
 115 M-edge GAT graph) the checks are size-independent properties of the math: attention rows sum
 to one, zero attention is the neighbour mean, linearity in the features, the column-sum checksum
-of grad_feat, the slope == 1 shift invariance, and the transpose round trip of csr2csc.  EdgeConv
+of grad_feat, the slope == 1 shift invariance, and the transpose round trip of csr2csc; on top of
+that a sample of rows and columns of the full-size graph is compared with float64 torch math.  EdgeConv
 (C3) and GMMConv (C4) are small enough to compare with the oracle at full size."""
 import numpy as np
 import pytest
@@ -207,3 +208,78 @@ def test_c5_gat_properties(c5_graph, h, f):
     gx3 = gat_native.gat_backward(0.2, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, o3[1], o3[2], x * 3.0, ar, ac, go,
                                   out_feat=o3[0], out2=o3[3], cc=o3[4])[0]
     assert torch.equal(gx3, gx)
+
+
+def _segment_sums(vals, deg):
+    """Sums of consecutive segments of `vals` ([P, H], float64) with lengths `deg` (all >= 1), by
+    differences of a running sum (float64 index_add_ serialises on its atomics)."""
+    c = torch.cumsum(vals, 0)[torch.cumsum(deg, 0) - 1]
+    return c - torch.cat([torch.zeros_like(c[:1]), c[:-1]])
+
+
+def _rows_float64(g, rows, ar, ac, x, slope, go=None, need_out=True):
+    """Float64 restatement of the GAT math for the given destination rows only (all their edges), on
+    the device with plain torch ops: returns out[rows] and, with go, grad_attn_row[rows] and the
+    per-edge (position, g) pairs needed for column sums."""
+    rp = g.row_ptr.long()
+    deg = rp[rows + 1] - rp[rows]
+    seg = torch.repeat_interleave(torch.arange(rows.numel(), device=DEV), deg)            # edge -> index into rows
+    first = torch.cumsum(deg, 0) - deg                                                      # index of each row's first edge in the list
+    pos = rp[rows][seg] + (torch.arange(seg.numel(), device=DEV) - first[seg])              # CSR positions of the listed edges
+    src = g.col_ind[pos].long()
+    e = torch.nn.functional.leaky_relu(ar[rows].double()[seg] + ac[src].double(), slope)   # [P, H]
+    m = torch.full((rows.numel(), e.shape[1]), -float("inf"), dtype=torch.float64, device=DEV).scatter_reduce(
+        0, seg.view(-1, 1).expand_as(e), e, "amax")
+    w = torch.exp(e - m[seg])
+    s = _segment_sums(w, deg)
+    alpha = w / s[seg]
+    h, f = x.shape[1], x.shape[2]
+    out = torch.zeros(rows.numel(), h, f, dtype=torch.float64, device=DEV)
+    ge = torch.empty_like(alpha) if go is not None else None
+    for a in range(0, pos.numel(), 1 << 20):                                               # chunks: [P, H, F] in float64 is large
+        sl = slice(a, min(a + (1 << 20), pos.numel()))
+        xs = x[src[sl]].double()
+        if need_out:
+            out.index_add_(0, seg[sl], alpha[sl].unsqueeze(-1) * xs)
+        if go is not None:
+            ge[sl] = (go[rows].double()[seg[sl]] * xs).sum(-1)
+    if go is None:
+        return out
+    ws = _segment_sums(alpha * ge, deg)
+    gscore = alpha * (ge - ws[seg]) * torch.where(e > 0, 1.0, slope)
+    gar = _segment_sums(gscore, deg)
+    return out, gar, pos, src, seg, alpha, gscore
+
+
+def test_c2_gat_sampled_rows_and_columns_vs_float64(c2_graph):
+    """Direct parity at full size on a sample: 100 destination rows (forward, grad_attn_row) and 6
+    source columns with all the rows they touch (grad_feat, grad_attn_col), against float64 torch math."""
+    from ae_mlsys_gnn_amd.operators.fused_gat import gat_native
+    g = c2_graph
+    n, h, f, slope = g.n, 8, 32, 0.2
+    gen = torch.Generator(device=DEV).manual_seed(7)
+    ar = torch.randn(n, h, device=DEV, generator=gen)
+    ac = torch.randn(n, h, device=DEV, generator=gen)
+    x = torch.randn(n, h, f, device=DEV, generator=gen)
+    go = torch.randn(n, h, f, device=DEV, generator=gen)
+    o = gat_native.gat_forward(ar, ac, g.row_ptr, g.col_ind, slope, x)
+    gx, gar, gac = gat_native.gat_backward(slope, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, o[1], o[2], x, ar, ac, go,
+                                           out_feat=o[0], out2=o[3], cc=o[4])
+    rows = torch.randperm(n, device=DEV, generator=gen)[:100]
+    ref_out, ref_gar = _rows_float64(g, rows, ar, ac, x, slope, go)[:2]
+    assert_close(o[0][rows], ref_out, "out on sampled rows at C2")
+    scale = float(go.abs().max() * x.abs().max() * f)
+    assert_close(gar[rows], ref_gar, "grad_attn_row on sampled rows at C2", atol=1e-5 * scale)
+    # columns of modest length, so that the rows they touch stay a few million edges
+    cp = g.col_ptr.long()
+    cdeg = cp[1:] - cp[:-1]
+    cand = torch.nonzero((cdeg >= 20) & (cdeg <= 60)).squeeze(1)
+    cols = cand[torch.randperm(cand.numel(), device=DEV, generator=gen)[:6]]
+    touched = torch.unique(torch.cat([g.row_ind[a:b].long() for a, b in zip(cp[cols].tolist(), cp[cols + 1].tolist())]))
+    _, _, pos, src, seg, alpha, gscore = _rows_float64(g, touched, ar, ac, x, slope, go, need_out=False)
+    for j in cols.tolist():
+        mine = src == j
+        rws = touched[seg[mine]]
+        want_gx = (alpha[mine].unsqueeze(-1) * go[rws].double()).sum(0)
+        assert_close(gx[j], want_gx, "grad_feat of column %d at C2" % j)
+        assert_close(gac[j], gscore[mine].sum(0), "grad_attn_col of column %d at C2" % j, atol=1e-5 * scale)

@@ -24,7 +24,7 @@ _SIGNATURES = {
     "fgnn_version": (c_int, []),
     "fgnn_last_error": (ctypes.c_char_p, []),
     "fgnn_schedule_create": (c_int, [c_void_p, c_int, c_int, c_void_p, ctypes.POINTER(c_void_p)]),
-    "fgnn_schedule_create_bucketed": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, ctypes.POINTER(c_void_p)]),
+    "fgnn_schedule_create_bucketed": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, ctypes.POINTER(c_void_p)]),
     "fgnn_schedule_destroy": (None, [c_void_p]),
     "fgnn_schedule_num_items": (c_int, [c_void_p]),
     "fgnn_schedule_num_partials": (c_int, [c_void_p]),
@@ -124,7 +124,7 @@ class Schedule:
     """Degree-binned work list of one pointer array (row_ptr or col_ptr).  With `idx_tensor` it is
     the XCD-aware form: long rows are cut by source bucket and each XCD gets one bucket."""
 
-    def __init__(self, ptr_tensor, seg_len=0, idx_tensor=None, min_deg=0):
+    def __init__(self, ptr_tensor, seg_len=0, idx_tensor=None, min_deg=0, with_positions=True):
         require_cuda(ptr_tensor)
         self.ptr_tensor = as_i32(ptr_tensor)      # keeps the device memory alive
         self.idx_tensor = None if idx_tensor is None else as_i32(idx_tensor)
@@ -136,7 +136,7 @@ class Schedule:
                                                  ctypes.byref(handle)), "fgnn_schedule_create")
             else:
                 check(lib().fgnn_schedule_create_bucketed(ptr(self.ptr_tensor), ptr(self.idx_tensor), self.n_rows, int(seg_len),
-                                                          int(min_deg), stream_ptr(), ctypes.byref(handle)),
+                                                          int(min_deg), int(bool(with_positions)), stream_ptr(), ctypes.byref(handle)),
                       "fgnn_schedule_create_bucketed")
         self.handle = handle
         self.n_items = lib().fgnn_schedule_num_items(handle)
@@ -167,25 +167,33 @@ def xcd_buckets_enabled(n_rows: int, n_edges: int) -> bool:
     return n_rows > 0 and n_edges >= 64 * n_rows
 
 
-def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None) -> Schedule:
+def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True) -> Schedule:
     """Cached schedule of a pointer array.  The cache entry holds the tensors, so their device
     addresses cannot be reused while the entry lives; in-place edits bump `_version`.
-    idx_tensor: the index array, for operators that may use an XCD-aware schedule."""
+    idx_tensor: the index array, for operators that may use an XCD-aware schedule.
+    need_positions: whether the operator has per-edge tensors (an XCD-aware schedule then also keeps
+    the caller's position of every entry, 4*E bytes more); a schedule with positions serves both."""
     if seg_len is None:
         seg_len = default_seg_len()
     if idx_tensor is not None and not xcd_buckets_enabled(ptr_tensor.numel() - 1, idx_tensor.numel()):
         idx_tensor = None
     min_deg = int(os.environ.get("FGNN_BUCKET_MIN_DEG", "0"))
-    key = (ptr_tensor.data_ptr(), ptr_tensor.numel(), ptr_tensor.device.index, ptr_tensor._version, int(seg_len),
-           None if idx_tensor is None else (idx_tensor.data_ptr(), idx_tensor._version, min_deg))
-    s = _sched_cache.get(key)
+
+    def key(pos):
+        return (ptr_tensor.data_ptr(), ptr_tensor.numel(), ptr_tensor.device.index, ptr_tensor._version, int(seg_len),
+                None if idx_tensor is None else (idx_tensor.data_ptr(), idx_tensor._version, min_deg, pos))
+    k = key(True)
+    s = _sched_cache.get(k)
+    if s is None and not need_positions and idx_tensor is not None:
+        k = key(False)
+        s = _sched_cache.get(k)
     if s is None:
-        s = Schedule(ptr_tensor, seg_len, idx_tensor, min_deg)
-        _sched_cache[key] = s
+        s = Schedule(ptr_tensor, seg_len, idx_tensor, min_deg, with_positions=need_positions)
+        _sched_cache[k] = s
         while len(_sched_cache) > _SCHED_CACHE_MAX:
             _sched_cache.popitem(last=False)
     else:
-        _sched_cache.move_to_end(key)
+        _sched_cache.move_to_end(k)
     return s
 
 

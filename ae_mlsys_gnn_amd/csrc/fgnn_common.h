@@ -71,6 +71,8 @@ struct fgnn_schedule {
 // caller's edge positions (NULL = identity).
 static inline const int32_t *fgnn_sched_idx(const fgnn_schedule *s, const int32_t *idx) { return (s && s->n_buckets > 0) ? s->bidx_dev : idx; }
 static inline const int32_t *fgnn_sched_pos(const fgnn_schedule *s) { return (s && s->n_buckets > 0) ? s->bpos_dev : nullptr; }
+// false for an XCD-aware schedule built without the position map: operators with per-edge tensors must refuse it
+static inline bool fgnn_sched_has_pos(const fgnn_schedule *s) { return !s || s->n_buckets == 0 || s->n_edges == 0 || s->bpos_dev != nullptr; }
 
 #define FGNN_NUM_XCD 8      // workgroup w of a dispatch runs on XCD w % 8 (gfx942 / gfx950, SPX mode)
 // Source bucket of a node id: the top 3 bits of a multiplicative hash, so hot ids spread evenly.

@@ -23,7 +23,7 @@
 
 struct GatFwdP {
     const fgnn_item *items; int n_items;
-    const int *ptr; const int *idx; const int *pos;     // pos: caller's edge position of entry q of idx (NULL = q)
+    const int *ptr; const int *idx;
     const float *ar; const float *ac; const float *x;
     float *out; float *emax; float *esum; float *out2; float *cc;
     float *part;
@@ -718,7 +718,7 @@ static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_
     GatFwdP p;
     p.items = sched ? sched->items_dev : nullptr;
     p.n_items = sched ? sched->n_items : N;
-    p.ptr = row_ptr; p.idx = fgnn_sched_idx(sched, col_ind); p.pos = fgnn_sched_pos(sched); p.ar = attn_row; p.ac = attn_col; p.x = in_feat;
+    p.ptr = row_ptr; p.idx = fgnn_sched_idx(sched, col_ind); p.ar = attn_row; p.ac = attn_col; p.x = in_feat;
     p.out = out; p.emax = edge_max; p.esum = edge_sum; p.out2 = aux_out2; p.cc = aux_c;
     p.part = (float *)workspace; p.N = N; p.H = H; p.F = F; p.HF = HF; p.slope = slope;
     if (sched && sched->n_partials > 0) {
@@ -815,6 +815,7 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
                  FGNN_ERR_NULL, "fgnn_gat_backward: NULL argument");
     const bool stash = e_softmax != nullptr;
     FGNN_REQUIRE(!stash || permute, FGNN_ERR_NULL, "fgnn_gat_backward: stashed attention needs permute");
+    FGNN_REQUIRE(!stash || fgnn_sched_has_pos(sched_csc), FGNN_ERR_SCHEDULE, "fgnn_gat_backward: stashed attention needs a schedule built with edge positions");
     (void)e_lrelu;      // the sign of the pre-activation is taken from attn_row + attn_col
     const bool recompute = !(out_feat && aux_out2 && aux_c);
     FGNN_REQUIRE(!recompute || (row_ptr && (col_ind || E == 0)), FGNN_ERR_NULL, "fgnn_gat_backward: recomputing the forward needs row_ptr/col_ind");

@@ -61,7 +61,7 @@ __global__ __launch_bounds__(FGNN_TPB) void bucket_partition_kernel(int n_rows, 
             if (bk == b) dst = off[b] + __popcll(m & lt);
             off[b] += __popcll(m);
         }
-        if (ok) { bidx[dst] = id; bpos[dst] = q; }
+        if (ok) { bidx[dst] = id; if (bpos) bpos[dst] = q; }
     }
 }
 
@@ -178,7 +178,7 @@ extern "C" int fgnn_schedule_create(const int32_t *ptr_dev, int n_rows, int seg_
 // XCD's L2 then sees one eighth of the gathered rows, which is what lets the hot ones stay resident.
 // Shorter rows stay whole and are dealt round-robin.  Segments are partial results merged by row.
 extern "C" int fgnn_schedule_create_bucketed(const int32_t *ptr_dev, const int32_t *idx_dev, int n_rows, int seg_len, int min_deg,
-                                             void *stream, fgnn_schedule_t **out)
+                                             int with_positions, void *stream, fgnn_schedule_t **out)
 {
     FGNN_REQUIRE(ptr_dev && out, FGNN_ERR_NULL, "fgnn_schedule_create_bucketed: NULL argument");
     FGNN_REQUIRE(n_rows >= 0, FGNN_ERR_SHAPE, "fgnn_schedule_create_bucketed: n_rows=%d", n_rows);
@@ -200,7 +200,7 @@ extern "C" int fgnn_schedule_create_bucketed(const int32_t *ptr_dev, const int32
         int32_t *bcnt_dev = nullptr;
         hipError_t err = hipMalloc((void **)&bcnt_dev, bcnt.size() * sizeof(int32_t));
         if (err == hipSuccess && n_edges > 0) err = hipMalloc((void **)&s->bidx_dev, (size_t)n_edges * sizeof(int32_t));
-        if (err == hipSuccess && n_edges > 0) err = hipMalloc((void **)&s->bpos_dev, (size_t)n_edges * sizeof(int32_t));
+        if (err == hipSuccess && n_edges > 0 && with_positions) err = hipMalloc((void **)&s->bpos_dev, (size_t)n_edges * sizeof(int32_t));
         if (err == hipSuccess) {
             hipLaunchKernelGGL(bucket_partition_kernel, dim3((unsigned)((n_rows + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, st,
                                n_rows, ptr_dev, idx_dev, s->bidx_dev, s->bpos_dev, bcnt_dev);

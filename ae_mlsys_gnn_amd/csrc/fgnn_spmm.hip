@@ -204,6 +204,7 @@ static int spmm_checks(const char *fn, int N, int64_t E, int H, int F, const fgn
                      "%s: schedule was built for another pointer array", fn);
         FGNN_REQUIRE(sched->n_buckets == 0 || sched->idx_src_dev == idx, FGNN_ERR_SCHEDULE,
                      "%s: XCD-aware schedule was built from another index array", fn);
+        FGNN_REQUIRE(fgnn_sched_has_pos(sched), FGNN_ERR_SCHEDULE, "%s: the schedule was built without edge positions", fn);
     }
     return 0;
 }

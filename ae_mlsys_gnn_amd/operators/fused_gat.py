@@ -41,7 +41,7 @@ class gat_native:
         cc = torch.empty((n, h), dtype=torch.float32, device=dev) if need_aux else None
         e_lrelu = torch.empty((e, h), dtype=torch.float32, device=dev) if stash else None
         e_soft = torch.empty((e, h), dtype=torch.float32, device=dev) if stash else None
-        sched = schedule_for(row_ptr, idx_tensor=col_ind) if use_schedule else None
+        sched = schedule_for(row_ptr, idx_tensor=col_ind, need_positions=False) if use_schedule else None
         sh = sched.handle if sched is not None else None
         with torch.cuda.device(dev):
             ws, wsb = workspace(lib().fgnn_gat_forward_workspace_bytes(sh, h, f), dev)
@@ -65,8 +65,8 @@ class gat_native:
         grad_attn_row = torch.empty((n, h), dtype=torch.float32, device=dev)
         grad_attn_col = torch.empty((n, h), dtype=torch.float32, device=dev)
         recompute = out_feat is None or out2 is None or cc is None
-        sched_csc = schedule_for(col_ptr, idx_tensor=row_ind) if use_schedule else None
-        sched_csr = schedule_for(row_ptr, idx_tensor=col_ind) if (use_schedule and recompute) else None
+        sched_csc = schedule_for(col_ptr, idx_tensor=row_ind, need_positions=e_soft is not None) if use_schedule else None
+        sched_csr = schedule_for(row_ptr, idx_tensor=col_ind, need_positions=False) if (use_schedule and recompute) else None
         hc = sched_csc.handle if sched_csc is not None else None
         hr = sched_csr.handle if sched_csr is not None else None
         with torch.cuda.device(dev):

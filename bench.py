@@ -190,8 +190,8 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
     g, t_gen, t_csc = build_gat_graph(n, e_target, dev)
     e = g.n_edges
     t0 = time.time()
-    s_csr = _lib.schedule_for(g.row_ptr, idx_tensor=g.col_ind)
-    s_csc = _lib.schedule_for(g.col_ptr, idx_tensor=g.row_ind)
+    s_csr = _lib.schedule_for(g.row_ptr, idx_tensor=g.col_ind, need_positions=False)
+    s_csc = _lib.schedule_for(g.col_ptr, idx_tensor=g.row_ind, need_positions=False)
     torch.cuda.synchronize()
     t_sched = time.time() - t0
     slope = 0.2

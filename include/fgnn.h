@@ -51,10 +51,14 @@ int     fgnn_schedule_create(const int32_t *ptr_dev, int n_rows, int seg_len, vo
 /* XCD-aware variant for the gather kernels (fused GAT, mhspmm, GMMConv): rows longer than min_deg
  * (<= 0: 64) entries are cut by source bucket (8 buckets, one per XCD) and workgroup w only gets
  * segments of bucket w % 8, so each XCD's L2 sees one eighth of the gathered feature rows.  The
- * schedule keeps its own bucket-ordered copy of `idx` and the original position of every entry
- * (8*E bytes of device memory); `idx` must be the array later passed to the operator. */
+ * schedule keeps its own bucket-ordered copy of `idx` (4*E bytes of device memory) and, with
+ * with_positions != 0, the original position of every entry (another 4*E bytes): operators with
+ * per-edge tensors (stashed GAT attention, mhspmm weights, GMMConv pseudo-coordinates) need it and
+ * return FGNN_ERR_SCHEDULE without; the recomputing fused GAT does not.  `idx` must be the array later
+ * passed to the operator. */
 int     fgnn_schedule_create_bucketed(const int32_t *ptr_dev, const int32_t *idx_dev, int n_rows,
-                                      int seg_len, int min_deg, void *stream, fgnn_schedule_t **out);
+                                      int seg_len, int min_deg, int with_positions, void *stream,
+                                      fgnn_schedule_t **out);
 void    fgnn_schedule_destroy(fgnn_schedule_t *s);
 int     fgnn_schedule_num_items(const fgnn_schedule_t *s);
 int     fgnn_schedule_num_partials(const fgnn_schedule_t *s);   /* segments of split rows */

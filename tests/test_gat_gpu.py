@@ -149,6 +149,27 @@ def test_xcd_schedule_must_match_index_array():
     assert rc == -6 and b"another index array" in lib().fgnn_last_error()
 
 
+def test_schedule_without_positions_is_refused_by_per_edge_operators():
+    """An XCD-aware schedule built without the position map serves the recomputing GAT (the default
+    path of fused_gat_op) but not operators with per-edge tensors."""
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd._lib import lib, ptr, stream_ptr
+    g = graphs.add_csc_torch(graphs.rmat_graph(500, 20000, seed=1)).to("cuda:0")
+    s = _lib.Schedule(g.row_ptr, 0, g.col_ind, 16, with_positions=False)
+    n, h, f = g.n, 2, 8
+    x = torch.randn(n, h, f, device="cuda:0")
+    att = torch.rand(g.n_edges, h, device="cuda:0")
+    out = torch.empty_like(x)
+    ws = torch.empty(lib().fgnn_mhspmm_workspace_bytes(s.handle, h, f) // 4 + 4, device="cuda:0")
+    rc = lib().fgnn_mhspmm(n, g.n_edges, h, f, ptr(g.row_ptr), ptr(g.col_ind), None, ptr(att), ptr(x), ptr(out), s.handle, ptr(ws),
+                           ws.numel() * 4, stream_ptr())
+    assert rc == -6 and b"without edge positions" in lib().fgnn_last_error()
+    s2 = _lib.Schedule(g.row_ptr, 0, g.col_ind, 16, with_positions=True)
+    rc = lib().fgnn_mhspmm(n, g.n_edges, h, f, ptr(g.row_ptr), ptr(g.col_ind), None, ptr(att), ptr(x), ptr(out), s2.handle, ptr(ws),
+                           ws.numel() * 4, stream_ptr())
+    assert rc == 0
+
+
 def test_gat_degenerate_graphs():
     """No edges at all, isolated nodes between connected ones, a single node with a self loop."""
     from ae_mlsys_gnn_amd.operators import fused_gat as fg

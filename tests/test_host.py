@@ -152,5 +152,5 @@ def test_more_argument_errors_without_gpu():
     assert l.fgnn_coo2csr(4, 4, 3, None, None, 1, None, None, None, None, None, 0, None) == -1
     out = ctypes.c_void_p()
     assert l.fgnn_schedule_create(None, 4, 0, None, ctypes.byref(out)) == -1
-    assert l.fgnn_schedule_create_bucketed(None, None, 4, 0, 0, None, ctypes.byref(out)) == -1
+    assert l.fgnn_schedule_create_bucketed(None, None, 4, 0, 0, 1, None, ctypes.byref(out)) == -1
     l.fgnn_schedule_destroy(None)                                                  # no-op on NULL

@@ -207,6 +207,19 @@ struct fg_lanemap {
             hd[r] = ok[r] ? eoff[r] / F : 0;
         }
     }
+    // Head-aligned variant for kernels that reduce inside heads with DPP: head h takes lanes
+    // [h*lphp, (h+1)*lphp) (lphp a power of two >= F/VEC), the lanes past F/VEC of a head stay idle.
+    __device__ __forceinline__ void init_padded(int lane, int H, int F, int lphp)
+    {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int li = lane + 64 * r;
+            int h = li / lphp, sub = li - h * lphp;
+            ok[r] = h < H && sub * VEC < F;
+            hd[r] = ok[r] ? h : 0;
+            eoff[r] = ok[r] ? h * F + sub * VEC : 0;
+        }
+    }
 };
 
 // Decode the work item of this wave.  Returns false when there is none.
@@ -289,6 +302,17 @@ static inline int fgnn_pick_lph(int vec, int F)
     if (vec == 4 && (lph == 1 || lph == 2 || lph == 4 || lph == 8 || lph == 16 || lph == 32)) return lph;
     return 0;
 }
+// Lanes per head of the head-aligned lane map (fg_lanemap::init_padded) for a width that is a multiple
+// of 4 but whose quarter is not a power of two; 0 when the dense map already is head-aligned or the
+// padded row would not fit 4 slabs.
+static inline int fgnn_pad_lph(int vec, int H, int F)
+{
+    if (vec != 4 || F % 4 != 0) return 0;
+    int l = 1;
+    while (l * 4 < F) l *= 2;
+    if (l * 4 == F || l > 32 || (int64_t)H * l * 4 > 1024) return 0;
+    return l;
+}
 // Entries of a narrow row gathered per load instruction (1 = one row per wave).
 static inline int fgnn_pick_pack(int vec, int HF)
 {
@@ -358,6 +382,15 @@ struct fg_packmap {
         eoff = (lane % LPR) * 4;
         ok = eoff < HF;
         hd = ok ? eoff / F : 0;
+    }
+    __device__ __forceinline__ void init_padded(int lane, int H, int F, int lphp)      // see fg_lanemap::init_padded
+    {
+        grp = lane / LPR;
+        int li = lane % LPR;
+        int h = li / lphp, sub = li - h * lphp;
+        ok = h < H && sub * 4 < F;
+        hd = ok ? h : 0;
+        eoff = ok ? h * F + sub * 4 : 0;
     }
 };
 // Sum over the G groups; every group ends with the total.

@@ -6,7 +6,7 @@
 // out[p,h] = <a[row,h,:], b[col_ind[p],h,:]> (src/sddmm/mhsddmm.cu:5-81 of the reference, which
 // finds the row of each edge by binary search; here the row is the work item).
 template <int VEC, int R, bool FULL, int LPH>
-__global__ __launch_bounds__(FGNN_TPB) void mhsddmm_kernel(int N, int H, int F, int HF, const int *ptr, const int *idx,
+__global__ __launch_bounds__(FGNN_TPB) void mhsddmm_kernel(int N, int H, int F, int HF, int lphp, const int *ptr, const int *idx,
                                                            const float *a, const float *b, float *out)
 {
     extern __shared__ float lds[];
@@ -16,7 +16,7 @@ __global__ __launch_bounds__(FGNN_TPB) void mhsddmm_kernel(int N, int H, int F, 
     float *scr = lds + fg_wave() * (64 * R);
     const int pb = fg_uni(ptr[row]), pe = fg_uni(ptr[row + 1]);
     fg_lanemap<VEC, R> lm;
-    lm.init(lane, HF, F);
+    if (lphp) lm.init_padded(lane, H, F, lphp); else lm.init(lane, HF, F);      // lphp: head-aligned lanes for DPP sums
     fg_vec<VEC> ar[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ar[r].load(a + (size_t)row * HF + lm.eoff[r]); else ar[r].zero(); }
@@ -64,13 +64,15 @@ extern "C" int fgnn_mhsddmm(int N, int64_t E, int H, int F, const int32_t *row_p
     const int HF = H * F;
     fgnn_rowcfg cfg;
     FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, fgnn_aligned16(a) && fgnn_aligned16(b), &cfg), FGNN_ERR_LIMIT, "fgnn_mhsddmm: unsupported row width %d", HF);
-    const int lph = fgnn_pick_lph(cfg.vec, F);
+    const int lphp = fgnn_pad_lph(cfg.vec, H, F);
+    if (lphp) { int w = H * lphp * 4; cfg.r = w <= 256 ? 1 : w <= 512 ? 2 : 4; cfg.full = false; }
+    const int lph = lphp ? lphp : fgnn_pick_lph(cfg.vec, F);
     const unsigned grid = (unsigned)((N + FGNN_WPB - 1) / FGNN_WPB);
     hipStream_t st = (hipStream_t)stream;
     return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
         return fgnn_dispatch_lph(VEC == 4 ? lph : 0, [&]<int LPH>() -> int {
             hipLaunchKernelGGL((mhsddmm_kernel<VEC, R, FULL, (VEC == 4 ? LPH : 0)>), dim3(grid), dim3(FGNN_TPB),
-                               (size_t)FGNN_WPB * 64 * R * sizeof(float), st, N, H, F, HF, row_ptr, col_ind, a, b, out);
+                               (size_t)FGNN_WPB * 64 * R * sizeof(float), st, N, H, F, HF, lphp, row_ptr, col_ind, a, b, out);
             return fgnn_launch_status("mhsddmm_kernel");
         });
     });
@@ -80,7 +82,7 @@ extern "C" int fgnn_mhsddmm(int N, int64_t E, int H, int F, const int32_t *row_p
 // reference, src/sddmm/sddmm.cpp:12-27, with H heads).  One wave per 64 edges; both rows of an edge
 // are fetched by base-plus-lane-offset loads, four edges in flight.
 template <int VEC, int R, bool FULL, int LPH>
-__global__ __launch_bounds__(FGNN_TPB) void sddmm_coo_kernel(int64_t E, int H, int F, int HF, const int *rows, const int *cols,
+__global__ __launch_bounds__(FGNN_TPB) void sddmm_coo_kernel(int64_t E, int H, int F, int HF, int lphp, const int *rows, const int *cols,
                                                              const float *a, const float *b, float *out)
 {
     extern __shared__ float lds[];
@@ -89,7 +91,7 @@ __global__ __launch_bounds__(FGNN_TPB) void sddmm_coo_kernel(int64_t E, int H, i
     const int lane = fg_lane();
     float *scr = lds + fg_wave() * (64 * R);
     fg_lanemap<VEC, R> lm;
-    lm.init(lane, HF, F);
+    if (lphp) lm.init_padded(lane, H, F, lphp); else lm.init(lane, HF, F);      // lphp: head-aligned lanes for DPP sums
     const int cnt = (int)min((int64_t)64, E - c);
     const int64_t q = c + (lane < cnt ? lane : 0);
     const int ri = rows[q], ci = cols[q];
@@ -136,14 +138,16 @@ extern "C" int fgnn_sddmm_coo(int64_t E, int n_rows, int n_cols, int H, int F, c
     const int HF = H * F;
     fgnn_rowcfg cfg;
     FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, fgnn_aligned16(a) && fgnn_aligned16(b), &cfg), FGNN_ERR_LIMIT, "fgnn_sddmm_coo: unsupported row width %d", HF);
-    const int lph = fgnn_pick_lph(cfg.vec, F);
+    const int lphp = fgnn_pad_lph(cfg.vec, H, F);
+    if (lphp) { int w = H * lphp * 4; cfg.r = w <= 256 ? 1 : w <= 512 ? 2 : 4; cfg.full = false; }
+    const int lph = lphp ? lphp : fgnn_pick_lph(cfg.vec, F);
     const int64_t waves = (E + 63) / 64;
     const unsigned grid = (unsigned)((waves + FGNN_WPB - 1) / FGNN_WPB);
     hipStream_t st = (hipStream_t)stream;
     return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
         return fgnn_dispatch_lph(VEC == 4 ? lph : 0, [&]<int LPH>() -> int {
             hipLaunchKernelGGL((sddmm_coo_kernel<VEC, R, FULL, (VEC == 4 ? LPH : 0)>), dim3(grid), dim3(FGNN_TPB),
-                               (size_t)FGNN_WPB * 64 * R * sizeof(float), st, E, H, F, HF, row_ind, col_ind, a, b, out);
+                               (size_t)FGNN_WPB * 64 * R * sizeof(float), st, E, H, F, HF, lphp, row_ind, col_ind, a, b, out);
             return fgnn_launch_status("sddmm_coo_kernel");
         });
     });

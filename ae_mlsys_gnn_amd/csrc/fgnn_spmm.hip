@@ -294,6 +294,7 @@ struct GmmBwdP {
     float *gfeat; float *gww; float *part;      // gww: [E,K] in CSR position order, gw * w per edge and kernel
     int N, K, dim, F, HF;
     int g_stride;   // floats per grad_out row: HF, or F when grad_out is the gradient of the sum over kernels
+    int lphp;       // > 0: head-aligned lane map with this many lanes per mixture kernel
 };
 
 // One pass over CSC column j (x[j] stays in registers): per in-edge gather grad_out[i], accumulate
@@ -315,7 +316,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p)
     float *wl = lds + fg_wave() * per_wave;
     float *scr = wl + K * 64;
     fg_lanemap<VEC, R> lm;
-    lm.init(lane, p.HF, p.F);
+    if (p.lphp) lm.init_padded(lane, p.K, p.F, p.lphp); else lm.init(lane, p.HF, p.F);
     fg_vec<VEC> T[R], xr[R];
     int goff[R];        // float offset of the lane's slab inside a grad_out row
 #pragma unroll
@@ -330,7 +331,8 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p)
         int cnt = min(64, e - c);
         int qq = ok ? q : c;
         int id = p.idx[qq];
-        int posv = p.permute[p.pos ? p.pos[qq] : qq];
+        int posv = p.pos ? p.pos[qq] : qq;
+        if (p.permute) posv = p.permute[posv];      // NULL: pseudo and gww are in this pass's own (CSC) order
         // the first rows are requested before the weights are formed: the pseudo-coordinate fetch
         // (itself behind the permute fetch) then overlaps with the row fetches
         constexpr int UG = (R >= 8) ? 1 : 8 / R;
@@ -405,7 +407,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_packed_kernel(GmmBwdP p)
     const int lane = fg_lane();
     float *wl = lds + fg_wave() * per_wave;
     fg_packmap<G> pm;
-    pm.init(lane, p.HF, p.F);
+    if (p.lphp) pm.init_padded(lane, p.K, p.F, p.lphp); else pm.init(lane, p.HF, p.F);
     fg_vec<4> T, xr;
     T.zero();
     if (pm.ok) xr.load(p.x + (size_t)col * p.HF + pm.eoff); else xr.zero();
@@ -418,7 +420,8 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_packed_kernel(GmmBwdP p)
         int cnt = min(64, e - c);
         int qq = ok ? q : c;
         int id = p.idx[qq];
-        int posv = p.permute[p.pos ? p.pos[qq] : qq];
+        int posv = p.pos ? p.pos[qq] : qq;
+        if (p.permute) posv = p.permute[posv];      // NULL: pseudo and gww are in this pass's own (CSC) order
         const float *ps = p.pseudo + (size_t)(unsigned)posv * dim;
         for (int k = 0; k < K; ++k) {
             float acc = 0.f;
@@ -596,7 +599,7 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
     int rc = spmm_checks("fgnn_gmm_backward", N, E, K, F, sched_csc, col_ptr, row_ind);
     if (rc) return rc;
     FGNN_REQUIRE(dim >= 1 && dim <= 64 && K * dim <= 1024, FGNN_ERR_LIMIT, "fgnn_gmm_backward: dim=%d K*dim=%d unsupported", dim, K * dim);
-    FGNN_REQUIRE(col_ptr && (row_ind || E == 0) && (permute || E == 0) && node_feat && (pseudo || E == 0) && mu && inv_sigma &&
+    FGNN_REQUIRE(col_ptr && (row_ind || E == 0) && node_feat && (pseudo || E == 0) && mu && inv_sigma &&
                      grad_out && grad_feat && (grad_pseudo || E == 0) && grad_mu && grad_sigma,
                  FGNN_ERR_NULL, "fgnn_gmm_backward: NULL argument");
     FGNN_REQUIRE(sched_csc, FGNN_ERR_SCHEDULE, "fgnn_gmm_backward: a schedule of col_ptr is required");
@@ -618,12 +621,21 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
         p.pos = fgnn_sched_pos(sched_csc); p.permute = permute;
         p.x = node_feat; p.g = grad_out; p.pseudo = pseudo; p.mu = mu; p.isg = inv_sigma; p.gfeat = grad_feat; p.gww = gww;
         p.part = part; p.N = N; p.K = K; p.dim = dim; p.F = F; p.HF = HF; p.g_stride = sum_kernels ? F : HF;
-        const int lph = fgnn_pick_lph(cfg.vec, F);
+        // widths like 44 or 48 (quarter not a power of two): head-aligned lane map, so the per-edge dot
+        // products still reduce with DPP and narrow rows still pack
+        p.lphp = fgnn_pad_lph(cfg.vec, K, F);
+        int lanes_hf = HF;          // floats the lane map spans
+        if (p.lphp) {
+            lanes_hf = K * p.lphp * 4;
+            cfg.r = lanes_hf <= 256 ? 1 : lanes_hf <= 512 ? 2 : 4;
+            cfg.full = false;
+        }
+        const int lph = p.lphp ? p.lphp : fgnn_pick_lph(cfg.vec, F);
         const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
         rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
             size_t shm = ((size_t)FGNN_WPB * (K * 64 + 64 * R) + 2 * KD) * sizeof(float);
             FGNN_REQUIRE(shm <= 64 * 1024, FGNN_ERR_LIMIT, "fgnn_gmm_backward: K=%d, dim=%d need %zu bytes of LDS per workgroup (limit 64 KiB)", K, dim, shm);
-            const int pack = lph > 0 ? fgnn_pick_pack(cfg.vec, HF) : 1;
+            const int pack = lph > 0 ? fgnn_pick_pack(cfg.vec, lanes_hf) : 1;
             int rc2 = fgnn_dispatch_lph(VEC == 4 ? lph : 0, [&]<int LPH>() -> int {
                 if constexpr (VEC == 4 && R == 1 && LPH > 0 && LPH <= 32) {
                     // a mixture kernel's LPH lanes must fit inside one group of 64/pack lanes

@@ -6,7 +6,7 @@ import torch as th
 from torch import nn
 from torch.nn import init
 
-from ..operators.fused_gmmconv import GmmConvFuseSum, GmmConvStash
+from ..operators.fused_gmmconv import GmmConvFuseSum, GmmConvFuseSumTwoOrders, GmmConvStash
 
 
 class _GMMBase(nn.Module):
@@ -48,12 +48,20 @@ class _GMMBase(nn.Module):
     def set_allow_zero_in_degree(self, set_value):
         self._allow_zero_in_degree = set_value
 
-    def forward(self, rowptr, colind, colptr, rowind, permute, feat, pseudo):
+    def forward(self, rowptr, colind, colptr, rowind, permute, feat, pseudo, pseudo_csc=None):
+        """pseudo_csc (GMMConv only): the same pseudo-coordinates in CSC order, pseudo[permute], built by
+        the caller from its own CSC-ordered edge data.  The backward then works in CSC order throughout
+        and the gradient of the pseudo-coordinates flows through pseudo_csc instead of pseudo."""
         node_feat = self.fc(feat).view(-1, self._n_kernels, self._out_feats)
         pad = (-self._out_feats) % 4
         if pad:         # zero columns up to a multiple of 4: the operator then takes its 128-bit row layout
             node_feat = th.nn.functional.pad(node_feat, (0, pad))
-        rst = type(self)._op(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, self.mu, self.inv_sigma)
+        if pseudo_csc is not None:
+            if type(self)._op is not GmmConvFuseSum:
+                raise ValueError("pseudo_csc is supported by the recomputing GMMConv layer only")
+            rst = GmmConvFuseSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo.detach(), pseudo_csc, self.mu, self.inv_sigma)
+        else:
+            rst = type(self)._op(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, self.mu, self.inv_sigma)
         if pad:
             rst = rst[..., :self._out_feats]
         if self.res_fc is not None:

@@ -38,7 +38,8 @@ class gmm_native:
     @staticmethod
     def gmmconv_backward(colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out, sum_kernels=False):
         require_cuda(colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out)
-        colptr, rowind, permute = as_i32(colptr), as_i32(rowind), as_i32(permute)
+        colptr, rowind = as_i32(colptr), as_i32(rowind)
+        permute = None if permute is None else as_i32(permute)      # None: pseudo / grad_pseudo in CSC order
         grad_out = as_f32(grad_out)
         n, k, f = node_feat.shape
         e = rowind.numel()
@@ -106,6 +107,30 @@ def GmmConvFuseSum(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, m
     """GmmConvFuse(...).sum(1) as one operator: the sum over the K mixture kernels is fused into the
     forward's store and the backward gathers [N,F] gradient rows.  Returns [N,F]."""
     return GmmFuseSumFunction.apply(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma)
+
+
+def GmmConvFuseSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma):
+    """GmmConvFuseSum for a caller that has the pseudo-coordinates in both edge orders
+    (pseudo_csc == pseudo_csr[permute], e.g. the same elementwise projection applied to constant
+    edge data stored both ways).  The forward reads pseudo_csr, the backward reads pseudo_csc and
+    returns its gradient in CSC order: no per-edge gather or scatter through permute.  pseudo_csr
+    gets no gradient; the caller's parameters receive theirs through pseudo_csc."""
+    return GmmFuseSumTwoOrdersFunction.apply(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma)
+
+
+class GmmFuseSumTwoOrdersFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma):
+        out = gmm_native.gmmconv(rowptr, colind, node_feat, pseudo_csr, mu, sigma, sum_kernels=True)      # [N, F]
+        ctx.save_for_backward(colptr, rowind, node_feat, pseudo_csc, mu, sigma)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        colptr, rowind, node_feat, pseudo_csc, mu, sigma = ctx.saved_tensors
+        grad_feat, grad_pseudo_csc, grad_mu, grad_sigma = gmm_native.gmmconv_backward(
+            colptr, rowind, None, node_feat, pseudo_csc, mu, sigma, grad_out.contiguous(), sum_kernels=True)
+        return None, None, None, None, grad_feat, None, grad_pseudo_csc, grad_mu, grad_sigma
 
 
 class GmmFuseSumFunction(torch.autograd.Function):

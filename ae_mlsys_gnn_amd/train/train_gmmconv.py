@@ -40,12 +40,20 @@ class MoNet(nn.Module):
         self.pseudo_proj = nn.ModuleList(PseudoProj(2, dim) for _ in self.layers)
         self.dropout = nn.Dropout(dropout)
 
-    def forward(self, g, feat, pseudo):
+    def forward(self, g, feat, pseudo, pseudo_csc=None):
+        """pseudo: raw per-edge coordinates [E, 2] in CSR order; pseudo_csc: the same rows in CSC order
+        (pseudo[permute]).  With both, each layer projects both copies (the projection is elementwise per
+        edge, so the results are each other's permutation) and the layer's backward runs in CSC order."""
         h = feat
         for i, (layer, proj) in enumerate(zip(self.layers, self.pseudo_proj)):
             if i:
                 h = self.dropout(h)
-            h = layer(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, g.permute, h, proj(pseudo))
+            if pseudo_csc is not None and torch.is_grad_enabled():
+                with torch.no_grad():
+                    ps = proj(pseudo)
+                h = layer(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, g.permute, h, ps, pseudo_csc=proj(pseudo_csc))
+            else:
+                h = layer(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, g.permute, h, proj(pseudo))
         return h
 
 
@@ -63,6 +71,8 @@ def build_parser():
     p.add_argument("--weight-decay", type=float, default=5e-4)
     p.add_argument("--output", type=str, default="figure7.csv")
     p.add_argument("--variant", choices=sorted(VARIANTS), default="our")
+    p.add_argument("--csc-pseudo", type=int, default=1, help="1: keep the edge coordinates in CSR and CSC order (variant our), so the "
+                   "backward needs no per-edge transposition; 0: one copy, as the reference")
     p.add_argument("--data-root", type=str, default=None)
     p.add_argument("--cache-dir", type=str, default=None)
     p.add_argument("--scale", type=float, default=1.0)
@@ -81,6 +91,7 @@ def main(argv=None):
     print("----Data statistics------ (%s)\n  #Nodes %d\n  #Edges %d\n  #Classes %d\n  #Train samples %d\n  #Val samples %d\n  #Test samples %d"
           % (data.source, g.n, g.n_edges, data.n_classes, int(data.train_mask.sum()), int(data.val_mask.sum()), int(data.test_mask.sum())))
     pseudo = datasets.degree_pseudo(g)
+    pseudo_csc = pseudo[g.permute.long()].contiguous() if (args.csc_pseudo and args.variant == "our") else None
     torch.manual_seed(args.seed)
     model = MoNet(VARIANTS[args.variant], data.feat.shape[1], args.n_hidden, data.n_classes, args.n_layers, args.pseudo_dim, args.n_kernels,
                   args.dropout).to(dev)
@@ -92,11 +103,11 @@ def main(argv=None):
     def evaluate(mask):
         model.eval()
         with torch.no_grad():
-            return common.accuracy(model(g, data.feat, pseudo)[mask], data.label[mask])
+            return common.accuracy(model(g, data.feat, pseudo)[mask], data.label[mask])      # no gradients: one copy is enough
 
     def train_step():
         model.train()
-        loss = loss_fcn(model(g, data.feat, pseudo)[train_idx], train_labels)
+        loss = loss_fcn(model(g, data.feat, pseudo, pseudo_csc)[train_idx], train_labels)
         opt.zero_grad(set_to_none=False)
         loss.backward()
         opt.step()

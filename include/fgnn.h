@@ -149,7 +149,11 @@ int    fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F,
  * grad_feat [N,K,F], grad_pseudo [E,dim] (CSR order), grad_mu, grad_sigma [K,dim].
  * The pass writes gw*w per edge into the workspace; a second edge-parallel kernel finishes the
  * Gaussian derivatives, grad_mu / grad_sigma reduced in a fixed order (bit-reproducible).
- * A schedule of col_ptr is required. */
+ * A schedule of col_ptr is required.
+ * permute == NULL: pseudo is given in the order of (col_ptr, row_ind) itself and grad_pseudo comes back
+ * in that order.  A caller that keeps its per-edge inputs in both orders (they are often an
+ * elementwise function of constant edge data) thereby avoids the per-edge gather and scatter through
+ * permute, which is most of this pass on large graphs. */
 size_t fgnn_gmm_backward_workspace_bytes(const fgnn_schedule_t *sched_csc, int K, int dim, int F);
 /* sum_kernels != 0: grad_out is [N,F], the gradient of the fused sum over kernels (every kernel of a
  * node sees the same row, so the pass gathers F instead of K*F floats per edge). */

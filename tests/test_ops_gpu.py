@@ -136,7 +136,10 @@ def _gmm_case(g, k, dim, f, seed):
                                               (5, 2, 33, "sum"), (2, 1, 41, "fuse"), (9, 2, 5, "fuse"), (12, 1, 12, "sum"),
                                               # rows narrower than a wave: several edges per load instruction
                                               (1, 2, 8, "fuse"), (4, 2, 32, "fuse"), (1, 1, 128, "sum"), (2, 2, 32, "stash"), (2, 1, 16, "sum"),
-                                              (3, 1, 4, "fuse")])
+                                              (3, 1, 4, "fuse"),
+                                              # quarter of the width not a power of two: head-aligned lane map
+                                              (2, 1, 44, "fuse"), (3, 2, 12, "sum"), (2, 2, 20, "stash"), (5, 1, 48, "fuse"), (4, 2, 100, "fuse"),
+                                              (9, 1, 12, "fuse")])
 def test_gmm_forward_backward(k, dim, f, variant, monkeypatch):
     from ae_mlsys_gnn_amd.operators import fused_gmmconv as fg
     from ae_mlsys_gnn_amd import _lib
@@ -254,7 +257,8 @@ def _small_graph():
     return graphs.add_csc_torch(degree_edge_graph(n=300, seed=4))
 
 
-@pytest.mark.parametrize("h,f", [(4, 16), (8, 32), (1, 47), (3, 20), (2, 128), (2, 41), (9, 5), (12, 12), (1, 4), (2, 8), (1, 128)])
+@pytest.mark.parametrize("h,f", [(4, 16), (8, 32), (1, 47), (3, 20), (2, 128), (2, 41), (9, 5), (12, 12), (1, 4), (2, 8), (1, 128),
+                                 (2, 44), (5, 48), (4, 100), (16, 12)])
 def test_mhspmm_and_mhsddmm(h, f):
     from ae_mlsys_gnn_amd.operators import mhspmm as op
     g = _small_graph()
@@ -352,7 +356,7 @@ def test_error_paths_return_codes_not_aborts():
         fg.fused_gat_op(a, a, g.row_ptr.long(), g.col_ind, g.col_ptr, g.row_ind, 0.2, torch.randn(64, 8, 4, device=DEV))
 
 
-@pytest.mark.parametrize("h,f", [(1, 64), (1, 47), (4, 16), (3, 20), (9, 5), (2, 256)])
+@pytest.mark.parametrize("h,f", [(1, 64), (1, 47), (4, 16), (3, 20), (9, 5), (2, 256), (2, 44), (12, 12)])
 def test_coo_and_csr_sddmm(h, f):
     """sddmm.coo_sddmm / csr_sddmm: per-edge dot products, against float64 gathers."""
     from ae_mlsys_gnn_amd.operators import sddmm
@@ -542,3 +546,36 @@ def test_edgeconv_step_replays_from_a_hip_graph():
         torch.cuda.synchronize()
         assert torch.equal(out, e_out) and torch.equal(arg, e_arg), "replay %d: forward differs from eager" % rep
         assert torch.equal(gs, e_gs), "replay %d: backward differs from eager" % rep
+
+
+@pytest.mark.parametrize("k,dim,f", [(3, 2, 16), (2, 1, 41), (2, 1, 16)])
+def test_gmm_layer_with_csc_ordered_pseudo(k, dim, f, monkeypatch):
+    """GMMConv(..., pseudo_csc=pseudo[permute]): same output; the gradient that arrives at pseudo_csc is
+    the oracle's grad_pseudo in CSC order; all other gradients unchanged.  With an XCD-aware schedule too."""
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd.layers import GMMConv
+    for buckets in ("0", "1"):
+        monkeypatch.setenv("FGNN_XCD_BUCKETS", buckets)
+        monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+        _lib.clear_schedule_cache()
+        torch.manual_seed(4)
+        g = graphs.add_csc_torch(graphs.rmat_graph(600, 30000, seed=6))
+        layer = GMMConv(24, f, dim=dim, n_kernels=k)
+        feat, pseudo, go = torch.randn(g.n, 24), torch.rand(g.n_edges, dim), torch.randn(g.n, f)
+        leaves = [t.detach().double().requires_grad_(True) for t in (layer.fc.weight, layer.mu, layer.inv_sigma, layer.bias, feat, pseudo)]
+        ref = orc.gmm_layer_dgl(leaves[0], leaves[1], leaves[2], leaves[3], g.row_ptr, g.col_ind, leaves[4], leaves[5])
+        ref.backward(go.double())
+        gd = g.to(DEV)
+        layer = layer.to(DEV)
+        fd = feat.to(DEV).requires_grad_(True)
+        pd = pseudo.to(DEV)
+        pc = pd[gd.permute.long()].contiguous().requires_grad_(True)
+        out = layer(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, pd, pseudo_csc=pc)
+        out.backward(go.to(DEV))
+        assert_close(out, ref.detach(), "GMMConv (two orders)", atol=1e-4)
+        assert_close(fd.grad, leaves[4].grad, "grad feat (two orders)", atol=1e-4)
+        assert_close(pc.grad, leaves[5].grad[g.permute.long()], "grad pseudo in CSC order", atol=1e-3)
+        assert_close(layer.mu.grad, leaves[1].grad, "grad mu (two orders)", rtol=1e-3, atol=5e-2)
+        assert_close(layer.inv_sigma.grad, leaves[2].grad, "grad inv_sigma (two orders)", rtol=1e-3, atol=5e-2)
+        assert_close(layer.fc.weight.grad, leaves[0].grad, "grad fc (two orders)", rtol=1e-3, atol=5e-2)
+    _lib.clear_schedule_cache()

@@ -28,7 +28,7 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published peak
 
 # L2<->fabric bytes per launch of the dominant kernels measured with rocprofv3 --pmc (FETCH_SIZE scaled
 # x2.000 and WRITE_SIZE x1.000 by the 1 GiB copy of --calibrate-copy; profiles/gat_kernels_gat_c2.md and
-# profiles/other_workloads.md); all kernels of the entry point summed.
+# profiles/kernels_edgeconv_c3_gmm_c4_gat_c5_drivers.md); all kernels of the entry point summed.
 # They bound the HBM traffic from above.  None = not measured for that workload.
 MEASURED_TRAFFIC_BYTES = {
     "gat_c2": {"fwd": 37136911667, "bwd": 33567448883},

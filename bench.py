@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gat_c2|gat_c5|gat_c5_train|edgeconv_c3|gmm_c4]
 
-Default workload = BASELINE config 2: one fused GAT layer forward+backward (dense projection by
+Default workload = benchmark configuration 2: one fused GAT layer forward+backward (dense projection by
 torch.matmul, fused sparse op by libfgnn_hip.so) on a seeded R-MAT power-law graph with 232,965
 nodes and ~114.6 M edges plus self loops, features [N,256], 8 heads x 32, fp32.  A step is one
 layer forward + backward; inputs are resident in HBM before the timed region; graph
@@ -151,7 +151,7 @@ def cpu_baseline_gat(g, x_feat, layer, slope, target_edges, go):
 
 
 def cpu_baseline_c1():
-    """BASELINE config 1 at its real size on the host: the DGL-composed GAT layer forward+backward,
+    """benchmark configuration 1 at its real size on the host: the DGL-composed GAT layer forward+backward,
     N=4096, 32,768 uniform random edges + self loops, X [4096,64], 4 heads x 16, slope 0.2, loss = sum."""
     import torch
     from ae_mlsys_gnn_amd import graphs
@@ -394,7 +394,7 @@ def run_gmm(args):
 
 
 def run_gat_train(args):
-    """BASELINE config 5: full 2-layer GAT training step (forward, cross-entropy over all nodes,
+    """benchmark configuration 5: full 2-layer GAT training step (forward, cross-entropy over all nodes,
     backward, Adam) with the model of the reference's script/train/train_gatconv_our.py:33-53
     (GATConv(100, 32, 8) -> flatten -> GATConv(256, 47, 1) -> mean over heads; no activation in
     between), recompute variant against stash variant; reports ms/step and peak HBM of both."""

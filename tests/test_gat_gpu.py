@@ -104,7 +104,7 @@ def test_gat_self_loops_only_is_identity():
 
 
 def test_gat_c1_config():
-    # BASELINE config 1: N=4096, 32k uniform edges + self loops, 4 heads x 16
+    # benchmark configuration 1: N=4096, 32k uniform edges + self loops, 4 heads x 16
     _run(graphs.uniform_graph(4096, 32768, seed=0), 4, 16)
 
 

@@ -119,3 +119,105 @@ extern "C" int fgnn_edgeconv_backward(int N, int n_src, int F, const int32_t *ar
     hipLaunchKernelGGL(edgeconv_bwd_kernel, dim3(grid), dim3(256), 0, st, total, F, argmax, grad_out, grad_src);
     return fgnn_launch_status("edgeconv_bwd_kernel");
 }
+
+// ---------------------------------------------------------------------------------------------------
+// Backward for batched point clouds.  `block` is a hint: the neighbours of destination rows
+// [b*block, (b+1)*block) mostly lie in source rows of the same range (a kNN graph of clouds of `block`
+// points each has them all there).  A workgroup owns block b and FS feature columns, accumulates its
+// contributions in an LDS tile with LDS float atomics and writes the tile out with plain stores: no
+// clearing pass, no global atomics.  A contribution whose source lies outside the block is appended to
+// an overflow list and applied by a second, normally empty, kernel with global atomics, so a wrong
+// hint costs time, never correctness.
+#define EC_OVF_HEADER 64        // ints in front of the overflow list (counter + padding)
+
+#define EC_BT 1024      // threads per workgroup of the blocked backward
+template <int FS>
+__global__ __launch_bounds__(EC_BT) void edgeconv_bwd_blocked_kernel(int N, int F, int block, const int *__restrict__ argmax,
+                                                                     const float *__restrict__ grad_out, float *__restrict__ grad_src,
+                                                                     int *__restrict__ ovf)
+{
+    extern __shared__ float tile[];                 // [rows of the block][FS]
+    const int b = (int)blockIdx.y, f0 = (int)blockIdx.x * FS;
+    const int r0 = b * block, rows = min(block, N - r0), fs = min(FS, F - f0);
+    const int total = rows * FS;
+    for (int i = (int)threadIdx.x; i < total; i += EC_BT) tile[i] = 0.f;
+    __syncthreads();
+    constexpr int U = 4;                            // elements in flight per thread
+    for (int i0 = (int)threadIdx.x; i0 < total; i0 += EC_BT * U) {
+        int g[U], a[U];
+        float v[U];
+        bool ok[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + u * EC_BT;
+            const int r = i / FS, ff = i - r * FS;
+            ok[u] = i < total && ff < fs;
+            g[u] = (r0 + r) * F + f0 + ff;           // N*F < 2^31 is checked on the host
+            a[u] = ok[u] ? argmax[g[u]] : 0;
+            v[u] = ok[u] ? grad_out[g[u]] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (!ok[u]) continue;
+            const int i = i0 + u * EC_BT;
+            const int ff = i % FS;
+            const int local = a[u] - r0;
+            if ((unsigned)local < (unsigned)rows) {
+                __hip_atomic_fetch_add(&tile[local * FS + ff], v[u], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            } else {
+                int slot = atomicAdd(ovf, 1);
+                ovf[EC_OVF_HEADER + slot] = g[u];
+            }
+        }
+    }
+    __syncthreads();
+    for (int i = (int)threadIdx.x; i < total; i += EC_BT) {
+        const int r = i / FS, ff = i - r * FS;
+        if (ff < fs) grad_src[(size_t)(r0 + r) * F + f0 + ff] = tile[i];
+    }
+}
+
+__global__ __launch_bounds__(256) void edgeconv_bwd_overflow_kernel(int F, const int *__restrict__ argmax, const float *__restrict__ grad_out,
+                                                                    float *__restrict__ grad_src, const int *__restrict__ ovf)
+{
+    const int count = ovf[0];
+    for (int i = (int)(blockIdx.x * 256 + threadIdx.x); i < count; i += (int)(gridDim.x * 256)) {
+        const int g = ovf[EC_OVF_HEADER + i];
+        unsafeAtomicAdd(grad_src + (size_t)argmax[g] * F + (g % F), grad_out[g]);
+    }
+}
+
+extern "C" size_t fgnn_edgeconv_backward_blocked_workspace_bytes(int N, int F)
+{
+    return ((size_t)N * F + EC_OVF_HEADER) * sizeof(int32_t);
+}
+
+extern "C" int fgnn_edgeconv_backward_blocked(int N, int n_src, int F, int block, const int32_t *argmax, const float *grad_out,
+                                              float *grad_src, void *workspace, size_t workspace_bytes, void *stream)
+{
+    FGNN_REQUIRE(N >= 0 && n_src >= 0 && F >= 1 && block >= 1, FGNN_ERR_SHAPE, "fgnn_edgeconv_backward_blocked: bad sizes");
+    FGNN_REQUIRE(argmax && grad_out && grad_src, FGNN_ERR_NULL, "fgnn_edgeconv_backward_blocked: NULL argument");
+    FGNN_REQUIRE((int64_t)N * F <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_edgeconv_backward_blocked: N*F exceeds int32");
+    // tile of the largest FS that fits 64 KiB of LDS; without a usable tile, or with source rows that no
+    // destination block covers, the plain scatter does the job
+    const int fs = block <= 2048 ? 8 : block <= 4096 ? 4 : 0;
+    if (fs == 0 || n_src != N || (size_t)block * fs * sizeof(float) > 64 * 1024)
+        return fgnn_edgeconv_backward(N, n_src, F, argmax, grad_out, grad_src, stream);
+    size_t need = fgnn_edgeconv_backward_blocked_workspace_bytes(N, F);
+    FGNN_REQUIRE(N == 0 || (workspace && workspace_bytes >= need), FGNN_ERR_WORKSPACE, "fgnn_edgeconv_backward_blocked: workspace %zu < %zu bytes",
+                 workspace_bytes, need);
+    if (N == 0) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    int *ovf = (int *)workspace;
+    int rc = fgnn_fill_f32((float *)ovf, 1, 0.f, st);        // the counter (bit pattern of 0.0f is integer 0)
+    if (rc) return rc;
+    dim3 grid((unsigned)((F + fs - 1) / fs), (unsigned)((N + block - 1) / block));
+    FGNN_REQUIRE(grid.y <= 65535, FGNN_ERR_LIMIT, "fgnn_edgeconv_backward_blocked: more than 65535 blocks");
+    const size_t shm = (size_t)block * fs * sizeof(float);
+    if (fs == 8) hipLaunchKernelGGL(edgeconv_bwd_blocked_kernel<8>, grid, dim3(EC_BT), shm, st, N, F, block, argmax, grad_out, grad_src, ovf);
+    else hipLaunchKernelGGL(edgeconv_bwd_blocked_kernel<4>, grid, dim3(EC_BT), shm, st, N, F, block, argmax, grad_out, grad_src, ovf);
+    rc = fgnn_launch_status("edgeconv_bwd_blocked_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(edgeconv_bwd_overflow_kernel, dim3(64), dim3(256), 0, st, F, argmax, grad_out, grad_src, ovf);
+    return fgnn_launch_status("edgeconv_bwd_overflow_kernel");
+}

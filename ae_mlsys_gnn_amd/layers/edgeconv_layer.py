@@ -22,8 +22,9 @@ class EdgeConv(nn.Module):
     def set_allow_zero_in_degree(self, set_value):
         self._allow_zero_in_degree = set_value
 
-    def forward(self, k, src_ind, feat):
+    def forward(self, k, src_ind, feat, block=None):
+        """block: points per cloud when src_ind is a kNN graph of equally sized clouds (see fused_edgeconv_op)."""
         h_theta = self.theta(feat)
         h_src = h_theta
         h_dst = self.phi(feat) - h_theta
-        return fused_edgeconv_op(k, src_ind, h_src, h_dst)
+        return fused_edgeconv_op(k, src_ind, h_src, h_dst, block)

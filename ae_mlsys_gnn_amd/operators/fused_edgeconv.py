@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .._lib import FgnnError, as_f32, as_i32, check, lib, ptr, require_cuda, stream_ptr
+from .._lib import FgnnError, as_f32, as_i32, check, lib, ptr, require_cuda, stream_ptr, workspace
 
 
 class edgeconv_native:
@@ -25,20 +25,29 @@ class edgeconv_native:
         return out, max_idx
 
     @staticmethod
-    def edgeconv_backward(grad_out, max_idx, n_src=None):
+    def edgeconv_backward(grad_out, max_idx, n_src=None, block=None):
+        """block: points per cloud when the graph is a kNN graph of equally sized point clouds (a hint:
+        neighbours outside a node's own block are still handled, just more slowly)."""
         require_cuda(grad_out, max_idx)
         grad_out, max_idx = as_f32(grad_out), as_i32(max_idx)
         n, f = grad_out.shape
         n_src = n if n_src is None else n_src
         grad_src = torch.empty((n_src, f), dtype=torch.float32, device=grad_out.device)
         with torch.cuda.device(grad_out.device):
-            check(lib().fgnn_edgeconv_backward(n, n_src, f, ptr(max_idx), ptr(grad_out), ptr(grad_src), stream_ptr()),
-                  "fgnn_edgeconv_backward")
+            if block:
+                ws, wsb = workspace(lib().fgnn_edgeconv_backward_blocked_workspace_bytes(n, f), grad_out.device)
+                check(lib().fgnn_edgeconv_backward_blocked(n, n_src, f, int(block), ptr(max_idx), ptr(grad_out), ptr(grad_src), ptr(ws), wsb,
+                                                           stream_ptr()), "fgnn_edgeconv_backward_blocked")
+            else:
+                check(lib().fgnn_edgeconv_backward(n, n_src, f, ptr(max_idx), ptr(grad_out), ptr(grad_src), stream_ptr()),
+                      "fgnn_edgeconv_backward")
         return grad_src
 
 
-def fused_edgeconv_op(k, src_ind, h_src, h_dst):
-    return FusedEdgeConvFunction.apply(k, src_ind, h_src, h_dst)
+def fused_edgeconv_op(k, src_ind, h_src, h_dst, block=None):
+    """block (optional, not in the reference): points per cloud of a batched kNN graph; lets the backward
+    accumulate per cloud in LDS instead of scattering with global atomics."""
+    return FusedEdgeConvFunction.apply(k, src_ind, h_src, h_dst, block)
 
 
 class FusedEdgeConvFunction(torch.autograd.Function):
@@ -46,15 +55,16 @@ class FusedEdgeConvFunction(torch.autograd.Function):
     node id, first maximum wins) is kept for the backward (operators/fused_edgeconv.py:18-29)."""
 
     @staticmethod
-    def forward(ctx, k, src_ind, h_src, h_dst):
+    def forward(ctx, k, src_ind, h_src, h_dst, block=None):
         out_feat, max_idx = edgeconv_native.edgeconv_forward(k, src_ind, h_src, h_dst)
         ctx.save_for_backward(max_idx)
         ctx.n_src = h_src.shape[0]
+        ctx.block = block
         return out_feat
 
     @staticmethod
     def backward(ctx, grad_out):
         max_idx = ctx.saved_tensors[0]
         grad_out = grad_out.contiguous()
-        grad_src = edgeconv_native.edgeconv_backward(grad_out, max_idx, ctx.n_src)
-        return None, None, grad_src, grad_out
+        grad_src = edgeconv_native.edgeconv_backward(grad_out, max_idx, ctx.n_src, ctx.block)
+        return None, None, grad_src, grad_out, None

@@ -44,7 +44,7 @@ class Model(nn.Module):
         h, hs = x, []
         for conv in self.conv:
             src = self.knn(h.detach(), self.k)
-            h = F.leaky_relu(conv(self.k, src, h.reshape(b * p, -1)), 0.2).view(b, p, -1)
+            h = F.leaky_relu(conv(self.k, src, h.reshape(b * p, -1), block=p), 0.2).view(b, p, -1)
             hs.append(h)
         h = self.proj(torch.cat(hs, 2))
         h = torch.cat([h.max(1).values, h.mean(1)], 1)

@@ -119,6 +119,17 @@ int fgnn_edgeconv_forward(int N, int n_src, int F, int k, const int32_t *src_ind
 int fgnn_edgeconv_backward(int N, int n_src, int F, const int32_t *argmax, const float *grad_out,
                            float *grad_src, void *stream);
 
+/* The same backward for batched point clouds.  `block` is a hint that the neighbours of destination
+ * rows [b*block, (b+1)*block) lie in source rows of the same range, as in a kNN graph of clouds of
+ * `block` points (fgnn_knn_graph): those contributions are accumulated in LDS and written with plain
+ * stores; any others go through an overflow list in the workspace and global atomics, so a wrong hint
+ * only costs time.  Falls back to fgnn_edgeconv_backward when n_src != N or block > 4096.  No
+ * counterpart in the reference (its backward is the plain scatter, fused_edgeconv.cu:175-187). */
+size_t fgnn_edgeconv_backward_blocked_workspace_bytes(int N, int F);
+int    fgnn_edgeconv_backward_blocked(int N, int n_src, int F, int block, const int32_t *argmax,
+                                      const float *grad_out, float *grad_src, void *workspace,
+                                      size_t workspace_bytes, void *stream);
+
 /* k-nearest-neighbour graph of batched point clouds, the input of fgnn_edgeconv_forward: points
  * [n_clouds*P, D]; src_ind [n_clouds*P*k] gets, for every point, the global ids of the k nearest
  * points of its own cloud (itself included), nearest first, ties to the smaller id; 1 <= k <= min(P,

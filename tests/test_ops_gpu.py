@@ -433,6 +433,46 @@ def test_knn_graph_feeds_edgeconv():
     assert out.shape == (1024, 64) and bool(torch.isfinite(out).all())
 
 
+@pytest.mark.parametrize("b,p,k,f,block", [(4, 256, 20, 64, 256), (3, 1000, 8, 20, 1000), (2, 2048, 10, 8, 2048), (5, 100, 5, 130, 100),
+                                            (4, 256, 20, 64, 128), (4, 256, 20, 64, 1024), (2, 300, 6, 16, 8192)])
+def test_edgeconv_backward_blocked(b, p, k, f, block):
+    """The blocked backward (LDS tiles per cloud) against the oracle's scatter-add; block sizes that
+    match the clouds, cut them in two, span several of them (overflow path) or exceed the LDS tile
+    (fallback to the plain scatter)."""
+    from ae_mlsys_gnn_amd.operators.fused_edgeconv import edgeconv_native
+    from ae_mlsys_gnn_amd.operators.knn import knn_graph
+    gen = torch.Generator().manual_seed(b * p + f)
+    pts = (torch.rand(b, p, 3, generator=gen) * 2 - 1).to(DEV)
+    src = knn_graph(pts, k)
+    n = b * p
+    hs, hd = torch.randn(n, f, generator=gen), torch.randn(n, f, generator=gen)
+    go = torch.randn(n, f, generator=gen)
+    out, arg = edgeconv_native.edgeconv_forward(k, src, hs.to(DEV), hd.to(DEV))
+    want = torch.zeros(n, f, dtype=torch.float64).scatter_add_(0, arg.cpu().long(), go.double())
+    got = edgeconv_native.edgeconv_backward(go.to(DEV), arg, n, block=block)
+    assert_close(got, want, "blocked edgeconv backward", atol=1e-5)
+    plain = edgeconv_native.edgeconv_backward(go.to(DEV), arg, n)
+    assert_close(plain, want, "plain edgeconv backward", atol=1e-5)
+
+
+def test_edgeconv_backward_blocked_with_a_wrong_hint():
+    """Neighbours anywhere in the graph: every contribution outside a node's own block goes through the
+    overflow list, the result is still the scatter-add."""
+    from ae_mlsys_gnn_amd.operators.fused_edgeconv import fused_edgeconv_op
+    gen = torch.Generator().manual_seed(3)
+    n, k, f = 3000, 7, 24
+    src = torch.randint(0, n, (n * k,), generator=gen, dtype=torch.int32)
+    hs, hd, go = (torch.randn(n, f, generator=gen) for _ in range(3))
+    ref_s = hs.double().requires_grad_(True)
+    ref = orc.edgeconv_forward_autograd(k, src, ref_s, hd.double())
+    ref.backward(go.double())
+    hsd = hs.to(DEV).requires_grad_(True)
+    out = fused_edgeconv_op(k, src.to(DEV), hsd, hd.to(DEV), block=512)
+    out.backward(go.to(DEV))
+    assert torch.equal(out.detach().cpu(), ref.detach().float())
+    assert_close(hsd.grad, ref_s.grad, "grad_src with a wrong block hint", atol=1e-5)
+
+
 # ------------------------------------------------------------------ coo2csr (bit-exact)
 @pytest.mark.parametrize("n,e,dedupe", [(1, 1, True), (50, 400, True), (50, 400, False), (3000, 200000, True), (70000, 500000, True), (300, 0, True)])
 def test_coo2csr_bit_exact(n, e, dedupe):

@@ -13,12 +13,14 @@
 // dimension by dimension in ascending order with one subtract and one fma each, so a point is at
 // distance exactly 0 from itself.
 //
-// Selection: k rounds per query; a round takes the wave-wide minimum (DPP butterfly), finds the
-// holder with the smallest node id by ballots, records it in lane (round % 64) of the result
-// registers and retires it.  The order is total (smaller distance first, smaller node id on equal
-// distance), so the result is deterministic.  Clouds with more points than one tile keep the best
-// k of the tiles seen so far in registers and run them through the next tile's selection, where
-// they win ties because their ids are smaller.
+// Selection (k <= 64): the k-th smallest of the 64 lane minima is a threshold that at least k
+// candidates pass; the candidates under it (usually k to 2k of the 1024) are compacted into LDS with
+// ballots and ordered by one bitonic sort over the wave.  When more than 64 pass (many equal distances)
+// and for 64 < k <= 128 the selection runs k extraction rounds instead: wave-wide minimum (DPP
+// butterfly), holder with the smallest node id by ballots, retire it.  Either way the order is total
+// (smaller distance first, smaller node id on equal distance), so the result is deterministic.  Clouds
+// with more points than one tile keep the best k of the tiles seen so far in registers and run them
+// through the next tile's selection, where they win ties because their ids are smaller.
 #include "fgnn_common.h"
 #include <float.h>
 
@@ -30,7 +32,7 @@
 // Takes the k best of {prior list (pd, pi), the tile's distances} in order; the new list replaces
 // the prior one.  List position p lives in lane p % 64 of register p / 64.
 template <int NR, int KR>
-__device__ __forceinline__ void knn_select(float (&dist)[NR], int tile0, float (&pd)[KR], int (&pi)[KR], int k, int lane, int fallback_id)
+__device__ __forceinline__ void knn_select_rounds(float (&dist)[NR], int tile0, float (&pd)[KR], int (&pi)[KR], int k, int lane, int fallback_id)
 {
     float nd[KR];
     int ni[KR];
@@ -83,12 +85,82 @@ __device__ __forceinline__ void knn_select(float (&dist)[NR], int tile0, float (
     for (int t = 0; t < KR; ++t) { pd[t] = nd[t]; pi[t] = ni[t]; }
 }
 
+// Bitonic sort of one value per lane over the wave, ascending by (d, i).
+__device__ __forceinline__ void knn_sort_wave(float &d, int &i, int lane)
+{
+#pragma unroll
+    for (int size = 2; size <= 64; size <<= 1) {
+#pragma unroll
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            const float od = fg_bperm(d, lane ^ stride);
+            const int oi = __builtin_amdgcn_ds_bpermute((lane ^ stride) << 2, i);
+            const bool keep_small = (((lane & size) == 0) || size == 64) == ((lane & stride) == 0);
+            const bool other_smaller = od < d || (od == d && oi < i);
+            if (keep_small == other_smaller) { d = od; i = oi; }
+        }
+    }
+}
+
+// The k best of {prior list, tile} for k <= 64: (1) a threshold that at least k candidates pass, the
+// k-th smallest of the 64 lane minima; (2) the candidates under it (usually k to 2k) are compacted
+// into wave-private LDS with ballots; (3) one bitonic sort over the wave orders them.  More than 64
+// candidates under the threshold (many equal distances, or fewer than k lanes with a candidate) fall
+// back to the extraction rounds.  sd/si: 64 floats / ints of LDS owned by this wave.
+template <int NR>
+__device__ __forceinline__ void knn_select(float (&dist)[NR], int tile0, float (&pd)[1], int (&pi)[1], int k, int lane, int fallback_id,
+                                           float *sd, int *si)
+{
+    float lm = pd[0];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) lm = fminf(lm, dist[r]);
+    int dummy = lane;
+    knn_sort_wave(lm, dummy, lane);
+    const float tau = fg_readlane(lm, k - 1);
+    int cnt = __popcll(__ballot(pd[0] <= tau));
+#pragma unroll
+    for (int r = 0; r < NR; ++r) cnt += __popcll(__ballot(dist[r] <= tau));
+    if (cnt > 64 || !(tau < INFINITY)) {
+        knn_select_rounds<NR, 1>(dist, tile0, pd, pi, k, lane, fallback_id);
+        return;
+    }
+    const unsigned long long lt = (1ull << lane) - 1ull;
+    int base = 0;
+    {
+        const bool in = pd[0] <= tau;
+        const unsigned long long m = __ballot(in);
+        if (in) { int pos = base + __popcll(m & lt); sd[pos] = pd[0]; si[pos] = pi[0]; }
+        base += __popcll(m);
+    }
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        const bool in = dist[r] <= tau;
+        const unsigned long long m = __ballot(in);
+        if (in) { int pos = base + __popcll(m & lt); sd[pos] = dist[r]; si[pos] = tile0 + (r / 4) * 256 + lane * 4 + (r % 4); }
+        base += __popcll(m);
+    }
+    fg_wave_lds_sync();
+    float cd = lane < cnt ? sd[lane] : INFINITY;
+    int ci = lane < cnt ? si[lane] : 0x7fffffff;
+    fg_wave_lds_sync();
+    knn_sort_wave(cd, ci, lane);
+    pd[0] = lane < k ? cd : INFINITY;
+    pi[0] = lane < k ? ci : fallback_id;
+}
+template <int NR>
+__device__ __forceinline__ void knn_select(float (&dist)[NR], int tile0, float (&pd)[2], int (&pi)[2], int k, int lane, int fallback_id,
+                                           float *, int *)
+{
+    knn_select_rounds<NR, 2>(dist, tile0, pd, pi, k, lane, fallback_id);       // 64 < k <= 128
+}
+
 template <int RG, int KR>
 __global__ __launch_bounds__(KNN_WAVES * 64) void knn_kernel(int P, int D, int k, int rows_aligned, const float *__restrict__ pts, int *__restrict__ out)
 {
     constexpr int NR = 4 * RG;                  // distances per lane and query
     constexpr int TILE = 256 * RG;              // candidate points per tile
     __shared__ __attribute__((aligned(16))) float cs[KNN_DC * TILE];        // [dimension of the slice][point of the tile]
+    __shared__ float sel_d[KNN_WAVES * 64];                                 // selection scratch, 64 entries per wave
+    __shared__ int sel_i[KNN_WAVES * 64];
     const int tid = (int)threadIdx.x;
     const int lane = fg_lane();
     const int cloud = (int)blockIdx.y;
@@ -162,7 +234,7 @@ __global__ __launch_bounds__(KNN_WAVES * 64) void knn_kernel(int P, int D, int k
                 for (int a = 0; a < KNN_QW; ++a) acc[a][4 * g + u] = ok ? fminf(acc[a][4 * g + u], FLT_MAX) : INFINITY;
             }
 #pragma unroll
-        for (int a = 0; a < KNN_QW; ++a) knn_select<NR, KR>(acc[a], tile0, pd[a], pi[a], k, lane, qrow[a]);
+        for (int a = 0; a < KNN_QW; ++a) knn_select<NR>(acc[a], tile0, pd[a], pi[a], k, lane, qrow[a], sel_d + fg_wave() * 64, sel_i + fg_wave() * 64);
     }
 #pragma unroll
     for (int a = 0; a < KNN_QW; ++a) {

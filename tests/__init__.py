@@ -1,0 +1,1 @@
+"""Test package (parity tests of the fused sparse operators)."""

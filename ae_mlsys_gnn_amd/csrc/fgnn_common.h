@@ -255,10 +255,7 @@ __device__ __forceinline__ void fg_accum_chunk(const float *__restrict__ feat, i
             int id = __builtin_amdgcn_readlane(idv, t + u);
             const float *base = feat + (size_t)id * (size_t)HF;
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                if (FULL || lm.ok[r]) ld[u][r].load(base + lm.eoff[r]);
-                else ld[u][r].zero();
-            }
+            for (int r = 0; r < R; ++r) ld[u][r].load(base + ((FULL || lm.ok[r]) ? lm.eoff[r] : 0));   // idle lanes re-read float 0: no branch
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) {

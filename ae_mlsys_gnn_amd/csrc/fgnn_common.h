@@ -123,7 +123,9 @@ __device__ __forceinline__ float fg_bperm(float v, int src_lane) { return __int_
 template <int CTRL>
 __device__ __forceinline__ float fg_dpp(float v)
 {
-    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xf, 0xf, false));
+    // every control used here is a permutation inside a row, so no lane lacks a source; "old = 0,
+    // bound_ctrl" lets the compiler fold the move into the add / max that consumes it
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
 }
 // Butterfly inside each row of 16 lanes (quad xor 1, quad xor 2, half-row mirror, row mirror),
 // then the four row results are combined through scalar registers.  All lanes get the result.

@@ -14,6 +14,26 @@ struct SpmmP {
 };
 __host__ __device__ static inline int spmm_pw(int HF) { return (HF + 3) & ~3; }
 
+// Gaussian mixture weight of one edge for kernel k: exp(-0.5 sum_d ((ps[d]-mu[k,d])*isg[k,d])^2).  The
+// first GMM_PV pseudo-coordinates of the edge are fetched once, up front and together (pv); fetched
+// inside the k / d loops every one of them would be a separate round trip to memory.
+#define GMM_PV 4
+__device__ __forceinline__ void gmm_load_pseudo(const float *ps, int dim, float (&pv)[GMM_PV])
+{
+#pragma unroll
+    for (int d = 0; d < GMM_PV; ++d) pv[d] = d < dim ? ps[d] : 0.f;
+}
+__device__ __forceinline__ float gmm_weight(const float (&pv)[GMM_PV], const float *ps, const float *mu_k, const float *isg_k, int dim)
+{
+    float acc = 0.f;
+#pragma unroll
+    for (int d = 0; d < GMM_PV; ++d) {
+        if (d < dim) { float t = (pv[d] - mu_k[d]) * isg_k[d]; acc = fmaf(t, t, acc); }
+    }
+    for (int d = GMM_PV; d < dim; ++d) { float t = (ps[d] - mu_k[d]) * isg_k[d]; acc = fmaf(t, t, acc); }
+    return __expf(-0.5f * acc);
+}
+
 // Final store of an accumulated row: either the [H,F] row itself or, with sum_h, its sum over heads.
 // scr: wave-private LDS of HF floats (only touched with sum_h).
 template <int VEC, int R, bool FULL>
@@ -59,13 +79,10 @@ struct WGauss {
     __device__ __forceinline__ void fill(float *wl, const float *shared, int lane, size_t pos, bool ok, int K) const
     {
         const float *ps = pseudo + pos * dim;
+        float pv[GMM_PV];
+        gmm_load_pseudo(ps, dim, pv);
         for (int k = 0; k < K; ++k) {
-            float acc = 0.f;
-            for (int d = 0; d < dim; ++d) {
-                float t = (ps[d] - shared[k * dim + d]) * shared[K * dim + k * dim + d];
-                acc = fmaf(t, t, acc);
-            }
-            float w = __expf(-0.5f * acc);
+            float w = gmm_weight(pv, ps, shared + k * dim, shared + K * dim + k * dim, dim);
             wl[k * 64 + lane] = ok ? w : 0.f;
             if (gauss_out && ok) gauss_out[pos * K + k] = w;
         }
@@ -348,14 +365,9 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p)
         };
         request(0);
         const float *ps = p.pseudo + (size_t)(unsigned)posv * dim;
-        for (int k = 0; k < K; ++k) {
-            float acc = 0.f;
-            for (int d = 0; d < dim; ++d) {
-                float t = (ps[d] - shared[k * dim + d]) * shared[KD + k * dim + d];
-                acc = fmaf(t, t, acc);
-            }
-            wl[k * 64 + lane] = ok ? __expf(-0.5f * acc) : 0.f;
-        }
+        float pv[GMM_PV];
+        gmm_load_pseudo(ps, dim, pv);
+        for (int k = 0; k < K; ++k) wl[k * 64 + lane] = ok ? gmm_weight(pv, ps, shared + k * dim, shared + KD + k * dim, dim) : 0.f;
         fg_wave_lds_sync();
         for (int t = 0; t < cnt; t += UG) {
             if (t > 0) request(t);
@@ -423,14 +435,9 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_packed_kernel(GmmBwdP p)
         int posv = p.pos ? p.pos[qq] : qq;
         if (p.permute) posv = p.permute[posv];      // NULL: pseudo and gww are in this pass's own (CSC) order
         const float *ps = p.pseudo + (size_t)(unsigned)posv * dim;
-        for (int k = 0; k < K; ++k) {
-            float acc = 0.f;
-            for (int d = 0; d < dim; ++d) {
-                float t = (ps[d] - shared[k * dim + d]) * shared[KD + k * dim + d];
-                acc = fmaf(t, t, acc);
-            }
-            wl[k * 64 + lane] = ok ? __expf(-0.5f * acc) : 0.f;
-        }
+        float pv[GMM_PV];
+        gmm_load_pseudo(ps, dim, pv);
+        for (int k = 0; k < K; ++k) wl[k * 64 + lane] = ok ? gmm_weight(pv, ps, shared + k * dim, shared + KD + k * dim, dim) : 0.f;
         fg_wave_lds_sync();
         for (int t = 0; t < cnt; t += U * G) {
             fg_vec<4> ld[U];

@@ -75,6 +75,25 @@ def test_gat_rows_narrower_than_a_wave(h, f, variant, monkeypatch):
     _lib.clear_schedule_cache()
 
 
+@pytest.mark.parametrize("variant", ["sm", "stash"])
+@pytest.mark.parametrize("h,f", [(8, 32), (4, 64), (1, 256), (2, 72), (5, 52), (16, 32), (16, 16), (3, 50), (7, 36), (64, 16), (33, 31)])
+def test_gat_long_rows_pair_layout(h, f, variant, monkeypatch):
+    """Graphs averaging 64 or more entries per row take the kernels that compute the attention weights
+    once per (edge, head) on one lane and hand them to the feature lanes (where edges-per-batch x heads
+    fits the wave; (16, 16) and (33, 31) do not and keep the per-lane form).  Degrees 0..3000 with
+    ragged batch tails, whole and split rows, and an XCD-aware schedule."""
+    from ae_mlsys_gnn_amd import _lib
+    g = degree_edge_graph(n=80, seed=21)
+    assert g.n_edges >= 64 * g.n
+    _run(g, h, f, variant=variant)
+    monkeypatch.setenv("FGNN_SEG_LEN", "256")
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
+    monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+    _lib.clear_schedule_cache()
+    _run(degree_edge_graph(n=75, seed=22), h, f, variant=variant)
+    _lib.clear_schedule_cache()
+
+
 def test_gat_split_rows(monkeypatch):
     monkeypatch.setenv("FGNN_SEG_LEN", "256")
     from ae_mlsys_gnn_amd import _lib

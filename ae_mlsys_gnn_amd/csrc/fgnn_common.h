@@ -120,6 +120,22 @@ __device__ __forceinline__ int fg_uni(int v) { return __builtin_amdgcn_readfirst
 __device__ __forceinline__ float fg_readlane(float v, int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l)); }
 __device__ __forceinline__ float fg_bperm(float v, int src_lane) { return __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane << 2, __float_as_int(v))); }
 
+// Marks a wave-uniform address as such for the compiler: the halves go through readfirstlane (free
+// for values that already sit in scalar registers), which keeps the address arithmetic before it on
+// the scalar unit and lets `base + 32-bit lane offset` loads use the scalar-base addressing mode.
+typedef float fg_f4 __attribute__((ext_vector_type(4)));
+typedef const __attribute__((address_space(1))) char *fg_gptr;        // a pointer known to be to global memory
+__device__ __forceinline__ fg_gptr fg_uniform_ptr(const void *p)
+{
+    uint64_t a = (uint64_t)p;
+    uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a), hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32));
+    return (fg_gptr)(((uint64_t)hi << 32) | lo);
+}
+// The empty asm re-defines a 32-bit lane offset inside the block it is called from.  Loads of that block
+// then show instruction selection "scalar base + zero-extended 32-bit offset" and get the scalar-base
+// form, with no address arithmetic on the vector unit (a zero-extension hoisted out of the loop hides it).
+__device__ __forceinline__ uint32_t fg_pin(uint32_t off) { asm volatile("" : "+v"(off)); return off; }
+
 template <int CTRL>
 __device__ __forceinline__ float fg_dpp(float v)
 {
@@ -156,6 +172,8 @@ __device__ __forceinline__ void fg_wave_lds_sync()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 __device__ __forceinline__ float fg_lrelu(float x, float slope) { return x > 0.f ? x : x * slope; }
+// max(x, 0) of a finite x as one integer maximum on the bit pattern (negative floats are negative integers)
+__device__ __forceinline__ float fg_relu_bits(float x) { return __int_as_float(max(__float_as_int(x), 0)); }
 // SLE1: the slope is known to lie in [0, 1], where LeakyReLU(x) == max(x, slope*x)
 template <bool SLE1>
 __device__ __forceinline__ float fg_lrelu_t(float x, float slope) { return SLE1 ? fmaxf(x, x * slope) : (x > 0.f ? x : x * slope); }
@@ -169,6 +187,7 @@ template <> struct fg_vec<4> {
     __device__ __forceinline__ void load(const float *p) { v = *reinterpret_cast<const float4 *>(p); }
     // wave-uniform base + unsigned 32-bit byte offset: lets the load use a scalar base register
     __device__ __forceinline__ void load_off(const char *base, uint32_t off) { v = *reinterpret_cast<const float4 *>(base + off); }
+    __device__ __forceinline__ void load_off(fg_gptr base, uint32_t off) { fg_f4 t = *(const __attribute__((address_space(1))) fg_f4 *)(base + off); v = make_float4(t.x, t.y, t.z, t.w); }
     __device__ __forceinline__ void store(float *p) const { *reinterpret_cast<float4 *>(p) = v; }
     // streaming store: the line is not kept in L2 (results nobody gathers again in this kernel)
     __device__ __forceinline__ void store_nt(float *p) const { __builtin_nontemporal_store(v.x, p); __builtin_nontemporal_store(v.y, p + 1); __builtin_nontemporal_store(v.z, p + 2); __builtin_nontemporal_store(v.w, p + 3); }
@@ -184,6 +203,7 @@ template <> struct fg_vec<1> {
     __device__ __forceinline__ void zero() { v = 0.f; }
     __device__ __forceinline__ void load(const float *p) { v = *p; }
     __device__ __forceinline__ void load_off(const char *base, uint32_t off) { v = *reinterpret_cast<const float *>(base + off); }
+    __device__ __forceinline__ void load_off(fg_gptr base, uint32_t off) { v = *(const __attribute__((address_space(1))) float *)(base + off); }
     __device__ __forceinline__ void store(float *p) const { *p = v; }
     __device__ __forceinline__ void store_nt(float *p) const { __builtin_nontemporal_store(v, p); }
     __device__ __forceinline__ void fma(float w, const fg_vec &x) { v = fmaf(w, x.v, v); }

@@ -124,14 +124,17 @@ __device__ __forceinline__ void gat_fwd_pair_batch(const GatFwdP &p, const fg_la
     float acn = 0.f;
     if (t + UB < cnt) acn = gat_fwd_pair_fetch(p, pr, idv, t + UB, cnt);        // wave-uniform
     fg_vec<VEC> ld[UB][R];
-    const size_t row_bytes = (size_t)p.HF * sizeof(float);
+    const uint32_t row_bytes = (uint32_t)p.HF * 4u;
+    uint32_t bo[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) bo[r] = fg_pin(boff[r]);
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
-        size_t j = (size_t)(unsigned)__builtin_amdgcn_readlane(idv, (t + u) & 63);      // past the chunk: any valid row, weight 0
-        const char *base = (const char *)p.x + j * row_bytes;
+        uint64_t j = (uint64_t)(uint32_t)__builtin_amdgcn_readlane(idv, (t + u) & 63);      // past the chunk: any valid row, weight 0
+        fg_gptr base = fg_uniform_ptr((const char *)p.x + j * row_bytes);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            if (FULL || lm.ok[r]) ld[u][r].load_off(base, boff[r]); else ld[u][r].zero();
+            if (FULL || lm.ok[r]) ld[u][r].load_off(base, bo[r]); else ld[u][r].zero();
         }
     }
     const bool live = pr.ok && t + pr.u < cnt;
@@ -161,7 +164,7 @@ __device__ __forceinline__ void gat_fwd_pair_batch(const GatFwdP &p, const fg_la
             const int src = ((u << p.hp_shift) + lm.hd[r]) << 2;
             const float a = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(ws)));
             T[r].fma(AUX ? fabsf(a) : a, ld[u][r]);
-            if (AUX) P[r].fma(fmaxf(a, 0.f), ld[u][r]);
+            if (AUX) P[r].fma(fg_relu_bits(a), ld[u][r]);
         }
     }
     acv = acn;
@@ -642,14 +645,17 @@ __device__ __forceinline__ void gat_bwd_pair_batch(const GatBwdP &p, const fg_la
     nxt.rc = make_float4(0.f, 0.f, 0.f, 0.f); nxt.esm = 0.f;
     if (t + UB < cnt) nxt = gat_bwd_pair_fetch<STASH>(p, pr, idv, posv, t + UB, cnt);      // wave-uniform
     fg_vec<VEC> ld[UB][R];
-    const size_t row_bytes = (size_t)p.HF * sizeof(float);
+    const uint32_t row_bytes = (uint32_t)p.HF * 4u;
+    uint32_t bo[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) bo[r] = fg_pin(boff[r]);
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
-        size_t i = (size_t)(unsigned)__builtin_amdgcn_readlane(idv, (t + u) & 63);      // past the chunk: any valid row, weight 0
-        const char *base = (const char *)p.g + i * row_bytes;
+        uint64_t i = (uint64_t)(uint32_t)__builtin_amdgcn_readlane(idv, (t + u) & 63);      // past the chunk: any valid row, weight 0
+        fg_gptr base = fg_uniform_ptr((const char *)p.g + i * row_bytes);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            if (FULL || lm.ok[r]) ld[u][r].load_off(base, boff[r]); else ld[u][r].zero();
+            if (FULL || lm.ok[r]) ld[u][r].load_off(base, bo[r]); else ld[u][r].zero();
         }
     }
     const float4 rc = cur.rc;
@@ -667,7 +673,7 @@ __device__ __forceinline__ void gat_bwd_pair_batch(const GatBwdP &p, const fg_la
             const int src = ((u << p.hp_shift) + lm.hd[r]) << 2;
             const float a = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(als)));
             T[r].fma(fabsf(a), ld[u][r]);
-            P[r].fma(fmaxf(a, 0.f), ld[u][r]);
+            P[r].fma(fg_relu_bits(a), ld[u][r]);
         }
     }
     cur = nxt;

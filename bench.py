@@ -31,9 +31,9 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published peak
 # profiles/kernels_edgeconv_c3_gmm_c4_gat_c5_drivers.md); all kernels of the entry point summed.
 # They bound the HBM traffic from above.  None = not measured for that workload.
 MEASURED_TRAFFIC_BYTES = {
-    "gat_c2": {"fwd": 37136911667, "bwd": 33567448883},
+    "gat_c2": {"fwd": 38_905_487_360, "bwd": 39_145_359_872},
     "gat_c5_layer1": {"fwd": 72_099_949_465, "bwd": 81_156_805_427},
-    "gmm_c4": {"fwd": 1_154_166_988, "bwd": 1_514_758_144},
+    "gmm_c4": {"fwd": 1161785548, "bwd": 1468256256},
     "edgeconv_c3": {"fwd": 123_305_574, "bwd": 73_504_972},
 }
 

@@ -75,33 +75,57 @@ __global__ __launch_bounds__(256) void rs_digit_base_kernel(const int *__restric
 }
 
 // Stable scatter of one pass.  pay_in == NULL: the payload is the element's own index (first pass).
+// The tile is first sorted by digit inside LDS (local position = the digit's base inside the tile +
+// rank among the tile's earlier elements of that digit), then written out in local order: all
+// elements of a digit leave as one contiguous run, so neighbouring lanes write neighbouring addresses
+// instead of 4-byte stores scattered over 256 destinations.
 __global__ __launch_bounds__(RS_TPB) void rs_scatter_kernel(const int *__restrict__ keys_in, const int *__restrict__ pay_in, int64_t n, int shift,
                                                             int nblocks, const int *__restrict__ hist, const int *__restrict__ digit_base,
                                                             int *__restrict__ keys_out, int *__restrict__ pay_out)
 {
-    __shared__ int wcnt[4][256];
+    __shared__ int wcnt[4][256];        // per wave and digit: count, then the running local position
+    __shared__ int gofs[256];           // per digit: global position of the tile's run minus its local base
+    __shared__ int wave_tot[4];
+    __shared__ int skey[RS_TILE], spay[RS_TILE];
     const int wave = fg_wave(), lane = fg_lane();
     for (int i = (int)threadIdx.x; i < 4 * 256; i += RS_TPB) (&wcnt[0][0])[i] = 0;
     __syncthreads();
+    const int64_t tile0 = (int64_t)blockIdx.x * RS_TILE;
     int key[RS_ITEMS];
 #pragma unroll
     for (int it = 0; it < RS_ITEMS; ++it) {
-        int64_t i = (int64_t)blockIdx.x * RS_TILE + wave * RS_SUB + it * 64 + lane;
+        int64_t i = tile0 + wave * RS_SUB + it * 64 + lane;
         key[it] = i < n ? keys_in[i] : 0;
         if (i < n) atomicAdd(&wcnt[wave][(key[it] >> shift) & 255], 1);
     }
     __syncthreads();
     {
-        int d = (int)threadIdx.x;
-        int base = digit_base[d] + hist[(size_t)d * nblocks + blockIdx.x];
+        // thread d owns digit d: exclusive scan of the tile's digit counts (inside the wave by shuffles,
+        // across the four waves through LDS), then the per-wave starting positions
+        const int d = (int)threadIdx.x;
+        int c[4], tot = 0;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) { int t = wcnt[w][d]; wcnt[w][d] = base; base += t; }
+        for (int w = 0; w < 4; ++w) { c[w] = wcnt[w][d]; tot += c[w]; }
+        int incl = tot;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            int t = __shfl_up(incl, off);
+            if (lane >= off) incl += t;
+        }
+        if (lane == 63) wave_tot[wave] = incl;
+        __syncthreads();
+        int lbase = incl - tot;
+        for (int w = 0; w < wave; ++w) lbase += wave_tot[w];
+        gofs[d] = digit_base[d] + hist[(size_t)d * nblocks + blockIdx.x] - lbase;
+        int run = lbase;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) { wcnt[w][d] = run; run += c[w]; }
     }
     __syncthreads();
     const unsigned long long lt = (1ull << lane) - 1ull;
 #pragma unroll
     for (int it = 0; it < RS_ITEMS; ++it) {
-        int64_t i = (int64_t)blockIdx.x * RS_TILE + wave * RS_SUB + it * 64 + lane;
+        int64_t i = tile0 + wave * RS_SUB + it * 64 + lane;
         bool ok = i < n;
         int d = (key[it] >> shift) & 255;
         unsigned long long peers = __builtin_amdgcn_ballot_w64(ok);
@@ -113,20 +137,51 @@ __global__ __launch_bounds__(RS_TPB) void rs_scatter_kernel(const int *__restric
         int rank = __popcll(peers & lt);
         int base = wcnt[wave][d];
         if (ok) {
-            int dst = base + rank;
-            keys_out[dst] = key[it];
-            pay_out[dst] = pay_in ? pay_in[i] : (int)i;
+            skey[base + rank] = key[it];
+            spay[base + rank] = pay_in ? pay_in[i] : (int)i;
         }
         fg_wave_lds_sync();
         // the highest lane of every peer group advances the wave's counter of that digit
         if (ok && (peers >> lane) == 1ull) wcnt[wave][d] = base + __popcll(peers);
         fg_wave_lds_sync();
     }
+    __syncthreads();
+    const int count = (int)((n - tile0) < (int64_t)RS_TILE ? (n - tile0) : (int64_t)RS_TILE);
+#pragma unroll 4
+    for (int i = (int)threadIdx.x; i < count; i += RS_TPB) {
+        int k = skey[i];
+        int dst = gofs[(k >> shift) & 255] + i;
+        keys_out[dst] = k;
+        pay_out[dst] = spay[i];
+    }
+}
+
+// Row of CSR position p: the last r with row_ptr[r] <= p, searched in [lo, hi) with row_ptr[lo] <= p < row_ptr[hi].
+__device__ __forceinline__ int csc_row_of(const int *__restrict__ row_ptr, int lo, int hi, int p)
+{
+    while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if (row_ptr[mid] <= p) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+// hint[k] = row of position min(k << CSC_HINT_SHIFT, n - 1), k = 0 .. n_hint - 1: a coarse inverse of
+// row_ptr, so that the per-entry search of csc_finalize_kernel covers the few rows of one bucket of
+// positions instead of the whole pointer array.
+#define CSC_HINT_SHIFT 9
+__global__ __launch_bounds__(256) void csc_row_hint_kernel(int64_t n, int n_rows, int n_hint, const int *__restrict__ row_ptr, int *__restrict__ hint)
+{
+    int k = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    if (k >= n_hint) return;
+    int64_t p = (int64_t)k << CSC_HINT_SHIFT;
+    if (p > n - 1) p = n - 1;
+    hint[k] = csc_row_of(row_ptr, 0, n_rows, (int)p);
 }
 
 __global__ __launch_bounds__(256) void csc_finalize_kernel(int64_t n, int n_rows, int n_cols, const int *__restrict__ sorted_keys,
                                                            const int *__restrict__ permute, const int *__restrict__ row_ptr,
-                                                           int *__restrict__ col_ptr, int *__restrict__ row_ind)
+                                                           const int *__restrict__ hint, int *__restrict__ col_ptr, int *__restrict__ row_ind)
 {
     int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (q >= n) return;
@@ -135,14 +190,9 @@ __global__ __launch_bounds__(256) void csc_finalize_kernel(int64_t n, int n_rows
     for (int c = prev + 1; c <= key; ++c) col_ptr[c] = (int)q;
     if (q == n - 1)
         for (int c = key + 1; c <= n_cols; ++c) col_ptr[c] = (int)n;
-    // row of CSR position p: the last r with row_ptr[r] <= p
     int p = permute[q];
-    int lo = 0, hi = n_rows;            // invariant: row_ptr[lo] <= p < row_ptr[hi]
-    while (hi - lo > 1) {
-        int mid = (lo + hi) >> 1;
-        if (row_ptr[mid] <= p) lo = mid; else hi = mid;
-    }
-    row_ind[q] = lo;
+    int k = p >> CSC_HINT_SHIFT;
+    row_ind[q] = csc_row_of(row_ptr, hint[k], hint[k + 1] + 1, p);
 }
 
 __global__ __launch_bounds__(256) void fill_i32_kernel(int *p, size_t n, int v)
@@ -208,10 +258,12 @@ static int rs_sort_pairs(const int *keys_in, const int *pay_in, int64_t n, int p
     return 0;
 }
 
+static int csc_num_hints(int64_t E) { return E > 0 ? (int)((E - 1) >> CSC_HINT_SHIFT) + 2 : 0; }
+
 extern "C" size_t fgnn_csr2csc_workspace_bytes(int n_rows, int n_cols, int64_t E)
 {
     (void)n_rows; (void)n_cols;
-    return rs_sort_workspace(E);
+    return rs_sort_workspace(E) + fgnn_align256((size_t)csc_num_hints(E) * sizeof(int));
 }
 
 extern "C" int fgnn_csr2csc(int n_rows, int n_cols, int64_t E, const int32_t *row_ptr, const int32_t *col_ind, int32_t *col_ptr,
@@ -231,7 +283,12 @@ extern "C" int fgnn_csr2csc(int n_rows, int n_cols, int64_t E, const int32_t *ro
     const int *sorted = nullptr;
     int rc = rs_sort_pairs(col_ind, nullptr, E, rs_num_passes(n_cols), permute, &sorted, workspace, st);
     if (rc) return rc;
-    hipLaunchKernelGGL(csc_finalize_kernel, dim3((unsigned)((E + 255) / 256)), dim3(256), 0, st, E, n_rows, n_cols, sorted, permute, row_ptr, col_ptr, row_ind);
+    int *hint = (int *)((char *)workspace + rs_sort_workspace(E));
+    const int n_hint = csc_num_hints(E);
+    hipLaunchKernelGGL(csc_row_hint_kernel, dim3((unsigned)((n_hint + 255) / 256)), dim3(256), 0, st, E, n_rows, n_hint, row_ptr, hint);
+    rc = fgnn_launch_status("csc_row_hint_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(csc_finalize_kernel, dim3((unsigned)((E + 255) / 256)), dim3(256), 0, st, E, n_rows, n_cols, sorted, permute, row_ptr, hint, col_ptr, row_ind);
     return fgnn_launch_status("csc_finalize_kernel");
 }
 

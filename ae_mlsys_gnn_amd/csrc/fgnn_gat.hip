@@ -279,7 +279,10 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_kernel(GatFwdP p)
 // cut into G lane groups (fg_packmap) that take different edges of the row with the same load
 // instruction, each with its own online softmax state; the groups are combined by a log-sum-exp
 // butterfly before the row is written.
-template <int G, bool AUX, bool SLE1>
+// PAIR: the scores are handled in the pair layout of gat_fwd_pair_batch, one lane per (entry of the
+// batch of 8*G, head); the wave then keeps ONE running maximum per head, so the groups' accumulators
+// are plain partial sums.
+template <int G, bool AUX, bool SLE1, bool PAIR>
 __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_packed_kernel(GatFwdP p)
 {
     int row, b, e, slot;
@@ -294,13 +297,55 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_packed_kernel(GatFwdP p)
     float s = 0.f, cp = 0.f, m = -INFINITY;
     const float arh = p.ar[(size_t)row * H + pm.hd] * FGNN_LOG2E;
     constexpr int U = 8;
+    GatFwdPair pr;
+    pr.u = lane >> p.hp_shift; pr.h = lane & ((1 << p.hp_shift) - 1);
+    pr.ok = PAIR && pr.h < H && pr.u < U * G;
+    pr.arh = pr.ok ? p.ar[(size_t)row * H + pr.h] * FGNN_LOG2E : 0.f;
+    pr.m = pr.ok ? -INFINITY : 0.f; pr.s = 0.f; pr.cp = 0.f;
     for (int c = b; c < e; c += 64) {
         int q = c + lane;
         int cnt = min(64, e - c);
         int idv = p.idx[q < e ? q : c];
+        float acv = 0.f;
+        if constexpr (PAIR) acv = gat_fwd_pair_fetch(p, pr, idv, 0, cnt);
         for (int t = 0; t < cnt; t += U * G) {
             fg_vec<4> ld[U];
             float ev[U];
+            if constexpr (PAIR) {
+                float acn = 0.f;
+                if (t + U * G < cnt) acn = gat_fwd_pair_fetch(p, pr, idv, t + U * G, cnt);      // wave-uniform
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int ei = t + u * G + pm.grp;
+                    const size_t j = (size_t)(unsigned)__builtin_amdgcn_ds_bpermute((ei & 63) << 2, idv);
+                    if (ei < cnt && pm.ok) ld[u].load(p.x + j * p.HF + pm.eoff); else ld[u].zero();
+                }
+                const bool live = pr.ok && t + pr.u < cnt;
+                const float v = live ? fg_lrelu_t<SLE1>(fmaf(acv, FGNN_LOG2E, pr.arh), slope) : -INFINITY;
+                float bm = v;
+                for (int sft = 1 << p.hp_shift; sft < 64; sft <<= 1) bm = fmaxf(bm, fg_bperm(bm, lane ^ sft));
+                if (__builtin_amdgcn_ballot_w64(bm > pr.m) != 0ull) {
+                    const float mn = fmaxf(pr.m, bm);
+                    const float sc = __builtin_amdgcn_exp2f(pr.m - mn);
+                    pr.m = mn; pr.s *= sc; pr.cp *= sc;
+                    const float scf = fg_bperm(sc, pm.hd);
+                    T.scale(scf);
+                    if (AUX) P.scale(scf);
+                }
+                const float w = __builtin_amdgcn_exp2f(v - pr.m);       // 0 for the slots without an edge
+                const float wp = v > 0.f ? w : 0.f;
+                pr.s += w; pr.cp += wp;
+                const float ws = (!AUX || v > 0.f) ? w : -w;            // the sign carries "pre-activation positive"
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int src = (((u * G + pm.grp) << p.hp_shift) + pm.hd) << 2;
+                    const float a = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(ws)));
+                    T.fma(AUX ? fabsf(a) : a, ld[u]);
+                    if (AUX) P.fma(fg_relu_bits(a), ld[u]);
+                }
+                acv = acn;
+                continue;
+            }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int ei = t + u * G + pm.grp;
@@ -337,9 +382,17 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_packed_kernel(GatFwdP p)
             }
         }
     }
+    if constexpr (PAIR) {
+        // one maximum per head for the whole wave: the groups add up; sums over the entry slots
+        fg_pack_reduce<G>(T, lane);
+        if (AUX) fg_pack_reduce<G>(P, lane);
+        float st = pr.s, ct = pr.cp;
+        for (int sft = 1 << p.hp_shift; sft < 64; sft <<= 1) { st += fg_bperm(st, lane ^ sft); ct += fg_bperm(ct, lane ^ sft); }
+        m = fg_bperm(pr.m, pm.hd); s = fg_bperm(st, pm.hd); cp = fg_bperm(ct, pm.hd);
+    }
     // combine the lane groups: (m, s, cp, T, P) of the partner group, rescaled to the common maximum
 #pragma unroll
-    for (int step = 64 / G; step < 64; step <<= 1) {
+    for (int step = PAIR ? 64 : 64 / G; step < 64; step <<= 1) {
         const int o = lane ^ step;
         float mo = fg_bperm(m, o);
         float mn = fmaxf(m, mo);
@@ -759,7 +812,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_kernel(GatBwdP p)
 
 // The column pass for rows narrower than a wave: G entries of the column per load instruction
 // (see gat_fwd_packed_kernel); T, P and z are plain sums, so the groups are added by a butterfly.
-template <int G, bool STASH, bool SLE1>
+template <int G, bool STASH, bool SLE1, bool PAIR>
 __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
 {
     extern __shared__ float lds[];
@@ -775,14 +828,51 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
     float z = 0.f;
     const float ach = p.ac[(size_t)col * H + pm.hd];
     constexpr int U = 8;
+    // PAIR: the attention weights are formed in the pair layout of gat_bwd_pair_batch, one lane per
+    // (entry of the batch of 8*G, head)
+    GatPair pr;
+    pr.u = lane >> p.hp_shift; pr.h = lane & ((1 << p.hp_shift) - 1);
+    pr.ok = PAIR && pr.h < H && pr.u < U * G;
+    pr.ach = pr.ok ? p.ac[(size_t)col * H + pr.h] : 0.f;
+    pr.z = 0.f;
     for (int c = b; c < e; c += 64) {
         int q = c + lane;
         int cnt = min(64, e - c);
         int qq = q < e ? q : c;
         int idv = p.idx[qq];
         int posv = STASH ? p.permute[p.pos ? p.pos[qq] : qq] : 0;
+        GatPairRec cur;
+        cur.rc = make_float4(0.f, 0.f, 0.f, 0.f); cur.esm = 0.f;
+        if constexpr (PAIR) cur = gat_bwd_pair_fetch<STASH>(p, pr, idv, posv, 0, cnt);
         for (int t = 0; t < cnt; t += U * G) {
             fg_vec<4> ld[U];
+            if constexpr (PAIR) {
+                GatPairRec nxt;
+                nxt.rc = make_float4(0.f, 0.f, 0.f, 0.f); nxt.esm = 0.f;
+                if (t + U * G < cnt) nxt = gat_bwd_pair_fetch<STASH>(p, pr, idv, posv, t + U * G, cnt);     // wave-uniform
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int ei = t + u * G + pm.grp;
+                    const size_t i = (size_t)(unsigned)__builtin_amdgcn_ds_bpermute((ei & 63) << 2, idv);
+                    if (ei < cnt && pm.ok) ld[u].load(p.g + i * p.HF + pm.eoff); else ld[u].zero();
+                }
+                const float4 rc = cur.rc;
+                float ev, al;
+                if (STASH) { ev = fmaf(pr.ach, FGNN_LOG2E, rc.x); al = cur.esm; }
+                else { ev = fg_lrelu_t<SLE1>(fmaf(pr.ach, FGNN_LOG2E, rc.x), p.slope); al = __builtin_amdgcn_exp2f(ev - rc.y) * rc.z; }
+                al = (pr.ok && t + pr.u < cnt) ? al : 0.f;
+                pr.z = fmaf(ev > 0.f ? al : al * p.slope, rc.w, pr.z);
+                const float als = ev > 0.f ? al : -al;      // the sign carries "pre-activation positive"
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int src = (((u * G + pm.grp) << p.hp_shift) + pm.hd) << 2;
+                    const float a = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(als)));
+                    T.fma(fabsf(a), ld[u]);
+                    P.fma(fg_relu_bits(a), ld[u]);
+                }
+                cur = nxt;
+                continue;
+            }
             float4 rc[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
@@ -813,8 +903,14 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
     }
     fg_pack_reduce<G>(T, lane);
     fg_pack_reduce<G>(P, lane);
+    if constexpr (PAIR) {
+        float zt = pr.z;
+        for (int sft = 1 << p.hp_shift; sft < 64; sft <<= 1) zt += fg_bperm(zt, lane ^ sft);
+        z = fg_bperm(zt, pm.hd);
+    } else {
 #pragma unroll
-    for (int step = 64 / G; step < 64; step <<= 1) z += fg_bperm(z, lane ^ step);
+        for (int step = 64 / G; step < 64; step <<= 1) z += fg_bperm(z, lane ^ step);
+    }
     fg_lanemap<4, 1> lm;
     lm.eoff[0] = pm.eoff; lm.hd[0] = pm.hd; lm.ok[0] = pm.ok && pm.grp == 0;
     if (slot < 0) {
@@ -919,11 +1015,18 @@ static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_
         const bool sle1 = slope >= 0.f && slope <= 1.f;
         const int pack = fgnn_pick_pack(cfg.vec, HF);
         if (pack > 1) {
+            p.hp_shift = 0;
+            while ((1 << p.hp_shift) < H) ++p.hp_shift;
+            // the pair layout needs 8*G entry slots x heads (rounded up to a power of two) <= 64 lanes
+            const bool pair = ((8 * pack) << p.hp_shift) <= 64 && E >= 64 * (int64_t)N;
             auto launch = [&]<int G>() {
-                if (aux && sle1) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, true>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
-                else if (aux) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, false>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
-                else if (sle1) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, false, true>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
-                else hipLaunchKernelGGL((gat_fwd_packed_kernel<G, false, false>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
+                auto go = [&]<bool PAIR>() {
+                    if (aux && sle1) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, true, PAIR>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
+                    else if (aux) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, false, PAIR>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
+                    else if (sle1) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, false, true, PAIR>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
+                    else hipLaunchKernelGGL((gat_fwd_packed_kernel<G, false, false, PAIR>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
+                };
+                if (pair) go.template operator()<true>(); else go.template operator()<false>();
             };
             if (pack == 8) launch.template operator()<8>();
             else if (pack == 4) launch.template operator()<4>();
@@ -1065,10 +1168,16 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
         const bool sle1 = negative_slope >= 0.f && negative_slope <= 1.f;
         const int pack = fgnn_pick_pack(cfg.vec, HF);
         if (pack > 1) {
+            p.hp_shift = 0;
+            while ((1 << p.hp_shift) < H) ++p.hp_shift;
+            const bool pair = ((8 * pack) << p.hp_shift) <= 64 && E >= 64 * (int64_t)N;
             auto launch = [&]<int G>() {
-                if (stash) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, true, true>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
-                else if (sle1) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, false, true>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
-                else hipLaunchKernelGGL((gat_bwd_packed_kernel<G, false, false>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                auto go = [&]<bool PAIR>() {
+                    if (stash) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, true, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                    else if (sle1) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, false, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                    else hipLaunchKernelGGL((gat_bwd_packed_kernel<G, false, false, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                };
+                if (pair) go.template operator()<true>(); else go.template operator()<false>();
             };
             if (pack == 8) launch.template operator()<8>();
             else if (pack == 4) launch.template operator()<4>();

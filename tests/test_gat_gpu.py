@@ -76,12 +76,14 @@ def test_gat_rows_narrower_than_a_wave(h, f, variant, monkeypatch):
 
 
 @pytest.mark.parametrize("variant", ["sm", "stash"])
-@pytest.mark.parametrize("h,f", [(8, 32), (4, 64), (1, 256), (2, 72), (5, 52), (16, 32), (16, 16), (3, 50), (7, 36), (64, 16), (33, 31)])
+@pytest.mark.parametrize("h,f", [(8, 32), (4, 64), (1, 256), (2, 72), (5, 52), (16, 32), (16, 16), (3, 50), (7, 36), (64, 16), (33, 31),
+                                 (1, 128), (1, 44), (1, 64), (2, 64), (2, 24), (1, 16), (1, 32), (3, 40), (4, 16), (1, 4)])
 def test_gat_long_rows_pair_layout(h, f, variant, monkeypatch):
     """Graphs averaging 64 or more entries per row take the kernels that compute the attention weights
     once per (edge, head) on one lane and hand them to the feature lanes (where edges-per-batch x heads
-    fits the wave; (16, 16) and (33, 31) do not and keep the per-lane form).  Degrees 0..3000 with
-    ragged batch tails, whole and split rows, and an XCD-aware schedule."""
+    fits the wave; (16, 16), (33, 31) and (4, 16) do not and keep the per-lane form), in the kernels for
+    wide rows and in the packed ones for H*F <= 128.  Degrees 0..3000 with ragged batch tails, whole and
+    split rows, and an XCD-aware schedule."""
     from ae_mlsys_gnn_amd import _lib
     g = degree_edge_graph(n=80, seed=21)
     assert g.n_edges >= 64 * g.n

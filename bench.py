@@ -262,9 +262,10 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
         "sparse_fwd_bwd": {"ms": round(ms_fwd + ms_bwd, 4), "alg_bytes": b_fwd + b_bwd,
                            "achieved_GBps": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6, 1),
                            "frac_of_peak": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6 / HBM_PEAK_GBPS, 4)},
-        "cpu_baseline": {"value": round(cpu_ms * e / cpu_e, 1), "unit": "ms/iter", "cores": cores, "kind": "port",
-                         "sample": "DGL-composed GAT layer (torch CPU, %d threads) fwd+bwd on the first %d rows = %d edges of the same graph: "
-                                   "median %.1f ms over %d iters, scaled by E/E_sample = %.1f" % (cores, cpu_rows, cpu_e, cpu_ms, cpu_iters, e / cpu_e)},
+        "cpu_baseline": None if args.no_cpu_baseline else {
+            "value": round(cpu_ms * e / cpu_e, 1), "unit": "ms/iter", "cores": cores, "kind": "port",
+            "sample": "DGL-composed GAT layer (torch CPU, %d threads) fwd+bwd on the first %d rows = %d edges of the same graph: "
+                      "median %.1f ms over %d iters, scaled by E/E_sample = %.1f" % (cores, cpu_rows, cpu_e, cpu_ms, cpu_iters, e / cpu_e)},
         "cpu_baseline_c1": c1,
         "preprocess_s": {"graph_gen": round(t_gen, 3), "csr2csc_first_call": round(t_csc, 4), "schedules": round(t_sched, 4), **prep},
         "schedule": {"xcd_aware": s_csr.idx_tensor is not None, "csr_items": s_csr.n_items, "csr_partials": s_csr.n_partials,

@@ -58,6 +58,9 @@ _SIGNATURES = {
     "fgnn_edge_softmax_backward": (c_int, [c_int, c_int64, c_int] + [c_void_p] * 4 + [c_void_p]),
     "fgnn_u_add_v": (c_int, [c_int, c_int64, c_int] + [c_void_p] * 5 + [c_void_p]),
     "fgnn_u_add_v_backward": (c_int, [c_int, c_int64, c_int] + [c_void_p] * 5 + [c_void_p]),
+    "fgnn_edge_linear_tanh": (c_int, [c_int64, c_int] + [c_void_p] * 4 + [c_void_p]),
+    "fgnn_edge_linear_tanh_backward_workspace_bytes": (c_size_t, [c_int64, c_int]),
+    "fgnn_edge_linear_tanh_backward": (c_int, [c_int64, c_int] + [c_void_p] * 5 + [c_void_p, c_size_t, c_void_p]),
     "fgnn_coo2csr_workspace_bytes": (c_size_t, [c_int, c_int, c_int64]),
     "fgnn_coo2csr": (c_int, [c_int, c_int, c_int64, c_void_p, c_void_p, c_int] + [c_void_p] * 4 + [c_void_p, c_size_t, c_void_p]),
     "fgnn_csr2csc_workspace_bytes": (c_size_t, [c_int, c_int, c_int64]),

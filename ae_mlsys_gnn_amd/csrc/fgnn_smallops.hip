@@ -288,3 +288,120 @@ extern "C" int fgnn_u_add_v_backward(int N, int64_t E, int W, const int32_t *row
                        grad_row, grad_col);
     return fgnn_launch_status("u_add_v_bwd_kernel");
 }
+
+// ------------------------------------------------------------------------------- per-edge Linear(2, D) + tanh
+// The pseudo-coordinate projection of the MoNet drivers (script/train/train_gmmconv_our.py:46-57:
+// nn.Sequential(nn.Linear(2, dim), nn.Tanh()) applied to the [E, 2] edge coordinates), as one pass
+// over the edges each way instead of a chain of elementwise kernels; its weight gradient is a
+// reduction over all E edges, done here with per-thread partial sums, a fixed-order workgroup
+// reduction and a fixed-order sum over the workgroups (deterministic).
+#define ELT_BLOCKS 1024
+template <int D>
+__global__ __launch_bounds__(256) void edge_linear_tanh_kernel(int64_t E, const float2 *__restrict__ x, const float *__restrict__ W,
+                                                               const float *__restrict__ b, float *__restrict__ y)
+{
+    float w0[D], w1[D], bb[D];
+#pragma unroll
+    for (int o = 0; o < D; ++o) { w0[o] = W[2 * o]; w1[o] = W[2 * o + 1]; bb[o] = b[o]; }
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < E; e += (int64_t)gridDim.x * 256) {
+        const float2 v = x[e];
+#pragma unroll
+        for (int o = 0; o < D; ++o) y[e * D + o] = tanhf(fmaf(v.y, w1[o], fmaf(v.x, w0[o], bb[o])));
+    }
+}
+
+// part[block][3*D]: per output o the partial sums of gt*x0, gt*x1, gt with gt = g * (1 - y^2).
+template <int D>
+__global__ __launch_bounds__(256) void edge_linear_tanh_bwd_kernel(int64_t E, const float2 *__restrict__ x, const float *__restrict__ y,
+                                                                   const float *__restrict__ g, float *__restrict__ part)
+{
+    __shared__ float sh[4][3 * D];
+    float acc[3 * D];
+#pragma unroll
+    for (int i = 0; i < 3 * D; ++i) acc[i] = 0.f;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < E; e += (int64_t)gridDim.x * 256) {
+        const float2 v = x[e];
+#pragma unroll
+        for (int o = 0; o < D; ++o) {
+            const float yy = y[e * D + o];
+            const float gt = g[e * D + o] * (1.f - yy * yy);
+            acc[3 * o] = fmaf(gt, v.x, acc[3 * o]);
+            acc[3 * o + 1] = fmaf(gt, v.y, acc[3 * o + 1]);
+            acc[3 * o + 2] += gt;
+        }
+    }
+    const int lane = fg_lane(), wave = fg_wave();
+#pragma unroll
+    for (int i = 0; i < 3 * D; ++i) {
+        float s = fg_wave_sum(acc[i]);
+        if (lane == 0) sh[wave][i] = s;
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < 3 * D)
+        part[(size_t)blockIdx.x * 3 * D + threadIdx.x] = (sh[0][threadIdx.x] + sh[1][threadIdx.x]) + (sh[2][threadIdx.x] + sh[3][threadIdx.x]);
+}
+
+__global__ __launch_bounds__(64) void edge_linear_tanh_finish_kernel(int nblk, int D, const float *__restrict__ part, float *__restrict__ gW,
+                                                                     float *__restrict__ gb)
+{
+    const int i = (int)threadIdx.x;
+    if (i >= 3 * D) return;
+    float s = 0.f;
+    for (int k = 0; k < nblk; ++k) s += part[(size_t)k * 3 * D + i];
+    const int o = i / 3, c = i - 3 * o;
+    if (c < 2) gW[2 * o + c] = s; else gb[o] = s;
+}
+
+static int elt_blocks(int64_t E) { return (int)std::min<int64_t>(ELT_BLOCKS, (E + 255) / 256); }
+
+extern "C" int fgnn_edge_linear_tanh(int64_t E, int D, const float *x, const float *W, const float *b, float *y, void *stream)
+{
+    FGNN_REQUIRE(E >= 0, FGNN_ERR_SHAPE, "fgnn_edge_linear_tanh: E=%lld", (long long)E);
+    FGNN_REQUIRE(D >= 1 && D <= 4, FGNN_ERR_LIMIT, "fgnn_edge_linear_tanh: %d output columns unsupported (1..4)", D);
+    if (E == 0) return 0;
+    FGNN_REQUIRE(x && W && b && y, FGNN_ERR_NULL, "fgnn_edge_linear_tanh: NULL argument");
+    FGNN_REQUIRE((((uintptr_t)x) & 7u) == 0, FGNN_ERR_ALIGN, "fgnn_edge_linear_tanh: x not 8-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid((unsigned)std::min<int64_t>(8192, (E + 255) / 256));
+    switch (D) {
+    case 1: hipLaunchKernelGGL(edge_linear_tanh_kernel<1>, grid, dim3(256), 0, st, E, (const float2 *)x, W, b, y); break;
+    case 2: hipLaunchKernelGGL(edge_linear_tanh_kernel<2>, grid, dim3(256), 0, st, E, (const float2 *)x, W, b, y); break;
+    case 3: hipLaunchKernelGGL(edge_linear_tanh_kernel<3>, grid, dim3(256), 0, st, E, (const float2 *)x, W, b, y); break;
+    default: hipLaunchKernelGGL(edge_linear_tanh_kernel<4>, grid, dim3(256), 0, st, E, (const float2 *)x, W, b, y); break;
+    }
+    return fgnn_launch_status("edge_linear_tanh_kernel");
+}
+
+extern "C" size_t fgnn_edge_linear_tanh_backward_workspace_bytes(int64_t E, int D)
+{
+    return (size_t)elt_blocks(E) * 3 * (size_t)(D > 0 ? D : 1) * sizeof(float);
+}
+
+extern "C" int fgnn_edge_linear_tanh_backward(int64_t E, int D, const float *x, const float *y, const float *grad_y, float *grad_W,
+                                              float *grad_b, void *workspace, size_t workspace_bytes, void *stream)
+{
+    FGNN_REQUIRE(E >= 0, FGNN_ERR_SHAPE, "fgnn_edge_linear_tanh_backward: E=%lld", (long long)E);
+    FGNN_REQUIRE(D >= 1 && D <= 4, FGNN_ERR_LIMIT, "fgnn_edge_linear_tanh_backward: %d output columns unsupported (1..4)", D);
+    FGNN_REQUIRE(grad_W && grad_b, FGNN_ERR_NULL, "fgnn_edge_linear_tanh_backward: NULL argument");
+    hipStream_t st = (hipStream_t)stream;
+    if (E == 0) {
+        int rc = fgnn_fill_f32(grad_W, 2 * (size_t)D, 0.f, st);
+        return rc ? rc : fgnn_fill_f32(grad_b, (size_t)D, 0.f, st);
+    }
+    FGNN_REQUIRE(x && y && grad_y, FGNN_ERR_NULL, "fgnn_edge_linear_tanh_backward: NULL argument");
+    FGNN_REQUIRE((((uintptr_t)x) & 7u) == 0, FGNN_ERR_ALIGN, "fgnn_edge_linear_tanh_backward: x not 8-byte aligned");
+    const size_t need = fgnn_edge_linear_tanh_backward_workspace_bytes(E, D);
+    FGNN_REQUIRE(workspace && workspace_bytes >= need, FGNN_ERR_WORKSPACE, "fgnn_edge_linear_tanh_backward: workspace %zu < %zu bytes", workspace_bytes, need);
+    const int nblk = elt_blocks(E);
+    float *part = (float *)workspace;
+    switch (D) {
+    case 1: hipLaunchKernelGGL(edge_linear_tanh_bwd_kernel<1>, dim3(nblk), dim3(256), 0, st, E, (const float2 *)x, y, grad_y, part); break;
+    case 2: hipLaunchKernelGGL(edge_linear_tanh_bwd_kernel<2>, dim3(nblk), dim3(256), 0, st, E, (const float2 *)x, y, grad_y, part); break;
+    case 3: hipLaunchKernelGGL(edge_linear_tanh_bwd_kernel<3>, dim3(nblk), dim3(256), 0, st, E, (const float2 *)x, y, grad_y, part); break;
+    default: hipLaunchKernelGGL(edge_linear_tanh_bwd_kernel<4>, dim3(nblk), dim3(256), 0, st, E, (const float2 *)x, y, grad_y, part); break;
+    }
+    int rc = fgnn_launch_status("edge_linear_tanh_bwd_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(edge_linear_tanh_finish_kernel, dim3(1), dim3(64), 0, st, nblk, D, part, grad_W, grad_b);
+    return fgnn_launch_status("edge_linear_tanh_finish_kernel");
+}

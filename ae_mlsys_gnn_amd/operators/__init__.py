@@ -1,6 +1,7 @@
 """Python mirror of the reference's ``operators/`` package for the fused sparse-operator path.
 Same callables and signatures; the work is done by libfgnn_hip.so."""
 from .csr2csc import sparsetrans  # noqa: F401  (the csr2csc function lives in the csr2csc submodule)
+from .edge_proj import EdgeLinearTanhFunction, edge_linear_tanh  # noqa: F401
 from .edge_softmax import EdgeSoftmaxFunction, csr_edge_softmax  # noqa: F401
 from .fused_edgeconv import FusedEdgeConvFunction, fused_edgeconv_op  # noqa: F401
 from .fused_gat import (FusedGATFunction, FusedGATFunction_SM, FusedGATFunction_stash,  # noqa: F401

@@ -16,6 +16,7 @@ import torch
 from torch import nn
 
 from ..layers import GMMConv, GMMConv_stash
+from ..operators import edge_proj
 from . import common, datasets
 
 VARIANTS = {"our": GMMConv, "stash": GMMConv_stash}
@@ -23,11 +24,15 @@ VARIANTS = {"our": GMMConv, "stash": GMMConv_stash}
 
 class PseudoProj(nn.Linear):
     """Linear(2, dim) + Tanh over the per-edge pseudo-coordinates (train_gmmconv_our.py:46-57), same
-    parameters as nn.Linear.  With only two input columns and one row per edge the product is written
-    as two broadcast multiplies: its weight gradient is then a column reduction over the edges rather
-    than a 2 x dim GEMM with a reduction length of E, which GEMM libraries run on a single workgroup."""
+    parameters as nn.Linear.  Up to 4 output columns run as one fused pass over the edges each way
+    (operators.edge_proj; the coordinates are data, only the parameters get gradients).  Wider
+    projections are written as two broadcast multiplies: the weight gradient is then a column reduction
+    over the edges rather than a 2 x dim GEMM with a reduction length of E, which GEMM libraries run
+    on a single workgroup."""
 
     def forward(self, pseudo):
+        if self.out_features <= edge_proj.MAX_OUT and pseudo.is_cuda and not pseudo.requires_grad:
+            return edge_proj.edge_linear_tanh(pseudo, self.weight, self.bias)
         out = pseudo[:, 0:1] * self.weight[:, 0] + pseudo[:, 1:2] * self.weight[:, 1]
         return torch.tanh(out + self.bias)
 

@@ -222,6 +222,19 @@ int    fgnn_u_add_v(int N, int64_t E, int W, const int32_t *row_ptr, const int32
 int    fgnn_u_add_v_backward(int N, int64_t E, int W, const int32_t *row_ptr, const int32_t *col_ind,
                              const float *grad_out, float *grad_row, float *grad_col, void *stream);
 
+/* The per-edge pseudo-coordinate projection of the MoNet drivers, nn.Sequential(nn.Linear(2, D),
+ * nn.Tanh()) on the [E, 2] edge coordinates (script/train/train_gmmconv_our.py:46-57), in one pass
+ * over the edges each way: y[e,o] = tanh(x[e,0]*W[o,0] + x[e,1]*W[o,1] + b[o]), 1 <= D <= 4,
+ * W [D,2] and b [D] as in nn.Linear.  The backward returns the parameter gradients (the coordinates are
+ * data): grad_W[o,c] = sum_e gt[e,o]*x[e,c], grad_b[o] = sum_e gt[e,o], gt = grad_y*(1 - y^2), summed in
+ * a fixed order.  x must be 8-byte aligned. */
+int    fgnn_edge_linear_tanh(int64_t E, int D, const float *x, const float *W, const float *b, float *y,
+                             void *stream);
+size_t fgnn_edge_linear_tanh_backward_workspace_bytes(int64_t E, int D);
+int    fgnn_edge_linear_tanh_backward(int64_t E, int D, const float *x, const float *y,
+                                      const float *grad_y, float *grad_W, float *grad_b,
+                                      void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---------------------------------------------------------------- csr2csc
  * Replaces csrtocsc.csr2csc (src/csr2csc/csr2csc.cc; csr2csc.cu:7-43, a cuSPARSE
  * cusparseCsr2cscEx2 call).  Stable: entries of a column keep ascending CSR position.

@@ -619,3 +619,42 @@ def test_gmm_layer_with_csc_ordered_pseudo(k, dim, f, monkeypatch):
         assert_close(layer.inv_sigma.grad, leaves[2].grad, "grad inv_sigma (two orders)", rtol=1e-3, atol=5e-2)
         assert_close(layer.fc.weight.grad, leaves[0].grad, "grad fc (two orders)", rtol=1e-3, atol=5e-2)
     _lib.clear_schedule_cache()
+
+
+@pytest.mark.parametrize("d", [1, 2, 3, 4])
+@pytest.mark.parametrize("e", [1, 257, 300001])
+def test_edge_linear_tanh_matches_torch(d, e):
+    """Linear(2, d) + Tanh over the edges (the MoNet drivers' pseudo projection): forward and the
+    parameter gradients against torch in float64; the gradient sums are reproducible run to run."""
+    from ae_mlsys_gnn_amd.operators import edge_proj
+    torch.manual_seed(d * 1000 + e)
+    x = torch.rand(e, 2, dtype=torch.float64) * 2 - 1
+    w = torch.randn(d, 2, dtype=torch.float64, requires_grad=True)
+    b = torch.randn(d, dtype=torch.float64, requires_grad=True)
+    go = torch.randn(e, d, dtype=torch.float64)
+    want = torch.tanh(torch.nn.functional.linear(x, w, b))
+    want.backward(go)
+    xd = x.float().to(DEV)
+    wd = w.detach().float().to(DEV).requires_grad_(True)
+    bd = b.detach().float().to(DEV).requires_grad_(True)
+    got = edge_proj.edge_linear_tanh(xd, wd, bd)
+    got.backward(go.float().to(DEV))
+    assert_close(got, want, "y", atol=2e-6)
+    # sums of e terms of either sign: the absolute bar scales with sqrt(e) summands of magnitude ~|go|
+    bar = 1e-5 * max(1.0, float(go.abs().max()) * e ** 0.5)
+    assert_close(wd.grad, w.grad, "grad_W", atol=bar)
+    assert_close(bd.grad, b.grad, "grad_b", atol=bar)
+    w2 = wd.detach().clone().requires_grad_(True)
+    b2 = bd.detach().clone().requires_grad_(True)
+    edge_proj.edge_linear_tanh(xd, w2, b2).backward(go.float().to(DEV))
+    assert torch.equal(w2.grad, wd.grad) and torch.equal(b2.grad, bd.grad)
+
+
+def test_edge_linear_tanh_limits():
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd.operators import edge_proj
+    with pytest.raises(ValueError):
+        edge_proj.edge_linear_tanh(torch.rand(5, 2, device=DEV), torch.rand(5, 2, device=DEV), torch.rand(5, device=DEV))
+    assert _lib.lib().fgnn_edge_linear_tanh(4, 5, None, None, None, None, None) == -4
+    y = edge_proj.edge_linear_tanh(torch.rand(0, 2, device=DEV), torch.rand(2, 2, device=DEV), torch.rand(2, device=DEV))
+    assert y.shape == (0, 2)

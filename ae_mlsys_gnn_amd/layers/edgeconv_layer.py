@@ -1,9 +1,11 @@
 """EdgeConv layer on the fused operator (interface of the reference's layers/edgeconv_layer.py:6-43)."""
 from __future__ import annotations
 
+import torch
 from torch import nn
 
 from ..operators.fused_edgeconv import fused_edgeconv_op
+from .dense import tall_linear
 
 
 class EdgeConv(nn.Module):
@@ -24,7 +26,11 @@ class EdgeConv(nn.Module):
 
     def forward(self, k, src_ind, feat, block=None):
         """block: points per cloud when src_ind is a kNN graph of equally sized clouds (see fused_edgeconv_op)."""
-        h_theta = self.theta(feat)
-        h_src = h_theta
-        h_dst = self.phi(feat) - h_theta
+        # theta and phi read the same rows: one product with the stacked weights (its weight gradient
+        # reduced over the points in chunks), split afterwards
+        out_feat = self.theta.out_features
+        h = tall_linear(feat, torch.cat([self.theta.weight, self.phi.weight], 0))
+        h_theta, h_phi = h[:, :out_feat], h[:, out_feat:]
+        h_src = h_theta.contiguous()
+        h_dst = h_phi - h_theta
         return fused_edgeconv_op(k, src_ind, h_src, h_dst, block)

@@ -9,6 +9,7 @@ import torch
 from torch import nn
 
 from ..operators.fused_gat import fused_gat_fusescatter, fused_gat_op, fused_gat_stash_op
+from .dense import reduce_over_rows
 
 
 class _GATBase(nn.Module):
@@ -40,22 +41,6 @@ class _GATBase(nn.Module):
         return out if out.shape[-1] == self.out_feats else out[..., :self.out_feats]
 
 
-def _reduce_over_nodes(x, g):
-    """x^T @ g for tall x [N, a], g [N, b] (a weight gradient: the reduction runs over the nodes).
-    As one GEMM the reduction length N lands on a few workgroups (4.6 ms for N = 2.4 M, a = 100,
-    b = 272); cut into chunks of rows it is a batched matmul over all of them plus a small sum (1.5 ms)."""
-    n = x.shape[0]
-    chunks = min(256, n // 4096)
-    if chunks < 2:
-        return torch.matmul(x.t(), g)
-    rows = n // chunks
-    body = chunks * rows
-    out = torch.bmm(x[:body].view(chunks, rows, -1).transpose(1, 2), g[:body].view(chunks, rows, -1)).sum(0)
-    if body < n:
-        out = out + torch.matmul(x[body:].t(), g[body:])
-    return out
-
-
 class _ProjectScores(torch.autograd.Function):
     """The dense part of the layer.  The scores are formed as feat @ ((W * attn).sum(-1)): the same
     sums taken in another order, as one thin GEMM over `feat` instead of two strided reductions over
@@ -84,7 +69,7 @@ class _ProjectScores(torch.autograd.Function):
         g = torch.cat([zeros(hfp) if dh is None else dh.reshape(n, hfp), zeros(hh) if drow is None else drow,
                        zeros(hh) if dcol is None else dcol], dim=1)                        # [N, H*Fp + 2H]
         dfeat = torch.matmul(g, w_all.t()) if ctx.needs_input_grad[0] else None
-        dw_ext = _reduce_over_nodes(feat, g)                                              # [in, H*Fp + 2H]
+        dw_ext = reduce_over_rows(feat, g)                                              # [in, H*Fp + 2H]
         dwl, dwr = dw_ext[:, hfp:hfp + hh].unsqueeze(-1), dw_ext[:, hfp + hh:].unsqueeze(-1)   # [in, H, 1]
         wv = W.view(W.shape[0], hh, ff)
         dW = dw_ext[:, :hfp].view(W.shape[0], hh, ff + ctx.pad)[:, :, :ff] + dwl * attn_l + dwr * attn_r

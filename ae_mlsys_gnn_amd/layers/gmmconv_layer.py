@@ -7,6 +7,7 @@ from torch import nn
 from torch.nn import init
 
 from ..operators.fused_gmmconv import GmmConvFuseSum, GmmConvFuseSumTwoOrders, GmmConvStash
+from .dense import tall_linear
 
 
 class _GMMBase(nn.Module):
@@ -52,7 +53,7 @@ class _GMMBase(nn.Module):
         """pseudo_csc (GMMConv only): the same pseudo-coordinates in CSC order, pseudo[permute], built by
         the caller from its own CSC-ordered edge data.  The backward then works in CSC order throughout
         and the gradient of the pseudo-coordinates flows through pseudo_csc instead of pseudo."""
-        node_feat = self.fc(feat).view(-1, self._n_kernels, self._out_feats)
+        node_feat = tall_linear(feat, self.fc.weight).view(-1, self._n_kernels, self._out_feats)    # = self.fc(feat)
         pad = (-self._out_feats) % 4
         if pad:         # zero columns up to a multiple of 4: the operator then takes its 128-bit row layout
             node_feat = th.nn.functional.pad(node_feat, (0, pad))

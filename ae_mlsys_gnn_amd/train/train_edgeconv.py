@@ -21,6 +21,7 @@ from torch import nn
 
 from .. import graphs
 from ..layers import EdgeConv
+from ..layers.dense import tall_linear
 from ..operators.knn import knn_graph
 from . import common, datasets
 
@@ -46,7 +47,7 @@ class Model(nn.Module):
             src = self.knn(h.detach(), self.k)
             h = F.leaky_relu(conv(self.k, src, h.reshape(b * p, -1), block=p), 0.2).view(b, p, -1)
             hs.append(h)
-        h = self.proj(torch.cat(hs, 2))
+        h = tall_linear(torch.cat(hs, 2).view(b * p, -1), self.proj.weight, self.proj.bias).view(b, p, -1)
         h = torch.cat([h.max(1).values, h.mean(1)], 1)
         for emb, bn, drop in zip(self.embs, self.bn_embs, self.dropouts):
             h = drop(F.leaky_relu(bn(emb(h)), 0.2))

@@ -227,3 +227,24 @@ def test_training_step_replays_from_a_hip_graph(model):
     # last bits and 16 optimizer steps amplify that; a wrong replay would be off by far more
     assert abs(eager["last_loss"] - graphed["last_loss"]) <= 5e-4 * abs(eager["last_loss"]), (eager, graphed)
     assert abs(eager["test_acc"] - graphed["test_acc"]) < 0.02
+
+
+def test_tall_linear_equals_linear():
+    """layers.dense: the chunked reduction over the rows gives the weight gradient of an ordinary Linear
+    (row counts that do and do not divide into the chunks, with and without bias / input gradient)."""
+    from ae_mlsys_gnn_amd.layers.dense import reduce_over_rows, tall_linear
+    torch.manual_seed(0)
+    for n, need_gx in ((100, True), (4096 + 17, True), (3 * 2048, False), (70001, True)):
+        x = torch.randn(n, 5, dtype=torch.float64, requires_grad=need_gx)
+        w = torch.randn(7, 5, dtype=torch.float64, requires_grad=True)
+        b = torch.randn(7, dtype=torch.float64, requires_grad=True)
+        go = torch.randn(n, 7, dtype=torch.float64)
+        for bias in (b, None):
+            want = torch.nn.functional.linear(x, w, bias)
+            got = tall_linear(x, w, bias)
+            assert torch.allclose(got, want, atol=1e-12)
+            leaves = [t for t in (x, w, bias) if t is not None and t.requires_grad]
+            gw = torch.autograd.grad((want * go).sum(), leaves)
+            gg = torch.autograd.grad((got * go).sum(), leaves)
+            assert all(torch.allclose(a, c, rtol=1e-10, atol=1e-10) for a, c in zip(gg, gw))
+        assert torch.allclose(reduce_over_rows(x.detach(), go), x.detach().t() @ go, rtol=1e-10, atol=1e-10)

@@ -254,3 +254,26 @@ def test_gat_random_shapes_and_graphs(seed):
     else:
         g = degree_edge_graph(seed=100 + seed)
     _run(g, h, f, slope=slope, seed=seed, variant=variant)
+
+
+@pytest.mark.parametrize("dense", [False, True])
+@pytest.mark.parametrize("h,f", [(8, 32), (1, 128), (3, 20)])
+def test_gat_without_schedules_and_reference_backward_signature(h, f, dense):
+    """The C ABI as a caller with only the reference's tensors uses it: no schedules (one wave per row
+    or column) and a backward that gets neither out nor the auxiliary outputs and recomputes them."""
+    from ae_mlsys_gnn_amd.operators.fused_gat import gat_native
+    g = graphs.add_csc_torch(degree_edge_graph(n=80, seed=31) if dense else graphs.rmat_graph(400, 5000, seed=31))
+    x, ar, ac, go = gat_inputs(g, h, f, 3)
+    ref = _oracle_fwd_bwd(g, x, ar, ac, go, 0.2)
+    dev = torch.device("cuda:0")
+    gd = g.to(dev)
+    xd, ard, acd, god = (t.float().to(dev) for t in (x, ar, ac, go))
+    out, emax, esum, _, _, _, _ = gat_native.gat_forward(ard, acd, gd.row_ptr, gd.col_ind, 0.2, xd, need_aux=False, use_schedule=False)
+    gx, gar, gac = gat_native.gat_backward(0.2, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, emax, esum, xd, ard, acd, god,
+                                           use_schedule=False)
+    torch.cuda.synchronize()
+    assert_close(out, ref[0], "out")
+    assert_close(gx, ref[1], "grad_feat")
+    scale = max(1.0, float(go.abs().max() * x.abs().max() * f))
+    assert_close(gar, ref[2], "grad_attn_row", atol=1e-5 * scale)
+    assert_close(gac, ref[3], "grad_attn_col", atol=1e-5 * scale)

@@ -467,6 +467,90 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_packed_kernel(GmmBwdP p)
     if (pm.ok && pm.grp == 0) T.store_nt(dst + pm.eoff);
 }
 
+// The column pass when grad_out is the gradient of the SUM over the mixture kernels ([N, F], the
+// GMMConv layers): the gathered row is the same for every kernel, so the lanes spread over F only
+// (LPF = lanes per row, a power of two >= F/4) and keep the K accumulators and the K slices of x[col]
+// in registers.  One load instruction then fetches 64/LPF different rows, every lane of it is used,
+// and a row is read once instead of once per mixture kernel.  K <= GMM_SUMK_MAX, F % 4 == 0, F <= 256.
+#define GMM_SUMK_MAX 4
+template <int LPF>
+__global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_sum_kernel(GmmBwdP p)
+{
+    extern __shared__ float lds[];
+    constexpr int G = 64 / LPF;         // rows per load instruction
+    constexpr int U = G > 8 ? 64 / G : 8;       // load instructions in flight; U * G divides 64
+    const int K = p.K, dim = p.dim, KD = K * dim, F = p.F;
+    const int per_wave = K * 64;
+    float *shared = lds + FGNN_WPB * per_wave;          // mu | inv_sigma
+    for (int i = (int)threadIdx.x; i < KD; i += FGNN_TPB) { shared[i] = p.mu[i]; shared[KD + i] = p.isg[i]; }
+    __syncthreads();
+    int col, b, e, slot;
+    if (!fg_get_item(p.items, p.n_items, p.ptr, col, b, e, slot)) return;
+    const int lane = fg_lane();
+    float *wl = lds + fg_wave() * per_wave;
+    const int grp = lane / LPF, sub = lane % LPF;
+    const bool fok = sub * 4 < F;
+    const int foff = fok ? sub * 4 : 0;
+    fg_vec<4> T[GMM_SUMK_MAX], xr[GMM_SUMK_MAX];
+#pragma unroll
+    for (int k = 0; k < GMM_SUMK_MAX; ++k) {
+        T[k].zero();
+        if (k < K && fok) xr[k].load(p.x + (size_t)col * p.HF + k * F + foff); else xr[k].zero();
+    }
+    for (int c = b; c < e; c += 64) {
+        int q = c + lane;
+        bool ok = q < e;
+        int cnt = min(64, e - c);
+        int qq = ok ? q : c;
+        int id = p.idx[qq];
+        int posv = p.pos ? p.pos[qq] : qq;
+        if (p.permute) posv = p.permute[posv];      // NULL: pseudo and gww are in this pass's own (CSC) order
+        const float *ps = p.pseudo + (size_t)(unsigned)posv * dim;
+        float pv[GMM_PV];
+        gmm_load_pseudo(ps, dim, pv);
+        for (int k = 0; k < K; ++k) wl[k * 64 + lane] = ok ? gmm_weight(pv, ps, shared + k * dim, shared + KD + k * dim, dim) : 0.f;
+        fg_wave_lds_sync();
+        for (int t = 0; t < cnt; t += U * G) {
+            fg_vec<4> ld[U];
+            int pe[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u * G + grp;                     // < 64: U*G divides 64
+                const int rid = __builtin_amdgcn_ds_bpermute(ei << 2, id);
+                pe[u] = __builtin_amdgcn_ds_bpermute(ei << 2, posv);
+                if (ei < cnt && fok) ld[u].load(p.g + (size_t)rid * F + foff); else ld[u].zero();
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u * G + grp;
+                float *gdst = p.gww + (size_t)(unsigned)pe[u] * K;
+                float mine = 0.f;                                   // lane `sub` of a row keeps the value of kernel `sub`
+#pragma unroll
+                for (int k = 0; k < GMM_SUMK_MAX; ++k) {
+                    if (k < K) {
+                        const float w = wl[k * 64 + ei];            // 0 past the end of the chunk
+                        T[k].fma(w, ld[u]);
+                        const float sum = fg_group_sum<LPF>(ld[u].dot(xr[k]));
+                        if constexpr (LPF >= GMM_SUMK_MAX) mine = sub == k ? sum * w : mine;
+                        else if (ei < cnt && sub == 0) gdst[k] = sum * w;
+                    }
+                }
+                // the K values of an edge leave with one store instruction, K adjacent lanes writing K adjacent floats
+                if constexpr (LPF >= GMM_SUMK_MAX) { if (ei < cnt && sub < K) gdst[sub] = mine; }
+            }
+        }
+        fg_wave_lds_sync();
+    }
+    float *dst = slot < 0 ? p.gfeat + (size_t)col * p.HF : p.part + (size_t)slot * spmm_pw(p.HF);
+#pragma unroll
+    for (int k = 0; k < GMM_SUMK_MAX; ++k) {
+        if (k < K) {
+            fg_pack_reduce<G>(T[k], lane);
+            if (fok && grp == 0) T[k].store_nt(dst + k * F + foff);
+        }
+    }
+}
+
 // Closed-form derivatives of w[p,k] = exp(-0.5 sum_d ((pseudo[p,d]-mu[k,d])*isg[k,d])^2), one edge per
 // thread.  src[p,k] is either dL/dw (premultiplied == 0: the weight is recomputed here) or dL/dw * w.
 //   d/dpseudo[p,d] = -sum_k gww*diff*isg^2,  d/dmu[k,d] = sum_p gww*diff*isg^2,  d/disg[k,d] = -sum_p gww*diff^2*isg
@@ -639,7 +723,38 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
         }
         const int lph = p.lphp ? p.lphp : fgnn_pick_lph(cfg.vec, F);
         const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
-        rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
+        const bool sumk = sum_kernels && cfg.vec == 4 && F % 4 == 0 && F <= 256 && K <= GMM_SUMK_MAX;
+        rc = sumk ? 0 : 1;
+        if (sumk) {
+            // lanes over F only, the K mixture kernels in registers (see gmm_bwd_sum_kernel)
+            int lpf = 1;
+            while (lpf * 4 < F) lpf *= 2;
+            const size_t shm = ((size_t)FGNN_WPB * K * 64 + 2 * KD) * sizeof(float);
+            FGNN_REQUIRE(shm <= 64 * 1024, FGNN_ERR_LIMIT, "fgnn_gmm_backward: K=%d, dim=%d need %zu bytes of LDS per workgroup (limit 64 KiB)", K, dim, shm);
+            p.lphp = 0;
+            switch (lpf) {
+            case 1: hipLaunchKernelGGL(gmm_bwd_sum_kernel<1>, dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
+            case 2: hipLaunchKernelGGL(gmm_bwd_sum_kernel<2>, dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
+            case 4: hipLaunchKernelGGL(gmm_bwd_sum_kernel<4>, dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
+            case 8: hipLaunchKernelGGL(gmm_bwd_sum_kernel<8>, dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
+            case 16: hipLaunchKernelGGL(gmm_bwd_sum_kernel<16>, dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
+            case 32: hipLaunchKernelGGL(gmm_bwd_sum_kernel<32>, dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
+            default: hipLaunchKernelGGL(gmm_bwd_sum_kernel<64>, dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
+            }
+            rc = fgnn_launch_status("gmm_bwd_sum_kernel");
+            if (rc) return rc;
+            if (sched_csc->n_split > 0) {
+                SpmmP mp{};
+                mp.part = part; mp.out = grad_feat; mp.N = N; mp.H = K; mp.F = F; mp.HF = HF;
+                unsigned g2 = (unsigned)((sched_csc->n_split + FGNN_WPB - 1) / FGNN_WPB);
+                rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
+                    hipLaunchKernelGGL((spmm_merge_kernel<VEC, R>), dim3(g2), dim3(FGNN_TPB), 0, st, mp, sched_csc->split_dev, sched_csc->n_split);
+                    return fgnn_launch_status("spmm_merge_kernel");
+                });
+                if (rc) return rc;
+            }
+        }
+        if (!sumk) rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
             size_t shm = ((size_t)FGNN_WPB * (K * 64 + 64 * R) + 2 * KD) * sizeof(float);
             FGNN_REQUIRE(shm <= 64 * 1024, FGNN_ERR_LIMIT, "fgnn_gmm_backward: K=%d, dim=%d need %zu bytes of LDS per workgroup (limit 64 KiB)", K, dim, shm);
             const int pack = lph > 0 ? fgnn_pick_pack(cfg.vec, lanes_hf) : 1;

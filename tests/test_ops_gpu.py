@@ -139,7 +139,10 @@ def _gmm_case(g, k, dim, f, seed):
                                               (3, 1, 4, "fuse"),
                                               # quarter of the width not a power of two: head-aligned lane map
                                               (2, 1, 44, "fuse"), (3, 2, 12, "sum"), (2, 2, 20, "stash"), (5, 1, 48, "fuse"), (4, 2, 100, "fuse"),
-                                              (9, 1, 12, "fuse")])
+                                              (9, 1, 12, "fuse"),
+                                              # summed kernels: lanes over F only, 1 to 64 rows per load instruction
+                                              (3, 2, 4, "sum"), (4, 1, 8, "sum"), (2, 2, 256, "sum"), (4, 2, 128, "sum"), (1, 2, 44, "sum"),
+                                              (3, 1, 100, "sum"), (2, 1, 252, "sum"), (4, 3, 32, "sum")])
 def test_gmm_forward_backward(k, dim, f, variant, monkeypatch):
     from ae_mlsys_gnn_amd.operators import fused_gmmconv as fg
     from ae_mlsys_gnn_amd import _lib

@@ -179,7 +179,7 @@ __global__ __launch_bounds__(256) void csc_row_hint_kernel(int64_t n, int n_rows
     hint[k] = csc_row_of(row_ptr, 0, n_rows, (int)p);
 }
 
-__global__ __launch_bounds__(256) void csc_finalize_kernel(int64_t n, int n_rows, int n_cols, const int *__restrict__ sorted_keys,
+__global__ __launch_bounds__(256) void csc_finalize_kernel(int64_t n, int n_cols, const int *__restrict__ sorted_keys,
                                                            const int *__restrict__ permute, const int *__restrict__ row_ptr,
                                                            const int *__restrict__ hint, int *__restrict__ col_ptr, int *__restrict__ row_ind)
 {
@@ -288,7 +288,7 @@ extern "C" int fgnn_csr2csc(int n_rows, int n_cols, int64_t E, const int32_t *ro
     hipLaunchKernelGGL(csc_row_hint_kernel, dim3((unsigned)((n_hint + 255) / 256)), dim3(256), 0, st, E, n_rows, n_hint, row_ptr, hint);
     rc = fgnn_launch_status("csc_row_hint_kernel");
     if (rc) return rc;
-    hipLaunchKernelGGL(csc_finalize_kernel, dim3((unsigned)((E + 255) / 256)), dim3(256), 0, st, E, n_rows, n_cols, sorted, permute, row_ptr, hint, col_ptr, row_ind);
+    hipLaunchKernelGGL(csc_finalize_kernel, dim3((unsigned)((E + 255) / 256)), dim3(256), 0, st, E, n_cols, sorted, permute, row_ptr, hint, col_ptr, row_ind);
     return fgnn_launch_status("csc_finalize_kernel");
 }
 
@@ -394,7 +394,7 @@ __global__ __launch_bounds__(256) void coo_compact_kernel(int64_t n, const int *
 }
 
 // row_ptr from the compacted destinations (ascending); *n_out entries are valid.
-__global__ __launch_bounds__(256) void coo_rowptr_kernel(int64_t n, int n_rows, const int *__restrict__ dstc, const int *__restrict__ n_out_dev,
+__global__ __launch_bounds__(256) void coo_rowptr_kernel(int n_rows, const int *__restrict__ dstc, const int *__restrict__ n_out_dev,
                                                          int *__restrict__ row_ptr, int64_t *__restrict__ n_out)
 {
     int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -474,6 +474,6 @@ extern "C" int fgnn_coo2csr(int n_rows, int n_cols, int64_t E, const int32_t *ds
     hipLaunchKernelGGL(coo_compact_kernel, dim3(ge), dim3(256), 0, st, E, dsts, tmp, perm2, flag, incl, col_ind, dstc, edge_pos);
     rc = fgnn_launch_status("coo_compact_kernel");
     if (rc) return rc;
-    hipLaunchKernelGGL(coo_rowptr_kernel, dim3(ge), dim3(256), 0, st, E, n_rows, dstc, total, row_ptr, n_out);
+    hipLaunchKernelGGL(coo_rowptr_kernel, dim3(ge), dim3(256), 0, st, n_rows, dstc, total, row_ptr, n_out);
     return fgnn_launch_status("coo_rowptr_kernel");
 }

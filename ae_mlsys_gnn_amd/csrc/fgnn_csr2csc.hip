@@ -1,8 +1,8 @@
 // GPU CSR -> CSC transpose (stable), replacing the reference's cuSPARSE call
 // (src/csr2csc/csr2csc.cu:10-23).
 //
-// The transpose is a stable sort of the CSR positions by column: an LSD radix sort with 8-bit
-// digits over key = col_ind[p], payload = p.  Each pass is histogram -> scan -> stable scatter:
+// The transpose is a stable sort of the CSR positions by column: an LSD radix sort with digits of
+// up to 8 bits over key = col_ind[p], payload = p.  Each pass is histogram -> scan -> stable scatter:
 // a workgroup owns a contiguous tile, each of its 4 waves a contiguous quarter of it, and a wave
 // walks its quarter 64 elements at a time, ranking equal digits inside the wave with ballots, so
 // equal keys keep their order (the order of CSR positions).  After the last pass the payload IS
@@ -15,54 +15,62 @@
 #define RS_TILE (RS_TPB * RS_ITEMS)    // 4096 elements per workgroup
 #define RS_SUB (64 * RS_ITEMS)         // 1024 per wave
 
-__global__ __launch_bounds__(RS_TPB) void rs_hist_kernel(const int *__restrict__ keys, int64_t n, int shift, int nblocks, int *__restrict__ hist)
+__global__ __launch_bounds__(RS_TPB) void rs_hist_kernel(const int *__restrict__ keys, int64_t n, int shift, int mask, int nblocks, int *__restrict__ hist)
 {
-    __shared__ int cnt[256];
-    cnt[threadIdx.x] = 0;
+    __shared__ int cnt[4][256];         // one set of counters per wave: a quarter of the collisions
+    for (int i = (int)threadIdx.x; i < 4 * 256; i += RS_TPB) (&cnt[0][0])[i] = 0;
     __syncthreads();
     const int wave = fg_wave(), lane = fg_lane();
 #pragma unroll 4
     for (int it = 0; it < RS_ITEMS; ++it) {
         int64_t i = (int64_t)blockIdx.x * RS_TILE + wave * RS_SUB + it * 64 + lane;
-        if (i < n) atomicAdd(&cnt[(keys[i] >> shift) & 255], 1);
+        if (i < n) atomicAdd(&cnt[wave][(keys[i] >> shift) & mask], 1);
     }
     __syncthreads();
-    hist[(size_t)threadIdx.x * nblocks + blockIdx.x] = cnt[threadIdx.x];
+    if ((int)threadIdx.x <= mask)
+        hist[(size_t)threadIdx.x * nblocks + blockIdx.x] = (cnt[0][threadIdx.x] + cnt[1][threadIdx.x]) + (cnt[2][threadIdx.x] + cnt[3][threadIdx.x]);
 }
 
-// One workgroup per digit: exclusive scan of that digit's per-block counts in place.
+// One workgroup per digit: exclusive scan of that digit's per-block counts in place.  The row is walked
+// in chunks of RS_TPB * 8 counts: every thread scans 8 consecutive counts serially, the 256 thread totals
+// are scanned with wave shuffles and one exchange through LDS, and the chunk's total carries over.
 __global__ __launch_bounds__(RS_TPB) void rs_scan_kernel(int *__restrict__ hist, int nblocks, int *__restrict__ digit_total)
 {
-    __shared__ int sh[RS_TPB];
-    __shared__ int carry;
+    constexpr int PER = 8;
+    __shared__ int wave_tot[4];
     int *row = hist + (size_t)blockIdx.x * nblocks;
-    if (threadIdx.x == 0) carry = 0;
-    __syncthreads();
-    for (int base = 0; base < nblocks; base += RS_TPB) {
-        int i = base + (int)threadIdx.x;
-        int v = i < nblocks ? row[i] : 0;
-        sh[threadIdx.x] = v;
-        __syncthreads();
-        for (int off = 1; off < RS_TPB; off <<= 1) {
-            int t = (int)threadIdx.x >= off ? sh[threadIdx.x - off] : 0;
-            __syncthreads();
-            sh[threadIdx.x] += t;
-            __syncthreads();
+    const int lane = fg_lane(), wave = fg_wave();
+    int carry = 0;
+    for (int base = 0; base < nblocks; base += RS_TPB * PER) {
+        const int i0 = base + (int)threadIdx.x * PER;
+        int v[PER], tot = 0;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) { v[j] = i0 + j < nblocks ? row[i0 + j] : 0; tot += v[j]; }
+        int incl = tot;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            int t = __shfl_up(incl, off);
+            if (lane >= off) incl += t;
         }
-        int incl = sh[threadIdx.x];
-        int c = carry;
-        if (i < nblocks) row[i] = c + incl - v;
+        __syncthreads();                        // the previous chunk's wave totals have been read
+        if (lane == 63) wave_tot[wave] = incl;
         __syncthreads();
-        if (threadIdx.x == RS_TPB - 1) carry = c + incl;
-        __syncthreads();
+        int run = carry + incl - tot;
+        for (int w = 0; w < wave; ++w) run += wave_tot[w];
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            if (i0 + j < nblocks) row[i0 + j] = run;
+            run += v[j];
+        }
+        carry += wave_tot[0] + wave_tot[1] + wave_tot[2] + wave_tot[3];
     }
     if (threadIdx.x == 0) digit_total[blockIdx.x] = carry;
 }
 
-__global__ __launch_bounds__(256) void rs_digit_base_kernel(const int *__restrict__ digit_total, int *__restrict__ digit_base)
+__global__ __launch_bounds__(256) void rs_digit_base_kernel(const int *__restrict__ digit_total, int n_digits, int *__restrict__ digit_base)
 {
     __shared__ int sh[256];
-    int v = digit_total[threadIdx.x];
+    int v = (int)threadIdx.x < n_digits ? digit_total[threadIdx.x] : 0;
     sh[threadIdx.x] = v;
     __syncthreads();
     for (int off = 1; off < 256; off <<= 1) {
@@ -80,7 +88,7 @@ __global__ __launch_bounds__(256) void rs_digit_base_kernel(const int *__restric
 // elements of a digit leave as one contiguous run, so neighbouring lanes write neighbouring addresses
 // instead of 4-byte stores scattered over 256 destinations.
 __global__ __launch_bounds__(RS_TPB) void rs_scatter_kernel(const int *__restrict__ keys_in, const int *__restrict__ pay_in, int64_t n, int shift,
-                                                            int nblocks, const int *__restrict__ hist, const int *__restrict__ digit_base,
+                                                            int bits, int nblocks, const int *__restrict__ hist, const int *__restrict__ digit_base,
                                                             int *__restrict__ keys_out, int *__restrict__ pay_out)
 {
     __shared__ int wcnt[4][256];        // per wave and digit: count, then the running local position
@@ -88,15 +96,17 @@ __global__ __launch_bounds__(RS_TPB) void rs_scatter_kernel(const int *__restric
     __shared__ int wave_tot[4];
     __shared__ int skey[RS_TILE], spay[RS_TILE];
     const int wave = fg_wave(), lane = fg_lane();
+    const int mask = (1 << bits) - 1;
     for (int i = (int)threadIdx.x; i < 4 * 256; i += RS_TPB) (&wcnt[0][0])[i] = 0;
     __syncthreads();
     const int64_t tile0 = (int64_t)blockIdx.x * RS_TILE;
-    int key[RS_ITEMS];
+    int key[RS_ITEMS], pay[RS_ITEMS];
 #pragma unroll
     for (int it = 0; it < RS_ITEMS; ++it) {
         int64_t i = tile0 + wave * RS_SUB + it * 64 + lane;
         key[it] = i < n ? keys_in[i] : 0;
-        if (i < n) atomicAdd(&wcnt[wave][(key[it] >> shift) & 255], 1);
+        pay[it] = (pay_in && i < n) ? pay_in[i] : (int)i;      // fetched up front: the ranking loop below is a dependent chain
+        if (i < n) atomicAdd(&wcnt[wave][(key[it] >> shift) & mask], 1);
     }
     __syncthreads();
     {
@@ -116,7 +126,7 @@ __global__ __launch_bounds__(RS_TPB) void rs_scatter_kernel(const int *__restric
         __syncthreads();
         int lbase = incl - tot;
         for (int w = 0; w < wave; ++w) lbase += wave_tot[w];
-        gofs[d] = digit_base[d] + hist[(size_t)d * nblocks + blockIdx.x] - lbase;
+        gofs[d] = d <= mask ? digit_base[d] + hist[(size_t)d * nblocks + blockIdx.x] - lbase : 0;
         int run = lbase;
 #pragma unroll
         for (int w = 0; w < 4; ++w) { wcnt[w][d] = run; run += c[w]; }
@@ -127,18 +137,20 @@ __global__ __launch_bounds__(RS_TPB) void rs_scatter_kernel(const int *__restric
     for (int it = 0; it < RS_ITEMS; ++it) {
         int64_t i = tile0 + wave * RS_SUB + it * 64 + lane;
         bool ok = i < n;
-        int d = (key[it] >> shift) & 255;
+        int d = (key[it] >> shift) & mask;
         unsigned long long peers = __builtin_amdgcn_ballot_w64(ok);
 #pragma unroll
         for (int bit = 0; bit < 8; ++bit) {
-            unsigned long long bal = __builtin_amdgcn_ballot_w64(((d >> bit) & 1) != 0);
-            peers &= ((d >> bit) & 1) ? bal : ~bal;
+            if (bit < bits) {
+                unsigned long long bal = __builtin_amdgcn_ballot_w64(((d >> bit) & 1) != 0);
+                peers &= ((d >> bit) & 1) ? bal : ~bal;
+            }
         }
         int rank = __popcll(peers & lt);
         int base = wcnt[wave][d];
         if (ok) {
             skey[base + rank] = key[it];
-            spay[base + rank] = pay_in ? pay_in[i] : (int)i;
+            spay[base + rank] = pay[it];
         }
         fg_wave_lds_sync();
         // the highest lane of every peer group advances the wave's counter of that digit
@@ -150,7 +162,7 @@ __global__ __launch_bounds__(RS_TPB) void rs_scatter_kernel(const int *__restric
 #pragma unroll 4
     for (int i = (int)threadIdx.x; i < count; i += RS_TPB) {
         int k = skey[i];
-        int dst = gofs[(k >> shift) & 255] + i;
+        int dst = gofs[(k >> shift) & mask] + i;
         keys_out[dst] = k;
         pay_out[dst] = spay[i];
     }
@@ -201,11 +213,12 @@ __global__ __launch_bounds__(256) void fill_i32_kernel(int *p, size_t n, int v)
     if (i < n) p[i] = v;
 }
 
-static int rs_num_passes(int n_cols)
+// Key bits to sort for ids below n_cols.
+static int rs_key_bits(int n_cols)
 {
     int bits = 1;
     while (bits < 31 && (1LL << bits) < (long long)n_cols) ++bits;
-    return (bits + 7) / 8;
+    return bits;
 }
 
 // Scratch of one radix sort of n (key, payload) pairs: two key buffers, one payload buffer,
@@ -216,12 +229,15 @@ static size_t rs_sort_workspace(int64_t n)
     return 3 * fgnn_align256((size_t)n * sizeof(int)) + fgnn_align256(256 * nblocks * sizeof(int)) + 2 * fgnn_align256(256 * sizeof(int));
 }
 
-// Stable LSD radix sort of n pairs by the low 8*passes key bits.  keys_in is not modified; pay_in ==
-// NULL sorts the element indices.  The sorted payload lands in pay_out; *sorted_keys points at the
-// sorted keys (inside the workspace).
-static int rs_sort_pairs(const int *keys_in, const int *pay_in, int64_t n, int passes, int *pay_out, const int **sorted_keys, void *workspace,
+// Stable LSD radix sort of n pairs by the low `key_bits` key bits, in ceil(key_bits / 8) passes of equal
+// digit width (18 bits: 6 + 6 + 6 rather than 8 + 8 + 2 -- fewer digits mean longer contiguous runs per
+// tile in the scatter).  keys_in is not modified; pay_in == NULL sorts the element indices.  The sorted
+// payload lands in pay_out; *sorted_keys points at the sorted keys (inside the workspace).
+static int rs_sort_pairs(const int *keys_in, const int *pay_in, int64_t n, int key_bits, int *pay_out, const int **sorted_keys, void *workspace,
                          hipStream_t st)
 {
+    const int passes = (key_bits + 7) / 8;
+    const int bits = (key_bits + passes - 1) / passes;      // digit width of every pass, <= 8
     const int nblocks = (int)((n + RS_TILE - 1) / RS_TILE);
     char *w = (char *)workspace;
     int *keys[2];
@@ -236,19 +252,19 @@ static int rs_sort_pairs(const int *keys_in, const int *pay_in, int64_t n, int p
     const int *kin = keys_in;
     const int *pin = pay_in;
     for (int i = 0; i < passes; ++i) {
-        int shift = 8 * i;
+        int shift = bits * i;
         int *kout = keys[i & 1];
         int *pout = pay[(passes - 1 - i) & 1];      // the last pass lands in pay_out
-        hipLaunchKernelGGL(rs_hist_kernel, dim3(nblocks), dim3(RS_TPB), 0, st, kin, n, shift, nblocks, hist);
+        hipLaunchKernelGGL(rs_hist_kernel, dim3(nblocks), dim3(RS_TPB), 0, st, kin, n, shift, (1 << bits) - 1, nblocks, hist);
         int rc = fgnn_launch_status("rs_hist_kernel");
         if (rc) return rc;
-        hipLaunchKernelGGL(rs_scan_kernel, dim3(256), dim3(RS_TPB), 0, st, hist, nblocks, digit_total);
+        hipLaunchKernelGGL(rs_scan_kernel, dim3(1 << bits), dim3(RS_TPB), 0, st, hist, nblocks, digit_total);
         rc = fgnn_launch_status("rs_scan_kernel");
         if (rc) return rc;
-        hipLaunchKernelGGL(rs_digit_base_kernel, dim3(1), dim3(256), 0, st, digit_total, digit_base);
+        hipLaunchKernelGGL(rs_digit_base_kernel, dim3(1), dim3(256), 0, st, digit_total, 1 << bits, digit_base);
         rc = fgnn_launch_status("rs_digit_base_kernel");
         if (rc) return rc;
-        hipLaunchKernelGGL(rs_scatter_kernel, dim3(nblocks), dim3(RS_TPB), 0, st, kin, pin, n, shift, nblocks, hist, digit_base, kout, pout);
+        hipLaunchKernelGGL(rs_scatter_kernel, dim3(nblocks), dim3(RS_TPB), 0, st, kin, pin, n, shift, bits, nblocks, hist, digit_base, kout, pout);
         rc = fgnn_launch_status("rs_scatter_kernel");
         if (rc) return rc;
         kin = kout;
@@ -281,7 +297,7 @@ extern "C" int fgnn_csr2csc(int n_rows, int n_cols, int64_t E, const int32_t *ro
     size_t need = fgnn_csr2csc_workspace_bytes(n_rows, n_cols, E);
     FGNN_REQUIRE(workspace && workspace_bytes >= need, FGNN_ERR_WORKSPACE, "fgnn_csr2csc: workspace %zu < %zu bytes", workspace_bytes, need);
     const int *sorted = nullptr;
-    int rc = rs_sort_pairs(col_ind, nullptr, E, rs_num_passes(n_cols), permute, &sorted, workspace, st);
+    int rc = rs_sort_pairs(col_ind, nullptr, E, rs_key_bits(n_cols), permute, &sorted, workspace, st);
     if (rc) return rc;
     int *hint = (int *)((char *)workspace + rs_sort_workspace(E));
     const int n_hint = csc_num_hints(E);
@@ -448,13 +464,13 @@ extern "C" int fgnn_coo2csr(int n_rows, int n_cols, int64_t E, const int32_t *ds
     const unsigned ge = (unsigned)((E + 255) / 256);
 
     const int *sorted = nullptr;
-    int rc = rs_sort_pairs(src, nullptr, E, rs_num_passes(n_cols), perm1, &sorted, sort_ws, st);
+    int rc = rs_sort_pairs(src, nullptr, E, rs_key_bits(n_cols), perm1, &sorted, sort_ws, st);
     if (rc) return rc;
     hipLaunchKernelGGL(gather_i32_kernel, dim3(ge), dim3(256), 0, st, E, perm1, dst, tmp);
     rc = fgnn_launch_status("gather_i32_kernel");
     if (rc) return rc;
     const int *dsts = nullptr;
-    rc = rs_sort_pairs(tmp, perm1, E, rs_num_passes(n_rows), perm2, &dsts, sort_ws, st);
+    rc = rs_sort_pairs(tmp, perm1, E, rs_key_bits(n_rows), perm2, &dsts, sort_ws, st);
     if (rc) return rc;
     hipLaunchKernelGGL(gather_i32_kernel, dim3(ge), dim3(256), 0, st, E, perm2, src, tmp);       // sources in (dst, src) order
     rc = fgnn_launch_status("gather_i32_kernel");

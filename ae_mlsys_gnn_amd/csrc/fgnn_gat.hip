@@ -531,8 +531,8 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_edge_stash_kernel(int N, int64_t
         if (k < k1) {
             const size_t rh = (size_t)row * H + h;
             const float ev = fg_lrelu(ar[rh] + ac[(size_t)idx[q] * H + h], slope);
-            __builtin_nontemporal_store(ev, e_lrelu + k);
-            __builtin_nontemporal_store(__expf(ev - emax[rh]) / esum[rh], e_softmax + k);
+            if (e_lrelu) __builtin_nontemporal_store(ev, e_lrelu + k);
+            __builtin_nontemporal_store(__builtin_amdgcn_exp2f((ev - emax[rh]) * FGNN_LOG2E) * __builtin_amdgcn_rcpf(esum[rh]), e_softmax + k);
         }
         rem += 64u;
         const unsigned adv = rem / uh;
@@ -1060,7 +1060,7 @@ static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_
         return 0;
     });
     if (rc) return rc;
-    if (e_lrelu && E > 0) {
+    if (e_softmax && E > 0) {
         const int64_t waves = (E * H + 64 * GAT_STASH_CHUNKS - 1) / (64 * GAT_STASH_CHUNKS);
         hipLaunchKernelGGL(gat_edge_stash_kernel, dim3((unsigned)((waves + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, st, N, E, H, row_ptr,
                            col_ind, attn_row, attn_col, edge_max, edge_sum, slope, e_lrelu, e_softmax);
@@ -1080,7 +1080,7 @@ extern "C" int fgnn_gat_forward(int N, int64_t E, int H, int F, const float *att
     FGNN_REQUIRE(attn_row && attn_col && row_ptr && in_feat && out && edge_max && edge_sum && (col_ind || E == 0),
                  FGNN_ERR_NULL, "fgnn_gat_forward: NULL argument");
     FGNN_REQUIRE((aux_out2 == nullptr) == (aux_c == nullptr), FGNN_ERR_NULL, "fgnn_gat_forward: aux_out2 and aux_c go together");
-    FGNN_REQUIRE((e_lrelu == nullptr) == (e_softmax == nullptr), FGNN_ERR_NULL, "fgnn_gat_forward: e_lrelu and e_softmax go together");
+    FGNN_REQUIRE(e_lrelu == nullptr || e_softmax != nullptr, FGNN_ERR_NULL, "fgnn_gat_forward: e_lrelu is only written together with e_softmax");
     rc = check_sched(sched, row_ptr, col_ind, N, E, "fgnn_gat_forward");
     if (rc) return rc;
     return gat_forward_launch(N, E, H, F, attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, out, edge_max,

@@ -22,7 +22,7 @@ class gat_native:
 
     @staticmethod
     def gat_forward(attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, *, need_aux=True, stash=False,
-                    use_schedule=True):
+                    stash_lrelu=True, use_schedule=True):
         require_cuda(attn_row, attn_col, row_ptr, col_ind, in_feat)
         attn_row, attn_col, in_feat = as_f32(attn_row), as_f32(attn_col), as_f32(in_feat)
         row_ptr, col_ind = as_i32(row_ptr), as_i32(col_ind)
@@ -39,7 +39,7 @@ class gat_native:
         edge_sum = torch.empty((n, h), dtype=torch.float32, device=dev)
         out2 = torch.empty_like(in_feat) if need_aux else None
         cc = torch.empty((n, h), dtype=torch.float32, device=dev) if need_aux else None
-        e_lrelu = torch.empty((e, h), dtype=torch.float32, device=dev) if stash else None
+        e_lrelu = torch.empty((e, h), dtype=torch.float32, device=dev) if (stash and stash_lrelu) else None
         e_soft = torch.empty((e, h), dtype=torch.float32, device=dev) if stash else None
         sched = schedule_for(row_ptr, idx_tensor=col_ind, need_positions=False) if use_schedule else None
         sh = sched.handle if sched is not None else None
@@ -121,24 +121,27 @@ class FusedGATFunction_SM(torch.autograd.Function):
 
 
 class FusedGATFunction_stash(torch.autograd.Function):
-    """Stash variant: the forward also writes edge LeakyReLU / softmax [E,H]; the backward reads them."""
+    """Stash variant: the forward also writes the edge softmax [E,H] and the backward reads it instead
+    of recomputing.  (The reference stashes the edge LeakyReLU values too, fused_gat_stash.cu:420-442;
+    the backward here takes the one thing it needs from them, the sign of the pre-activation, from
+    attn_row + attn_col, so they are not written: half the stash.)"""
 
     @staticmethod
     def forward(ctx, attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute):
-        out, edge_max, edge_sum, out2, cc, e_lrelu, e_soft = gat_native.gat_forward(
-            attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, need_aux=True, stash=True)
-        ctx.save_for_backward(row_ptr, col_ind, col_ptr, row_ind, permute, e_soft, e_lrelu, in_feat, attn_row, attn_col,
+        out, edge_max, edge_sum, out2, cc, _, e_soft = gat_native.gat_forward(
+            attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, need_aux=True, stash=True, stash_lrelu=False)
+        ctx.save_for_backward(row_ptr, col_ind, col_ptr, row_ind, permute, e_soft, in_feat, attn_row, attn_col,
                               edge_max, edge_sum, out, out2, cc)
         ctx.negative_slope = negative_slope
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
-        (row_ptr, col_ind, col_ptr, row_ind, permute, e_soft, e_lrelu, in_feat, attn_row, attn_col,
+        (row_ptr, col_ind, col_ptr, row_ind, permute, e_soft, in_feat, attn_row, attn_col,
          edge_max, edge_sum, out, out2, cc) = ctx.saved_tensors
         grad_feat, grad_attn_row, grad_attn_col = gat_native.gat_backward(
             ctx.negative_slope, row_ptr, col_ind, col_ptr, row_ind, edge_max, edge_sum, in_feat, attn_row, attn_col,
-            grad_out.contiguous(), out_feat=out, out2=out2, cc=cc, permute=as_i32(permute), e_lrelu=e_lrelu, e_soft=e_soft)
+            grad_out.contiguous(), out_feat=out, out2=out2, cc=cc, permute=as_i32(permute), e_soft=e_soft)
         return grad_attn_row, grad_attn_col, None, None, None, None, None, grad_feat, None
 
 

@@ -72,7 +72,8 @@ int64_t fgnn_schedule_num_edges(const fgnn_schedule_t *s);
  * Outputs: out [N,H,F], edge_max, edge_sum [N,H].  Optional (NULL to skip):
  *   aux_out2 [N,H,F], aux_c [N,H]  -- sum_p alpha*lrelu'(e) * in_feat and sum_p alpha*lrelu'(e);
  *                                     they let the backward run in a single gather pass
- *   e_lrelu, e_softmax [E,H]       -- the stashed per-edge tensors of the stash variants
+ *   e_lrelu, e_softmax [E,H]       -- the stashed per-edge tensors of the stash variants; e_lrelu may be
+ *                                     NULL alone (fgnn_gat_backward does not read it)
  * Workspace: fgnn_gat_forward_workspace_bytes(sched, H, F) bytes (0 when sched is NULL). */
 size_t fgnn_gat_forward_workspace_bytes(const fgnn_schedule_t *sched, int H, int F);
 int    fgnn_gat_forward(int N, int64_t E, int H, int F,

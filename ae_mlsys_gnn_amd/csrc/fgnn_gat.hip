@@ -504,6 +504,7 @@ __device__ __forceinline__ int gat_row_of(const int *__restrict__ ptr, int lo, i
     return lo;
 }
 #define GAT_STASH_CHUNKS 32     // 64-element chunks per wave: the two wave-wide bisections are paid once per 2048 elements
+#define GAT_STASH_UJ 4          // chunks in flight; divides GAT_STASH_CHUNKS
 __global__ __launch_bounds__(FGNN_TPB) void gat_edge_stash_kernel(int N, int64_t E, int H, const int *__restrict__ ptr,
                                                                   const int *__restrict__ idx, const float *__restrict__ ar,
                                                                   const float *__restrict__ ac, const float *__restrict__ emax,
@@ -516,29 +517,50 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_edge_stash_kernel(int N, int64_t
     const int64_t k1 = min(k0 + 64 * GAT_STASH_CHUNKS, total);
     const int lane = fg_lane();
     const unsigned uh = (unsigned)H;
+    const unsigned inv_h = (65536u + uh - 1u) / uh;          // ceil(2^16 / H)
     int qbase = fg_uni((int)(k0 / H));                       // edge of the chunk's first element
     unsigned rem = (unsigned)fg_uni((int)(k0 - (int64_t)qbase * H));
     const int qlast = fg_uni((int)((k1 - 1) / H));
     int rlo = gat_row_of(ptr, 0, N - 1, qbase);
     const int rhi = gat_row_of(ptr, rlo, N - 1, qlast);
-    for (int64_t kk = k0; kk < k1; kk += 64) {
-        const unsigned x = rem + (unsigned)lane;
-        const unsigned dq = x / uh;
-        const int h = (int)(x - dq * uh);
-        const int q = min(qbase + (int)dq, qlast);
-        const int row = gat_row_of(ptr, rlo, rhi, q);
-        const int64_t k = kk + lane;
-        if (k < k1) {
-            const size_t rh = (size_t)row * H + h;
-            const float ev = fg_lrelu(ar[rh] + ac[(size_t)idx[q] * H + h], slope);
-            if (e_lrelu) __builtin_nontemporal_store(ev, e_lrelu + k);
-            __builtin_nontemporal_store(__builtin_amdgcn_exp2f((ev - emax[rh]) * FGNN_LOG2E) * __builtin_amdgcn_rcpf(esum[rh]), e_softmax + k);
+    // GAT_STASH_UJ chunks per trip, their bisections and loads side by side: one chunk is a chain of
+    // dependent loads (row bounds, source id, attn_col of the source), several in flight hide it
+    constexpr int UJ = GAT_STASH_UJ;
+    for (int64_t kk = k0; kk < k1; kk += 64 * UJ) {
+        int q[UJ], h[UJ], lo[UJ], hi[UJ];
+#pragma unroll
+        for (int j = 0; j < UJ; ++j) {
+            const unsigned x = rem + (unsigned)(64 * j + lane);           // < H + 64 * UJ <= 320
+            const unsigned dq = (x * inv_h) >> 16;                          // = x / H for x < 1024 (H <= 64)
+            h[j] = (int)(x - dq * uh);
+            q[j] = min(qbase + (int)dq, qlast);
+            lo[j] = rlo; hi[j] = rhi;
         }
-        rem += 64u;
+        for (int w = rhi - rlo; w > 0; w >>= 1) {           // wave-uniform trip count: ceil(log2(window))
+#pragma unroll
+            for (int j = 0; j < UJ; ++j) {
+                const int mid = (lo[j] + hi[j] + 1) >> 1;   // lo == hi: mid == lo, nothing changes
+                if (lo[j] < hi[j]) { if (ptr[mid] <= q[j]) lo[j] = mid; else hi[j] = mid - 1; }
+            }
+        }
+        int src[UJ];
+#pragma unroll
+        for (int j = 0; j < UJ; ++j) src[j] = idx[q[j]];
+#pragma unroll
+        for (int j = 0; j < UJ; ++j) {
+            const int64_t k = kk + 64 * j + lane;
+            if (k < k1) {
+                const size_t rh = (size_t)lo[j] * H + h[j];
+                const float ev = fg_lrelu(ar[rh] + ac[(size_t)src[j] * H + h[j]], slope);
+                if (e_lrelu) __builtin_nontemporal_store(ev, e_lrelu + k);
+                __builtin_nontemporal_store(__builtin_amdgcn_exp2f((ev - emax[rh]) * FGNN_LOG2E) * __builtin_amdgcn_rcpf(esum[rh]), e_softmax + k);
+            }
+        }
+        rem += 64u * UJ;
         const unsigned adv = rem / uh;
         qbase += (int)adv;
         rem -= adv * uh;
-        rlo = __builtin_amdgcn_readlane(row, 63);           // rows only grow along the chunk
+        rlo = __builtin_amdgcn_readlane(lo[UJ - 1], 63);    // rows only grow along the chunks
     }
 }
 

@@ -163,13 +163,37 @@ def default_seg_len() -> int:
     return int(os.environ.get("FGNN_SEG_LEN", "0"))
 
 
-def xcd_buckets_enabled(n_rows: int, n_edges: int) -> bool:
-    """XCD-aware schedules pay off when rows are long enough to be cut in eight: on by default for
-    graphs with an average degree of at least 64 (FGNN_XCD_BUCKETS=0/1 overrides)."""
+_bucket_rule_cache: "collections.OrderedDict" = collections.OrderedDict()
+BUCKET_ROW_LEN = 64          # rows longer than this are the ones an XCD-aware schedule cuts by source bucket
+BUCKET_MIN_SHARE = 0.25      # ...and they must hold at least this share of the entries
+BUCKET_MIN_SKEW = 4          # longest row / mean row length
+
+
+def xcd_buckets_enabled(ptr_tensor) -> bool:
+    """Whether operators get the XCD-aware schedule for this pointer array (FGNN_XCD_BUCKETS=0/1
+    overrides).  It pays off on skewed graphs, where the rows longer than 64 entries hold a good part
+    of the work: cutting them by source bucket keeps each XCD's L2 on one eighth of the gathered rows
+    and shortens the longest work item.  It costs time on graphs without hubs (every row of a
+    uniform degree-100 graph would become eight short segments with nothing to reuse between them),
+    so the rule asks for both: rows longer than 64 hold a quarter of the entries, and the longest row
+    is at least 4x the mean.  The two numbers are read from the device once per array and cached."""
     env = os.environ.get("FGNN_XCD_BUCKETS")
     if env is not None:
         return env not in ("0", "")
-    return n_rows > 0 and n_edges >= 64 * n_rows
+    n_rows = ptr_tensor.numel() - 1
+    if n_rows <= 0:
+        return False
+    key = (ptr_tensor.data_ptr(), ptr_tensor.numel(), ptr_tensor.device.index, ptr_tensor._version)
+    hit = _bucket_rule_cache.get(key)
+    if hit is None:
+        deg = (ptr_tensor[1:] - ptr_tensor[:-1]).long()
+        long_rows = torch.where(deg > BUCKET_ROW_LEN, deg, torch.zeros_like(deg)).sum()
+        n_edges, n_long, longest = torch.stack([deg.sum(), long_rows, deg.max()]).tolist()
+        hit = n_edges > 0 and n_long >= BUCKET_MIN_SHARE * n_edges and longest * n_rows >= BUCKET_MIN_SKEW * n_edges
+        _bucket_rule_cache[key] = hit
+        while len(_bucket_rule_cache) > 4 * _SCHED_CACHE_MAX:
+            _bucket_rule_cache.popitem(last=False)
+    return hit
 
 
 def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True) -> Schedule:
@@ -180,7 +204,7 @@ def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True)
     the caller's position of every entry, 4*E bytes more); a schedule with positions serves both."""
     if seg_len is None:
         seg_len = default_seg_len()
-    if idx_tensor is not None and not xcd_buckets_enabled(ptr_tensor.numel() - 1, idx_tensor.numel()):
+    if idx_tensor is not None and not xcd_buckets_enabled(ptr_tensor):
         idx_tensor = None
     min_deg = int(os.environ.get("FGNN_BUCKET_MIN_DEG", "0"))
 
@@ -204,6 +228,7 @@ def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True)
 
 def clear_schedule_cache():
     _sched_cache.clear()
+    _bucket_rule_cache.clear()
 
 
 def workspace(nbytes: int, device):

@@ -23,6 +23,36 @@ def reduce_over_rows(x, g):
     return out
 
 
+def column_sum(g):
+    """g.sum(0) for tall g [N, c].  torch's reduction over the rows falls off a cliff when c is not a
+    multiple of 4 (19 ms for 2.4 M x 47, 1.2 ms for 233 k x 41, against 40 us and 14 us for 16
+    columns): the rows are cut into chunks that are summed side by side, then the chunk sums are added
+    (0.15 ms and 0.04 ms).  Narrow, aligned, moderately sized inputs keep the single reduction."""
+    n, c = g.shape
+    chunks = min(256, n // 2048)
+    if chunks < 2 or (c % 4 == 0 and n * c < (1 << 25)):
+        return g.sum(0)
+    rows = n // chunks
+    body = chunks * rows
+    out = g[:body].view(chunks, rows, c).sum(1).sum(0)
+    return out + g[body:].sum(0) if body < n else out
+
+
+class _AddBias(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, bias):
+        return x + bias
+
+    @staticmethod
+    def backward(ctx, g):
+        return g, (column_sum(g.contiguous()) if ctx.needs_input_grad[1] else None)
+
+
+def add_bias(x, bias):
+    """x + bias for x [N, c], bias [c]; the bias gradient is taken by `column_sum`."""
+    return _AddBias.apply(x, bias)
+
+
 class _TallLinear(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, bias):
@@ -37,7 +67,7 @@ class _TallLinear(torch.autograd.Function):
         g = g.contiguous()
         gx = torch.matmul(g, weight) if ctx.needs_input_grad[0] else None
         gw = reduce_over_rows(g, x) if ctx.needs_input_grad[1] else None
-        gb = g.sum(0) if (ctx.has_bias and ctx.needs_input_grad[2]) else None
+        gb = column_sum(g) if (ctx.has_bias and ctx.needs_input_grad[2]) else None
         return gx, gw, gb
 
 

@@ -7,7 +7,7 @@ from torch import nn
 from torch.nn import init
 
 from ..operators.fused_gmmconv import GmmConvFuseSum, GmmConvFuseSumTwoOrders, GmmConvStash
-from .dense import tall_linear
+from .dense import add_bias, tall_linear
 
 
 class _GMMBase(nn.Module):
@@ -68,7 +68,7 @@ class _GMMBase(nn.Module):
         if self.res_fc is not None:
             rst = rst + self.res_fc(feat)
         if self.bias is not None:
-            rst = rst + self.bias
+            rst = add_bias(rst, self.bias)
         return rst
 
 

@@ -248,3 +248,20 @@ def test_tall_linear_equals_linear():
             gg = torch.autograd.grad((got * go).sum(), leaves)
             assert all(torch.allclose(a, c, rtol=1e-10, atol=1e-10) for a, c in zip(gg, gw))
         assert torch.allclose(reduce_over_rows(x.detach(), go), x.detach().t() @ go, rtol=1e-10, atol=1e-10)
+
+
+def test_column_sum_and_add_bias_equal_the_plain_forms():
+    """layers.dense: the chunked column sum (bias gradients of tall matrices) equals g.sum(0) for widths
+    that are and are not multiples of 4 and row counts on both sides of the chunking threshold."""
+    from ae_mlsys_gnn_amd.layers.dense import add_bias, column_sum
+    torch.manual_seed(0)
+    for n, c in ((10, 3), (4096, 7), (4096 + 17, 7), (3 * 2048 + 5, 8), (70001, 47), (600000, 64)):
+        g = torch.randn(n, c, dtype=torch.float64)
+        assert torch.allclose(column_sum(g), g.sum(0), rtol=1e-10, atol=1e-9)
+    x = torch.randn(5000, 6, dtype=torch.float64, requires_grad=True)
+    b = torch.randn(6, dtype=torch.float64, requires_grad=True)
+    go = torch.randn(5000, 6, dtype=torch.float64)
+    want = torch.autograd.grad(((x + b) * go).sum(), (x, b))
+    got = torch.autograd.grad((add_bias(x, b) * go).sum(), (x, b))
+    assert torch.equal(add_bias(x, b), x + b)
+    assert all(torch.allclose(a, w, rtol=1e-10, atol=1e-10) for a, w in zip(got, want))

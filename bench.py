@@ -32,8 +32,8 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published peak
 # They bound the HBM traffic from above.  None = not measured for that workload.
 MEASURED_TRAFFIC_BYTES = {
     "gat_c2": {"fwd": 38_905_487_360, "bwd": 39_145_359_872},
-    "gat_c5_layer1": {"fwd": 72_099_949_465, "bwd": 81_156_805_427},
-    "gmm_c4": {"fwd": 1161785548, "bwd": 1468256256},
+    "gat_c5_layer1": {"fwd": 60_759_466_188, "bwd": 68_750_860_697},
+    "gmm_c4": {"fwd": 995_238_707, "bwd": 1_676_252_057},
     "edgeconv_c3": {"fwd": 123_305_574, "bwd": 73_504_972},
 }
 

@@ -96,6 +96,33 @@ def test_gat_long_rows_pair_layout(h, f, variant, monkeypatch):
     _lib.clear_schedule_cache()
 
 
+def test_xcd_aware_schedule_is_chosen_by_row_length_skew(monkeypatch):
+    """Without an override the operators take the XCD-aware work list on graphs where the rows longer
+    than 64 entries hold a quarter of the entries and the longest row is 4x the mean (an R-MAT graph of
+    average degree 5 qualifies, a uniform graph of average degree 100 does not); the decision is cached
+    per pointer array, the results agree with the oracle either way, and FGNN_XCD_BUCKETS overrides."""
+    from ae_mlsys_gnn_amd import _lib
+    monkeypatch.delenv("FGNN_XCD_BUCKETS", raising=False)
+    monkeypatch.delenv("FGNN_BUCKET_MIN_DEG", raising=False)
+    _lib.clear_schedule_cache()
+    skewed_host, flat_host = graphs.rmat_graph(20000, 100000, seed=31), graphs.uniform_graph(3000, 300000, seed=32)
+    skewed, flat, short = skewed_host.to("cuda:0"), flat_host.to("cuda:0"), graphs.uniform_graph(3000, 30000, seed=33).to("cuda:0")
+    assert _lib.xcd_buckets_enabled(skewed.row_ptr) is True
+    assert _lib.xcd_buckets_enabled(flat.row_ptr) is False and _lib.xcd_buckets_enabled(short.row_ptr) is False
+    assert len(_lib._bucket_rule_cache) == 3
+    assert _lib.xcd_buckets_enabled(skewed.row_ptr) is True and len(_lib._bucket_rule_cache) == 3
+    assert _lib.schedule_for(skewed.row_ptr, idx_tensor=skewed.col_ind).n_partials > 0
+    assert _lib.schedule_for(flat.row_ptr, idx_tensor=flat.col_ind).n_partials == 0
+    for g in (skewed_host, flat_host):
+        _run(g, 4, 16, variant="sm")
+        _run(g, 2, 64, variant="stash")
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "0")
+    assert _lib.xcd_buckets_enabled(skewed.row_ptr) is False
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
+    assert _lib.xcd_buckets_enabled(flat.row_ptr) is True
+    _lib.clear_schedule_cache()
+
+
 def test_gat_split_rows(monkeypatch):
     monkeypatch.setenv("FGNN_SEG_LEN", "256")
     from ae_mlsys_gnn_amd import _lib

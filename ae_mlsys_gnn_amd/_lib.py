@@ -25,6 +25,7 @@ _SIGNATURES = {
     "fgnn_last_error": (ctypes.c_char_p, []),
     "fgnn_schedule_create": (c_int, [c_void_p, c_int, c_int, c_void_p, ctypes.POINTER(c_void_p)]),
     "fgnn_schedule_create_bucketed": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, ctypes.POINTER(c_void_p)]),
+    "fgnn_schedule_take_positions": (c_int, [c_void_p, c_void_p, c_void_p]),
     "fgnn_schedule_destroy": (None, [c_void_p]),
     "fgnn_schedule_num_items": (c_int, [c_void_p]),
     "fgnn_schedule_num_partials": (c_int, [c_void_p]),
@@ -147,6 +148,16 @@ class Schedule:
         self.n_items = lib().fgnn_schedule_num_items(handle)
         self.n_partials = lib().fgnn_schedule_num_partials(handle)
         self.n_edges = lib().fgnn_schedule_num_edges(handle)
+        self.own_order = False
+
+    def take_positions(self):
+        """int32 [E]: caller's edge position of every entry in the schedule's own order.  The schedule gives
+        up its copy; operators called with it afterwards take per-edge tensors in that order."""
+        out = torch.empty(self.n_edges, dtype=torch.int32, device=self.ptr_tensor.device)
+        with torch.cuda.device(self.ptr_tensor.device):
+            check(lib().fgnn_schedule_take_positions(self.handle, ptr(out), stream_ptr()), "fgnn_schedule_take_positions")
+        self.own_order = True
+        return out
 
     def __del__(self):
         h = getattr(self, "handle", None)
@@ -196,12 +207,14 @@ def xcd_buckets_enabled(ptr_tensor) -> bool:
     return hit
 
 
-def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True) -> Schedule:
+def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True, own_order=False) -> Schedule:
     """Cached schedule of a pointer array.  The cache entry holds the tensors, so their device
     addresses cannot be reused while the entry lives; in-place edits bump `_version`.
     idx_tensor: the index array, for operators that may use an XCD-aware schedule.
     need_positions: whether the operator has per-edge tensors (an XCD-aware schedule then also keeps
-    the caller's position of every entry, 4*E bytes more); a schedule with positions serves both."""
+    the caller's position of every entry, 4*E bytes more); a schedule with positions serves both.
+    own_order: a schedule of its own (never shared with the other kinds) whose position map was taken
+    out (`edge_positions`): operators called with it take per-edge tensors in the schedule's order."""
     if seg_len is None:
         seg_len = default_seg_len()
     if idx_tensor is not None and not xcd_buckets_enabled(ptr_tensor):
@@ -211,6 +224,14 @@ def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True)
     def key(pos):
         return (ptr_tensor.data_ptr(), ptr_tensor.numel(), ptr_tensor.device.index, ptr_tensor._version, int(seg_len),
                 None if idx_tensor is None else (idx_tensor.data_ptr(), idx_tensor._version, min_deg, pos))
+    if own_order:
+        k = key("own")
+        s = _sched_cache.get(k)
+        if s is None:
+            raise FgnnError("no own-order schedule for these arrays: call edge_positions(ptr, idx) first and pass per-edge "
+                            "tensors permuted by its result")
+        _sched_cache.move_to_end(k)
+        return s
     k = key(True)
     s = _sched_cache.get(k)
     if s is None and not need_positions and idx_tensor is not None:
@@ -224,6 +245,30 @@ def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True)
     else:
         _sched_cache.move_to_end(k)
     return s
+
+
+def edge_positions(ptr_tensor, idx_tensor, seg_len=None):
+    """Builds (once) the own-order schedule of (ptr, idx) and returns int32 [E]: the caller's position of
+    every entry in that schedule's order, or None when the order is the caller's (plain schedule).
+    Per-edge tensors passed to operators with edge_order="schedule" must be t[edge_positions]."""
+    if seg_len is None:
+        seg_len = default_seg_len()
+    bucketed = xcd_buckets_enabled(ptr_tensor)
+    min_deg = int(os.environ.get("FGNN_BUCKET_MIN_DEG", "0"))
+    k = (ptr_tensor.data_ptr(), ptr_tensor.numel(), ptr_tensor.device.index, ptr_tensor._version, int(seg_len),
+         (idx_tensor.data_ptr(), idx_tensor._version, min_deg, "own") if bucketed else None)
+    if not bucketed:
+        schedule_for(ptr_tensor, seg_len)          # the plain schedule serves both orders
+        return None
+    s = Schedule(ptr_tensor, seg_len, idx_tensor, min_deg, with_positions=True)
+    pos = s.take_positions()
+    if k in _sched_cache:                   # asked again: the map is a function of the arrays, the cached schedule stays
+        _sched_cache.move_to_end(k)
+        return pos
+    _sched_cache[k] = s
+    while len(_sched_cache) > _SCHED_CACHE_MAX:
+        _sched_cache.popitem(last=False)
+    return pos
 
 
 def clear_schedule_cache():

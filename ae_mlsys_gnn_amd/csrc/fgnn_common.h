@@ -66,13 +66,14 @@ struct fgnn_schedule {
     const int32_t *idx_src_dev;
     int32_t *bidx_dev;
     int32_t *bpos_dev;      // original position of every bucket-ordered entry (for per-edge arrays)
+    int own_order;          // the position map was handed to the caller: per-edge arrays come in the schedule's entry order
 };
 // The index array a kernel walks under schedule `s`, and the map from its positions back to the
 // caller's edge positions (NULL = identity).
 static inline const int32_t *fgnn_sched_idx(const fgnn_schedule *s, const int32_t *idx) { return (s && s->n_buckets > 0) ? s->bidx_dev : idx; }
 static inline const int32_t *fgnn_sched_pos(const fgnn_schedule *s) { return (s && s->n_buckets > 0) ? s->bpos_dev : nullptr; }
 // false for an XCD-aware schedule built without the position map: operators with per-edge tensors must refuse it
-static inline bool fgnn_sched_has_pos(const fgnn_schedule *s) { return !s || s->n_buckets == 0 || s->n_edges == 0 || s->bpos_dev != nullptr; }
+static inline bool fgnn_sched_has_pos(const fgnn_schedule *s) { return !s || s->n_buckets == 0 || s->n_edges == 0 || s->bpos_dev != nullptr || s->own_order; }
 
 #define FGNN_NUM_XCD 8      // workgroup w of a dispatch runs on XCD w % 8 (gfx942 / gfx950, SPX mode)
 // Source bucket of a node id: the top 3 bits of a multiplicative hash, so hot ids spread evenly.

@@ -127,7 +127,7 @@ static fgnn_schedule *new_schedule(const int32_t *ptr_dev, int n_rows, int64_t n
     s->n_rows = n_rows; s->n_edges = n_edges; s->seg_len = seg_len;
     s->n_items = s->n_partials = s->n_split = 0;
     s->items_dev = nullptr; s->split_dev = nullptr; s->ptr_dev = ptr_dev;
-    s->n_buckets = 0; s->idx_src_dev = nullptr; s->bidx_dev = nullptr; s->bpos_dev = nullptr;
+    s->n_buckets = 0; s->idx_src_dev = nullptr; s->bidx_dev = nullptr; s->bpos_dev = nullptr; s->own_order = 0;
     (void)hipGetDevice(&s->device);
     return s;
 }
@@ -260,6 +260,38 @@ extern "C" int fgnn_schedule_create_bucketed(const int32_t *ptr_dev, const int32
     rc = upload_schedule(s, items, splits, st);
     if (rc) { fgnn_schedule_destroy(s); return rc; }
     *out = s;
+    return 0;
+}
+
+__global__ __launch_bounds__(256) void iota_i32_kernel(int64_t n, int *__restrict__ out)
+{
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = (int)i;
+}
+
+// Hands the map (schedule entry order -> caller's edge position) to the caller and drops the
+// schedule's own copy.  From then on operators index per-edge tensors (and `permute`) by the
+// schedule's entry order: an XCD then reads and writes the per-edge data of its segments as
+// contiguous runs instead of scattered elements of lines that all eight XCDs touch.
+extern "C" int fgnn_schedule_take_positions(fgnn_schedule_t *s, int32_t *pos_out_dev, void *stream)
+{
+    FGNN_REQUIRE(s, FGNN_ERR_NULL, "fgnn_schedule_take_positions: NULL schedule");
+    FGNN_REQUIRE(pos_out_dev || s->n_edges == 0, FGNN_ERR_NULL, "fgnn_schedule_take_positions: NULL output");
+    FGNN_REQUIRE(!s->own_order, FGNN_ERR_SCHEDULE, "fgnn_schedule_take_positions: the positions of this schedule were taken before");
+    FGNN_REQUIRE(fgnn_sched_has_pos(s), FGNN_ERR_SCHEDULE, "fgnn_schedule_take_positions: the schedule was built without edge positions");
+    hipStream_t st = (hipStream_t)stream;
+    if (s->n_edges > 0) {
+        if (s->n_buckets > 0) {
+            FGNN_HIP(hipMemcpyAsync(pos_out_dev, s->bpos_dev, (size_t)s->n_edges * sizeof(int32_t), hipMemcpyDeviceToDevice, st));
+        } else {        // plain schedules walk the caller's arrays: identity
+            hipLaunchKernelGGL(iota_i32_kernel, dim3((unsigned)((s->n_edges + 255) / 256)), dim3(256), 0, st, s->n_edges, pos_out_dev);
+            int rc = fgnn_launch_status("iota_i32_kernel");
+            if (rc) return rc;
+        }
+        FGNN_HIP(hipStreamSynchronize(st));      // the copy must be done before the source is freed
+    }
+    if (s->bpos_dev) { (void)hipFree(s->bpos_dev); s->bpos_dev = nullptr; }
+    s->own_order = 1;
     return 0;
 }
 

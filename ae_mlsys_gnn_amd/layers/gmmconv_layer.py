@@ -49,18 +49,23 @@ class _GMMBase(nn.Module):
     def set_allow_zero_in_degree(self, set_value):
         self._allow_zero_in_degree = set_value
 
-    def forward(self, rowptr, colind, colptr, rowind, permute, feat, pseudo, pseudo_csc=None):
+    def forward(self, rowptr, colind, colptr, rowind, permute, feat, pseudo, pseudo_csc=None, own_order=False):
         """pseudo_csc (GMMConv only): the same pseudo-coordinates in CSC order, pseudo[permute], built by
         the caller from its own CSC-ordered edge data.  The backward then works in CSC order throughout
-        and the gradient of the pseudo-coordinates flows through pseudo_csc instead of pseudo."""
+        and the gradient of the pseudo-coordinates flows through pseudo_csc instead of pseudo.
+        own_order (GMMConv only): pseudo and pseudo_csc are in the entry order of the operators' schedules
+        (operators.fused_gmmconv.gmm_edge_positions); without pseudo_csc the layer is forward-only."""
         node_feat = tall_linear(feat, self.fc.weight).view(-1, self._n_kernels, self._out_feats)    # = self.fc(feat)
         pad = (-self._out_feats) % 4
         if pad:         # zero columns up to a multiple of 4: the operator then takes its 128-bit row layout
             node_feat = th.nn.functional.pad(node_feat, (0, pad))
-        if pseudo_csc is not None:
+        if pseudo_csc is not None or own_order:
             if type(self)._op is not GmmConvFuseSum:
-                raise ValueError("pseudo_csc is supported by the recomputing GMMConv layer only")
-            rst = GmmConvFuseSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo.detach(), pseudo_csc, self.mu, self.inv_sigma)
+                raise ValueError("pseudo_csc / own_order are supported by the recomputing GMMConv layer only")
+            if own_order and pseudo_csc is None and th.is_grad_enabled() and (node_feat.requires_grad or pseudo.requires_grad):
+                raise ValueError("own_order without pseudo_csc is forward-only")
+            rst = GmmConvFuseSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo.detach(), pseudo_csc, self.mu, self.inv_sigma,
+                                          own_order=own_order)
         else:
             rst = type(self)._op(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, self.mu, self.inv_sigma)
         if pad:

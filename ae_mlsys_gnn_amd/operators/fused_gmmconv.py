@@ -6,14 +6,14 @@ from __future__ import annotations
 
 import torch
 
-from .._lib import FgnnError, as_f32, as_i32, check, lib, ptr, require_cuda, schedule_for, stream_ptr, workspace
+from .._lib import FgnnError, as_f32, as_i32, check, edge_positions, lib, ptr, require_cuda, schedule_for, stream_ptr, workspace
 
 
 class gmm_native:
     """gmmconv.gmmconv / gmmconvstash / Gaussian / GaussianBp (src/fused_gmmconv/gmmconv.cc:36-94)."""
 
     @staticmethod
-    def gmmconv(rowptr, colind, node_feat, pseudo, mu, sigma, *, pos_map=None, want_gauss=False, sum_kernels=False):
+    def gmmconv(rowptr, colind, node_feat, pseudo, mu, sigma, *, pos_map=None, want_gauss=False, sum_kernels=False, own_order=False):
         require_cuda(rowptr, colind, node_feat, pseudo, mu, sigma)
         rowptr, colind = as_i32(rowptr), as_i32(colind)
         node_feat, pseudo, mu, sigma = as_f32(node_feat), as_f32(pseudo), as_f32(mu), as_f32(sigma)
@@ -27,7 +27,8 @@ class gmm_native:
                 tuple(mu.shape), tuple(sigma.shape), tuple(pseudo.shape), k, e))
         out = torch.empty((n, f), dtype=torch.float32, device=node_feat.device) if sum_kernels else torch.empty_like(node_feat)
         gauss = torch.empty((e, k), dtype=torch.float32, device=node_feat.device) if want_gauss else None
-        sched = schedule_for(rowptr, idx_tensor=colind)
+        # own_order: pseudo (and gauss) are indexed by the schedule's entry order, pseudo_caller[edge_positions(rowptr, colind)]
+        sched = schedule_for(rowptr, idx_tensor=colind, own_order=own_order)
         with torch.cuda.device(node_feat.device):
             ws, wsb = workspace(lib().fgnn_gmm_forward_workspace_bytes(sched.handle, k, f), node_feat.device)
             check(lib().fgnn_gmm_forward(n, e, k, dim, f, ptr(rowptr), ptr(colind), ptr(pos_map), ptr(node_feat), ptr(pseudo),
@@ -36,7 +37,7 @@ class gmm_native:
         return (out, gauss) if want_gauss else out
 
     @staticmethod
-    def gmmconv_backward(colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out, sum_kernels=False):
+    def gmmconv_backward(colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out, sum_kernels=False, own_order=False):
         require_cuda(colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out)
         colptr, rowind = as_i32(colptr), as_i32(rowind)
         permute = None if permute is None else as_i32(permute)      # None: pseudo / grad_pseudo in CSC order
@@ -50,7 +51,9 @@ class gmm_native:
         grad_mu = torch.empty_like(mu)
         grad_sigma = torch.empty_like(sigma)
         # the summed form gathers narrow rows ([N,F]); below an average degree of 64 it measured faster on the plain work list
-        sched = schedule_for(colptr, idx_tensor=None if (sum_kernels and e < 64 * n) else rowind)
+        # own_order: pseudo, grad_pseudo (and permute) are indexed by the schedule's entry order (edge_positions(colptr, rowind))
+        sched = (schedule_for(colptr, idx_tensor=rowind, own_order=True) if own_order else
+                 schedule_for(colptr, idx_tensor=None if (sum_kernels and e < 64 * n) else rowind))
         with torch.cuda.device(dev):
             ws, wsb = workspace(lib().fgnn_gmm_backward_workspace_bytes(sched.handle, k, dim, f), dev)
             check(lib().fgnn_gmm_backward(n, e, k, dim, f, ptr(colptr), ptr(rowind), ptr(permute), ptr(node_feat), ptr(pseudo),
@@ -110,28 +113,41 @@ def GmmConvFuseSum(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, m
     return GmmFuseSumFunction.apply(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma)
 
 
-def GmmConvFuseSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma):
+def GmmConvFuseSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order=False):
     """GmmConvFuseSum for a caller that has the pseudo-coordinates in both edge orders
     (pseudo_csc == pseudo_csr[permute], e.g. the same elementwise projection applied to constant
     edge data stored both ways).  The forward reads pseudo_csr, the backward reads pseudo_csc and
     returns its gradient in CSC order: no per-edge gather or scatter through permute.  pseudo_csr
-    gets no gradient; the caller's parameters receive theirs through pseudo_csc."""
-    return GmmFuseSumTwoOrdersFunction.apply(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma)
+    gets no gradient; the caller's parameters receive theirs through pseudo_csc (None: forward only).
+    own_order: the two tensors are in the entry order of the operators' own schedules,
+    pseudo_csr[gmm_edge_positions(rowptr, colind)] and pseudo_csc[gmm_edge_positions(colptr, rowind)]:
+    every pass then streams its per-edge data."""
+    if pseudo_csc is None:
+        return gmm_native.gmmconv(rowptr, colind, node_feat, pseudo_csr, mu, sigma, sum_kernels=True, own_order=own_order)
+    return GmmFuseSumTwoOrdersFunction.apply(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order)
+
+
+def gmm_edge_positions(ptr_arr, idx):
+    """int32 [E] (or None = identity): caller's position of every entry in the order in which the GMMConv
+    operators walk (ptr_arr, idx) when called with own_order=True."""
+    require_cuda(ptr_arr, idx)
+    return edge_positions(as_i32(ptr_arr), as_i32(idx))
 
 
 class GmmFuseSumTwoOrdersFunction(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma):
-        out = gmm_native.gmmconv(rowptr, colind, node_feat, pseudo_csr, mu, sigma, sum_kernels=True)      # [N, F]
+    def forward(ctx, rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order):
+        out = gmm_native.gmmconv(rowptr, colind, node_feat, pseudo_csr, mu, sigma, sum_kernels=True, own_order=own_order)      # [N, F]
         ctx.save_for_backward(colptr, rowind, node_feat, pseudo_csc, mu, sigma)
+        ctx.own_order = own_order
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
         colptr, rowind, node_feat, pseudo_csc, mu, sigma = ctx.saved_tensors
         grad_feat, grad_pseudo_csc, grad_mu, grad_sigma = gmm_native.gmmconv_backward(
-            colptr, rowind, None, node_feat, pseudo_csc, mu, sigma, grad_out.contiguous(), sum_kernels=True)
-        return None, None, None, None, grad_feat, None, grad_pseudo_csc, grad_mu, grad_sigma
+            colptr, rowind, None, node_feat, pseudo_csc, mu, sigma, grad_out.contiguous(), sum_kernels=True, own_order=ctx.own_order)
+        return None, None, None, None, grad_feat, None, grad_pseudo_csc, grad_mu, grad_sigma, None
 
 
 class GmmFuseSumFunction(torch.autograd.Function):

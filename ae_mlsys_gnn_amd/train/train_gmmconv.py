@@ -17,6 +17,7 @@ from torch import nn
 
 from ..layers import GMMConv, GMMConv_stash
 from ..operators import edge_proj
+from ..operators.fused_gmmconv import gmm_edge_positions
 from . import common, datasets
 
 VARIANTS = {"our": GMMConv, "stash": GMMConv_stash}
@@ -45,10 +46,11 @@ class MoNet(nn.Module):
         self.pseudo_proj = nn.ModuleList(PseudoProj(2, dim) for _ in self.layers)
         self.dropout = nn.Dropout(dropout)
 
-    def forward(self, g, feat, pseudo, pseudo_csc=None):
+    def forward(self, g, feat, pseudo, pseudo_csc=None, own_order=False):
         """pseudo: raw per-edge coordinates [E, 2] in CSR order; pseudo_csc: the same rows in CSC order
         (pseudo[permute]).  With both, each layer projects both copies (the projection is elementwise per
-        edge, so the results are each other's permutation) and the layer's backward runs in CSC order."""
+        edge, so the results are each other's permutation) and the layer's backward runs in CSC order.
+        own_order: both copies are in the entry order of the operators' schedules instead (`schedule_order_copies`)."""
         h = feat
         for i, (layer, proj) in enumerate(zip(self.layers, self.pseudo_proj)):
             if i:
@@ -56,10 +58,22 @@ class MoNet(nn.Module):
             if pseudo_csc is not None and torch.is_grad_enabled():
                 with torch.no_grad():
                     ps = proj(pseudo)
-                h = layer(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, g.permute, h, ps, pseudo_csc=proj(pseudo_csc))
+                h = layer(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, g.permute, h, ps, pseudo_csc=proj(pseudo_csc), own_order=own_order)
             else:
-                h = layer(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, g.permute, h, proj(pseudo))
+                h = layer(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, g.permute, h, proj(pseudo), own_order=own_order)
         return h
+
+
+def schedule_order_copies(g, pseudo):
+    """The raw coordinates in the entry order of the forward (CSR) and backward (CSC) schedules of the
+    GMMConv operators.  The coordinates are constant and their projection is elementwise, so the whole
+    per-edge pipeline (projection, Gaussian weights, their gradients) can run in those orders and every
+    pass streams its per-edge data instead of reaching it through a position map."""
+    pos_r = gmm_edge_positions(g.row_ptr, g.col_ind)
+    pos_c = gmm_edge_positions(g.col_ptr, g.row_ind)
+    fwd = pseudo if pos_r is None else pseudo[pos_r.long()].contiguous()
+    to_csc = g.permute.long() if pos_c is None else g.permute[pos_c.long()].long()
+    return fwd, pseudo[to_csc].contiguous()
 
 
 def build_parser():
@@ -76,8 +90,9 @@ def build_parser():
     p.add_argument("--weight-decay", type=float, default=5e-4)
     p.add_argument("--output", type=str, default="figure7.csv")
     p.add_argument("--variant", choices=sorted(VARIANTS), default="our")
-    p.add_argument("--csc-pseudo", type=int, default=1, help="1: keep the edge coordinates in CSR and CSC order (variant our), so the "
-                   "backward needs no per-edge transposition; 0: one copy, as the reference")
+    p.add_argument("--csc-pseudo", type=int, default=2, help="2: keep the edge coordinates in the entry order of the forward and the backward "
+                   "schedule (variant our), so every pass streams its per-edge data; 1: in CSR and CSC order (no per-edge transposition in "
+                   "the backward); 0: one copy, as the reference")
     p.add_argument("--data-root", type=str, default=None)
     p.add_argument("--cache-dir", type=str, default=None)
     p.add_argument("--scale", type=float, default=1.0)
@@ -96,7 +111,11 @@ def main(argv=None):
     print("----Data statistics------ (%s)\n  #Nodes %d\n  #Edges %d\n  #Classes %d\n  #Train samples %d\n  #Val samples %d\n  #Test samples %d"
           % (data.source, g.n, g.n_edges, data.n_classes, int(data.train_mask.sum()), int(data.val_mask.sum()), int(data.test_mask.sum())))
     pseudo = datasets.degree_pseudo(g)
-    pseudo_csc = pseudo[g.permute.long()].contiguous() if (args.csc_pseudo and args.variant == "our") else None
+    own_order = args.csc_pseudo == 2 and args.variant == "our"
+    if own_order:
+        pseudo, pseudo_csc = schedule_order_copies(g, pseudo)
+    else:
+        pseudo_csc = pseudo[g.permute.long()].contiguous() if (args.csc_pseudo and args.variant == "our") else None
     torch.manual_seed(args.seed)
     model = MoNet(VARIANTS[args.variant], data.feat.shape[1], args.n_hidden, data.n_classes, args.n_layers, args.pseudo_dim, args.n_kernels,
                   args.dropout).to(dev)
@@ -108,11 +127,11 @@ def main(argv=None):
     def evaluate(mask):
         model.eval()
         with torch.no_grad():
-            return common.accuracy(model(g, data.feat, pseudo)[mask], data.label[mask])      # no gradients: one copy is enough
+            return common.accuracy(model(g, data.feat, pseudo, own_order=own_order)[mask], data.label[mask])      # no gradients: one copy is enough
 
     def train_step():
         model.train()
-        loss = loss_fcn(model(g, data.feat, pseudo, pseudo_csc)[train_idx], train_labels)
+        loss = loss_fcn(model(g, data.feat, pseudo, pseudo_csc, own_order=own_order)[train_idx], train_labels)
         opt.zero_grad(set_to_none=False)
         loss.backward()
         opt.step()

@@ -624,6 +624,88 @@ def test_gmm_layer_with_csc_ordered_pseudo(k, dim, f, monkeypatch):
     _lib.clear_schedule_cache()
 
 
+@pytest.mark.parametrize("k,dim,f", [(3, 2, 16), (2, 1, 41), (2, 1, 16)])
+def test_gmm_layer_with_pseudo_in_schedule_order(k, dim, f, monkeypatch):
+    """GMMConv(..., own_order=True) with the pseudo-coordinates permuted into the entry order of the
+    operators' schedules (gmm_edge_positions): same output and gradients as the oracle, the gradient of
+    the pseudo-coordinates arrives in the backward schedule's order.  XCD-aware (a real permutation) and
+    plain schedules (identity, positions None); a forward-only call; asking for the positions twice."""
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd.layers import GMMConv
+    from ae_mlsys_gnn_amd.operators.fused_gmmconv import gmm_edge_positions
+    for buckets in ("1", "0"):
+        monkeypatch.setenv("FGNN_XCD_BUCKETS", buckets)
+        monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+        _lib.clear_schedule_cache()
+        torch.manual_seed(4)
+        g = graphs.add_csc_torch(graphs.rmat_graph(600, 30000, seed=6))
+        layer = GMMConv(24, f, dim=dim, n_kernels=k)
+        feat, pseudo, go = torch.randn(g.n, 24), torch.rand(g.n_edges, dim), torch.randn(g.n, f)
+        leaves = [t.detach().double().requires_grad_(True) for t in (layer.fc.weight, layer.mu, layer.inv_sigma, layer.bias, feat, pseudo)]
+        ref = orc.gmm_layer_dgl(leaves[0], leaves[1], leaves[2], leaves[3], g.row_ptr, g.col_ind, leaves[4], leaves[5])
+        ref.backward(go.double())
+        gd = g.to(DEV)
+        layer = layer.to(DEV)
+        fd = feat.to(DEV).requires_grad_(True)
+        pos_r, pos_c = gmm_edge_positions(gd.row_ptr, gd.col_ind), gmm_edge_positions(gd.col_ptr, gd.row_ind)
+        if buckets == "0":
+            assert pos_r is None and pos_c is None
+            pos_r = pos_c = torch.arange(g.n_edges, device=DEV, dtype=torch.int32)
+        else:
+            for pos, ptr_arr in ((pos_r, g.row_ptr), (pos_c, g.col_ptr)):        # a permutation that stays inside every row
+                assert torch.equal(pos.long().sort().values.cpu(), torch.arange(g.n_edges))
+                row_of = torch.repeat_interleave(torch.arange(g.n), (ptr_arr[1:] - ptr_arr[:-1]).long())
+                assert torch.equal(row_of[pos.long().cpu()], row_of)
+            assert not torch.equal(pos_r.cpu(), torch.arange(g.n_edges, dtype=torch.int32))
+            assert torch.equal(gmm_edge_positions(gd.row_ptr, gd.col_ind), pos_r)           # asked again: same map
+        to_csc = gd.permute.long()[pos_c.long()]
+        pd = pseudo.to(DEV)[pos_r.long()].contiguous()
+        pc = pseudo.to(DEV)[to_csc].contiguous().requires_grad_(True)
+        out = layer(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, pd, pseudo_csc=pc, own_order=True)
+        out.backward(go.to(DEV))
+        assert_close(out, ref.detach(), "GMMConv (schedule order)", atol=1e-4)
+        assert_close(fd.grad, leaves[4].grad, "grad feat (schedule order)", atol=1e-4)
+        assert_close(pc.grad, leaves[5].grad[to_csc.cpu()], "grad pseudo in the backward schedule's order", atol=1e-3)
+        assert_close(layer.mu.grad, leaves[1].grad, "grad mu (schedule order)", rtol=1e-3, atol=5e-2)
+        assert_close(layer.inv_sigma.grad, leaves[2].grad, "grad inv_sigma (schedule order)", rtol=1e-3, atol=5e-2)
+        assert_close(layer.fc.weight.grad, leaves[0].grad, "grad fc (schedule order)", rtol=1e-3, atol=5e-2)
+        with torch.no_grad():
+            assert_close(layer(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, pd, own_order=True), ref.detach(),
+                         "GMMConv forward only (schedule order)", atol=1e-4)
+        with pytest.raises(ValueError, match="forward-only"):
+            layer(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, pd, own_order=True)
+    _lib.clear_schedule_cache()
+
+
+def test_schedule_take_positions_c_abi(monkeypatch):
+    """fgnn_schedule_take_positions: the map of an XCD-aware schedule is handed over once; a schedule built
+    without positions refuses; a plain schedule returns the identity; afterwards mhspmm takes its per-edge
+    weights in the schedule's order."""
+    from ae_mlsys_gnn_amd import _lib
+    g = graphs.rmat_graph(500, 20000, seed=9).to(DEV)
+    s = _lib.Schedule(g.row_ptr, 0, g.col_ind, 16, with_positions=True)
+    pos = s.take_positions()
+    assert s.own_order and torch.equal(pos.long().sort().values.cpu(), torch.arange(g.n_edges))
+    with pytest.raises(_lib.FgnnError, match="taken before"):
+        s.take_positions()
+    with pytest.raises(_lib.FgnnError, match="without edge positions"):
+        _lib.Schedule(g.row_ptr, 0, g.col_ind, 16, with_positions=False).take_positions()
+    plain = _lib.Schedule(g.row_ptr, 0)
+    assert torch.equal(plain.take_positions().cpu(), torch.arange(g.n_edges, dtype=torch.int32))
+    # the operator under the own-order schedule: weights permuted by `pos` give the caller-order result
+    torch.manual_seed(1)
+    h, f = 2, 16
+    x, w = torch.randn(g.n, h, f, device=DEV), torch.rand(g.n_edges, h, device=DEV)
+    out = torch.empty(g.n, h, f, device=DEV)
+    wo = w[pos.long()].contiguous()
+    ws, wsb = _lib.workspace(_lib.lib().fgnn_mhspmm_workspace_bytes(s.handle, h, f), x.device)
+    _lib.check(_lib.lib().fgnn_mhspmm(g.n, g.n_edges, h, f, _lib.ptr(g.row_ptr), _lib.ptr(g.col_ind), None, _lib.ptr(wo), _lib.ptr(x),
+                                       _lib.ptr(out), s.handle, _lib.ptr(ws), wsb, _lib.stream_ptr()), "fgnn_mhspmm")
+    torch.cuda.synchronize()
+    want = orc.mhspmm(g.row_ptr.cpu(), g.col_ind.cpu(), w.cpu().double(), x.cpu().double())
+    assert_close(out, want, "mhspmm under an own-order schedule", atol=1e-4)
+
+
 @pytest.mark.parametrize("d", [1, 2, 3, 4])
 @pytest.mark.parametrize("e", [1, 257, 300001])
 def test_edge_linear_tanh_matches_torch(d, e):

@@ -9,6 +9,12 @@ import torch
 from .._lib import FgnnError, as_f32, as_i32, check, edge_positions, lib, ptr, require_cuda, schedule_for, stream_ptr, workspace
 
 
+def _plain_list_for_summed_backward(n, e):
+    """The summed backward gathers narrow rows ([N,F]); below an average degree of 64 it measured faster
+    on the plain work list than on the XCD-aware one."""
+    return e < 64 * n
+
+
 class gmm_native:
     """gmmconv.gmmconv / gmmconvstash / Gaussian / GaussianBp (src/fused_gmmconv/gmmconv.cc:36-94)."""
 
@@ -50,10 +56,8 @@ class gmm_native:
         grad_pseudo = torch.empty((e, dim), dtype=torch.float32, device=dev)
         grad_mu = torch.empty_like(mu)
         grad_sigma = torch.empty_like(sigma)
-        # the summed form gathers narrow rows ([N,F]); below an average degree of 64 it measured faster on the plain work list
-        # own_order: pseudo, grad_pseudo (and permute) are indexed by the schedule's entry order (edge_positions(colptr, rowind))
-        sched = (schedule_for(colptr, idx_tensor=rowind, own_order=True) if own_order else
-                 schedule_for(colptr, idx_tensor=None if (sum_kernels and e < 64 * n) else rowind))
+        # own_order: pseudo, grad_pseudo (and permute) are indexed by the schedule's entry order (gmm_edge_positions(colptr, rowind, True))
+        sched = schedule_for(colptr, idx_tensor=None if (sum_kernels and _plain_list_for_summed_backward(n, e)) else rowind, own_order=own_order)
         with torch.cuda.device(dev):
             ws, wsb = workspace(lib().fgnn_gmm_backward_workspace_bytes(sched.handle, k, dim, f), dev)
             check(lib().fgnn_gmm_backward(n, e, k, dim, f, ptr(colptr), ptr(rowind), ptr(permute), ptr(node_feat), ptr(pseudo),
@@ -120,18 +124,24 @@ def GmmConvFuseSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo_cs
     returns its gradient in CSC order: no per-edge gather or scatter through permute.  pseudo_csr
     gets no gradient; the caller's parameters receive theirs through pseudo_csc (None: forward only).
     own_order: the two tensors are in the entry order of the operators' own schedules,
-    pseudo_csr[gmm_edge_positions(rowptr, colind)] and pseudo_csc[gmm_edge_positions(colptr, rowind)]:
+    pseudo_csr[gmm_edge_positions(rowptr, colind)] and pseudo_csc[gmm_edge_positions(colptr, rowind, True)]:
     every pass then streams its per-edge data."""
     if pseudo_csc is None:
         return gmm_native.gmmconv(rowptr, colind, node_feat, pseudo_csr, mu, sigma, sum_kernels=True, own_order=own_order)
     return GmmFuseSumTwoOrdersFunction.apply(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order)
 
 
-def gmm_edge_positions(ptr_arr, idx):
+def gmm_edge_positions(ptr_arr, idx, summed_backward=False):
     """int32 [E] (or None = identity): caller's position of every entry in the order in which the GMMConv
-    operators walk (ptr_arr, idx) when called with own_order=True."""
+    operators walk (ptr_arr, idx) when called with own_order=True.  summed_backward: for the (col_ptr,
+    row_ind) arrays of the summed backward (GmmConvFuseSumTwoOrders), which keeps the caller's order on
+    graphs of low average degree."""
     require_cuda(ptr_arr, idx)
-    return edge_positions(as_i32(ptr_arr), as_i32(idx))
+    ptr_arr, idx = as_i32(ptr_arr), as_i32(idx)
+    if summed_backward and _plain_list_for_summed_backward(ptr_arr.numel() - 1, idx.numel()):
+        schedule_for(ptr_arr)
+        return None
+    return edge_positions(ptr_arr, idx)
 
 
 class GmmFuseSumTwoOrdersFunction(torch.autograd.Function):

@@ -70,7 +70,7 @@ def schedule_order_copies(g, pseudo):
     per-edge pipeline (projection, Gaussian weights, their gradients) can run in those orders and every
     pass streams its per-edge data instead of reaching it through a position map."""
     pos_r = gmm_edge_positions(g.row_ptr, g.col_ind)
-    pos_c = gmm_edge_positions(g.col_ptr, g.row_ind)
+    pos_c = gmm_edge_positions(g.col_ptr, g.row_ind, summed_backward=True)
     fwd = pseudo if pos_r is None else pseudo[pos_r.long()].contiguous()
     to_csc = g.permute.long() if pos_c is None else g.permute[pos_c.long()].long()
     return fwd, pseudo[to_csc].contiguous()

@@ -633,12 +633,14 @@ def test_gmm_layer_with_pseudo_in_schedule_order(k, dim, f, monkeypatch):
     from ae_mlsys_gnn_amd import _lib
     from ae_mlsys_gnn_amd.layers import GMMConv
     from ae_mlsys_gnn_amd.operators.fused_gmmconv import gmm_edge_positions
-    for buckets in ("1", "0"):
+    # 250 nodes: rows average 160 entries, both passes take an XCD-aware schedule; 600 nodes: 50 entries, the
+    # summed backward keeps the caller's order there
+    for buckets, n_nodes in (("1", 250), ("1", 600), ("0", 600)):
         monkeypatch.setenv("FGNN_XCD_BUCKETS", buckets)
         monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
         _lib.clear_schedule_cache()
         torch.manual_seed(4)
-        g = graphs.add_csc_torch(graphs.rmat_graph(600, 30000, seed=6))
+        g = graphs.add_csc_torch(graphs.rmat_graph(n_nodes, 30000 if n_nodes == 600 else 40000, seed=6))
         layer = GMMConv(24, f, dim=dim, n_kernels=k)
         feat, pseudo, go = torch.randn(g.n, 24), torch.rand(g.n_edges, dim), torch.randn(g.n, f)
         leaves = [t.detach().double().requires_grad_(True) for t in (layer.fc.weight, layer.mu, layer.inv_sigma, layer.bias, feat, pseudo)]
@@ -647,17 +649,18 @@ def test_gmm_layer_with_pseudo_in_schedule_order(k, dim, f, monkeypatch):
         gd = g.to(DEV)
         layer = layer.to(DEV)
         fd = feat.to(DEV).requires_grad_(True)
-        pos_r, pos_c = gmm_edge_positions(gd.row_ptr, gd.col_ind), gmm_edge_positions(gd.col_ptr, gd.row_ind)
-        if buckets == "0":
-            assert pos_r is None and pos_c is None
-            pos_r = pos_c = torch.arange(g.n_edges, device=DEV, dtype=torch.int32)
-        else:
-            for pos, ptr_arr in ((pos_r, g.row_ptr), (pos_c, g.col_ptr)):        # a permutation that stays inside every row
+        pos_r, pos_c = gmm_edge_positions(gd.row_ptr, gd.col_ind), gmm_edge_positions(gd.col_ptr, gd.row_ind, summed_backward=True)
+        assert (pos_r is None) == (buckets == "0") and (pos_c is None) == (buckets == "0" or n_nodes == 600)
+        for pos, ptr_arr in ((pos_r, g.row_ptr), (pos_c, g.col_ptr)):        # a permutation that stays inside every row
+            if pos is not None:
                 assert torch.equal(pos.long().sort().values.cpu(), torch.arange(g.n_edges))
                 row_of = torch.repeat_interleave(torch.arange(g.n), (ptr_arr[1:] - ptr_arr[:-1]).long())
                 assert torch.equal(row_of[pos.long().cpu()], row_of)
-            assert not torch.equal(pos_r.cpu(), torch.arange(g.n_edges, dtype=torch.int32))
+                assert not torch.equal(pos.cpu(), torch.arange(g.n_edges, dtype=torch.int32))
+        if pos_r is not None:
             assert torch.equal(gmm_edge_positions(gd.row_ptr, gd.col_ind), pos_r)           # asked again: same map
+        identity = torch.arange(g.n_edges, device=DEV, dtype=torch.int32)
+        pos_r, pos_c = identity if pos_r is None else pos_r, identity if pos_c is None else pos_c
         to_csc = gd.permute.long()[pos_c.long()]
         pd = pseudo.to(DEV)[pos_r.long()].contiguous()
         pc = pseudo.to(DEV)[to_csc].contiguous().requires_grad_(True)

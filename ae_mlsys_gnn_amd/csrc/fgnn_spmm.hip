@@ -613,6 +613,77 @@ __global__ __launch_bounds__(256) void gauss_grad_kernel(int64_t E, int K, int d
         red[(size_t)blockIdx.x * 2 * KD + i] = (wsum[i] + wsum[2 * KD + i]) + (wsum[4 * KD + i] + wsum[6 * KD + i]);
 }
 
+// The same derivatives for small mixtures (K <= 4, dim <= 3: the MoNet models), K and dim known at
+// compile time: mu and inv_sigma live in registers, a thread handles GG_EPT edges 256 apart and keeps
+// its partial mu / isg sums in registers, so the wave reductions run once per GG_EPT * 64 edges.
+#define GG_EPT 4
+template <int K, int DIM>
+__global__ __launch_bounds__(256) void gauss_grad_small_kernel(int64_t E, const float *__restrict__ pseudo, const float *__restrict__ mu,
+                                                               const float *__restrict__ isg, const float *__restrict__ src,
+                                                               int premultiplied, float *__restrict__ gp, float *__restrict__ red)
+{
+    constexpr int KD = K * DIM;
+    __shared__ float wsum[4][2 * KD];
+    float m[KD], s[KD], amu[KD], asg[KD];
+#pragma unroll
+    for (int i = 0; i < KD; ++i) { m[i] = mu[i]; s[i] = isg[i]; amu[i] = 0.f; asg[i] = 0.f; }
+    const int64_t base = (int64_t)blockIdx.x * (256 * GG_EPT) + threadIdx.x;
+#pragma unroll
+    for (int t = 0; t < GG_EPT; ++t) {
+        const int64_t e = base + t * 256;
+        if (e < E) {
+            float p[DIM], g[K], gpd[DIM];
+#pragma unroll
+            for (int d = 0; d < DIM; ++d) { p[d] = pseudo[e * DIM + d]; gpd[d] = 0.f; }
+#pragma unroll
+            for (int k = 0; k < K; ++k) g[k] = src[e * K + k];
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                float diff[DIM], acc = 0.f;
+#pragma unroll
+                for (int d = 0; d < DIM; ++d) {
+                    diff[d] = p[d] - m[k * DIM + d];
+                    const float u = diff[d] * s[k * DIM + d];
+                    acc = fmaf(u, u, acc);
+                }
+                float gww = g[k];
+                if (!premultiplied) gww *= __expf(-0.5f * acc);
+#pragma unroll
+                for (int d = 0; d < DIM; ++d) {
+                    const float sg = s[k * DIM + d];
+                    const float a = gww * diff[d] * sg;
+                    amu[k * DIM + d] += a * sg;
+                    asg[k * DIM + d] -= a * diff[d];
+                    gpd[d] = fmaf(-gww * diff[d], sg * sg, gpd[d]);
+                }
+            }
+#pragma unroll
+            for (int d = 0; d < DIM; ++d) gp[e * DIM + d] = gpd[d];
+        }
+    }
+    const int lane = fg_lane(), wave = fg_wave();
+#pragma unroll
+    for (int i = 0; i < KD; ++i) {
+        const float sm = fg_wave_sum(amu[i]), ss = fg_wave_sum(asg[i]);
+        if (lane == 0) { wsum[wave][i] = sm; wsum[wave][KD + i] = ss; }
+    }
+    __syncthreads();
+    for (int i = (int)threadIdx.x; i < 2 * KD; i += 256)
+        red[(size_t)blockIdx.x * 2 * KD + i] = (wsum[0][i] + wsum[1][i]) + (wsum[2][i] + wsum[3][i]);
+}
+
+template <int K>
+static bool gauss_grad_small_launch(int dim, int nblk, hipStream_t st, int64_t E, const float *pseudo, const float *mu, const float *isg,
+                                    const float *src, int premultiplied, float *gp, float *red)
+{
+    switch (dim) {
+    case 1: hipLaunchKernelGGL((gauss_grad_small_kernel<K, 1>), dim3(nblk), dim3(256), 0, st, E, pseudo, mu, isg, src, premultiplied, gp, red); return true;
+    case 2: hipLaunchKernelGGL((gauss_grad_small_kernel<K, 2>), dim3(nblk), dim3(256), 0, st, E, pseudo, mu, isg, src, premultiplied, gp, red); return true;
+    case 3: hipLaunchKernelGGL((gauss_grad_small_kernel<K, 3>), dim3(nblk), dim3(256), 0, st, E, pseudo, mu, isg, src, premultiplied, gp, red); return true;
+    default: return false;
+    }
+}
+
 // Column sums of red[rows, width] in two deterministic levels.
 __global__ __launch_bounds__(256) void colsum_level1(const float *red, int rows, int width, float *tmp /*[gridDim.x, width]*/)
 {
@@ -657,11 +728,24 @@ static int gauss_grad_launch(int64_t E, int K, int dim, const float *pseudo, con
         int rc = fgnn_fill_f32(gmu, KD, 0.f, st);
         return rc ? rc : fgnn_fill_f32(gsig, KD, 0.f, st);
     }
-    const int nblk = (int)((E + 255) / 256);
+    int nblk = (int)((E + 255) / 256);
     float *red = (float *)ws;
-    float *tmp = (float *)((char *)ws + fgnn_align256((size_t)nblk * 2 * KD * sizeof(float)));
-    size_t shm = (size_t)(2 * KD + 4 * 2 * KD) * sizeof(float);
-    hipLaunchKernelGGL(gauss_grad_kernel, dim3(nblk), dim3(256), shm, st, E, K, dim, pseudo, mu, isg, src, premultiplied, gp, red);
+    float *tmp = (float *)((char *)ws + fgnn_align256((size_t)nblk * 2 * KD * sizeof(float)));     // layout sized for one edge per thread
+    const int nblk_small = (int)((E + 256 * GG_EPT - 1) / (256 * GG_EPT));
+    bool small = false;
+    switch (K) {
+    case 1: small = gauss_grad_small_launch<1>(dim, nblk_small, st, E, pseudo, mu, isg, src, premultiplied, gp, red); break;
+    case 2: small = gauss_grad_small_launch<2>(dim, nblk_small, st, E, pseudo, mu, isg, src, premultiplied, gp, red); break;
+    case 3: small = gauss_grad_small_launch<3>(dim, nblk_small, st, E, pseudo, mu, isg, src, premultiplied, gp, red); break;
+    case 4: small = gauss_grad_small_launch<4>(dim, nblk_small, st, E, pseudo, mu, isg, src, premultiplied, gp, red); break;
+    default: break;
+    }
+    if (small) {
+        nblk = nblk_small;
+    } else {
+        size_t shm = (size_t)(2 * KD + 4 * 2 * KD) * sizeof(float);
+        hipLaunchKernelGGL(gauss_grad_kernel, dim3(nblk), dim3(256), shm, st, E, K, dim, pseudo, mu, isg, src, premultiplied, gp, red);
+    }
     int rc = fgnn_launch_status("gauss_grad_kernel");
     if (rc) return rc;
     hipLaunchKernelGGL(colsum_level1, dim3(kColsumBlocks), dim3(256), 0, st, red, nblk, 2 * KD, tmp);

@@ -173,13 +173,16 @@ def test_gmm_forward_backward(k, dim, f, variant, monkeypatch):
     assert_close(dl[3].grad, leaves[3].grad, "grad inv_sigma", rtol=1e-3, atol=1e-2)
 
 
-def test_gaussian_op():
+@pytest.mark.parametrize("e,k,dim", [(1000, 3, 2), (1, 1, 1), (1025, 2, 1), (5000, 4, 3), (3000, 5, 2), (2049, 2, 4), (700, 7, 5)])
+def test_gaussian_op(e, k, dim):
+    """GaussianCp and its closed-form backward: mixtures with K <= 4, dim <= 3 take the kernel specialised at
+    compile time (several edges per thread: edge counts around its 1024-edge blocks), the others the general one."""
     from ae_mlsys_gnn_amd.operators import fused_gmmconv as fg
-    gen = torch.Generator().manual_seed(3)
-    pseudo = torch.rand(1000, 2, generator=gen, dtype=torch.float64)
-    mu = torch.rand(3, 2, generator=gen, dtype=torch.float64)
-    isg = 0.5 + torch.rand(3, 2, generator=gen, dtype=torch.float64)
-    go = torch.randn(1000, 3, generator=gen, dtype=torch.float64)
+    gen = torch.Generator().manual_seed(3 + e)
+    pseudo = torch.rand(e, dim, generator=gen, dtype=torch.float64)
+    mu = torch.rand(k, dim, generator=gen, dtype=torch.float64)
+    isg = 0.5 + torch.rand(k, dim, generator=gen, dtype=torch.float64)
+    go = torch.randn(e, k, generator=gen, dtype=torch.float64)
     leaves = [t.clone().requires_grad_(True) for t in (pseudo, mu, isg)]
     ref = orc.gaussian(*leaves)
     ref.backward(go)

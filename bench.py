@@ -392,7 +392,7 @@ def run_gmm(args):
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "gmm_c4", "nodes": n, "edges": e, "K": kk, "dim": dim, "F": f},
         "roofline": roofline_record("spmm_kernel<WGauss>", b_f, ms_f, MEASURED_TRAFFIC_BYTES["gmm_c4"]["fwd"]),
-        "roofline_bwd": roofline_record("gmm_bwd_kernel + gauss_grad_kernel + column sums", b_b, ms_b, MEASURED_TRAFFIC_BYTES["gmm_c4"]["bwd"]),
+        "roofline_bwd": roofline_record("gmm_bwd_kernel + gauss_grad_small_kernel + column sums", b_b, ms_b, MEASURED_TRAFFIC_BYTES["gmm_c4"]["bwd"]),
         "fused_sum_over_kernels": {"fwd_ms": round(ms_fs, 4), "bwd_ms": round(ms_bs, 4)},
         "cpu_baseline": {"value": round(sorted(ts)[1], 1), "unit": "ms/iter", "cores": cores, "kind": "port",
                          "sample": "GMMConv_dgl composed math (torch CPU) fwd+bwd at full size, median of 3"},

@@ -286,6 +286,10 @@ extern "C" size_t fgnn_gmm_forward_workspace_bytes(const fgnn_schedule_t *sched,
     return fgnn_mhspmm_workspace_bytes(sched, K, F);
 }
 
+static int gmm_forward_shared(int N, int K, int dim, int F, const int32_t *ptr, const int32_t *idx, const int32_t *pos_map, const float *feat,
+                              const float *pseudo, const float *mu, const float *isg, float *out, const fgnn_schedule_t *sched,
+                              void *workspace, size_t workspace_bytes, hipStream_t st);
+
 extern "C" int fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F, const int32_t *ptr, const int32_t *idx,
                                 const int32_t *pos_map, const float *node_feat, const float *pseudo, const float *mu,
                                 const float *inv_sigma, float *out, float *gauss_out, int sum_kernels,
@@ -295,6 +299,12 @@ extern "C" int fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F, const i
     if (rc) return rc;
     FGNN_REQUIRE(dim >= 1 && dim <= 64 && K * dim <= 1024, FGNN_ERR_LIMIT, "fgnn_gmm_forward: dim=%d K*dim=%d unsupported", dim, K * dim);
     FGNN_REQUIRE(ptr && (idx || E == 0) && node_feat && (pseudo || E == 0) && mu && inv_sigma && out, FGNN_ERR_NULL, "fgnn_gmm_forward: NULL argument");
+    FGNN_REQUIRE(sum_kernels >= 0 && sum_kernels <= 2, FGNN_ERR_SHAPE, "fgnn_gmm_forward: sum_kernels=%d (0, 1 or 2)", sum_kernels);
+    if (sum_kernels == 2) {
+        FGNN_REQUIRE(!gauss_out, FGNN_ERR_SHAPE, "fgnn_gmm_forward: gauss_out is not available with shared node features");
+        return gmm_forward_shared(N, K, dim, F, ptr, idx, pos_map, node_feat, pseudo, mu, inv_sigma, out, sched, workspace, workspace_bytes,
+                                  (hipStream_t)stream);
+    }
     SpmmP p{};
     p.ptr = ptr; p.idx = idx; p.pos_map = pos_map; p.feat = node_feat; p.out = out; p.N = N; p.H = K; p.F = F; p.HF = K * F;
     p.sum_h = sum_kernels;
@@ -311,6 +321,7 @@ struct GmmBwdP {
     float *gfeat; float *gww; float *part;      // gww: [E,K] in CSR position order, gw * w per edge and kernel
     int N, K, dim, F, HF;
     int g_stride;   // floats per grad_out row: HF, or F when grad_out is the gradient of the sum over kernels
+    int x_stride;   // floats per node_feat row: HF, or F when all mixture kernels share one [N,F] feature matrix
     int lphp;       // > 0: head-aligned lane map with this many lanes per mixture kernel
 };
 
@@ -339,7 +350,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p)
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         T[r].zero();
-        if (FULL || lm.ok[r]) xr[r].load(p.x + (size_t)col * p.HF + lm.eoff[r]); else xr[r].zero();
+        if (FULL || lm.ok[r]) xr[r].load(p.x + (size_t)col * p.x_stride + (p.x_stride == p.HF ? lm.eoff[r] : lm.eoff[r] % p.F)); else xr[r].zero();
         goff[r] = (p.g_stride == p.HF) ? lm.eoff[r] : lm.eoff[r] % p.F;
     }
     for (int c = b; c < e; c += 64) {
@@ -422,7 +433,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_packed_kernel(GmmBwdP p)
     if (p.lphp) pm.init_padded(lane, p.K, p.F, p.lphp); else pm.init(lane, p.HF, p.F);
     fg_vec<4> T, xr;
     T.zero();
-    if (pm.ok) xr.load(p.x + (size_t)col * p.HF + pm.eoff); else xr.zero();
+    if (pm.ok) xr.load(p.x + (size_t)col * p.x_stride + (p.x_stride == p.HF ? pm.eoff : pm.eoff % p.F)); else xr.zero();
     const int goff = (p.g_stride == p.HF) ? pm.eoff : pm.eoff % p.F;
     const bool writer = pm.ok && pm.eoff % p.F == 0;
     constexpr int U = 8;
@@ -472,8 +483,11 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_packed_kernel(GmmBwdP p)
 // (LPF = lanes per row, a power of two >= F/4) and keep the K accumulators and the K slices of x[col]
 // in registers.  One load instruction then fetches 64/LPF different rows, every lane of it is used,
 // and a row is read once instead of once per mixture kernel.  K <= GMM_SUMK_MAX, F % 4 == 0, F <= 256.
+// With GWW == false the same loop is the forward of a layer whose K mixture kernels share one [N,F]
+// feature matrix (aggregate first, transform afterwards): out[i,k,:] = sum_p w[p,k] * g[idx[p],:], nothing
+// per edge is written and x is not read.
 #define GMM_SUMK_MAX 4
-template <int LPF>
+template <int LPF, bool GWW = true>
 __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_sum_kernel(GmmBwdP p)
 {
     extern __shared__ float lds[];
@@ -495,7 +509,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_sum_kernel(GmmBwdP p)
 #pragma unroll
     for (int k = 0; k < GMM_SUMK_MAX; ++k) {
         T[k].zero();
-        if (k < K && fok) xr[k].load(p.x + (size_t)col * p.HF + k * F + foff); else xr[k].zero();
+        if (GWW && k < K && fok) xr[k].load(p.x + (size_t)col * p.HF + k * F + foff); else xr[k].zero();
     }
     for (int c = b; c < e; c += 64) {
         int q = c + lane;
@@ -530,13 +544,15 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_sum_kernel(GmmBwdP p)
                     if (k < K) {
                         const float w = wl[k * 64 + ei];            // 0 past the end of the chunk
                         T[k].fma(w, ld[u]);
-                        const float sum = fg_group_sum<LPF>(ld[u].dot(xr[k]));
-                        if constexpr (LPF >= GMM_SUMK_MAX) mine = sub == k ? sum * w : mine;
-                        else if (ei < cnt && sub == 0) gdst[k] = sum * w;
+                        if constexpr (GWW) {
+                            const float sum = fg_group_sum<LPF>(ld[u].dot(xr[k]));
+                            if constexpr (LPF >= GMM_SUMK_MAX) mine = sub == k ? sum * w : mine;
+                            else if (ei < cnt && sub == 0) gdst[k] = sum * w;
+                        }
                     }
                 }
                 // the K values of an edge leave with one store instruction, K adjacent lanes writing K adjacent floats
-                if constexpr (LPF >= GMM_SUMK_MAX) { if (ei < cnt && sub < K) gdst[sub] = mine; }
+                if constexpr (GWW && LPF >= GMM_SUMK_MAX) { if (ei < cnt && sub < K) gdst[sub] = mine; }
             }
         }
         fg_wave_lds_sync();
@@ -549,6 +565,62 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_sum_kernel(GmmBwdP p)
             if (fok && grp == 0) T[k].store_nt(dst + k * F + foff);
         }
     }
+}
+
+template <bool GWW>
+static void gmm_sum_launch(int lpf, unsigned grid, size_t shm, hipStream_t st, const GmmBwdP &p)
+{
+    switch (lpf) {
+    case 1: hipLaunchKernelGGL((gmm_bwd_sum_kernel<1, GWW>), dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
+    case 2: hipLaunchKernelGGL((gmm_bwd_sum_kernel<2, GWW>), dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
+    case 4: hipLaunchKernelGGL((gmm_bwd_sum_kernel<4, GWW>), dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
+    case 8: hipLaunchKernelGGL((gmm_bwd_sum_kernel<8, GWW>), dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
+    case 16: hipLaunchKernelGGL((gmm_bwd_sum_kernel<16, GWW>), dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
+    case 32: hipLaunchKernelGGL((gmm_bwd_sum_kernel<32, GWW>), dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
+    default: hipLaunchKernelGGL((gmm_bwd_sum_kernel<64, GWW>), dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
+    }
+}
+
+// Forward with one [N,F] feature matrix shared by the K mixture kernels: out[i,k,:] = sum_p w[p,k] * feat[idx[p],:].
+static int gmm_forward_shared(int N, int K, int dim, int F, const int32_t *ptr, const int32_t *idx, const int32_t *pos_map, const float *feat,
+                              const float *pseudo, const float *mu, const float *isg, float *out, const fgnn_schedule_t *sched,
+                              void *workspace, size_t workspace_bytes, hipStream_t st)
+{
+    const int HF = K * F, KD = K * dim;
+    FGNN_REQUIRE(F % 4 == 0 && F <= 256 && K <= GMM_SUMK_MAX && fgnn_aligned16(feat) && fgnn_aligned16(out), FGNN_ERR_LIMIT,
+                 "fgnn_gmm_forward: shared node features need F %% 4 == 0, F <= 256, K <= %d and 16-byte aligned tensors (F=%d, K=%d)",
+                 GMM_SUMK_MAX, F, K);
+    if (sched && sched->n_partials > 0) {
+        size_t need = (size_t)sched->n_partials * spmm_pw(HF) * sizeof(float);
+        FGNN_REQUIRE(workspace && workspace_bytes >= need && fgnn_aligned16(workspace), FGNN_ERR_WORKSPACE,
+                     "fgnn_gmm_forward: workspace %zu < %zu bytes (or unaligned)", workspace_bytes, need);
+    }
+    GmmBwdP p{};
+    p.items = sched ? sched->items_dev : nullptr; p.n_items = sched ? sched->n_items : N;
+    if (p.n_items == 0) return 0;
+    p.ptr = ptr; p.idx = fgnn_sched_idx(sched, idx); p.pos = fgnn_sched_pos(sched); p.permute = pos_map;
+    p.g = feat; p.pseudo = pseudo; p.mu = mu; p.isg = isg; p.gfeat = out; p.part = (float *)workspace;
+    p.N = N; p.K = K; p.dim = dim; p.F = F; p.HF = HF; p.g_stride = F; p.x_stride = HF;
+    int lpf = 1;
+    while (lpf * 4 < F) lpf *= 2;
+    const size_t shm = ((size_t)FGNN_WPB * K * 64 + 2 * KD) * sizeof(float);
+    FGNN_REQUIRE(shm <= 64 * 1024, FGNN_ERR_LIMIT, "fgnn_gmm_forward: K=%d, dim=%d need %zu bytes of LDS per workgroup (limit 64 KiB)", K, dim, shm);
+    const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
+    gmm_sum_launch<false>(lpf, grid, shm, st, p);
+    int rc = fgnn_launch_status("gmm_bwd_sum_kernel (forward, shared features)");
+    if (rc) return rc;
+    if (sched && sched->n_split > 0) {
+        fgnn_rowcfg cfg;
+        FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, true, &cfg), FGNN_ERR_LIMIT, "fgnn_gmm_forward: unsupported row width %d", HF);
+        SpmmP mp{};
+        mp.part = p.part; mp.out = out; mp.N = N; mp.H = K; mp.F = F; mp.HF = HF;
+        unsigned g2 = (unsigned)((sched->n_split + FGNN_WPB - 1) / FGNN_WPB);
+        rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
+            hipLaunchKernelGGL((spmm_merge_kernel<VEC, R>), dim3(g2), dim3(FGNN_TPB), 0, st, mp, sched->split_dev, sched->n_split);
+            return fgnn_launch_status("spmm_merge_kernel");
+        });
+    }
+    return rc;
 }
 
 // Closed-form derivatives of w[p,k] = exp(-0.5 sum_d ((pseudo[p,d]-mu[k,d])*isg[k,d])^2), one edge per
@@ -778,6 +850,7 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
                      grad_out && grad_feat && (grad_pseudo || E == 0) && grad_mu && grad_sigma,
                  FGNN_ERR_NULL, "fgnn_gmm_backward: NULL argument");
     FGNN_REQUIRE(sched_csc, FGNN_ERR_SCHEDULE, "fgnn_gmm_backward: a schedule of col_ptr is required");
+    FGNN_REQUIRE(sum_kernels >= 0 && sum_kernels <= 2, FGNN_ERR_SHAPE, "fgnn_gmm_backward: sum_kernels=%d (0, 1 or 2)", sum_kernels);
     size_t need = fgnn_gmm_backward_workspace_bytes(sched_csc, K, dim, F);
     FGNN_REQUIRE(workspace && workspace_bytes >= need && fgnn_aligned16(workspace), FGNN_ERR_WORKSPACE,
                  "fgnn_gmm_backward: workspace %zu < %zu bytes (or unaligned)", workspace_bytes, need);
@@ -795,7 +868,9 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
         p.items = sched_csc->items_dev; p.n_items = sched_csc->n_items; p.ptr = col_ptr; p.idx = fgnn_sched_idx(sched_csc, row_ind);
         p.pos = fgnn_sched_pos(sched_csc); p.permute = permute;
         p.x = node_feat; p.g = grad_out; p.pseudo = pseudo; p.mu = mu; p.isg = inv_sigma; p.gfeat = grad_feat; p.gww = gww;
-        p.part = part; p.N = N; p.K = K; p.dim = dim; p.F = F; p.HF = HF; p.g_stride = sum_kernels ? F : HF;
+        p.part = part; p.N = N; p.K = K; p.dim = dim; p.F = F; p.HF = HF;
+        p.g_stride = sum_kernels == 1 ? F : HF;
+        p.x_stride = sum_kernels == 2 ? F : HF;
         // widths like 44 or 48 (quarter not a power of two): head-aligned lane map, so the per-edge dot
         // products still reduce with DPP and narrow rows still pack
         p.lphp = fgnn_pad_lph(cfg.vec, K, F);
@@ -807,7 +882,7 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
         }
         const int lph = p.lphp ? p.lphp : fgnn_pick_lph(cfg.vec, F);
         const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
-        const bool sumk = sum_kernels && cfg.vec == 4 && F % 4 == 0 && F <= 256 && K <= GMM_SUMK_MAX;
+        const bool sumk = sum_kernels == 1 && cfg.vec == 4 && F % 4 == 0 && F <= 256 && K <= GMM_SUMK_MAX;
         rc = sumk ? 0 : 1;
         if (sumk) {
             // lanes over F only, the K mixture kernels in registers (see gmm_bwd_sum_kernel)
@@ -816,15 +891,7 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
             const size_t shm = ((size_t)FGNN_WPB * K * 64 + 2 * KD) * sizeof(float);
             FGNN_REQUIRE(shm <= 64 * 1024, FGNN_ERR_LIMIT, "fgnn_gmm_backward: K=%d, dim=%d need %zu bytes of LDS per workgroup (limit 64 KiB)", K, dim, shm);
             p.lphp = 0;
-            switch (lpf) {
-            case 1: hipLaunchKernelGGL(gmm_bwd_sum_kernel<1>, dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
-            case 2: hipLaunchKernelGGL(gmm_bwd_sum_kernel<2>, dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
-            case 4: hipLaunchKernelGGL(gmm_bwd_sum_kernel<4>, dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
-            case 8: hipLaunchKernelGGL(gmm_bwd_sum_kernel<8>, dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
-            case 16: hipLaunchKernelGGL(gmm_bwd_sum_kernel<16>, dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
-            case 32: hipLaunchKernelGGL(gmm_bwd_sum_kernel<32>, dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
-            default: hipLaunchKernelGGL(gmm_bwd_sum_kernel<64>, dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
-            }
+            gmm_sum_launch<true>(lpf, grid, shm, st, p);
             rc = fgnn_launch_status("gmm_bwd_sum_kernel");
             if (rc) return rc;
             if (sched_csc->n_split > 0) {

@@ -6,7 +6,8 @@ import torch as th
 from torch import nn
 from torch.nn import init
 
-from ..operators.fused_gmmconv import GmmConvFuseSum, GmmConvFuseSumTwoOrders, GmmConvStash
+from ..operators.fused_gmmconv import (GmmAggregate, GmmAggregateTwoOrders, GmmConvFuseSum, GmmConvFuseSumTwoOrders, GmmConvStash,
+                                        gmm_native)
 from .dense import add_bias, tall_linear
 
 
@@ -55,6 +56,8 @@ class _GMMBase(nn.Module):
         and the gradient of the pseudo-coordinates flows through pseudo_csc instead of pseudo.
         own_order (GMMConv only): pseudo and pseudo_csc are in the entry order of the operators' schedules
         (operators.fused_gmmconv.gmm_edge_positions); without pseudo_csc the layer is forward-only."""
+        if self._aggregate_first(feat):
+            return self._finish(self._forward_aggregate_first(rowptr, colind, colptr, rowind, permute, feat, pseudo, pseudo_csc, own_order), feat)
         node_feat = tall_linear(feat, self.fc.weight).view(-1, self._n_kernels, self._out_feats)    # = self.fc(feat)
         pad = (-self._out_feats) % 4
         if pad:         # zero columns up to a multiple of 4: the operator then takes its 128-bit row layout
@@ -70,11 +73,36 @@ class _GMMBase(nn.Module):
             rst = type(self)._op(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, self.mu, self.inv_sigma)
         if pad:
             rst = rst[..., :self._out_feats]
+        return self._finish(rst, feat)
+
+    def _finish(self, rst, feat):
         if self.res_fc is not None:
             rst = rst + self.res_fc(feat)
         if self.bias is not None:
             rst = add_bias(rst, self.bias)
         return rst
+
+    def _aggregate_first(self, feat):
+        """Whether the layer aggregates its input before the fc (recomputing layer only): when the input is
+        narrower than the K x out floats an edge would gather otherwise, and the operator takes the shape."""
+        k, fin = self._n_kernels, feat.shape[1]
+        return (type(self)._op is GmmConvFuseSum and feat.dim() == 2 and fin < k * self._out_feats
+                and gmm_native.shared_supported(k, fin))
+
+    def _forward_aggregate_first(self, rowptr, colind, colptr, rowind, permute, feat, pseudo, pseudo_csc, own_order):
+        """sum_k (sum_p w[p,k] feat[col(p),:]) @ W_k: the reference's sum over k of the aggregated fc(feat)[:,k,:]
+        (layers/gmmconv_layer.py:67-69) with the two linear steps exchanged."""
+        k, fin, fout = self._n_kernels, feat.shape[1], self._out_feats
+        feat = feat.contiguous()
+        if pseudo_csc is not None or own_order:
+            if own_order and pseudo_csc is None and th.is_grad_enabled() and (feat.requires_grad or pseudo.requires_grad):
+                raise ValueError("own_order without pseudo_csc is forward-only")
+            agg = GmmAggregateTwoOrders(rowptr, colind, colptr, rowind, feat, pseudo.detach(), pseudo_csc, self.mu, self.inv_sigma,
+                                        own_order=own_order)
+        else:
+            agg = GmmAggregate(rowptr, colind, colptr, rowind, permute, feat, pseudo, self.mu, self.inv_sigma)
+        w = self.fc.weight.view(k, fout, fin).permute(1, 0, 2).reshape(fout, k * fin)       # [out, K*in]: rst = agg.view(N, K*in) @ w^T
+        return tall_linear(agg.view(-1, k * fin), w)
 
 
 class GMMConv(_GMMBase):

@@ -66,6 +66,62 @@ class gmm_native:
         return grad_feat, grad_pseudo, grad_mu, grad_sigma
 
     @staticmethod
+    def shared_supported(k, f):
+        """Shapes the shared-feature (aggregate first) entry points take: the [N,f] rows as 128-bit slabs over
+        at most a wave, the K accumulators in registers."""
+        return f % 4 == 0 and 0 < f <= 256 and 0 < k <= 4
+
+    @staticmethod
+    def gmmconv_shared(rowptr, colind, feat, pseudo, mu, sigma, *, pos_map=None, own_order=False):
+        """out[i,k,:] = sum_p w[p,k] * feat[colind[p],:] for one [N,F] feature matrix shared by the K mixture
+        kernels (the reference's gmmconv with node_feat[:,k,:] == feat for every k).  Returns [N,K,F]."""
+        require_cuda(rowptr, colind, feat, pseudo, mu, sigma)
+        rowptr, colind = as_i32(rowptr), as_i32(colind)
+        feat, pseudo, mu, sigma = as_f32(feat), as_f32(pseudo), as_f32(mu), as_f32(sigma)
+        if feat.dim() != 2:
+            raise FgnnError("feat must be [N,F], got %s" % (tuple(feat.shape),))
+        n, f = feat.shape
+        k, dim = mu.shape
+        e = colind.numel()
+        if sigma.shape != (k, dim) or pseudo.shape != (e, dim) or rowptr.numel() != n + 1:
+            raise FgnnError("gmmconv_shared: shape mismatch mu %s sigma %s pseudo %s for E=%d" % (
+                tuple(mu.shape), tuple(sigma.shape), tuple(pseudo.shape), e))
+        out = torch.empty((n, k, f), dtype=torch.float32, device=feat.device)
+        sched = schedule_for(rowptr, idx_tensor=colind, own_order=own_order)
+        with torch.cuda.device(feat.device):
+            ws, wsb = workspace(lib().fgnn_gmm_forward_workspace_bytes(sched.handle, k, f), feat.device)
+            check(lib().fgnn_gmm_forward(n, e, k, dim, f, ptr(rowptr), ptr(colind), ptr(pos_map), ptr(feat), ptr(pseudo),
+                                         ptr(mu), ptr(sigma), ptr(out), None, 2, sched.handle, ptr(ws), wsb, stream_ptr()),
+                  "fgnn_gmm_forward (shared features)")
+        return out
+
+    @staticmethod
+    def gmmconv_shared_backward(colptr, rowind, permute, feat, pseudo, mu, sigma, grad_out, own_order=False):
+        """Backward of gmmconv_shared for grad_out [N,K,F]: (grad_feat [N,F], grad_pseudo, grad_mu, grad_sigma)."""
+        require_cuda(colptr, rowind, permute, feat, pseudo, mu, sigma, grad_out)
+        colptr, rowind = as_i32(colptr), as_i32(rowind)
+        permute = None if permute is None else as_i32(permute)
+        grad_out = as_f32(grad_out)
+        n, f = feat.shape
+        k, dim = mu.shape
+        e = rowind.numel()
+        dev = feat.device
+        if grad_out.shape != (n, k, f):
+            raise FgnnError("gmmconv_shared_backward: grad_out is %s, expected (%d, %d, %d)" % (tuple(grad_out.shape), n, k, f))
+        parts = torch.empty((n, k, f), dtype=torch.float32, device=dev)      # kernel k's share of grad_feat
+        grad_pseudo = torch.empty((e, dim), dtype=torch.float32, device=dev)
+        grad_mu = torch.empty_like(mu)
+        grad_sigma = torch.empty_like(sigma)
+        # same work list as the summed backward, so that one CSC-side copy of own-order edge data serves both kinds of layer
+        sched = schedule_for(colptr, idx_tensor=None if _plain_list_for_summed_backward(n, e) else rowind, own_order=own_order)
+        with torch.cuda.device(dev):
+            ws, wsb = workspace(lib().fgnn_gmm_backward_workspace_bytes(sched.handle, k, dim, f), dev)
+            check(lib().fgnn_gmm_backward(n, e, k, dim, f, ptr(colptr), ptr(rowind), ptr(permute), ptr(feat), ptr(pseudo),
+                                          ptr(mu), ptr(sigma), ptr(grad_out), 2, ptr(parts), ptr(grad_pseudo), ptr(grad_mu),
+                                          ptr(grad_sigma), sched.handle, ptr(ws), wsb, stream_ptr()), "fgnn_gmm_backward (shared features)")
+        return parts.sum(1), grad_pseudo, grad_mu, grad_sigma
+
+    @staticmethod
     def Gaussian(pseudo, mu, sigma):
         require_cuda(pseudo, mu, sigma)
         pseudo, mu, sigma = as_f32(pseudo), as_f32(mu), as_f32(sigma)
@@ -134,8 +190,8 @@ def GmmConvFuseSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo_cs
 def gmm_edge_positions(ptr_arr, idx, summed_backward=False):
     """int32 [E] (or None = identity): caller's position of every entry in the order in which the GMMConv
     operators walk (ptr_arr, idx) when called with own_order=True.  summed_backward: for the (col_ptr,
-    row_ind) arrays of the summed backward (GmmConvFuseSumTwoOrders), which keeps the caller's order on
-    graphs of low average degree."""
+    row_ind) arrays of the layers' backward passes (GmmConvFuseSumTwoOrders, GmmAggregateTwoOrders), which
+    keep the caller's order on graphs of low average degree."""
     require_cuda(ptr_arr, idx)
     ptr_arr, idx = as_i32(ptr_arr), as_i32(idx)
     if summed_backward and _plain_list_for_summed_backward(ptr_arr.numel() - 1, idx.numel()):
@@ -157,6 +213,53 @@ class GmmFuseSumTwoOrdersFunction(torch.autograd.Function):
         colptr, rowind, node_feat, pseudo_csc, mu, sigma = ctx.saved_tensors
         grad_feat, grad_pseudo_csc, grad_mu, grad_sigma = gmm_native.gmmconv_backward(
             colptr, rowind, None, node_feat, pseudo_csc, mu, sigma, grad_out.contiguous(), sum_kernels=True, own_order=ctx.own_order)
+        return None, None, None, None, grad_feat, None, grad_pseudo_csc, grad_mu, grad_sigma, None
+
+
+def GmmAggregate(rowptr, colind, colptr, rowind, permute, feat, pseudo, mu, sigma):
+    """Aggregate first: agg[i,k,:] = sum_p w[p,k] * feat[colind[p],:] for feat [N,F] -> [N,K,F].  A GMMConv
+    layer whose input is narrower than K x its output multiplies by the fc weights afterwards
+    (sum_k agg[:,k,:] @ W_k equals the reference's sum over k of the aggregated fc(feat)[:,k,:]), so an
+    edge gathers F floats instead of K x out."""
+    return GmmAggregateFunction.apply(rowptr, colind, colptr, rowind, permute, feat, pseudo, mu, sigma)
+
+
+class GmmAggregateFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, rowptr, colind, colptr, rowind, permute, feat, pseudo, mu, sigma):
+        out = gmm_native.gmmconv_shared(rowptr, colind, feat, pseudo, mu, sigma)
+        ctx.save_for_backward(colptr, rowind, permute, feat, pseudo, mu, sigma)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        colptr, rowind, permute, feat, pseudo, mu, sigma = ctx.saved_tensors
+        grad_feat, grad_pseudo, grad_mu, grad_sigma = gmm_native.gmmconv_shared_backward(
+            colptr, rowind, permute, feat, pseudo, mu, sigma, grad_out.contiguous())
+        return None, None, None, None, None, grad_feat, grad_pseudo, grad_mu, grad_sigma
+
+
+def GmmAggregateTwoOrders(rowptr, colind, colptr, rowind, feat, pseudo_csr, pseudo_csc, mu, sigma, own_order=False):
+    """GmmAggregate for a caller that has the pseudo-coordinates in both edge orders (see
+    GmmConvFuseSumTwoOrders; pseudo_csc None: forward only)."""
+    if pseudo_csc is None:
+        return gmm_native.gmmconv_shared(rowptr, colind, feat, pseudo_csr, mu, sigma, own_order=own_order)
+    return GmmAggregateTwoOrdersFunction.apply(rowptr, colind, colptr, rowind, feat, pseudo_csr, pseudo_csc, mu, sigma, own_order)
+
+
+class GmmAggregateTwoOrdersFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, rowptr, colind, colptr, rowind, feat, pseudo_csr, pseudo_csc, mu, sigma, own_order):
+        out = gmm_native.gmmconv_shared(rowptr, colind, feat, pseudo_csr, mu, sigma, own_order=own_order)
+        ctx.save_for_backward(colptr, rowind, feat, pseudo_csc, mu, sigma)
+        ctx.own_order = own_order
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        colptr, rowind, feat, pseudo_csc, mu, sigma = ctx.saved_tensors
+        grad_feat, grad_pseudo_csc, grad_mu, grad_sigma = gmm_native.gmmconv_shared_backward(
+            colptr, rowind, None, feat, pseudo_csc, mu, sigma, grad_out.contiguous(), own_order=ctx.own_order)
         return None, None, None, None, grad_feat, None, grad_pseudo_csc, grad_mu, grad_sigma, None
 
 

@@ -155,8 +155,13 @@ int fgnn_knn_graph(int n_clouds, int P, int D, int k, const float *points, int32
  * pseudo [E,dim] is in the position order of (ptr, idx); when pos_map is non-NULL the row
  * pseudo[pos_map[p]] is used instead (lets a CSC pass read CSR-ordered pseudo without the
  * mhtranspose copy of operators/fused_gmmconv.py:55).  gauss_out [E,K] optional.
- * sum_kernels != 0 fuses the layer's `.sum(1)` (layers/gmmconv_layer.py:69) into the store:
- * out is then [N,F] = sum_k out[i,k,:]. */
+ * sum_kernels == 1 fuses the layer's `.sum(1)` (layers/gmmconv_layer.py:69) into the store:
+ * out is then [N,F] = sum_k out[i,k,:].
+ * sum_kernels == 2: node_feat is ONE [N,F] matrix shared by the K kernels (node_feat[j,k,:] == node_feat[j,:]
+ * for every k), out stays [N,K,F].  A layer whose input is narrower than K x its output aggregates the
+ * input this way and multiplies by the fc weights afterwards, which is the same sum with the two linear
+ * steps exchanged; an edge then gathers F floats instead of K x out.  Needs F % 4 == 0, F <= 256, K <= 4,
+ * gauss_out == NULL (FGNN_ERR_LIMIT / FGNN_ERR_SHAPE otherwise). */
 size_t fgnn_gmm_forward_workspace_bytes(const fgnn_schedule_t *sched, int K, int F);
 int    fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F,
                         const int32_t *ptr, const int32_t *idx, const int32_t *pos_map,
@@ -176,8 +181,10 @@ int    fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F,
  * elementwise function of constant edge data) thereby avoids the per-edge gather and scatter through
  * permute, which is most of this pass on large graphs. */
 size_t fgnn_gmm_backward_workspace_bytes(const fgnn_schedule_t *sched_csc, int K, int dim, int F);
-/* sum_kernels != 0: grad_out is [N,F], the gradient of the fused sum over kernels (every kernel of a
- * node sees the same row, so the pass gathers F instead of K*F floats per edge). */
+/* sum_kernels == 1: grad_out is [N,F], the gradient of the fused sum over kernels (every kernel of a
+ * node sees the same row, so the pass gathers F instead of K*F floats per edge).
+ * sum_kernels == 2: node_feat is [N,F], shared by the K kernels (see fgnn_gmm_forward); grad_out is [N,K,F]
+ * and grad_feat [N,K,F] receives kernel k's share in slice k: the gradient of node_feat is their sum over k. */
 int    fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F,
                          const int32_t *col_ptr, const int32_t *row_ind, const int32_t *permute,
                          const float *node_feat, const float *pseudo, const float *mu,

@@ -173,6 +173,41 @@ def test_gmm_forward_backward(k, dim, f, variant, monkeypatch):
     assert_close(dl[3].grad, leaves[3].grad, "grad inv_sigma", rtol=1e-3, atol=1e-2)
 
 
+@pytest.mark.parametrize("k,dim,f", [(2, 1, 16), (3, 2, 64), (4, 3, 32), (1, 1, 128), (2, 2, 256), (3, 2, 4), (2, 1, 44), (4, 1, 100), (1, 2, 8)])
+def test_gmm_aggregate_shared_features(k, dim, f, monkeypatch):
+    """GmmAggregate: one [N,F] feature matrix shared by the K mixture kernels (the aggregate-first form of the
+    layers).  Oracle: the reference operator on the features repeated K times; its gradient summed over the
+    copies.  Degrees 0..3000 with split rows, plain and XCD-aware schedules; unsupported shapes are refused."""
+    from ae_mlsys_gnn_amd.operators import fused_gmmconv as fg
+    from ae_mlsys_gnn_amd import _lib
+    g = graphs.add_csc_torch(degree_edge_graph(n=400, seed=k + f))
+    x, pseudo, mu, isg, go = _gmm_case(g, k, dim, f, seed=2)
+    x = x[:, 0, :].contiguous()
+    leaves = [t.clone().requires_grad_(True) for t in (x, pseudo, mu, isg)]
+    ref = orc.gmm_forward(g.row_ptr, g.col_ind, leaves[0].unsqueeze(1).expand(-1, k, -1), *leaves[1:])
+    ref.backward(go)
+    gd = g.to(DEV)
+    for buckets in ("0", "1"):
+        monkeypatch.setenv("FGNN_SEG_LEN", "256")
+        monkeypatch.setenv("FGNN_XCD_BUCKETS", buckets)
+        monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+        _lib.clear_schedule_cache()
+        dl = [t.float().to(DEV).requires_grad_(True) for t in (x, pseudo, mu, isg)]
+        out = fg.GmmAggregate(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, *dl)
+        assert out.shape == (g.n, k, f)
+        out.backward(go.float().to(DEV))
+        assert_close(out, ref.detach(), "aggregate out (buckets %s)" % buckets, atol=1e-5)
+        assert_close(dl[0].grad, leaves[0].grad, "grad feat", atol=1e-4)
+        assert_close(dl[1].grad, leaves[1].grad, "grad pseudo", atol=1e-4)
+        assert_close(dl[2].grad, leaves[2].grad, "grad mu", rtol=1e-3, atol=1e-2)
+        assert_close(dl[3].grad, leaves[3].grad, "grad inv_sigma", rtol=1e-3, atol=1e-2)
+    _lib.clear_schedule_cache()
+    assert not fg.gmm_native.shared_supported(5, 16) and not fg.gmm_native.shared_supported(2, 18) and not fg.gmm_native.shared_supported(2, 260)
+    with pytest.raises(_lib.FgnnError, match="shared node features"):
+        fg.gmm_native.gmmconv_shared(gd.row_ptr, gd.col_ind, torch.zeros(g.n, 18, device=DEV), torch.zeros(g.n_edges, 1, device=DEV),
+                                     torch.zeros(2, 1, device=DEV), torch.ones(2, 1, device=DEV))
+
+
 @pytest.mark.parametrize("e,k,dim", [(1000, 3, 2), (1, 1, 1), (1025, 2, 1), (5000, 4, 3), (3000, 5, 2), (2049, 2, 4), (700, 7, 5)])
 def test_gaussian_op(e, k, dim):
     """GaussianCp and its closed-form backward: mixtures with K <= 4, dim <= 3 take the kernel specialised at
@@ -195,17 +230,22 @@ def test_gaussian_op(e, k, dim):
     assert_close(dl[2].grad, leaves[2].grad, "grad sigma", rtol=1e-3, atol=1e-3)
 
 
-@pytest.mark.parametrize("fout,k,dim,variant", [(16, 3, 2, "our"), (41, 2, 1, "our"), (7, 3, 2, "stash"), (16, 2, 3, "stash")])
-def test_gmm_layer_matches_dgl_composed(fout, k, dim, variant):
+@pytest.mark.parametrize("fin,fout,k,dim,variant,agg_first", [(32, 16, 3, 2, "our", True), (32, 41, 2, 1, "our", True), (16, 24, 2, 1, "our", True),
+                                                               (100, 16, 2, 1, "our", False), (30, 41, 2, 1, "our", False), (32, 7, 5, 2, "our", False),
+                                                               (32, 7, 3, 2, "stash", False), (32, 16, 2, 3, "stash", False)])
+def test_gmm_layer_matches_dgl_composed(fin, fout, k, dim, variant, agg_first):
     """Output and the gradients of the input, the pseudo-coordinates and every parameter against
-    autograd through the float64 DGL-composed layer; odd widths go through the layer's zero padding."""
+    autograd through the float64 DGL-composed layer; odd widths go through the layer's zero padding.
+    The recomputing layer aggregates its input before the fc when the input is narrower than K x out
+    (and the operator takes the shape); the other cases transform first, as the reference does."""
     from ae_mlsys_gnn_amd.layers import GMMConv, GMMConv_stash
     torch.manual_seed(1)
     g = graphs.add_csc_torch(graphs.rmat_graph(500, 6000, seed=2))
-    layer = (GMMConv if variant == "our" else GMMConv_stash)(32, fout, dim=dim, n_kernels=k, residual=True, bias=True)
+    layer = (GMMConv if variant == "our" else GMMConv_stash)(fin, fout, dim=dim, n_kernels=k, residual=True, bias=True)
     with torch.no_grad():
         layer.bias.normal_()
-    feat = torch.randn(g.n, 32)
+    feat = torch.randn(g.n, fin)
+    assert layer._aggregate_first(feat) == agg_first
     pseudo = torch.rand(g.n_edges, dim)
     go = torch.randn(g.n, fout)
     params = [layer.fc.weight, layer.mu, layer.inv_sigma, layer.bias, layer.res_fc.weight]

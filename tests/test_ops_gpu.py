@@ -202,6 +202,15 @@ def test_gmm_aggregate_shared_features(k, dim, f, monkeypatch):
         assert_close(dl[2].grad, leaves[2].grad, "grad mu", rtol=1e-3, atol=1e-2)
         assert_close(dl[3].grad, leaves[3].grad, "grad inv_sigma", rtol=1e-3, atol=1e-2)
     _lib.clear_schedule_cache()
+    # through the C ABI without a schedule (one wave per row)
+    direct = torch.empty(g.n, k, f, device=DEV)
+    dl = [t.float().to(DEV) for t in (x, pseudo, mu, isg)]
+    _lib.check(_lib.lib().fgnn_gmm_forward(g.n, g.n_edges, k, dim, f, _lib.ptr(gd.row_ptr), _lib.ptr(gd.col_ind), None, _lib.ptr(dl[0]),
+                                            _lib.ptr(dl[1]), _lib.ptr(dl[2]), _lib.ptr(dl[3]), _lib.ptr(direct), None, 2, None, None, 0,
+                                            _lib.stream_ptr()), "fgnn_gmm_forward")
+    torch.cuda.synchronize()
+    # rows of up to 3000 entries summed by one wave in one go: the absolute bar of the summed variants
+    assert_close(direct, ref.detach(), "aggregate out (no schedule)", atol=1e-4)
     assert not fg.gmm_native.shared_supported(5, 16) and not fg.gmm_native.shared_supported(2, 18) and not fg.gmm_native.shared_supported(2, 260)
     with pytest.raises(_lib.FgnnError, match="shared node features"):
         fg.gmm_native.gmmconv_shared(gd.row_ptr, gd.col_ind, torch.zeros(g.n, 18, device=DEV), torch.zeros(g.n_edges, 1, device=DEV),

@@ -747,6 +747,18 @@ def test_schedule_take_positions_c_abi(monkeypatch):
         _lib.Schedule(g.row_ptr, 0, g.col_ind, 16, with_positions=False).take_positions()
     plain = _lib.Schedule(g.row_ptr, 0)
     assert torch.equal(plain.take_positions().cpu(), torch.arange(g.n_edges, dtype=torch.int32))
+    # the cached own-order schedule exists only after edge_positions was asked for
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
+    _lib.clear_schedule_cache()
+    with pytest.raises(_lib.FgnnError, match="edge_positions"):
+        _lib.schedule_for(g.row_ptr, idx_tensor=g.col_ind, own_order=True)
+    again = _lib.edge_positions(g.row_ptr, g.col_ind)
+    assert _lib.schedule_for(g.row_ptr, idx_tensor=g.col_ind, own_order=True).own_order
+    assert _lib.schedule_for(g.row_ptr, idx_tensor=g.col_ind) is not _lib.schedule_for(g.row_ptr, idx_tensor=g.col_ind, own_order=True)
+    monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+    _lib.clear_schedule_cache()
+    assert torch.equal(_lib.edge_positions(g.row_ptr, g.col_ind), pos) and again.numel() == g.n_edges
+    _lib.clear_schedule_cache()
     # the operator under the own-order schedule: weights permuted by `pos` give the caller-order result
     torch.manual_seed(1)
     h, f = 2, 16

@@ -45,8 +45,8 @@ class _ProjectScores(torch.autograd.Function):
     """The dense part of the layer.  The scores are formed as feat @ ((W * attn).sum(-1)): the same
     sums taken in another order, as one thin GEMM over `feat` instead of two strided reductions over
     the [N,H,F] projection.  The backward stacks the gradients of the projection and of the scores
-    into one [N, H*F + 2H] operand, so `feat` is reduced over the nodes once (that tall-skinny
-    product costs the same for 16 columns as for 272) and the input gradient is one GEMM."""
+    into one [N, H*F + 2H] operand when the input gradient is wanted, so that it is one GEMM and `feat` is
+    reduced over the nodes once; a first layer reduces the two parts separately instead of copying the wide one."""
 
     @staticmethod
     def forward(ctx, feat, W, attn_l, attn_r, pad):
@@ -66,10 +66,17 @@ class _ProjectScores(torch.autograd.Function):
         _, hh, ff = attn_l.shape
         n, hfp = feat.shape[0], hh * (ff + ctx.pad)
         zeros = lambda cols: feat.new_zeros(n, cols)
-        g = torch.cat([zeros(hfp) if dh is None else dh.reshape(n, hfp), zeros(hh) if drow is None else drow,
-                       zeros(hh) if dcol is None else dcol], dim=1)                        # [N, H*Fp + 2H]
-        dfeat = torch.matmul(g, w_all.t()) if ctx.needs_input_grad[0] else None
-        dw_ext = reduce_over_rows(feat, g)                                              # [in, H*Fp + 2H]
+        if ctx.needs_input_grad[0] or dh is None:
+            g = torch.cat([zeros(hfp) if dh is None else dh.reshape(n, hfp), zeros(hh) if drow is None else drow,
+                           zeros(hh) if dcol is None else dcol], dim=1)                    # [N, H*Fp + 2H]
+            dfeat = torch.matmul(g, w_all.t()) if ctx.needs_input_grad[0] else None
+            dw_ext = reduce_over_rows(feat, g)                                          # [in, H*Fp + 2H]
+        else:
+            # first layer (no input gradient): nothing needs the stacked operand, so the wide gradient is not copied;
+            # two reductions over feat (2.45 M x 100 -> 256 + 16 columns: 1.2 + 0.3 ms against 1.3 ms of copy + 1.7 ms)
+            dfeat = None
+            gs = torch.cat([zeros(hh) if drow is None else drow, zeros(hh) if dcol is None else dcol], dim=1)
+            dw_ext = torch.cat([reduce_over_rows(feat, dh.reshape(n, hfp)), reduce_over_rows(feat, gs)], dim=1)
         dwl, dwr = dw_ext[:, hfp:hfp + hh].unsqueeze(-1), dw_ext[:, hfp + hh:].unsqueeze(-1)   # [in, H, 1]
         wv = W.view(W.shape[0], hh, ff)
         dW = dw_ext[:, :hfp].view(W.shape[0], hh, ff + ctx.pad)[:, :, :ff] + dwl * attn_l + dwr * attn_r

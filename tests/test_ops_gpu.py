@@ -305,6 +305,15 @@ def test_gat_layer_matches_dgl_composed(fin, f, h, variant):
     assert_close(layer.W.grad, leaves[0].grad, "GATConv grad W", rtol=1e-4, atol=2e-3)
     assert_close(layer.attn_l.grad, leaves[1].grad, "GATConv grad attn_l", rtol=1e-4, atol=2e-3)
     assert_close(layer.attn_r.grad, leaves[2].grad, "GATConv grad attn_r", rtol=1e-4, atol=2e-3)
+    # as a first layer (input without gradient: the backward reduces the two gradient parts separately)
+    for p_ in layer.parameters():
+        p_.grad = None
+    out = layer(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, feat.to(DEV), True if variant == "our" else gd.permute)
+    out.backward(go.to(DEV))
+    assert_close(out, ref.detach(), "GATConv layer (first layer)")
+    assert_close(layer.W.grad, leaves[0].grad, "GATConv grad W (first layer)", rtol=1e-4, atol=2e-3)
+    assert_close(layer.attn_l.grad, leaves[1].grad, "GATConv grad attn_l (first layer)", rtol=1e-4, atol=2e-3)
+    assert_close(layer.attn_r.grad, leaves[2].grad, "GATConv grad attn_r (first layer)", rtol=1e-4, atol=2e-3)
 
 
 # ------------------------------------------------------------------ small operators

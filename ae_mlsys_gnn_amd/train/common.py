@@ -8,6 +8,12 @@ import time
 import torch
 
 
+def head_mean(t):
+    """Mean over the heads of [N, H, C] (the reference's `.mean(1)` on the output layer); with one head it is
+    the same values without a pass over the tensor."""
+    return t.squeeze(1) if t.shape[1] == 1 else t.mean(1)
+
+
 def accuracy(logits, labels):
     if labels.numel() == 0:
         return float("nan")

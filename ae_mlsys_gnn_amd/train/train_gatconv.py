@@ -31,7 +31,7 @@ class GAT(nn.Module):
     def forward(self, g, x, extra):
         for layer in self.hidden:
             x = layer(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, x, extra).flatten(1)
-        return self.out(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, x, extra).mean(1)
+        return common.head_mean(self.out(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, x, extra))
 
 
 def build_parser():

@@ -408,7 +408,7 @@ def run_gat_train(args):
     from torch import nn
     from ae_mlsys_gnn_amd import _lib
     from ae_mlsys_gnn_amd.layers import GATConv, GATConv_stash
-    from ae_mlsys_gnn_amd.train.common import cross_entropy
+    from ae_mlsys_gnn_amd.train.common import cross_entropy, head_mean
     dev = torch.device("cuda:0")
     n, e_t, in_dim, hidden, heads, classes = 2449029, 61_900_000, 100, 32, 8, 47
     g, t_gen, t_csc = build_gat_graph(n, e_t, dev)
@@ -426,7 +426,7 @@ def run_gat_train(args):
 
         def forward(self, extra):
             h = self.l1(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, x, extra).flatten(1)
-            return self.l2(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, h, extra).mean(1)
+            return head_mean(self.l2(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, h, extra))
 
     res = {}
     for name, conv, extra in (("recompute", GATConv, True), ("stash", GATConv_stash, g.permute)):

@@ -250,7 +250,7 @@ def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True,
 def edge_positions(ptr_tensor, idx_tensor, seg_len=None):
     """Builds (once) the own-order schedule of (ptr, idx) and returns int32 [E]: the caller's position of
     every entry in that schedule's order, or None when the order is the caller's (plain schedule).
-    Per-edge tensors passed to operators with edge_order="schedule" must be t[edge_positions]."""
+    Per-edge tensors passed to operators with own_order=True must be t[edge_positions]."""
     if seg_len is None:
         seg_len = default_seg_len()
     bucketed = xcd_buckets_enabled(ptr_tensor)

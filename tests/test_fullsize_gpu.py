@@ -283,3 +283,55 @@ def test_c2_gat_sampled_rows_and_columns_vs_float64(c2_graph):
         want_gx = (alpha[mine].unsqueeze(-1) * go[rws].double()).sum(0)
         assert_close(gx[j], want_gx, "grad_feat of column %d at C2" % j)
         assert_close(gac[j], gscore[mine].sum(0), "grad_attn_col of column %d at C2" % j, atol=1e-5 * scale)
+
+
+def test_c2_graph_gmm_layer_two_dataflows_agree(c2_graph, monkeypatch):
+    """MoNet's second layer at the reddit shape (16 -> 41, K=2, dim=1, 114.8 M edges): the layer that aggregates
+    its input before the fc and the layer that transforms first (the reference's order) are the same sums in
+    another order, computed by different kernels (shared-feature forward / column pass against the packed
+    SpMM / summed column pass); outputs and every gradient must agree.  With the per-edge coordinates in
+    the schedules' own orders on the aggregate-first side, in CSR / CSC order on the other."""
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd.layers import GMMConv
+    from ae_mlsys_gnn_amd.operators.fused_gmmconv import gmm_edge_positions
+    g = c2_graph
+    torch.manual_seed(7)
+    layer = GMMConv(16, 41, dim=1, n_kernels=2).to(DEV)
+    with torch.no_grad():
+        layer.mu.uniform_(0.2, 0.8)
+        layer.bias.normal_()
+    feat = torch.randn(g.n, 16, device=DEV)
+    pseudo = torch.rand(g.n_edges, 1, device=DEV)
+    go = torch.randn(g.n, 41, device=DEV) / 16
+    results = []
+    for aggregate in (True, False):
+        monkeypatch.setattr(GMMConv, "_aggregate_first", lambda self, x, a=aggregate: a)
+        for p_ in layer.parameters():
+            p_.grad = None
+        fd = feat.clone().requires_grad_(True)
+        if aggregate:
+            pos_r, pos_c = gmm_edge_positions(g.row_ptr, g.col_ind), gmm_edge_positions(g.col_ptr, g.row_ind, summed_backward=True)
+            assert pos_r is not None and pos_c is not None
+            to_csc = g.permute.long()[pos_c.long()]
+            pc = pseudo[to_csc].contiguous().requires_grad_(True)
+            out = layer(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, g.permute, fd, pseudo[pos_r.long()].contiguous(), pseudo_csc=pc, own_order=True)
+            del pos_r, pos_c
+        else:
+            to_csc = g.permute.long()
+            pc = pseudo[to_csc].contiguous().requires_grad_(True)
+            out = layer(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, g.permute, fd, pseudo, pseudo_csc=pc)
+        out.backward(go)
+        gp = torch.zeros(g.n_edges, 1, device=DEV)
+        gp[to_csc] = pc.grad                                    # back to CSR order
+        results.append([out.detach(), fd.grad, gp, layer.fc.weight.grad.clone(), layer.mu.grad.clone(), layer.inv_sigma.grad.clone(),
+                        layer.bias.grad.clone()])
+        del pc, to_csc, out, fd
+    a, b = results
+    names = ("out", "grad feat", "grad pseudo", "grad fc.weight", "grad mu", "grad inv_sigma", "grad bias")
+    # rows sum ~490 terms of either sign; the parameter gradients sum over all nodes / all 114.8 M edges
+    # (observed: 7e-4 on outputs up to 1100, 7e-5 on grad feat, 5e-7 on grad pseudo, 1.5e-3 / 3e-4 / 6e-5 on parameter
+    # gradients of magnitude 500-2000)
+    bars = ((1e-4, 2e-3), (1e-4, 5e-4), (1e-4, 1e-5), (1e-5, 1e-2), (1e-5, 5e-3), (1e-5, 2e-3), (1e-5, 1e-3))
+    for name, x, y, (rtol, atol) in zip(names, a, b, bars):
+        assert_close(x, y, "aggregate first vs transform first: " + name, rtol=rtol, atol=atol)
+    _lib.clear_schedule_cache()

@@ -7,7 +7,7 @@ from torch import nn
 from torch.nn import init
 
 from ..operators.fused_gmmconv import (GmmAggregate, GmmAggregateTwoOrders, GmmConvFuseSum, GmmConvFuseSumTwoOrders, GmmConvStash,
-                                        gmm_native)
+                                        GmmConvStashSumTwoOrders, gmm_native)
 from .dense import add_bias, tall_linear
 
 
@@ -51,10 +51,10 @@ class _GMMBase(nn.Module):
         self._allow_zero_in_degree = set_value
 
     def forward(self, rowptr, colind, colptr, rowind, permute, feat, pseudo, pseudo_csc=None, own_order=False):
-        """pseudo_csc (GMMConv only): the same pseudo-coordinates in CSC order, pseudo[permute], built by
+        """pseudo_csc: the same pseudo-coordinates in CSC order, pseudo[permute], built by
         the caller from its own CSC-ordered edge data.  The backward then works in CSC order throughout
         and the gradient of the pseudo-coordinates flows through pseudo_csc instead of pseudo.
-        own_order (GMMConv only): pseudo and pseudo_csc are in the entry order of the operators' schedules
+        own_order: pseudo and pseudo_csc are in the entry order of the operators' schedules
         (operators.fused_gmmconv.gmm_edge_positions); without pseudo_csc the layer is forward-only."""
         if self._aggregate_first(feat):
             return self._finish(self._forward_aggregate_first(rowptr, colind, colptr, rowind, permute, feat, pseudo, pseudo_csc, own_order), feat)
@@ -63,12 +63,11 @@ class _GMMBase(nn.Module):
         if pad:         # zero columns up to a multiple of 4: the operator then takes its 128-bit row layout
             node_feat = th.nn.functional.pad(node_feat, (0, pad))
         if pseudo_csc is not None or own_order:
-            if type(self)._op is not GmmConvFuseSum:
-                raise ValueError("pseudo_csc / own_order are supported by the recomputing GMMConv layer only")
             if own_order and pseudo_csc is None and th.is_grad_enabled() and (node_feat.requires_grad or pseudo.requires_grad):
                 raise ValueError("own_order without pseudo_csc is forward-only")
-            rst = GmmConvFuseSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo.detach(), pseudo_csc, self.mu, self.inv_sigma,
-                                          own_order=own_order)
+            two_orders = GmmConvFuseSumTwoOrders if (type(self)._op is GmmConvFuseSum or pseudo_csc is None) else GmmConvStashSumTwoOrders
+            rst = two_orders(rowptr, colind, colptr, rowind, node_feat, pseudo.detach(), pseudo_csc, self.mu, self.inv_sigma,
+                             own_order=own_order)
         else:
             rst = type(self)._op(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, self.mu, self.inv_sigma)
         if pad:

@@ -187,6 +187,32 @@ def GmmConvFuseSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo_cs
     return GmmFuseSumTwoOrdersFunction.apply(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order)
 
 
+def GmmConvStashSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order=False):
+    """The stash variant with the pseudo-coordinates in both edge orders: as GmmConvFuseSumTwoOrders, and the
+    forward also writes the Gaussian weights [E,K] (in the order of pseudo_csr) and keeps them until the
+    backward, the memory cost of the reference's stash variant (operators/fused_gmmconv.py:100-118).  The
+    backward is the same single pass: recomputing a weight is cheaper than reading it back through a
+    transposition."""
+    return GmmStashSumTwoOrdersFunction.apply(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order)
+
+
+class GmmStashSumTwoOrdersFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order):
+        out, gauss = gmm_native.gmmconv(rowptr, colind, node_feat, pseudo_csr, mu, sigma, want_gauss=True, sum_kernels=True,
+                                        own_order=own_order)
+        ctx.save_for_backward(colptr, rowind, node_feat, pseudo_csc, mu, sigma, gauss)
+        ctx.own_order = own_order
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        colptr, rowind, node_feat, pseudo_csc, mu, sigma, _gauss = ctx.saved_tensors
+        grad_feat, grad_pseudo_csc, grad_mu, grad_sigma = gmm_native.gmmconv_backward(
+            colptr, rowind, None, node_feat, pseudo_csc, mu, sigma, grad_out.contiguous(), sum_kernels=True, own_order=ctx.own_order)
+        return None, None, None, None, grad_feat, None, grad_pseudo_csc, grad_mu, grad_sigma, None
+
+
 def gmm_edge_positions(ptr_arr, idx, summed_backward=False):
     """int32 [E] (or None = identity): caller's position of every entry in the order in which the GMMConv
     operators walk (ptr_arr, idx) when called with own_order=True.  summed_backward: for the (col_ptr,

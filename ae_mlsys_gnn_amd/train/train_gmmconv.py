@@ -91,7 +91,7 @@ def build_parser():
     p.add_argument("--output", type=str, default="figure7.csv")
     p.add_argument("--variant", choices=sorted(VARIANTS), default="our")
     p.add_argument("--csc-pseudo", type=int, default=2, help="2: keep the edge coordinates in the entry order of the forward and the backward "
-                   "schedule (variant our), so every pass streams its per-edge data; 1: in CSR and CSC order (no per-edge transposition in "
+                   "schedule, so every pass streams its per-edge data; 1: in CSR and CSC order (no per-edge transposition in "
                    "the backward); 0: one copy, as the reference")
     p.add_argument("--data-root", type=str, default=None)
     p.add_argument("--cache-dir", type=str, default=None)
@@ -111,11 +111,11 @@ def main(argv=None):
     print("----Data statistics------ (%s)\n  #Nodes %d\n  #Edges %d\n  #Classes %d\n  #Train samples %d\n  #Val samples %d\n  #Test samples %d"
           % (data.source, g.n, g.n_edges, data.n_classes, int(data.train_mask.sum()), int(data.val_mask.sum()), int(data.test_mask.sum())))
     pseudo = datasets.degree_pseudo(g)
-    own_order = args.csc_pseudo == 2 and args.variant == "our"
+    own_order = args.csc_pseudo == 2
     if own_order:
         pseudo, pseudo_csc = schedule_order_copies(g, pseudo)
     else:
-        pseudo_csc = pseudo[g.permute.long()].contiguous() if (args.csc_pseudo and args.variant == "our") else None
+        pseudo_csc = pseudo[g.permute.long()].contiguous() if args.csc_pseudo else None
     torch.manual_seed(args.seed)
     model = MoNet(VARIANTS[args.variant], data.feat.shape[1], args.n_hidden, data.n_classes, args.n_layers, args.pseudo_dim, args.n_kernels,
                   args.dropout).to(dev)

@@ -685,14 +685,15 @@ def test_gmm_layer_with_csc_ordered_pseudo(k, dim, f, monkeypatch):
     _lib.clear_schedule_cache()
 
 
+@pytest.mark.parametrize("stash", [False, True])
 @pytest.mark.parametrize("k,dim,f", [(3, 2, 16), (2, 1, 41), (2, 1, 16)])
-def test_gmm_layer_with_pseudo_in_schedule_order(k, dim, f, monkeypatch):
+def test_gmm_layer_with_pseudo_in_schedule_order(k, dim, f, stash, monkeypatch):
     """GMMConv(..., own_order=True) with the pseudo-coordinates permuted into the entry order of the
     operators' schedules (gmm_edge_positions): same output and gradients as the oracle, the gradient of
     the pseudo-coordinates arrives in the backward schedule's order.  XCD-aware (a real permutation) and
     plain schedules (identity, positions None); a forward-only call; asking for the positions twice."""
     from ae_mlsys_gnn_amd import _lib
-    from ae_mlsys_gnn_amd.layers import GMMConv
+    from ae_mlsys_gnn_amd.layers import GMMConv, GMMConv_stash
     from ae_mlsys_gnn_amd.operators.fused_gmmconv import gmm_edge_positions
     # 250 nodes: rows average 160 entries, both passes take an XCD-aware schedule; 600 nodes: 50 entries, the
     # summed backward keeps the caller's order there
@@ -702,7 +703,7 @@ def test_gmm_layer_with_pseudo_in_schedule_order(k, dim, f, monkeypatch):
         _lib.clear_schedule_cache()
         torch.manual_seed(4)
         g = graphs.add_csc_torch(graphs.rmat_graph(n_nodes, 30000 if n_nodes == 600 else 40000, seed=6))
-        layer = GMMConv(24, f, dim=dim, n_kernels=k)
+        layer = (GMMConv_stash if stash else GMMConv)(24, f, dim=dim, n_kernels=k)      # the stash layer keeps the weights [E,K] as well
         feat, pseudo, go = torch.randn(g.n, 24), torch.rand(g.n_edges, dim), torch.randn(g.n, f)
         leaves = [t.detach().double().requires_grad_(True) for t in (layer.fc.weight, layer.mu, layer.inv_sigma, layer.bias, feat, pseudo)]
         ref = orc.gmm_layer_dgl(leaves[0], leaves[1], leaves[2], leaves[3], g.row_ptr, g.col_ind, leaves[4], leaves[5])

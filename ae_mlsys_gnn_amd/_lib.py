@@ -30,6 +30,8 @@ _SIGNATURES = {
     "fgnn_schedule_num_items": (c_int, [c_void_p]),
     "fgnn_schedule_num_partials": (c_int, [c_void_p]),
     "fgnn_schedule_num_edges": (c_int64, [c_void_p]),
+    "fgnn_schedule_device_bytes": (c_size_t, [c_void_p]),
+    "fgnn_validate_graph": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int64, c_void_p]),
     "fgnn_gat_forward_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int]),
     "fgnn_gat_forward": (c_int, [c_int, c_int64, c_int, c_int] + [c_void_p] * 4 + [c_float] + [c_void_p] * 8
                          + [c_void_p, c_void_p, c_size_t, c_void_p]),
@@ -137,6 +139,10 @@ class Schedule:
         self.n_rows = self.ptr_tensor.numel() - 1
         handle = c_void_p()
         with torch.cuda.device(self.ptr_tensor.device):
+            if self.idx_tensor is not None and os.environ.get("FGNN_VALIDATE", "0") not in ("0", ""):
+                # opt-in: range-check the graph once, when its work list is built, before any gather kernel runs
+                check(lib().fgnn_validate_graph(ptr(self.ptr_tensor), ptr(self.idx_tensor), self.n_rows, self.n_rows,
+                                                self.idx_tensor.numel(), stream_ptr()), "fgnn_validate_graph")
             if self.idx_tensor is None:
                 check(lib().fgnn_schedule_create(ptr(self.ptr_tensor), self.n_rows, int(seg_len), stream_ptr(),
                                                  ctypes.byref(handle)), "fgnn_schedule_create")
@@ -149,6 +155,10 @@ class Schedule:
         self.n_partials = lib().fgnn_schedule_num_partials(handle)
         self.n_edges = lib().fgnn_schedule_num_edges(handle)
         self.own_order = False
+
+    def device_bytes(self):
+        """Device memory the schedule holds outside torch's allocator."""
+        return int(lib().fgnn_schedule_device_bytes(self.handle))
 
     def take_positions(self):
         """int32 [E]: caller's edge position of every entry in the schedule's own order.  The schedule gives
@@ -200,11 +210,12 @@ def xcd_buckets_enabled(ptr_tensor) -> bool:
         deg = (ptr_tensor[1:] - ptr_tensor[:-1]).long()
         long_rows = torch.where(deg > BUCKET_ROW_LEN, deg, torch.zeros_like(deg)).sum()
         n_edges, n_long, longest = torch.stack([deg.sum(), long_rows, deg.max()]).tolist()
-        hit = n_edges > 0 and n_long >= BUCKET_MIN_SHARE * n_edges and longest * n_rows >= BUCKET_MIN_SKEW * n_edges
+        hit = (n_edges > 0 and n_long >= BUCKET_MIN_SHARE * n_edges and longest * n_rows >= BUCKET_MIN_SKEW * n_edges,
+               ptr_tensor)         # the entry holds the tensor: its address cannot be reused while the entry lives
         _bucket_rule_cache[key] = hit
         while len(_bucket_rule_cache) > 4 * _SCHED_CACHE_MAX:
             _bucket_rule_cache.popitem(last=False)
-    return hit
+    return hit[0]
 
 
 def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True, own_order=False) -> Schedule:
@@ -269,6 +280,12 @@ def edge_positions(ptr_tensor, idx_tensor, seg_len=None):
     while len(_sched_cache) > _SCHED_CACHE_MAX:
         _sched_cache.popitem(last=False)
     return pos
+
+
+def schedule_device_bytes() -> int:
+    """Device memory held by all cached schedules: the library allocates it itself, so torch's
+    max_memory_allocated does not see it and peak-memory reports add it."""
+    return sum(s.device_bytes() for s in _sched_cache.values())
 
 
 def clear_schedule_cache():

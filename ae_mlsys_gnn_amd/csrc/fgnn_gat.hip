@@ -1109,7 +1109,7 @@ extern "C" int fgnn_gat_forward(int N, int64_t E, int H, int F, const float *att
                               edge_sum, aux_out2, aux_c, e_lrelu, e_softmax, sched, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
-// Backward workspace: rec [N*H float4] | recompute area (out, out2 [N*HF each], c [N*H]) | partials
+// Backward workspace: rec [N*H float4] | recompute area (out, out2 [N*HF each], c, max, sum [N*H each]) | partials
 
 extern "C" size_t fgnn_gat_backward_workspace_bytes(int N, int H, int F, const fgnn_schedule_t *sched_csc,
                                                     const fgnn_schedule_t *sched_csr, int need_recompute)
@@ -1117,7 +1117,7 @@ extern "C" size_t fgnn_gat_backward_workspace_bytes(int N, int H, int F, const f
     size_t HF = (size_t)H * F;
     size_t b = fgnn_align256((size_t)N * H * sizeof(float4));
     if (need_recompute) {
-        b += 2 * fgnn_align256((size_t)N * HF * sizeof(float)) + fgnn_align256((size_t)N * H * sizeof(float));
+        b += 2 * fgnn_align256((size_t)N * HF * sizeof(float)) + 3 * fgnn_align256((size_t)N * H * sizeof(float));
         b += fgnn_align256(fgnn_gat_forward_workspace_bytes(sched_csr, H, F));
     }
     if (sched_csc) b += fgnn_align256((size_t)sched_csc->n_partials * gat_bwd_pw((int)HF, H) * sizeof(float));
@@ -1159,12 +1159,14 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
         float *r_out = (float *)w; w += fgnn_align256((size_t)N * HF * sizeof(float));
         float *r_out2 = (float *)w; w += fgnn_align256((size_t)N * HF * sizeof(float));
         float *r_c = (float *)w; w += fgnn_align256((size_t)N * H * sizeof(float));
+        float *r_max = (float *)w; w += fgnn_align256((size_t)N * H * sizeof(float));
+        float *r_sum = (float *)w; w += fgnn_align256((size_t)N * H * sizeof(float));
         void *fws = w; size_t fwb = fgnn_align256(fgnn_gat_forward_workspace_bytes(sched_csr, H, F)); w += fwb;
-        // edge_max / edge_sum are rewritten with identical values by the recomputation
+        // the recomputation writes its own row statistics (the same values): the caller's stay read-only
         rc = gat_forward_launch(N, E, H, F, attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, r_out,
-                                (float *)edge_max, (float *)edge_sum, r_out2, r_c, nullptr, nullptr, sched_csr, fws, fwb, st);
+                                r_max, r_sum, r_out2, r_c, nullptr, nullptr, sched_csr, fws, fwb, st);
         if (rc) return rc;
-        out_feat = r_out; aux_out2 = r_out2; aux_c = r_c;
+        out_feat = r_out; aux_out2 = r_out2; aux_c = r_c; edge_max = r_max; edge_sum = r_sum;
     }
     float *part = (float *)w;
 

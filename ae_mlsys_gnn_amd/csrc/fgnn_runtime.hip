@@ -305,6 +305,62 @@ extern "C" void fgnn_schedule_destroy(fgnn_schedule_t *s)
     delete s;
 }
 
+extern "C" size_t fgnn_schedule_device_bytes(const fgnn_schedule_t *s)
+{
+    if (!s) return 0;
+    size_t b = (size_t)s->n_items * sizeof(fgnn_item) + (size_t)s->n_split * sizeof(fgnn_split);
+    if (s->bidx_dev) b += (size_t)s->n_edges * sizeof(int32_t);
+    if (s->bpos_dev) b += (size_t)s->n_edges * sizeof(int32_t);
+    return b;
+}
+
+// flags[0] |= 1: ptr[0] != 0; 2: ptr decreases; 4: ptr[n_rows] != E; 8: an index outside [0, n_cols)
+__global__ __launch_bounds__(256) void validate_graph_kernel(const int *__restrict__ ptr, const int *__restrict__ idx, int n_rows, int n_cols,
+                                                             int64_t E, int *__restrict__ flags)
+{
+    int bad = 0;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i <= n_rows; i += stride) {
+        const int v = ptr[i];
+        if (i == 0 && v != 0) bad |= 1;
+        if (i < n_rows && ptr[i + 1] < v) bad |= 2;
+        if (i == n_rows && (int64_t)v != E) bad |= 4;
+    }
+    for (int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x; q < E; q += stride) {
+        const int j = idx[q];
+        if (j < 0 || j >= n_cols) bad |= 8;
+    }
+    if (bad) atomicOr(flags, bad);
+}
+
+extern "C" int fgnn_validate_graph(const int32_t *ptr_dev, const int32_t *idx_dev, int n_rows, int n_cols, int64_t E, void *stream)
+{
+    FGNN_REQUIRE(ptr_dev && (idx_dev || E == 0), FGNN_ERR_NULL, "fgnn_validate_graph: NULL argument");
+    FGNN_REQUIRE(n_rows >= 0 && n_cols >= 0 && E >= 0 && E <= 2147483647LL, FGNN_ERR_SHAPE, "fgnn_validate_graph: bad sizes n_rows=%d n_cols=%d E=%lld",
+                 n_rows, n_cols, (long long)E);
+    hipStream_t st = (hipStream_t)stream;
+    int *flags_dev = nullptr;
+    int flags = 0;
+    FGNN_HIP(hipMalloc((void **)&flags_dev, sizeof(int)));
+    hipError_t err = hipMemcpyAsync(flags_dev, &flags, sizeof(int), hipMemcpyHostToDevice, st);
+    if (err == hipSuccess) {
+        const int64_t work = std::max<int64_t>(E, (int64_t)n_rows + 1);
+        const unsigned grid = (unsigned)std::min<int64_t>((work + 255) / 256, 8192);
+        hipLaunchKernelGGL(validate_graph_kernel, dim3(grid), dim3(256), 0, st, ptr_dev, idx_dev, n_rows, n_cols, E, flags_dev);
+        err = hipGetLastError();
+    }
+    if (err == hipSuccess) err = hipMemcpyAsync(&flags, flags_dev, sizeof(int), hipMemcpyDeviceToHost, st);
+    if (err == hipSuccess) err = hipStreamSynchronize(st);
+    (void)hipFree(flags_dev);
+    if (err != hipSuccess) {
+        fgnn_set_error("fgnn_validate_graph: %s", hipGetErrorString(err));
+        return (int)err;
+    }
+    FGNN_REQUIRE(flags == 0, FGNN_ERR_SHAPE, "fgnn_validate_graph: malformed graph:%s%s%s%s", (flags & 1) ? " ptr[0] != 0;" : "",
+                 (flags & 2) ? " ptr decreases;" : "", (flags & 4) ? " ptr[n_rows] != E;" : "", (flags & 8) ? " an index lies outside [0, n_cols);" : "");
+    return 0;
+}
+
 extern "C" int fgnn_schedule_num_items(const fgnn_schedule_t *s) { return s ? s->n_items : 0; }
 extern "C" int fgnn_schedule_num_partials(const fgnn_schedule_t *s) { return s ? s->n_partials : 0; }
 extern "C" int64_t fgnn_schedule_num_edges(const fgnn_schedule_t *s) { return s ? s->n_edges : 0; }

@@ -32,6 +32,35 @@ class Graph:
         return Graph(self.n, mv(self.row_ptr), mv(self.col_ind), mv(self.col_ptr), mv(self.row_ind), mv(self.permute))
 
 
+def validate_graph(g: "Graph", what: str = "graph") -> None:
+    """Raises ValueError unless the arrays describe a graph the gather kernels can walk: integer index
+    arrays, pointer arrays that start at 0, never decrease and end at E, every node id in [0, n) and every
+    permute entry in [0, E).  Plain torch reductions (host or device), to be called BEFORE any operator
+    sees arrays that came from a file or another untrusted source: the kernels index feature rows with
+    these ids unchecked."""
+    int_types = (torch.int8, torch.int16, torch.int32, torch.int64, torch.uint8)
+    e = int(g.col_ind.numel())
+    for name, ptr_arr, idx in (("row_ptr/col_ind", g.row_ptr, g.col_ind), ("col_ptr/row_ind", g.col_ptr, g.row_ind)):
+        if ptr_arr is None and idx is None:
+            continue
+        if ptr_arr is None or idx is None:
+            raise ValueError("%s: %s must be given together" % (what, name))
+        if ptr_arr.dtype not in int_types or idx.dtype not in int_types:
+            raise ValueError("%s: %s must be integer arrays, got %s / %s" % (what, name, ptr_arr.dtype, idx.dtype))
+        if ptr_arr.dim() != 1 or idx.dim() != 1 or ptr_arr.numel() != g.n + 1 or idx.numel() != e:
+            raise ValueError("%s: %s have %d / %d entries, expected %d / %d" % (what, name, ptr_arr.numel(), idx.numel(), g.n + 1, e))
+        p = ptr_arr.to(torch.int64)
+        if int(p[0]) != 0 or int(p[-1]) != e or (g.n > 0 and bool((p[1:] < p[:-1]).any())):
+            raise ValueError("%s: %s: the pointer array must start at 0, never decrease and end at E=%d" % (what, name, e))
+        if e and (int(idx.min()) < 0 or int(idx.max()) >= g.n):
+            raise ValueError("%s: %s: node ids must lie in [0, %d), found [%d, %d]" % (what, name, g.n, int(idx.min()), int(idx.max())))
+    if g.permute is not None:
+        if g.permute.dtype not in int_types or g.permute.numel() != e:
+            raise ValueError("%s: permute must be an integer array of %d entries" % (what, e))
+        if e and (int(g.permute.min()) < 0 or int(g.permute.max()) >= e):
+            raise ValueError("%s: permute entries must lie in [0, %d)" % (what, e))
+
+
 def csr_from_keys(keys: torch.Tensor, n: int) -> Graph:
     """keys = dst * n + src, sorted and unique (int64)."""
     dst = torch.div(keys, n, rounding_mode="floor")

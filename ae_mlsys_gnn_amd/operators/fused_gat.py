@@ -55,12 +55,31 @@ class gat_native:
     def gat_backward(negative_slope, row_ptr, col_ind, col_ptr, row_ind, edge_max, edge_sum, in_feat, attn_row, attn_col,
                      grad, *, out_feat=None, out2=None, cc=None, permute=None, e_lrelu=None, e_soft=None,
                      use_schedule=True):
-        require_cuda(grad, in_feat, col_ptr, row_ind)
-        grad = as_f32(grad)
+        require_cuda(grad, in_feat, col_ptr, row_ind, attn_row, attn_col, edge_max, edge_sum, row_ptr, col_ind, out_feat, out2, cc,
+                     permute, e_soft)
+        # the kernels take raw pointers: every tensor is made contiguous and checked here, so a strided view
+        # (or a tensor of another shape) can neither give wrong gradients nor be read past its storage
+        grad, in_feat, attn_row, attn_col = as_f32(grad), as_f32(in_feat), as_f32(attn_row), as_f32(attn_col)
+        edge_max, edge_sum = as_f32(edge_max), as_f32(edge_sum)
+        if in_feat.dim() != 3:
+            raise _lib.FgnnError("in_feat must be [N,H,F], got %s" % (tuple(in_feat.shape),))
         n, h, f = in_feat.shape
         e = row_ind.numel()
         dev = in_feat.device
         col_ptr, row_ind = as_i32(col_ptr), as_i32(row_ind)
+        row_ptr = None if row_ptr is None else as_i32(row_ptr)
+        col_ind = None if col_ind is None else as_i32(col_ind)
+        out_feat, out2, cc = (None if t is None else as_f32(t) for t in (out_feat, out2, cc))
+        permute = None if permute is None else as_i32(permute)
+        e_soft = None if e_soft is None else as_f32(e_soft)
+        for name, t, shape in (("grad", grad, (n, h, f)), ("attn_row", attn_row, (n, h)), ("attn_col", attn_col, (n, h)),
+                               ("edge_max", edge_max, (n, h)), ("edge_sum", edge_sum, (n, h)), ("out_feat", out_feat, (n, h, f)),
+                               ("out2", out2, (n, h, f)), ("cc", cc, (n, h)), ("e_soft", e_soft, (e, h))):
+            if t is not None and tuple(t.shape) != shape:
+                raise _lib.FgnnError("gat_backward: %s has shape %s, expected %s" % (name, tuple(t.shape), shape))
+        for name, t, numel in (("col_ptr", col_ptr, n + 1), ("row_ptr", row_ptr, n + 1), ("col_ind", col_ind, e), ("permute", permute, e)):
+            if t is not None and t.numel() != numel:
+                raise _lib.FgnnError("gat_backward: %s has %d elements, expected %d" % (name, t.numel(), numel))
         grad_feat = torch.empty_like(in_feat)
         grad_attn_row = torch.empty((n, h), dtype=torch.float32, device=dev)
         grad_attn_col = torch.empty((n, h), dtype=torch.float32, device=dev)
@@ -97,12 +116,19 @@ def _needs_grad(ctx):
     return any(ctx.needs_input_grad)
 
 
+def _contig(t):
+    return t if t.is_contiguous() else t.contiguous()
+
+
 class FusedGATFunction_SM(torch.autograd.Function):
     """Recompute ("save memory") variant: nothing edge-sized is kept between forward and backward."""
 
     @staticmethod
     def forward(ctx, attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat):
         need = _needs_grad(ctx)
+        # contiguous copies of strided views are made once, here, and these are what the backward gets
+        attn_row, attn_col, in_feat = _contig(attn_row), _contig(attn_col), _contig(in_feat)
+        row_ptr, col_ind, col_ptr, row_ind = _contig(row_ptr), _contig(col_ind), _contig(col_ptr), _contig(row_ind)
         out, edge_max, edge_sum, out2, cc, _, _ = gat_native.gat_forward(
             attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, need_aux=need)
         if need:
@@ -128,6 +154,8 @@ class FusedGATFunction_stash(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute):
+        attn_row, attn_col, in_feat = _contig(attn_row), _contig(attn_col), _contig(in_feat)
+        row_ptr, col_ind, col_ptr, row_ind, permute = _contig(row_ptr), _contig(col_ind), _contig(col_ptr), _contig(row_ind), _contig(permute)
         out, edge_max, edge_sum, out2, cc, _, e_soft = gat_native.gat_forward(
             attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, need_aux=True, stash=True, stash_lrelu=False)
         ctx.save_for_backward(row_ptr, col_ind, col_ptr, row_ind, permute, e_soft, in_feat, attn_row, attn_col,

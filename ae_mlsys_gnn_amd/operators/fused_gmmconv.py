@@ -47,11 +47,19 @@ class gmm_native:
         require_cuda(colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out)
         colptr, rowind = as_i32(colptr), as_i32(rowind)
         permute = None if permute is None else as_i32(permute)      # None: pseudo / grad_pseudo in CSC order
-        grad_out = as_f32(grad_out)
+        # raw pointers go to the kernels: contiguous copies of strided views, and every shape checked
+        grad_out, node_feat, pseudo, mu, sigma = as_f32(grad_out), as_f32(node_feat), as_f32(pseudo), as_f32(mu), as_f32(sigma)
+        if node_feat.dim() != 3 or mu.dim() != 2:
+            raise FgnnError("gmmconv_backward: node_feat must be [N,K,F] and mu [K,dim], got %s and %s" % (tuple(node_feat.shape), tuple(mu.shape)))
         n, k, f = node_feat.shape
         e = rowind.numel()
         dim = mu.shape[1]
         dev = node_feat.device
+        want_go = (n, f) if sum_kernels else (n, k, f)
+        if (mu.shape != (k, dim) or sigma.shape != (k, dim) or pseudo.shape != (e, dim) or colptr.numel() != n + 1
+                or tuple(grad_out.shape) != want_go or (permute is not None and permute.numel() != e)):
+            raise FgnnError("gmmconv_backward: shape mismatch mu %s sigma %s pseudo %s grad_out %s col_ptr %d for N=%d K=%d F=%d E=%d" % (
+                tuple(mu.shape), tuple(sigma.shape), tuple(pseudo.shape), tuple(grad_out.shape), colptr.numel(), n, k, f, e))
         grad_feat = torch.empty_like(node_feat)
         grad_pseudo = torch.empty((e, dim), dtype=torch.float32, device=dev)
         grad_mu = torch.empty_like(mu)
@@ -101,13 +109,18 @@ class gmm_native:
         require_cuda(colptr, rowind, permute, feat, pseudo, mu, sigma, grad_out)
         colptr, rowind = as_i32(colptr), as_i32(rowind)
         permute = None if permute is None else as_i32(permute)
-        grad_out = as_f32(grad_out)
+        grad_out, feat, pseudo, mu, sigma = as_f32(grad_out), as_f32(feat), as_f32(pseudo), as_f32(mu), as_f32(sigma)
+        if feat.dim() != 2 or mu.dim() != 2:
+            raise FgnnError("gmmconv_shared_backward: feat must be [N,F] and mu [K,dim], got %s and %s" % (tuple(feat.shape), tuple(mu.shape)))
         n, f = feat.shape
         k, dim = mu.shape
         e = rowind.numel()
         dev = feat.device
         if grad_out.shape != (n, k, f):
             raise FgnnError("gmmconv_shared_backward: grad_out is %s, expected (%d, %d, %d)" % (tuple(grad_out.shape), n, k, f))
+        if sigma.shape != (k, dim) or pseudo.shape != (e, dim) or colptr.numel() != n + 1 or (permute is not None and permute.numel() != e):
+            raise FgnnError("gmmconv_shared_backward: shape mismatch sigma %s pseudo %s col_ptr %d for N=%d K=%d E=%d" % (
+                tuple(sigma.shape), tuple(pseudo.shape), colptr.numel(), n, k, e))
         parts = torch.empty((n, k, f), dtype=torch.float32, device=dev)      # kernel k's share of grad_feat
         grad_pseudo = torch.empty((e, dim), dtype=torch.float32, device=dev)
         grad_mu = torch.empty_like(mu)

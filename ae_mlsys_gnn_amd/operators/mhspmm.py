@@ -11,6 +11,11 @@ def mhspmm(ptr_arr, idx, attention, feat, pos_map=None):
     require_cuda(ptr_arr, idx, feat)
     ptr_arr, idx, feat = as_i32(ptr_arr), as_i32(idx), as_f32(feat)
     attention = None if attention is None else as_f32(attention)
+    if pos_map is not None:
+        require_cuda(pos_map)
+        pos_map = as_i32(pos_map)
+        if pos_map.numel() != idx.numel():
+            raise FgnnError("mhspmm: pos_map has %d entries, expected %d" % (pos_map.numel(), idx.numel()))
     n, h, f = feat.shape
     e = idx.numel()
     if attention is not None and attention.shape != (e, h):

@@ -54,8 +54,20 @@ def graph_from_edges(src, dst, n, device, self_loops=True, dedupe=False) -> grap
     """Directed edges src -> dst (any integer tensors) -> CSR by destination + CSC + permute, all on
     `device` through fgnn_coo2csr / fgnn_csr2csc.  Duplicate edges stay independent edges unless
     `dedupe`; with `self_loops` every node ends up with exactly one."""
-    src = torch.as_tensor(src).to(device=device, dtype=torch.int32)
-    dst = torch.as_tensor(dst).to(device=device, dtype=torch.int32)
+    src, dst = torch.as_tensor(src), torch.as_tensor(dst)
+    # checked in the file's own integer type, before the cast to int32 could wrap an id into range and
+    # before any kernel indexes a feature row with it
+    for name, t in (("src", src), ("dst", dst)):
+        if t.dtype.is_floating_point or t.dtype == torch.bool or t.dim() != 1:
+            raise ValueError("graph_from_edges: %s must be a 1-D integer array, got %s %s" % (name, t.dtype, tuple(t.shape)))
+        if t.numel() and (int(t.min()) < 0 or int(t.max()) >= n):
+            raise ValueError("graph_from_edges: %s ids must lie in [0, %d), found [%d, %d]" % (name, n, int(t.min()), int(t.max())))
+    if src.numel() != dst.numel():
+        raise ValueError("graph_from_edges: %d sources for %d destinations" % (src.numel(), dst.numel()))
+    if not 0 <= n <= 2147483647 or src.numel() + (n if self_loops else 0) > 2147483647:
+        raise ValueError("graph_from_edges: node or edge count exceeds int32")
+    src = src.to(device=device, dtype=torch.int32)
+    dst = dst.to(device=device, dtype=torch.int32)
     if self_loops:
         keep = src != dst
         ar = torch.arange(n, dtype=torch.int32, device=device)
@@ -73,12 +85,11 @@ def save_graph(path, g: graphs.Graph):
 
 def load_graph(path, device) -> graphs.Graph:
     with np.load(path, allow_pickle=False) as z:
-        arr = {k: torch.from_numpy(z[k]).to(device) for k in ("row_ptr", "col_ind", "col_ptr", "row_ind", "permute")}
+        host = {k: torch.from_numpy(z[k]) for k in ("row_ptr", "col_ind", "col_ptr", "row_ind", "permute")}
         n = int(z["n"])
-    if arr["row_ptr"].numel() != n + 1 or arr["col_ptr"].numel() != n + 1 or not (
-            arr["col_ind"].numel() == arr["row_ind"].numel() == arr["permute"].numel() == int(arr["row_ptr"][-1])):
-        raise ValueError("%s: inconsistent graph arrays" % path)
-    return graphs.Graph(n, **arr)
+    # a cache file is untrusted input: every id is range-checked on the host before anything reaches the device
+    graphs.validate_graph(graphs.Graph(n, **host), what=str(path))
+    return graphs.Graph(n, **{k: v.to(device=device, dtype=torch.int32) for k, v in host.items()})
 
 
 def _masks_from_types(node_types):

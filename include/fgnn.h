@@ -72,6 +72,18 @@ void    fgnn_schedule_destroy(fgnn_schedule_t *s);
 int     fgnn_schedule_num_items(const fgnn_schedule_t *s);
 int     fgnn_schedule_num_partials(const fgnn_schedule_t *s);   /* segments of split rows */
 int64_t fgnn_schedule_num_edges(const fgnn_schedule_t *s);
+/* Device memory the schedule itself holds (work items, split table, the bucket-ordered index copy and the
+ * position map of an XCD-aware schedule): allocated by the library outside the caller's allocator, so a
+ * caller that reports peak memory adds it.  No counterpart in the reference. */
+size_t  fgnn_schedule_device_bytes(const fgnn_schedule_t *s);
+
+/* Checks a CSR (or CSC) pair before any gather kernel sees it: ptr[0] == 0, ptr non-decreasing,
+ * ptr[n_rows] == E and every idx in [0, n_cols).  One reduction kernel and a 4-byte read-back (synchronises
+ * `stream`); returns FGNN_ERR_SHAPE with the findings in fgnn_last_error().  The operators themselves do not
+ * range-check indices (the reference's do not either: src/fused_gat/fused_gat_SM.cpp:22-36 only asserts
+ * device, dtype and contiguity), so a loader of untrusted files calls this first. */
+int     fgnn_validate_graph(const int32_t *ptr_dev, const int32_t *idx_dev, int n_rows, int n_cols, int64_t E,
+                            void *stream);
 
 /* ---------------------------------------------------------------- fused GAT
  * Replaces fused_gat_SM.gat_forward (src/fused_gat/fused_gat_SM.cpp:14-38, host launcher

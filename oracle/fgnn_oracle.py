@@ -31,6 +31,19 @@ What each function follows in the reference, and what pins it:
   ``cusparseCsr2cscEx2`` (CUDA 11.3, src/csr2csc/csr2csc.cu:10-23), third-party and
   absent here: parity with *that* routine is unpinned; the contract is the stable
   (ascending CSR position) transpose.
+* ``gmm_layer_dgl`` -- the whole ``GMMConv_dgl.forward`` (layers/gmmconv_layer.py:130-149: fc,
+  ``view(-1, K, out)``, Gaussian-weighted sum, ``.sum(1)``, residual, bias).  Pinned by K = 1,
+  inv_sigma = 0 (a scipy SpMM of ``feat @ W.T``), by a hand-built 3-node case with residual and
+  bias worked out with python loops and ``math.exp``, and by a check that the other (out, K)
+  view order gives a different result.
+* ``gat_abs_sums`` / ``gmm_abs_sums`` -- not reference functions: for every output of the two
+  fused operators the sum of the ABSOLUTE values of its elementary summands (products of inputs,
+  no cancellation inside), which is what an fp32 rounding-error bound of a cancellation sum
+  scales with.  Pinned by construction checks in tests (equal to |output| when all inputs are
+  non-negative; never below |output|).
+* ``gat_reference_chunked`` -- the same GAT math with the analytic backward and the scales, written
+  without any [E,H,F] tensor so that it runs at the full benchmark sizes.  Pinned in tests against
+  ``gat_forward`` + autograd and ``gat_abs_sums`` on small graphs with chunk sizes that cut rows.
 * small operators -- one-line gather/scatter identities
   (operators/edge_softmax.py:30-42, operators/u_add_v.py:19-29,
   operators/mhspmm.py:24-41, operators/spmm.py:25-66).
@@ -48,17 +61,17 @@ def row_of_edge(row_ptr: torch.Tensor) -> torch.Tensor:
     """Destination node of every CSR position (int64)."""
     rp = row_ptr.to(torch.int64)
     deg = rp[1:] - rp[:-1]
-    return torch.repeat_interleave(torch.arange(deg.numel(), dtype=torch.int64), deg)
+    return torch.repeat_interleave(torch.arange(deg.numel(), dtype=torch.int64, device=rp.device), deg)
 
 
 def _segment_softmax(e: torch.Tensor, dst: torch.Tensor, n: int):
     """Softmax of e[E,H] over edges sharing a destination.  Returns (alpha, max, sum)."""
     h = e.shape[1]
     idx = dst.view(-1, 1).expand(-1, h)
-    mx = torch.full((n, h), -float("inf"), dtype=e.dtype)
+    mx = torch.full((n, h), -float("inf"), dtype=e.dtype, device=e.device)
     mx = mx.scatter_reduce(0, idx, e, reduce="amax", include_self=True)
     ex = torch.exp(e - mx[dst])
-    sm = torch.zeros((n, h), dtype=e.dtype).index_add_(0, dst, ex)
+    sm = torch.zeros((n, h), dtype=e.dtype, device=e.device).index_add_(0, dst, ex)
     return ex / sm[dst], mx, sm
 
 
@@ -124,6 +137,122 @@ def gat_layer_dgl(fc_weight, attn_l, attn_r, row_ptr, col_ind, negative_slope, f
     return torch.zeros_like(ft).index_add_(0, dst, a.unsqueeze(-1) * ft[src])
 
 
+def gat_abs_sums(attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, grad_out):
+    """Sum of |elementary summand| for every output of the fused GAT forward and backward (the scale
+    of their fp32 rounding error).  With alpha the attention, d = lrelu'(e) and
+    geA[p,h] = sum_f |g[i,h,f]| |x[j,h,f]|, wsA[i,h] = sum_p alpha geA:
+      out           sum_p alpha |x_j|
+      grad_feat     sum_i alpha |g_i|
+      grad_attn_row sum_p alpha |d| (geA + wsA[i])      (terms of src/fused_gat/fused_gat_SM.cu:656-732)
+      grad_attn_col the same terms summed per source."""
+    n = attn_row.shape[0]
+    dst = row_of_edge(row_ptr)
+    src = col_ind.to(torch.int64)
+    _, e, alpha, _, _ = gat_forward(attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, return_edge=True)
+    ax, ag = in_feat.abs(), grad_out.abs()
+    s_out = torch.zeros_like(ax).index_add_(0, dst, alpha.unsqueeze(-1) * ax[src])
+    s_gfeat = torch.zeros_like(ax).index_add_(0, src, alpha.unsqueeze(-1) * ag[dst])
+    ge_a = (ag[dst] * ax[src]).sum(-1)
+    ws_a = torch.zeros_like(attn_row).index_add_(0, dst, alpha * ge_a)
+    d = torch.where(e > 0, torch.ones_like(e), torch.full_like(e, abs(negative_slope)))
+    t_a = alpha * d * (ge_a + ws_a[dst])
+    s_gar = torch.zeros_like(attn_row).index_add_(0, dst, t_a)
+    s_gac = torch.zeros_like(attn_row).index_add_(0, src, t_a)
+    return {"out": s_out, "grad_feat": s_gfeat, "grad_attn_row": s_gar, "grad_attn_col": s_gac}
+
+
+def segment_sums(ptr, vals):
+    """out[r] = sum of vals[ptr[r]:ptr[r+1]] along dim 0 (empty segments give 0), by differences of one
+    running sum -- usable at 10^8 entries, where index_add_ of float64 serialises on its atomics."""
+    c = torch.cat([torch.zeros_like(vals[:1]), torch.cumsum(vals, 0)])
+    p = ptr.to(torch.int64)
+    return c[p[1:]] - c[p[:-1]]
+
+
+def segment_weighted_rows(ptr, ids, weights, feat, chunk=1 << 20):
+    """out[r,h,:] = sum_{p in [ptr[r], ptr[r+1])} weights[p,h] * feat[ids[p],h,:] in float64, the entries walked in
+    chunks (the [E,H,F] message tensor of gat_forward is never materialised).  feat may be float32."""
+    p = ptr.to(torch.int64)
+    n_e = int(p[-1])
+    out = torch.zeros((p.numel() - 1,) + tuple(feat.shape[1:]), dtype=torch.float64, device=feat.device)
+    for a in range(0, n_e, chunk):
+        b = min(a + chunk, n_e)
+        c = torch.cumsum(weights[a:b].unsqueeze(-1) * feat[ids[a:b].to(torch.int64)].double(), 0)
+        r_lo = int(torch.searchsorted(p, torch.tensor(a, device=p.device), right=True)) - 1
+        r_hi = int(torch.searchsorted(p, torch.tensor(b - 1, device=p.device), right=True)) - 1
+        rows = torch.arange(r_lo, r_hi + 1, device=p.device)
+        st = torch.clamp(p[rows], min=a) - a
+        en = torch.clamp(p[rows + 1], max=b) - a
+        live = en > st
+        rows, st, en = rows[live], st[live], en[live]
+        seg = c[en - 1] - torch.where((st > 0).view(-1, 1, 1), c[torch.clamp(st - 1, min=0)], torch.zeros_like(c[:1]))
+        out[rows] += seg                      # rows are distinct inside a chunk
+    return out
+
+
+def edge_dots(dst, src, a, b, chunk=1 << 20, absolute=False):
+    """[E,H]: <a[dst[p],h,:], b[src[p],h,:]> in float64 (of the absolute values when `absolute`), in chunks."""
+    out = torch.empty((dst.numel(), a.shape[1]), dtype=torch.float64, device=a.device)
+    for s0 in range(0, dst.numel(), chunk):
+        sl = slice(s0, min(s0 + chunk, dst.numel()))
+        u, v = a[dst[sl]].double(), b[src[sl]].double()
+        out[sl] = (u.abs() * v.abs()).sum(-1) if absolute else (u * v).sum(-1)
+    return out
+
+
+def gat_reference_chunked(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, permute, negative_slope, in_feat, grad_out,
+                          chunk=1 << 20):
+    """The whole fused GAT forward and backward in float64 with explicit formulas instead of autograd, and the
+    scales of gat_abs_sums next to them, without any [E,H,F] tensor: usable on the 10^8-edge graphs (on whatever
+    device the inputs live on; they may be float32).  Same math as gat_forward; the backward terms are
+    ge = <g_i, x_j>, ws_i = sum_p alpha ge, g_score = alpha (ge - ws_i) lrelu'(e)
+    (src/fused_gat/fused_gat_SM.cu:656-732).  Returns a dict of out, grad_feat, grad_attn_row, grad_attn_col
+    and S_<name> for each."""
+    ar, ac = attn_row.double(), attn_col.double()
+    dst = row_of_edge(row_ptr)
+    src = col_ind.to(torch.int64)
+    pm = permute.to(torch.int64)
+    e = torch.nn.functional.leaky_relu(ar[dst] + ac[src], negative_slope)
+    alpha, _, _ = _segment_softmax(e, dst, ar.shape[0])
+    d = torch.where(e > 0, 1.0, abs(negative_slope))
+    del e
+    res = {"out": segment_weighted_rows(row_ptr, col_ind, alpha, in_feat, chunk),
+           "S_out": segment_weighted_rows(row_ptr, col_ind, alpha, in_feat.abs(), chunk)}
+    a_csc = alpha[pm]
+    res["grad_feat"] = segment_weighted_rows(col_ptr, row_ind, a_csc, grad_out, chunk)
+    res["S_grad_feat"] = segment_weighted_rows(col_ptr, row_ind, a_csc, grad_out.abs(), chunk)
+    del a_csc
+    ge = edge_dots(dst, src, grad_out, in_feat, chunk)
+    ws = segment_sums(row_ptr, alpha * ge)
+    gs = alpha * (ge - ws[dst]) * torch.where(d == 1.0, 1.0, negative_slope)
+    del ge, ws
+    res["grad_attn_row"] = segment_sums(row_ptr, gs)
+    res["grad_attn_col"] = segment_sums(col_ptr, gs[pm])
+    del gs
+    ge_a = edge_dots(dst, src, grad_out, in_feat, chunk, absolute=True)
+    ws_a = segment_sums(row_ptr, alpha * ge_a)
+    t_a = alpha * d * (ge_a + ws_a[dst])
+    del ge_a, ws_a
+    res["S_grad_attn_row"] = segment_sums(row_ptr, t_a)
+    res["S_grad_attn_col"] = segment_sums(col_ptr, t_a[pm])
+    return res
+
+
+def gat_layer_abs_sums(W, attn_l, attn_r, row_ptr, col_ind, negative_slope, feat, grad_out):
+    """gat_abs_sums carried through the dense part of the layer (gat_layer_ours): the projected features
+    are themselves sums, so their scale |feat| @ |W| takes the place of |in_feat|, and the parameter
+    gradients are the op-level scales pushed through |feat|, |W|, |attn|."""
+    hh, ff = attn_l.shape[1], attn_l.shape[2]
+    n = feat.shape[0]
+    h = torch.matmul(feat, W).view(-1, hh, ff)
+    s_h = torch.matmul(feat.abs(), W.abs()).view(-1, hh, ff)
+    s = gat_abs_sums((attn_l * h).sum(-1), (attn_r * h).sum(-1), row_ptr, col_ind, negative_slope, s_h, grad_out)
+    s_gh = s["grad_feat"] + s["grad_attn_row"].unsqueeze(-1) * attn_l.abs() + s["grad_attn_col"].unsqueeze(-1) * attn_r.abs()
+    return {"out": s["out"], "grad_feat": s_gh.view(n, -1) @ W.abs().t(), "grad_W": feat.abs().t() @ s_gh.view(n, -1),
+            "grad_attn_l": (s["grad_attn_row"].unsqueeze(-1) * s_h).sum(0, keepdim=True),
+            "grad_attn_r": (s["grad_attn_col"].unsqueeze(-1) * s_h).sum(0, keepdim=True)}
+
+
 # --------------------------------------------------------------------------- EdgeConv
 def edgeconv_forward(k, src_ind, h_src, h_dst):
     """out[i,f] = max_p (h_dst[i,f] + h_src[src_ind[p],f]), p in [i*k,(i+1)*k); argmax is the
@@ -182,6 +311,24 @@ def gmm_forward(row_ptr, col_ind, node_feat, pseudo, mu, inv_sigma):
     return torch.zeros_like(node_feat).index_add_(0, dst, msg)
 
 
+def gmm_abs_sums(row_ptr, col_ind, node_feat, pseudo, mu, inv_sigma, grad_out):
+    """Sum of |elementary summand| for every output of the fused GMMConv forward and backward
+    (see gat_abs_sums).  With gwA[p,k] = sum_f |g[i,k,f]| |x[j,k,f]| and t = pseudo - mu:
+      out sum_p w |x_j|;  grad_feat sum_i w |g_i|;  grad_pseudo[p,d] sum_k gwA w |t| s^2;
+      grad_mu[k,d] sum_p gwA w |t| s^2;  grad_sigma[k,d] sum_p gwA w t^2 |s|."""
+    dst = row_of_edge(row_ptr)
+    src = col_ind.to(torch.int64)
+    w = gaussian(pseudo, mu, inv_sigma)
+    ax, ag = node_feat.abs(), grad_out.abs()
+    s_out = torch.zeros_like(ax).index_add_(0, dst, w.unsqueeze(-1) * ax[src])
+    s_gx = torch.zeros_like(ax).index_add_(0, src, w.unsqueeze(-1) * ag[dst])
+    gw_a = ((ag[dst] * ax[src]).sum(-1) * w).unsqueeze(-1)                  # [E,K,1]
+    t = (pseudo.unsqueeze(1) - mu.unsqueeze(0)).abs()                       # [E,K,dim]
+    sg = inv_sigma.abs().unsqueeze(0)
+    return {"out": s_out, "grad_feat": s_gx, "grad_pseudo": (gw_a * t * sg * sg).sum(1),
+            "grad_mu": (gw_a * t * sg * sg).sum(0), "grad_sigma": (gw_a * t * t * sg).sum(0)}
+
+
 def gmm_layer_dgl(fc_weight, mu, inv_sigma, bias, row_ptr, col_ind, feat, pseudo, res_weight=None):
     """GMMConv_dgl.forward (layers/gmmconv_layer.py:130-149)."""
     kk = mu.shape[0]
@@ -193,6 +340,38 @@ def gmm_layer_dgl(fc_weight, mu, inv_sigma, bias, row_ptr, col_ind, feat, pseudo
     if bias is not None:
         rst = rst + bias
     return rst
+
+
+def gmm_layer_abs_sums(fc_weight, mu, inv_sigma, bias, row_ptr, col_ind, feat, pseudo, res_weight, grad_out):
+    """gmm_abs_sums carried through the dense part of gmm_layer_dgl (fc, sum over kernels, residual, bias)."""
+    kk = mu.shape[0]
+    n = feat.shape[0]
+    af, ag = feat.abs(), grad_out.abs()
+    s_h = (af @ fc_weight.abs().t()).view(n, kk, -1)
+    s = gmm_abs_sums(row_ptr, col_ind, s_h, pseudo, mu, inv_sigma, ag.unsqueeze(1).expand(-1, kk, -1))
+    out = s["out"].sum(1)
+    gfeat = s["grad_feat"].reshape(n, -1) @ fc_weight.abs()
+    res = {"grad_fc": s["grad_feat"].reshape(n, -1).t() @ af, "grad_pseudo": s["grad_pseudo"], "grad_mu": s["grad_mu"],
+           "grad_sigma": s["grad_sigma"], "grad_bias": ag.sum(0)}
+    if res_weight is not None:
+        out = out + af @ res_weight.abs().t()
+        gfeat = gfeat + ag @ res_weight.abs()
+        res["grad_res"] = ag.t() @ af
+    if bias is not None:
+        out = out + bias.abs()
+    res["out"] = out
+    res["grad_feat"] = gfeat
+    return res
+
+
+def multilinear_abs_sums(fn, inputs, grad_out):
+    """For an operator that is a sum of products of its float inputs with no other sign in it (SpMM,
+    SDDMM, u_add_v, a scatter-add): the scales of the output and of every input gradient are the operator
+    and its autograd evaluated on the absolute values.  Returns (S_out, [S_grad of every input])."""
+    leaves = [t.detach().abs().clone().requires_grad_(True) for t in inputs]
+    out = fn(*leaves)
+    out.backward(grad_out.abs())
+    return out.detach(), [t.grad for t in leaves]
 
 
 # --------------------------------------------------------------------------- csr2csc

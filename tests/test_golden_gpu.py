@@ -6,11 +6,23 @@ import numpy as np
 import pytest
 import torch
 
-from tests.util import assert_close
+from oracle import fgnn_oracle as orc
+from tests.util import assert_close, assert_close_sum, c_exp
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 HERE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _gat_check(d, got):
+    """(out, grad_x, grad_attn_row, grad_attn_col) against the fixture; the bar of every output comes from the sum of
+    its absolute summands (oracle.gat_abs_sums on the fixture's inputs)."""
+    h = {k: torch.from_numpy(d[k]).double() for k in ("attn_row", "attn_col", "x", "grad_out")}
+    s = orc.gat_abs_sums(h["attn_row"], h["attn_col"], torch.from_numpy(d["row_ptr"]), torch.from_numpy(d["col_ind"]), float(d["slope"]),
+                         h["x"], h["grad_out"])
+    c = c_exp(float(h["attn_row"].abs().max() + h["attn_col"].abs().max()))
+    for val, key, sk in zip(got, ("out", "grad_x", "grad_attn_row", "grad_attn_col"), ("out", "grad_feat", "grad_attn_row", "grad_attn_col")):
+        assert_close_sum(val, torch.from_numpy(d[key]), s[sk], key, c=c)
 
 
 def _t(a, dtype=None):
@@ -30,10 +42,7 @@ def test_gat_golden(name, variant):
     else:
         out = fg.fused_gat_stash_op(ar, ac, rp, ci, cp, ri, float(d["slope"]), x, pm)
     out.backward(_t(d["grad_out"]))
-    assert_close(out, torch.from_numpy(d["out"]), "out")
-    assert_close(x.grad, torch.from_numpy(d["grad_x"]), "grad_x")
-    assert_close(ar.grad, torch.from_numpy(d["grad_attn_row"]), "grad_attn_row", atol=1e-4)
-    assert_close(ac.grad, torch.from_numpy(d["grad_attn_col"]), "grad_attn_col", atol=1e-4)
+    _gat_check(d, (out, x.grad, ar.grad, ac.grad))
 
 
 def test_gat_backward_without_saved_aux_recomputes():
@@ -44,10 +53,7 @@ def test_gat_backward_without_saved_aux_recomputes():
     rp, ci, cp, ri = (_t(d[k]) for k in ("row_ptr", "col_ind", "col_ptr", "row_ind"))
     out, emax, esum, _, _, _, _ = gat_native.gat_forward(ar, ac, rp, ci, float(d["slope"]), x, need_aux=False)
     gx, gar, gac = gat_native.gat_backward(float(d["slope"]), rp, ci, cp, ri, emax, esum, x, ar, ac, _t(d["grad_out"]))
-    assert_close(out, torch.from_numpy(d["out"]), "out")
-    assert_close(gx, torch.from_numpy(d["grad_x"]), "grad_x")
-    assert_close(gar, torch.from_numpy(d["grad_attn_row"]), "grad_attn_row", atol=1e-4)
-    assert_close(gac, torch.from_numpy(d["grad_attn_col"]), "grad_attn_col", atol=1e-4)
+    _gat_check(d, (out, gx, gar, gac))
 
 
 def test_gat_is_bit_reproducible():
@@ -79,11 +85,12 @@ def test_gmm_golden():
     rp, ci, cp, ri, pm = (_t(d[k]) for k in ("row_ptr", "col_ind", "col_ptr", "row_ind", "permute"))
     out = fg.GmmConvFuse(rp, ci, cp, ri, pm, *leaves)
     out.backward(_t(d["grad_out"]))
-    assert_close(out, torch.from_numpy(d["out"]), "out")
-    assert_close(leaves[0].grad, torch.from_numpy(d["grad_x"]), "grad_x")
-    assert_close(leaves[1].grad, torch.from_numpy(d["grad_pseudo"]), "grad_pseudo", atol=1e-4)
-    assert_close(leaves[2].grad, torch.from_numpy(d["grad_mu"]), "grad_mu", rtol=1e-3, atol=1e-2)
-    assert_close(leaves[3].grad, torch.from_numpy(d["grad_sigma"]), "grad_sigma", rtol=1e-3, atol=1e-2)
+    h = [torch.from_numpy(d[k]).double() for k in ("x", "pseudo", "mu", "inv_sigma", "grad_out")]
+    s = orc.gmm_abs_sums(torch.from_numpy(d["row_ptr"]), torch.from_numpy(d["col_ind"]), *h)
+    c = c_exp(float((0.5 * (((h[1].unsqueeze(1) - h[2].unsqueeze(0)) * h[3].unsqueeze(0)) ** 2).sum(-1)).max()))
+    for val, key, sk in zip((out,) + tuple(t.grad for t in leaves), ("out", "grad_x", "grad_pseudo", "grad_mu", "grad_sigma"),
+                            ("out", "grad_feat", "grad_pseudo", "grad_mu", "grad_sigma")):
+        assert_close_sum(val, torch.from_numpy(d[key]), s[sk], key, c=c)
 
 
 def test_csr2csc_golden_bit_exact():

@@ -6,7 +6,7 @@ import torch
 
 from oracle import fgnn_oracle as orc
 from oracle import c_oracle
-from tests.util import assert_close, custom_graph, degree_edge_graph
+from tests.util import assert_close, assert_close_sum, c_exp, custom_graph, degree_edge_graph
 from ae_mlsys_gnn_amd import graphs
 
 pytestmark = pytest.mark.gpu
@@ -106,8 +106,12 @@ def test_edgeconv_backward_and_layer():
     out = layer(k, src.to(DEV), x.to(DEV))
     out.backward(go.float().to(DEV))
     assert_close(out, ref.detach(), "edgeconv out")
-    assert_close(layer.theta.weight.grad, th.grad, "theta grad", atol=1e-4)
-    assert_close(layer.phi.weight.grad, ph.grad, "phi grad", atol=1e-4)
+    # the weight gradients are sums over the 192 points (and, for theta, the scattered neighbours) of terms
+    # of either sign: bar from the sum of their absolute values
+    _, arg = orc.edgeconv_forward(k, src, h_src.detach(), h_dst.detach())
+    gsrc_abs = orc.edgeconv_backward(arg, go.abs(), xd.shape[0])[0]
+    assert_close_sum(layer.theta.weight.grad, th.grad, (gsrc_abs + go.abs()).t() @ xd.abs(), "theta grad")
+    assert_close_sum(layer.phi.weight.grad, ph.grad, go.abs().t() @ xd.abs(), "phi grad")
 
 
 def test_edgeconv_backward_scatter_exact_counts():
@@ -129,6 +133,28 @@ def _gmm_case(g, k, dim, f, seed):
     isg = 0.5 + torch.rand(k, dim, generator=gen, dtype=torch.float64)
     go = torch.randn(g.n, k, f, generator=gen, dtype=torch.float64)
     return x, pseudo, mu, isg, go
+
+
+def _gmm_c(pseudo, mu, isg):
+    """Constant of the derived bar for Gaussian weights: grows with the largest exponent magnitude."""
+    v = 0.5 * (((pseudo.detach().double().unsqueeze(1) - mu.detach().double().unsqueeze(0)) * isg.detach().double().unsqueeze(0)) ** 2).sum(-1)
+    return c_exp(float(v.max())) if v.numel() else c_exp(0.0)
+
+
+def _gmm_check(got, want, g, x, pseudo, mu, isg, go, tag="", summed=False, shared=False):
+    """(out, grad_feat, grad_pseudo, grad_mu, grad_sigma) against the oracle under the derived bar (rtol 1e-4 plus
+    the rounding scale of each output's sum of absolute summands).  summed: the sum over the kernels is fused
+    (out and go are [N,F]); shared: one [N,F] feature matrix serves all kernels."""
+    k = mu.shape[0]
+    xs = x.detach().unsqueeze(1).expand(-1, k, -1) if shared else x.detach()
+    gs = go.unsqueeze(1).expand(-1, k, -1) if summed else go
+    s = orc.gmm_abs_sums(g.row_ptr, g.col_ind, xs, pseudo.detach(), mu.detach(), isg.detach(), gs)
+    scales = (s["out"].sum(1) if summed else s["out"], s["grad_feat"].sum(1) if shared else s["grad_feat"], s["grad_pseudo"],
+              s["grad_mu"], s["grad_sigma"])
+    c = _gmm_c(pseudo, mu, isg)
+    for val, ref, sc, name in zip(got, want, scales, ("out", "grad node_feat", "grad pseudo", "grad mu", "grad inv_sigma")):
+        if val is not None:
+            assert_close_sum(val, ref, sc, "gmm " + name + tag, c=c)
 
 
 @pytest.mark.parametrize("k,dim,f,variant", [(3, 2, 64, "fuse"), (2, 1, 16, "fuse"), (3, 2, 64, "stash"), (1, 3, 47, "fuse"),
@@ -165,12 +191,8 @@ def test_gmm_forward_backward(k, dim, f, variant, monkeypatch):
         ref.backward(go)
     out.backward(go.float().to(DEV))
     _lib.clear_schedule_cache()
-    assert_close(out, ref.detach(), "gmm out", atol=1e-4 if variant == "sum" else 1e-5)
-    assert_close(dl[0].grad, leaves[0].grad, "grad node_feat")
-    assert_close(dl[1].grad, leaves[1].grad, "grad pseudo", atol=1e-4)
-    # sums over all E edges: absolute bar scales with the number of summands
-    assert_close(dl[2].grad, leaves[2].grad, "grad mu", rtol=1e-3, atol=1e-2)
-    assert_close(dl[3].grad, leaves[3].grad, "grad inv_sigma", rtol=1e-3, atol=1e-2)
+    _gmm_check((out, dl[0].grad, dl[1].grad, dl[2].grad, dl[3].grad), (ref.detach(),) + tuple(t.grad for t in leaves),
+               g, x, pseudo, mu, isg, go, summed=variant == "sum")
 
 
 @pytest.mark.parametrize("k,dim,f", [(2, 1, 16), (3, 2, 64), (4, 3, 32), (1, 1, 128), (2, 2, 256), (3, 2, 4), (2, 1, 44), (4, 1, 100), (1, 2, 8)])
@@ -196,11 +218,8 @@ def test_gmm_aggregate_shared_features(k, dim, f, monkeypatch):
         out = fg.GmmAggregate(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, *dl)
         assert out.shape == (g.n, k, f)
         out.backward(go.float().to(DEV))
-        assert_close(out, ref.detach(), "aggregate out (buckets %s)" % buckets, atol=1e-5)
-        assert_close(dl[0].grad, leaves[0].grad, "grad feat", atol=1e-4)
-        assert_close(dl[1].grad, leaves[1].grad, "grad pseudo", atol=1e-4)
-        assert_close(dl[2].grad, leaves[2].grad, "grad mu", rtol=1e-3, atol=1e-2)
-        assert_close(dl[3].grad, leaves[3].grad, "grad inv_sigma", rtol=1e-3, atol=1e-2)
+        _gmm_check((out, dl[0].grad, dl[1].grad, dl[2].grad, dl[3].grad), (ref.detach(),) + tuple(t.grad for t in leaves),
+                   g, x, pseudo, mu, isg, go, tag=" (aggregate, buckets %s)" % buckets, shared=True)
     _lib.clear_schedule_cache()
     # through the C ABI without a schedule (one wave per row)
     direct = torch.empty(g.n, k, f, device=DEV)
@@ -209,8 +228,8 @@ def test_gmm_aggregate_shared_features(k, dim, f, monkeypatch):
                                             _lib.ptr(dl[1]), _lib.ptr(dl[2]), _lib.ptr(dl[3]), _lib.ptr(direct), None, 2, None, None, 0,
                                             _lib.stream_ptr()), "fgnn_gmm_forward")
     torch.cuda.synchronize()
-    # rows of up to 3000 entries summed by one wave in one go: the absolute bar of the summed variants
-    assert_close(direct, ref.detach(), "aggregate out (no schedule)", atol=1e-4)
+    _gmm_check((direct, None, None, None, None), (ref.detach(),) + tuple(t.grad for t in leaves), g, x, pseudo, mu, isg, go,
+               tag=" (aggregate, no schedule)", shared=True)
     assert not fg.gmm_native.shared_supported(5, 16) and not fg.gmm_native.shared_supported(2, 18) and not fg.gmm_native.shared_supported(2, 260)
     with pytest.raises(_lib.FgnnError, match="shared node features"):
         fg.gmm_native.gmmconv_shared(gd.row_ptr, gd.col_ind, torch.zeros(g.n, 18, device=DEV), torch.zeros(g.n_edges, 1, device=DEV),
@@ -234,9 +253,14 @@ def test_gaussian_op(e, k, dim):
     out = fg.GaussianCp(*dl)
     out.backward(go.float().to(DEV))
     assert_close(out, ref.detach(), "gaussian")
-    assert_close(dl[0].grad, leaves[0].grad, "grad pseudo")
-    assert_close(dl[1].grad, leaves[1].grad, "grad mu", rtol=1e-3, atol=1e-3)
-    assert_close(dl[2].grad, leaves[2].grad, "grad sigma", rtol=1e-3, atol=1e-3)
+    # closed-form derivatives, summed over k (pseudo) or over all edges (mu, sigma): scales = sums of |terms|
+    t = (pseudo.unsqueeze(1) - mu.unsqueeze(0)).abs()
+    gw = (go.abs() * ref.detach()).unsqueeze(-1)
+    s2 = (isg ** 2).unsqueeze(0)
+    c = _gmm_c(pseudo, mu, isg)
+    assert_close_sum(dl[0].grad, leaves[0].grad, (gw * t * s2).sum(1), "grad pseudo", c=c)
+    assert_close_sum(dl[1].grad, leaves[1].grad, (gw * t * s2).sum(0), "grad mu", c=c)
+    assert_close_sum(dl[2].grad, leaves[2].grad, (gw * t * t * isg.unsqueeze(0)).sum(0), "grad sigma", c=c)
 
 
 @pytest.mark.parametrize("fin,fout,k,dim,variant,agg_first", [(32, 16, 3, 2, "our", True), (32, 41, 2, 1, "our", True), (16, 24, 2, 1, "our", True),
@@ -267,14 +291,17 @@ def test_gmm_layer_matches_dgl_composed(fin, fout, k, dim, variant, agg_first):
     out = layer(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, pd)
     assert out.shape == (g.n, fout)
     out.backward(go.to(DEV))
-    assert_close(out, ref.detach(), "GMMConv layer", atol=1e-4)
-    assert_close(fd.grad, leaves[5].grad, "GMMConv grad feat", atol=1e-4)
-    assert_close(pd.grad, leaves[6].grad, "GMMConv grad pseudo", atol=1e-3)
-    # parameter gradients are sums over all nodes / edges of terms of either sign
-    for name, got, want in zip(("fc.weight", "mu", "inv_sigma", "bias", "res_fc.weight"),
-                               (layer.fc.weight.grad, layer.mu.grad, layer.inv_sigma.grad, layer.bias.grad, layer.res_fc.weight.grad),
-                               (l.grad for l in leaves[:5])):
-        assert_close(got, want, "GMMConv grad " + name, rtol=1e-3, atol=5e-2)
+    # every output is a sum of terms of either sign (rows, then all nodes / edges for the parameters): derived bar
+    d = [t.detach() for t in leaves]
+    s = orc.gmm_layer_abs_sums(d[0], d[1], d[2], d[3], g.row_ptr, g.col_ind, d[5], d[6], d[4], go.double())
+    c = _gmm_c(d[6], d[1], d[2])
+    assert_close_sum(out, ref.detach(), s["out"], "GMMConv layer", c=c)
+    assert_close_sum(fd.grad, leaves[5].grad, s["grad_feat"], "GMMConv grad feat", c=c)
+    assert_close_sum(pd.grad, leaves[6].grad, s["grad_pseudo"], "GMMConv grad pseudo", c=c)
+    for name, key, got, want in zip(("fc.weight", "mu", "inv_sigma", "bias", "res_fc.weight"), ("grad_fc", "grad_mu", "grad_sigma", "grad_bias", "grad_res"),
+                                    (layer.fc.weight.grad, layer.mu.grad, layer.inv_sigma.grad, layer.bias.grad, layer.res_fc.weight.grad),
+                                    (l.grad for l in leaves[:5])):
+        assert_close_sum(got, want, s[key], "GMMConv grad " + name, c=c)
 
 
 # ------------------------------------------------------------------ GAT layer vs the DGL-composed layer
@@ -299,21 +326,26 @@ def test_gat_layer_matches_dgl_composed(fin, f, h, variant):
     out = layer(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, fd, True if variant == "our" else gd.permute)
     assert out.shape == (g.n, h, f)
     out.backward(go.to(DEV))
-    assert_close(out, ref.detach(), "GATConv layer")
-    assert_close(fd.grad, leaves[3].grad, "GATConv grad feat", atol=1e-4)
-    # parameter gradients are sums over 4096 nodes (and their edges) of terms of either sign
-    assert_close(layer.W.grad, leaves[0].grad, "GATConv grad W", rtol=1e-4, atol=2e-3)
-    assert_close(layer.attn_l.grad, leaves[1].grad, "GATConv grad attn_l", rtol=1e-4, atol=2e-3)
-    assert_close(layer.attn_r.grad, leaves[2].grad, "GATConv grad attn_r", rtol=1e-4, atol=2e-3)
+    # projected features, outputs and gradients are all sums of terms of either sign (over the input width, the
+    # neighbours, then the 4096 nodes for the parameters): derived bar from the sums of absolute summands
+    d = [t.detach() for t in leaves]
+    s = orc.gat_layer_abs_sums(d[0], d[1], d[2], g.row_ptr, g.col_ind, 0.2, d[3], go.double())
+    hp = (d[3] @ d[0]).view(-1, h, f)
+    c = c_exp(float((d[1] * hp).sum(-1).abs().max() + (d[2] * hp).sum(-1).abs().max()))
+    assert_close_sum(out, ref.detach(), s["out"], "GATConv layer", c=c)
+    assert_close_sum(fd.grad, leaves[3].grad, s["grad_feat"], "GATConv grad feat", c=c)
+    assert_close_sum(layer.W.grad, leaves[0].grad, s["grad_W"], "GATConv grad W", c=c)
+    assert_close_sum(layer.attn_l.grad, leaves[1].grad, s["grad_attn_l"], "GATConv grad attn_l", c=c)
+    assert_close_sum(layer.attn_r.grad, leaves[2].grad, s["grad_attn_r"], "GATConv grad attn_r", c=c)
     # as a first layer (input without gradient: the backward reduces the two gradient parts separately)
     for p_ in layer.parameters():
         p_.grad = None
     out = layer(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, feat.to(DEV), True if variant == "our" else gd.permute)
     out.backward(go.to(DEV))
-    assert_close(out, ref.detach(), "GATConv layer (first layer)")
-    assert_close(layer.W.grad, leaves[0].grad, "GATConv grad W (first layer)", rtol=1e-4, atol=2e-3)
-    assert_close(layer.attn_l.grad, leaves[1].grad, "GATConv grad attn_l (first layer)", rtol=1e-4, atol=2e-3)
-    assert_close(layer.attn_r.grad, leaves[2].grad, "GATConv grad attn_r (first layer)", rtol=1e-4, atol=2e-3)
+    assert_close_sum(out, ref.detach(), s["out"], "GATConv layer (first layer)", c=c)
+    assert_close_sum(layer.W.grad, leaves[0].grad, s["grad_W"], "GATConv grad W (first layer)", c=c)
+    assert_close_sum(layer.attn_l.grad, leaves[1].grad, s["grad_attn_l"], "GATConv grad attn_l (first layer)", c=c)
+    assert_close_sum(layer.attn_r.grad, leaves[2].grad, s["grad_attn_r"], "GATConv grad attn_r (first layer)", c=c)
 
 
 # ------------------------------------------------------------------ small operators
@@ -337,9 +369,10 @@ def test_mhspmm_and_mhsddmm(h, f):
     fd, ad = feat.float().to(DEV).requires_grad_(True), att.float().to(DEV).requires_grad_(True)
     out = op.csrmhspmm(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, ad)
     out.backward(go.float().to(DEV))
-    assert_close(out, ref.detach(), "mhspmm", atol=1e-4)
-    assert_close(fd.grad, fl.grad, "mhspmm grad feat", atol=1e-4)
-    assert_close(ad.grad, al.grad, "mhspmm grad att (mhsddmm)", atol=1e-4)
+    s_out, (s_att, s_feat) = orc.multilinear_abs_sums(lambda a, x: orc.mhspmm(g.row_ptr, g.col_ind, a, x), (att, feat), go)
+    assert_close_sum(out, ref.detach(), s_out, "mhspmm")
+    assert_close_sum(fd.grad, fl.grad, s_feat, "mhspmm grad feat")
+    assert_close_sum(ad.grad, al.grad, s_att, "mhspmm grad att (mhsddmm)")
     tr = op.mhtranspose(gd.permute, ad.detach())
     assert torch.equal(tr.cpu(), att.float()[g.permute.long()])
 
@@ -372,8 +405,9 @@ def test_u_add_v():
     out = op.u_add_v_op(g.row_ptr.to(DEV), g.col_ind.to(DEV), rd, cd)
     out.backward(go.float().to(DEV))
     assert_close(out, ref.detach(), "u_add_v")
-    assert_close(rd.grad, rl.grad, "u_add_v grad row", atol=1e-4)
-    assert_close(cd.grad, cl.grad, "u_add_v grad col", atol=1e-4)
+    _, (s_row, s_col) = orc.multilinear_abs_sums(lambda a, b: orc.u_add_v(g.row_ptr, g.col_ind, a, b), (rv, cv), go)
+    assert_close_sum(rd.grad, rl.grad, s_row, "u_add_v grad row")
+    assert_close_sum(cd.grad, cl.grad, s_col, "u_add_v grad col")
 
 
 @pytest.mark.parametrize("weighted,sym", [(True, False), (False, False), (True, True)])
@@ -400,10 +434,14 @@ def test_csrspmm(weighted, sym):
     wd = None if w is None else w.float().to(DEV).requires_grad_(True)
     out = op.csrspmm(g.row_ptr.to(DEV), g.col_ind.to(DEV), xd, wd, sym)
     out.backward(go.float().to(DEV))
-    assert_close(out, ref.detach(), "csrspmm", atol=1e-4)
-    assert_close(xd.grad, xl.grad, "csrspmm grad x", atol=1e-4)
     if weighted:
-        assert_close(wd.grad, wl.grad, "csrspmm grad w", atol=1e-4)
+        s_out, (s_x, s_w) = orc.multilinear_abs_sums(lambda a, b: orc.spmm(g.row_ptr, g.col_ind, a, b), (x, w), go)
+    else:
+        s_out, (s_x,) = orc.multilinear_abs_sums(lambda a: orc.spmm(g.row_ptr, g.col_ind, a), (x,), go)
+    assert_close_sum(out, ref.detach(), s_out, "csrspmm")
+    assert_close_sum(xd.grad, xl.grad, s_x, "csrspmm grad x")
+    if weighted:
+        assert_close_sum(wd.grad, wl.grad, s_w, "csrspmm grad w")
 
 
 def test_error_paths_return_codes_not_aborts():
@@ -433,14 +471,14 @@ def test_coo_and_csr_sddmm(h, f):
     b = torch.randn(g.n, h, f, generator=gen, dtype=torch.float64)
     want = (a[rows.long()] * b[cols.long()]).sum(-1)
     got = sddmm.coo_sddmm(rows.to(DEV), cols.to(DEV), a.float().to(DEV), b.float().to(DEV))
-    assert_close(got, want, "coo_sddmm", atol=2e-5 * f ** 0.5)
+    assert_close_sum(got, want, (a[rows.long()].abs() * b[cols.long()].abs()).sum(-1), "coo_sddmm")
     if h == 1:
         got1 = sddmm.coo_sddmm(rows.to(DEV), cols.to(DEV), a[:, 0].float().to(DEV), b[:, 0].float().to(DEV))
         assert torch.equal(got1, got[:, 0])
         dst = torch.repeat_interleave(torch.arange(g.n), (g.row_ptr[1:] - g.row_ptr[:-1]).long())
         want_csr = (a[dst, 0] * b[g.col_ind.long(), 0]).sum(-1)
         got_csr = sddmm.csr_sddmm(g.row_ptr.to(DEV), g.col_ind.to(DEV), a[:, 0].float().to(DEV), b[:, 0].float().to(DEV))
-        assert_close(got_csr, want_csr, "csr_sddmm", atol=2e-5 * f ** 0.5)
+        assert_close_sum(got_csr, want_csr, (a[dst, 0].abs() * b[g.col_ind.long(), 0].abs()).sum(-1), "csr_sddmm")
     assert sddmm.coo_sddmm(rows[:0].to(DEV), cols[:0].to(DEV), a.float().to(DEV), b.float().to(DEV)).shape == (0, h)
 
 
@@ -514,9 +552,10 @@ def test_edgeconv_backward_blocked(b, p, k, f, block):
     out, arg = edgeconv_native.edgeconv_forward(k, src, hs.to(DEV), hd.to(DEV))
     want = torch.zeros(n, f, dtype=torch.float64).scatter_add_(0, arg.cpu().long(), go.double())
     got = edgeconv_native.edgeconv_backward(go.to(DEV), arg, n, block=block)
-    assert_close(got, want, "blocked edgeconv backward", atol=1e-5)
+    s_abs = torch.zeros(n, f, dtype=torch.float64).scatter_add_(0, arg.cpu().long(), go.double().abs())
+    assert_close_sum(got, want, s_abs, "blocked edgeconv backward")
     plain = edgeconv_native.edgeconv_backward(go.to(DEV), arg, n)
-    assert_close(plain, want, "plain edgeconv backward", atol=1e-5)
+    assert_close_sum(plain, want, s_abs, "plain edgeconv backward")
 
 
 def test_edgeconv_backward_blocked_with_a_wrong_hint():
@@ -534,7 +573,8 @@ def test_edgeconv_backward_blocked_with_a_wrong_hint():
     out = fused_edgeconv_op(k, src.to(DEV), hsd, hd.to(DEV), block=512)
     out.backward(go.to(DEV))
     assert torch.equal(out.detach().cpu(), ref.detach().float())
-    assert_close(hsd.grad, ref_s.grad, "grad_src with a wrong block hint", atol=1e-5)
+    _, arg = orc.edgeconv_forward(k, src, hs.double(), hd.double())
+    assert_close_sum(hsd.grad, ref_s.grad, orc.edgeconv_backward(arg, go.double().abs(), n)[0], "grad_src with a wrong block hint")
 
 
 # ------------------------------------------------------------------ coo2csr (bit-exact)
@@ -594,9 +634,10 @@ def test_mhspmm_and_gmm_with_xcd_buckets(monkeypatch):
     fd, ad = feat.float().to(DEV).requires_grad_(True), att.float().to(DEV).requires_grad_(True)
     out = op.csrmhspmm(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, ad)
     out.backward(go.float().to(DEV))
-    assert_close(out, ref.detach(), "mhspmm (buckets)", atol=2e-4)
-    assert_close(fd.grad, fl.grad, "mhspmm grad feat (buckets)", atol=2e-4)
-    assert_close(ad.grad, al.grad, "mhspmm grad att (buckets)", atol=2e-4)
+    s_out, (s_att, s_feat) = orc.multilinear_abs_sums(lambda a, x: orc.mhspmm(g.row_ptr, g.col_ind, a, x), (att, feat), go)
+    assert_close_sum(out, ref.detach(), s_out, "mhspmm (buckets)")
+    assert_close_sum(fd.grad, fl.grad, s_feat, "mhspmm grad feat (buckets)")
+    assert_close_sum(ad.grad, al.grad, s_att, "mhspmm grad att (buckets)")
     for (k, dim, f) in [(3, 2, 64), (2, 1, 16)]:            # a full-width row and one narrower than a wave
         x, pseudo, mu, isg, go = _gmm_case(g, k, dim, f, seed=2)
         leaves = [t.clone().requires_grad_(True) for t in (x, pseudo, mu, isg)]
@@ -605,11 +646,8 @@ def test_mhspmm_and_gmm_with_xcd_buckets(monkeypatch):
         dl = [t.float().to(DEV).requires_grad_(True) for t in (x, pseudo, mu, isg)]
         out = fg.GmmConvStash(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, *dl)
         out.backward(go.float().to(DEV))
-        assert_close(out, ref.detach(), "gmm out (buckets)", atol=1e-4)
-        assert_close(dl[0].grad, leaves[0].grad, "gmm grad node_feat (buckets)", atol=1e-4)
-        assert_close(dl[1].grad, leaves[1].grad, "gmm grad pseudo (buckets)", atol=1e-3)
-        assert_close(dl[2].grad, leaves[2].grad, "gmm grad mu (buckets)", rtol=1e-3, atol=5e-2)
-        assert_close(dl[3].grad, leaves[3].grad, "gmm grad inv_sigma (buckets)", rtol=1e-3, atol=5e-2)
+        _gmm_check((out, dl[0].grad, dl[1].grad, dl[2].grad, dl[3].grad), (ref.detach(),) + tuple(t.grad for t in leaves),
+                   g, x, pseudo, mu, isg, go, tag=" (buckets)")
     _lib.clear_schedule_cache()
 
 
@@ -676,12 +714,15 @@ def test_gmm_layer_with_csc_ordered_pseudo(k, dim, f, monkeypatch):
         pc = pd[gd.permute.long()].contiguous().requires_grad_(True)
         out = layer(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, pd, pseudo_csc=pc)
         out.backward(go.to(DEV))
-        assert_close(out, ref.detach(), "GMMConv (two orders)", atol=1e-4)
-        assert_close(fd.grad, leaves[4].grad, "grad feat (two orders)", atol=1e-4)
-        assert_close(pc.grad, leaves[5].grad[g.permute.long()], "grad pseudo in CSC order", atol=1e-3)
-        assert_close(layer.mu.grad, leaves[1].grad, "grad mu (two orders)", rtol=1e-3, atol=5e-2)
-        assert_close(layer.inv_sigma.grad, leaves[2].grad, "grad inv_sigma (two orders)", rtol=1e-3, atol=5e-2)
-        assert_close(layer.fc.weight.grad, leaves[0].grad, "grad fc (two orders)", rtol=1e-3, atol=5e-2)
+        d = [t.detach() for t in leaves]
+        s = orc.gmm_layer_abs_sums(d[0], d[1], d[2], d[3], g.row_ptr, g.col_ind, d[4], d[5], None, go.double())
+        c = _gmm_c(d[5], d[1], d[2])
+        assert_close_sum(out, ref.detach(), s["out"], "GMMConv (two orders)", c=c)
+        assert_close_sum(fd.grad, leaves[4].grad, s["grad_feat"], "grad feat (two orders)", c=c)
+        assert_close_sum(pc.grad, leaves[5].grad[g.permute.long()], s["grad_pseudo"][g.permute.long()], "grad pseudo in CSC order", c=c)
+        assert_close_sum(layer.mu.grad, leaves[1].grad, s["grad_mu"], "grad mu (two orders)", c=c)
+        assert_close_sum(layer.inv_sigma.grad, leaves[2].grad, s["grad_sigma"], "grad inv_sigma (two orders)", c=c)
+        assert_close_sum(layer.fc.weight.grad, leaves[0].grad, s["grad_fc"], "grad fc (two orders)", c=c)
     _lib.clear_schedule_cache()
 
 
@@ -728,15 +769,18 @@ def test_gmm_layer_with_pseudo_in_schedule_order(k, dim, f, stash, monkeypatch):
         pc = pseudo.to(DEV)[to_csc].contiguous().requires_grad_(True)
         out = layer(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, pd, pseudo_csc=pc, own_order=True)
         out.backward(go.to(DEV))
-        assert_close(out, ref.detach(), "GMMConv (schedule order)", atol=1e-4)
-        assert_close(fd.grad, leaves[4].grad, "grad feat (schedule order)", atol=1e-4)
-        assert_close(pc.grad, leaves[5].grad[to_csc.cpu()], "grad pseudo in the backward schedule's order", atol=1e-3)
-        assert_close(layer.mu.grad, leaves[1].grad, "grad mu (schedule order)", rtol=1e-3, atol=5e-2)
-        assert_close(layer.inv_sigma.grad, leaves[2].grad, "grad inv_sigma (schedule order)", rtol=1e-3, atol=5e-2)
-        assert_close(layer.fc.weight.grad, leaves[0].grad, "grad fc (schedule order)", rtol=1e-3, atol=5e-2)
+        d = [t.detach() for t in leaves]
+        s = orc.gmm_layer_abs_sums(d[0], d[1], d[2], d[3], g.row_ptr, g.col_ind, d[4], d[5], None, go.double())
+        c = _gmm_c(d[5], d[1], d[2])
+        assert_close_sum(out, ref.detach(), s["out"], "GMMConv (schedule order)", c=c)
+        assert_close_sum(fd.grad, leaves[4].grad, s["grad_feat"], "grad feat (schedule order)", c=c)
+        assert_close_sum(pc.grad, leaves[5].grad[to_csc.cpu()], s["grad_pseudo"][to_csc.cpu()], "grad pseudo in the backward schedule's order", c=c)
+        assert_close_sum(layer.mu.grad, leaves[1].grad, s["grad_mu"], "grad mu (schedule order)", c=c)
+        assert_close_sum(layer.inv_sigma.grad, leaves[2].grad, s["grad_sigma"], "grad inv_sigma (schedule order)", c=c)
+        assert_close_sum(layer.fc.weight.grad, leaves[0].grad, s["grad_fc"], "grad fc (schedule order)", c=c)
         with torch.no_grad():
-            assert_close(layer(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, pd, own_order=True), ref.detach(),
-                         "GMMConv forward only (schedule order)", atol=1e-4)
+            assert_close_sum(layer(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, pd, own_order=True), ref.detach(),
+                             s["out"], "GMMConv forward only (schedule order)", c=c)
         with pytest.raises(ValueError, match="forward-only"):
             layer(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, pd, own_order=True)
     _lib.clear_schedule_cache()
@@ -780,7 +824,8 @@ def test_schedule_take_positions_c_abi(monkeypatch):
                                        _lib.ptr(out), s.handle, _lib.ptr(ws), wsb, _lib.stream_ptr()), "fgnn_mhspmm")
     torch.cuda.synchronize()
     want = orc.mhspmm(g.row_ptr.cpu(), g.col_ind.cpu(), w.cpu().double(), x.cpu().double())
-    assert_close(out, want, "mhspmm under an own-order schedule", atol=1e-4)
+    assert_close_sum(out, want, orc.mhspmm(g.row_ptr.cpu(), g.col_ind.cpu(), w.cpu().double(), x.cpu().double().abs()),
+                     "mhspmm under an own-order schedule")
 
 
 @pytest.mark.parametrize("d", [1, 2, 3, 4])
@@ -801,11 +846,11 @@ def test_edge_linear_tanh_matches_torch(d, e):
     bd = b.detach().float().to(DEV).requires_grad_(True)
     got = edge_proj.edge_linear_tanh(xd, wd, bd)
     got.backward(go.float().to(DEV))
-    assert_close(got, want, "y", atol=2e-6)
-    # sums of e terms of either sign: the absolute bar scales with sqrt(e) summands of magnitude ~|go|
-    bar = 1e-5 * max(1.0, float(go.abs().max()) * e ** 0.5)
-    assert_close(wd.grad, w.grad, "grad_W", atol=bar)
-    assert_close(bd.grad, b.grad, "grad_b", atol=bar)
+    assert_close(got, want, "y")
+    # sums over the e edges of terms of either sign: derived bar from the sums of their absolute values
+    gt = (go * (1 - want.detach() ** 2)).abs()
+    assert_close_sum(wd.grad, w.grad, gt.t() @ x.abs(), "grad_W")
+    assert_close_sum(bd.grad, b.grad, gt.sum(0), "grad_b")
     w2 = wd.detach().clone().requires_grad_(True)
     b2 = bd.detach().clone().requires_grad_(True)
     edge_proj.edge_linear_tanh(xd, w2, b2).backward(go.float().to(DEV))

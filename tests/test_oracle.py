@@ -195,6 +195,117 @@ def test_gmm_special_cases_and_c_oracle():
     _close(leaves[0].grad, gx); _close(leaves[1].grad, gp, 1e-9); _close(leaves[2].grad, gm, 1e-9); _close(leaves[3].grad, gs, 1e-9)
 
 
+def test_gmm_layer_dgl_reduces_to_scipy_spmm():
+    """K = 1 and inv_sigma = 0 (every Gaussian weight is 1), no bias, no residual: the layer of
+    layers/gmmconv_layer.py:130-149 is A @ (feat @ W.T) with A the 0/1 adjacency."""
+    g = graphs.rmat_graph(70, 600, seed=12)
+    gen = torch.Generator().manual_seed(5)
+    fin, fout = 6, 5
+    feat = torch.randn(g.n, fin, generator=gen, dtype=torch.float64)
+    w = torch.randn(fout, fin, generator=gen, dtype=torch.float64)
+    ps = torch.rand(g.n_edges, 2, generator=gen, dtype=torch.float64)
+    mu = torch.rand(1, 2, generator=gen, dtype=torch.float64)
+    a = sp.csr_matrix((np.ones(g.n_edges), g.col_ind.numpy(), g.row_ptr.numpy()), shape=(g.n, g.n))
+    _close(orc.gmm_layer_dgl(w, mu, torch.zeros(1, 2, dtype=torch.float64), None, g.row_ptr, g.col_ind, feat, ps),
+           a @ (feat.numpy() @ w.numpy().T))
+
+
+def test_gmm_layer_dgl_hand_built_with_residual_bias_and_view_order():
+    """3 nodes, 4 edges, K = 2, out = 2, dim = 1, worked out with python loops and math.exp.  Kernel k
+    uses rows [k*out, (k+1)*out) of fc.weight (the `view(-1, K, out)` of layers/gmmconv_layer.py:133);
+    reading the same fc output as (out, K) gives another number, so a swapped view cannot pass."""
+    import math
+    rows = [[1, 2], [0], [2]]                       # destination -> sources, CSR order
+    g = custom_graph(rows)
+    kk, fout, fin = 2, 2, 2
+    feat = [[1.0, 2.0], [0.5, -1.0], [-2.0, 0.25]]
+    wfc = [[1.0, 0.0], [0.0, 1.0], [2.0, -1.0], [0.5, 0.5]]          # [K*out, in]
+    wres = [[0.1, 0.2], [-0.3, 0.4]]
+    bias = [0.5, -0.25]
+    pseudo = [0.2, 0.9, 0.4, 0.7]                   # one coordinate per CSR position
+    mu = [0.1, 0.8]
+    isg = [2.0, 0.5]
+
+    def layer(view_k_major=True):
+        out = [[0.0] * fout for _ in range(3)]
+        pos = 0
+        for i, srcs in enumerate(rows):
+            for j in srcs:
+                fc = [sum(wfc[r][c] * feat[j][c] for c in range(fin)) for r in range(kk * fout)]
+                for k in range(kk):
+                    wgt = math.exp(-0.5 * ((pseudo[pos] - mu[k]) * isg[k]) ** 2)
+                    for o in range(fout):
+                        out[i][o] += wgt * (fc[k * fout + o] if view_k_major else fc[o * kk + k])
+                pos += 1
+            for o in range(fout):
+                out[i][o] += sum(wres[o][c] * feat[i][c] for c in range(fin)) + bias[o]
+        return out
+
+    t = lambda v: torch.tensor(v, dtype=torch.float64)
+    got = orc.gmm_layer_dgl(t(wfc), t(mu).view(kk, 1), t(isg).view(kk, 1), t(bias), g.row_ptr, g.col_ind, t(feat),
+                            t(pseudo).view(-1, 1), t(wres))
+    _close(got, layer(True), 1e-14)
+    assert float((got - t(layer(False))).abs().max()) > 0.1
+    # residual and bias really are added: dropping either changes every row
+    no_res = orc.gmm_layer_dgl(t(wfc), t(mu).view(kk, 1), t(isg).view(kk, 1), t(bias), g.row_ptr, g.col_ind, t(feat), t(pseudo).view(-1, 1))
+    no_bias = orc.gmm_layer_dgl(t(wfc), t(mu).view(kk, 1), t(isg).view(kk, 1), None, g.row_ptr, g.col_ind, t(feat), t(pseudo).view(-1, 1), t(wres))
+    _close(got - no_res, t(feat) @ t(wres).t(), 1e-14)
+    _close(got - no_bias, t(bias).view(1, -1).expand(3, -1), 1e-14)
+
+
+# ------------------------------------------------------------------ the error-bound scales (sums of |summands|)
+def test_abs_sums_equal_outputs_for_non_negative_inputs_and_bound_them_otherwise():
+    g = graphs.rmat_graph(60, 500, seed=13)
+    x, ar, ac, go = gat_inputs(g, 2, 4, 5)
+    slope = 0.2
+    # slope = 1 and non-negative features / gradients: forward sums have no cancellation, so S == output
+    s = orc.gat_abs_sums(ar, ac, g.row_ptr, g.col_ind, 1.0, x.abs(), go.abs())
+    xr = x.abs().clone().requires_grad_(True)
+    out = orc.gat_forward(ar, ac, g.row_ptr, g.col_ind, 1.0, xr)
+    out.backward(go.abs())
+    _close(s["out"], out.detach()); _close(s["grad_feat"], xr.grad)
+    # general signs: S bounds |output| for every output, and is strictly larger somewhere
+    leaves = [t.clone().requires_grad_(True) for t in (ar, ac, x)]
+    out = orc.gat_forward(leaves[0], leaves[1], g.row_ptr, g.col_ind, slope, leaves[2])
+    out.backward(go)
+    s = orc.gat_abs_sums(ar, ac, g.row_ptr, g.col_ind, slope, x, go)
+    for name, val in (("out", out.detach()), ("grad_feat", leaves[2].grad), ("grad_attn_row", leaves[0].grad), ("grad_attn_col", leaves[1].grad)):
+        assert bool((s[name] >= val.abs() - 1e-12).all()), name
+        assert float((s[name] - val.abs()).max()) > 1e-3, name
+    # GMM: with x, g >= 0 the forward and grad_feat sums are cancellation-free; t >= 0 when pseudo >= mu
+    k, dim, f = 2, 2, 3
+    gen = torch.Generator().manual_seed(6)
+    xm = torch.rand(g.n, k, f, generator=gen, dtype=torch.float64)
+    gm = torch.rand(g.n, k, f, generator=gen, dtype=torch.float64)
+    ps = 1.0 + torch.rand(g.n_edges, dim, generator=gen, dtype=torch.float64)
+    mu = torch.rand(k, dim, generator=gen, dtype=torch.float64)
+    sg = 0.5 + torch.rand(k, dim, generator=gen, dtype=torch.float64)
+    lv = [t.clone().requires_grad_(True) for t in (xm, ps, mu, sg)]
+    o = orc.gmm_forward(g.row_ptr, g.col_ind, *lv)
+    o.backward(gm)
+    sm = orc.gmm_abs_sums(g.row_ptr, g.col_ind, xm, ps, mu, sg, gm)
+    _close(sm["out"], o.detach()); _close(sm["grad_feat"], lv[0].grad)
+    _close(sm["grad_mu"], lv[2].grad.abs(), 1e-9); _close(sm["grad_sigma"], lv[3].grad.abs(), 1e-9); _close(sm["grad_pseudo"], lv[1].grad.abs(), 1e-9)
+
+
+@pytest.mark.parametrize("chunk", [5, 64, 1 << 20])
+def test_gat_reference_chunked_equals_autograd_oracle(chunk):
+    """The chunked float64 form used at full size (no [E,H,F] tensor, analytic backward) against gat_forward +
+    autograd and gat_abs_sums; the graph has empty rows, a hub and duplicate edges, the chunks cut rows."""
+    g = graphs.add_csc_torch(degree_edge_graph(n=90, seed=8))
+    x, ar, ac, go = gat_inputs(g, 2, 5, 6)
+    for slope in (0.2, 1.0):
+        leaves = [t.clone().requires_grad_(True) for t in (ar, ac, x)]
+        out = orc.gat_forward(leaves[0], leaves[1], g.row_ptr, g.col_ind, slope, leaves[2])
+        out.backward(go)
+        s = orc.gat_abs_sums(ar, ac, g.row_ptr, g.col_ind, slope, x, go)
+        r = orc.gat_reference_chunked(ar.float(), ac.float(), g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, g.permute, slope, x.float(), go.float(),
+                                      chunk=chunk)
+        for name, want in (("out", out.detach()), ("grad_feat", leaves[2].grad), ("grad_attn_row", leaves[0].grad), ("grad_attn_col", leaves[1].grad)):
+            _close(r[name], want, 1e-6)              # inputs went through float32
+            _close(r["S_" + name], s[name], 1e-6)
+
+
 # ------------------------------------------------------------------ csr2csc
 @pytest.mark.parametrize("seed", [0, 1])
 def test_csr2csc_vs_scipy_bruteforce_and_c(seed):

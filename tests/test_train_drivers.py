@@ -44,7 +44,7 @@ def test_graph_cache_round_trip_and_point_cloud_files(tmp_path):
     assert h.n == g.n and all(torch.equal(getattr(g, k), getattr(h, k)) for k in ("row_ptr", "col_ind", "col_ptr", "row_ind", "permute"))
     np.savez(tmp_path / "bad.npz", n=np.int64(50), row_ptr=g.row_ptr.numpy()[:-1], col_ind=g.col_ind.numpy(), col_ptr=g.col_ptr.numpy(),
              row_ind=g.row_ind.numpy(), permute=g.permute.numpy())
-    with pytest.raises(ValueError, match="inconsistent"):
+    with pytest.raises(ValueError, match="entries, expected"):
         datasets.load_graph(str(tmp_path / "bad.npz"), "cpu")
     data = np.random.default_rng(0).standard_normal((6, 40, 3)).astype(np.float32)
     np.savez(tmp_path / "clouds.npz", data=data, label=np.array([[0], [3], [1], [2], [3], [0]]))
@@ -54,6 +54,51 @@ def test_graph_cache_round_trip_and_point_cloud_files(tmp_path):
     assert s.source == "synthetic" and s.data.shape == (5, 16, 3) and float(s.data.abs().max()) <= 1
     with pytest.raises(RuntimeError, match="h5py"):
         datasets.load_point_clouds("cpu", str(tmp_path / "clouds.h5"))
+
+
+def test_malformed_graphs_are_rejected_on_the_host_before_any_kernel(tmp_path):
+    """Node ids outside [0, n), int64 ids that an int32 cast would wrap into range, broken pointer arrays and
+    permutations: the loaders raise ValueError from host-side reductions; nothing is handed to the device (the
+    target device here is the CPU, which the operators refuse, so reaching them would raise FgnnError instead)."""
+    from ae_mlsys_gnn_amd.train import datasets
+    n = 20
+    src = torch.arange(n, dtype=torch.int64)
+    dst = torch.flip(src, [0])
+    for bad_src, bad_dst, msg in ((src.clone().index_fill_(0, torch.tensor([3]), n), dst, r"src ids must lie in \[0, 20\)"),
+                                  (src, dst.clone().index_fill_(0, torch.tensor([0]), -1), r"dst ids must lie"),
+                                  (src.clone().index_fill_(0, torch.tensor([5]), (1 << 32) + 4), dst, r"src ids must lie"),   # wraps to 4 as int32
+                                  (src.double(), dst, "integer array"), (src[:-1], dst, "sources for")):
+        with pytest.raises(ValueError, match=msg):
+            datasets.graph_from_edges(bad_src, bad_dst, n, "cpu")
+    g = graphs.add_csc_torch(graphs.uniform_graph(n, 90, seed=2))
+    good = {k: getattr(g, k).numpy().copy() for k in ("row_ptr", "col_ind", "col_ptr", "row_ind", "permute")}
+    graphs.validate_graph(g)
+
+    def broken(key, fn, match):
+        arr = {k: v.copy() for k, v in good.items()}
+        fn(arr[key])
+        np.savez(tmp_path / "b.npz", n=np.int64(n), **arr)
+        with pytest.raises(ValueError, match=match):
+            datasets.load_graph(str(tmp_path / "b.npz"), "cpu")
+
+    def set_(i, v):
+        def f(a):
+            a[i] = v
+        return f
+    broken("col_ind", set_(7, n), "node ids must lie")
+    broken("row_ind", set_(0, -2), "node ids must lie")
+    broken("row_ptr", set_(3, good["row_ptr"][4] + 1), "never decrease")
+    broken("row_ptr", set_(0, 1), "start at 0")
+    broken("col_ptr", set_(n, good["col_ptr"][n] + 5), "end at E")
+    broken("permute", set_(2, g.n_edges), "permute entries")
+    arr = dict(good, col_ind=good["col_ind"].astype(np.float32))
+    np.savez(tmp_path / "b.npz", n=np.int64(n), **arr)
+    with pytest.raises(ValueError, match="integer arrays"):
+        datasets.load_graph(str(tmp_path / "b.npz"), "cpu")
+    # the C-ABI check refuses bad sizes without a GPU (its kernel path is covered by the GPU tests)
+    from ae_mlsys_gnn_amd import _lib
+    assert _lib.lib().fgnn_validate_graph(None, None, 4, 4, 3, None) == -1
+    assert _lib.lib().fgnn_schedule_device_bytes(None) == 0
 
 
 def test_driver_command_lines_and_loss():

@@ -23,6 +23,39 @@ def assert_close(got, ref, what, rtol=RTOL, atol=ATOL):
             float(got.flatten()[i]), float(ref.flatten()[i])))
 
 
+# Outputs that are sums of terms of either sign (the score / parameter gradients: up to E summands that
+# largely cancel) cannot be held to a bar relative to the RESULT: fp32 rounding scales with the sum of
+# the absolute summands S.  Their bar is  rtol*|ref| + max(atol, C_SUM * 2^-24 * S)  with S from the
+# oracle (gat_abs_sums / gmm_abs_sums: elementary products of the inputs, no cancellation inside).
+# C_SUM counts the roundings a summand carries at unit roundoff 2^-24 apart from its exponent: exp2, the
+# 1/sum normalisation, the weight product, the dot product feeding it, the accumulation (partial sums,
+# merges) -- 16 is that count with a factor of ~2 to spare and is not tuned per test.  A weight
+# exp(v) inherits the ABSOLUTE rounding of v as a relative error: forming v and subtracting the maximum
+# are 4 roundings of size 2^-24 * |v|, so operators with an exponential add 4 * max|v| (c_exp).
+EPS32 = 2.0 ** -24
+C_SUM = 16.0
+
+
+def c_exp(max_abs_exponent):
+    return C_SUM + 4.0 * float(max_abs_exponent)
+
+
+def assert_close_sum(got, ref, s_abs, what, rtol=RTOL, atol=ATOL, c=C_SUM):
+    got = got.detach().cpu().double()
+    ref = ref.detach().cpu().double()
+    s_abs = torch.as_tensor(s_abs).detach().cpu().double()
+    assert got.shape == ref.shape, "%s: shape %s vs %s" % (what, tuple(got.shape), tuple(ref.shape))
+    s_abs = s_abs.expand_as(ref)
+    err = (got - ref).abs()
+    tol = rtol * ref.abs() + torch.clamp(c * EPS32 * s_abs, min=atol)
+    bad = err > tol
+    if bad.any():
+        i = int(torch.argmax(err - tol))
+        raise AssertionError("%s: %d/%d outside rtol=%g + max(%g, %g*2^-24*S); worst |err|=%.3e at flat %d (got %.7g ref %.7g S %.4g)" % (
+            what, int(bad.sum()), bad.numel(), rtol, atol, c, float(err.flatten()[i]), i,
+            float(got.flatten()[i]), float(ref.flatten()[i]), float(s_abs.flatten()[i])))
+
+
 def gat_inputs(g, h, f, seed=0, attn_scale=1.0, dtype=torch.float64):
     gen = torch.Generator().manual_seed(seed)
     x = torch.randn(g.n, h, f, generator=gen, dtype=dtype)

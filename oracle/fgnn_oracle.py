@@ -162,31 +162,26 @@ def gat_abs_sums(attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, 
 
 
 def segment_sums(ptr, vals):
-    """out[r] = sum of vals[ptr[r]:ptr[r+1]] along dim 0 (empty segments give 0), by differences of one
-    running sum -- usable at 10^8 entries, where index_add_ of float64 serialises on its atomics."""
-    c = torch.cat([torch.zeros_like(vals[:1]), torch.cumsum(vals, 0)])
+    """out[r] = sum of vals[ptr[r]:ptr[r+1]] along dim 0 of vals [E,H] (empty segments give 0), by differences of
+    one running sum per column (taken along the contiguous dimension of the transposed array: fast at 10^8
+    entries, where index_add_ of float64 serialises on its atomics)."""
+    c = torch.cumsum(vals.t().contiguous(), 1)
+    c = torch.cat([torch.zeros_like(c[:, :1]), c], 1)
     p = ptr.to(torch.int64)
-    return c[p[1:]] - c[p[:-1]]
+    return (c[:, p[1:]] - c[:, p[:-1]]).t().contiguous()
 
 
-def segment_weighted_rows(ptr, ids, weights, feat, chunk=1 << 20):
-    """out[r,h,:] = sum_{p in [ptr[r], ptr[r+1])} weights[p,h] * feat[ids[p],h,:] in float64, the entries walked in
-    chunks (the [E,H,F] message tensor of gat_forward is never materialised).  feat may be float32."""
-    p = ptr.to(torch.int64)
-    n_e = int(p[-1])
-    out = torch.zeros((p.numel() - 1,) + tuple(feat.shape[1:]), dtype=torch.float64, device=feat.device)
-    for a in range(0, n_e, chunk):
-        b = min(a + chunk, n_e)
-        c = torch.cumsum(weights[a:b].unsqueeze(-1) * feat[ids[a:b].to(torch.int64)].double(), 0)
-        r_lo = int(torch.searchsorted(p, torch.tensor(a, device=p.device), right=True)) - 1
-        r_hi = int(torch.searchsorted(p, torch.tensor(b - 1, device=p.device), right=True)) - 1
-        rows = torch.arange(r_lo, r_hi + 1, device=p.device)
-        st = torch.clamp(p[rows], min=a) - a
-        en = torch.clamp(p[rows + 1], max=b) - a
-        live = en > st
-        rows, st, en = rows[live], st[live], en[live]
-        seg = c[en - 1] - torch.where((st > 0).view(-1, 1, 1), c[torch.clamp(st - 1, min=0)], torch.zeros_like(c[:1]))
-        out[rows] += seg                      # rows are distinct inside a chunk
+def segment_weighted_rows(ptr, ids, weights, feat):
+    """out[r,h,:] = sum_{p in [ptr[r], ptr[r+1])} weights[p,h] * feat[ids[p],h,:] in float64 without the [E,H,F]
+    message tensor of gat_forward: per head one sparse-matrix product by the library routine
+    (torch.sparse.mm on a CSR matrix holding the weights; duplicate entries of a row are separate terms).
+    feat may be float32."""
+    n_rows = ptr.numel() - 1
+    out = torch.empty((n_rows,) + tuple(feat.shape[1:]), dtype=torch.float64, device=feat.device)
+    crow, col = ptr.to(torch.int64), ids.to(torch.int64)
+    for h in range(feat.shape[1]):
+        a = torch.sparse_csr_tensor(crow, col, weights[:, h].contiguous(), size=(n_rows, feat.shape[0]))
+        out[:, h, :] = torch.sparse.mm(a, feat[:, h, :].double().contiguous())
     return out
 
 
@@ -201,31 +196,45 @@ def edge_dots(dst, src, a, b, chunk=1 << 20, absolute=False):
 
 
 def gat_reference_chunked(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, permute, negative_slope, in_feat, grad_out,
-                          chunk=1 << 20):
+                          chunk=1 << 20, log=None):
     """The whole fused GAT forward and backward in float64 with explicit formulas instead of autograd, and the
-    scales of gat_abs_sums next to them, without any [E,H,F] tensor: usable on the 10^8-edge graphs (on whatever
-    device the inputs live on; they may be float32).  Same math as gat_forward; the backward terms are
+    scales of gat_abs_sums next to them, without any [E,H,F] tensor (sparse-matrix products per head, per-edge dot
+    products in chunks): usable on the 10^8-edge graphs (on whatever device the inputs live on; they may be float32).  Same math as gat_forward; the backward terms are
     ge = <g_i, x_j>, ws_i = sum_p alpha ge, g_score = alpha (ge - ws_i) lrelu'(e)
-    (src/fused_gat/fused_gat_SM.cu:656-732).  Returns a dict of out, grad_feat, grad_attn_row, grad_attn_col
-    and S_<name> for each."""
+    (src/fused_gat/fused_gat_SM.cu:656-732).  Returns a dict of out, grad_feat, grad_attn_row, grad_attn_col,
+    S_<name> for each, and A_grad_attn_row / A_grad_attn_col (see below)."""
+    log = log or (lambda msg: None)
     ar, ac = attn_row.double(), attn_col.double()
     dst = row_of_edge(row_ptr)
     src = col_ind.to(torch.int64)
     pm = permute.to(torch.int64)
-    e = torch.nn.functional.leaky_relu(ar[dst] + ac[src], negative_slope)
+    raw = ar[dst] + ac[src]
+    # LeakyReLU' jumps at 0: an fp32 evaluation may land on the other side when the exact pre-activation is within
+    # its rounding of the operands (2 * 2^-24 * (|attn_row| + |attn_col|)).  Such edges are marked; what the jump can
+    # change in the score gradients is returned as an allowance (A_grad_attn_*), zero everywhere else.
+    amb = raw.abs() <= 2.0 * 2.0 ** -24 * (ar.abs()[dst] + ac.abs()[src])
+    e = torch.nn.functional.leaky_relu(raw, negative_slope)
+    del raw
     alpha, _, _ = _segment_softmax(e, dst, ar.shape[0])
     d = torch.where(e > 0, 1.0, abs(negative_slope))
     del e
-    res = {"out": segment_weighted_rows(row_ptr, col_ind, alpha, in_feat, chunk),
-           "S_out": segment_weighted_rows(row_ptr, col_ind, alpha, in_feat.abs(), chunk)}
+    log("attention weights done")
+    res = {"out": segment_weighted_rows(row_ptr, col_ind, alpha, in_feat)}
+    log("out done")
+    res["S_out"] = segment_weighted_rows(row_ptr, col_ind, alpha, in_feat.abs())
     a_csc = alpha[pm]
-    res["grad_feat"] = segment_weighted_rows(col_ptr, row_ind, a_csc, grad_out, chunk)
-    res["S_grad_feat"] = segment_weighted_rows(col_ptr, row_ind, a_csc, grad_out.abs(), chunk)
+    res["grad_feat"] = segment_weighted_rows(col_ptr, row_ind, a_csc, grad_out)
+    log("grad_feat done")
+    res["S_grad_feat"] = segment_weighted_rows(col_ptr, row_ind, a_csc, grad_out.abs())
     del a_csc
     ge = edge_dots(dst, src, grad_out, in_feat, chunk)
+    log("edge dot products done")
     ws = segment_sums(row_ptr, alpha * ge)
     gs = alpha * (ge - ws[dst]) * torch.where(d == 1.0, 1.0, negative_slope)
-    del ge, ws
+    jump = torch.where(amb, (alpha * (ge - ws[dst])).abs() * abs(1.0 - negative_slope), 0.0)
+    res["A_grad_attn_row"] = segment_sums(row_ptr, jump)
+    res["A_grad_attn_col"] = segment_sums(col_ptr, jump[pm])
+    del ge, ws, jump, amb
     res["grad_attn_row"] = segment_sums(row_ptr, gs)
     res["grad_attn_col"] = segment_sums(col_ptr, gs[pm])
     del gs

@@ -304,6 +304,14 @@ def test_gat_reference_chunked_equals_autograd_oracle(chunk):
         for name, want in (("out", out.detach()), ("grad_feat", leaves[2].grad), ("grad_attn_row", leaves[0].grad), ("grad_attn_col", leaves[1].grad)):
             _close(r[name], want, 1e-6)              # inputs went through float32
             _close(r["S_" + name], s[name], 1e-6)
+        assert float(r["A_grad_attn_row"].abs().max()) == 0.0 and float(r["A_grad_attn_col"].abs().max()) == 0.0
+    # a pre-activation of exactly zero (attn_row[i] == -attn_col[j]) is a point where LeakyReLU' jumps: the edge's
+    # possible contribution shows up as an allowance on its row and its column, nowhere else
+    i, j = 3, int(g.col_ind[int(g.row_ptr[3])])
+    ar2 = ar.float().clone(); ar2[i, 0] = -ac.float()[j, 0]
+    r = orc.gat_reference_chunked(ar2, ac.float(), g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, g.permute, 0.2, x.float(), go.float())
+    assert float(r["A_grad_attn_row"][i, 0]) > 0 and float(r["A_grad_attn_col"][j, 0]) > 0
+    assert int((r["A_grad_attn_row"] != 0).sum()) == 1
 
 
 # ------------------------------------------------------------------ csr2csc

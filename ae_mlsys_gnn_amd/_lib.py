@@ -42,6 +42,8 @@ _SIGNATURES = {
     "fgnn_edgeconv_backward": (c_int, [c_int, c_int, c_int] + [c_void_p] * 3 + [c_void_p]),
     "fgnn_edgeconv_backward_blocked_workspace_bytes": (c_size_t, [c_int, c_int]),
     "fgnn_edgeconv_backward_blocked": (c_int, [c_int, c_int, c_int, c_int] + [c_void_p] * 4 + [c_size_t, c_void_p]),
+    "fgnn_edgeconv_backward_blocked_static_max_elems": (c_size_t, []),
+    "fgnn_edgeconv_backward_blocked_static": (c_int, [c_int, c_int, c_int, c_int] + [c_void_p] * 3 + [c_void_p]),
     "fgnn_knn_graph": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "fgnn_gmm_forward_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int]),
     "fgnn_gmm_forward": (c_int, [c_int, c_int64, c_int, c_int, c_int] + [c_void_p] * 9 + [c_int]

@@ -9,6 +9,7 @@
 // Mapping: a thread owns VEC consecutive features of one node and walks the k neighbours in
 // position order with 4 row loads in flight; the F/VEC threads of a node read one contiguous
 // feature row per neighbour.  The problem is tiny (hundreds of MB), so there is no LDS staging.
+#include <mutex>
 #include "fgnn_common.h"
 
 template <int VEC>
@@ -192,24 +193,14 @@ extern "C" size_t fgnn_edgeconv_backward_blocked_workspace_bytes(int N, int F)
     return ((size_t)N * F + EC_OVF_HEADER) * sizeof(int32_t);
 }
 
-extern "C" int fgnn_edgeconv_backward_blocked(int N, int n_src, int F, int block, const int32_t *argmax, const float *grad_out,
-                                              float *grad_src, void *workspace, size_t workspace_bytes, void *stream)
+// Tile width of the blocked kernel for a block size (0: no usable LDS tile)
+static inline int ec_blocked_fs(int block) { return block <= 2048 ? 8 : block <= 4096 ? 4 : 0; }
+
+// The two launches of the blocked backward; ovf: (N*F + EC_OVF_HEADER) ints of device scratch.
+static int edgeconv_backward_blocked_run(int N, int F, int block, int fs, const int32_t *argmax, const float *grad_out, float *grad_src,
+                                         int *ovf, hipStream_t st)
 {
-    FGNN_REQUIRE(N >= 0 && n_src >= 0 && F >= 1 && block >= 1, FGNN_ERR_SHAPE, "fgnn_edgeconv_backward_blocked: bad sizes");
-    FGNN_REQUIRE(argmax && grad_out && grad_src, FGNN_ERR_NULL, "fgnn_edgeconv_backward_blocked: NULL argument");
-    FGNN_REQUIRE((int64_t)N * F <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_edgeconv_backward_blocked: N*F exceeds int32");
-    // tile of the largest FS that fits 64 KiB of LDS; without a usable tile, or with source rows that no
-    // destination block covers, the plain scatter does the job
-    const int fs = block <= 2048 ? 8 : block <= 4096 ? 4 : 0;
-    if (fs == 0 || n_src != N || (size_t)block * fs * sizeof(float) > 64 * 1024)
-        return fgnn_edgeconv_backward(N, n_src, F, argmax, grad_out, grad_src, stream);
-    size_t need = fgnn_edgeconv_backward_blocked_workspace_bytes(N, F);
-    FGNN_REQUIRE(N == 0 || (workspace && workspace_bytes >= need), FGNN_ERR_WORKSPACE, "fgnn_edgeconv_backward_blocked: workspace %zu < %zu bytes",
-                 workspace_bytes, need);
-    if (N == 0) return 0;
-    hipStream_t st = (hipStream_t)stream;
-    int *ovf = (int *)workspace;
-    int rc = fgnn_fill_f32((float *)ovf, 1, 0.f, st);        // the counter (bit pattern of 0.0f is integer 0)
+    int rc = fgnn_fill_f32((float *)ovf, 1, 0.f, st);        // the counter (bit pattern of 0.0f is integer 0); a kernel, so capturable
     if (rc) return rc;
     dim3 grid((unsigned)((F + fs - 1) / fs), (unsigned)((N + block - 1) / block));
     FGNN_REQUIRE(grid.y <= 65535, FGNN_ERR_LIMIT, "fgnn_edgeconv_backward_blocked: more than 65535 blocks");
@@ -220,4 +211,70 @@ extern "C" int fgnn_edgeconv_backward_blocked(int N, int n_src, int F, int block
     if (rc) return rc;
     hipLaunchKernelGGL(edgeconv_bwd_overflow_kernel, dim3(64), dim3(256), 0, st, F, argmax, grad_out, grad_src, ovf);
     return fgnn_launch_status("edgeconv_bwd_overflow_kernel");
+}
+
+extern "C" int fgnn_edgeconv_backward_blocked(int N, int n_src, int F, int block, const int32_t *argmax, const float *grad_out,
+                                              float *grad_src, void *workspace, size_t workspace_bytes, void *stream)
+{
+    FGNN_REQUIRE(N >= 0 && n_src >= 0 && F >= 1 && block >= 1, FGNN_ERR_SHAPE, "fgnn_edgeconv_backward_blocked: bad sizes");
+    FGNN_REQUIRE(argmax && grad_out && grad_src, FGNN_ERR_NULL, "fgnn_edgeconv_backward_blocked: NULL argument");
+    FGNN_REQUIRE((int64_t)N * F <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_edgeconv_backward_blocked: N*F exceeds int32");
+    // tile of the largest FS that fits 64 KiB of LDS; without a usable tile, or with source rows that no
+    // destination block covers, the plain scatter does the job
+    const int fs = ec_blocked_fs(block);
+    if (fs == 0 || n_src != N || (size_t)block * fs * sizeof(float) > 64 * 1024)
+        return fgnn_edgeconv_backward(N, n_src, F, argmax, grad_out, grad_src, stream);
+    size_t need = fgnn_edgeconv_backward_blocked_workspace_bytes(N, F);
+    FGNN_REQUIRE(N == 0 || (workspace && workspace_bytes >= need), FGNN_ERR_WORKSPACE, "fgnn_edgeconv_backward_blocked: workspace %zu < %zu bytes",
+                 workspace_bytes, need);
+    if (N == 0) return 0;
+    return edgeconv_backward_blocked_run(N, F, block, fs, argmax, grad_out, grad_src, (int *)workspace, (hipStream_t)stream);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// The blocked backward for callers that cannot allocate.  Its overflow list lives in a file-scope device
+// array of a fixed size: every GPU the library runs on holds one copy (at its own address) until the
+// process ends.  The array's name is only a host-side handle; the device address is looked up once per
+// device with hipGetSymbolAddress and that pointer is what the kernels get.
+#define EC_STATIC_MAX_ELEMS (4 * 1024 * 1024)         // largest N*F the static scratch serves (16 MiB + header)
+#define EC_STATIC_MAX_DEVICES 64
+static __device__ __align__(256) int32_t ec_static_scratch[EC_STATIC_MAX_ELEMS + EC_OVF_HEADER];
+static std::mutex ec_static_mutex;
+static int32_t *ec_static_ptr[EC_STATIC_MAX_DEVICES];   // per device: address of that device's copy (NULL until looked up)
+
+static int ec_static_scratch_for_current_device(int32_t **out)
+{
+    int dev = -1;
+    FGNN_HIP(hipGetDevice(&dev));
+    FGNN_REQUIRE(dev >= 0 && dev < EC_STATIC_MAX_DEVICES, FGNN_ERR_LIMIT, "fgnn_edgeconv_backward_blocked_static: device %d out of range", dev);
+    std::lock_guard<std::mutex> lock(ec_static_mutex);
+    if (!ec_static_ptr[dev]) {
+        void *p = nullptr;
+        FGNN_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(ec_static_scratch)));
+        FGNN_REQUIRE(p != nullptr, FGNN_ERR_NULL, "fgnn_edgeconv_backward_blocked_static: no device address for the scratch array");
+        ec_static_ptr[dev] = (int32_t *)p;
+    }
+    *out = ec_static_ptr[dev];
+    return 0;
+}
+
+extern "C" size_t fgnn_edgeconv_backward_blocked_static_max_elems(void) { return (size_t)EC_STATIC_MAX_ELEMS; }
+
+extern "C" int fgnn_edgeconv_backward_blocked_static(int N, int n_src, int F, int block, const int32_t *argmax, const float *grad_out,
+                                                     float *grad_src, void *stream)
+{
+    FGNN_REQUIRE(N >= 0 && n_src >= 0 && F >= 1 && block >= 1, FGNN_ERR_SHAPE, "fgnn_edgeconv_backward_blocked_static: bad sizes");
+    FGNN_REQUIRE(argmax && grad_out && grad_src, FGNN_ERR_NULL, "fgnn_edgeconv_backward_blocked_static: NULL argument");
+    FGNN_REQUIRE((int64_t)N * F <= (int64_t)EC_STATIC_MAX_ELEMS, FGNN_ERR_LIMIT,
+                 "fgnn_edgeconv_backward_blocked_static: N*F = %lld exceeds the static scratch of %d elements; use fgnn_edgeconv_backward_blocked with a workspace",
+                 (long long)N * F, EC_STATIC_MAX_ELEMS);
+    const int fs = ec_blocked_fs(block);
+    if (fs == 0 || n_src != N || (size_t)block * fs * sizeof(float) > 64 * 1024)
+        return fgnn_edgeconv_backward(N, n_src, F, argmax, grad_out, grad_src, stream);      // fill + scatter: no scratch, no allocation
+    if (N == 0) return 0;
+    int32_t *ovf = nullptr;
+    int rc = ec_static_scratch_for_current_device(&ovf);
+    if (rc) return rc;
+    // the list is rebuilt from its counter (cleared first) on every call: nothing of an earlier call is read
+    return edgeconv_backward_blocked_run(N, F, block, fs, argmax, grad_out, grad_src, ovf, (hipStream_t)stream);
 }

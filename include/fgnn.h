@@ -152,6 +152,17 @@ int    fgnn_edgeconv_backward_blocked(int N, int n_src, int F, int block, const 
                                       const float *grad_out, float *grad_src, void *workspace,
                                       size_t workspace_bytes, void *stream);
 
+/* fgnn_edgeconv_backward_blocked for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): same arguments without the workspace.  The overflow list
+ * lives in a fixed device array inside the library (16 MiB + 256 B, held by every GPU the library runs on until
+ * the process ends); the call allocates nothing and rejects N*F above
+ * fgnn_edgeconv_backward_blocked_static_max_elems() (4 Mi elements) with FGNN_ERR_LIMIT.  All calls on one GPU
+ * share that array: calls that overlap on one GPU (different streams, different threads) race; calls on one
+ * stream are safe, each call rebuilds the list from a counter it clears first.  No counterpart in the reference. */
+size_t fgnn_edgeconv_backward_blocked_static_max_elems(void);
+int    fgnn_edgeconv_backward_blocked_static(int N, int n_src, int F, int block, const int32_t *argmax,
+                                             const float *grad_out, float *grad_src, void *stream);
+
 /* k-nearest-neighbour graph of batched point clouds, the input of fgnn_edgeconv_forward: points
  * [n_clouds*P, D]; src_ind [n_clouds*P*k] gets, for every point, the global ids of the k nearest
  * points of its own cloud (itself included), nearest first, ties to the smaller id; 1 <= k <= min(P,

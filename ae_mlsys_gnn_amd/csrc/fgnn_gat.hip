@@ -564,11 +564,49 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_edge_stash_kernel(int N, int64_t
     }
 }
 
+// The stashed attention in the ORDER OF THE BACKWARD PASS: esm[q,h] = alpha of entry q of the (col_ptr, row_ind)
+// walk under the given schedule (its bucket-ordered entry order when it is XCD-aware), so that the column pass
+// streams the stash instead of gathering 32 bytes per edge through `permute`.  The value stored is alpha with the sign
+// bit set when the pre-activation is not positive, so the column pass needs nothing else per (destination, head) than
+// delta: no 16-byte record, a quarter of the gathered bytes next to the feature rows.  Same traversal as that pass (work
+// items, one wave each), pair layout: lane (u << hp_shift) | h owns (entry u of a batch, head h), gathers the three
+// row statistics of (destination, h) and writes one float; a batch writes 64 consecutive floats.
+__global__ __launch_bounds__(FGNN_TPB) void gat_stash_own_order_kernel(const fgnn_item *items, int n_items, const int *__restrict__ ptr,
+                                                                       const int *__restrict__ idx, int H, int hp_shift,
+                                                                       const float *__restrict__ ar, const float *__restrict__ ac,
+                                                                       const float *__restrict__ emax, const float *__restrict__ esum,
+                                                                       float slope, float *__restrict__ esm)
+{
+    int col, b, e, slot;
+    if (!fg_get_item(items, n_items, ptr, col, b, e, slot)) return;
+    const int lane = fg_lane();
+    const int u = lane >> hp_shift, h = lane & ((1 << hp_shift) - 1);
+    const int U = 64 >> hp_shift;                         // entries per batch
+    const bool okh = h < H;
+    const float ach = okh ? ac[(size_t)col * H + h] : 0.f;
+    for (int c = b; c < e; c += 64) {
+        const int q = c + lane;
+        const int cnt = min(64, e - c);
+        const int idv = idx[q < e ? q : c];
+        for (int t = 0; t < cnt; t += U) {
+            const int i = __builtin_amdgcn_ds_bpermute(((t + u) & 63) << 2, idv);
+            if (okh && t + u < cnt) {
+                const size_t rh = (size_t)(unsigned)i * H + h;
+                const float ev = fg_lrelu(ar[rh] + ach, slope);
+                const float al = __builtin_amdgcn_exp2f((ev - emax[rh]) * FGNN_LOG2E) * __builtin_amdgcn_rcpf(esum[rh]);
+                // alpha >= 0: its sign bit carries "pre-activation positive" (clear) / "not positive" (set, -0.0 included)
+                __builtin_nontemporal_store(ev > 0.f ? al : -al, esm + (size_t)(c + t + u) * H + h);
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------- backward
 struct GatBwdP {
     const fgnn_item *items; int n_items;
     const int *ptr; const int *idx; const int *pos; const int *permute;
     const float4 *rec;
+    const float *delta;     // own-order stash only: <g[i,h,:], out[i,h,:]> per (node, head), in place of rec
     const float *ac; const float *x; const float *g;
     const float *esm;
     float *gfeat; float *gac; float *part;
@@ -582,7 +620,8 @@ __host__ __device__ static inline int gat_bwd_pw(int HF, int H) { return (2 * HF
 template <int VEC, int R>
 __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_node_kernel(int N, int H, int F, int HF, const float *g, const float *out,
                                                                 const float *out2, const float *cc, const float *ar,
-                                                                const float *emax, const float *esum, float4 *rec, float *gar)
+                                                                const float *emax, const float *esum, float4 *rec, float *delta_out,
+                                                                float *gar)
 {
     extern __shared__ float lds[];
     int i = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
@@ -607,8 +646,10 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_node_kernel(int N, int H, in
     if (lane < H) {
         size_t q = (size_t)i * H + lane;
         float s = esum[q];
-        // attn_row and the maximum are stored in log2 units for the column pass
-        rec[q] = make_float4(ar[q] * FGNN_LOG2E, emax[q] * FGNN_LOG2E, s > 0.f ? 1.f / s : 0.f, delta);
+        // attn_row and the maximum are stored in log2 units for the column pass; with a signed own-order stash that
+        // pass only needs delta
+        if (delta_out) delta_out[q] = delta;
+        else rec[q] = make_float4(ar[q] * FGNN_LOG2E, emax[q] * FGNN_LOG2E, s > 0.f ? 1.f / s : 0.f, delta);
         gar[q] = dd2 - delta * cc[q];
     }
 }
@@ -640,7 +681,9 @@ __device__ __forceinline__ void gat_bwd_finish(const GatBwdP &p, int col, int la
 // One batch of UB edges of the backward column pass.  Every lane reads the 16-byte record
 // (attn_row, max, 1/sum, delta) of the head its features belong to (the first two in log2 units)
 // and recomputes alpha itself.
-template <int VEC, int R, bool STASH, bool FULL, int UB, bool TAIL, bool SLE1>
+// STASH: 0 = alpha recomputed from the record; 1 = alpha read from a stash in the caller's order (through permute), the
+// sign of the pre-activation from attn_row + attn_col; 2 = signed alpha read from a stash in this pass's own order.
+template <int VEC, int R, int STASH, bool FULL, int UB, bool TAIL, bool SLE1>
 __device__ __forceinline__ void gat_bwd_batch(const GatBwdP &p, const fg_lanemap<VEC, R> &lm, const uint32_t (&boff)[R],
                                               const uint32_t (&roff)[R], const uint32_t (&hoff)[R], int idv, int posv, int t, int cnt,
                                               const float (&ach)[R], float (&z)[R], fg_vec<VEC> (&T)[R], fg_vec<VEC> (&P)[R])
@@ -653,13 +696,15 @@ __device__ __forceinline__ void gat_bwd_batch(const GatBwdP &p, const fg_lanemap
         size_t i = (size_t)(unsigned)__builtin_amdgcn_readlane(idv, t + u);
         const char *base = (const char *)p.g + i * row_bytes;
         const char *rb = (const char *)p.rec + i * rec_bytes;
+        const char *db = (const char *)p.delta + i * sc_bytes;
         size_t pos = STASH ? (size_t)(unsigned)__builtin_amdgcn_readlane(posv, t + u) * sc_bytes : 0;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if (FULL || lm.ok[r]) {
                 ld[u][r].load_off(base, boff[r]);
-                rc[u][r] = *(const float4 *)(rb + roff[r]);
-                if (STASH) rc[u][r].y = *(const float *)((const char *)p.esm + pos + hoff[r]);
+                if (STASH == 2) rc[u][r] = make_float4(0.f, *(const float *)((const char *)p.esm + pos + hoff[r]), 0.f, *(const float *)(db + hoff[r]));
+                else rc[u][r] = *(const float4 *)(rb + roff[r]);
+                if (STASH == 1) rc[u][r].y = *(const float *)((const char *)p.esm + pos + hoff[r]);
             } else {
                 ld[u][r].zero();
                 rc[u][r] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -673,7 +718,8 @@ __device__ __forceinline__ void gat_bwd_batch(const GatBwdP &p, const fg_lanemap
             float ev, al;
             // stash variants: alpha comes from the stash; only the sign of the pre-activation is still
             // needed, and that is the sign of attn_row + attn_col (no second per-edge gather)
-            if (STASH) { ev = fmaf(ach[r], FGNN_LOG2E, rc[u][r].x); al = rc[u][r].y; }
+            if (STASH == 2) { ev = __float_as_int(rc[u][r].y) >= 0 ? 1.f : -1.f; al = fabsf(rc[u][r].y); }
+            else if (STASH == 1) { ev = fmaf(ach[r], FGNN_LOG2E, rc[u][r].x); al = rc[u][r].y; }
             else { ev = fg_lrelu_t<SLE1>(fmaf(ach[r], FGNN_LOG2E, rc[u][r].x), p.slope); al = __builtin_amdgcn_exp2f(ev - rc[u][r].y) * rc[u][r].z; }
             if (TAIL) al = ((t + u) < cnt) ? al : 0.f;
             const bool pos_e = ev > 0.f;
@@ -694,7 +740,7 @@ struct GatPair { int u, h; bool ok; float ach, z; };
 struct GatPairRec { float4 rc; float esm; };
 // The record (and stashed alpha) of the lane's pair in the batch that starts at entry t of the chunk.
 // Issued one batch ahead of its use, so that the feature-row loads of a batch never wait behind it.
-template <bool STASH>
+template <int STASH>
 __device__ __forceinline__ GatPairRec gat_bwd_pair_fetch(const GatBwdP &p, const GatPair &pr, int idv, int posv, int t, int cnt)
 {
     const int eu = (t + pr.u) & 63;
@@ -706,12 +752,13 @@ __device__ __forceinline__ GatPairRec gat_bwd_pair_fetch(const GatBwdP &p, const
     f.rc = make_float4(0.f, 0.f, 0.f, 0.f);
     f.esm = 0.f;
     if (live) {
-        f.rc = p.rec[(size_t)(unsigned)ip * p.H + pr.h];
-        if (STASH) f.esm = p.esm[(size_t)(unsigned)pp * p.H + pr.h];
+        if (STASH == 2) f.rc.w = p.delta[(size_t)(unsigned)ip * p.H + pr.h];
+        else f.rc = p.rec[(size_t)(unsigned)ip * p.H + pr.h];
+        if (STASH) f.esm = __builtin_nontemporal_load(p.esm + (size_t)(unsigned)pp * p.H + pr.h);     // read once
     }
     return f;
 }
-template <int VEC, int R, bool STASH, bool FULL, int UB, bool SLE1>
+template <int VEC, int R, int STASH, bool FULL, int UB, bool SLE1>
 __device__ __forceinline__ void gat_bwd_pair_batch(const GatBwdP &p, const fg_lanemap<VEC, R> &lm, const uint32_t (&boff)[R],
                                                    int idv, int posv, int t, int cnt, GatPair &pr, GatPairRec &cur,
                                                    fg_vec<VEC> (&T)[R], fg_vec<VEC> (&P)[R])
@@ -735,7 +782,8 @@ __device__ __forceinline__ void gat_bwd_pair_batch(const GatBwdP &p, const fg_la
     }
     const float4 rc = cur.rc;
     float ev, al;
-    if (STASH) { ev = fmaf(pr.ach, FGNN_LOG2E, rc.x); al = cur.esm; }
+    if (STASH == 2) { ev = __float_as_int(cur.esm) >= 0 ? 1.f : -1.f; al = fabsf(cur.esm); }
+    else if (STASH == 1) { ev = fmaf(pr.ach, FGNN_LOG2E, rc.x); al = cur.esm; }
     else { ev = fg_lrelu_t<SLE1>(fmaf(pr.ach, FGNN_LOG2E, rc.x), p.slope); al = __builtin_amdgcn_exp2f(ev - rc.y) * rc.z; }
     al = (pr.ok && t + pr.u < cnt) ? al : 0.f;
     pr.z = fmaf(ev > 0.f ? al : al * p.slope, rc.w, pr.z);
@@ -754,7 +802,7 @@ __device__ __forceinline__ void gat_bwd_pair_batch(const GatBwdP &p, const fg_la
     cur = nxt;
 }
 
-template <int VEC, int R, bool STASH, bool FULL, bool SLE1, bool PAIR>
+template <int VEC, int R, int STASH, bool FULL, bool SLE1, bool PAIR>
 __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_kernel(GatBwdP p)
 {
     extern __shared__ float lds[];
@@ -789,7 +837,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_kernel(GatBwdP p)
         int cnt = min(64, e - c);
         int qq = q < e ? q : c;
         int idv = p.idx[qq];
-        int posv = STASH ? p.permute[p.pos ? p.pos[qq] : qq] : 0;
+        int posv = STASH ? (p.permute ? p.permute[p.pos ? p.pos[qq] : qq] : qq) : 0;      // no permute: the stash is in this pass's own entry order
         int t = 0;
         if constexpr (PAIR) {
             GatPairRec cur = gat_bwd_pair_fetch<STASH>(p, pr, idv, posv, 0, cnt);
@@ -834,7 +882,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_kernel(GatBwdP p)
 
 // The column pass for rows narrower than a wave: G entries of the column per load instruction
 // (see gat_fwd_packed_kernel); T, P and z are plain sums, so the groups are added by a butterfly.
-template <int G, bool STASH, bool SLE1, bool PAIR>
+template <int G, int STASH, bool SLE1, bool PAIR>
 __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
 {
     extern __shared__ float lds[];
@@ -862,7 +910,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
         int cnt = min(64, e - c);
         int qq = q < e ? q : c;
         int idv = p.idx[qq];
-        int posv = STASH ? p.permute[p.pos ? p.pos[qq] : qq] : 0;
+        int posv = STASH ? (p.permute ? p.permute[p.pos ? p.pos[qq] : qq] : qq) : 0;
         GatPairRec cur;
         cur.rc = make_float4(0.f, 0.f, 0.f, 0.f); cur.esm = 0.f;
         if constexpr (PAIR) cur = gat_bwd_pair_fetch<STASH>(p, pr, idv, posv, 0, cnt);
@@ -880,7 +928,8 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
                 }
                 const float4 rc = cur.rc;
                 float ev, al;
-                if (STASH) { ev = fmaf(pr.ach, FGNN_LOG2E, rc.x); al = cur.esm; }
+                if (STASH == 2) { ev = __float_as_int(cur.esm) >= 0 ? 1.f : -1.f; al = fabsf(cur.esm); }
+                else if (STASH == 1) { ev = fmaf(pr.ach, FGNN_LOG2E, rc.x); al = cur.esm; }
                 else { ev = fg_lrelu_t<SLE1>(fmaf(pr.ach, FGNN_LOG2E, rc.x), p.slope); al = __builtin_amdgcn_exp2f(ev - rc.y) * rc.z; }
                 al = (pr.ok && t + pr.u < cnt) ? al : 0.f;
                 pr.z = fmaf(ev > 0.f ? al : al * p.slope, rc.w, pr.z);
@@ -903,8 +952,9 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
                 const size_t pos = STASH ? (size_t)(unsigned)__builtin_amdgcn_ds_bpermute((ei & 63) << 2, posv) : 0;
                 if (ei < cnt && pm.ok) {
                     ld[u].load(p.g + i * p.HF + pm.eoff);
-                    rc[u] = p.rec[i * H + pm.hd];
-                    if (STASH) rc[u].y = p.esm[pos * H + pm.hd];
+                    if (STASH == 2) rc[u] = make_float4(0.f, p.esm[pos * H + pm.hd], 0.f, p.delta[i * H + pm.hd]);
+                    else rc[u] = p.rec[i * H + pm.hd];
+                    if (STASH == 1) rc[u].y = p.esm[pos * H + pm.hd];
                 } else {
                     ld[u].zero();
                     rc[u] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -913,7 +963,8 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 float ev, al;
-                if (STASH) { ev = fmaf(ach, FGNN_LOG2E, rc[u].x); al = rc[u].y; }
+                if (STASH == 2) { ev = __float_as_int(rc[u].y) >= 0 ? 1.f : -1.f; al = fabsf(rc[u].y); }
+                else if (STASH == 1) { ev = fmaf(ach, FGNN_LOG2E, rc[u].x); al = rc[u].y; }
                 else { ev = fg_lrelu_t<SLE1>(fmaf(ach, FGNN_LOG2E, rc[u].x), p.slope); al = __builtin_amdgcn_exp2f(ev - rc[u].y) * rc[u].z; }
                 al = ((t + u * G + pm.grp) < cnt && pm.ok) ? al : 0.f;
                 const bool pos_e = ev > 0.f;
@@ -1139,8 +1190,8 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
                      grad_feat && grad_attn_row && grad_attn_col,
                  FGNN_ERR_NULL, "fgnn_gat_backward: NULL argument");
     const bool stash = e_softmax != nullptr;
-    FGNN_REQUIRE(!stash || permute, FGNN_ERR_NULL, "fgnn_gat_backward: stashed attention needs permute");
-    FGNN_REQUIRE(!stash || fgnn_sched_has_pos(sched_csc), FGNN_ERR_SCHEDULE, "fgnn_gat_backward: stashed attention needs a schedule built with edge positions");
+    // permute == NULL with a stash: e_softmax is in the entry order of this pass under sched_csc (fgnn_gat_stash_own_order)
+    FGNN_REQUIRE(!stash || !permute || fgnn_sched_has_pos(sched_csc), FGNN_ERR_SCHEDULE, "fgnn_gat_backward: stashed attention in the caller's order needs a schedule built with edge positions");
     (void)e_lrelu;      // the sign of the pre-activation is taken from attn_row + attn_col
     const bool recompute = !(out_feat && aux_out2 && aux_c);
     FGNN_REQUIRE(!recompute || (row_ptr && (col_ind || E == 0)), FGNN_ERR_NULL, "fgnn_gat_backward: recomputing the forward needs row_ptr/col_ind");
@@ -1178,13 +1229,16 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
     p.items = sched_csc ? sched_csc->items_dev : nullptr;
     p.n_items = sched_csc ? sched_csc->n_items : N;
     p.ptr = col_ptr; p.idx = fgnn_sched_idx(sched_csc, row_ind); p.pos = fgnn_sched_pos(sched_csc); p.permute = permute; p.rec = rec; p.ac = attn_col; p.x = in_feat; p.g = grad_out;
+    const int stash_mode = !stash ? 0 : (permute ? 1 : 2);
+    p.delta = (const float *)rec;       // own-order stash: the record area holds the compact [N,H] delta array instead
     p.esm = e_softmax; p.gfeat = grad_feat; p.gac = grad_attn_col; p.part = part;
     p.N = N; p.H = H; p.F = F; p.HF = HF; p.slope = negative_slope;
 
     return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
         const unsigned gn = (unsigned)((N + FGNN_WPB - 1) / FGNN_WPB);
         hipLaunchKernelGGL((gat_bwd_node_kernel<VEC, R>), dim3(gn), dim3(FGNN_TPB), (size_t)FGNN_WPB * 64 * R * sizeof(float), st,
-                           N, H, F, HF, grad_out, out_feat, aux_out2, aux_c, attn_row, edge_max, edge_sum, rec, grad_attn_row);
+                           N, H, F, HF, grad_out, out_feat, aux_out2, aux_c, attn_row, edge_max, edge_sum, rec,
+                           stash_mode == 2 ? (float *)rec : nullptr, grad_attn_row);
         int rc2 = fgnn_launch_status("gat_bwd_node_kernel");
         if (rc2) return rc2;
         const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
@@ -1197,9 +1251,10 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
             const bool pair = ((8 * pack) << p.hp_shift) <= 64 && E >= 64 * (int64_t)N;
             auto launch = [&]<int G>() {
                 auto go = [&]<bool PAIR>() {
-                    if (stash) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, true, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
-                    else if (sle1) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, false, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
-                    else hipLaunchKernelGGL((gat_bwd_packed_kernel<G, false, false, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                    if (stash_mode == 2) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 2, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                    else if (stash_mode == 1) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 1, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                    else if (sle1) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 0, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                    else hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 0, false, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
                 };
                 if (pair) go.template operator()<true>(); else go.template operator()<false>();
             };
@@ -1215,9 +1270,10 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
             while ((1 << p.hp_shift) < H) ++p.hp_shift;
             const bool pair = (U << p.hp_shift) <= 64 && E >= 64 * (int64_t)N;
             auto launch = [&]<bool PAIR>() {
-                if (stash) hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, true, FULL, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
-                else if (sle1) hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, false, FULL, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
-                else hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, false, FULL, false, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                if (stash_mode == 2) hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, 2, FULL, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                else if (stash_mode == 1) hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, 1, FULL, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                else if (sle1) hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, 0, FULL, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                else hipLaunchKernelGGL((gat_bwd_kernel<VEC, R, 0, FULL, false, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
             };
             if (pair) launch.template operator()<true>(); else launch.template operator()<false>();
         }
@@ -1231,4 +1287,25 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
         }
         return 0;
     });
+}
+
+extern "C" int fgnn_gat_stash_own_order(int N, int64_t E, int H, float negative_slope, const int32_t *col_ptr, const int32_t *row_ind,
+                                        const float *attn_row, const float *attn_col, const float *edge_max, const float *edge_sum,
+                                        float *e_softmax_own, const fgnn_schedule_t *sched_csc, void *stream)
+{
+    int rc = gat_common_checks("fgnn_gat_stash_own_order", N, E, H, 1);
+    if (rc) return rc;
+    FGNN_REQUIRE(col_ptr && (row_ind || E == 0) && attn_row && attn_col && edge_max && edge_sum && (e_softmax_own || E == 0), FGNN_ERR_NULL,
+                 "fgnn_gat_stash_own_order: NULL argument");
+    rc = check_sched(sched_csc, col_ptr, row_ind, N, E, "fgnn_gat_stash_own_order");
+    if (rc) return rc;
+    if (N == 0 || E == 0) return 0;
+    int hp_shift = 0;
+    while ((1 << hp_shift) < H) ++hp_shift;
+    const int n_items = sched_csc ? sched_csc->n_items : N;
+    const unsigned grid = (unsigned)((n_items + FGNN_WPB - 1) / FGNN_WPB);
+    hipLaunchKernelGGL(gat_stash_own_order_kernel, dim3(grid), dim3(FGNN_TPB), 0, (hipStream_t)stream, sched_csc ? sched_csc->items_dev : nullptr,
+                       n_items, col_ptr, fgnn_sched_idx(sched_csc, row_ind), H, hp_shift, attn_row, attn_col, edge_max, edge_sum, negative_slope,
+                       e_softmax_own);
+    return fgnn_launch_status("gat_stash_own_order_kernel");
 }

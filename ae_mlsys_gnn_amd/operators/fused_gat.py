@@ -84,7 +84,7 @@ class gat_native:
         grad_attn_row = torch.empty((n, h), dtype=torch.float32, device=dev)
         grad_attn_col = torch.empty((n, h), dtype=torch.float32, device=dev)
         recompute = out_feat is None or out2 is None or cc is None
-        sched_csc = schedule_for(col_ptr, idx_tensor=row_ind, need_positions=e_soft is not None) if use_schedule else None
+        sched_csc = schedule_for(col_ptr, idx_tensor=row_ind, need_positions=e_soft is not None and permute is not None) if use_schedule else None
         sched_csr = schedule_for(row_ptr, idx_tensor=col_ind, need_positions=False) if (use_schedule and recompute) else None
         hc = sched_csc.handle if sched_csc is not None else None
         hr = sched_csr.handle if sched_csr is not None else None
@@ -98,6 +98,26 @@ class gat_native:
                                           ptr(grad_attn_col), hc, hr, ptr(ws), wsb, stream_ptr()),
                   "fgnn_gat_backward")
         return grad_feat, grad_attn_row, grad_attn_col
+
+
+    @staticmethod
+    def gat_stash_own_order(negative_slope, col_ptr, row_ind, edge_max, edge_sum, attn_row, attn_col, use_schedule=True):
+        """The attention weights [E,H] in the entry order of the backward pass over (col_ptr, row_ind): what
+        gat_backward(..., e_soft=<this>, permute=None) streams instead of gathering a CSR-ordered stash."""
+        require_cuda(col_ptr, row_ind, edge_max, edge_sum, attn_row, attn_col)
+        col_ptr, row_ind = as_i32(col_ptr), as_i32(row_ind)
+        edge_max, edge_sum, attn_row, attn_col = as_f32(edge_max), as_f32(edge_sum), as_f32(attn_row), as_f32(attn_col)
+        n, h = attn_row.shape
+        e = row_ind.numel()
+        if col_ptr.numel() != n + 1 or any(tuple(t.shape) != (n, h) for t in (attn_col, edge_max, edge_sum)):
+            raise _lib.FgnnError("gat_stash_own_order: shape mismatch for N=%d H=%d" % (n, h))
+        out = torch.empty((e, h), dtype=torch.float32, device=attn_row.device)
+        sched = schedule_for(col_ptr, idx_tensor=row_ind, need_positions=False) if use_schedule else None
+        with torch.cuda.device(attn_row.device):
+            check(lib().fgnn_gat_stash_own_order(n, e, h, float(negative_slope), ptr(col_ptr), ptr(row_ind), ptr(attn_row), ptr(attn_col),
+                                                 ptr(edge_max), ptr(edge_sum), ptr(out), sched.handle if sched is not None else None,
+                                                 stream_ptr()), "fgnn_gat_stash_own_order")
+        return out
 
 
 def fused_gat_fusescatter(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute):
@@ -150,14 +170,18 @@ class FusedGATFunction_stash(torch.autograd.Function):
     """Stash variant: the forward also writes the edge softmax [E,H] and the backward reads it instead
     of recomputing.  (The reference stashes the edge LeakyReLU values too, fused_gat_stash.cu:420-442;
     the backward here takes the one thing it needs from them, the sign of the pre-activation, from
-    attn_row + attn_col, so they are not written: half the stash.)"""
+    attn_row + attn_col, so they are not written: half the stash.)  The stash is kept in the entry order
+    of the backward pass, so that pass streams it; the CSR-ordered stash of the reference's signature
+    (gat_forward(stash=True) + gat_backward(permute=...)) stays available through gat_native."""
 
     @staticmethod
     def forward(ctx, attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute):
         attn_row, attn_col, in_feat = _contig(attn_row), _contig(attn_col), _contig(in_feat)
         row_ptr, col_ind, col_ptr, row_ind, permute = _contig(row_ptr), _contig(col_ind), _contig(col_ptr), _contig(row_ind), _contig(permute)
-        out, edge_max, edge_sum, out2, cc, _, e_soft = gat_native.gat_forward(
-            attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, need_aux=True, stash=True, stash_lrelu=False)
+        out, edge_max, edge_sum, out2, cc, _, _ = gat_native.gat_forward(
+            attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, need_aux=True)
+        # the stash is this function's own tensor: it is written in the order in which the backward walks the edges
+        e_soft = gat_native.gat_stash_own_order(negative_slope, col_ptr, row_ind, edge_max, edge_sum, attn_row, attn_col)
         ctx.save_for_backward(row_ptr, col_ind, col_ptr, row_ind, permute, e_soft, in_feat, attn_row, attn_col,
                               edge_max, edge_sum, out, out2, cc)
         ctx.negative_slope = negative_slope
@@ -169,7 +193,7 @@ class FusedGATFunction_stash(torch.autograd.Function):
          edge_max, edge_sum, out, out2, cc) = ctx.saved_tensors
         grad_feat, grad_attn_row, grad_attn_col = gat_native.gat_backward(
             ctx.negative_slope, row_ptr, col_ind, col_ptr, row_ind, edge_max, edge_sum, in_feat, attn_row, attn_col,
-            grad_out.contiguous(), out_feat=out, out2=out2, cc=cc, permute=as_i32(permute), e_soft=e_soft)
+            grad_out.contiguous(), out_feat=out, out2=out2, cc=cc, permute=None, e_soft=e_soft)
         return grad_attn_row, grad_attn_col, None, None, None, None, None, grad_feat, None
 
 

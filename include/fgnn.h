@@ -108,7 +108,8 @@ int    fgnn_gat_forward(int N, int64_t E, int H, int F,
 /* Replaces fused_gat_SM.gat_backward (src/fused_gat/fused_gat_SM.cpp:40-124, host launcher
  * fused_gat_SM.cu:865-893); with permute/e_softmax non-NULL it reads the stashed attention
  * instead of recomputing it (fused_gat_stash.gat_backward, fused_gat_stash.cu:776-804;
- * fused_gat.gat_backward, fused_gat.cu:641-670).  e_lrelu is accepted for the reference's argument
+ * fused_gat.gat_backward, fused_gat.cu:641-670); with e_softmax non-NULL and permute == NULL the stash is taken to
+ * be in this pass's own entry order (fgnn_gat_stash_own_order).  e_lrelu is accepted for the reference's argument
  * list and not read: the sign of the pre-activation is that of attn_row + attn_col.
  * Inputs as the reference's plus out_feat/aux_out2/aux_c from the forward; when those three are
  * NULL they are recomputed into the workspace from (row_ptr, col_ind) first.
@@ -128,6 +129,20 @@ int    fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_slope,
                          float *grad_feat, float *grad_attn_row, float *grad_attn_col,
                          const fgnn_schedule_t *sched_csc, const fgnn_schedule_t *sched_csr,
                          void *workspace, size_t workspace_bytes, void *stream);
+
+/* The stashed attention of the stash variants in the ORDER OF THE BACKWARD PASS: e_softmax_own[q,h] = alpha of
+ * entry q of the walk of (col_ptr, row_ind) under sched_csc (its bucket-ordered entry order when it is XCD-aware,
+ * plain CSC order otherwise or with sched_csc == NULL), computed from the forward's row statistics; the sign bit of
+ * the stored value is set when the edge's pre-activation is not positive (alpha itself is >= 0), so the backward
+ * needs no other per-edge or per-destination data than <grad_out, out>.
+ * fgnn_gat_backward called with this array as e_softmax, permute == NULL and the same sched_csc then streams the
+ * stash instead of gathering it through permute (114.8 M edges, 8 heads: backward 10.5 -> about 7 ms).  The
+ * reference keeps its stash in CSR order and transposes while reading (src/fused_gat/fused_gat_stash.cu:444-464);
+ * a caller that owns the stashed tensor (the autograd function does) is free to keep it in this order instead. */
+int    fgnn_gat_stash_own_order(int N, int64_t E, int H, float negative_slope, const int32_t *col_ptr,
+                                const int32_t *row_ind, const float *attn_row, const float *attn_col,
+                                const float *edge_max, const float *edge_sum, float *e_softmax_own,
+                                const fgnn_schedule_t *sched_csc, void *stream);
 
 /* ---------------------------------------------------------------- fused EdgeConv
  * Replaces fused_edgeconv.edgeconv_forward / edgeconv_backward

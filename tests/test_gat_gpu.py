@@ -402,3 +402,52 @@ def test_validate_graph_rejects_malformed_arrays_before_any_gather(monkeypatch):
     assert s.device_bytes() >= 4 * g.n_edges + 16 * s.n_items and _lib.schedule_device_bytes() >= s.device_bytes()
     assert _lib.Schedule(g.row_ptr, 0).device_bytes() == 16 * (g.n)       # plain: one 16-byte item per row, nothing split
     _lib.clear_schedule_cache()
+
+
+@pytest.mark.parametrize("h,f", [(8, 32), (1, 47), (4, 16), (3, 20)])
+def test_gat_stash_in_both_orders_through_native_calls(h, f, monkeypatch):
+    """The two forms of the stash behind the C ABI: the reference's (e_softmax [E,H] in CSR order from
+    gat_forward, read through permute by gat_backward) and the one the autograd function keeps (in the entry
+    order of the backward pass, fgnn_gat_stash_own_order, permute == NULL).  Plain, XCD-aware and no schedules;
+    the own-order stash under an XCD-aware schedule is a per-column permutation of the CSC-ordered one."""
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd.operators.fused_gat import gat_native
+    dev = torch.device("cuda:0")
+    for buckets, use_schedule in (("0", True), ("1", True), ("0", False)):
+        monkeypatch.setenv("FGNN_XCD_BUCKETS", buckets)
+        monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+        monkeypatch.setenv("FGNN_SEG_LEN", "256")
+        _lib.clear_schedule_cache()
+        g = graphs.add_csc_torch(degree_edge_graph(n=300, seed=51))
+        x, ar, ac, go = gat_inputs(g, h, f, 5)
+        ref = _oracle_fwd_bwd(g, x, ar, ac, go, 0.2)
+        alpha = orc.gat_forward(ar, ac, g.row_ptr, g.col_ind, 0.2, x, return_edge=True)[2]
+        gd = g.to(dev)
+        xd, ard, acd, god = (t.float().to(dev) for t in (x, ar, ac, go))
+        o = gat_native.gat_forward(ard, acd, gd.row_ptr, gd.col_ind, 0.2, xd, stash=True, stash_lrelu=False, use_schedule=use_schedule)
+        assert_close(o[6], alpha, "e_softmax in CSR order")
+        res_csr = gat_native.gat_backward(0.2, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, o[1], o[2], xd, ard, acd, god, out_feat=o[0],
+                                          out2=o[3], cc=o[4], permute=gd.permute, e_soft=o[6], use_schedule=use_schedule)
+        own = gat_native.gat_stash_own_order(0.2, gd.col_ptr, gd.row_ind, o[1], o[2], ard, acd, use_schedule=use_schedule)
+        res_own = gat_native.gat_backward(0.2, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, o[1], o[2], xd, ard, acd, god, out_feat=o[0],
+                                          out2=o[3], cc=o[4], permute=None, e_soft=own, use_schedule=use_schedule)
+        torch.cuda.synchronize()
+        for tag, res in (("CSR-ordered stash", res_csr), ("own-order stash", res_own)):
+            _check((o[0],) + tuple(res), ref, g, x, ar, ac, go, 0.2, tag=" (%s, buckets %s, schedule %s)" % (tag, buckets, use_schedule))
+        # the own-order stash holds alpha with the sign bit set where the pre-activation is not positive
+        e_csr = orc.gat_forward(ar, ac, g.row_ptr, g.col_ind, 0.2, x, return_edge=True)[1]
+        csc_alpha = alpha[g.permute.long()]
+        csc_signed = torch.where(e_csr[g.permute.long()] > 0, csc_alpha, -csc_alpha)
+        if buckets == "0":
+            assert_close(own, csc_signed, "own-order stash == signed alpha in CSC order without buckets")
+        else:       # same multiset of values inside every column
+            cp = g.col_ptr.long()
+            seg = torch.repeat_interleave(torch.arange(g.n), cp[1:] - cp[:-1])
+            a = torch.zeros(g.n, h, dtype=torch.float64).index_add_(0, seg, own.cpu().double())
+            b = torch.zeros(g.n, h, dtype=torch.float64).index_add_(0, seg, csc_signed)
+            assert_close(a, b, "column sums of the own-order stash")
+            a = torch.zeros(g.n, h, dtype=torch.float64).index_add_(0, seg, own.cpu().double().abs())
+            b = torch.zeros(g.n, h, dtype=torch.float64).index_add_(0, seg, csc_alpha)
+            assert_close(a, b, "column sums of |own-order stash|")
+            assert not torch.allclose(own.cpu().double(), csc_signed)
+    _lib.clear_schedule_cache()

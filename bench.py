@@ -1,16 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the fused GNN sparse-operator path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gat_c2|gat_c5|gat_c5_train|edgeconv_c3|gmm_c4]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gat_c2|gat_c5|gat_c5_train|edgeconv_c3|gmm_c4|gather_ceiling]
 
 Default workload = benchmark configuration 2: one fused GAT layer forward+backward (dense projection by
 torch.matmul, fused sparse op by libfgnn_hip.so) on a seeded R-MAT power-law graph with 232,965
 nodes and ~114.6 M edges plus self loops, features [N,256], 8 heads x 32, fp32.  A step is one
 layer forward + backward; inputs are resident in HBM before the timed region; graph
 preprocessing (csr2csc, schedules) is reported separately.  One JSON line is printed with the
-metric, the roofline record of the dominant kernel (algorithmic bytes / live HIP-event time) and
-a CPU baseline (the torch-composed DGL-style layer of oracle/ on the host cores, on a bounded
-sample of the same graph).
+metric, the roofline record of the dominant kernel and a CPU baseline (the torch-composed DGL-style
+layer of oracle/ on the host cores, on a bounded sample of the same graph).  The default run also
+measures the other benchmark configurations (EdgeConv C3, GMMConv C4, GAT C5 layer 1 and the C5
+training step) and appends them to the same line under "other_configs" (--no-others skips them).
+
+Roofline record: `achieved` is MEASURED bytes (rocprofv3 FETCH_SIZE + WRITE_SIZE of the entry point's
+kernels, kept in profiles/traffic.json) over the live HIP-event time, `frac` its share of the 8 TB/s HBM
+peak; the counters sit between L2 and the fabric, so this bounds the HBM traffic from above.  The rate of
+the no-reuse gather model (one full feature row per edge and pass) is reported next to it as
+`effective_gather_GBps`: it exceeds the HBM peak wherever gathered rows are served from the per-XCD L2.
 """
 from __future__ import annotations
 
@@ -26,28 +33,67 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published peak
 
-# L2<->fabric bytes per launch of the dominant kernels measured with rocprofv3 --pmc (FETCH_SIZE scaled
-# x2.000 and WRITE_SIZE x1.000 by the 1 GiB copy of --calibrate-copy; profiles/gat_kernels_gat_c2.md and
-# profiles/kernels_edgeconv_c3_gmm_c4_gat_c5_drivers.md); all kernels of the entry point summed.
-# They bound the HBM traffic from above.  None = not measured for that workload.
-MEASURED_TRAFFIC_BYTES = {
-    "gat_c2": {"fwd": 38_905_487_360, "bwd": 39_145_359_872},
-    "gat_c5_layer1": {"fwd": 60_759_466_188, "bwd": 68_750_860_697},
-    "gmm_c4": {"fwd": 995_238_707, "bwd": 1_676_252_057},
-    "edgeconv_c3": {"fwd": 123_305_574, "bwd": 73_504_972},
-}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+CSRC_DIR = os.path.join(ROOT, "ae_mlsys_gnn_amd", "csrc")
 
 
-def roofline_record(kernel, alg_bytes, ms, traffic):
-    """`achieved` is the algorithmic (no-reuse gather model) rate.  It can exceed the HBM peak when
-    gathered rows are served from the per-XCD L2; `traffic` / `traffic_frac` give the measured
-    L2<->fabric bytes and their share of the HBM peak next to it."""
-    rec = {"bound": "hbm", "kernel": kernel, "achieved": round(alg_bytes / ms / 1e6, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-           "frac": round(alg_bytes / ms / 1e6 / HBM_PEAK_GBPS, 4), "traffic": traffic, "alg_bytes": alg_bytes, "ms": round(ms, 4)}
+def csrc_digest():
+    """sha256 over the kernel sources: profiles/traffic.json records the digest its byte counts were measured at."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    for f in sorted(glob.glob(os.path.join(CSRC_DIR, "*.hip")) + glob.glob(os.path.join(CSRC_DIR, "*.h"))):
+        h.update(os.path.basename(f).encode())
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
+
+
+def measured_traffic(workload):
+    """L2<->fabric bytes per call of the entry points of `workload`, measured with rocprofv3 --pmc (FETCH_SIZE and
+    WRITE_SIZE, scaled by what the same counters read for a 1 GiB copy), from profiles/traffic.json.  Returns
+    (dict or None, stale): stale when the kernel sources have changed since the measurement."""
+    try:
+        with open(TRAFFIC_FILE) as fh:
+            t = json.load(fh)
+    except (OSError, ValueError):
+        return None, False
+    stale = t.get("csrc_sha256") != csrc_digest()
+    if stale:
+        print("bench.py: the kernel sources changed after profiles/traffic.json was measured (commit %s): byte counts may be stale"
+              % t.get("measured_at_commit"), file=sys.stderr)
+    return t.get("workloads", {}).get(workload), stale
+
+
+def roofline_record(kernel, alg_bytes, ms, traffic, stale=False, note=None):
+    """achieved / frac: measured L2<->fabric bytes (an upper bound on the HBM bytes) over the kernel time, against the
+    HBM peak.  effective_gather_GBps: the no-reuse gather model's bytes over the same time (cache-served rows count
+    in full, so it can exceed the peak).  Without a byte measurement the record falls back to the model and says so."""
+    eff = alg_bytes / ms / 1e6
+    rec = {"bound": "hbm", "kernel": kernel, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "traffic": traffic, "alg_bytes": alg_bytes, "ms": round(ms, 4),
+           "effective_gather_GBps": round(eff, 1), "effective_gather_frac": round(eff / HBM_PEAK_GBPS, 4)}
     if traffic:
-        rec["traffic_GBps"] = round(traffic / ms / 1e6, 1)
-        rec["traffic_frac"] = round(traffic / ms / 1e6 / HBM_PEAK_GBPS, 4)
+        rec["achieved"] = round(traffic / ms / 1e6, 1)
+        rec["frac"] = round(traffic / ms / 1e6 / HBM_PEAK_GBPS, 4)
+        rec["achieved_basis"] = "measured L2<->fabric bytes (rocprofv3 FETCH_SIZE + WRITE_SIZE, profiles/traffic.json) / live HIP-event time"
+        rec["limiter"] = ("L2<->fabric path; %.0f %% of the gathered bytes are served by the per-XCD L2" % (100 * (1 - traffic / alg_bytes))
+                          if traffic < 0.9 * alg_bytes else "HBM")
+        if stale:
+            rec["traffic_stale"] = True
+    else:
+        rec["achieved"] = round(eff, 1)
+        rec["frac"] = round(eff / HBM_PEAK_GBPS, 4)
+        rec["achieved_basis"] = "algorithmic bytes (no byte-counter measurement for this kernel)"
+    if note:
+        rec["note"] = note
     return rec
+
+
+def peak_hbm_gib():
+    """Peak device memory: torch's allocator plus what the library's schedules hold outside it."""
+    import torch
+    from ae_mlsys_gnn_amd import _lib
+    return (torch.cuda.max_memory_allocated() + _lib.schedule_device_bytes()) / 2**30
 
 
 def gat_alg_bytes(n, e, h, f):
@@ -114,19 +160,26 @@ def time_device_preprocessing(g):
 
 def cpu_baseline_gat(g, x_feat, layer, slope, target_edges, go):
     """The DGL-composed GAT layer (oracle.gat_layer_dgl: u_add_v, LeakyReLU, edge softmax,
-    u_mul_e + sum in plain torch) forward+backward on the host cores, on the sub-graph formed by the
-    first rows of the benchmark graph holding about `target_edges` edges; scaled to the full edge
-    count."""
+    u_mul_e + sum in plain torch) forward+backward on the host cores, on the sub-graph formed by a
+    seeded random sample of destination rows of the benchmark graph holding about `target_edges` edges
+    (all other rows empty; every source node kept); scaled to the full edge count."""
     import torch
     from oracle import fgnn_oracle as orc
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
-    rp = g.row_ptr.cpu()
-    r = int(torch.searchsorted(rp.long(), torch.tensor([target_edges])).item())
+    rp = g.row_ptr.cpu().long()
+    deg = rp[1:] - rp[:-1]
+    order = torch.randperm(g.n, generator=torch.Generator().manual_seed(12345))
+    r = int(torch.searchsorted(torch.cumsum(deg[order], 0), torch.tensor([target_edges])).item()) + 1
     r = max(1, min(r, g.n))
-    e_s = int(rp[r])
-    rp_s = torch.cat([rp[: r + 1], torch.full((g.n - r,), e_s, dtype=rp.dtype)])     # rows >= r are empty
-    ci_s = g.col_ind[:e_s].cpu()
+    rows = torch.sort(order[:r]).values
+    keep = torch.zeros(g.n, dtype=torch.long)
+    keep[rows] = deg[rows]
+    rp_s = torch.cat([torch.zeros(1, dtype=torch.long), torch.cumsum(keep, 0)]).to(torch.int32)
+    e_s = int(rp_s[-1])
+    seg = torch.repeat_interleave(torch.arange(r), deg[rows])
+    pos = rp[rows][seg] + (torch.arange(e_s) - (torch.cumsum(deg[rows], 0) - deg[rows])[seg])
+    ci_s = g.col_ind.cpu()[pos]
     feat = x_feat.detach().cpu()
     w_t = layer.W.detach().cpu().t().contiguous().requires_grad_(True)
     # weight mapping to GATConv_dgl: attn_l(dgl) = attn_r(ours), attn_r(dgl) = attn_l(ours)
@@ -230,18 +283,19 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
         lambda: gat_native.gat_backward(slope, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, o[1], o[2], h, a_row, a_col, go,
                                         out_feat=o[0], out2=o[3], cc=o[4]), args.steps, 2)
     b_fwd, b_bwd = gat_alg_bytes(n, e, heads, out_feats)
-    peak_mem = torch.cuda.max_memory_allocated() / 2**30
-    # stash variant of the same operator as the autograd function runs it: the per-edge softmax [E,H] written by the
-    # forward and read by the backward (the edge LeakyReLU values of the reference's stash are not needed and not written)
-    so = gat_native.gat_forward(a_row, a_col, g.row_ptr, g.col_ind, slope, h, stash=True, stash_lrelu=False)
-    ms_sf, _, _ = time_calls(lambda: gat_native.gat_forward(a_row, a_col, g.row_ptr, g.col_ind, slope, h, stash=True, stash_lrelu=False),
-                             max(3, args.steps // 4), 1)
+    traffic, stale = measured_traffic(workload)
+    peak_mem = peak_hbm_gib()
+    # stash variant as the autograd function runs it: the attention [E,H] written after the forward in the entry order of
+    # the backward pass (signed: the sign bit says whether the pre-activation was positive) and streamed by the backward
+    own = gat_native.gat_stash_own_order(slope, g.col_ptr, g.row_ind, o[1], o[2], a_row, a_col)
+    ms_sw, _, _ = time_calls(lambda: gat_native.gat_stash_own_order(slope, g.col_ptr, g.row_ind, o[1], o[2], a_row, a_col), max(3, args.steps // 4), 1)
+    ms_sf = ms_fwd + ms_sw
     ms_sb, _, _ = time_calls(
-        lambda: gat_native.gat_backward(slope, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, so[1], so[2], h, a_row, a_col, go,
-                                        out_feat=so[0], out2=so[3], cc=so[4], permute=g.permute, e_soft=so[6]),
+        lambda: gat_native.gat_backward(slope, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, o[1], o[2], h, a_row, a_col, go,
+                                        out_feat=o[0], out2=o[3], cc=o[4], permute=None, e_soft=own),
         max(3, args.steps // 4), 1)
     stash_bytes = e * heads * 4
-    del so
+    del own
     prep = time_device_preprocessing(g)
 
     if args.no_cpu_baseline:
@@ -257,21 +311,23 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
         "config": {"workload": workload, "graph": "R-MAT a=0.57 b=0.19 c=0.19 d=0.05 seed 0, unique edges + self loops",
                    "nodes": n, "edges": e, "in_feats": in_feats, "heads": heads, "out_feats": out_feats,
                    "negative_slope": slope, "step": "GATConv forward + backward (torch.matmul projection + fused sparse op)"},
-        "roofline": roofline_record("gat_fwd_kernel (+gat_fwd_merge_kernel)", b_fwd, ms_fwd, (MEASURED_TRAFFIC_BYTES.get(workload) or {}).get("fwd")),
+        "roofline": roofline_record("gat_fwd_kernel (+gat_fwd_merge_kernel)", b_fwd, ms_fwd, (traffic or {}).get("fwd"), stale),
         "roofline_bwd": roofline_record("gat_bwd_node_kernel + gat_bwd_kernel (+gat_bwd_merge_kernel)", b_bwd, ms_bwd,
-                                        (MEASURED_TRAFFIC_BYTES.get(workload) or {}).get("bwd")),
-        "stash_variant": {"fwd_ms": round(ms_sf, 4), "bwd_ms": round(ms_sb, 4), "stashed_GiB": round(stash_bytes / 2**30, 3)},
+                                        (traffic or {}).get("bwd"), stale),
+        "stash_variant": {"fwd_ms": round(ms_sf, 4), "stash_writer_ms": round(ms_sw, 4), "bwd_ms": round(ms_sb, 4),
+                          "stashed_GiB": round(stash_bytes / 2**30, 3)},
         "sparse_fwd_bwd": {"ms": round(ms_fwd + ms_bwd, 4), "alg_bytes": b_fwd + b_bwd,
                            "achieved_GBps": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6, 1),
                            "frac_of_peak": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6 / HBM_PEAK_GBPS, 4)},
         "cpu_baseline": None if args.no_cpu_baseline else {
             "value": round(cpu_ms * e / cpu_e, 1), "unit": "ms/iter", "cores": cores, "kind": "port",
-            "sample": "DGL-composed GAT layer (torch CPU, %d threads) fwd+bwd on the first %d rows = %d edges of the same graph: "
-                      "median %.1f ms over %d iters, scaled by E/E_sample = %.1f" % (cores, cpu_rows, cpu_e, cpu_ms, cpu_iters, e / cpu_e)},
+            "sample": "DGL-composed GAT layer (torch CPU, %d threads) fwd+bwd on a seeded random sample of %d destination rows = %d edges of the "
+                      "same graph: median %.1f ms over %d iters, scaled by E/E_sample = %.1f" % (cores, cpu_rows, cpu_e, cpu_ms, cpu_iters, e / cpu_e)},
         "cpu_baseline_c1": c1,
         "preprocess_s": {"graph_gen": round(t_gen, 3), "csr2csc_first_call": round(t_csc, 4), "schedules": round(t_sched, 4), **prep},
         "schedule": {"xcd_aware": s_csr.idx_tensor is not None, "csr_items": s_csr.n_items, "csr_partials": s_csr.n_partials,
-                     "csc_items": s_csc.n_items, "csc_partials": s_csc.n_partials},
+                     "csc_items": s_csc.n_items, "csc_partials": s_csc.n_partials,
+                     "device_GiB": round((s_csr.device_bytes() + s_csc.device_bytes()) / 2**30, 3)},
         "peak_hbm_GiB": round(peak_mem, 3),
     }
     return rec
@@ -316,6 +372,7 @@ def run_edgeconv(args):
     knn_graph(pts, k)
     ms_knn, _, _ = time_calls(lambda: knn_graph(pts, k), args.steps, args.warmup)
     e = n * k
+    traffic, stale = measured_traffic("edgeconv_c3")
     b_f = e * (4 * f + 4) + n * f * 12
     b_b = n * f * 20
     # CPU baseline: EdgeConv_reorg composed math on the host, full size (it is small)
@@ -338,8 +395,9 @@ def run_edgeconv(args):
         "config": {"workload": "edgeconv_c3", "clouds": bsz, "points": npts, "k": k, "F": f, "edges": e},
         "hip_graph_replay": {"fwd_bwd_us": round(ms_graph * 1e3, 2), "matches_eager": graph_ok},
         "knn_graph_ms": round(ms_knn, 3),
-        "roofline": roofline_record("edgeconv_fwd_kernel", b_f, ms_f, MEASURED_TRAFFIC_BYTES["edgeconv_c3"]["fwd"]),
-        "roofline_bwd": roofline_record("edgeconv_bwd_blocked_kernel (+ overflow kernel)", b_b, ms_b, None),
+        "roofline": roofline_record("edgeconv_fwd_kernel", b_f, ms_f, (traffic or {}).get("fwd"), stale,
+                                    note="237 MB of algorithmic bytes: launch-latency bound, not bandwidth bound"),
+        "roofline_bwd": roofline_record("edgeconv_bwd_blocked_kernel (+ overflow kernel)", b_b, ms_b, (traffic or {}).get("bwd_blocked"), stale),
         "backward_plain_scatter_us": round(ms_b_plain * 1e3, 2),
         "cpu_baseline": {"value": round(sorted(ts)[len(ts) // 2] * 1e3, 1), "unit": "us/iter", "cores": cores, "kind": "port",
                          "sample": "EdgeConv_reorg composed math (torch CPU gather + max over k) fwd+bwd at full size, median of 5"},
@@ -372,6 +430,7 @@ def run_gmm(args):
     ms_fs, _, _ = time_calls(lambda: gmm_native.gmmconv(g.row_ptr, g.col_ind, x, pseudo, mu, isg, sum_kernels=True), args.steps, args.warmup)
     ms_bs, _, _ = time_calls(lambda: gmm_native.gmmconv_backward(g.col_ptr, g.row_ind, g.permute, x, pseudo, mu, isg, go_s, sum_kernels=True),
                              args.steps, args.warmup)
+    traffic, stale = measured_traffic("gmm_c4")
     b_f = e * (4 * kk * f + 4 * dim + 4) + n * (4 * kk * f + 4)
     b_b = e * (4 * kk * f + 8 * dim + 12) + n * (8 * kk * f + 4)
     cores = os.cpu_count() or 1
@@ -391,8 +450,8 @@ def run_gmm(args):
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "gmm_c4", "nodes": n, "edges": e, "K": kk, "dim": dim, "F": f},
-        "roofline": roofline_record("spmm_kernel<WGauss>", b_f, ms_f, MEASURED_TRAFFIC_BYTES["gmm_c4"]["fwd"]),
-        "roofline_bwd": roofline_record("gmm_bwd_kernel + gauss_grad_small_kernel + column sums", b_b, ms_b, MEASURED_TRAFFIC_BYTES["gmm_c4"]["bwd"]),
+        "roofline": roofline_record("spmm_kernel<WGauss>", b_f, ms_f, (traffic or {}).get("fwd"), stale),
+        "roofline_bwd": roofline_record("gmm_bwd_kernel + gauss_grad_small_kernel + column sums", b_b, ms_b, (traffic or {}).get("bwd"), stale),
         "fused_sum_over_kernels": {"fwd_ms": round(ms_fs, 4), "bwd_ms": round(ms_bs, 4)},
         "cpu_baseline": {"value": round(sorted(ts)[1], 1), "unit": "ms/iter", "cores": cores, "kind": "port",
                          "sample": "GMMConv_dgl composed math (torch CPU) fwd+bwd at full size, median of 3"},
@@ -454,8 +513,9 @@ def run_gat_train(args):
             loss = step()
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) * 1e3 / args.steps
-        res[name] = {"ms_per_step": round(ms, 3), "peak_hbm_GiB": round(torch.cuda.max_memory_allocated() / 2**30, 3),
-                     "resident_before_GiB": round(base / 2**30, 3), "final_loss": round(float(loss), 5)}
+        res[name] = {"ms_per_step": round(ms, 3), "peak_hbm_GiB": round(peak_hbm_gib(), 3),
+                     "of_which_schedules_GiB": round(_lib.schedule_device_bytes() / 2**30, 3),
+                     "resident_before_GiB": round(base / 2**30, 3), "final_loss": round(float(loss.detach()), 5)}
         del model, opt
     b1 = gat_alg_bytes(n, e, heads, hidden)
     b2 = gat_alg_bytes(n, e, 1, classes)
@@ -468,10 +528,50 @@ def run_gat_train(args):
         "config": {"workload": "gat_c5_train", "nodes": n, "edges": e, "in_feats": in_dim, "hidden": "8x32", "classes": classes,
                    "optimizer": "Adam(lr=5e-3, weight_decay=5e-4)", "loss": "mean cross-entropy over all nodes (logsumexp - true-class logit)"},
         "variants": res,
-        "roofline": {"bound": "hbm", "kernel": "whole step (sparse ops of both layers, no-reuse gather model)", "achieved": round(alg / ms / 1e6, 1),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(alg / ms / 1e6 / HBM_PEAK_GBPS, 4), "traffic": None, "alg_bytes": alg},
+        "roofline": roofline_record("whole step (sparse ops of both layers; dense GEMMs, loss and Adam included in the time)", alg, ms, None),
         "cpu_baseline": None,
     }
+
+
+def run_gather_ceiling(args):
+    """What a bare feature-row gather reaches on this part, with the library's own unweighted SpMM (fgnn_mhspmm
+    without weights: one 1 KiB row gathered and added per edge, nothing else per edge): on the C2 graph as it is
+    (skewed sources, XCD-aware work list) and with every source replaced by a uniform random node (no reuse to
+    speak of: the rate of the L2<->fabric path itself), likewise at the C5 size (features far larger than the caches)."""
+    import torch
+    from ae_mlsys_gnn_amd import _lib, graphs
+    from ae_mlsys_gnn_amd.operators import mhspmm as mh
+    dev = torch.device("cuda:0")
+    h, f = 8, 32
+    out = {}
+    for name, n, e_t in (("c2_graph", 232965, 114_600_000), ("c5_graph", 2449029, 61_900_000)):
+        g = graphs.rmat_graph(n, e_t, seed=0, device=dev)
+        e = g.n_edges
+        x = torch.randn(n, h, f, device=dev)
+        alg = e * (4 * h * f + 4) + n * 4 * h * f
+        ms_skew, _, _ = time_calls(lambda: mh.mhspmm(g.row_ptr, g.col_ind, None, x), args.steps, 2)
+        ci = torch.randint(0, n, (e,), device=dev, dtype=torch.int32)
+        ms_unif, _, _ = time_calls(lambda: mh.mhspmm(g.row_ptr, ci, None, x), args.steps, 2)
+        out[name] = {"nodes": n, "edges": e, "row_bytes": 4 * h * f, "alg_bytes": alg,
+                     "own_sources": {"ms": round(ms_skew, 4), "effective_gather_GBps": round(alg / ms_skew / 1e6, 1)},
+                     "uniform_random_sources": {"ms": round(ms_unif, 4), "effective_gather_GBps": round(alg / ms_unif / 1e6, 1),
+                                                "frac_of_hbm_peak": round(alg / ms_unif / 1e6 / HBM_PEAK_GBPS, 4)}}
+        del g, x, ci
+        _lib.clear_schedule_cache()
+        torch.cuda.empty_cache()
+    ms = out["c2_graph"]["uniform_random_sources"]["ms"]
+    return {"metric": "bare 1 KiB feature-row gather (unweighted SpMM) ms + GB/s, 1 MI355X", "value": ms, "unit": "ms/iter", "n_gpus": 1,
+            "steps": args.steps, "warmup": 2, "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+            "dtype": "f32", "data": "synthetic", "config": {"workload": "gather_ceiling", "heads": h, "out_feats": f}, "graphs": out,
+            "roofline": roofline_record("spmm_kernel (unweighted), uniform random sources on the C2 degree sequence",
+                                        out["c2_graph"]["alg_bytes"], ms, None), "cpu_baseline": None}
+
+
+def brief(rec):
+    """The part of a workload's record that goes under "other_configs" of the default line."""
+    keep = ("metric", "value", "unit", "ms_per_step", "config", "roofline", "roofline_bwd", "variants", "stash_variant", "sparse_fwd_bwd",
+            "fused_sum_over_kernels", "hip_graph_replay", "knn_graph_ms", "backward_plain_scatter_us", "cpu_baseline", "peak_hbm_GiB")
+    return {k: rec[k] for k in keep if k in rec}
 
 
 def main():
@@ -479,7 +579,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="gat_c2", choices=["gat_c2", "gat_c5", "gat_c5_train", "edgeconv_c3", "gmm_c4"])
+    ap.add_argument("--workload", default="gat_c2", choices=["gat_c2", "gat_c5", "gat_c5_train", "edgeconv_c3", "gmm_c4", "gather_ceiling"])
+    ap.add_argument("--no-others", action="store_true", help="gat_c2 only: do not append the other benchmark configurations to the line")
     ap.add_argument("--cpu-sample-edges", type=int, default=1_500_000)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline (profiling runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -502,6 +603,29 @@ def main():
         del a, b
     if args.workload == "gat_c2":
         rec = run_gat(args, 232965, 114_600_000, 256, 8, 32, "gat_c2")
+        if not args.no_others:
+            # the other benchmark configurations, each on its own graph, after this one's memory has been returned
+            from ae_mlsys_gnn_amd import _lib
+            import gc
+            others = {}
+            sub = argparse.Namespace(**vars(args))
+            sub.steps, sub.warmup, sub.no_cpu_baseline = min(args.steps, 10), min(args.warmup, 3), True
+            for name, fn in (("edgeconv_c3", lambda: run_edgeconv(args)), ("gmm_c4", lambda: run_gmm(args)),
+                             ("gat_c5_layer1", lambda: run_gat(sub, 2449029, 61_900_000, 100, 8, 32, "gat_c5_layer1")),
+                             ("gat_c5_train", lambda: run_gat_train(sub))):
+                gc.collect()
+                _lib.clear_schedule_cache()
+                torch.cuda.empty_cache()
+                torch.cuda.reset_peak_memory_stats()
+                t0 = time.time()
+                try:
+                    others[name] = brief(fn())
+                except Exception as exc:          # a failing side measurement must not take the headline with it
+                    others[name] = {"error": "%s: %s" % (type(exc).__name__, exc)}
+                others[name]["wall_s"] = round(time.time() - t0, 1)
+            rec["other_configs"] = others
+    elif args.workload == "gather_ceiling":
+        rec = run_gather_ceiling(args)
     elif args.workload == "gat_c5":
         rec = run_gat(args, 2449029, 61_900_000, 100, 8, 32, "gat_c5_layer1")
     elif args.workload == "gat_c5_train":

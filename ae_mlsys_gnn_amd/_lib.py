@@ -31,6 +31,8 @@ _SIGNATURES = {
     "fgnn_schedule_num_partials": (c_int, [c_void_p]),
     "fgnn_schedule_num_edges": (c_int64, [c_void_p]),
     "fgnn_schedule_device_bytes": (c_size_t, [c_void_p]),
+    "fgnn_schedule_num_splits": (c_int, [c_void_p]),
+    "fgnn_schedule_export": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p]),
     "fgnn_validate_graph": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int64, c_void_p]),
     "fgnn_gat_forward_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int]),
     "fgnn_gat_forward": (c_int, [c_int, c_int64, c_int, c_int] + [c_void_p] * 4 + [c_float] + [c_void_p] * 8
@@ -158,6 +160,16 @@ class Schedule:
         self.n_partials = lib().fgnn_schedule_num_partials(handle)
         self.n_edges = lib().fgnn_schedule_num_edges(handle)
         self.own_order = False
+
+    def export(self):
+        """(items int32 [n_items, 4], splits int32 [n_split, 4]) on the device: the work list itself."""
+        dev = self.ptr_tensor.device
+        n_split = lib().fgnn_schedule_num_splits(self.handle)
+        items = torch.empty((self.n_items, 4), dtype=torch.int32, device=dev)
+        splits = torch.empty((n_split, 4), dtype=torch.int32, device=dev)
+        with torch.cuda.device(dev):
+            check(lib().fgnn_schedule_export(self.handle, ptr(items), ptr(splits), stream_ptr()), "fgnn_schedule_export")
+        return items, splits
 
     def device_bytes(self):
         """Device memory the schedule holds outside torch's allocator."""

@@ -43,6 +43,14 @@ static inline size_t fgnn_align256(size_t x) { return (x + 255) & ~(size_t)255; 
 // Fills n floats with v on `st` (a kernel, so it may be captured into a HIP graph).
 int fgnn_fill_f32(float *p, size_t n, float v, hipStream_t st);
 
+// Stable LSD radix sort of (key, payload) pairs and an inclusive int32 scan (fgnn_csr2csc.hip); device pointers.
+size_t fgnn_rs_sort_workspace(int64_t n);
+int fgnn_rs_key_bits(int n_keys);
+int fgnn_rs_sort_pairs(const int *keys_in, const int *pay_in, int64_t n, int key_bits, int *pay_out, const int **sorted_keys, void *workspace,
+                       hipStream_t st);
+size_t fgnn_scan_workspace(int64_t n);
+int fgnn_inclusive_scan_i32(const int *in, int64_t n, int *out, int *tile_sums, int *total_dev, hipStream_t st);
+
 // One work item: the edge range [begin, end) of `row`.  slot < 0: the item covers the whole
 // row and writes final results; slot >= 0: a segment of a split row, written as partial `slot`.
 struct fgnn_item { int row, begin, end, slot; };

@@ -396,6 +396,29 @@ __global__ __launch_bounds__(256) void scan_apply_kernel(int64_t n, const int *_
     }
 }
 
+// Library-internal entry points to the sort and the scan (the schedule builder uses them too).
+size_t fgnn_rs_sort_workspace(int64_t n) { return rs_sort_workspace(n); }
+int fgnn_rs_key_bits(int n_keys) { return rs_key_bits(n_keys); }
+int fgnn_rs_sort_pairs(const int *keys_in, const int *pay_in, int64_t n, int key_bits, int *pay_out, const int **sorted_keys, void *workspace,
+                       hipStream_t st)
+{
+    return rs_sort_pairs(keys_in, pay_in, n, key_bits, pay_out, sorted_keys, workspace, st);
+}
+size_t fgnn_scan_workspace(int64_t n) { return fgnn_align256(((size_t)((n + SC_TILE - 1) / SC_TILE) + 1) * sizeof(int)); }
+// out[i] = in[0] + ... + in[i]; *total_dev = the sum of all.  tile_sums: fgnn_scan_workspace(n) bytes.
+int fgnn_inclusive_scan_i32(const int *in, int64_t n, int *out, int *tile_sums, int *total_dev, hipStream_t st)
+{
+    const int nt = (int)((n + SC_TILE - 1) / SC_TILE);
+    hipLaunchKernelGGL(scan_tile_sums_kernel, dim3(nt), dim3(256), 0, st, n, in, tile_sums);
+    int rc = fgnn_launch_status("scan_tile_sums_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(scan_sums_kernel, dim3(1), dim3(256), 0, st, nt, tile_sums, total_dev);
+    rc = fgnn_launch_status("scan_sums_kernel");
+    if (rc) return rc;
+    hipLaunchKernelGGL(scan_apply_kernel, dim3(nt), dim3(256), 0, st, n, in, tile_sums, out);
+    return fgnn_launch_status("scan_apply_kernel");
+}
+
 // Compaction: the first entry of every group writes its source and destination at the group's
 // position; every input edge learns the position of its group.
 __global__ __launch_bounds__(256) void coo_compact_kernel(int64_t n, const int *__restrict__ dsts, const int *__restrict__ srcs,

@@ -1,6 +1,7 @@
 // Error reporting, version and row schedules of libfgnn_hip.so.
 #include <algorithm>
 #include <cstdarg>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 #include "fgnn_common.h"
@@ -132,12 +133,10 @@ static fgnn_schedule *new_schedule(const int32_t *ptr_dev, int n_rows, int64_t n
     return s;
 }
 
-extern "C" int fgnn_schedule_create(const int32_t *ptr_dev, int n_rows, int seg_len, void *stream, fgnn_schedule_t **out)
+// The work list built on the host from a read-back of the pointer array: the first implementation, kept as the
+// cross-check of the device builder below (FGNN_SCHEDULE_BUILDER=host selects it).
+static int schedule_create_host(const int32_t *ptr_dev, int n_rows, int seg_len, void *stream, fgnn_schedule_t **out)
 {
-    FGNN_REQUIRE(ptr_dev && out, FGNN_ERR_NULL, "fgnn_schedule_create: NULL argument");
-    FGNN_REQUIRE(n_rows >= 0, FGNN_ERR_SHAPE, "fgnn_schedule_create: n_rows=%d", n_rows);
-    if (seg_len <= 0) seg_len = 2048;
-    seg_len = (seg_len + 63) & ~63;
     hipStream_t st = (hipStream_t)stream;
     std::vector<int32_t> ptr;
     int rc = read_ptr(ptr_dev, n_rows, st, ptr);
@@ -177,14 +176,9 @@ extern "C" int fgnn_schedule_create(const int32_t *ptr_dev, int n_rows, int seg_
 // bucket, and lays the work items out so that workgroup w only gets segments of bucket w % 8.  Each
 // XCD's L2 then sees one eighth of the gathered rows, which is what lets the hot ones stay resident.
 // Shorter rows stay whole and are dealt round-robin.  Segments are partial results merged by row.
-extern "C" int fgnn_schedule_create_bucketed(const int32_t *ptr_dev, const int32_t *idx_dev, int n_rows, int seg_len, int min_deg,
-                                             int with_positions, void *stream, fgnn_schedule_t **out)
+static int schedule_create_bucketed_host(const int32_t *ptr_dev, const int32_t *idx_dev, int n_rows, int seg_len, int min_deg,
+                                         int with_positions, void *stream, fgnn_schedule_t **out)
 {
-    FGNN_REQUIRE(ptr_dev && out, FGNN_ERR_NULL, "fgnn_schedule_create_bucketed: NULL argument");
-    FGNN_REQUIRE(n_rows >= 0, FGNN_ERR_SHAPE, "fgnn_schedule_create_bucketed: n_rows=%d", n_rows);
-    if (seg_len <= 0) seg_len = 2048;
-    seg_len = (seg_len + 63) & ~63;
-    if (min_deg <= 0) min_deg = 64;
     hipStream_t st = (hipStream_t)stream;
     std::vector<int32_t> ptr;
     int rc = read_ptr(ptr_dev, n_rows, st, ptr);
@@ -262,6 +256,326 @@ extern "C" int fgnn_schedule_create_bucketed(const int32_t *ptr_dev, const int32
     *out = s;
     return 0;
 }
+
+// ------------------------------------------------------------------------------------------------
+// The same work lists built on the device.  Per row: how many segments it is cut into (count kernel), two scans
+// (first partial slot of every split row, rank of every split row), ONE read-back of a dozen counters for the
+// allocation sizes, then the segments and the whole rows are emitted in the host builder's generation order,
+// stably sorted longest first with the library's radix sort (per source bucket for an XCD-aware list) and placed.
+// Item for item the result equals the host builder's.
+struct SchedCounts { int err, n_part, n_split, e_total; int cntb[FGNN_NUM_XCD]; };
+
+// Pieces a range of `len` entries is cut into, as split_range does it; step = length of all but the last.
+static __host__ __device__ inline int sched_pieces(int len, int seg_len, int &step)
+{
+    const int nseg = (len + seg_len - 1) / seg_len;
+    step = (((len + nseg - 1) / nseg) + 63) & ~63;
+    return (len + step - 1) / step;
+}
+
+__global__ __launch_bounds__(256) void sched_count_kernel(int n_rows, const int *__restrict__ ptr, const int *__restrict__ bcnt, int cut, int seg_len,
+                                                          int *__restrict__ segs, int *__restrict__ longf, SchedCounts *__restrict__ c)
+{
+    __shared__ int cb[FGNN_NUM_XCD];
+    if (threadIdx.x < FGNN_NUM_XCD) cb[threadIdx.x] = 0;
+    __syncthreads();
+    const int row = (int)(blockIdx.x * 256 + threadIdx.x);
+    if (row < n_rows) {
+        const int pb = ptr[row], pe = ptr[row + 1];
+        const int deg = pe - pb;
+        int err = (row == 0 && pb != 0) ? 1 : 0;
+        if (deg < 0) err |= 2;
+        if (row == n_rows - 1) c->e_total = pe;
+        if (err) atomicOr(&c->err, err);
+        const bool lng = deg > cut;
+        int nseg = 0, step;
+        if (lng) {
+            if (bcnt) {
+#pragma unroll
+                for (int b = 0; b < FGNN_NUM_XCD; ++b) {
+                    const int cnt = bcnt[(size_t)row * FGNN_NUM_XCD + b];
+                    if (cnt > 0) { const int pc = sched_pieces(cnt, seg_len, step); nseg += pc; atomicAdd(&cb[b], pc); }
+                }
+            } else {
+                nseg = sched_pieces(deg, seg_len, step);
+            }
+        }
+        segs[row] = nseg;
+        longf[row] = lng ? 1 : 0;
+    }
+    __syncthreads();
+    if (bcnt && threadIdx.x < FGNN_NUM_XCD && cb[threadIdx.x]) atomicAdd(&c->cntb[threadIdx.x], cb[threadIdx.x]);
+}
+
+// Segments of the split rows into gen[slot] (slot order = rows ascending, buckets ascending, pieces ascending), with
+// the sort key of an XCD-aware list (bucket major, longest first); the split table; the whole rows into (wkey, wrow).
+__global__ __launch_bounds__(256) void sched_emit_kernel(int n_rows, const int *__restrict__ ptr, const int *__restrict__ bcnt, int cut, int seg_len,
+                                                         const int *__restrict__ segs, const int *__restrict__ seg_incl,
+                                                         const int *__restrict__ long_incl, fgnn_item *__restrict__ gen, int *__restrict__ key,
+                                                         fgnn_split *__restrict__ splits, int *__restrict__ wkey, int *__restrict__ wrow)
+{
+    const int row = (int)(blockIdx.x * 256 + threadIdx.x);
+    if (row >= n_rows) return;
+    const int pb = ptr[row], deg = ptr[row + 1] - pb;
+    if (deg > cut) {
+        int slot = seg_incl[row] - segs[row];
+        splits[long_incl[row] - 1] = fgnn_split{row, slot, segs[row], 0};
+        int b0 = pb;
+        const int nb = bcnt ? FGNN_NUM_XCD : 1;
+        for (int b = 0; b < nb; ++b) {
+            const int cnt = bcnt ? bcnt[(size_t)row * FGNN_NUM_XCD + b] : deg;
+            if (cnt > 0) {
+                int step;
+                (void)sched_pieces(cnt, seg_len, step);
+                for (int sb = b0; sb < b0 + cnt; sb += step) {
+                    const int se = min(b0 + cnt, sb + step);
+                    gen[slot] = fgnn_item{row, sb, se, slot};
+                    if (key) key[slot] = b * (seg_len + 1) + (seg_len - (se - sb));
+                    ++slot;
+                }
+            }
+            b0 += cnt;
+        }
+    } else {
+        const int w = row - long_incl[row];
+        wkey[w] = cut - deg;
+        wrow[w] = row;
+    }
+}
+
+struct SchedBucketStart { int v[FGNN_NUM_XCD]; };
+// XCD-aware list: sorted segment p of bucket b, k-th of its bucket, goes to workgroup (k / WPB) * 8 + b, wave k % WPB.
+__global__ __launch_bounds__(256) void sched_place_segments_kernel(int n_part, const int *__restrict__ sorted_slot, const int *__restrict__ sorted_key,
+                                                                   int seg_len, SchedBucketStart bs, const fgnn_item *__restrict__ gen,
+                                                                   fgnn_item *__restrict__ items)
+{
+    const int p = (int)(blockIdx.x * 256 + threadIdx.x);
+    if (p >= n_part) return;
+    const int b = sorted_key[p] / (seg_len + 1);
+    const int k = p - bs.v[b];
+    items[((size_t)(k / FGNN_WPB) * FGNN_NUM_XCD + b) * FGNN_WPB + (k % FGNN_WPB)] = gen[sorted_slot[p]];
+}
+// Whole rows, longest first: rank w goes to slot base + w (plain list) or is dealt round-robin over the eight buckets.
+__global__ __launch_bounds__(256) void sched_place_whole_kernel(int n_whole, const int *__restrict__ sorted_row, const int *__restrict__ ptr,
+                                                                int bucketed, size_t base, fgnn_item *__restrict__ items)
+{
+    const int w = (int)(blockIdx.x * 256 + threadIdx.x);
+    if (w >= n_whole) return;
+    const int row = sorted_row[w];
+    size_t dest = base + (size_t)w;
+    if (bucketed) {
+        const int b = w % FGNN_NUM_XCD, k = w / FGNN_NUM_XCD;
+        dest = base + ((size_t)(k / FGNN_WPB) * FGNN_NUM_XCD + b) * FGNN_WPB + (k % FGNN_WPB);
+    }
+    items[dest] = fgnn_item{row, ptr[row], ptr[row + 1], -1};
+}
+__global__ __launch_bounds__(256) void sched_fill_padding_kernel(size_t n, fgnn_item *__restrict__ items)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) items[i] = fgnn_item{-1, 0, 0, -1};
+}
+
+#define SCHED_HIP(call)                                                                 \
+    do {                                                                                \
+        hipError_t e__ = (call);                                                        \
+        if (e__ != hipSuccess && rc == 0) {                                             \
+            fgnn_set_error("schedule: %s failed: %s", #call, hipGetErrorString(e__));   \
+            rc = (int)e__;                                                              \
+        }                                                                               \
+    } while (0)
+
+// bcnt_dev: per (row, bucket) entry counts of an XCD-aware list (NULL: plain list); cut: rows longer than this are split.
+static int schedule_build_device(fgnn_schedule *s, const int32_t *ptr_dev, const int *bcnt_dev, int n_rows, int cut, int seg_len, hipStream_t st)
+{
+    if (n_rows == 0) return 0;
+    const bool bucketed = bcnt_dev != nullptr;
+    int rc = 0;
+    char *tmp1 = nullptr, *tmp2 = nullptr;
+    const size_t rb = fgnn_align256((size_t)n_rows * sizeof(int));
+    const size_t scan_b = fgnn_scan_workspace(n_rows);
+    SCHED_HIP(hipMalloc((void **)&tmp1, 4 * rb + scan_b + 512));
+    if (rc) return rc;
+    int *segs = (int *)tmp1, *longf = (int *)(tmp1 + rb), *seg_incl = (int *)(tmp1 + 2 * rb), *long_incl = (int *)(tmp1 + 3 * rb);
+    int *scan_ws = (int *)(tmp1 + 4 * rb);
+    SchedCounts *cnt_dev = (SchedCounts *)(tmp1 + 4 * rb + scan_b);          // 48 bytes, then two scan totals
+    int *tot = (int *)(cnt_dev + 1);
+    SchedCounts cnt;
+    memset(&cnt, 0, sizeof(cnt));
+    SCHED_HIP(hipMemcpyAsync(cnt_dev, &cnt, sizeof(cnt), hipMemcpyHostToDevice, st));
+    const unsigned gr = (unsigned)((n_rows + 255) / 256);
+    if (!rc) {
+        hipLaunchKernelGGL(sched_count_kernel, dim3(gr), dim3(256), 0, st, n_rows, ptr_dev, bcnt_dev, cut, seg_len, segs, longf, cnt_dev);
+        rc = fgnn_launch_status("sched_count_kernel");
+    }
+    if (!rc) rc = fgnn_inclusive_scan_i32(segs, n_rows, seg_incl, scan_ws, tot, st);
+    if (!rc) rc = fgnn_inclusive_scan_i32(longf, n_rows, long_incl, scan_ws, tot + 1, st);
+    int totals[2] = {0, 0};
+    SCHED_HIP(hipMemcpyAsync(&cnt, cnt_dev, sizeof(cnt), hipMemcpyDeviceToHost, st));
+    SCHED_HIP(hipMemcpyAsync(totals, tot, sizeof(totals), hipMemcpyDeviceToHost, st));
+    SCHED_HIP(hipStreamSynchronize(st));                                     // the one read-back: a dozen counters
+    if (!rc && cnt.err) {
+        fgnn_set_error("schedule: %s", (cnt.err & 1) ? "ptr[0] != 0" : "ptr decreases");
+        rc = FGNN_ERR_SHAPE;
+    }
+    if (rc) { (void)hipFree(tmp1); return rc; }
+    const int n_part = totals[0], n_split = totals[1], n_whole = n_rows - n_split;
+    s->n_edges = cnt.e_total;
+    s->n_partials = n_part;
+    s->n_split = n_split;
+    size_t base2 = (size_t)n_part;
+    SchedBucketStart bs;
+    if (bucketed) {
+        int longest = 0, run = 0;
+        for (int b = 0; b < FGNN_NUM_XCD; ++b) { bs.v[b] = run; run += cnt.cntb[b]; longest = std::max(longest, cnt.cntb[b]); }
+        base2 = (size_t)((longest + FGNN_WPB - 1) / FGNN_WPB) * FGNN_NUM_XCD * FGNN_WPB;
+        const int longest_tail = (n_whole + FGNN_NUM_XCD - 1) / FGNN_NUM_XCD;
+        s->n_items = (int)(base2 + (size_t)((longest_tail + FGNN_WPB - 1) / FGNN_WPB) * FGNN_NUM_XCD * FGNN_WPB);
+    } else {
+        for (int b = 0; b < FGNN_NUM_XCD; ++b) bs.v[b] = 0;
+        s->n_items = n_part + n_whole;
+    }
+    // second stage: sized by the counters
+    const size_t pb = fgnn_align256((size_t)std::max(n_part, 1) * sizeof(int)), wb = fgnn_align256((size_t)std::max(n_whole, 1) * sizeof(int));
+    const size_t gen_b = fgnn_align256((size_t)std::max(n_part, 1) * sizeof(fgnn_item));
+    const size_t sort_b = fgnn_align256(fgnn_rs_sort_workspace(std::max(std::max(n_part, n_whole), 1)));
+    SCHED_HIP(hipMalloc((void **)&tmp2, gen_b + 2 * pb + 3 * wb + sort_b));
+    if (!rc && s->n_items > 0) SCHED_HIP(hipMalloc((void **)&s->items_dev, (size_t)s->n_items * sizeof(fgnn_item)));
+    if (!rc && n_split > 0) SCHED_HIP(hipMalloc((void **)&s->split_dev, (size_t)n_split * sizeof(fgnn_split)));
+    if (!rc) {
+        fgnn_item *gen = (fgnn_item *)tmp2;
+        int *key = (int *)(tmp2 + gen_b), *pay = (int *)(tmp2 + gen_b + pb);
+        int *wkey = (int *)(tmp2 + gen_b + 2 * pb), *wrow = wkey + wb / sizeof(int), *wsorted = wrow + wb / sizeof(int);
+        void *sort_ws = tmp2 + gen_b + 2 * pb + 3 * wb;
+        // a plain list keeps its segments in generation order: they go straight into the item array
+        hipLaunchKernelGGL(sched_emit_kernel, dim3(gr), dim3(256), 0, st, n_rows, ptr_dev, bcnt_dev, cut, seg_len, segs, seg_incl, long_incl,
+                           bucketed ? gen : s->items_dev, bucketed ? key : nullptr, s->split_dev, wkey, wrow);
+        rc = fgnn_launch_status("sched_emit_kernel");
+        if (!rc && bucketed) {
+            hipLaunchKernelGGL(sched_fill_padding_kernel, dim3((unsigned)((s->n_items + 255) / 256)), dim3(256), 0, st, (size_t)s->n_items, s->items_dev);
+            rc = fgnn_launch_status("sched_fill_padding_kernel");
+            if (!rc && n_part > 0) {
+                const int *sorted_key = nullptr;
+                rc = fgnn_rs_sort_pairs(key, nullptr, n_part, fgnn_rs_key_bits(FGNN_NUM_XCD * (seg_len + 1)), pay, &sorted_key, sort_ws, st);
+                if (!rc) {
+                    hipLaunchKernelGGL(sched_place_segments_kernel, dim3((unsigned)((n_part + 255) / 256)), dim3(256), 0, st, n_part, pay, sorted_key,
+                                       seg_len, bs, gen, s->items_dev);
+                    rc = fgnn_launch_status("sched_place_segments_kernel");
+                }
+            }
+        }
+        if (!rc && n_whole > 0) {
+            const int *sorted_key = nullptr;
+            rc = fgnn_rs_sort_pairs(wkey, wrow, n_whole, fgnn_rs_key_bits(cut + 1), wsorted, &sorted_key, sort_ws, st);
+            if (!rc) {
+                hipLaunchKernelGGL(sched_place_whole_kernel, dim3((unsigned)((n_whole + 255) / 256)), dim3(256), 0, st, n_whole, wsorted, ptr_dev,
+                                   bucketed ? 1 : 0, base2, s->items_dev);
+                rc = fgnn_launch_status("sched_place_whole_kernel");
+            }
+        }
+    }
+    SCHED_HIP(hipStreamSynchronize(st));          // the temporaries are freed below
+    if (tmp2) (void)hipFree(tmp2);
+    (void)hipFree(tmp1);
+    return rc;
+}
+
+// out[0] |= 1: ptr[0] != 0; 2: ptr decreases somewhere; out[1] = ptr[n_rows]
+__global__ __launch_bounds__(256) void sched_check_ptr_kernel(int n_rows, const int *__restrict__ ptr, int *__restrict__ out)
+{
+    int bad = 0;
+    for (int i = (int)(blockIdx.x * 256 + threadIdx.x); i < n_rows; i += (int)(gridDim.x * 256)) {
+        if (i == 0 && ptr[0] != 0) bad |= 1;
+        if (ptr[i + 1] < ptr[i]) bad |= 2;
+        if (i == n_rows - 1) out[1] = ptr[n_rows];
+    }
+    if (bad) atomicOr(out, bad);
+}
+
+static bool schedule_builder_is_host()
+{
+    const char *v = getenv("FGNN_SCHEDULE_BUILDER");
+    return v && strcmp(v, "host") == 0;
+}
+
+extern "C" int fgnn_schedule_create(const int32_t *ptr_dev, int n_rows, int seg_len, void *stream, fgnn_schedule_t **out)
+{
+    FGNN_REQUIRE(ptr_dev && out, FGNN_ERR_NULL, "fgnn_schedule_create: NULL argument");
+    FGNN_REQUIRE(n_rows >= 0, FGNN_ERR_SHAPE, "fgnn_schedule_create: n_rows=%d", n_rows);
+    if (seg_len <= 0) seg_len = 2048;
+    seg_len = (seg_len + 63) & ~63;
+    if (schedule_builder_is_host()) return schedule_create_host(ptr_dev, n_rows, seg_len, stream, out);
+    fgnn_schedule *s = new_schedule(ptr_dev, n_rows, 0, seg_len);
+    int rc = schedule_build_device(s, ptr_dev, nullptr, n_rows, seg_len, seg_len, (hipStream_t)stream);
+    if (rc) { fgnn_schedule_destroy(s); return rc; }
+    *out = s;
+    return 0;
+}
+
+extern "C" int fgnn_schedule_create_bucketed(const int32_t *ptr_dev, const int32_t *idx_dev, int n_rows, int seg_len, int min_deg,
+                                             int with_positions, void *stream, fgnn_schedule_t **out)
+{
+    FGNN_REQUIRE(ptr_dev && out, FGNN_ERR_NULL, "fgnn_schedule_create_bucketed: NULL argument");
+    FGNN_REQUIRE(n_rows >= 0, FGNN_ERR_SHAPE, "fgnn_schedule_create_bucketed: n_rows=%d", n_rows);
+    if (seg_len <= 0) seg_len = 2048;
+    seg_len = (seg_len + 63) & ~63;
+    if (min_deg <= 0) min_deg = 64;
+    if (schedule_builder_is_host()) return schedule_create_bucketed_host(ptr_dev, idx_dev, n_rows, seg_len, min_deg, with_positions, stream, out);
+    hipStream_t st = (hipStream_t)stream;
+    // the pointer array is checked before the partition kernel walks the index array with it; the same 8-byte
+    // read-back brings the edge count, which sizes the bucket-ordered copies
+    int32_t e32 = 0;
+    if (n_rows > 0) {
+        int *chk_dev = nullptr, chk[2] = {0, 0};
+        FGNN_HIP(hipMalloc((void **)&chk_dev, sizeof(chk)));
+        hipError_t err = hipMemcpyAsync(chk_dev, chk, sizeof(chk), hipMemcpyHostToDevice, st);
+        if (err == hipSuccess) {
+            hipLaunchKernelGGL(sched_check_ptr_kernel, dim3((unsigned)std::min((n_rows + 255) / 256, 4096)), dim3(256), 0, st, n_rows, ptr_dev, chk_dev);
+            err = hipGetLastError();
+        }
+        if (err == hipSuccess) err = hipMemcpyAsync(chk, chk_dev, sizeof(chk), hipMemcpyDeviceToHost, st);
+        if (err == hipSuccess) err = hipStreamSynchronize(st);
+        (void)hipFree(chk_dev);
+        if (err != hipSuccess) { fgnn_set_error("fgnn_schedule_create_bucketed: %s", hipGetErrorString(err)); return (int)err; }
+        FGNN_REQUIRE(chk[0] == 0, FGNN_ERR_SHAPE, "schedule: %s", (chk[0] & 1) ? "ptr[0] != 0" : "ptr decreases");
+        e32 = chk[1];
+    }
+    FGNN_REQUIRE(e32 >= 0, FGNN_ERR_SHAPE, "schedule: ptr[n_rows]=%d", e32);
+    FGNN_REQUIRE(idx_dev || e32 == 0, FGNN_ERR_NULL, "fgnn_schedule_create_bucketed: idx is NULL");
+    fgnn_schedule *s = new_schedule(ptr_dev, n_rows, e32, seg_len);
+    s->n_buckets = FGNN_NUM_XCD;
+    s->idx_src_dev = idx_dev;
+    int rc = 0;
+    int32_t *bcnt_dev = nullptr;
+    if (n_rows > 0) {
+        SCHED_HIP(hipMalloc((void **)&bcnt_dev, (size_t)n_rows * FGNN_NUM_XCD * sizeof(int32_t)));
+        if (!rc && e32 > 0) SCHED_HIP(hipMalloc((void **)&s->bidx_dev, (size_t)e32 * sizeof(int32_t)));
+        if (!rc && e32 > 0 && with_positions) SCHED_HIP(hipMalloc((void **)&s->bpos_dev, (size_t)e32 * sizeof(int32_t)));
+        if (!rc) {
+            hipLaunchKernelGGL(bucket_partition_kernel, dim3((unsigned)((n_rows + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, st,
+                               n_rows, ptr_dev, idx_dev, s->bidx_dev, s->bpos_dev, bcnt_dev);
+            rc = fgnn_launch_status("bucket_partition_kernel");
+        }
+        if (!rc) rc = schedule_build_device(s, ptr_dev, bcnt_dev, n_rows, min_deg, seg_len, st);
+        if (bcnt_dev) (void)hipFree(bcnt_dev);
+    }
+    if (rc) { fgnn_schedule_destroy(s); return rc; }
+    *out = s;
+    return 0;
+}
+
+// Copies the work items (4 ints each: row, begin, end, slot) and the split table (4 ints each: row, first slot,
+// segments, 0) to caller memory on the device; either pointer may be NULL.
+extern "C" int fgnn_schedule_export(const fgnn_schedule_t *s, int32_t *items_out, int32_t *splits_out, void *stream)
+{
+    FGNN_REQUIRE(s, FGNN_ERR_NULL, "fgnn_schedule_export: NULL schedule");
+    hipStream_t st = (hipStream_t)stream;
+    if (items_out && s->n_items > 0)
+        FGNN_HIP(hipMemcpyAsync(items_out, s->items_dev, (size_t)s->n_items * sizeof(fgnn_item), hipMemcpyDeviceToDevice, st));
+    if (splits_out && s->n_split > 0)
+        FGNN_HIP(hipMemcpyAsync(splits_out, s->split_dev, (size_t)s->n_split * sizeof(fgnn_split), hipMemcpyDeviceToDevice, st));
+    return 0;
+}
+extern "C" int fgnn_schedule_num_splits(const fgnn_schedule_t *s) { return s ? s->n_split : 0; }
 
 __global__ __launch_bounds__(256) void iota_i32_kernel(int64_t n, int *__restrict__ out)
 {

@@ -44,7 +44,11 @@ const char *fgnn_last_error(void);
  * reduced separately and merged, and the work items are ordered longest first.  The reference
  * has no counterpart (it launches one block per row: src/fused_gat/fused_gat_SM.cu:518-532);
  * passing sched == NULL to an operator selects the same one-wave-per-row mapping.
- * fgnn_schedule_create reads `ptr` back to the host once (it synchronises `stream`). */
+ * The list is built on the device (segment counts per row, two scans, a stable radix sort by length); only a dozen
+ * counters come back to the host for the allocation sizes, which synchronises `stream` once or twice.  The
+ * reference prepares its graphs on the host with scipy (script/train/train_gatconv_our.py:87-121).
+ * FGNN_SCHEDULE_BUILDER=host in the environment selects the first implementation instead (the pointer array read
+ * back and the list built by the host): item for item the same list, kept as the cross-check. */
 typedef struct fgnn_schedule fgnn_schedule_t;
 int     fgnn_schedule_create(const int32_t *ptr_dev, int n_rows, int seg_len, void *stream,
                              fgnn_schedule_t **out);
@@ -76,6 +80,12 @@ int64_t fgnn_schedule_num_edges(const fgnn_schedule_t *s);
  * position map of an XCD-aware schedule): allocated by the library outside the caller's allocator, so a
  * caller that reports peak memory adds it.  No counterpart in the reference. */
 size_t  fgnn_schedule_device_bytes(const fgnn_schedule_t *s);
+/* For inspection and tests: the work items (4 ints each: row, begin, end, partial slot or -1; row -1 = padding of an
+ * XCD-aware list) and the table of split rows (4 ints each: row, first slot, segments, 0) copied to device memory of
+ * the caller; items_out holds 4 * fgnn_schedule_num_items ints, splits_out 4 * fgnn_schedule_num_splits; either
+ * may be NULL. */
+int     fgnn_schedule_num_splits(const fgnn_schedule_t *s);
+int     fgnn_schedule_export(const fgnn_schedule_t *s, int32_t *items_out, int32_t *splits_out, void *stream);
 
 /* Checks a CSR (or CSC) pair before any gather kernel sees it: ptr[0] == 0, ptr non-decreasing,
  * ptr[n_rows] == E and every idx in [0, n_cols).  One reduction kernel and a 4-byte read-back (synchronises

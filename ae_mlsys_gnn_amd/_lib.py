@@ -43,6 +43,9 @@ _SIGNATURES = {
     "fgnn_gat_stash_own_order": (c_int, [c_int, c_int64, c_int, c_float] + [c_void_p] * 7 + [c_void_p, c_void_p]),
     "fgnn_edgeconv_forward": (c_int, [c_int, c_int, c_int, c_int] + [c_void_p] * 5 + [c_void_p]),
     "fgnn_edgeconv_backward": (c_int, [c_int, c_int, c_int] + [c_void_p] * 3 + [c_void_p]),
+    "fgnn_edgeconv_forward_lrelu": (c_int, [c_int, c_int, c_int, c_int] + [c_void_p] * 3 + [c_float] + [c_void_p] * 2 + [c_void_p]),
+    "fgnn_edgeconv_backward_lrelu": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float] + [c_void_p] * 3
+                                     + [c_void_p, c_size_t, c_void_p]),
     "fgnn_edgeconv_backward_blocked_workspace_bytes": (c_size_t, [c_int, c_int]),
     "fgnn_edgeconv_backward_blocked": (c_int, [c_int, c_int, c_int, c_int] + [c_void_p] * 4 + [c_size_t, c_void_p]),
     "fgnn_edgeconv_backward_blocked_static_max_elems": (c_size_t, []),
@@ -51,6 +54,7 @@ _SIGNATURES = {
     "fgnn_gmm_forward_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int]),
     "fgnn_gmm_forward": (c_int, [c_int, c_int64, c_int, c_int, c_int] + [c_void_p] * 9 + [c_int]
                          + [c_void_p, c_void_p, c_size_t, c_void_p]),
+    "fgnn_gmm_forward_epilogue": (c_int, [c_int, c_int64, c_int, c_int, c_int] + [c_void_p] * 11 + [c_void_p, c_void_p, c_size_t, c_void_p]),
     "fgnn_gmm_backward_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int, c_int]),
     "fgnn_gmm_backward": (c_int, [c_int, c_int64, c_int, c_int, c_int] + [c_void_p] * 8 + [c_int] + [c_void_p] * 4
                           + [c_void_p, c_void_p, c_size_t, c_void_p]),

@@ -15,7 +15,7 @@
 template <int VEC>
 __global__ __launch_bounds__(256) void edgeconv_fwd_kernel(int N, int F, int k, const int *__restrict__ src_ind,
                                                            const float *__restrict__ h_src, const float *__restrict__ h_dst,
-                                                           float *__restrict__ out, int *__restrict__ argmax)
+                                                           float out_slope, float *__restrict__ out, int *__restrict__ argmax)
 {
     const int per = F / VEC;
     const long long tid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -57,7 +57,8 @@ __global__ __launch_bounds__(256) void edgeconv_fwd_kernel(int N, int F, int k, 
     }
 #pragma unroll
     for (int c = 0; c < VEC; ++c) {
-        out[(size_t)node * F + fo + c] = best[c];
+        // optional LeakyReLU on the way out (out_slope == 1: the identity, bit for bit)
+        out[(size_t)node * F + fo + c] = best[c] > 0.f ? best[c] : best[c] * out_slope;
         argmax[(size_t)node * F + fo + c] = arg[c];
     }
 }
@@ -72,13 +73,23 @@ __global__ __launch_bounds__(256) void fgnn_fill_f32_kernel(float *p, size_t n, 
 // grad_src[argmax[i,f], f] += grad_out[i,f].  grad_src is cleared by a fill kernel on the same
 // stream first (the reference clears inside the scattering kernel and races,
 // src/fused_edgeconv/fused_edgeconv.cu:184-185).
+// act_out != NULL: the forward ended in LeakyReLU(act_slope) and act_out is its output; the gradient of the
+// pre-activation, grad_out * (act_out > 0 ? 1 : act_slope), is what gets scattered, and it is written to grad_dst
+// (the gradient of h_dst) on the way.
+__device__ __forceinline__ float ec_masked(float g, const float *act_out, float act_slope, long long i)
+{
+    return act_out ? (act_out[i] > 0.f ? g : g * act_slope) : g;
+}
 __global__ __launch_bounds__(256) void edgeconv_bwd_kernel(long long total, int F, const int *__restrict__ argmax,
-                                                           const float *__restrict__ grad_out, float *__restrict__ grad_src)
+                                                           const float *__restrict__ grad_out, const float *__restrict__ act_out, float act_slope,
+                                                           float *__restrict__ grad_src, float *__restrict__ grad_dst)
 {
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;
     int f = (int)(i % F);
-    unsafeAtomicAdd(grad_src + (size_t)argmax[i] * F + f, grad_out[i]);     // hardware float add (device memory), no CAS loop
+    const float g = ec_masked(grad_out[i], act_out, act_slope, i);
+    if (grad_dst) grad_dst[i] = g;
+    unsafeAtomicAdd(grad_src + (size_t)argmax[i] * F + f, g);     // hardware float add (device memory), no CAS loop
 }
 
 int fgnn_fill_f32(float *p, size_t n, float v, hipStream_t st)
@@ -90,24 +101,38 @@ int fgnn_fill_f32(float *p, size_t n, float v, hipStream_t st)
     return fgnn_launch_status("fill");
 }
 
-extern "C" int fgnn_edgeconv_forward(int N, int n_src, int F, int k, const int32_t *src_ind, const float *h_src,
-                                     const float *h_dst, float *out, int32_t *argmax, void *stream)
+static int edgeconv_forward_run(const char *fn, int N, int n_src, int F, int k, const int32_t *src_ind, const float *h_src,
+                                const float *h_dst, float out_slope, float *out, int32_t *argmax, void *stream)
 {
-    FGNN_REQUIRE(N >= 0 && n_src >= 0 && F >= 1 && k >= 1, FGNN_ERR_SHAPE, "fgnn_edgeconv_forward: bad sizes N=%d n_src=%d F=%d k=%d", N, n_src, F, k);
-    FGNN_REQUIRE(src_ind && h_src && h_dst && out && argmax, FGNN_ERR_NULL, "fgnn_edgeconv_forward: NULL argument");
-    FGNN_REQUIRE((int64_t)N * k <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_edgeconv_forward: N*k exceeds int32");
+    FGNN_REQUIRE(N >= 0 && n_src >= 0 && F >= 1 && k >= 1, FGNN_ERR_SHAPE, "%s: bad sizes N=%d n_src=%d F=%d k=%d", fn, N, n_src, F, k);
+    FGNN_REQUIRE(src_ind && h_src && h_dst && out && argmax, FGNN_ERR_NULL, "%s: NULL argument", fn);
+    FGNN_REQUIRE((int64_t)N * k <= 2147483647LL, FGNN_ERR_LIMIT, "%s: N*k exceeds int32", fn);
     if (N == 0) return 0;
     hipStream_t st = (hipStream_t)stream;
     bool v4 = (F % 4 == 0) && fgnn_aligned16(h_src) && fgnn_aligned16(h_dst);
     long long threads = (long long)N * (v4 ? F / 4 : F);
     unsigned grid = (unsigned)((threads + 255) / 256);
-    if (v4) hipLaunchKernelGGL(edgeconv_fwd_kernel<4>, dim3(grid), dim3(256), 0, st, N, F, k, src_ind, h_src, h_dst, out, argmax);
-    else hipLaunchKernelGGL(edgeconv_fwd_kernel<1>, dim3(grid), dim3(256), 0, st, N, F, k, src_ind, h_src, h_dst, out, argmax);
+    if (v4) hipLaunchKernelGGL(edgeconv_fwd_kernel<4>, dim3(grid), dim3(256), 0, st, N, F, k, src_ind, h_src, h_dst, out_slope, out, argmax);
+    else hipLaunchKernelGGL(edgeconv_fwd_kernel<1>, dim3(grid), dim3(256), 0, st, N, F, k, src_ind, h_src, h_dst, out_slope, out, argmax);
     return fgnn_launch_status("edgeconv_fwd_kernel");
 }
 
-extern "C" int fgnn_edgeconv_backward(int N, int n_src, int F, const int32_t *argmax, const float *grad_out,
-                                      float *grad_src, void *stream)
+extern "C" int fgnn_edgeconv_forward(int N, int n_src, int F, int k, const int32_t *src_ind, const float *h_src,
+                                     const float *h_dst, float *out, int32_t *argmax, void *stream)
+{
+    return edgeconv_forward_run("fgnn_edgeconv_forward", N, n_src, F, k, src_ind, h_src, h_dst, 1.f, out, argmax, stream);
+}
+
+extern "C" int fgnn_edgeconv_forward_lrelu(int N, int n_src, int F, int k, const int32_t *src_ind, const float *h_src,
+                                           const float *h_dst, float out_slope, float *out, int32_t *argmax, void *stream)
+{
+    FGNN_REQUIRE(out_slope > 0.f, FGNN_ERR_LIMIT, "fgnn_edgeconv_forward_lrelu: out_slope=%g; the backward reads the sign of the pre-activation "
+                 "off the output, which needs a positive slope", (double)out_slope);
+    return edgeconv_forward_run("fgnn_edgeconv_forward_lrelu", N, n_src, F, k, src_ind, h_src, h_dst, out_slope, out, argmax, stream);
+}
+
+static int edgeconv_backward_run(int N, int n_src, int F, const int32_t *argmax, const float *grad_out, const float *act_out, float act_slope,
+                                 float *grad_src, float *grad_dst, void *stream)
 {
     FGNN_REQUIRE(N >= 0 && n_src >= 0 && F >= 1, FGNN_ERR_SHAPE, "fgnn_edgeconv_backward: bad sizes");
     FGNN_REQUIRE(argmax && grad_out && grad_src, FGNN_ERR_NULL, "fgnn_edgeconv_backward: NULL argument");
@@ -117,8 +142,14 @@ extern "C" int fgnn_edgeconv_backward(int N, int n_src, int F, const int32_t *ar
     long long total = (long long)N * F;
     if (total == 0) return 0;
     unsigned grid = (unsigned)((total + 255) / 256);
-    hipLaunchKernelGGL(edgeconv_bwd_kernel, dim3(grid), dim3(256), 0, st, total, F, argmax, grad_out, grad_src);
+    hipLaunchKernelGGL(edgeconv_bwd_kernel, dim3(grid), dim3(256), 0, st, total, F, argmax, grad_out, act_out, act_slope, grad_src, grad_dst);
     return fgnn_launch_status("edgeconv_bwd_kernel");
+}
+
+extern "C" int fgnn_edgeconv_backward(int N, int n_src, int F, const int32_t *argmax, const float *grad_out,
+                                      float *grad_src, void *stream)
+{
+    return edgeconv_backward_run(N, n_src, F, argmax, grad_out, nullptr, 1.f, grad_src, nullptr, stream);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -134,7 +165,8 @@ extern "C" int fgnn_edgeconv_backward(int N, int n_src, int F, const int32_t *ar
 #define EC_BT 1024      // threads per workgroup of the blocked backward
 template <int FS>
 __global__ __launch_bounds__(EC_BT) void edgeconv_bwd_blocked_kernel(int N, int F, int block, const int *__restrict__ argmax,
-                                                                     const float *__restrict__ grad_out, float *__restrict__ grad_src,
+                                                                     const float *__restrict__ grad_out, const float *__restrict__ act_out,
+                                                                     float act_slope, float *__restrict__ grad_src, float *__restrict__ grad_dst,
                                                                      int *__restrict__ ovf)
 {
     extern __shared__ float tile[];                 // [rows of the block][FS]
@@ -155,7 +187,8 @@ __global__ __launch_bounds__(EC_BT) void edgeconv_bwd_blocked_kernel(int N, int 
             ok[u] = i < total && ff < fs;
             g[u] = (r0 + r) * F + f0 + ff;           // N*F < 2^31 is checked on the host
             a[u] = ok[u] ? argmax[g[u]] : 0;
-            v[u] = ok[u] ? grad_out[g[u]] : 0.f;
+            v[u] = ok[u] ? ec_masked(grad_out[g[u]], act_out, act_slope, g[u]) : 0.f;
+            if (ok[u] && grad_dst) grad_dst[g[u]] = v[u];
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -179,12 +212,13 @@ __global__ __launch_bounds__(EC_BT) void edgeconv_bwd_blocked_kernel(int N, int 
 }
 
 __global__ __launch_bounds__(256) void edgeconv_bwd_overflow_kernel(int F, const int *__restrict__ argmax, const float *__restrict__ grad_out,
+                                                                    const float *__restrict__ act_out, float act_slope,
                                                                     float *__restrict__ grad_src, const int *__restrict__ ovf)
 {
     const int count = ovf[0];
     for (int i = (int)(blockIdx.x * 256 + threadIdx.x); i < count; i += (int)(gridDim.x * 256)) {
         const int g = ovf[EC_OVF_HEADER + i];
-        unsafeAtomicAdd(grad_src + (size_t)argmax[g] * F + (g % F), grad_out[g]);
+        unsafeAtomicAdd(grad_src + (size_t)argmax[g] * F + (g % F), ec_masked(grad_out[g], act_out, act_slope, g));
     }
 }
 
@@ -198,18 +232,18 @@ static inline int ec_blocked_fs(int block) { return block <= 2048 ? 8 : block <=
 
 // The two launches of the blocked backward; ovf: (N*F + EC_OVF_HEADER) ints of device scratch.
 static int edgeconv_backward_blocked_run(int N, int F, int block, int fs, const int32_t *argmax, const float *grad_out, float *grad_src,
-                                         int *ovf, hipStream_t st)
+                                         int *ovf, hipStream_t st, const float *act_out = nullptr, float act_slope = 1.f, float *grad_dst = nullptr)
 {
     int rc = fgnn_fill_f32((float *)ovf, 1, 0.f, st);        // the counter (bit pattern of 0.0f is integer 0); a kernel, so capturable
     if (rc) return rc;
     dim3 grid((unsigned)((F + fs - 1) / fs), (unsigned)((N + block - 1) / block));
     FGNN_REQUIRE(grid.y <= 65535, FGNN_ERR_LIMIT, "fgnn_edgeconv_backward_blocked: more than 65535 blocks");
     const size_t shm = (size_t)block * fs * sizeof(float);
-    if (fs == 8) hipLaunchKernelGGL(edgeconv_bwd_blocked_kernel<8>, grid, dim3(EC_BT), shm, st, N, F, block, argmax, grad_out, grad_src, ovf);
-    else hipLaunchKernelGGL(edgeconv_bwd_blocked_kernel<4>, grid, dim3(EC_BT), shm, st, N, F, block, argmax, grad_out, grad_src, ovf);
+    if (fs == 8) hipLaunchKernelGGL(edgeconv_bwd_blocked_kernel<8>, grid, dim3(EC_BT), shm, st, N, F, block, argmax, grad_out, act_out, act_slope, grad_src, grad_dst, ovf);
+    else hipLaunchKernelGGL(edgeconv_bwd_blocked_kernel<4>, grid, dim3(EC_BT), shm, st, N, F, block, argmax, grad_out, act_out, act_slope, grad_src, grad_dst, ovf);
     rc = fgnn_launch_status("edgeconv_bwd_blocked_kernel");
     if (rc) return rc;
-    hipLaunchKernelGGL(edgeconv_bwd_overflow_kernel, dim3(64), dim3(256), 0, st, F, argmax, grad_out, grad_src, ovf);
+    hipLaunchKernelGGL(edgeconv_bwd_overflow_kernel, dim3(64), dim3(256), 0, st, F, argmax, grad_out, act_out, act_slope, grad_src, ovf);
     return fgnn_launch_status("edgeconv_bwd_overflow_kernel");
 }
 
@@ -277,4 +311,26 @@ extern "C" int fgnn_edgeconv_backward_blocked_static(int N, int n_src, int F, in
     if (rc) return rc;
     // the list is rebuilt from its counter (cleared first) on every call: nothing of an earlier call is read
     return edgeconv_backward_blocked_run(N, F, block, fs, argmax, grad_out, grad_src, ovf, (hipStream_t)stream);
+}
+
+// The backward of fgnn_edgeconv_forward_lrelu: the LeakyReLU mask is replayed from the forward's output while the
+// gradient is scattered, and the masked gradient (the gradient of h_dst) is written on the way: no separate
+// elementwise pass in either direction.  block <= 0: plain scatter; block > 0: the blocked form (workspace as for
+// fgnn_edgeconv_backward_blocked).
+extern "C" int fgnn_edgeconv_backward_lrelu(int N, int n_src, int F, int block, const int32_t *argmax, const float *out, float out_slope,
+                                            const float *grad_out, float *grad_src, float *grad_dst, void *workspace, size_t workspace_bytes,
+                                            void *stream)
+{
+    FGNN_REQUIRE(N >= 0 && n_src >= 0 && F >= 1, FGNN_ERR_SHAPE, "fgnn_edgeconv_backward_lrelu: bad sizes");
+    FGNN_REQUIRE(argmax && out && grad_out && grad_src && grad_dst, FGNN_ERR_NULL, "fgnn_edgeconv_backward_lrelu: NULL argument");
+    FGNN_REQUIRE(out_slope > 0.f, FGNN_ERR_LIMIT, "fgnn_edgeconv_backward_lrelu: out_slope=%g must be positive", (double)out_slope);
+    FGNN_REQUIRE((int64_t)N * F <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_edgeconv_backward_lrelu: N*F exceeds int32");
+    const int fs = block > 0 ? ec_blocked_fs(block) : 0;
+    if (fs == 0 || n_src != N || (size_t)block * fs * sizeof(float) > 64 * 1024)
+        return edgeconv_backward_run(N, n_src, F, argmax, grad_out, out, out_slope, grad_src, grad_dst, stream);
+    size_t need = fgnn_edgeconv_backward_blocked_workspace_bytes(N, F);
+    FGNN_REQUIRE(N == 0 || (workspace && workspace_bytes >= need), FGNN_ERR_WORKSPACE, "fgnn_edgeconv_backward_lrelu: workspace %zu < %zu bytes",
+                 workspace_bytes, need);
+    if (N == 0) return 0;
+    return edgeconv_backward_blocked_run(N, F, block, fs, argmax, grad_out, grad_src, (int *)workspace, (hipStream_t)stream, out, out_slope, grad_dst);
 }

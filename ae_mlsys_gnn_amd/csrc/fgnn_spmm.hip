@@ -11,6 +11,7 @@ struct SpmmP {
     const float *feat; float *out; float *part;
     int N, H, F, HF;
     int sum_h;      // != 0: out is [N,F], the sum over the H heads (GMMConv's .sum(1) fused into the store)
+    const float *bias; const float *res;     // with sum_h: out[i,:] += bias[:] (+ res[i,:]) in the same store (either may be NULL)
 };
 __host__ __device__ static inline int spmm_pw(int HF) { return (HF + 3) & ~3; }
 
@@ -54,6 +55,9 @@ __device__ __forceinline__ void spmm_store_row(const SpmmP &p, int row, const fg
         if ((FULL || lm.ok[r]) && lm.eoff[r] < p.F) {
             fg_vec<VEC> acc; acc.zero();
             for (int h = 0; h < p.H; ++h) { fg_vec<VEC> t; t.load(scr + h * p.F + lm.eoff[r]); acc.add(t); }
+            // the layer's epilogue (layers/gmmconv_layer.py:69-75 of the reference): residual, then bias
+            if (p.res) { fg_vec<VEC> t; t.load(p.res + (size_t)row * p.F + lm.eoff[r]); acc.add(t); }
+            if (p.bias) { fg_vec<VEC> t; t.load(p.bias + lm.eoff[r]); acc.add(t); }
             acc.store(p.out + (size_t)row * p.F + lm.eoff[r]);
         }
     }
@@ -311,6 +315,26 @@ extern "C" int fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F, const i
     WGauss wf{pseudo, mu, inv_sigma, gauss_out, dim};
     return spmm_launch("fgnn_gmm_forward", p, wf, 2 * K * dim, sched, fgnn_aligned16(node_feat) && fgnn_aligned16(out), workspace,
                        workspace_bytes, (hipStream_t)stream);
+}
+
+// fgnn_gmm_forward with sum_kernels == 1 and the rest of the layer's forward in the store: out[i,:] = sum_k sum_p ... +
+// residual[i,:] + bias[:].
+extern "C" int fgnn_gmm_forward_epilogue(int N, int64_t E, int K, int dim, int F, const int32_t *ptr, const int32_t *idx,
+                                         const int32_t *pos_map, const float *node_feat, const float *pseudo, const float *mu,
+                                         const float *inv_sigma, const float *bias, const float *residual, float *out, float *gauss_out,
+                                         const fgnn_schedule_t *sched, void *workspace, size_t workspace_bytes, void *stream)
+{
+    int rc = spmm_checks("fgnn_gmm_forward_epilogue", N, E, K, F, sched, ptr, idx);
+    if (rc) return rc;
+    FGNN_REQUIRE(dim >= 1 && dim <= 64 && K * dim <= 1024, FGNN_ERR_LIMIT, "fgnn_gmm_forward_epilogue: dim=%d K*dim=%d unsupported", dim, K * dim);
+    FGNN_REQUIRE(ptr && (idx || E == 0) && node_feat && (pseudo || E == 0) && mu && inv_sigma && out, FGNN_ERR_NULL,
+                 "fgnn_gmm_forward_epilogue: NULL argument");
+    SpmmP p{};
+    p.ptr = ptr; p.idx = idx; p.pos_map = pos_map; p.feat = node_feat; p.out = out; p.N = N; p.H = K; p.F = F; p.HF = K * F;
+    p.sum_h = 1; p.bias = bias; p.res = residual;
+    WGauss wf{pseudo, mu, inv_sigma, gauss_out, dim};
+    const bool aligned = fgnn_aligned16(node_feat) && fgnn_aligned16(out) && (!bias || fgnn_aligned16(bias)) && (!residual || fgnn_aligned16(residual));
+    return spmm_launch("fgnn_gmm_forward_epilogue", p, wf, 2 * K * dim, sched, aligned, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 // ------------------------------------------------------------------------------- GMM backward

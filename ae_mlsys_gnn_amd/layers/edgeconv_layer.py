@@ -24,8 +24,10 @@ class EdgeConv(nn.Module):
     def set_allow_zero_in_degree(self, set_value):
         self._allow_zero_in_degree = set_value
 
-    def forward(self, k, src_ind, feat, block=None):
-        """block: points per cloud when src_ind is a kNN graph of equally sized clouds (see fused_edgeconv_op)."""
+    def forward(self, k, src_ind, feat, block=None, negative_slope_out=None):
+        """block: points per cloud when src_ind is a kNN graph of equally sized clouds (see fused_edgeconv_op).
+        negative_slope_out: apply LeakyReLU with this slope to the result inside the operator (the activation that
+        follows every EdgeConv of the reference's DGCNN, script/train/train_edgeconv_our.py:56)."""
         # theta and phi read the same rows: one product with the stacked weights (its weight gradient
         # reduced over the points in chunks), split afterwards
         out_feat = self.theta.out_features
@@ -33,4 +35,4 @@ class EdgeConv(nn.Module):
         h_theta, h_phi = h[:, :out_feat], h[:, out_feat:]
         h_src = h_theta.contiguous()
         h_dst = h_phi - h_theta
-        return fused_edgeconv_op(k, src_ind, h_src, h_dst, block)
+        return fused_edgeconv_op(k, src_ind, h_src, h_dst, block, negative_slope_out)

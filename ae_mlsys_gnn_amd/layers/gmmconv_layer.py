@@ -62,14 +62,23 @@ class _GMMBase(nn.Module):
         pad = (-self._out_feats) % 4
         if pad:         # zero columns up to a multiple of 4: the operator then takes its 128-bit row layout
             node_feat = th.nn.functional.pad(node_feat, (0, pad))
+        # residual and bias (layers/gmmconv_layer.py:69-75 of the reference) go into the operator's store when the
+        # width needs no padding; otherwise they are added afterwards
+        fuse_tail = pad == 0 and (self.bias is not None or self.res_fc is not None)
+        tail = lambda: {"bias": self.bias, "residual": None if self.res_fc is None else self.res_fc(feat)} if fuse_tail else {}
         if pseudo_csc is not None or own_order:
             if own_order and pseudo_csc is None and th.is_grad_enabled() and (node_feat.requires_grad or pseudo.requires_grad):
                 raise ValueError("own_order without pseudo_csc is forward-only")
             two_orders = GmmConvFuseSumTwoOrders if (type(self)._op is GmmConvFuseSum or pseudo_csc is None) else GmmConvStashSumTwoOrders
             rst = two_orders(rowptr, colind, colptr, rowind, node_feat, pseudo.detach(), pseudo_csc, self.mu, self.inv_sigma,
-                             own_order=own_order)
+                             own_order=own_order, **tail())
+        elif type(self)._op is GmmConvFuseSum:
+            rst = GmmConvFuseSum(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, self.mu, self.inv_sigma, **tail())
         else:
             rst = type(self)._op(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, self.mu, self.inv_sigma)
+            fuse_tail = False
+        if fuse_tail:
+            return rst
         if pad:
             rst = rst[..., :self._out_feats]
         return self._finish(rst, feat)

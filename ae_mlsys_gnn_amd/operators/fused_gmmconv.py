@@ -19,8 +19,10 @@ class gmm_native:
     """gmmconv.gmmconv / gmmconvstash / Gaussian / GaussianBp (src/fused_gmmconv/gmmconv.cc:36-94)."""
 
     @staticmethod
-    def gmmconv(rowptr, colind, node_feat, pseudo, mu, sigma, *, pos_map=None, want_gauss=False, sum_kernels=False, own_order=False):
-        require_cuda(rowptr, colind, node_feat, pseudo, mu, sigma)
+    def gmmconv(rowptr, colind, node_feat, pseudo, mu, sigma, *, pos_map=None, want_gauss=False, sum_kernels=False, own_order=False,
+                bias=None, residual=None):
+        """bias [F] / residual [N,F] (with sum_kernels only): added to the summed output inside the operator's store."""
+        require_cuda(rowptr, colind, node_feat, pseudo, mu, sigma, bias, residual)
         rowptr, colind = as_i32(rowptr), as_i32(colind)
         node_feat, pseudo, mu, sigma = as_f32(node_feat), as_f32(pseudo), as_f32(mu), as_f32(sigma)
         if node_feat.dim() != 3:
@@ -35,11 +37,24 @@ class gmm_native:
         gauss = torch.empty((e, k), dtype=torch.float32, device=node_feat.device) if want_gauss else None
         # own_order: pseudo (and gauss) are indexed by the schedule's entry order, pseudo_caller[edge_positions(rowptr, colind)]
         sched = schedule_for(rowptr, idx_tensor=colind, own_order=own_order)
+        epilogue = bias is not None or residual is not None
+        if epilogue:
+            if not sum_kernels:
+                raise FgnnError("gmmconv: bias / residual are added to the sum over the kernels (sum_kernels=True)")
+            bias = None if bias is None else as_f32(bias)
+            residual = None if residual is None else as_f32(residual)
+            if (bias is not None and tuple(bias.shape) != (f,)) or (residual is not None and tuple(residual.shape) != (n, f)):
+                raise FgnnError("gmmconv: bias must be [%d] and residual [%d, %d]" % (f, n, f))
         with torch.cuda.device(node_feat.device):
             ws, wsb = workspace(lib().fgnn_gmm_forward_workspace_bytes(sched.handle, k, f), node_feat.device)
-            check(lib().fgnn_gmm_forward(n, e, k, dim, f, ptr(rowptr), ptr(colind), ptr(pos_map), ptr(node_feat), ptr(pseudo),
-                                         ptr(mu), ptr(sigma), ptr(out), ptr(gauss), int(sum_kernels), sched.handle, ptr(ws), wsb, stream_ptr()),
-                  "fgnn_gmm_forward")
+            if epilogue:
+                check(lib().fgnn_gmm_forward_epilogue(n, e, k, dim, f, ptr(rowptr), ptr(colind), ptr(pos_map), ptr(node_feat), ptr(pseudo),
+                                                      ptr(mu), ptr(sigma), ptr(bias), ptr(residual), ptr(out), ptr(gauss), sched.handle,
+                                                      ptr(ws), wsb, stream_ptr()), "fgnn_gmm_forward_epilogue")
+            else:
+                check(lib().fgnn_gmm_forward(n, e, k, dim, f, ptr(rowptr), ptr(colind), ptr(pos_map), ptr(node_feat), ptr(pseudo),
+                                             ptr(mu), ptr(sigma), ptr(out), ptr(gauss), int(sum_kernels), sched.handle, ptr(ws), wsb, stream_ptr()),
+                      "fgnn_gmm_forward")
         return (out, gauss) if want_gauss else out
 
     @staticmethod
@@ -161,6 +176,14 @@ class gmm_native:
         return gp, gm, gs
 
 
+def _epilogue_grads(ctx, grad_out, first):
+    """Gradients of the optional (bias, residual) inputs at positions first, first + 1 of a Function's inputs."""
+    from ..layers.dense import column_sum
+    gb = column_sum(grad_out) if (ctx.has_bias and ctx.needs_input_grad[first]) else None
+    gr = grad_out if (ctx.has_res and ctx.needs_input_grad[first + 1]) else None
+    return gb, gr
+
+
 def GmmConvFuse(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma):
     return GmmFuseFunction.apply(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma)
 
@@ -180,13 +203,16 @@ class GmmFuseFunction(torch.autograd.Function):
         return None, None, None, None, None, grad_feat, grad_pseudo, grad_mu, grad_sigma
 
 
-def GmmConvFuseSum(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma):
+def GmmConvFuseSum(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma, bias=None, residual=None):
     """GmmConvFuse(...).sum(1) as one operator: the sum over the K mixture kernels is fused into the
-    forward's store and the backward gathers [N,F] gradient rows.  Returns [N,F]."""
-    return GmmFuseSumFunction.apply(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma)
+    forward's store and the backward gathers [N,F] gradient rows.  Returns [N,F].
+    bias [F], residual [N,F] (optional): the rest of the layer's forward (layers/gmmconv_layer.py:69-75), added in
+    the same store."""
+    return GmmFuseSumFunction.apply(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma, bias, residual)
 
 
-def GmmConvFuseSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order=False):
+def GmmConvFuseSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order=False, bias=None,
+                            residual=None):
     """GmmConvFuseSum for a caller that has the pseudo-coordinates in both edge orders
     (pseudo_csc == pseudo_csr[permute], e.g. the same elementwise projection applied to constant
     edge data stored both ways).  The forward reads pseudo_csr, the backward reads pseudo_csc and
@@ -196,26 +222,29 @@ def GmmConvFuseSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo_cs
     pseudo_csr[gmm_edge_positions(rowptr, colind)] and pseudo_csc[gmm_edge_positions(colptr, rowind, True)]:
     every pass then streams its per-edge data."""
     if pseudo_csc is None:
-        return gmm_native.gmmconv(rowptr, colind, node_feat, pseudo_csr, mu, sigma, sum_kernels=True, own_order=own_order)
-    return GmmFuseSumTwoOrdersFunction.apply(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order)
+        return gmm_native.gmmconv(rowptr, colind, node_feat, pseudo_csr, mu, sigma, sum_kernels=True, own_order=own_order, bias=bias,
+                                  residual=residual)
+    return GmmFuseSumTwoOrdersFunction.apply(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order, bias, residual)
 
 
-def GmmConvStashSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order=False):
+def GmmConvStashSumTwoOrders(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order=False, bias=None,
+                             residual=None):
     """The stash variant with the pseudo-coordinates in both edge orders: as GmmConvFuseSumTwoOrders, and the
     forward also writes the Gaussian weights [E,K] (in the order of pseudo_csr) and keeps them until the
     backward, the memory cost of the reference's stash variant (operators/fused_gmmconv.py:100-118).  The
     backward is the same single pass: recomputing a weight is cheaper than reading it back through a
     transposition."""
-    return GmmStashSumTwoOrdersFunction.apply(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order)
+    return GmmStashSumTwoOrdersFunction.apply(rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order, bias, residual)
 
 
 class GmmStashSumTwoOrdersFunction(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order):
+    def forward(ctx, rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order, bias=None, residual=None):
         out, gauss = gmm_native.gmmconv(rowptr, colind, node_feat, pseudo_csr, mu, sigma, want_gauss=True, sum_kernels=True,
-                                        own_order=own_order)
+                                        own_order=own_order, bias=bias, residual=residual)
         ctx.save_for_backward(colptr, rowind, node_feat, pseudo_csc, mu, sigma, gauss)
         ctx.own_order = own_order
+        ctx.has_bias, ctx.has_res = bias is not None, residual is not None
         return out
 
     @staticmethod
@@ -223,7 +252,7 @@ class GmmStashSumTwoOrdersFunction(torch.autograd.Function):
         colptr, rowind, node_feat, pseudo_csc, mu, sigma, _gauss = ctx.saved_tensors
         grad_feat, grad_pseudo_csc, grad_mu, grad_sigma = gmm_native.gmmconv_backward(
             colptr, rowind, None, node_feat, pseudo_csc, mu, sigma, grad_out.contiguous(), sum_kernels=True, own_order=ctx.own_order)
-        return None, None, None, None, grad_feat, None, grad_pseudo_csc, grad_mu, grad_sigma, None
+        return (None, None, None, None, grad_feat, None, grad_pseudo_csc, grad_mu, grad_sigma, None) + _epilogue_grads(ctx, grad_out.contiguous(), 10)
 
 
 def gmm_edge_positions(ptr_arr, idx, summed_backward=False):
@@ -241,10 +270,12 @@ def gmm_edge_positions(ptr_arr, idx, summed_backward=False):
 
 class GmmFuseSumTwoOrdersFunction(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order):
-        out = gmm_native.gmmconv(rowptr, colind, node_feat, pseudo_csr, mu, sigma, sum_kernels=True, own_order=own_order)      # [N, F]
+    def forward(ctx, rowptr, colind, colptr, rowind, node_feat, pseudo_csr, pseudo_csc, mu, sigma, own_order, bias=None, residual=None):
+        out = gmm_native.gmmconv(rowptr, colind, node_feat, pseudo_csr, mu, sigma, sum_kernels=True, own_order=own_order, bias=bias,
+                                 residual=residual)      # [N, F]
         ctx.save_for_backward(colptr, rowind, node_feat, pseudo_csc, mu, sigma)
         ctx.own_order = own_order
+        ctx.has_bias, ctx.has_res = bias is not None, residual is not None
         return out
 
     @staticmethod
@@ -252,7 +283,7 @@ class GmmFuseSumTwoOrdersFunction(torch.autograd.Function):
         colptr, rowind, node_feat, pseudo_csc, mu, sigma = ctx.saved_tensors
         grad_feat, grad_pseudo_csc, grad_mu, grad_sigma = gmm_native.gmmconv_backward(
             colptr, rowind, None, node_feat, pseudo_csc, mu, sigma, grad_out.contiguous(), sum_kernels=True, own_order=ctx.own_order)
-        return None, None, None, None, grad_feat, None, grad_pseudo_csc, grad_mu, grad_sigma, None
+        return (None, None, None, None, grad_feat, None, grad_pseudo_csc, grad_mu, grad_sigma, None) + _epilogue_grads(ctx, grad_out.contiguous(), 10)
 
 
 def GmmAggregate(rowptr, colind, colptr, rowind, permute, feat, pseudo, mu, sigma):
@@ -304,9 +335,10 @@ class GmmAggregateTwoOrdersFunction(torch.autograd.Function):
 
 class GmmFuseSumFunction(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma):
-        out = gmm_native.gmmconv(rowptr, colind, node_feat, pseudo, mu, sigma, sum_kernels=True)      # [N, F]
+    def forward(ctx, rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma, bias=None, residual=None):
+        out = gmm_native.gmmconv(rowptr, colind, node_feat, pseudo, mu, sigma, sum_kernels=True, bias=bias, residual=residual)      # [N, F]
         ctx.save_for_backward(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma)
+        ctx.has_bias, ctx.has_res = bias is not None, residual is not None
         return out
 
     @staticmethod
@@ -314,7 +346,7 @@ class GmmFuseSumFunction(torch.autograd.Function):
         rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma = ctx.saved_tensors
         grad_feat, grad_pseudo, grad_mu, grad_sigma = gmm_native.gmmconv_backward(
             colptr, rowind, permute, node_feat, pseudo, mu, sigma, grad_out.contiguous(), sum_kernels=True)
-        return None, None, None, None, None, grad_feat, grad_pseudo, grad_mu, grad_sigma
+        return (None, None, None, None, None, grad_feat, grad_pseudo, grad_mu, grad_sigma) + _epilogue_grads(ctx, grad_out.contiguous(), 9)
 
 
 def GmmConvFuseEb(rowptr, colind, colptr, rowind, permute, node_feat, pseudo, mu, sigma):

@@ -45,7 +45,7 @@ class Model(nn.Module):
         h, hs = x, []
         for conv in self.conv:
             src = self.knn(h.detach(), self.k)
-            h = F.leaky_relu(conv(self.k, src, h.reshape(b * p, -1), block=p), 0.2).view(b, p, -1)
+            h = conv(self.k, src, h.reshape(b * p, -1), block=p, negative_slope_out=0.2).view(b, p, -1)     # LeakyReLU(0.2) fused in
             hs.append(h)
         h = tall_linear(torch.cat(hs, 2).view(b * p, -1), self.proj.weight, self.proj.bias).view(b, p, -1)
         h = torch.cat([h.max(1).values, h.mean(1)], 1)

@@ -166,6 +166,18 @@ int fgnn_edgeconv_forward(int N, int n_src, int F, int k, const int32_t *src_ind
 int fgnn_edgeconv_backward(int N, int n_src, int F, const int32_t *argmax, const float *grad_out,
                            float *grad_src, void *stream);
 
+/* EdgeConv with the LeakyReLU that follows every EdgeConv of the reference's DGCNN stack
+ * (script/train/train_edgeconv_our.py:56, `h = F.leaky_relu(h, 0.2)`) fused in: the forward stores
+ * lrelu(max, out_slope); the backward replays the mask from that output (out > 0 <=> pre-activation > 0 for
+ * out_slope > 0, which is required) while it scatters, and writes the masked gradient -- the gradient of h_dst --
+ * to grad_dst.  block > 0 selects the blocked form (workspace of fgnn_edgeconv_backward_blocked_workspace_bytes),
+ * block <= 0 the plain scatter (workspace unused). */
+int fgnn_edgeconv_forward_lrelu(int N, int n_src, int F, int k, const int32_t *src_ind, const float *h_src,
+                                const float *h_dst, float out_slope, float *out, int32_t *argmax, void *stream);
+int fgnn_edgeconv_backward_lrelu(int N, int n_src, int F, int block, const int32_t *argmax, const float *out,
+                                 float out_slope, const float *grad_out, float *grad_src, float *grad_dst,
+                                 void *workspace, size_t workspace_bytes, void *stream);
+
 /* The same backward for batched point clouds.  `block` is a hint that the neighbours of destination
  * rows [b*block, (b+1)*block) lie in source rows of the same range, as in a kNN graph of clouds of
  * `block` points (fgnn_knn_graph): those contributions are accumulated in LDS and written with plain
@@ -217,6 +229,17 @@ int    fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F,
                         const float *inv_sigma, float *out, float *gauss_out, int sum_kernels,
                         const fgnn_schedule_t *sched, void *workspace, size_t workspace_bytes,
                         void *stream);
+
+/* fgnn_gmm_forward with sum_kernels == 1 and the layer's epilogue (layers/gmmconv_layer.py:69-75: `rst = rst +
+ * res_fc(feat)`, `rst = rst + bias`) in the same store: out[i,:] = sum_k out[i,k,:] + residual[i,:] + bias[:], bias [F]
+ * and residual [N,F] optional (NULL).  Their gradients are the gradient of out (summed over the nodes for the
+ * bias), so fgnn_gmm_backward serves unchanged. */
+int    fgnn_gmm_forward_epilogue(int N, int64_t E, int K, int dim, int F,
+                                 const int32_t *ptr, const int32_t *idx, const int32_t *pos_map,
+                                 const float *node_feat, const float *pseudo, const float *mu,
+                                 const float *inv_sigma, const float *bias, const float *residual,
+                                 float *out, float *gauss_out, const fgnn_schedule_t *sched,
+                                 void *workspace, size_t workspace_bytes, void *stream);
 
 /* Replaces the backward sequence of operators/fused_gmmconv.py:51-58 (mhsddmm + mhtranspose +
  * gmmconv over CSC + GaussianBp, gmmconv.cu:265-285) with one pass over the CSC arrays:

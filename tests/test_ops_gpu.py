@@ -865,3 +865,91 @@ def test_edge_linear_tanh_limits():
     assert _lib.lib().fgnn_edge_linear_tanh(4, 5, None, None, None, None, None) == -4
     y = edge_proj.edge_linear_tanh(torch.rand(0, 2, device=DEV), torch.rand(2, 2, device=DEV), torch.rand(2, device=DEV))
     assert y.shape == (0, 2)
+
+
+@pytest.mark.parametrize("b,p,k,fin,f,block,slope", [(3, 128, 10, 3, 64, 128, 0.2), (2, 100, 7, 5, 20, None, 0.2), (2, 256, 20, 3, 130, 256, 0.01),
+                                                       (4, 64, 5, 8, 8, 32, 1.0)])
+def test_edgeconv_with_fused_leaky_relu(b, p, k, fin, f, block, slope):
+    """EdgeConv(..., negative_slope_out=s) == LeakyReLU(s)(EdgeConv(...)) (script/train/train_edgeconv_our.py:56):
+    outputs bit-identical to the unfused pair on the GPU and equal to the float64 oracle's; gradients of theta and
+    phi against autograd through the oracle (plain and blocked backward, the mask replayed from the output)."""
+    from ae_mlsys_gnn_amd.layers import EdgeConv
+    torch.manual_seed(b * p + f)
+    pts = torch.rand(b, p, 3) * 2 - 1
+    src = graphs.knn_graph(pts, k)
+    x = torch.randn(b * p, fin)
+    layer = EdgeConv(fin, f)
+    th = layer.theta.weight.detach().double().requires_grad_(True)
+    ph = layer.phi.weight.detach().double().requires_grad_(True)
+    xd = x.double().requires_grad_(True)
+    h_src = xd @ th.t()
+    h_dst = xd @ ph.t() - h_src
+    ref = torch.nn.functional.leaky_relu(orc.edgeconv_forward_autograd(k, src, h_src, h_dst), slope)
+    go = torch.randn(ref.shape, dtype=torch.float64)
+    ref.backward(go)
+    layer = layer.to(DEV)
+    xg = x.to(DEV).requires_grad_(True)
+    out = layer(k, src.to(DEV), xg, block=block, negative_slope_out=slope)
+    out.backward(go.float().to(DEV))
+    unfused = torch.nn.functional.leaky_relu(layer(k, src.to(DEV), x.to(DEV), block=block), slope)
+    assert torch.equal(out.detach(), unfused.detach()), "fused activation is not bit-identical to the unfused pair"
+    assert_close(out, ref.detach(), "edgeconv + lrelu out")
+    # scales of the weight / input gradients: sums over points (and scattered neighbours) of |masked gradient| |x|
+    _, arg = orc.edgeconv_forward(k, src, h_src.detach(), h_dst.detach())
+    gm = (go * torch.where(ref.detach() > 0, 1.0, slope)).abs()
+    gsrc_abs = orc.edgeconv_backward(arg, gm, xd.shape[0])[0]
+    assert_close_sum(layer.theta.weight.grad, th.grad, (gsrc_abs + gm).t() @ xd.detach().abs(), "theta grad")
+    assert_close_sum(layer.phi.weight.grad, ph.grad, gm.t() @ xd.detach().abs(), "phi grad")
+    assert_close_sum(xg.grad, xd.grad, (gsrc_abs + gm) @ th.detach().abs() + gm @ ph.detach().abs(), "input grad")
+    from ae_mlsys_gnn_amd._lib import FgnnError
+    with pytest.raises(FgnnError, match="positive"):
+        layer(k, src.to(DEV), x.to(DEV), negative_slope_out=0.0)
+
+
+@pytest.mark.parametrize("k,dim,f,with_bias,with_res", [(3, 2, 64, True, True), (2, 1, 16, True, False), (4, 2, 32, False, True), (2, 2, 256, True, True),
+                                                         (3, 1, 44, True, True)])
+def test_gmm_sum_with_bias_and_residual_in_the_store(k, dim, f, with_bias, with_res, monkeypatch):
+    """GmmConvFuseSum(..., bias, residual): the rest of the layer's forward (layers/gmmconv_layer.py:69-75 of the
+    reference) added inside the operator's store, whole rows and merged split rows, plain and XCD-aware work lists;
+    output and every gradient (bias and residual included) against the float64 oracle."""
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd.operators import fused_gmmconv as fg
+    g = graphs.add_csc_torch(degree_edge_graph(n=400, seed=k + f))
+    x, pseudo, mu, isg, go = _gmm_case(g, k, dim, f, seed=3)
+    go = go[:, 0, :].contiguous()
+    gen = torch.Generator().manual_seed(9)
+    bias = torch.randn(f, generator=gen, dtype=torch.float64) if with_bias else None
+    res = torch.randn(g.n, f, generator=gen, dtype=torch.float64) if with_res else None
+    leaves = [t.clone().requires_grad_(True) for t in (x, pseudo, mu, isg)]
+    bl = None if bias is None else bias.clone().requires_grad_(True)
+    rl = None if res is None else res.clone().requires_grad_(True)
+    ref = orc.gmm_forward(g.row_ptr, g.col_ind, *leaves).sum(1)
+    if rl is not None:
+        ref = ref + rl
+    if bl is not None:
+        ref = ref + bl
+    ref.backward(go)
+    gd = g.to(DEV)
+    for buckets in ("0", "1"):
+        monkeypatch.setenv("FGNN_SEG_LEN", "256")
+        monkeypatch.setenv("FGNN_XCD_BUCKETS", buckets)
+        monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+        _lib.clear_schedule_cache()
+        dl = [t.float().to(DEV).requires_grad_(True) for t in (x, pseudo, mu, isg)]
+        bd = None if bias is None else bias.float().to(DEV).requires_grad_(True)
+        rd = None if res is None else res.float().to(DEV).requires_grad_(True)
+        out = fg.GmmConvFuseSum(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, *dl, bias=bd, residual=rd)
+        out.backward(go.float().to(DEV))
+        s = orc.gmm_abs_sums(g.row_ptr, g.col_ind, x, pseudo, mu, isg, go.unsqueeze(1).expand(-1, k, -1))
+        s_out = s["out"].sum(1) + (0 if res is None else res.abs()) + (0 if bias is None else bias.abs())
+        c = _gmm_c(pseudo, mu, isg)
+        assert_close_sum(out, ref.detach(), s_out, "out with epilogue (buckets %s)" % buckets, c=c)
+        for val, want, key in zip((t.grad for t in dl), (t.grad for t in leaves), ("grad_feat", "grad_pseudo", "grad_mu", "grad_sigma")):
+            assert_close_sum(val, want, s[key], key + " with epilogue", c=c)
+        if bd is not None:
+            assert_close_sum(bd.grad, bl.grad, go.abs().sum(0), "grad bias")
+        if rd is not None:
+            assert torch.equal(rd.grad.cpu(), go.float())
+    _lib.clear_schedule_cache()
+    with pytest.raises(_lib.FgnnError, match="sum over the kernels"):
+        fg.gmm_native.gmmconv(gd.row_ptr, gd.col_ind, dl[0].detach(), dl[1].detach(), dl[2].detach(), dl[3].detach(), bias=torch.zeros(f, device=DEV))

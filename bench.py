@@ -315,7 +315,9 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
         "roofline_bwd": roofline_record("gat_bwd_node_kernel + gat_bwd_kernel (+gat_bwd_merge_kernel)", b_bwd, ms_bwd,
                                         (traffic or {}).get("bwd"), stale),
         "stash_variant": {"fwd_ms": round(ms_sf, 4), "stash_writer_ms": round(ms_sw, 4), "bwd_ms": round(ms_sb, 4),
-                          "stashed_GiB": round(stash_bytes / 2**30, 3)},
+                          "stashed_GiB": round(stash_bytes / 2**30, 3),
+                          "roofline_bwd": roofline_record("gat_bwd_node_kernel + gat_bwd_kernel<own-order stash> (+merge)", b_bwd + stash_bytes, ms_sb,
+                                                          (traffic or {}).get("stash_bwd"), stale)},
         "sparse_fwd_bwd": {"ms": round(ms_fwd + ms_bwd, 4), "alg_bytes": b_fwd + b_bwd,
                            "achieved_GBps": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6, 1),
                            "frac_of_peak": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6 / HBM_PEAK_GBPS, 4)},

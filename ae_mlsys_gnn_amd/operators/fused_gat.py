@@ -198,5 +198,19 @@ class FusedGATFunction_stash(torch.autograd.Function):
 
 
 class FusedGATFunction(FusedGATFunction_stash):
-    """Fuse-scatter variant of the reference (edge softmax stashed, separate SpMM).  Here the
-    stashed tensors come out of the same fused forward, so it shares the stash implementation."""
+    """Fuse-scatter variant as ONE fused operator: it shares the stash implementation (same math, same
+    stashed tensor).  The reference's own fuse-scatter data flow -- a softmax kernel that materialises
+    [E,H], then a separate SpMM; backward by permuted SpMM, SDDMM and row / column sums
+    (src/fused_gat/fused_gat.cu:235-326, 641-670) -- is `fused_gat_fusescatter_pipeline` below."""
+
+
+def fused_gat_fusescatter_pipeline(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute):
+    """The fuse-scatter ablation of the reference as a pipeline of this package's small operators, each with
+    its own autograd function: u_add_v -> LeakyReLU -> edge softmax ([E,H] materialised twice) -> multi-head
+    SpMM; the backward runs the permuted SpMM over the CSC arrays, the SDDMM, the softmax backward and the
+    row / column sums of u_add_v.  Same results as the fused operators; several passes over [E,H] more."""
+    from .edge_softmax import csr_edge_softmax
+    from .mhspmm import csrmhspmm
+    from .u_add_v import u_add_v_op
+    e = torch.nn.functional.leaky_relu(u_add_v_op(row_ptr, col_ind, attn_row, attn_col), negative_slope)
+    return csrmhspmm(row_ptr, col_ind, col_ptr, row_ind, permute, in_feat, csr_edge_softmax(row_ptr, e))

@@ -296,6 +296,18 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
         max(3, args.steps // 4), 1)
     stash_bytes = e * heads * 4
     del own
+    # the reference's fuse-scatter data flow as a pipeline of the small operators (u_add_v, LeakyReLU, edge softmax with
+    # [E,H] materialised, multi-head SpMM; backward by permuted SpMM, SDDMM, softmax backward, row / column sums)
+    from ae_mlsys_gnn_amd.operators.fused_gat import fused_gat_fusescatter_pipeline
+    hp, arp, acp = (t.detach().clone().requires_grad_(True) for t in (h, a_row, a_col))
+
+    def pipeline_step():
+        fused_gat_fusescatter_pipeline(arp, acp, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, slope, hp, g.permute).backward(go)
+        hp.grad = None; arp.grad = None; acp.grad = None
+    torch.cuda.reset_peak_memory_stats()
+    ms_pipe, _, _ = time_calls(pipeline_step, max(3, args.steps // 4), 1)
+    pipe_peak = peak_hbm_gib()
+    del hp, arp, acp
     prep = time_device_preprocessing(g)
 
     if args.no_cpu_baseline:
@@ -318,6 +330,8 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
                           "stashed_GiB": round(stash_bytes / 2**30, 3),
                           "roofline_bwd": roofline_record("gat_bwd_node_kernel + gat_bwd_kernel<own-order stash> (+merge)", b_bwd + stash_bytes, ms_sb,
                                                           (traffic or {}).get("stash_bwd"), stale)},
+        "fusescatter_pipeline": {"fwd_bwd_ms": round(ms_pipe, 4), "peak_hbm_GiB": round(pipe_peak, 3),
+                                 "what": "the reference's fuse-scatter ablation composed from u_add_v, edge softmax and mhspmm"},
         "sparse_fwd_bwd": {"ms": round(ms_fwd + ms_bwd, 4), "alg_bytes": b_fwd + b_bwd,
                            "achieved_GBps": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6, 1),
                            "frac_of_peak": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6 / HBM_PEAK_GBPS, 4)},
@@ -571,7 +585,7 @@ def run_gather_ceiling(args):
 
 def brief(rec):
     """The part of a workload's record that goes under "other_configs" of the default line."""
-    keep = ("metric", "value", "unit", "ms_per_step", "config", "roofline", "roofline_bwd", "variants", "stash_variant", "sparse_fwd_bwd",
+    keep = ("metric", "value", "unit", "ms_per_step", "config", "roofline", "roofline_bwd", "variants", "stash_variant", "fusescatter_pipeline", "sparse_fwd_bwd",
             "fused_sum_over_kernels", "hip_graph_replay", "knn_graph_ms", "backward_plain_scatter_us", "cpu_baseline", "peak_hbm_GiB")
     return {k: rec[k] for k in keep if k in rec}
 

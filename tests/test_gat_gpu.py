@@ -39,6 +39,8 @@ def _run(g, h, f, slope=0.2, seed=0, attn_scale=1.0, variant="sm", seg_len=None,
     acd = ac.float().to(dev).requires_grad_(True)
     if variant == "sm":
         out = fg.fused_gat_op(ard, acd, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, slope, xd)
+    elif variant == "pipeline":
+        out = fg.fused_gat_fusescatter_pipeline(ard, acd, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, slope, xd, gd.permute)
     elif variant == "stash":
         out = fg.fused_gat_stash_op(ard, acd, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, slope, xd, gd.permute)
     else:
@@ -450,4 +452,17 @@ def test_gat_stash_in_both_orders_through_native_calls(h, f, monkeypatch):
             b = torch.zeros(g.n, h, dtype=torch.float64).index_add_(0, seg, csc_alpha)
             assert_close(a, b, "column sums of |own-order stash|")
             assert not torch.allclose(own.cpu().double(), csc_signed)
+    _lib.clear_schedule_cache()
+
+
+@pytest.mark.parametrize("h,f", [(8, 32), (1, 47), (4, 16)])
+def test_fusescatter_pipeline_of_small_operators(h, f, monkeypatch):
+    """The reference's fuse-scatter data flow (softmax kernel -> [E,H] -> SpMM; backward by permuted SpMM, SDDMM,
+    softmax backward, row / column sums) composed from u_add_v, edge softmax and mhspmm: same results as the oracle."""
+    from ae_mlsys_gnn_amd import _lib
+    _run(degree_edge_graph(seed=61), h, f, variant="pipeline")
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
+    monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+    _lib.clear_schedule_cache()
+    _run(graphs.rmat_graph(1500, 90000, seed=62), h, f, variant="pipeline", slope=0.05)
     _lib.clear_schedule_cache()

@@ -1,56 +1,80 @@
 // The small per-edge operators of the reference's operators/ package: multi-head SDDMM,
 // permuted row gather (mhtranspose), edge softmax and u_add_v, each with its backward.
-// One wave per CSR row, lanes over (edge, head) or (edge, column) pairs.
+// None of them takes a work list, so each balances its own load: the element-wise ones cut the
+// [E, W] array into fixed chunks and find the rows of a chunk by bisection of row_ptr, the row
+// reductions give short rows to single waves and long rows to whole workgroups.
 #include "fgnn_common.h"
 
+// largest r in [lo, hi] with ptr[r] <= q
+__device__ __forceinline__ int so_row_of(const int *__restrict__ ptr, int lo, int hi, int q)
+{
+    while (lo < hi) {
+        int mid = (lo + hi + 1) >> 1;
+        if (ptr[mid] <= q) lo = mid; else hi = mid - 1;
+    }
+    return lo;
+}
+
 // out[p,h] = <a[row,h,:], b[col_ind[p],h,:]> (src/sddmm/mhsddmm.cu:5-81 of the reference, which
-// finds the row of each edge by binary search; here the row is the work item).
+// finds the row of each edge by binary search).  One wave per SDDMM_CHUNK consecutive CSR positions:
+// the row of the first one by bisection, the following rows by walking row_ptr, so a hub row is
+// shared by as many waves as it has chunks and the a-row is loaded once per (wave, row).
+#define SDDMM_CHUNK 256
 template <int VEC, int R, bool FULL, int LPH>
-__global__ __launch_bounds__(FGNN_TPB) void mhsddmm_kernel(int N, int H, int F, int HF, int lphp, const int *ptr, const int *idx,
+__global__ __launch_bounds__(FGNN_TPB) void mhsddmm_kernel(int N, int64_t E, int H, int F, int HF, int lphp, const int *ptr, const int *idx,
                                                            const float *a, const float *b, float *out)
 {
     extern __shared__ float lds[];
-    int row = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
-    if (row >= N) return;
+    const int64_t c0 = ((int64_t)blockIdx.x * FGNN_WPB + fg_wave()) * SDDMM_CHUNK;
+    if (c0 >= E) return;
+    const int c1 = fg_uni((int)min(c0 + SDDMM_CHUNK, E));
     const int lane = fg_lane();
     float *scr = lds + fg_wave() * (64 * R);
-    const int pb = fg_uni(ptr[row]), pe = fg_uni(ptr[row + 1]);
     fg_lanemap<VEC, R> lm;
     if (lphp) lm.init_padded(lane, H, F, lphp); else lm.init(lane, HF, F);      // lphp: head-aligned lanes for DPP sums
-    fg_vec<VEC> ar[R];
+    int row = fg_uni(so_row_of(ptr, 0, N - 1, (int)c0));     // ptr[row] <= c0 < ptr[row + 1]
+    int pb = fg_uni((int)c0);
+    while (pb < c1 && row < N) {                             // ptr[N] = E >= c1 keeps row < N on a consistent graph
+        const int pe = min(fg_uni(ptr[row + 1]), c1);
+        if (pe > pb) {
+            fg_vec<VEC> ar[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ar[r].load(a + (size_t)row * HF + lm.eoff[r]); else ar[r].zero(); }
-    for (int c = pb; c < pe; c += 64) {
-        int q = c + lane;
-        int cnt = min(64, pe - c);
-        int id = idx[q < pe ? q : c];
-        for (int t = 0; t < cnt; t += 4) {
-            fg_vec<VEC> ld[4][R];
+            for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ar[r].load(a + (size_t)row * HF + lm.eoff[r]); else ar[r].zero(); }
+            for (int c = pb; c < pe; c += 64) {
+                int q = c + lane;
+                int cnt = min(64, pe - c);
+                int id = idx[q < pe ? q : c];
+                for (int t = 0; t < cnt; t += 4) {
+                    fg_vec<VEC> ld[4][R];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                int j = __builtin_amdgcn_readlane(id, t + u);
+                    for (int u = 0; u < 4; ++u) {
+                        int j = __builtin_amdgcn_readlane(id, (t + u) & 63);
 #pragma unroll
-                for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ld[u][r].load(b + (size_t)j * HF + lm.eoff[r]); else ld[u][r].zero(); }
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                if (t + u >= cnt) break;
-                float d[R];
-#pragma unroll
-                for (int r = 0; r < R; ++r) d[r] = ld[u][r].dot(ar[r]);
-                size_t o = (size_t)(c + t + u) * H;
-                if constexpr (LPH > 0) {
-#pragma unroll
-                    for (int r = 0; r < R; ++r) {
-                        float s = fg_group_sum<LPH>(d[r]);
-                        if ((FULL || lm.ok[r]) && lm.eoff[r] % F == 0) out[o + lm.hd[r]] = s;
+                        for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ld[u][r].load(b + (size_t)j * HF + lm.eoff[r]); else ld[u][r].zero(); }
                     }
-                } else {
-                    float s = H <= FGNN_FEW_HEADS ? fg_head_reduce_few<VEC, R>(d, lm, lane, H) : fg_head_reduce<VEC, R>(scr, d, lm, lane, H, F);
-                    if (lane < H) out[o + lane] = s;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        if (t + u >= cnt) break;
+                        float d[R];
+#pragma unroll
+                        for (int r = 0; r < R; ++r) d[r] = ld[u][r].dot(ar[r]);
+                        size_t o = (size_t)(c + t + u) * H;
+                        if constexpr (LPH > 0) {
+#pragma unroll
+                            for (int r = 0; r < R; ++r) {
+                                float s = fg_group_sum<LPH>(d[r]);
+                                if ((FULL || lm.ok[r]) && lm.eoff[r] % F == 0) out[o + lm.hd[r]] = s;
+                            }
+                        } else {
+                            float s = H <= FGNN_FEW_HEADS ? fg_head_reduce_few<VEC, R>(d, lm, lane, H) : fg_head_reduce<VEC, R>(scr, d, lm, lane, H, F);
+                            if (lane < H) out[o + lane] = s;
+                        }
+                    }
                 }
             }
         }
+        pb = pe;
+        ++row;
     }
 }
 
@@ -67,12 +91,14 @@ extern "C" int fgnn_mhsddmm(int N, int64_t E, int H, int F, const int32_t *row_p
     const int lphp = fgnn_pad_lph(cfg.vec, H, F);
     if (lphp) { int w = H * lphp * 4; cfg.r = w <= 256 ? 1 : w <= 512 ? 2 : 4; cfg.full = false; }
     const int lph = lphp ? lphp : fgnn_pick_lph(cfg.vec, F);
-    const unsigned grid = (unsigned)((N + FGNN_WPB - 1) / FGNN_WPB);
+    FGNN_REQUIRE(E <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_mhsddmm: E=%lld exceeds the 32-bit row_ptr", (long long)E);
+    const int64_t waves = (E + SDDMM_CHUNK - 1) / SDDMM_CHUNK;
+    const unsigned grid = (unsigned)((waves + FGNN_WPB - 1) / FGNN_WPB);
     hipStream_t st = (hipStream_t)stream;
     return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
         return fgnn_dispatch_lph(VEC == 4 ? lph : 0, [&]<int LPH>() -> int {
             hipLaunchKernelGGL((mhsddmm_kernel<VEC, R, FULL, (VEC == 4 ? LPH : 0)>), dim3(grid), dim3(FGNN_TPB),
-                               (size_t)FGNN_WPB * 64 * R * sizeof(float), st, N, H, F, HF, lphp, row_ptr, col_ind, a, b, out);
+                               (size_t)FGNN_WPB * 64 * R * sizeof(float), st, N, E, H, F, HF, lphp, row_ptr, col_ind, a, b, out);
             return fgnn_launch_status("mhsddmm_kernel");
         });
     });
@@ -174,9 +200,113 @@ extern "C" int fgnn_gather_rows(int64_t E, int W, const int32_t *permute, const 
     return fgnn_launch_status("gather_rows_kernel");
 }
 
+// ------------------------------------------------------------------- row reductions over [E, W] arrays, W <= 64
+// A row's entries are one contiguous run of (pe - pb) * W floats.  Lanes t < S0 = (64 / W) * W of a
+// wave take part and stride by a multiple of W, so lane t only ever sees column t % W and every
+// load is a contiguous run of S0 floats.  Rows of up to SO_LONG_ELEMS floats are taken by one wave
+// each (first launch), longer ones by a whole workgroup each (second launch, whose other
+// workgroups leave at once): a 100 k-entry hub row is then a few hundred trips of 512 threads
+// instead of tens of thousands of trips of one wave.
+#define SO_LONG_ELEMS 2048
+#define SO_LONG_TPB 512
+
+struct so_max { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
+struct so_add { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
+
+// Combines the values of the lanes t, t + W, t + 2W, ... < S0 (any count, by suffix doubling) and of
+// the workgroup's waves (LONG) in a fixed order; every lane gets the result of its column.
+template <bool LONG, class Op>
+__device__ __forceinline__ float so_column_reduce(float v, int lane, int W, int S0, float (*sh)[64], Op op)
+{
+    for (int off = W; off < S0; off <<= 1) {
+        const float o = __shfl(v, (lane + off) & 63);
+        if (lane + off < S0) v = op(v, o);
+    }
+    v = __shfl(v, lane % W);
+    if constexpr (LONG) {
+        const int w = fg_wave();
+        if (lane < W) sh[w][lane] = v;
+        __syncthreads();
+        float r = sh[0][lane % W];
+        for (int i = 1; i < SO_LONG_TPB / 64; ++i) r = op(r, sh[i][lane % W]);
+        __syncthreads();
+        v = r;
+    }
+    return v;
+}
+
+// The row of this wave (short rows) or workgroup (LONG); false when it belongs to the other launch.
+template <bool LONG>
+__device__ __forceinline__ bool so_take_row(int N, int W, const int *ptr, int &row, int &pb, int64_t &n)
+{
+    row = LONG ? (int)blockIdx.x : fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (row >= N) return false;
+    pb = fg_uni(ptr[row]);
+    n = (int64_t)(fg_uni(ptr[row + 1]) - pb) * W;
+    return LONG ? n > SO_LONG_ELEMS : (n > 0 && n <= SO_LONG_ELEMS);
+}
+
 // Per-row, per-head softmax over [E,H] (src/edge_softmax/edge_softmax.cu:7-61) and its backward
-// s*(g - sum_row s*g) (:63-98).  Lanes stride over the row's edges, one head at a time.
-__global__ __launch_bounds__(FGNN_TPB) void edge_softmax_kernel(int N, int H, const int *ptr, const float *in, float *out)
+// s*(g - sum_row s*g) (:63-98).
+template <bool LONG>
+__global__ __launch_bounds__(LONG ? SO_LONG_TPB : FGNN_TPB) void edge_softmax_kernel(int N, int H, const int *__restrict__ ptr,
+                                                                                     const float *__restrict__ in, float *__restrict__ out)
+{
+    __shared__ float sh[LONG ? SO_LONG_TPB / 64 : 1][64];
+    int row, pb;
+    int64_t n;
+    if (!so_take_row<LONG>(N, H, ptr, row, pb, n)) return;          // uniform over the workgroup when LONG
+    const int lane = fg_lane(), S0 = (64 / H) * H;
+    const int64_t first = (LONG ? fg_wave() * S0 : 0) + lane, step = (int64_t)S0 * (LONG ? SO_LONG_TPB / 64 : 1);
+    const bool act = lane < S0;
+    const float *src = in + (size_t)pb * H;
+    float *dst = out + (size_t)pb * H;
+    float m = -INFINITY;
+    if (act) {
+#pragma unroll 4
+        for (int64_t k = first; k < n; k += step) m = fmaxf(m, src[k]);
+    }
+    m = so_column_reduce<LONG>(m, lane, H, S0, sh, so_max());
+    float s = 0.f;
+    if (act) {
+#pragma unroll 4
+        for (int64_t k = first; k < n; k += step) s += __expf(src[k] - m);
+    }
+    s = so_column_reduce<LONG>(s, lane, H, S0, sh, so_add());
+    const float inv = 1.f / s;
+    if (act) {
+#pragma unroll 4
+        for (int64_t k = first; k < n; k += step) dst[k] = __expf(src[k] - m) * inv;
+    }
+}
+
+template <bool LONG>
+__global__ __launch_bounds__(LONG ? SO_LONG_TPB : FGNN_TPB) void edge_softmax_bwd_kernel(int N, int H, const int *__restrict__ ptr,
+                                                                                         const float *__restrict__ sm, const float *__restrict__ g,
+                                                                                         float *__restrict__ gin)
+{
+    __shared__ float sh[LONG ? SO_LONG_TPB / 64 : 1][64];
+    int row, pb;
+    int64_t n;
+    if (!so_take_row<LONG>(N, H, ptr, row, pb, n)) return;
+    const int lane = fg_lane(), S0 = (64 / H) * H;
+    const int64_t first = (LONG ? fg_wave() * S0 : 0) + lane, step = (int64_t)S0 * (LONG ? SO_LONG_TPB / 64 : 1);
+    const bool act = lane < S0;
+    const size_t base = (size_t)pb * H;
+    float acc = 0.f;
+    if (act) {
+#pragma unroll 4
+        for (int64_t k = first; k < n; k += step) acc = fmaf(sm[base + k], g[base + k], acc);
+    }
+    acc = so_column_reduce<LONG>(acc, lane, H, S0, sh, so_add());
+    if (act) {
+#pragma unroll 4
+        for (int64_t k = first; k < n; k += step) gin[base + k] = sm[base + k] * (g[base + k] - acc);
+    }
+}
+
+// More than 64 heads: one wave per row, one head at a time.
+__global__ __launch_bounds__(FGNN_TPB) void edge_softmax_wide_kernel(int N, int H, const int *ptr, const float *in, float *out)
 {
     int row = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
     if (row >= N) return;
@@ -194,7 +324,7 @@ __global__ __launch_bounds__(FGNN_TPB) void edge_softmax_kernel(int N, int H, co
     }
 }
 
-__global__ __launch_bounds__(FGNN_TPB) void edge_softmax_bwd_kernel(int N, int H, const int *ptr, const float *sm, const float *g, float *gin)
+__global__ __launch_bounds__(FGNN_TPB) void edge_softmax_bwd_wide_kernel(int N, int H, const int *ptr, const float *sm, const float *g, float *gin)
 {
     int row = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
     if (row >= N) return;
@@ -216,8 +346,17 @@ extern "C" int fgnn_edge_softmax(int N, int64_t E, int H, const int32_t *row_ptr
     FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1, FGNN_ERR_SHAPE, "fgnn_edge_softmax: bad sizes");
     FGNN_REQUIRE(row_ptr && (E == 0 || (in && out)), FGNN_ERR_NULL, "fgnn_edge_softmax: NULL argument");
     if (N == 0 || E == 0) return 0;
-    hipLaunchKernelGGL(edge_softmax_kernel, dim3((unsigned)((N + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, (hipStream_t)stream, N, H, row_ptr, in, out);
-    return fgnn_launch_status("edge_softmax_kernel");
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned waves = (unsigned)((N + FGNN_WPB - 1) / FGNN_WPB);
+    if (H > 64) {
+        hipLaunchKernelGGL(edge_softmax_wide_kernel, dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, in, out);
+        return fgnn_launch_status("edge_softmax_wide_kernel");
+    }
+    hipLaunchKernelGGL(edge_softmax_kernel<false>, dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, in, out);
+    int rc = fgnn_launch_status("edge_softmax_kernel");
+    if (rc || E * H <= SO_LONG_ELEMS) return rc;                    // no row can be long
+    hipLaunchKernelGGL(edge_softmax_kernel<true>, dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, H, row_ptr, in, out);
+    return fgnn_launch_status("edge_softmax_kernel (long rows)");
 }
 
 extern "C" int fgnn_edge_softmax_backward(int N, int64_t E, int H, const int32_t *row_ptr, const float *sm, const float *grad_out,
@@ -226,13 +365,75 @@ extern "C" int fgnn_edge_softmax_backward(int N, int64_t E, int H, const int32_t
     FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1, FGNN_ERR_SHAPE, "fgnn_edge_softmax_backward: bad sizes");
     FGNN_REQUIRE(row_ptr && (E == 0 || (sm && grad_out && grad_in)), FGNN_ERR_NULL, "fgnn_edge_softmax_backward: NULL argument");
     if (N == 0 || E == 0) return 0;
-    hipLaunchKernelGGL(edge_softmax_bwd_kernel, dim3((unsigned)((N + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, (hipStream_t)stream, N, H, row_ptr, sm,
-                       grad_out, grad_in);
-    return fgnn_launch_status("edge_softmax_bwd_kernel");
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned waves = (unsigned)((N + FGNN_WPB - 1) / FGNN_WPB);
+    if (H > 64) {
+        hipLaunchKernelGGL(edge_softmax_bwd_wide_kernel, dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, sm, grad_out, grad_in);
+        return fgnn_launch_status("edge_softmax_bwd_wide_kernel");
+    }
+    hipLaunchKernelGGL(edge_softmax_bwd_kernel<false>, dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, sm, grad_out, grad_in);
+    int rc = fgnn_launch_status("edge_softmax_bwd_kernel");
+    if (rc || E * H <= SO_LONG_ELEMS) return rc;
+    hipLaunchKernelGGL(edge_softmax_bwd_kernel<true>, dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, H, row_ptr, sm, grad_out, grad_in);
+    return fgnn_launch_status("edge_softmax_bwd_kernel (long rows)");
 }
 
-// out[p,w] = row_val[row(p),w] + col_val[col_ind[p],w]  (src/u_add_v/u_add_v.cu:4-26)
-__global__ __launch_bounds__(FGNN_TPB) void u_add_v_kernel(int N, int W, const int *ptr, const int *idx, const float *rv, const float *cv, float *out)
+// out[p,w] = row_val[row(p),w] + col_val[col_ind[p],w]  (src/u_add_v/u_add_v.cu:4-26).  W <= 64: one thread per
+// element of out, a wave takes 2048 consecutive ones; the row of an edge is found by bisection of row_ptr, first
+// for the wave's first and last edge (wave-uniform), then per lane inside that usually one- or two-row window.
+#define UAV_CHUNKS 32           // 64-element chunks per wave
+#define UAV_UJ 4                // chunks in flight; divides UAV_CHUNKS
+__global__ __launch_bounds__(FGNN_TPB) void u_add_v_kernel(int N, int64_t E, int W, const int *__restrict__ ptr, const int *__restrict__ idx,
+                                                           const float *__restrict__ rv, const float *__restrict__ cv, float *__restrict__ out)
+{
+    const int64_t total = E * W;
+    const int64_t k0 = ((int64_t)blockIdx.x * FGNN_WPB + fg_wave()) * (64 * UAV_CHUNKS);
+    if (k0 >= total) return;
+    const int64_t k1 = min(k0 + 64 * UAV_CHUNKS, total);
+    const int lane = fg_lane();
+    const unsigned uw = (unsigned)W;
+    const unsigned inv_w = (65536u + uw - 1u) / uw;          // ceil(2^16 / W)
+    int qbase = fg_uni((int)(k0 / W));                       // edge of the wave's first element
+    unsigned rem = (unsigned)fg_uni((int)(k0 - (int64_t)qbase * W));
+    const int qlast = fg_uni((int)((k1 - 1) / W));
+    int rlo = fg_uni(so_row_of(ptr, 0, N - 1, qbase));
+    const int rhi = fg_uni(so_row_of(ptr, rlo, N - 1, qlast));
+    constexpr int UJ = UAV_UJ;
+    for (int64_t kk = k0; kk < k1; kk += 64 * UJ) {
+        int q[UJ], w[UJ], lo[UJ], hi[UJ];
+#pragma unroll
+        for (int j = 0; j < UJ; ++j) {
+            const unsigned x = rem + (unsigned)(64 * j + lane);           // < W + 64 * UJ <= 320
+            const unsigned dq = (x * inv_w) >> 16;                          // = x / W for x < 1024 (W <= 64)
+            w[j] = (int)(x - dq * uw);
+            q[j] = min(qbase + (int)dq, qlast);
+            lo[j] = rlo; hi[j] = rhi;
+        }
+        for (int span = rhi - rlo; span > 0; span >>= 1) {   // wave-uniform trip count: ceil(log2(window))
+#pragma unroll
+            for (int j = 0; j < UJ; ++j) {
+                const int mid = (lo[j] + hi[j] + 1) >> 1;    // lo == hi: mid == lo, nothing changes
+                if (lo[j] < hi[j]) { if (ptr[mid] <= q[j]) lo[j] = mid; else hi[j] = mid - 1; }
+            }
+        }
+        int src[UJ];
+#pragma unroll
+        for (int j = 0; j < UJ; ++j) src[j] = idx[q[j]];
+#pragma unroll
+        for (int j = 0; j < UJ; ++j) {
+            const int64_t k = kk + 64 * j + lane;
+            if (k < k1) __builtin_nontemporal_store(rv[(size_t)lo[j] * W + w[j]] + cv[(size_t)src[j] * W + w[j]], out + k);
+        }
+        rem += 64u * UJ;
+        const unsigned adv = rem / uw;
+        qbase += (int)adv;
+        rem -= adv * uw;
+        rlo = __builtin_amdgcn_readlane(lo[UJ - 1], 63);     // rows only grow along the chunks
+    }
+}
+
+// More than 64 columns: one wave per row.
+__global__ __launch_bounds__(FGNN_TPB) void u_add_v_wide_kernel(int N, int W, const int *ptr, const int *idx, const float *rv, const float *cv, float *out)
 {
     int row = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
     if (row >= N) return;
@@ -245,9 +446,41 @@ __global__ __launch_bounds__(FGNN_TPB) void u_add_v_kernel(int N, int W, const i
     }
 }
 
-// grad_row[i,w] = sum over the row's edges; grad_col[j,w] += g[p,w] with float atomics into a
-// zero-filled buffer (the reference adds into uninitialised memory, src/u_add_v/u_add_v.cu:67,87).
-__global__ __launch_bounds__(FGNN_TPB) void u_add_v_bwd_kernel(int N, int W, const int *ptr, const int *idx, const float *g, float *grow, float *gcol)
+// grad_row[i,w] = sum over the row's edges (fixed order); grad_col[j,w] += g[p,w] with float atomics into a
+// zero-filled buffer (the reference adds into uninitialised memory, src/u_add_v/u_add_v.cu:67,87).  One pass
+// over grad_out, rows shared out as in the softmax kernels.
+template <bool LONG>
+__global__ __launch_bounds__(LONG ? SO_LONG_TPB : FGNN_TPB) void u_add_v_bwd_kernel(int N, int W, const int *__restrict__ ptr,
+                                                                                    const int *__restrict__ idx, const float *__restrict__ g,
+                                                                                    float *__restrict__ grow, float *__restrict__ gcol)
+{
+    __shared__ float sh[LONG ? SO_LONG_TPB / 64 : 1][64];
+    int row, pb;
+    int64_t n;
+    row = LONG ? (int)blockIdx.x : fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (row >= N) return;
+    pb = fg_uni(ptr[row]);
+    n = (int64_t)(fg_uni(ptr[row + 1]) - pb) * W;
+    if (LONG ? n <= SO_LONG_ELEMS : n > SO_LONG_ELEMS) return;      // empty rows stay with the short launch: they store zeros
+    const int lane = fg_lane(), S0 = (64 / W) * W, w = lane % W;
+    const int per = S0 / W;                                        // entries per wave-wide trip
+    const int nw = LONG ? SO_LONG_TPB / 64 : 1;
+    const bool act = lane < S0;
+    float acc = 0.f;
+    if (act) {
+        const int pe = pb + (int)(n / W);
+#pragma unroll 4
+        for (int q = pb + (LONG ? fg_wave() * per : 0) + lane / W; q < pe; q += per * nw) {
+            const float v = g[(size_t)q * W + w];
+            acc += v;
+            unsafeAtomicAdd(gcol + (size_t)idx[q] * W + w, v);
+        }
+    }
+    acc = so_column_reduce<LONG>(acc, lane, W, S0, sh, so_add());
+    if (lane < W && (!LONG || fg_wave() == 0)) grow[(size_t)row * W + lane] = acc;
+}
+
+__global__ __launch_bounds__(FGNN_TPB) void u_add_v_bwd_wide_kernel(int N, int W, const int *ptr, const int *idx, const float *g, float *grow, float *gcol)
 {
     int row = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
     if (row >= N) return;
@@ -271,8 +504,16 @@ extern "C" int fgnn_u_add_v(int N, int64_t E, int W, const int32_t *row_ptr, con
     FGNN_REQUIRE(N >= 0 && E >= 0 && W >= 1, FGNN_ERR_SHAPE, "fgnn_u_add_v: bad sizes");
     FGNN_REQUIRE(row_ptr && row_val && col_val && (E == 0 || (col_ind && out)), FGNN_ERR_NULL, "fgnn_u_add_v: NULL argument");
     if (N == 0 || E == 0) return 0;
-    hipLaunchKernelGGL(u_add_v_kernel, dim3((unsigned)((N + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, (hipStream_t)stream, N, W, row_ptr, col_ind,
-                       row_val, col_val, out);
+    hipStream_t st = (hipStream_t)stream;
+    if (W > 64) {
+        hipLaunchKernelGGL(u_add_v_wide_kernel, dim3((unsigned)((N + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, st, N, W, row_ptr, col_ind,
+                           row_val, col_val, out);
+        return fgnn_launch_status("u_add_v_wide_kernel");
+    }
+    FGNN_REQUIRE(E <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_u_add_v: E=%lld exceeds the 32-bit row_ptr", (long long)E);
+    const int64_t per_block = (int64_t)FGNN_WPB * 64 * UAV_CHUNKS;
+    const int64_t blocks = (E * W + per_block - 1) / per_block;
+    hipLaunchKernelGGL(u_add_v_kernel, dim3((unsigned)blocks), dim3(FGNN_TPB), 0, st, N, E, W, row_ptr, col_ind, row_val, col_val, out);
     return fgnn_launch_status("u_add_v_kernel");
 }
 
@@ -284,9 +525,16 @@ extern "C" int fgnn_u_add_v_backward(int N, int64_t E, int W, const int32_t *row
     hipStream_t st = (hipStream_t)stream;
     int rc = fgnn_fill_f32(grad_col, (size_t)N * W, 0.f, st);
     if (rc || N == 0) return rc;
-    hipLaunchKernelGGL(u_add_v_bwd_kernel, dim3((unsigned)((N + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, st, N, W, row_ptr, col_ind, grad_out,
-                       grad_row, grad_col);
-    return fgnn_launch_status("u_add_v_bwd_kernel");
+    const unsigned waves = (unsigned)((N + FGNN_WPB - 1) / FGNN_WPB);
+    if (W > 64) {
+        hipLaunchKernelGGL(u_add_v_bwd_wide_kernel, dim3(waves), dim3(FGNN_TPB), 0, st, N, W, row_ptr, col_ind, grad_out, grad_row, grad_col);
+        return fgnn_launch_status("u_add_v_bwd_wide_kernel");
+    }
+    hipLaunchKernelGGL(u_add_v_bwd_kernel<false>, dim3(waves), dim3(FGNN_TPB), 0, st, N, W, row_ptr, col_ind, grad_out, grad_row, grad_col);
+    rc = fgnn_launch_status("u_add_v_bwd_kernel");
+    if (rc || E * W <= SO_LONG_ELEMS) return rc;
+    hipLaunchKernelGGL(u_add_v_bwd_kernel<true>, dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, W, row_ptr, col_ind, grad_out, grad_row, grad_col);
+    return fgnn_launch_status("u_add_v_bwd_kernel (long rows)");
 }
 
 // ------------------------------------------------------------------------------- per-edge Linear(2, D) + tanh

@@ -136,6 +136,49 @@ def test_c2_gat_backward_properties(c2_graph):
     assert float(garc.abs().max()) < 5e-4 and float(gacc.abs().max()) < 5e-2
 
 
+def test_c2_small_operators_every_entry_vs_float64(c2_graph):
+    """u_add_v, edge softmax and the multi-head SDDMM over all 114.8 M entries of the C2 graph (rows of up to 10^5
+    entries: the kernels share such a row between many waves), each way, against float64 on the device."""
+    from ae_mlsys_gnn_amd.operators.u_add_v import u_add_v_native
+    from ae_mlsys_gnn_amd.operators.edge_softmax import edge_softmax_native
+    from ae_mlsys_gnn_amd.operators import mhspmm as mh
+    g = c2_graph
+    n, e, h, f = g.n, g.n_edges, 8, 32
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    ar = torch.randn(n, h, device=DEV, generator=gen)
+    ac = torch.randn(n, h, device=DEV, generator=gen)
+    dst = orc.row_of_edge(g.row_ptr)
+    src = g.col_ind.long()
+    # u_add_v forward: one fp32 addition per element, so the result is exact
+    ee = u_add_v_native.u_add_v_forward(g.row_ptr, g.col_ind, ar, ac)
+    assert torch.equal(ee, ar[dst] + ac[src])
+    # u_add_v backward: row sums in CSR order, column sums through the transposed pattern
+    ge = torch.randn(e, h, device=DEV, generator=gen)
+    grow, gcol = u_add_v_native.u_add_v_backward(g.row_ptr, g.col_ind, ge)
+    ged = ge.double()
+    assert_close_sum(grow, orc.segment_sums(g.row_ptr, ged), orc.segment_sums(g.row_ptr, ged.abs()), "u_add_v grad row at C2", where=DEV)
+    gperm = ged[g.permute.long()]
+    assert_close_sum(gcol, orc.segment_sums(g.col_ptr, gperm), orc.segment_sums(g.col_ptr, gperm.abs()), "u_add_v grad col at C2", where=DEV)
+    del gperm
+    # edge softmax: exponents are differences to the row maximum, at most max - min of the inputs
+    lo, hi = ee.aminmax()
+    c = c_exp(float(hi - lo))
+    sm = edge_softmax_native.edge_softmax(g.row_ptr, ee)
+    ref, _, _ = orc._segment_softmax(ee.double(), dst, n)
+    assert_close_sum(sm, ref, torch.ones((), device=DEV, dtype=torch.float64), "edge softmax at C2", c=c, where=DEV)
+    assert float((orc.segment_sums(g.row_ptr, sm.double()) - (g.row_ptr[1:] > g.row_ptr[:-1]).double().view(n, 1)).abs().max()) < 1e-5
+    gin = edge_softmax_native.edge_softmax_backward(g.row_ptr, sm, ge)
+    dot = orc.segment_sums(g.row_ptr, ref * ged)
+    dot_abs = orc.segment_sums(g.row_ptr, ref * ged.abs())
+    assert_close_sum(gin, ref * (ged - dot[dst]), ref * (ged.abs() + dot_abs[dst]), "edge softmax backward at C2", c=c, where=DEV)
+    del ref, dot, dot_abs, ged, gin, sm, ee
+    # multi-head SDDMM: <a[row], b[source]> per head
+    a = torch.randn(n, h, f, device=DEV, generator=gen)
+    b = torch.randn(n, h, f, device=DEV, generator=gen)
+    out = mh.mhsddmm(g.row_ptr, g.col_ind, a, b)
+    assert_close_sum(out, orc.edge_dots(dst, src, a, b), orc.edge_dots(dst, src, a, b, absolute=True), "mhsddmm at C2", where=DEV)
+
+
 def test_c3_edgeconv_full_size_vs_oracle():
     from ae_mlsys_gnn_amd.operators.fused_edgeconv import edgeconv_native
     from ae_mlsys_gnn_amd.operators import knn as knn_op

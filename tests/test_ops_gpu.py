@@ -377,11 +377,19 @@ def test_mhspmm_and_mhsddmm(h, f):
     assert torch.equal(tr.cpu(), att.float()[g.permute.long()])
 
 
-def test_edge_softmax():
+# widths either side of the lane maps: 1, odd, powers of two, 33 (one entry per wave trip), 64, and 70 (the one-wave-per-row
+# kernels); the graph has rows of 0..513 entries and a 3000-entry hub, so each width meets rows on both sides of the
+# single-wave / whole-workgroup threshold
+SMALL_OP_WIDTHS = [1, 3, 4, 8, 12, 33, 64, 70]
+
+
+@pytest.mark.parametrize("nh", SMALL_OP_WIDTHS)
+def test_edge_softmax(nh):
     from ae_mlsys_gnn_amd.operators import edge_softmax as op
     g = _small_graph()
-    h = torch.randn(g.n_edges, 4, dtype=torch.float64) * 3
-    go = torch.randn(g.n_edges, 4, dtype=torch.float64)
+    gen = torch.Generator().manual_seed(nh)
+    h = torch.randn(g.n_edges, nh, generator=gen, dtype=torch.float64) * 3
+    go = torch.randn(g.n_edges, nh, generator=gen, dtype=torch.float64)
     hl = h.clone().requires_grad_(True)
     ref = orc.edge_softmax(g.row_ptr, hl)
     ref.backward(go)
@@ -392,12 +400,14 @@ def test_edge_softmax():
     assert_close(hd.grad, hl.grad, "edge_softmax grad")
 
 
-def test_u_add_v():
+@pytest.mark.parametrize("nh", SMALL_OP_WIDTHS)
+def test_u_add_v(nh):
     from ae_mlsys_gnn_amd.operators import u_add_v as op
     g = _small_graph()
-    rv = torch.randn(g.n, 4, dtype=torch.float64)
-    cv = torch.randn(g.n, 4, dtype=torch.float64)
-    go = torch.randn(g.n_edges, 4, dtype=torch.float64)
+    gen = torch.Generator().manual_seed(100 + nh)
+    rv = torch.randn(g.n, nh, generator=gen, dtype=torch.float64)
+    cv = torch.randn(g.n, nh, generator=gen, dtype=torch.float64)
+    go = torch.randn(g.n_edges, nh, generator=gen, dtype=torch.float64)
     rl, cl = rv.clone().requires_grad_(True), cv.clone().requires_grad_(True)
     ref = orc.u_add_v(g.row_ptr, g.col_ind, rl, cl)
     ref.backward(go)

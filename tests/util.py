@@ -40,18 +40,19 @@ def c_exp(max_abs_exponent):
     return C_SUM + 4.0 * float(max_abs_exponent)
 
 
-def assert_close_sum(got, ref, s_abs, what, rtol=RTOL, atol=ATOL, c=C_SUM, extra=None):
+def assert_close_sum(got, ref, s_abs, what, rtol=RTOL, atol=ATOL, c=C_SUM, extra=None, where="cpu"):
     """extra: an additional absolute allowance per element (e.g. what a LeakyReLU' jump at a pre-activation of
-    zero can change), zero wherever it does not apply."""
-    got = got.detach().cpu().double()
-    ref = ref.detach().cpu().double()
-    s_abs = torch.as_tensor(s_abs).detach().cpu().double()
+    zero can change), zero wherever it does not apply.  where: the device the comparison runs on (arrays of
+    10^9 elements stay on the GPU)."""
+    got = got.detach().to(where).double()
+    ref = ref.detach().to(where).double()
+    s_abs = torch.as_tensor(s_abs).detach().to(where).double()
     assert got.shape == ref.shape, "%s: shape %s vs %s" % (what, tuple(got.shape), tuple(ref.shape))
     s_abs = s_abs.expand_as(ref)
     err = (got - ref).abs()
     tol = rtol * ref.abs() + torch.clamp(c * EPS32 * s_abs, min=atol)
     if extra is not None:
-        tol = tol + torch.as_tensor(extra).detach().cpu().double().expand_as(ref)
+        tol = tol + torch.as_tensor(extra).detach().to(where).double().expand_as(ref)
     bad = err > tol
     if bad.any():
         i = int(torch.argmax(err - tol))

@@ -34,6 +34,7 @@ _SIGNATURES = {
     "fgnn_schedule_num_splits": (c_int, [c_void_p]),
     "fgnn_schedule_export": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p]),
     "fgnn_validate_graph": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int64, c_void_p]),
+    "fgnn_row_length_stats": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "fgnn_gat_forward_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int]),
     "fgnn_gat_forward": (c_int, [c_int, c_int64, c_int, c_int] + [c_void_p] * 4 + [c_float] + [c_void_p] * 8
                          + [c_void_p, c_void_p, c_size_t, c_void_p]),
@@ -209,14 +210,15 @@ BUCKET_MIN_SHARE = 0.25      # ...and they must hold at least this share of the 
 BUCKET_MIN_SKEW = 4          # longest row / mean row length
 
 
-def xcd_buckets_enabled(ptr_tensor) -> bool:
+def xcd_buckets_enabled(ptr_tensor, idx_numel=None) -> bool:
     """Whether operators get the XCD-aware schedule for this pointer array (FGNN_XCD_BUCKETS=0/1
     overrides).  It pays off on skewed graphs, where the rows longer than 64 entries hold a good part
     of the work: cutting them by source bucket keeps each XCD's L2 on one eighth of the gathered rows
     and shortens the longest work item.  It costs time on graphs without hubs (every row of a
     uniform degree-100 graph would become eight short segments with nothing to reuse between them),
     so the rule asks for both: rows longer than 64 hold a quarter of the entries, and the longest row
-    is at least 4x the mean.  The two numbers are read from the device once per array and cached."""
+    is at least 4x the mean.  The two numbers come from one reduction kernel, once per array, and are cached.
+    idx_numel: the number of entries when the caller has it (saves reading ptr[-1] back)."""
     env = os.environ.get("FGNN_XCD_BUCKETS")
     if env is not None:
         return env not in ("0", "")
@@ -226,9 +228,12 @@ def xcd_buckets_enabled(ptr_tensor) -> bool:
     key = (ptr_tensor.data_ptr(), ptr_tensor.numel(), ptr_tensor.device.index, ptr_tensor._version)
     hit = _bucket_rule_cache.get(key)
     if hit is None:
-        deg = (ptr_tensor[1:] - ptr_tensor[:-1]).long()
-        long_rows = torch.where(deg > BUCKET_ROW_LEN, deg, torch.zeros_like(deg)).sum()
-        n_edges, n_long, longest = torch.stack([deg.sum(), long_rows, deg.max()]).tolist()
+        stats = (ctypes.c_int64 * 2)()
+        with torch.cuda.device(ptr_tensor.device):
+            check(lib().fgnn_row_length_stats(ptr(ptr_tensor), n_rows, BUCKET_ROW_LEN, ctypes.cast(stats, c_void_p), stream_ptr()),
+                  "fgnn_row_length_stats")
+        n_long, longest = int(stats[0]), int(stats[1])
+        n_edges = int(idx_numel) if idx_numel is not None else int(ptr_tensor[-1])
         hit = (n_edges > 0 and n_long >= BUCKET_MIN_SHARE * n_edges and longest * n_rows >= BUCKET_MIN_SKEW * n_edges,
                ptr_tensor)         # the entry holds the tensor: its address cannot be reused while the entry lives
         _bucket_rule_cache[key] = hit
@@ -247,7 +252,7 @@ def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True,
     out (`edge_positions`): operators called with it take per-edge tensors in the schedule's order."""
     if seg_len is None:
         seg_len = default_seg_len()
-    if idx_tensor is not None and not xcd_buckets_enabled(ptr_tensor):
+    if idx_tensor is not None and not xcd_buckets_enabled(ptr_tensor, idx_tensor.numel()):
         idx_tensor = None
     min_deg = int(os.environ.get("FGNN_BUCKET_MIN_DEG", "0"))
 

@@ -675,6 +675,61 @@ extern "C" int fgnn_validate_graph(const int32_t *ptr_dev, const int32_t *idx_de
     return 0;
 }
 
+// stats[0] += entries of the rows longer than long_len, stats[1] = max row length (both as unsigned 64-bit)
+__global__ __launch_bounds__(256) void row_length_stats_kernel(const int *__restrict__ ptr, int n_rows, int long_len,
+                                                               unsigned long long *__restrict__ stats)
+{
+    __shared__ unsigned long long sh_sum[4];
+    __shared__ int sh_max[4];
+    unsigned long long sum = 0;
+    int longest = 0;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n_rows; i += (int64_t)gridDim.x * 256) {
+        const int d = ptr[i + 1] - ptr[i];
+        if (d > long_len) sum += (unsigned long long)d;
+        longest = max(longest, d);
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        sum += __shfl_down(sum, off);
+        longest = max(longest, __shfl_down(longest, off));
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) { sh_sum[wave] = sum; sh_max[wave] = longest; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        sum = (sh_sum[0] + sh_sum[1]) + (sh_sum[2] + sh_sum[3]);
+        longest = max(max(sh_max[0], sh_max[1]), max(sh_max[2], sh_max[3]));
+        if (sum) atomicAdd(stats, sum);
+        if (longest > 0) atomicMax(stats + 1, (unsigned long long)longest);
+    }
+}
+
+extern "C" int fgnn_row_length_stats(const int32_t *ptr_dev, int n_rows, int long_len, int64_t *stats_host, void *stream)
+{
+    FGNN_REQUIRE(ptr_dev && stats_host, FGNN_ERR_NULL, "fgnn_row_length_stats: NULL argument");
+    FGNN_REQUIRE(n_rows >= 0 && long_len >= 0, FGNN_ERR_SHAPE, "fgnn_row_length_stats: bad sizes n_rows=%d long_len=%d", n_rows, long_len);
+    stats_host[0] = stats_host[1] = 0;
+    if (n_rows == 0) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    unsigned long long *dev = nullptr, host[2] = {0, 0};
+    FGNN_HIP(hipMalloc((void **)&dev, sizeof(host)));
+    hipError_t err = hipMemcpyAsync(dev, host, sizeof(host), hipMemcpyHostToDevice, st);
+    if (err == hipSuccess) {
+        const unsigned grid = (unsigned)std::min<int64_t>(((int64_t)n_rows + 255) / 256, 2048);
+        hipLaunchKernelGGL(row_length_stats_kernel, dim3(grid), dim3(256), 0, st, ptr_dev, n_rows, long_len, dev);
+        err = hipGetLastError();
+    }
+    if (err == hipSuccess) err = hipMemcpyAsync(host, dev, sizeof(host), hipMemcpyDeviceToHost, st);
+    if (err == hipSuccess) err = hipStreamSynchronize(st);
+    (void)hipFree(dev);
+    if (err != hipSuccess) {
+        fgnn_set_error("fgnn_row_length_stats: %s", hipGetErrorString(err));
+        return (int)err;
+    }
+    stats_host[0] = (int64_t)host[0];
+    stats_host[1] = (int64_t)host[1];
+    return 0;
+}
+
 extern "C" int fgnn_schedule_num_items(const fgnn_schedule_t *s) { return s ? s->n_items : 0; }
 extern "C" int fgnn_schedule_num_partials(const fgnn_schedule_t *s) { return s ? s->n_partials : 0; }
 extern "C" int64_t fgnn_schedule_num_edges(const fgnn_schedule_t *s) { return s ? s->n_edges : 0; }

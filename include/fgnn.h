@@ -95,6 +95,13 @@ int     fgnn_schedule_export(const fgnn_schedule_t *s, int32_t *items_out, int32
 int     fgnn_validate_graph(const int32_t *ptr_dev, const int32_t *idx_dev, int n_rows, int n_cols, int64_t E,
                             void *stream);
 
+/* Two numbers about the row lengths of a pointer array, for the caller's choice between the plain and the
+ * XCD-aware schedule: stats_host[0] = entries held by rows longer than long_len, stats_host[1] = the longest
+ * row.  One reduction kernel and a 16-byte read-back (synchronises `stream`).  No counterpart in the
+ * reference, whose kernels take one row per thread block whatever its length
+ * (src/fused_gat/fused_gat_SM.cu:139-145 launches N blocks). */
+int     fgnn_row_length_stats(const int32_t *ptr_dev, int n_rows, int long_len, int64_t *stats_host, void *stream);
+
 /* ---------------------------------------------------------------- fused GAT
  * Replaces fused_gat_SM.gat_forward (src/fused_gat/fused_gat_SM.cpp:14-38, host launcher
  * fused_gat_SM.cu:536-558) and, with e_lrelu/e_softmax non-NULL, fused_gat_stash.gat_forward

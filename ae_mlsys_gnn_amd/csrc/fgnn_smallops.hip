@@ -207,101 +207,209 @@ extern "C" int fgnn_gather_rows(int64_t E, int W, const int32_t *permute, const 
 // each (first launch), longer ones by a whole workgroup each (second launch, whose other
 // workgroups leave at once): a 100 k-entry hub row is then a few hundred trips of 512 threads
 // instead of tens of thousands of trips of one wave.
-#define SO_LONG_ELEMS 2048
+#define SO_LONG_ELEMS 8192
 #define SO_LONG_TPB 512
+#define SO_CACHE 8            // values per lane kept in registers by the softmax kernels
 
 struct so_max { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
 struct so_add { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
 
-// Combines the values of the lanes t, t + W, t + 2W, ... < S0 (any count, by suffix doubling) and of
-// the workgroup's waves (LONG) in a fixed order; every lane gets the result of its column.
-template <bool LONG, class Op>
-__device__ __forceinline__ float so_column_reduce(float v, int lane, int W, int S0, float (*sh)[64], Op op)
+template <int VEC> struct so_grp { float c[VEC]; };
+
+// Combines, per component, the values of the lanes t, t + W, t + 2W, ... < S0 (any count, by suffix doubling) and
+// of the workgroup's waves (LONG) in a fixed order; every lane gets the result of its column.  W * VEC <= 64.
+template <bool LONG, int VEC, class Op>
+__device__ __forceinline__ so_grp<VEC> so_column_reduce(so_grp<VEC> v, int lane, int W, int S0, float (*sh)[64], Op op)
 {
     for (int off = W; off < S0; off <<= 1) {
-        const float o = __shfl(v, (lane + off) & 63);
-        if (lane + off < S0) v = op(v, o);
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) {
+            const float o = __shfl(v.c[c], (lane + off) & 63);
+            if (lane + off < S0) v.c[c] = op(v.c[c], o);
+        }
     }
-    v = __shfl(v, lane % W);
+    const int col = lane % W;
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) v.c[c] = __shfl(v.c[c], col);
     if constexpr (LONG) {
         const int w = fg_wave();
-        if (lane < W) sh[w][lane] = v;
+        if (lane < W) {
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) sh[w][c * W + lane] = v.c[c];
+        }
         __syncthreads();
-        float r = sh[0][lane % W];
-        for (int i = 1; i < SO_LONG_TPB / 64; ++i) r = op(r, sh[i][lane % W]);
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) {
+            float r = sh[0][c * W + col];
+            for (int i = 1; i < SO_LONG_TPB / 64; ++i) r = op(r, sh[i][c * W + col]);
+            v.c[c] = r;
+        }
         __syncthreads();
-        v = r;
     }
     return v;
 }
 
-// The row of this wave (short rows) or workgroup (LONG); false when it belongs to the other launch.
-template <bool LONG>
+// The row of this wave (short rows) or workgroup (LONG); false when it belongs to the other launch.  W counts the
+// groups of VEC floats per entry, n the groups of the row.
+// Work unit u (a wave or a workgroup, in launch order) takes row (u * p) mod N with p a prime above 2^31: a
+// bijection of [0, N) that scatters neighbouring rows.  Workgroups go to the eight XCDs round-robin, and on a
+// power-law graph generated by recursive quadrants a row's length follows the low bits of its number (the
+// rows = 0 mod 8 of an R-MAT graph hold 44 % of the entries): in row order one XCD would get most of the work.
+__device__ __forceinline__ int so_scattered_row(unsigned u, int N) { return (int)(((unsigned long long)u * 2654435761ull) % (unsigned)N); }
+
+template <bool LONG, int VEC>
 __device__ __forceinline__ bool so_take_row(int N, int W, const int *ptr, int &row, int &pb, int64_t &n)
 {
-    row = LONG ? (int)blockIdx.x : fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
-    if (row >= N) return false;
+    const unsigned u = LONG ? blockIdx.x : (unsigned)fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (u >= (unsigned)N) return false;
+    row = fg_uni(so_scattered_row(u, N));
     pb = fg_uni(ptr[row]);
     n = (int64_t)(fg_uni(ptr[row + 1]) - pb) * W;
-    return LONG ? n > SO_LONG_ELEMS : (n > 0 && n <= SO_LONG_ELEMS);
+    return LONG ? n * VEC > SO_LONG_ELEMS : (n > 0 && n * VEC <= SO_LONG_ELEMS);
+}
+
+template <int VEC> __device__ __forceinline__ so_grp<VEC> so_load(const float *p)
+{
+    so_grp<VEC> r;
+    if constexpr (VEC == 4) { const float4 t = *reinterpret_cast<const float4 *>(p); r.c[0] = t.x; r.c[1] = t.y; r.c[2] = t.z; r.c[3] = t.w; }
+    else r.c[0] = *p;
+    return r;
+}
+template <int VEC> __device__ __forceinline__ void so_store(float *p, const so_grp<VEC> &r)
+{
+    if constexpr (VEC == 4) *reinterpret_cast<float4 *>(p) = make_float4(r.c[0], r.c[1], r.c[2], r.c[3]);
+    else *p = r.c[0];
+}
+template <int VEC> __device__ __forceinline__ so_grp<VEC> so_fill(float x)
+{
+    so_grp<VEC> r;
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) r.c[c] = x;
+    return r;
 }
 
 // Per-row, per-head softmax over [E,H] (src/edge_softmax/edge_softmax.cu:7-61) and its backward
-// s*(g - sum_row s*g) (:63-98).
-template <bool LONG>
-__global__ __launch_bounds__(LONG ? SO_LONG_TPB : FGNN_TPB) void edge_softmax_kernel(int N, int H, const int *__restrict__ ptr,
+// s*(g - sum_row s*g) (:63-98).  VEC = 4 (H % 4 == 0, 16-byte aligned arrays): a lane owns four consecutive
+// heads of an entry; with the eight trips unrolled a hub row keeps 128 bytes per lane in flight.
+template <bool LONG, int VEC>
+__global__ __launch_bounds__(LONG ? SO_LONG_TPB : FGNN_TPB) void edge_softmax_kernel(int N, int W, const int *__restrict__ ptr,
                                                                                      const float *__restrict__ in, float *__restrict__ out)
 {
     __shared__ float sh[LONG ? SO_LONG_TPB / 64 : 1][64];
     int row, pb;
     int64_t n;
-    if (!so_take_row<LONG>(N, H, ptr, row, pb, n)) return;          // uniform over the workgroup when LONG
-    const int lane = fg_lane(), S0 = (64 / H) * H;
+    if (!so_take_row<LONG, VEC>(N, W, ptr, row, pb, n)) return;      // uniform over the workgroup when LONG
+    const int lane = fg_lane(), S0 = (64 / W) * W;
     const int64_t first = (LONG ? fg_wave() * S0 : 0) + lane, step = (int64_t)S0 * (LONG ? SO_LONG_TPB / 64 : 1);
     const bool act = lane < S0;
-    const float *src = in + (size_t)pb * H;
-    float *dst = out + (size_t)pb * H;
-    float m = -INFINITY;
-    if (act) {
-#pragma unroll 4
-        for (int64_t k = first; k < n; k += step) m = fmaxf(m, src[k]);
+    const float *src = in + (size_t)pb * W * VEC;
+    float *dst = out + (size_t)pb * W * VEC;
+    // the first SO_CACHE groups of a lane stay in registers over the three phases; what a longer row has beyond
+    // them is read again (from the L2, which the first phase has just filled)
+    so_grp<VEC> v[SO_CACHE], m = so_fill<VEC>(-INFINITY), s = so_fill<VEC>(0.f);
+#pragma unroll
+    for (int i = 0; i < SO_CACHE; ++i) {
+        const int64_t k = first + i * step;
+        v[i] = (act && k < n) ? so_load<VEC>(src + k * VEC) : so_fill<VEC>(-INFINITY);
     }
-    m = so_column_reduce<LONG>(m, lane, H, S0, sh, so_max());
-    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < SO_CACHE; ++i)
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) m.c[c] = fmaxf(m.c[c], v[i].c[c]);
+    const int64_t rest = first + SO_CACHE * step;
     if (act) {
-#pragma unroll 4
-        for (int64_t k = first; k < n; k += step) s += __expf(src[k] - m);
+#pragma unroll 8
+        for (int64_t k = rest; k < n; k += step) {
+            const so_grp<VEC> t = so_load<VEC>(src + k * VEC);
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) m.c[c] = fmaxf(m.c[c], t.c[c]);
+        }
     }
-    s = so_column_reduce<LONG>(s, lane, H, S0, sh, so_add());
-    const float inv = 1.f / s;
+    m = so_column_reduce<LONG, VEC>(m, lane, W, S0, sh, so_max());
+#pragma unroll
+    for (int i = 0; i < SO_CACHE; ++i)
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) { v[i].c[c] = __expf(v[i].c[c] - m.c[c]); s.c[c] += v[i].c[c]; }      // exp(-inf) = 0 past the row
     if (act) {
-#pragma unroll 4
-        for (int64_t k = first; k < n; k += step) dst[k] = __expf(src[k] - m) * inv;
+#pragma unroll 8
+        for (int64_t k = rest; k < n; k += step) {
+            const so_grp<VEC> t = so_load<VEC>(src + k * VEC);
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) s.c[c] += __expf(t.c[c] - m.c[c]);
+        }
+    }
+    so_grp<VEC> inv = so_column_reduce<LONG, VEC>(s, lane, W, S0, sh, so_add());
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) inv.c[c] = 1.f / inv.c[c];
+#pragma unroll
+    for (int i = 0; i < SO_CACHE; ++i) {
+        const int64_t k = first + i * step;
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) v[i].c[c] *= inv.c[c];
+        if (act && k < n) so_store<VEC>(dst + k * VEC, v[i]);
+    }
+    if (act) {
+#pragma unroll 8
+        for (int64_t k = rest; k < n; k += step) {
+            so_grp<VEC> t = so_load<VEC>(src + k * VEC);
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) t.c[c] = __expf(t.c[c] - m.c[c]) * inv.c[c];
+            so_store<VEC>(dst + k * VEC, t);
+        }
     }
 }
 
-template <bool LONG>
-__global__ __launch_bounds__(LONG ? SO_LONG_TPB : FGNN_TPB) void edge_softmax_bwd_kernel(int N, int H, const int *__restrict__ ptr,
+template <bool LONG, int VEC>
+__global__ __launch_bounds__(LONG ? SO_LONG_TPB : FGNN_TPB) void edge_softmax_bwd_kernel(int N, int W, const int *__restrict__ ptr,
                                                                                          const float *__restrict__ sm, const float *__restrict__ g,
                                                                                          float *__restrict__ gin)
 {
     __shared__ float sh[LONG ? SO_LONG_TPB / 64 : 1][64];
     int row, pb;
     int64_t n;
-    if (!so_take_row<LONG>(N, H, ptr, row, pb, n)) return;
-    const int lane = fg_lane(), S0 = (64 / H) * H;
+    if (!so_take_row<LONG, VEC>(N, W, ptr, row, pb, n)) return;
+    const int lane = fg_lane(), S0 = (64 / W) * W;
     const int64_t first = (LONG ? fg_wave() * S0 : 0) + lane, step = (int64_t)S0 * (LONG ? SO_LONG_TPB / 64 : 1);
     const bool act = lane < S0;
-    const size_t base = (size_t)pb * H;
-    float acc = 0.f;
-    if (act) {
-#pragma unroll 4
-        for (int64_t k = first; k < n; k += step) acc = fmaf(sm[base + k], g[base + k], acc);
+    const size_t base = (size_t)pb * W * VEC;
+    so_grp<VEC> sv[SO_CACHE], gv[SO_CACHE], acc = so_fill<VEC>(0.f);
+#pragma unroll
+    for (int i = 0; i < SO_CACHE; ++i) {
+        const int64_t k = first + i * step;
+        const bool ok = act && k < n;
+        sv[i] = ok ? so_load<VEC>(sm + base + k * VEC) : so_fill<VEC>(0.f);
+        gv[i] = ok ? so_load<VEC>(g + base + k * VEC) : so_fill<VEC>(0.f);
     }
-    acc = so_column_reduce<LONG>(acc, lane, H, S0, sh, so_add());
+#pragma unroll
+    for (int i = 0; i < SO_CACHE; ++i)
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) acc.c[c] = fmaf(sv[i].c[c], gv[i].c[c], acc.c[c]);
+    const int64_t rest = first + SO_CACHE * step;
     if (act) {
 #pragma unroll 4
-        for (int64_t k = first; k < n; k += step) gin[base + k] = sm[base + k] * (g[base + k] - acc);
+        for (int64_t k = rest; k < n; k += step) {
+            const so_grp<VEC> a = so_load<VEC>(sm + base + k * VEC), b = so_load<VEC>(g + base + k * VEC);
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) acc.c[c] = fmaf(a.c[c], b.c[c], acc.c[c]);
+        }
+    }
+    acc = so_column_reduce<LONG, VEC>(acc, lane, W, S0, sh, so_add());
+#pragma unroll
+    for (int i = 0; i < SO_CACHE; ++i) {
+        const int64_t k = first + i * step;
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) sv[i].c[c] *= gv[i].c[c] - acc.c[c];
+        if (act && k < n) so_store<VEC>(gin + base + k * VEC, sv[i]);
+    }
+    if (act) {
+#pragma unroll 4
+        for (int64_t k = rest; k < n; k += step) {
+            so_grp<VEC> a = so_load<VEC>(sm + base + k * VEC);
+            const so_grp<VEC> b = so_load<VEC>(g + base + k * VEC);
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) a.c[c] *= b.c[c] - acc.c[c];
+            so_store<VEC>(gin + base + k * VEC, a);
+        }
     }
 }
 
@@ -352,11 +460,15 @@ extern "C" int fgnn_edge_softmax(int N, int64_t E, int H, const int32_t *row_ptr
         hipLaunchKernelGGL(edge_softmax_wide_kernel, dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, in, out);
         return fgnn_launch_status("edge_softmax_wide_kernel");
     }
-    hipLaunchKernelGGL(edge_softmax_kernel<false>, dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, in, out);
-    int rc = fgnn_launch_status("edge_softmax_kernel");
-    if (rc || E * H <= SO_LONG_ELEMS) return rc;                    // no row can be long
-    hipLaunchKernelGGL(edge_softmax_kernel<true>, dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, H, row_ptr, in, out);
-    return fgnn_launch_status("edge_softmax_kernel (long rows)");
+    const bool some_long = E * H > SO_LONG_ELEMS;                   // otherwise no row can be long
+    if (H % 4 == 0 && fgnn_aligned16(in) && fgnn_aligned16(out)) {
+        hipLaunchKernelGGL((edge_softmax_kernel<false, 4>), dim3(waves), dim3(FGNN_TPB), 0, st, N, H / 4, row_ptr, in, out);
+        if (some_long) hipLaunchKernelGGL((edge_softmax_kernel<true, 4>), dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, H / 4, row_ptr, in, out);
+    } else {
+        hipLaunchKernelGGL((edge_softmax_kernel<false, 1>), dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, in, out);
+        if (some_long) hipLaunchKernelGGL((edge_softmax_kernel<true, 1>), dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, H, row_ptr, in, out);
+    }
+    return fgnn_launch_status("edge_softmax_kernel");
 }
 
 extern "C" int fgnn_edge_softmax_backward(int N, int64_t E, int H, const int32_t *row_ptr, const float *sm, const float *grad_out,
@@ -371,11 +483,17 @@ extern "C" int fgnn_edge_softmax_backward(int N, int64_t E, int H, const int32_t
         hipLaunchKernelGGL(edge_softmax_bwd_wide_kernel, dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, sm, grad_out, grad_in);
         return fgnn_launch_status("edge_softmax_bwd_wide_kernel");
     }
-    hipLaunchKernelGGL(edge_softmax_bwd_kernel<false>, dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, sm, grad_out, grad_in);
-    int rc = fgnn_launch_status("edge_softmax_bwd_kernel");
-    if (rc || E * H <= SO_LONG_ELEMS) return rc;
-    hipLaunchKernelGGL(edge_softmax_bwd_kernel<true>, dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, H, row_ptr, sm, grad_out, grad_in);
-    return fgnn_launch_status("edge_softmax_bwd_kernel (long rows)");
+    const bool some_long = E * H > SO_LONG_ELEMS;
+    if (H % 4 == 0 && fgnn_aligned16(sm) && fgnn_aligned16(grad_out) && fgnn_aligned16(grad_in)) {
+        hipLaunchKernelGGL((edge_softmax_bwd_kernel<false, 4>), dim3(waves), dim3(FGNN_TPB), 0, st, N, H / 4, row_ptr, sm, grad_out, grad_in);
+        if (some_long)
+            hipLaunchKernelGGL((edge_softmax_bwd_kernel<true, 4>), dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, H / 4, row_ptr, sm, grad_out, grad_in);
+    } else {
+        hipLaunchKernelGGL((edge_softmax_bwd_kernel<false, 1>), dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, sm, grad_out, grad_in);
+        if (some_long)
+            hipLaunchKernelGGL((edge_softmax_bwd_kernel<true, 1>), dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, H, row_ptr, sm, grad_out, grad_in);
+    }
+    return fgnn_launch_status("edge_softmax_bwd_kernel");
 }
 
 // out[p,w] = row_val[row(p),w] + col_val[col_ind[p],w]  (src/u_add_v/u_add_v.cu:4-26).  W <= 64: one thread per
@@ -383,6 +501,8 @@ extern "C" int fgnn_edge_softmax_backward(int N, int64_t E, int H, const int32_t
 // for the wave's first and last edge (wave-uniform), then per lane inside that usually one- or two-row window.
 #define UAV_CHUNKS 32           // 64-element chunks per wave
 #define UAV_UJ 4                // chunks in flight; divides UAV_CHUNKS
+// VEC = 4: an element is four consecutive columns (W % 4 == 0, 16-byte aligned arrays), W counts such groups.
+template <int VEC>
 __global__ __launch_bounds__(FGNN_TPB) void u_add_v_kernel(int N, int64_t E, int W, const int *__restrict__ ptr, const int *__restrict__ idx,
                                                            const float *__restrict__ rv, const float *__restrict__ cv, float *__restrict__ out)
 {
@@ -422,7 +542,13 @@ __global__ __launch_bounds__(FGNN_TPB) void u_add_v_kernel(int N, int64_t E, int
 #pragma unroll
         for (int j = 0; j < UJ; ++j) {
             const int64_t k = kk + 64 * j + lane;
-            if (k < k1) __builtin_nontemporal_store(rv[(size_t)lo[j] * W + w[j]] + cv[(size_t)src[j] * W + w[j]], out + k);
+            if (k < k1) {
+                fg_vec<VEC> a, b;
+                a.load(rv + ((size_t)lo[j] * W + w[j]) * VEC);
+                b.load(cv + ((size_t)src[j] * W + w[j]) * VEC);
+                a.add(b);
+                a.store_nt(out + (size_t)k * VEC);
+            }
         }
         rem += 64u * UJ;
         const unsigned adv = rem / uw;
@@ -449,35 +575,34 @@ __global__ __launch_bounds__(FGNN_TPB) void u_add_v_wide_kernel(int N, int W, co
 // grad_row[i,w] = sum over the row's edges (fixed order); grad_col[j,w] += g[p,w] with float atomics into a
 // zero-filled buffer (the reference adds into uninitialised memory, src/u_add_v/u_add_v.cu:67,87).  One pass
 // over grad_out, rows shared out as in the softmax kernels.
-template <bool LONG>
+template <bool LONG, int VEC>
 __global__ __launch_bounds__(LONG ? SO_LONG_TPB : FGNN_TPB) void u_add_v_bwd_kernel(int N, int W, const int *__restrict__ ptr,
                                                                                     const int *__restrict__ idx, const float *__restrict__ g,
                                                                                     float *__restrict__ grow, float *__restrict__ gcol)
 {
     __shared__ float sh[LONG ? SO_LONG_TPB / 64 : 1][64];
-    int row, pb;
-    int64_t n;
-    row = LONG ? (int)blockIdx.x : fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
-    if (row >= N) return;
-    pb = fg_uni(ptr[row]);
-    n = (int64_t)(fg_uni(ptr[row + 1]) - pb) * W;
+    const unsigned u = LONG ? blockIdx.x : (unsigned)fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (u >= (unsigned)N) return;
+    const int row = fg_uni(so_scattered_row(u, N));
+    const int pb = fg_uni(ptr[row]), pe = fg_uni(ptr[row + 1]);
+    const int64_t n = (int64_t)(pe - pb) * W * VEC;
     if (LONG ? n <= SO_LONG_ELEMS : n > SO_LONG_ELEMS) return;      // empty rows stay with the short launch: they store zeros
     const int lane = fg_lane(), S0 = (64 / W) * W, w = lane % W;
     const int per = S0 / W;                                        // entries per wave-wide trip
     const int nw = LONG ? SO_LONG_TPB / 64 : 1;
     const bool act = lane < S0;
-    float acc = 0.f;
+    so_grp<VEC> acc = so_fill<VEC>(0.f);
     if (act) {
-        const int pe = pb + (int)(n / W);
-#pragma unroll 4
+#pragma unroll 8
         for (int q = pb + (LONG ? fg_wave() * per : 0) + lane / W; q < pe; q += per * nw) {
-            const float v = g[(size_t)q * W + w];
-            acc += v;
-            unsafeAtomicAdd(gcol + (size_t)idx[q] * W + w, v);
+            const so_grp<VEC> v = so_load<VEC>(g + ((size_t)q * W + w) * VEC);
+            float *dst = gcol + ((size_t)idx[q] * W + w) * VEC;
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) { acc.c[c] += v.c[c]; unsafeAtomicAdd(dst + c, v.c[c]); }
         }
     }
-    acc = so_column_reduce<LONG>(acc, lane, W, S0, sh, so_add());
-    if (lane < W && (!LONG || fg_wave() == 0)) grow[(size_t)row * W + lane] = acc;
+    acc = so_column_reduce<LONG, VEC>(acc, lane, W, S0, sh, so_add());
+    if (lane < W && (!LONG || fg_wave() == 0)) so_store<VEC>(grow + ((size_t)row * W + lane) * VEC, acc);
 }
 
 __global__ __launch_bounds__(FGNN_TPB) void u_add_v_bwd_wide_kernel(int N, int W, const int *ptr, const int *idx, const float *g, float *grow, float *gcol)
@@ -512,8 +637,13 @@ extern "C" int fgnn_u_add_v(int N, int64_t E, int W, const int32_t *row_ptr, con
     }
     FGNN_REQUIRE(E <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_u_add_v: E=%lld exceeds the 32-bit row_ptr", (long long)E);
     const int64_t per_block = (int64_t)FGNN_WPB * 64 * UAV_CHUNKS;
-    const int64_t blocks = (E * W + per_block - 1) / per_block;
-    hipLaunchKernelGGL(u_add_v_kernel, dim3((unsigned)blocks), dim3(FGNN_TPB), 0, st, N, E, W, row_ptr, col_ind, row_val, col_val, out);
+    if (W % 4 == 0 && fgnn_aligned16(row_val) && fgnn_aligned16(col_val) && fgnn_aligned16(out)) {
+        const int64_t blocks = (E * (W / 4) + per_block - 1) / per_block;
+        hipLaunchKernelGGL(u_add_v_kernel<4>, dim3((unsigned)blocks), dim3(FGNN_TPB), 0, st, N, E, W / 4, row_ptr, col_ind, row_val, col_val, out);
+    } else {
+        const int64_t blocks = (E * W + per_block - 1) / per_block;
+        hipLaunchKernelGGL(u_add_v_kernel<1>, dim3((unsigned)blocks), dim3(FGNN_TPB), 0, st, N, E, W, row_ptr, col_ind, row_val, col_val, out);
+    }
     return fgnn_launch_status("u_add_v_kernel");
 }
 
@@ -530,11 +660,12 @@ extern "C" int fgnn_u_add_v_backward(int N, int64_t E, int W, const int32_t *row
         hipLaunchKernelGGL(u_add_v_bwd_wide_kernel, dim3(waves), dim3(FGNN_TPB), 0, st, N, W, row_ptr, col_ind, grad_out, grad_row, grad_col);
         return fgnn_launch_status("u_add_v_bwd_wide_kernel");
     }
-    hipLaunchKernelGGL(u_add_v_bwd_kernel<false>, dim3(waves), dim3(FGNN_TPB), 0, st, N, W, row_ptr, col_ind, grad_out, grad_row, grad_col);
-    rc = fgnn_launch_status("u_add_v_bwd_kernel");
-    if (rc || E * W <= SO_LONG_ELEMS) return rc;
-    hipLaunchKernelGGL(u_add_v_bwd_kernel<true>, dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, W, row_ptr, col_ind, grad_out, grad_row, grad_col);
-    return fgnn_launch_status("u_add_v_bwd_kernel (long rows)");
+    // one float per lane: the atomics of a wave instruction then fall into the fewest cache lines (with four per lane
+    // the pass took three times as long on a 115 M-entry graph)
+    hipLaunchKernelGGL((u_add_v_bwd_kernel<false, 1>), dim3(waves), dim3(FGNN_TPB), 0, st, N, W, row_ptr, col_ind, grad_out, grad_row, grad_col);
+    if (E * W > SO_LONG_ELEMS)
+        hipLaunchKernelGGL((u_add_v_bwd_kernel<true, 1>), dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, W, row_ptr, col_ind, grad_out, grad_row, grad_col);
+    return fgnn_launch_status("u_add_v_bwd_kernel");
 }
 
 // ------------------------------------------------------------------------------- per-edge Linear(2, D) + tanh

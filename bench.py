@@ -11,7 +11,7 @@ preprocessing (csr2csc, schedules) is reported separately.  One JSON line is pri
 metric, the roofline record of the dominant kernel and a CPU baseline (the torch-composed DGL-style
 layer of oracle/ on the host cores, on a bounded sample of the same graph).  The default run also
 measures the other benchmark configurations (EdgeConv C3, GMMConv C4, GAT C5 layer 1 and the C5
-training step) and appends them to the same line under "other_configs" (--no-others skips them).
+training step, the small operators at C2) and appends them to the same line under "other_configs" (--no-others skips them).
 
 Roofline record: `achieved` is MEASURED bytes (rocprofv3 FETCH_SIZE + WRITE_SIZE of the entry point's
 kernels, kept in profiles/traffic.json) over the live HIP-event time, `frac` its share of the 8 TB/s HBM
@@ -583,10 +583,57 @@ def run_gather_ceiling(args):
                                         out["c2_graph"]["alg_bytes"], ms, None), "cpu_baseline": None}
 
 
+def run_small_ops(args):
+    """The per-edge operators of the reference's operators/ package on the C2 graph, each timed alone: u_add_v, edge
+    softmax, multi-head SpMM / SDDMM, the permuted row gather, csr2csc.  `bytes` is what one call must move when
+    nothing is reused: every array read or written once, gathered feature rows once per entry."""
+    import torch
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd.operators import csr2csc as csc_op
+    from ae_mlsys_gnn_amd.operators import mhspmm as mh
+    from ae_mlsys_gnn_amd.operators.edge_softmax import edge_softmax_native
+    from ae_mlsys_gnn_amd.operators.u_add_v import u_add_v_native
+    dev = torch.device("cuda:0")
+    n, h, f = 232965, 8, 32
+    g, _, _ = build_gat_graph(n, 114_600_000, dev)
+    e = g.n_edges
+    torch.manual_seed(0)
+    x = torch.randn(n, h, f, device=dev)
+    go = torch.randn(n, h, f, device=dev)
+    ar = torch.randn(n, h, device=dev)
+    ac = torch.randn(n, h, device=dev)
+    ee = u_add_v_native.u_add_v_forward(g.row_ptr, g.col_ind, ar, ac)
+    sm = edge_softmax_native.edge_softmax(g.row_ptr, ee)
+    eh, nh, row = 4 * e * h, 4 * n * h, 4 * h * f
+    ops = (
+        ("u_add_v", "fgnn_u_add_v", eh + 4 * e + 2 * nh, lambda: u_add_v_native.u_add_v_forward(g.row_ptr, g.col_ind, ar, ac)),
+        ("u_add_v_backward", "fgnn_u_add_v_backward", eh + 4 * e + 2 * nh, lambda: u_add_v_native.u_add_v_backward(g.row_ptr, g.col_ind, ee)),
+        ("edge_softmax", "fgnn_edge_softmax", 2 * eh, lambda: edge_softmax_native.edge_softmax(g.row_ptr, ee)),
+        ("edge_softmax_backward", "fgnn_edge_softmax_backward", 3 * eh, lambda: edge_softmax_native.edge_softmax_backward(g.row_ptr, sm, ee)),
+        ("mhspmm", "fgnn_mhspmm", e * (row + 4 + 4 * h) + n * row, lambda: mh.mhspmm(g.row_ptr, g.col_ind, sm, x)),
+        ("mhspmm_transposed", "fgnn_mhspmm (CSC walk, weights through permute)", e * (row + 8 + 4 * h) + n * row,
+         lambda: mh.mhspmm(g.col_ptr, g.row_ind, sm, go, pos_map=g.permute)),
+        ("mhsddmm", "fgnn_mhsddmm", e * (row + 4 + 4 * h) + n * row, lambda: mh.mhsddmm(g.row_ptr, g.col_ind, go, x)),
+        ("mhtranspose", "fgnn_gather_rows", 2 * eh + 4 * e, lambda: mh.mhtranspose(g.permute, sm)),
+        ("csr2csc", "fgnn_csr2csc", 0, lambda: csc_op.csr2csc(g.row_ptr, g.col_ind)),
+    )
+    out = {}
+    for name, entry, nbytes, fn in ops:
+        ms, _, _ = time_calls(fn, min(args.steps, 10), 2)
+        out[name] = {"entry_point": entry, "ms": round(ms, 3)}
+        if nbytes:
+            out[name].update({"bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)})
+    total = sum(v["ms"] for v in out.values())
+    return {"metric": "small per-edge operators on the C2 graph, ms per call, 1 MI355X", "value": round(total, 3), "unit": "ms (sum over the operators)",
+            "n_gpus": 1, "steps": min(args.steps, 10), "warmup": 2, "ms_per_step": round(total, 3), "higher_is_better": False, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "small_ops_c2", "nodes": n, "edges": e, "heads": h, "out_feats": f}, "operators": out, "cpu_baseline": None}
+
+
 def brief(rec):
     """The part of a workload's record that goes under "other_configs" of the default line."""
     keep = ("metric", "value", "unit", "ms_per_step", "config", "roofline", "roofline_bwd", "variants", "stash_variant", "fusescatter_pipeline", "sparse_fwd_bwd",
-            "fused_sum_over_kernels", "hip_graph_replay", "knn_graph_ms", "backward_plain_scatter_us", "cpu_baseline", "peak_hbm_GiB")
+            "operators", "fused_sum_over_kernels", "hip_graph_replay", "knn_graph_ms", "backward_plain_scatter_us", "cpu_baseline", "peak_hbm_GiB")
     return {k: rec[k] for k in keep if k in rec}
 
 
@@ -595,7 +642,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="gat_c2", choices=["gat_c2", "gat_c5", "gat_c5_train", "edgeconv_c3", "gmm_c4", "gather_ceiling"])
+    ap.add_argument("--workload", default="gat_c2", choices=["gat_c2", "gat_c5", "gat_c5_train", "edgeconv_c3", "gmm_c4", "small_ops_c2", "gather_ceiling"])
     ap.add_argument("--no-others", action="store_true", help="gat_c2 only: do not append the other benchmark configurations to the line")
     ap.add_argument("--cpu-sample-edges", type=int, default=1_500_000)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline (profiling runs)")
@@ -628,7 +675,7 @@ def main():
             sub.steps, sub.warmup, sub.no_cpu_baseline = min(args.steps, 10), min(args.warmup, 3), True
             for name, fn in (("edgeconv_c3", lambda: run_edgeconv(args)), ("gmm_c4", lambda: run_gmm(args)),
                              ("gat_c5_layer1", lambda: run_gat(sub, 2449029, 61_900_000, 100, 8, 32, "gat_c5_layer1")),
-                             ("gat_c5_train", lambda: run_gat_train(sub))):
+                             ("gat_c5_train", lambda: run_gat_train(sub)), ("small_ops_c2", lambda: run_small_ops(sub))):
                 gc.collect()
                 _lib.clear_schedule_cache()
                 torch.cuda.empty_cache()
@@ -642,6 +689,8 @@ def main():
             rec["other_configs"] = others
     elif args.workload == "gather_ceiling":
         rec = run_gather_ceiling(args)
+    elif args.workload == "small_ops_c2":
+        rec = run_small_ops(args)
     elif args.workload == "gat_c5":
         rec = run_gat(args, 2449029, 61_900_000, 100, 8, 32, "gat_c5_layer1")
     elif args.workload == "gat_c5_train":

@@ -575,6 +575,21 @@ def run_gather_ceiling(args):
         del g, x, ci
         _lib.clear_schedule_cache()
         torch.cuda.empty_cache()
+    # what plain streaming kernels of the installed libraries reach on this part (no gather at all): the practical
+    # ceiling next to the published 8 TB/s
+    stream = {}
+    for mib in (256, 4096):
+        nel = mib * 1024 * 1024 // 4
+        a = torch.randn(nel, device=dev)
+        b = torch.empty_like(a)
+        for name, nbytes, fn in (("copy", 8 * nel, lambda: b.copy_(a)), ("scale (read + write)", 8 * nel, lambda: torch.mul(a, 2.0, out=b)),
+                                 ("fill", 4 * nel, lambda: b.zero_()), ("sum (read only)", 4 * nel, lambda: a.sum())):
+            t, _, _ = time_calls(fn, args.steps, 3)
+            stream["%s, %d MiB arrays" % (name, mib)] = {"ms": round(t, 4), "GBps": round(nbytes / t / 1e6, 1),
+                                                         "frac_of_hbm_peak": round(nbytes / t / 1e6 / HBM_PEAK_GBPS, 4)}
+        del a, b
+        torch.cuda.empty_cache()
+    out["library_streaming_kernels"] = stream
     ms = out["c2_graph"]["uniform_random_sources"]["ms"]
     return {"metric": "bare 1 KiB feature-row gather (unweighted SpMM) ms + GB/s, 1 MI355X", "value": ms, "unit": "ms/iter", "n_gpus": 1,
             "steps": args.steps, "warmup": 2, "ms_per_step": ms, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,

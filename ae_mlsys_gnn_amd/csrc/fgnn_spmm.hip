@@ -12,6 +12,7 @@ struct SpmmP {
     int N, H, F, HF;
     int sum_h;      // != 0: out is [N,F], the sum over the H heads (GMMConv's .sum(1) fused into the store)
     const float *bias; const float *res;     // with sum_h: out[i,:] += bias[:] (+ res[i,:]) in the same store (either may be NULL)
+    int own_order;  // != 0: per-edge arrays are indexed by the work list's own entry positions (pos is not applied)
 };
 __host__ __device__ static inline int spmm_pw(int HF) { return (HF + 3) & ~3; }
 
@@ -239,7 +240,7 @@ static int spmm_launch(const char *name, SpmmP p, WF wf, int shared_floats, cons
     p.items = sched ? sched->items_dev : nullptr;
     p.n_items = sched ? sched->n_items : p.N;
     p.idx = fgnn_sched_idx(sched, p.idx);
-    p.pos = fgnn_sched_pos(sched);
+    p.pos = p.own_order ? nullptr : fgnn_sched_pos(sched);
     p.part = (float *)workspace;
     if (sched && sched->n_partials > 0) {
         size_t need = (size_t)sched->n_partials * spmm_pw(p.HF) * sizeof(float);
@@ -267,9 +268,43 @@ static int spmm_launch(const char *name, SpmmP p, WF wf, int shared_floats, cons
     });
 }
 
+static size_t spmm_partial_bytes(const fgnn_schedule_t *sched, int H, int F)
+{
+    return sched ? (((size_t)sched->n_partials * spmm_pw(H * F) * sizeof(float) + 255) & ~(size_t)255) : 0;
+}
+
 extern "C" size_t fgnn_mhspmm_workspace_bytes(const fgnn_schedule_t *sched, int H, int F)
 {
-    return sched ? (size_t)sched->n_partials * spmm_pw(H * F) * sizeof(float) : 0;
+    // partial results of the split rows, and for an XCD-aware work list room for the weights in the list's entry order
+    size_t own = (sched && sched->n_buckets > 0 && sched->bpos_dev) ? (size_t)sched->n_edges * H * sizeof(float) : 0;
+    return spmm_partial_bytes(sched, H, F) + own;
+}
+
+// own[q, :] = att[map(pos[q]), :]: the per-edge weights copied into the entry order of an XCD-aware work list, so that the
+// gather pass streams them.  Read through `pos` inside that pass, the eight source buckets of a row are eight workgroups on
+// eight XCDs that each pull every 128-byte line of the row's weights for a quarter of its bytes (measured at 115 M edges,
+// 8 heads: 70.6 GB moved, 35 GB of it weights, 11.2 ms; the bare gather moves 39 GB in 5.6 ms).  Here a workgroup takes a
+// run of ATT_RUN consecutive entries and workgroup w the run (w mod 8) * runs_per_xcd + w / 8: an XCD works through one
+// contiguous eighth of the list, so the bucket runs of a row follow each other on the same L2 and its lines are fetched once.
+#define ATT_RUN 2048
+template <int VEC>
+__global__ __launch_bounds__(256) void att_own_order_kernel(int64_t E, int H, int64_t runs_per_xcd, const int *__restrict__ pos,
+                                                            const int *__restrict__ pos_map, const float *__restrict__ att,
+                                                            float *__restrict__ own)
+{
+    const int64_t run = (int64_t)(blockIdx.x % FGNN_NUM_XCD) * runs_per_xcd + blockIdx.x / FGNN_NUM_XCD;
+    const int64_t q0 = run * ATT_RUN;
+    if (blockIdx.x / FGNN_NUM_XCD >= runs_per_xcd || q0 >= E) return;
+    const unsigned uh = (unsigned)H / VEC;                              // groups of VEC floats per entry
+    const unsigned n = (unsigned)(min(q0 + ATT_RUN, E) - q0) * uh;      // groups of this run (< 2^17)
+    for (unsigned k = threadIdx.x; k < n; k += 256) {
+        const unsigned dq = k / uh, g = k - dq * uh;
+        int o = pos[q0 + dq];
+        if (pos_map) o = pos_map[o];
+        fg_vec<VEC> v;
+        v.load(att + ((size_t)(unsigned)o * uh + g) * VEC);
+        v.store_nt(own + ((size_t)(q0 + dq) * uh + g) * VEC);
+    }
 }
 
 extern "C" int fgnn_mhspmm(int N, int64_t E, int H, int F, const int32_t *ptr, const int32_t *idx, const int32_t *pos_map,
@@ -282,12 +317,28 @@ extern "C" int fgnn_mhspmm(int N, int64_t E, int H, int F, const int32_t *ptr, c
     SpmmP p{};
     p.ptr = ptr; p.idx = idx; p.pos_map = pos_map; p.feat = feat; p.out = out; p.N = N; p.H = H; p.F = F; p.HF = H * F;
     WAtt wf{att};
-    return spmm_launch("fgnn_mhspmm", p, wf, 0, sched, fgnn_aligned16(feat) && fgnn_aligned16(out), workspace, workspace_bytes, (hipStream_t)stream);
+    hipStream_t st = (hipStream_t)stream;
+    const size_t part_bytes = spmm_partial_bytes(sched, H, F), own_bytes = (size_t)E * H * sizeof(float);
+    if (att && E > 0 && sched && sched->n_buckets > 0 && sched->bpos_dev && workspace && workspace_bytes >= part_bytes + own_bytes) {
+        float *own = (float *)((char *)workspace + part_bytes);
+        const int64_t runs = (E + ATT_RUN - 1) / ATT_RUN, runs_per_xcd = (runs + FGNN_NUM_XCD - 1) / FGNN_NUM_XCD;
+        const dim3 grid((unsigned)(runs_per_xcd * FGNN_NUM_XCD));
+        if (H % 4 == 0 && fgnn_aligned16(att) && fgnn_aligned16(own))
+            hipLaunchKernelGGL(att_own_order_kernel<4>, grid, dim3(256), 0, st, E, H, runs_per_xcd, sched->bpos_dev, pos_map, att, own);
+        else
+            hipLaunchKernelGGL(att_own_order_kernel<1>, grid, dim3(256), 0, st, E, H, runs_per_xcd, sched->bpos_dev, pos_map, att, own);
+        rc = fgnn_launch_status("att_own_order_kernel");
+        if (rc) return rc;
+        wf.att = own;
+        p.pos_map = nullptr;
+        p.own_order = 1;            // the weights are indexed by the list's own entry positions
+    }
+    return spmm_launch("fgnn_mhspmm", p, wf, 0, sched, fgnn_aligned16(feat) && fgnn_aligned16(out), workspace, workspace_bytes, st);
 }
 
 extern "C" size_t fgnn_gmm_forward_workspace_bytes(const fgnn_schedule_t *sched, int K, int F)
 {
-    return fgnn_mhspmm_workspace_bytes(sched, K, F);
+    return spmm_partial_bytes(sched, K, F);
 }
 
 static int gmm_forward_shared(int N, int K, int dim, int F, const int32_t *ptr, const int32_t *idx, const int32_t *pos_map, const float *feat,

@@ -23,7 +23,9 @@ def mhspmm(ptr_arr, idx, attention, feat, pos_map=None):
     out = torch.empty((ptr_arr.numel() - 1, h, f), dtype=torch.float32, device=feat.device)
     sched = schedule_for(ptr_arr, idx_tensor=idx)
     with torch.cuda.device(feat.device):
-        ws, wsb = workspace(lib().fgnn_mhspmm_workspace_bytes(sched.handle, h, f), feat.device)
+        # unweighted: only the partial results of split rows (the same figure as the GMMConv forward's)
+        need = (lib().fgnn_mhspmm_workspace_bytes if attention is not None else lib().fgnn_gmm_forward_workspace_bytes)(sched.handle, h, f)
+        ws, wsb = workspace(need, feat.device)
         check(lib().fgnn_mhspmm(ptr_arr.numel() - 1, e, h, f, ptr(ptr_arr), ptr(idx), ptr(pos_map), ptr(attention), ptr(feat),
                                 ptr(out), sched.handle, ptr(ws), wsb, stream_ptr()), "fgnn_mhspmm")
     return out

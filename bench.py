@@ -333,8 +333,9 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
         "fusescatter_pipeline": {"fwd_bwd_ms": round(ms_pipe, 4), "peak_hbm_GiB": round(pipe_peak, 3),
                                  "what": "the reference's fuse-scatter ablation composed from u_add_v, edge softmax and mhspmm"},
         "sparse_fwd_bwd": {"ms": round(ms_fwd + ms_bwd, 4), "alg_bytes": b_fwd + b_bwd,
-                           "achieved_GBps": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6, 1),
-                           "frac_of_peak": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6 / HBM_PEAK_GBPS, 4)},
+                           "effective_gather_GBps": round((b_fwd + b_bwd) / (ms_fwd + ms_bwd) / 1e6, 1),
+                           "measured_GBps": (round((traffic["fwd"] + traffic["bwd"]) / (ms_fwd + ms_bwd) / 1e6, 1)
+                                             if traffic and "fwd" in traffic and "bwd" in traffic else None)},
         "cpu_baseline": None if args.no_cpu_baseline else {
             "value": round(cpu_ms * e / cpu_e, 1), "unit": "ms/iter", "cores": cores, "kind": "port",
             "sample": "DGL-composed GAT layer (torch CPU, %d threads) fwd+bwd on a seeded random sample of %d destination rows = %d edges of the "

@@ -65,6 +65,7 @@ _SIGNATURES = {
     "fgnn_mhspmm_workspace_bytes": (c_size_t, [c_void_p, c_int, c_int]),
     "fgnn_mhspmm": (c_int, [c_int, c_int64, c_int, c_int] + [c_void_p] * 6 + [c_void_p, c_void_p, c_size_t, c_void_p]),
     "fgnn_mhsddmm": (c_int, [c_int, c_int64, c_int, c_int] + [c_void_p] * 5 + [c_void_p]),
+    "fgnn_mhsddmm_scheduled": (c_int, [c_int, c_int64, c_int, c_int] + [c_void_p] * 5 + [c_void_p, c_void_p]),
     "fgnn_sddmm_coo": (c_int, [c_int64, c_int, c_int, c_int, c_int] + [c_void_p] * 5 + [c_void_p]),
     "fgnn_gather_rows": (c_int, [c_int64, c_int] + [c_void_p] * 3 + [c_void_p]),
     "fgnn_edge_softmax": (c_int, [c_int, c_int64, c_int] + [c_void_p] * 3 + [c_void_p]),

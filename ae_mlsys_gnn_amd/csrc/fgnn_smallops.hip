@@ -16,9 +16,55 @@ __device__ __forceinline__ int so_row_of(const int *__restrict__ ptr, int lo, in
 }
 
 // out[p,h] = <a[row,h,:], b[col_ind[p],h,:]> (src/sddmm/mhsddmm.cu:5-81 of the reference, which
-// finds the row of each edge by binary search).  One wave per SDDMM_CHUNK consecutive CSR positions:
-// the row of the first one by bisection, the following rows by walking row_ptr, so a hub row is
-// shared by as many waves as it has chunks and the a-row is loaded once per (wave, row).
+// finds the row of each edge by binary search).  The entries [pb, pe) of one row, 64 at a time, four gathered
+// b-rows in flight; pos (NULL = identity) maps an entry to the position its result is stored at.
+template <int VEC, int R, bool FULL, int LPH>
+__device__ __forceinline__ void sddmm_row_piece(int row, int pb, int pe, int H, int F, int HF, const fg_lanemap<VEC, R> &lm, int lane, float *scr,
+                                                const int *__restrict__ idx, const int *__restrict__ pos, const float *__restrict__ a,
+                                                const float *__restrict__ b, float *__restrict__ out)
+{
+    fg_vec<VEC> ar[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ar[r].load(a + (size_t)row * HF + lm.eoff[r]); else ar[r].zero(); }
+    for (int c = pb; c < pe; c += 64) {
+        const int q = c + lane;
+        const int cnt = min(64, pe - c);
+        const int qq = q < pe ? q : c;
+        const int id = idx[qq];
+        const int pv = pos ? pos[qq] : qq;
+        for (int t = 0; t < cnt; t += 4) {
+            fg_vec<VEC> ld[4][R];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                int j = __builtin_amdgcn_readlane(id, (t + u) & 63);
+#pragma unroll
+                for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ld[u][r].load(b + (size_t)j * HF + lm.eoff[r]); else ld[u][r].zero(); }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (t + u >= cnt) break;
+                float d[R];
+#pragma unroll
+                for (int r = 0; r < R; ++r) d[r] = ld[u][r].dot(ar[r]);
+                const size_t o = (size_t)(unsigned)__builtin_amdgcn_readlane(pv, (t + u) & 63) * H;
+                if constexpr (LPH > 0) {
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        float s = fg_group_sum<LPH>(d[r]);
+                        if ((FULL || lm.ok[r]) && lm.eoff[r] % F == 0) out[o + lm.hd[r]] = s;
+                    }
+                } else {
+                    float s = H <= FGNN_FEW_HEADS ? fg_head_reduce_few<VEC, R>(d, lm, lane, H) : fg_head_reduce<VEC, R>(scr, d, lm, lane, H, F);
+                    if (lane < H) out[o + lane] = s;
+                }
+            }
+        }
+    }
+}
+
+// Without a work list: one wave per SDDMM_CHUNK consecutive CSR positions, the row of the first one by
+// bisection, the following rows by walking row_ptr, so a hub row is shared by as many waves as it has chunks
+// and the a-row is loaded once per (wave, row).
 #define SDDMM_CHUNK 256
 template <int VEC, int R, bool FULL, int LPH>
 __global__ __launch_bounds__(FGNN_TPB) void mhsddmm_kernel(int N, int64_t E, int H, int F, int HF, int lphp, const int *ptr, const int *idx,
@@ -36,72 +82,77 @@ __global__ __launch_bounds__(FGNN_TPB) void mhsddmm_kernel(int N, int64_t E, int
     int pb = fg_uni((int)c0);
     while (pb < c1 && row < N) {                             // ptr[N] = E >= c1 keeps row < N on a consistent graph
         const int pe = min(fg_uni(ptr[row + 1]), c1);
-        if (pe > pb) {
-            fg_vec<VEC> ar[R];
-#pragma unroll
-            for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ar[r].load(a + (size_t)row * HF + lm.eoff[r]); else ar[r].zero(); }
-            for (int c = pb; c < pe; c += 64) {
-                int q = c + lane;
-                int cnt = min(64, pe - c);
-                int id = idx[q < pe ? q : c];
-                for (int t = 0; t < cnt; t += 4) {
-                    fg_vec<VEC> ld[4][R];
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        int j = __builtin_amdgcn_readlane(id, (t + u) & 63);
-#pragma unroll
-                        for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ld[u][r].load(b + (size_t)j * HF + lm.eoff[r]); else ld[u][r].zero(); }
-                    }
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        if (t + u >= cnt) break;
-                        float d[R];
-#pragma unroll
-                        for (int r = 0; r < R; ++r) d[r] = ld[u][r].dot(ar[r]);
-                        size_t o = (size_t)(c + t + u) * H;
-                        if constexpr (LPH > 0) {
-#pragma unroll
-                            for (int r = 0; r < R; ++r) {
-                                float s = fg_group_sum<LPH>(d[r]);
-                                if ((FULL || lm.ok[r]) && lm.eoff[r] % F == 0) out[o + lm.hd[r]] = s;
-                            }
-                        } else {
-                            float s = H <= FGNN_FEW_HEADS ? fg_head_reduce_few<VEC, R>(d, lm, lane, H) : fg_head_reduce<VEC, R>(scr, d, lm, lane, H, F);
-                            if (lane < H) out[o + lane] = s;
-                        }
-                    }
-                }
-            }
-        }
+        if (pe > pb) sddmm_row_piece<VEC, R, FULL, LPH>(row, pb, pe, H, F, HF, lm, lane, scr, idx, nullptr, a, b, out);
         pb = pe;
         ++row;
     }
 }
 
-extern "C" int fgnn_mhsddmm(int N, int64_t E, int H, int F, const int32_t *row_ptr, const int32_t *col_ind, const float *a,
-                            const float *b, float *out, void *stream)
+// Under a work list (one wave per item; an XCD-aware list keeps each XCD on one eighth of the gathered b-rows):
+// the entries are walked in the list's order and every result goes to its caller's position.
+template <int VEC, int R, bool FULL, int LPH>
+__global__ __launch_bounds__(FGNN_TPB) void mhsddmm_items_kernel(const fgnn_item *items, int n_items, int H, int F, int HF, int lphp, const int *ptr,
+                                                                 const int *idx, const int *pos, const float *a, const float *b, float *out)
 {
-    FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1 && F >= 1, FGNN_ERR_SHAPE, "fgnn_mhsddmm: bad sizes");
-    FGNN_REQUIRE(H <= 64 && (int64_t)H * F <= 1024, FGNN_ERR_LIMIT, "fgnn_mhsddmm: H=%d H*F=%lld unsupported", H, (long long)H * F);
-    FGNN_REQUIRE(row_ptr && (col_ind || E == 0) && a && b && (out || E == 0), FGNN_ERR_NULL, "fgnn_mhsddmm: NULL argument");
+    extern __shared__ float lds[];
+    int row, pb, pe, slot;
+    if (!fg_get_item(items, n_items, ptr, row, pb, pe, slot)) return;
+    const int lane = fg_lane();
+    float *scr = lds + fg_wave() * (64 * R);
+    fg_lanemap<VEC, R> lm;
+    if (lphp) lm.init_padded(lane, H, F, lphp); else lm.init(lane, HF, F);
+    sddmm_row_piece<VEC, R, FULL, LPH>(row, pb, pe, H, F, HF, lm, lane, scr, idx, pos, a, b, out);
+}
+
+static int mhsddmm_run(const char *fn, int N, int64_t E, int H, int F, const int32_t *row_ptr, const int32_t *col_ind, const float *a,
+                       const float *b, float *out, const fgnn_schedule_t *sched, hipStream_t st)
+{
+    FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1 && F >= 1, FGNN_ERR_SHAPE, "%s: bad sizes", fn);
+    FGNN_REQUIRE(H <= 64 && (int64_t)H * F <= 1024, FGNN_ERR_LIMIT, "%s: H=%d H*F=%lld unsupported", fn, H, (long long)H * F);
+    FGNN_REQUIRE(row_ptr && (col_ind || E == 0) && a && b && (out || E == 0), FGNN_ERR_NULL, "%s: NULL argument", fn);
+    FGNN_REQUIRE(E <= 2147483647LL, FGNN_ERR_LIMIT, "%s: E=%lld exceeds the 32-bit row_ptr", fn, (long long)E);
+    if (sched) {
+        FGNN_REQUIRE(sched->ptr_dev == row_ptr && sched->n_rows == N && sched->n_edges == E, FGNN_ERR_SCHEDULE,
+                     "%s: schedule was built for another pointer array", fn);
+        FGNN_REQUIRE(sched->n_buckets == 0 || sched->idx_src_dev == col_ind, FGNN_ERR_SCHEDULE,
+                     "%s: XCD-aware schedule was built from another index array", fn);
+        FGNN_REQUIRE(fgnn_sched_has_pos(sched) && !sched->own_order, FGNN_ERR_SCHEDULE,
+                     "%s: the schedule must carry its edge positions (results are stored at the caller's positions)", fn);
+    }
     if (N == 0 || E == 0) return 0;
     const int HF = H * F;
     fgnn_rowcfg cfg;
-    FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, fgnn_aligned16(a) && fgnn_aligned16(b), &cfg), FGNN_ERR_LIMIT, "fgnn_mhsddmm: unsupported row width %d", HF);
+    FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, fgnn_aligned16(a) && fgnn_aligned16(b), &cfg), FGNN_ERR_LIMIT, "%s: unsupported row width %d", fn, HF);
     const int lphp = fgnn_pad_lph(cfg.vec, H, F);
     if (lphp) { int w = H * lphp * 4; cfg.r = w <= 256 ? 1 : w <= 512 ? 2 : 4; cfg.full = false; }
     const int lph = lphp ? lphp : fgnn_pick_lph(cfg.vec, F);
-    FGNN_REQUIRE(E <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_mhsddmm: E=%lld exceeds the 32-bit row_ptr", (long long)E);
-    const int64_t waves = (E + SDDMM_CHUNK - 1) / SDDMM_CHUNK;
+    const int64_t waves = sched ? sched->n_items : (E + SDDMM_CHUNK - 1) / SDDMM_CHUNK;
+    if (waves == 0) return 0;
     const unsigned grid = (unsigned)((waves + FGNN_WPB - 1) / FGNN_WPB);
-    hipStream_t st = (hipStream_t)stream;
     return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
         return fgnn_dispatch_lph(VEC == 4 ? lph : 0, [&]<int LPH>() -> int {
-            hipLaunchKernelGGL((mhsddmm_kernel<VEC, R, FULL, (VEC == 4 ? LPH : 0)>), dim3(grid), dim3(FGNN_TPB),
-                               (size_t)FGNN_WPB * 64 * R * sizeof(float), st, N, E, H, F, HF, lphp, row_ptr, col_ind, a, b, out);
+            const size_t shm = (size_t)FGNN_WPB * 64 * R * sizeof(float);
+            if (sched)
+                hipLaunchKernelGGL((mhsddmm_items_kernel<VEC, R, FULL, (VEC == 4 ? LPH : 0)>), dim3(grid), dim3(FGNN_TPB), shm, st, sched->items_dev,
+                                   sched->n_items, H, F, HF, lphp, row_ptr, fgnn_sched_idx(sched, col_ind), fgnn_sched_pos(sched), a, b, out);
+            else
+                hipLaunchKernelGGL((mhsddmm_kernel<VEC, R, FULL, (VEC == 4 ? LPH : 0)>), dim3(grid), dim3(FGNN_TPB), shm, st, N, E, H, F, HF, lphp,
+                                   row_ptr, col_ind, a, b, out);
             return fgnn_launch_status("mhsddmm_kernel");
         });
     });
+}
+
+extern "C" int fgnn_mhsddmm(int N, int64_t E, int H, int F, const int32_t *row_ptr, const int32_t *col_ind, const float *a,
+                            const float *b, float *out, void *stream)
+{
+    return mhsddmm_run("fgnn_mhsddmm", N, E, H, F, row_ptr, col_ind, a, b, out, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int fgnn_mhsddmm_scheduled(int N, int64_t E, int H, int F, const int32_t *row_ptr, const int32_t *col_ind, const float *a,
+                                      const float *b, float *out, const fgnn_schedule_t *sched, void *stream)
+{
+    return mhsddmm_run("fgnn_mhsddmm_scheduled", N, E, H, F, row_ptr, col_ind, a, b, out, sched, (hipStream_t)stream);
 }
 
 // out[e,h] = <a[row_ind[e],h,:], b[col_ind[e],h,:]> for an edge list (sddmm.coo_sddmm of the

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from .._lib import FgnnError, as_f32, as_i32, check, lib, ptr, require_cuda, schedule_for, stream_ptr, workspace
+from .._lib import FgnnError, as_f32, as_i32, check, lib, ptr, require_cuda, schedule_for, stream_ptr, workspace, xcd_buckets_enabled
 
 
 def mhspmm(ptr_arr, idx, attention, feat, pos_map=None):
@@ -38,9 +38,16 @@ def mhsddmm(rowptr, colind, grad, feat):
     n, h, f = feat.shape
     e = colind.numel()
     out = torch.empty((e, h), dtype=torch.float32, device=feat.device)
+    # a skewed graph is walked under its XCD-aware work list (each XCD then gathers from one eighth of the feature
+    # rows); otherwise the kernel cuts the entry array into equal chunks itself and needs no list
+    sched = schedule_for(rowptr, idx_tensor=colind) if e and xcd_buckets_enabled(rowptr, e) else None
     with torch.cuda.device(feat.device):
-        check(lib().fgnn_mhsddmm(rowptr.numel() - 1, e, h, f, ptr(rowptr), ptr(colind), ptr(grad), ptr(feat), ptr(out), stream_ptr()),
-              "fgnn_mhsddmm")
+        if sched is not None:
+            check(lib().fgnn_mhsddmm_scheduled(rowptr.numel() - 1, e, h, f, ptr(rowptr), ptr(colind), ptr(grad), ptr(feat), ptr(out),
+                                               sched.handle, stream_ptr()), "fgnn_mhsddmm_scheduled")
+        else:
+            check(lib().fgnn_mhsddmm(rowptr.numel() - 1, e, h, f, ptr(rowptr), ptr(colind), ptr(grad), ptr(feat), ptr(out), stream_ptr()),
+                  "fgnn_mhsddmm")
     return out
 
 

@@ -299,6 +299,12 @@ int    fgnn_mhspmm(int N, int64_t E, int H, int F, const int32_t *ptr, const int
  * (src/sddmm/sddmm.cpp): out[p,h] = <a[row(p),h,:], b[col_ind[p],h,:]>. */
 int    fgnn_mhsddmm(int N, int64_t E, int H, int F, const int32_t *row_ptr, const int32_t *col_ind,
                     const float *a, const float *b, float *out, void *stream);
+/* The same operator walked under a work list of (row_ptr, col_ind) that carries its edge positions (NULL = the
+ * call above): with an XCD-aware list every XCD gathers from one eighth of the b-rows; results are stored at the
+ * caller's CSR positions either way. */
+int    fgnn_mhsddmm_scheduled(int N, int64_t E, int H, int F, const int32_t *row_ptr, const int32_t *col_ind,
+                              const float *a, const float *b, float *out, const fgnn_schedule_t *sched,
+                              void *stream);
 /* sddmm.coo_sddmm (src/sddmm/sddmm.cpp:12-27), with heads: out[e,h] = <a[row_ind[e],h,:],
  * b[col_ind[e],h,:]> for an edge list; a is [n_rows,H,F], b is [n_cols,H,F].  Indices are not
  * range-checked on the device. */

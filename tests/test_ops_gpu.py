@@ -661,6 +661,12 @@ def test_mhspmm_and_gmm_with_xcd_buckets(monkeypatch):
         _lib.check(_lib.lib().fgnn_mhspmm(g.n, g.n_edges, 4, 16, _lib.ptr(ptr_arr), _lib.ptr(idx), _lib.ptr(pm), _lib.ptr(ad.detach()),
                                            _lib.ptr(fd.detach()), _lib.ptr(in_place), sc.handle, _lib.ptr(ws), wsb, _lib.stream_ptr()), "fgnn_mhspmm")
         assert torch.equal(copied, in_place)
+    # the SDDMM under the work list against the list-free kernel: the same dot product per entry, stored at the same place
+    sd = op.mhsddmm(gd.row_ptr, gd.col_ind, go.float().to(DEV), fd.detach())
+    plain = torch.empty_like(sd)
+    _lib.check(_lib.lib().fgnn_mhsddmm(g.n, g.n_edges, 4, 16, _lib.ptr(gd.row_ptr), _lib.ptr(gd.col_ind), _lib.ptr(go.float().to(DEV).contiguous()),
+                                        _lib.ptr(fd.detach()), _lib.ptr(plain), _lib.stream_ptr()), "fgnn_mhsddmm")
+    assert torch.equal(sd, plain)
     for (k, dim, f) in [(3, 2, 64), (2, 1, 16)]:            # a full-width row and one narrower than a wave
         x, pseudo, mu, isg, go = _gmm_case(g, k, dim, f, seed=2)
         leaves = [t.clone().requires_grad_(True) for t in (x, pseudo, mu, isg)]

@@ -63,3 +63,47 @@ def test_malformed_pointer_arrays_are_refused_by_both_builders(monkeypatch):
             for idx in (None, g.col_ind):
                 with pytest.raises(_lib.FgnnError, match=msg):
                     _lib.Schedule(bad, 0, idx, 16)
+
+
+@pytest.mark.parametrize("name", sorted(GRAPHS))
+def test_row_length_statistics(name):
+    """The two numbers behind the choice of the work list (entries held by rows longer than the limit, the longest row)
+    against torch reductions on the host."""
+    import ctypes
+    from ae_mlsys_gnn_amd import _lib
+    g = GRAPHS[name]()
+    deg = (g.row_ptr[1:] - g.row_ptr[:-1]).long()
+    ptr_dev = g.row_ptr.to(DEV)
+    for limit in (0, 1, 64, 512):
+        stats = (ctypes.c_int64 * 2)()
+        _lib.check(_lib.lib().fgnn_row_length_stats(_lib.ptr(ptr_dev), g.n, limit, ctypes.cast(stats, ctypes.c_void_p), _lib.stream_ptr()),
+                   "fgnn_row_length_stats")
+        assert int(stats[0]) == int(deg[deg > limit].sum()) and int(stats[1]) == int(deg.max() if g.n else 0)
+
+
+def test_scheduled_sddmm_refuses_lists_it_cannot_use(monkeypatch):
+    """fgnn_mhsddmm_scheduled stores its results at the caller's positions: a list of another graph, a list built
+    without the position map and one whose map was handed out are refused before any kernel runs."""
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd._lib import lib, ptr, stream_ptr
+    g = graphs.add_csc_torch(graphs.rmat_graph(500, 20000, seed=1)).to(DEV)
+    other = graphs.rmat_graph(500, 20000, seed=2).to(DEV)
+    n, h, f = g.n, 2, 8
+    a = torch.randn(n, h, f, device=DEV)
+    out = torch.empty(g.n_edges, h, device=DEV)
+
+    def call(sched, graph=g):
+        return lib().fgnn_mhsddmm_scheduled(n, graph.n_edges, h, f, ptr(graph.row_ptr), ptr(graph.col_ind), ptr(a), ptr(a), ptr(out), sched.handle,
+                                            stream_ptr())
+    good = _lib.Schedule(g.row_ptr, 0, g.col_ind, 16, with_positions=True)
+    assert call(good) == 0
+    plain = torch.empty_like(out)
+    _lib.check(lib().fgnn_mhsddmm(n, g.n_edges, h, f, ptr(g.row_ptr), ptr(g.col_ind), ptr(a), ptr(a), ptr(plain), stream_ptr()), "fgnn_mhsddmm")
+    assert torch.equal(out, plain)
+    assert call(_lib.Schedule(other.row_ptr, 0, other.col_ind, 16, with_positions=True)) == -6
+    assert b"another pointer array" in lib().fgnn_last_error()
+    assert call(_lib.Schedule(g.row_ptr, 0, g.col_ind, 16, with_positions=False)) == -6
+    assert b"edge positions" in lib().fgnn_last_error()
+    taken = _lib.Schedule(g.row_ptr, 0, g.col_ind, 16, with_positions=True)
+    taken.take_positions()
+    assert call(taken) == -6 and b"edge positions" in lib().fgnn_last_error()

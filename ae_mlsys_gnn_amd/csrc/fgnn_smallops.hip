@@ -51,11 +51,11 @@ __device__ __forceinline__ void sddmm_row_piece(int row, int pb, int pe, int H, 
 #pragma unroll
                     for (int r = 0; r < R; ++r) {
                         float s = fg_group_sum<LPH>(d[r]);
-                        if ((FULL || lm.ok[r]) && lm.eoff[r] % F == 0) out[o + lm.hd[r]] = s;
+                        if ((FULL || lm.ok[r]) && lm.eoff[r] % F == 0) __builtin_nontemporal_store(s, out + o + lm.hd[r]);
                     }
                 } else {
                     float s = H <= FGNN_FEW_HEADS ? fg_head_reduce_few<VEC, R>(d, lm, lane, H) : fg_head_reduce<VEC, R>(scr, d, lm, lane, H, F);
-                    if (lane < H) out[o + lane] = s;
+                    if (lane < H) __builtin_nontemporal_store(s, out + o + lane);
                 }
             }
         }

@@ -472,12 +472,12 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p)
 #pragma unroll
                     for (int r = 0; r < R; ++r) {
                         float sum = fg_group_sum<LPH>(dpart[r]);
-                        if ((FULL || lm.ok[r]) && lm.eoff[r] % p.F == 0) gdst[lm.hd[r]] = sum * w[r];
+                        if ((FULL || lm.ok[r]) && lm.eoff[r] % p.F == 0) __builtin_nontemporal_store(sum * w[r], gdst + lm.hd[r]);
                     }
                 } else {
                     float sum = K <= FGNN_FEW_HEADS ? fg_head_reduce_few<VEC, R>(dpart, lm, lane, K)
                                                     : fg_head_reduce<VEC, R>(scr, dpart, lm, lane, K, p.F);
-                    if (lane < K) gdst[lane] = sum * wl[lane * 64 + t + u];
+                    if (lane < K) __builtin_nontemporal_store(sum * wl[lane * 64 + t + u], gdst + lane);
                 }
             }
         }

@@ -543,7 +543,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_packed_kernel(GmmBwdP p)
                 const float w = live ? wl[pm.hd * 64 + ei] : 0.f;
                 T.fma(w, ld[u]);
                 const float sum = fg_group_sum<LPH>(ld[u].dot(xr));
-                if (live && writer) p.gww[(size_t)(unsigned)pv[u] * K + pm.hd] = sum * w;
+                if (live && writer) __builtin_nontemporal_store(sum * w, p.gww + (size_t)(unsigned)pv[u] * K + pm.hd);
             }
         }
         fg_wave_lds_sync();
@@ -622,12 +622,12 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_sum_kernel(GmmBwdP p)
                         if constexpr (GWW) {
                             const float sum = fg_group_sum<LPF>(ld[u].dot(xr[k]));
                             if constexpr (LPF >= GMM_SUMK_MAX) mine = sub == k ? sum * w : mine;
-                            else if (ei < cnt && sub == 0) gdst[k] = sum * w;
+                            else if (ei < cnt && sub == 0) __builtin_nontemporal_store(sum * w, gdst + k);
                         }
                     }
                 }
                 // the K values of an edge leave with one store instruction, K adjacent lanes writing K adjacent floats
-                if constexpr (GWW && LPF >= GMM_SUMK_MAX) { if (ei < cnt && sub < K) gdst[sub] = mine; }
+                if constexpr (GWW && LPF >= GMM_SUMK_MAX) { if (ei < cnt && sub < K) __builtin_nontemporal_store(mine, gdst + sub); }
             }
         }
         fg_wave_lds_sync();

@@ -420,6 +420,56 @@ def test_u_add_v(nh):
     assert_close_sum(cd.grad, cl.grad, s_col, "u_add_v grad col")
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_small_operators_on_random_heavy_tailed_graphs(seed):
+    """Random graphs whose row lengths straddle the kernels' thresholds (empty rows, rows of a few entries, rows around
+    8192 / width floats, one row of up to 12 k entries), random widths: edge softmax and u_add_v both ways, and the
+    multi-head SDDMM, against the oracle."""
+    from ae_mlsys_gnn_amd.operators import edge_softmax as es
+    from ae_mlsys_gnn_amd.operators import mhspmm as mh
+    from ae_mlsys_gnn_amd.operators import u_add_v as uav
+    rng = np.random.default_rng(1000 + seed)
+    n = int(rng.integers(1, 300))
+    w = int(rng.choice([1, 2, 4, 5, 8, 16, 24, 64]))
+    edge = 8192 // w
+    degs = rng.choice([0, 1, 3, 17, 64, edge - 1, edge, edge + 1, 2 * edge + 3], size=n, p=[.2, .2, .2, .15, .1, .04, .04, .04, .03])
+    degs[int(rng.integers(0, n))] = int(rng.integers(3000, 12000))
+    g = custom_graph([list(rng.integers(0, n, size=int(d))) for d in degs], n)
+    gen = torch.Generator().manual_seed(seed)
+    e = g.n_edges
+    x = torch.randn(e, w, generator=gen, dtype=torch.float64) * 2
+    go = torch.randn(e, w, generator=gen, dtype=torch.float64)
+    xl = x.clone().requires_grad_(True)
+    ref = orc.edge_softmax(g.row_ptr, xl)
+    ref.backward(go)
+    xd = x.float().to(DEV).requires_grad_(True)
+    out = es.csr_edge_softmax(g.row_ptr.to(DEV), xd)
+    out.backward(go.float().to(DEV))
+    c = c_exp(float(x.max() - x.min()))
+    one = torch.ones((), dtype=torch.float64)
+    assert_close_sum(out, ref.detach(), one, "edge_softmax (random graph, width %d)" % w, c=c)
+    dot_abs = orc.segment_sums(g.row_ptr, ref.detach() * go.abs())
+    dst = orc.row_of_edge(g.row_ptr)
+    assert_close_sum(xd.grad, xl.grad, ref.detach() * (go.abs() + dot_abs[dst]), "edge_softmax grad (random graph, width %d)" % w, c=c)
+    rv = torch.randn(n, w, generator=gen, dtype=torch.float64)
+    cv = torch.randn(n, w, generator=gen, dtype=torch.float64)
+    rd, cd = rv.float().to(DEV).requires_grad_(True), cv.float().to(DEV).requires_grad_(True)
+    o2 = uav.u_add_v_op(g.row_ptr.to(DEV), g.col_ind.to(DEV), rd, cd)
+    o2.backward(go.float().to(DEV))
+    assert torch.equal(o2.detach().cpu(), rv.float()[dst] + cv.float()[g.col_ind.long()])
+    _, (s_row, s_col) = orc.multilinear_abs_sums(lambda a, b: orc.u_add_v(g.row_ptr, g.col_ind, a, b), (rv, cv), go)
+    gl = [t.clone().requires_grad_(True) for t in (rv, cv)]
+    orc.u_add_v(g.row_ptr, g.col_ind, *gl).backward(go)
+    assert_close_sum(rd.grad, gl[0].grad, s_row, "u_add_v grad row (random graph)")
+    assert_close_sum(cd.grad, gl[1].grad, s_col, "u_add_v grad col (random graph)")
+    h, f = (w, 8) if w <= 16 else (4, 16)
+    a = torch.randn(n, h, f, generator=gen, dtype=torch.float64)
+    b = torch.randn(n, h, f, generator=gen, dtype=torch.float64)
+    sd = mh.mhsddmm(g.row_ptr.to(DEV), g.col_ind.to(DEV), a.float().to(DEV), b.float().to(DEV))
+    assert_close_sum(sd, orc.edge_dots(dst, g.col_ind.long(), a, b), orc.edge_dots(dst, g.col_ind.long(), a, b, absolute=True),
+                     "mhsddmm (random graph)")
+
+
 @pytest.mark.parametrize("weighted,sym", [(True, False), (False, False), (True, True)])
 def test_csrspmm(weighted, sym):
     from ae_mlsys_gnn_amd.operators import spmm as op

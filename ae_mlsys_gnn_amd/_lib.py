@@ -5,7 +5,9 @@ from __future__ import annotations
 
 import collections
 import ctypes
+import functools
 import os
+import threading
 from ctypes import c_float, c_int, c_int64, c_size_t, c_void_p
 
 import torch
@@ -72,6 +74,16 @@ _SIGNATURES = {
     "fgnn_edge_softmax_backward": (c_int, [c_int, c_int64, c_int] + [c_void_p] * 4 + [c_void_p]),
     "fgnn_u_add_v": (c_int, [c_int, c_int64, c_int] + [c_void_p] * 5 + [c_void_p]),
     "fgnn_u_add_v_backward": (c_int, [c_int, c_int64, c_int] + [c_void_p] * 5 + [c_void_p]),
+    "fgnn_colsum_plan_create": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_int, c_int, c_void_p, ctypes.POINTER(c_void_p)]),
+    "fgnn_colsum_plan_destroy": (None, [c_void_p]),
+    "fgnn_colsum_plan_device_bytes": (c_size_t, [c_void_p]),
+    "fgnn_colsum_plan_columns_per_range": (c_int, [c_void_p]),
+    "fgnn_colsum_plan_num_tasks": (c_int, [c_void_p]),
+    "fgnn_colsum_plan_matches": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64]),
+    "fgnn_colsum_workspace_bytes": (c_size_t, [c_void_p, c_int]),
+    "fgnn_edge_colsum": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "fgnn_edge_rowsum": (c_int, [c_int, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "fgnn_u_add_v_backward_planned": (c_int, [c_int, c_int64, c_int] + [c_void_p] * 5 + [c_void_p, c_void_p, c_size_t, c_void_p]),
     "fgnn_edge_linear_tanh": (c_int, [c_int64, c_int] + [c_void_p] * 4 + [c_void_p]),
     "fgnn_edge_linear_tanh_backward_workspace_bytes": (c_size_t, [c_int64, c_int]),
     "fgnn_edge_linear_tanh_backward": (c_int, [c_int64, c_int] + [c_void_p] * 5 + [c_void_p, c_size_t, c_void_p]),
@@ -199,6 +211,17 @@ class Schedule:
 
 _sched_cache: "collections.OrderedDict" = collections.OrderedDict()
 _SCHED_CACHE_MAX = 32
+# The caches below are read and filled by the thread that runs the forward pass and by autograd's backward
+# thread: one re-entrant lock serialises every look-up-then-insert sequence (and the builds inside them).
+_cache_lock = threading.RLock()
+
+
+def _locked(fn):
+    @functools.wraps(fn)
+    def wrapper(*args, **kwargs):
+        with _cache_lock:
+            return fn(*args, **kwargs)
+    return wrapper
 
 
 def default_seg_len() -> int:
@@ -211,6 +234,7 @@ BUCKET_MIN_SHARE = 0.25      # ...and they must hold at least this share of the 
 BUCKET_MIN_SKEW = 4          # longest row / mean row length
 
 
+@_locked
 def xcd_buckets_enabled(ptr_tensor, idx_numel=None) -> bool:
     """Whether operators get the XCD-aware schedule for this pointer array (FGNN_XCD_BUCKETS=0/1
     overrides).  It pays off on skewed graphs, where the rows longer than 64 entries hold a good part
@@ -243,6 +267,7 @@ def xcd_buckets_enabled(ptr_tensor, idx_numel=None) -> bool:
     return hit[0]
 
 
+@_locked
 def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True, own_order=False) -> Schedule:
     """Cached schedule of a pointer array.  The cache entry holds the tensors, so their device
     addresses cannot be reused while the entry lives; in-place edits bump `_version`.
@@ -283,6 +308,7 @@ def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True,
     return s
 
 
+@_locked
 def edge_positions(ptr_tensor, idx_tensor, seg_len=None):
     """Builds (once) the own-order schedule of (ptr, idx) and returns int32 [E]: the caller's position of
     every entry in that schedule's order, or None when the order is the caller's (plain schedule).
@@ -307,15 +333,82 @@ def edge_positions(ptr_tensor, idx_tensor, seg_len=None):
     return pos
 
 
+class ColsumPlan:
+    """Tile-ordered entry list of one (row_ptr, col_ind) pair for atomic-free column sums of per-edge arrays
+    (fgnn_colsum_plan_create).  Built for rows of `width` floats; serves every narrower array."""
+
+    def __init__(self, ptr_tensor, idx_tensor, n_cols, width, lds_bytes=0, task_len=0):
+        require_cuda(ptr_tensor, idx_tensor)
+        self.ptr_tensor = as_i32(ptr_tensor)      # keep the device memory alive
+        self.idx_tensor = as_i32(idx_tensor)
+        self.n_rows = self.ptr_tensor.numel() - 1
+        self.n_cols = int(n_cols)
+        self.width = int(width)
+        handle = c_void_p()
+        with torch.cuda.device(self.ptr_tensor.device):
+            check(lib().fgnn_colsum_plan_create(ptr(self.ptr_tensor), ptr(self.idx_tensor), self.n_rows, self.n_cols, self.idx_tensor.numel(),
+                                                self.width, int(lds_bytes), int(task_len), stream_ptr(), ctypes.byref(handle)),
+                  "fgnn_colsum_plan_create")
+        self.handle = handle
+        self.columns_per_range = lib().fgnn_colsum_plan_columns_per_range(handle)
+        self.n_tasks = lib().fgnn_colsum_plan_num_tasks(handle)
+
+    def device_bytes(self):
+        return int(lib().fgnn_colsum_plan_device_bytes(self.handle))
+
+    def colsum(self, g):
+        """[n_cols, ...] column sums of the per-edge array g [E, ...] (CSR position order)."""
+        require_cuda(g)
+        g = as_f32(g)
+        e = self.idx_tensor.numel()
+        if g.shape[0] != e:
+            raise FgnnError("colsum: the array has %d rows, the plan %d entries" % (g.shape[0], e))
+        w = g.numel() // max(e, 1) if e else int(torch.tensor(g.shape[1:]).prod()) if g.dim() > 1 else 1
+        out = torch.empty((self.n_cols,) + tuple(g.shape[1:]), dtype=torch.float32, device=g.device)
+        with torch.cuda.device(g.device):
+            ws, wsb = workspace(lib().fgnn_colsum_workspace_bytes(self.handle, w), g.device)
+            check(lib().fgnn_edge_colsum(self.handle, w, ptr(g), ptr(out), ptr(ws), wsb, stream_ptr()), "fgnn_edge_colsum")
+        return out
+
+    def __del__(self):
+        h = getattr(self, "handle", None)
+        if h is not None and _lib is not None:
+            _lib.fgnn_colsum_plan_destroy(h)
+            self.handle = None
+
+
+_colsum_cache: "collections.OrderedDict" = collections.OrderedDict()
+_COLSUM_CACHE_MAX = 8
+
+
+def colsum_plan_for(ptr_tensor, idx_tensor, n_cols, width) -> ColsumPlan:
+    """Cached plan of (row_ptr, col_ind); a cached plan built for wider rows is reused.  The entry holds the
+    tensors, so their addresses cannot be reused while it lives; in-place edits bump `_version`."""
+    key = (ptr_tensor.data_ptr(), ptr_tensor.numel(), ptr_tensor._version, idx_tensor.data_ptr(), idx_tensor.numel(), idx_tensor._version,
+           ptr_tensor.device.index, int(n_cols))
+    with _cache_lock:
+        p = _colsum_cache.get(key)
+        if p is None or p.width < width:
+            p = ColsumPlan(ptr_tensor, idx_tensor, n_cols, width)
+            _colsum_cache[key] = p
+        _colsum_cache.move_to_end(key)
+        while len(_colsum_cache) > _COLSUM_CACHE_MAX:
+            _colsum_cache.popitem(last=False)
+        return p
+
+
 def schedule_device_bytes() -> int:
-    """Device memory held by all cached schedules: the library allocates it itself, so torch's
-    max_memory_allocated does not see it and peak-memory reports add it."""
-    return sum(s.device_bytes() for s in _sched_cache.values())
+    """Device memory held by all cached schedules and column-sum plans: the library allocates it itself, so
+    torch's max_memory_allocated does not see it and peak-memory reports add it."""
+    with _cache_lock:
+        return sum(s.device_bytes() for s in _sched_cache.values()) + sum(p.device_bytes() for p in _colsum_cache.values())
 
 
 def clear_schedule_cache():
-    _sched_cache.clear()
-    _bucket_rule_cache.clear()
+    with _cache_lock:
+        _sched_cache.clear()
+        _bucket_rule_cache.clear()
+        _colsum_cache.clear()
 
 
 def workspace(nbytes: int, device):

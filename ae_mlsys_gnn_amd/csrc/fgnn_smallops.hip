@@ -230,14 +230,46 @@ extern "C" int fgnn_sddmm_coo(int64_t E, int n_rows, int n_cols, int H, int F, c
     });
 }
 
-// out[q,:] = in[permute[q],:]  (src/csr2csc/mhtranspose.cu:6-26)
-__global__ __launch_bounds__(256) void gather_rows_kernel(int64_t total, int W, const int *permute, const float *in, float *out)
+// out[q,:] = in[permute[q],:]  (src/csr2csc/mhtranspose.cu:6-47).  A row is G groups of VEC floats (VEC = 4: W % 4 == 0
+// and 16-byte aligned arrays, 128-bit lanes); a wave takes RW consecutive output rows = at most 64 * GR_U groups, lane j of
+// a trip owns group j of that span.  Its row inside the span is j / G by a multiply and a shift (inv = ceil(2^20 / G), exact
+// for j * G < 2^20; spans of one row pass inv = 0), so there is no division per element, and the GR_U loads of a lane are
+// all issued before the first store.
+#define GR_U 8
+template <int VEC>
+__global__ __launch_bounds__(FGNN_TPB) void gather_rows_kernel(int64_t E, int G, int RW, unsigned inv, const int *__restrict__ permute,
+                                                               const float *__restrict__ in, float *__restrict__ out)
 {
-    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= total) return;
-    int64_t q = i / W;
-    int w = (int)(i - q * W);
-    out[i] = in[(size_t)permute[q] * W + w];
+    const int64_t q0 = ((int64_t)blockIdx.x * FGNN_WPB + fg_wave()) * RW;
+    if (q0 >= E) return;
+    const int rows = (int)min((int64_t)RW, E - q0);
+    const int64_t n = (int64_t)rows * G;                 // groups of this wave: <= 64 * GR_U unless RW == 1
+    const int lane = fg_lane();
+    float *dst = out + (size_t)q0 * G * VEC;
+    for (int64_t j0 = 0; j0 < n; j0 += 64 * GR_U) {
+        fg_vec<VEC> v[GR_U];
+        int src[GR_U];
+        unsigned c[GR_U];
+#pragma unroll
+        for (int u = 0; u < GR_U; ++u) {
+            const int64_t j = j0 + 64 * u + lane;
+            const unsigned jj = j < n ? (unsigned)(j & 0x7fffffff) : 0u;       // RW > 1: j < 512
+            const unsigned ql = inv ? (jj * inv) >> 20 : 0u;
+            c[u] = inv ? jj - ql * (unsigned)G : 0u;
+            src[u] = permute[q0 + ql];
+        }
+#pragma unroll
+        for (int u = 0; u < GR_U; ++u) {
+            const int64_t j = j0 + 64 * u + lane;
+            const size_t col = inv ? (size_t)c[u] : (size_t)(j < n ? j : 0);
+            v[u].load(in + ((size_t)src[u] * G + col) * VEC);
+        }
+#pragma unroll
+        for (int u = 0; u < GR_U; ++u) {
+            const int64_t j = j0 + 64 * u + lane;
+            if (j < n) v[u].store_nt(dst + (size_t)j * VEC);
+        }
+    }
 }
 
 extern "C" int fgnn_gather_rows(int64_t E, int W, const int32_t *permute, const float *in, float *out, void *stream)
@@ -245,9 +277,17 @@ extern "C" int fgnn_gather_rows(int64_t E, int W, const int32_t *permute, const 
     FGNN_REQUIRE(E >= 0 && W >= 1, FGNN_ERR_SHAPE, "fgnn_gather_rows: bad sizes");
     FGNN_REQUIRE(E == 0 || (permute && in && out), FGNN_ERR_NULL, "fgnn_gather_rows: NULL argument");
     if (E == 0) return 0;
-    int64_t total = E * W;
-    FGNN_REQUIRE((total + 255) / 256 <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_gather_rows: too many elements");
-    hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, total, W, permute, in, out);
+    const bool vec4 = W % 4 == 0 && fgnn_aligned16(in) && fgnn_aligned16(out);
+    const int G = vec4 ? W / 4 : W;
+    const int RW = G >= 64 * GR_U ? 1 : (64 * GR_U) / G;          // whole rows per wave
+    const unsigned inv = RW > 1 ? (unsigned)(((1u << 20) + (unsigned)G - 1u) / (unsigned)G) : 0u;
+    const int64_t waves = (E + RW - 1) / RW;
+    const int64_t blocks = (waves + FGNN_WPB - 1) / FGNN_WPB;
+    FGNN_REQUIRE(blocks <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_gather_rows: too many rows");
+    if (vec4)
+        hipLaunchKernelGGL(gather_rows_kernel<4>, dim3((unsigned)blocks), dim3(FGNN_TPB), 0, (hipStream_t)stream, E, G, RW, inv, permute, in, out);
+    else
+        hipLaunchKernelGGL(gather_rows_kernel<1>, dim3((unsigned)blocks), dim3(FGNN_TPB), 0, (hipStream_t)stream, E, G, RW, inv, permute, in, out);
     return fgnn_launch_status("gather_rows_kernel");
 }
 
@@ -255,12 +295,18 @@ extern "C" int fgnn_gather_rows(int64_t E, int W, const int32_t *permute, const 
 // A row's entries are one contiguous run of (pe - pb) * W floats.  Lanes t < S0 = (64 / W) * W of a
 // wave take part and stride by a multiple of W, so lane t only ever sees column t % W and every
 // load is a contiguous run of S0 floats.  Rows of up to SO_LONG_ELEMS floats are taken by one wave
-// each (first launch), longer ones by a whole workgroup each (second launch, whose other
-// workgroups leave at once): a 100 k-entry hub row is then a few hundred trips of 512 threads
-// instead of tens of thousands of trips of one wave.
+// each (first launch), longer ones by a whole workgroup each (second launch): a 100 k-entry hub row is
+// then a few hundred trips of 512 threads instead of tens of thousands of trips of one wave.  The second
+// launch has one workgroup per SO_CAND candidate rows: its first wave looks at their lengths, a ballot
+// names the long ones, and the workgroup takes those one after the other (on a 233 k-row power-law graph
+// 31 k rows are long and hold 83 % of the entries; a workgroup per row would start 233 k workgroups of
+// which seven in eight leave at once).
 #define SO_LONG_ELEMS 8192
 #define SO_LONG_TPB 512
-#define SO_CACHE 8            // values per lane kept in registers by the softmax kernels
+#define SO_CAND 16            // candidate rows per workgroup of a long-row launch
+#define SO_CACHE 8            // groups per lane kept in registers by the short-row kernels
+#define SO_STREAM 8           // loads in flight per lane in the part of a row that is streamed
+#define SO_CACHE_LONG 16      // ... by the long-row softmax (512 threads x 16 groups x 4 floats = 4096 entries of 8 heads)
 
 struct so_max { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
 struct so_add { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
@@ -300,23 +346,40 @@ __device__ __forceinline__ so_grp<VEC> so_column_reduce(so_grp<VEC> v, int lane,
     return v;
 }
 
-// The row of this wave (short rows) or workgroup (LONG); false when it belongs to the other launch.  W counts the
-// groups of VEC floats per entry, n the groups of the row.
-// Work unit u (a wave or a workgroup, in launch order) takes row (u * p) mod N with p a prime above 2^31: a
-// bijection of [0, N) that scatters neighbouring rows.  Workgroups go to the eight XCDs round-robin, and on a
+// Work unit u (a wave of the short launch, a candidate of the long launch) takes row (u * p) mod N with p a prime
+// above 2^31: a bijection of [0, N) that scatters neighbouring rows.  Workgroups go to the eight XCDs round-robin, and on a
 // power-law graph generated by recursive quadrants a row's length follows the low bits of its number (the
 // rows = 0 mod 8 of an R-MAT graph hold 44 % of the entries): in row order one XCD would get most of the work.
 __device__ __forceinline__ int so_scattered_row(unsigned u, int N) { return (int)(((unsigned long long)u * 2654435761ull) % (unsigned)N); }
 
-template <bool LONG, int VEC>
-__device__ __forceinline__ bool so_take_row(int N, int W, const int *ptr, int &row, int &pb, int64_t &n)
+// Short launch: the row of this wave, false when it is empty or belongs to the long launch.  W counts the groups of VEC
+// floats per entry, n the groups of the row.
+template <int VEC>
+__device__ __forceinline__ bool so_take_short_row(unsigned u, int N, int W, const int *ptr, int &row, int &pb, int64_t &n)
 {
-    const unsigned u = LONG ? blockIdx.x : (unsigned)fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
     if (u >= (unsigned)N) return false;
     row = fg_uni(so_scattered_row(u, N));
     pb = fg_uni(ptr[row]);
     n = (int64_t)(fg_uni(ptr[row + 1]) - pb) * W;
-    return LONG ? n * VEC > SO_LONG_ELEMS : (n > 0 && n * VEC <= SO_LONG_ELEMS);
+    return n * VEC <= SO_LONG_ELEMS;
+}
+// Long launch: bit l of the result is set when candidate blockIdx.x * SO_CAND + l is a long row (uniform over the workgroup).
+template <int VEC>
+__device__ __forceinline__ unsigned long long so_long_candidates(int N, int W, const int *ptr, unsigned long long *sh_mask)
+{
+    if (fg_wave() == 0) {
+        const unsigned u = blockIdx.x * SO_CAND + (unsigned)fg_lane();
+        bool lng = false;
+        if (fg_lane() < SO_CAND && u < (unsigned)N) {
+            const int r = so_scattered_row(u, N);
+            lng = (int64_t)(ptr[r + 1] - ptr[r]) * W * VEC > SO_LONG_ELEMS;
+        }
+        const unsigned long long m = __builtin_amdgcn_ballot_w64(lng);
+        if (fg_lane() == 0) *sh_mask = m;
+    }
+    __syncthreads();
+    const unsigned long long m = *sh_mask;
+    return ((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane((int)(m >> 32)) << 32) | (unsigned)__builtin_amdgcn_readfirstlane((int)m);
 }
 
 template <int VEC> __device__ __forceinline__ so_grp<VEC> so_load(const float *p)
@@ -341,84 +404,111 @@ template <int VEC> __device__ __forceinline__ so_grp<VEC> so_fill(float x)
 
 // Per-row, per-head softmax over [E,H] (src/edge_softmax/edge_softmax.cu:7-61) and its backward
 // s*(g - sum_row s*g) (:63-98).  VEC = 4 (H % 4 == 0, 16-byte aligned arrays): a lane owns four consecutive
-// heads of an entry; with the eight trips unrolled a hub row keeps 128 bytes per lane in flight.
-template <bool LONG, int VEC>
-__global__ __launch_bounds__(LONG ? SO_LONG_TPB : FGNN_TPB) void edge_softmax_kernel(int N, int W, const int *__restrict__ ptr,
-                                                                                     const float *__restrict__ in, float *__restrict__ out)
+// heads of an entry.  One row: the first CACHE groups of a lane stay in registers over both phases; what a longer
+// row has beyond them is folded into a running (maximum, sum) pair while it streams by (one read instead of a
+// maximum pass and a sum pass) and read once more for the result.
+template <bool LONG, int VEC, int CACHE>
+__device__ __forceinline__ void so_softmax_row(int W, int pb, int64_t n, const float *__restrict__ in, float *__restrict__ out, float (*sh)[64])
 {
-    __shared__ float sh[LONG ? SO_LONG_TPB / 64 : 1][64];
-    int row, pb;
-    int64_t n;
-    if (!so_take_row<LONG, VEC>(N, W, ptr, row, pb, n)) return;      // uniform over the workgroup when LONG
     const int lane = fg_lane(), S0 = (64 / W) * W;
     const int64_t first = (LONG ? fg_wave() * S0 : 0) + lane, step = (int64_t)S0 * (LONG ? SO_LONG_TPB / 64 : 1);
     const bool act = lane < S0;
     const float *src = in + (size_t)pb * W * VEC;
     float *dst = out + (size_t)pb * W * VEC;
-    // the first SO_CACHE groups of a lane stay in registers over the three phases; what a longer row has beyond
-    // them is read again (from the L2, which the first phase has just filled)
-    so_grp<VEC> v[SO_CACHE], m = so_fill<VEC>(-INFINITY), s = so_fill<VEC>(0.f);
+    so_grp<VEC> v[CACHE], m = so_fill<VEC>(-INFINITY), s = so_fill<VEC>(0.f);
 #pragma unroll
-    for (int i = 0; i < SO_CACHE; ++i) {
+    for (int i = 0; i < CACHE; ++i) {
         const int64_t k = first + i * step;
         v[i] = (act && k < n) ? so_load<VEC>(src + k * VEC) : so_fill<VEC>(-INFINITY);
     }
 #pragma unroll
-    for (int i = 0; i < SO_CACHE; ++i)
+    for (int i = 0; i < CACHE; ++i)
 #pragma unroll
         for (int c = 0; c < VEC; ++c) m.c[c] = fmaxf(m.c[c], v[i].c[c]);
-    const int64_t rest = first + SO_CACHE * step;
+    const int64_t rest = first + CACHE * step;
+    // a lane that gets here has CACHE valid groups, so its m is finite and m - max(m, t) is never inf - inf.
+    // SO_STREAM loads are issued before the first is used: a row that one workgroup streams alone is bound by the
+    // bytes it keeps in flight.
     if (act) {
-#pragma unroll 8
-        for (int64_t k = rest; k < n; k += step) {
-            const so_grp<VEC> t = so_load<VEC>(src + k * VEC);
+        for (int64_t k0 = rest; k0 < n; k0 += SO_STREAM * step) {
+            so_grp<VEC> t[SO_STREAM];
 #pragma unroll
-            for (int c = 0; c < VEC; ++c) m.c[c] = fmaxf(m.c[c], t.c[c]);
+            for (int j = 0; j < SO_STREAM; ++j) t[j] = k0 + j * step < n ? so_load<VEC>(src + (k0 + j * step) * VEC) : so_fill<VEC>(-INFINITY);
+            so_grp<VEC> mn = m;
+#pragma unroll
+            for (int j = 0; j < SO_STREAM; ++j)
+#pragma unroll
+                for (int c = 0; c < VEC; ++c) mn.c[c] = fmaxf(mn.c[c], t[j].c[c]);
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) {
+                float acc = s.c[c] * __expf(m.c[c] - mn.c[c]);
+#pragma unroll
+                for (int j = 0; j < SO_STREAM; ++j) acc += __expf(t[j].c[c] - mn.c[c]);       // exp(-inf) = 0 past the row
+                s.c[c] = acc;
+                m.c[c] = mn.c[c];
+            }
         }
     }
-    m = so_column_reduce<LONG, VEC>(m, lane, W, S0, sh, so_max());
+    const so_grp<VEC> mall = so_column_reduce<LONG, VEC>(m, lane, W, S0, sh, so_max());
 #pragma unroll
-    for (int i = 0; i < SO_CACHE; ++i)
+    for (int c = 0; c < VEC; ++c) s.c[c] = s.c[c] > 0.f ? s.c[c] * __expf(m.c[c] - mall.c[c]) : 0.f;      // the streamed part, rebased
 #pragma unroll
-        for (int c = 0; c < VEC; ++c) { v[i].c[c] = __expf(v[i].c[c] - m.c[c]); s.c[c] += v[i].c[c]; }      // exp(-inf) = 0 past the row
-    if (act) {
-#pragma unroll 8
-        for (int64_t k = rest; k < n; k += step) {
-            const so_grp<VEC> t = so_load<VEC>(src + k * VEC);
+    for (int i = 0; i < CACHE; ++i)
 #pragma unroll
-            for (int c = 0; c < VEC; ++c) s.c[c] += __expf(t.c[c] - m.c[c]);
-        }
-    }
+        for (int c = 0; c < VEC; ++c) { v[i].c[c] = __expf(v[i].c[c] - mall.c[c]); s.c[c] += v[i].c[c]; }      // exp(-inf) = 0 past the row
     so_grp<VEC> inv = so_column_reduce<LONG, VEC>(s, lane, W, S0, sh, so_add());
 #pragma unroll
     for (int c = 0; c < VEC; ++c) inv.c[c] = 1.f / inv.c[c];
 #pragma unroll
-    for (int i = 0; i < SO_CACHE; ++i) {
+    for (int i = 0; i < CACHE; ++i) {
         const int64_t k = first + i * step;
 #pragma unroll
         for (int c = 0; c < VEC; ++c) v[i].c[c] *= inv.c[c];
         if (act && k < n) so_store<VEC>(dst + k * VEC, v[i]);
     }
     if (act) {
-#pragma unroll 8
-        for (int64_t k = rest; k < n; k += step) {
-            so_grp<VEC> t = so_load<VEC>(src + k * VEC);
+        for (int64_t k0 = rest; k0 < n; k0 += SO_STREAM * step) {
+            so_grp<VEC> t[SO_STREAM];
 #pragma unroll
-            for (int c = 0; c < VEC; ++c) t.c[c] = __expf(t.c[c] - m.c[c]) * inv.c[c];
-            so_store<VEC>(dst + k * VEC, t);
+            for (int j = 0; j < SO_STREAM; ++j) t[j] = k0 + j * step < n ? so_load<VEC>(src + (k0 + j * step) * VEC) : so_fill<VEC>(0.f);
+#pragma unroll
+            for (int j = 0; j < SO_STREAM; ++j) {
+#pragma unroll
+                for (int c = 0; c < VEC; ++c) t[j].c[c] = __expf(t[j].c[c] - mall.c[c]) * inv.c[c];
+                if (k0 + j * step < n) so_store<VEC>(dst + (k0 + j * step) * VEC, t[j]);
+            }
         }
     }
 }
 
-template <bool LONG, int VEC>
-__global__ __launch_bounds__(LONG ? SO_LONG_TPB : FGNN_TPB) void edge_softmax_bwd_kernel(int N, int W, const int *__restrict__ ptr,
-                                                                                         const float *__restrict__ sm, const float *__restrict__ g,
-                                                                                         float *__restrict__ gin)
+// One launch for both kinds of row: the first n_long_blocks workgroups take the long rows among their SO_CAND candidates
+// (they start first, so the longest rows are not left for the end), the workgroups after them give one short row to each
+// of their eight waves.
+template <int VEC>
+__global__ __launch_bounds__(SO_LONG_TPB) void edge_softmax_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
+                                                                   const float *__restrict__ in, float *__restrict__ out)
 {
-    __shared__ float sh[LONG ? SO_LONG_TPB / 64 : 1][64];
+    __shared__ float sh[SO_LONG_TPB / 64][64];
+    __shared__ unsigned long long sh_mask;
+    if (blockIdx.x < n_long_blocks) {
+        for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
+            const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
+            const int pb = fg_uni(ptr[row]);
+            so_softmax_row<true, VEC, SO_CACHE_LONG>(W, pb, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, in, out, sh);
+        }
+        return;
+    }
     int row, pb;
     int64_t n;
-    if (!so_take_row<LONG, VEC>(N, W, ptr, row, pb, n)) return;
+    const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (SO_LONG_TPB / 64)) + fg_wave());
+    if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n) || n == 0) return;
+    so_softmax_row<false, VEC, SO_CACHE>(W, pb, n, in, out, nullptr);
+}
+
+template <bool LONG, int VEC>
+__device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, const float *__restrict__ sm, const float *__restrict__ g,
+                                                   float *__restrict__ gin, float (*sh)[64])
+{
     const int lane = fg_lane(), S0 = (64 / W) * W;
     const int64_t first = (LONG ? fg_wave() * S0 : 0) + lane, step = (int64_t)S0 * (LONG ? SO_LONG_TPB / 64 : 1);
     const bool act = lane < S0;
@@ -437,11 +527,18 @@ __global__ __launch_bounds__(LONG ? SO_LONG_TPB : FGNN_TPB) void edge_softmax_bw
         for (int c = 0; c < VEC; ++c) acc.c[c] = fmaf(sv[i].c[c], gv[i].c[c], acc.c[c]);
     const int64_t rest = first + SO_CACHE * step;
     if (act) {
-#pragma unroll 4
-        for (int64_t k = rest; k < n; k += step) {
-            const so_grp<VEC> a = so_load<VEC>(sm + base + k * VEC), b = so_load<VEC>(g + base + k * VEC);
+        for (int64_t k0 = rest; k0 < n; k0 += (SO_STREAM / 2) * step) {
+            so_grp<VEC> a[SO_STREAM / 2], b[SO_STREAM / 2];
 #pragma unroll
-            for (int c = 0; c < VEC; ++c) acc.c[c] = fmaf(a.c[c], b.c[c], acc.c[c]);
+            for (int j = 0; j < SO_STREAM / 2; ++j) {
+                const bool ok = k0 + j * step < n;
+                a[j] = ok ? so_load<VEC>(sm + base + (k0 + j * step) * VEC) : so_fill<VEC>(0.f);
+                b[j] = ok ? so_load<VEC>(g + base + (k0 + j * step) * VEC) : so_fill<VEC>(0.f);
+            }
+#pragma unroll
+            for (int j = 0; j < SO_STREAM / 2; ++j)
+#pragma unroll
+                for (int c = 0; c < VEC; ++c) acc.c[c] = fmaf(a[j].c[c], b[j].c[c], acc.c[c]);
         }
     }
     acc = so_column_reduce<LONG, VEC>(acc, lane, W, S0, sh, so_add());
@@ -453,15 +550,44 @@ __global__ __launch_bounds__(LONG ? SO_LONG_TPB : FGNN_TPB) void edge_softmax_bw
         if (act && k < n) so_store<VEC>(gin + base + k * VEC, sv[i]);
     }
     if (act) {
-#pragma unroll 4
-        for (int64_t k = rest; k < n; k += step) {
-            so_grp<VEC> a = so_load<VEC>(sm + base + k * VEC);
-            const so_grp<VEC> b = so_load<VEC>(g + base + k * VEC);
+        for (int64_t k0 = rest; k0 < n; k0 += (SO_STREAM / 2) * step) {
+            so_grp<VEC> a[SO_STREAM / 2], b[SO_STREAM / 2];
 #pragma unroll
-            for (int c = 0; c < VEC; ++c) a.c[c] *= b.c[c] - acc.c[c];
-            so_store<VEC>(gin + base + k * VEC, a);
+            for (int j = 0; j < SO_STREAM / 2; ++j) {
+                const bool ok = k0 + j * step < n;
+                a[j] = ok ? so_load<VEC>(sm + base + (k0 + j * step) * VEC) : so_fill<VEC>(0.f);
+                b[j] = ok ? so_load<VEC>(g + base + (k0 + j * step) * VEC) : so_fill<VEC>(0.f);
+            }
+#pragma unroll
+            for (int j = 0; j < SO_STREAM / 2; ++j) {
+#pragma unroll
+                for (int c = 0; c < VEC; ++c) a[j].c[c] *= b[j].c[c] - acc.c[c];
+                if (k0 + j * step < n) so_store<VEC>(gin + base + (k0 + j * step) * VEC, a[j]);
+            }
         }
     }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(SO_LONG_TPB) void edge_softmax_bwd_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
+                                                                       const float *__restrict__ sm, const float *__restrict__ g,
+                                                                       float *__restrict__ gin)
+{
+    __shared__ float sh[SO_LONG_TPB / 64][64];
+    __shared__ unsigned long long sh_mask;
+    if (blockIdx.x < n_long_blocks) {
+        for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
+            const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
+            const int pb = fg_uni(ptr[row]);
+            so_softmax_bwd_row<true, VEC>(W, pb, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, sm, g, gin, sh);
+        }
+        return;
+    }
+    int row, pb;
+    int64_t n;
+    const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (SO_LONG_TPB / 64)) + fg_wave());
+    if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n) || n == 0) return;
+    so_softmax_bwd_row<false, VEC>(W, pb, n, sm, g, gin, nullptr);
 }
 
 // More than 64 heads: one wave per row, one head at a time.
@@ -511,14 +637,12 @@ extern "C" int fgnn_edge_softmax(int N, int64_t E, int H, const int32_t *row_ptr
         hipLaunchKernelGGL(edge_softmax_wide_kernel, dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, in, out);
         return fgnn_launch_status("edge_softmax_wide_kernel");
     }
-    const bool some_long = E * H > SO_LONG_ELEMS;                   // otherwise no row can be long
-    if (H % 4 == 0 && fgnn_aligned16(in) && fgnn_aligned16(out)) {
-        hipLaunchKernelGGL((edge_softmax_kernel<false, 4>), dim3(waves), dim3(FGNN_TPB), 0, st, N, H / 4, row_ptr, in, out);
-        if (some_long) hipLaunchKernelGGL((edge_softmax_kernel<true, 4>), dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, H / 4, row_ptr, in, out);
-    } else {
-        hipLaunchKernelGGL((edge_softmax_kernel<false, 1>), dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, in, out);
-        if (some_long) hipLaunchKernelGGL((edge_softmax_kernel<true, 1>), dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, H, row_ptr, in, out);
-    }
+    const unsigned n_long = E * H > SO_LONG_ELEMS ? (unsigned)((N + SO_CAND - 1) / SO_CAND) : 0u;      // otherwise no row can be long
+    const unsigned grid = n_long + (unsigned)((N + SO_LONG_TPB / 64 - 1) / (SO_LONG_TPB / 64));
+    if (H % 4 == 0 && fgnn_aligned16(in) && fgnn_aligned16(out))
+        hipLaunchKernelGGL(edge_softmax_kernel<4>, dim3(grid), dim3(SO_LONG_TPB), 0, st, N, H / 4, n_long, row_ptr, in, out);
+    else
+        hipLaunchKernelGGL(edge_softmax_kernel<1>, dim3(grid), dim3(SO_LONG_TPB), 0, st, N, H, n_long, row_ptr, in, out);
     return fgnn_launch_status("edge_softmax_kernel");
 }
 
@@ -534,16 +658,12 @@ extern "C" int fgnn_edge_softmax_backward(int N, int64_t E, int H, const int32_t
         hipLaunchKernelGGL(edge_softmax_bwd_wide_kernel, dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, sm, grad_out, grad_in);
         return fgnn_launch_status("edge_softmax_bwd_wide_kernel");
     }
-    const bool some_long = E * H > SO_LONG_ELEMS;
-    if (H % 4 == 0 && fgnn_aligned16(sm) && fgnn_aligned16(grad_out) && fgnn_aligned16(grad_in)) {
-        hipLaunchKernelGGL((edge_softmax_bwd_kernel<false, 4>), dim3(waves), dim3(FGNN_TPB), 0, st, N, H / 4, row_ptr, sm, grad_out, grad_in);
-        if (some_long)
-            hipLaunchKernelGGL((edge_softmax_bwd_kernel<true, 4>), dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, H / 4, row_ptr, sm, grad_out, grad_in);
-    } else {
-        hipLaunchKernelGGL((edge_softmax_bwd_kernel<false, 1>), dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, sm, grad_out, grad_in);
-        if (some_long)
-            hipLaunchKernelGGL((edge_softmax_bwd_kernel<true, 1>), dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, H, row_ptr, sm, grad_out, grad_in);
-    }
+    const unsigned n_long = E * H > SO_LONG_ELEMS ? (unsigned)((N + SO_CAND - 1) / SO_CAND) : 0u;
+    const unsigned grid = n_long + (unsigned)((N + SO_LONG_TPB / 64 - 1) / (SO_LONG_TPB / 64));
+    if (H % 4 == 0 && fgnn_aligned16(sm) && fgnn_aligned16(grad_out) && fgnn_aligned16(grad_in))
+        hipLaunchKernelGGL(edge_softmax_bwd_kernel<4>, dim3(grid), dim3(SO_LONG_TPB), 0, st, N, H / 4, n_long, row_ptr, sm, grad_out, grad_in);
+    else
+        hipLaunchKernelGGL(edge_softmax_bwd_kernel<1>, dim3(grid), dim3(SO_LONG_TPB), 0, st, N, H, n_long, row_ptr, sm, grad_out, grad_in);
     return fgnn_launch_status("edge_softmax_bwd_kernel");
 }
 
@@ -551,7 +671,7 @@ extern "C" int fgnn_edge_softmax_backward(int N, int64_t E, int H, const int32_t
 // element of out, a wave takes 2048 consecutive ones; the row of an edge is found by bisection of row_ptr, first
 // for the wave's first and last edge (wave-uniform), then per lane inside that usually one- or two-row window.
 #define UAV_CHUNKS 32           // 64-element chunks per wave
-#define UAV_UJ 4                // chunks in flight; divides UAV_CHUNKS
+#define UAV_UJ 8                // chunks in flight; divides UAV_CHUNKS
 // VEC = 4: an element is four consecutive columns (W % 4 == 0, 16-byte aligned arrays), W counts such groups.
 template <int VEC>
 __global__ __launch_bounds__(FGNN_TPB) void u_add_v_kernel(int N, int64_t E, int W, const int *__restrict__ ptr, const int *__restrict__ idx,
@@ -623,21 +743,14 @@ __global__ __launch_bounds__(FGNN_TPB) void u_add_v_wide_kernel(int N, int W, co
     }
 }
 
-// grad_row[i,w] = sum over the row's edges (fixed order); grad_col[j,w] += g[p,w] with float atomics into a
-// zero-filled buffer (the reference adds into uninitialised memory, src/u_add_v/u_add_v.cu:67,87).  One pass
-// over grad_out, rows shared out as in the softmax kernels.
-template <bool LONG, int VEC>
-__global__ __launch_bounds__(LONG ? SO_LONG_TPB : FGNN_TPB) void u_add_v_bwd_kernel(int N, int W, const int *__restrict__ ptr,
-                                                                                    const int *__restrict__ idx, const float *__restrict__ g,
-                                                                                    float *__restrict__ grow, float *__restrict__ gcol)
+// grad_row[i,w] = sum over the row's edges (fixed order) and, with COLS, grad_col[j,w] += g[p,w] with float atomics
+// into a zero-filled buffer as the reference does it (src/u_add_v/u_add_v.cu:43-90, which adds into uninitialised
+// memory); without COLS the column sums are left to the tile-ordered pass of fgnn_edge_colsum.  One pass over grad_out,
+// rows shared out as in the softmax kernels.
+template <bool LONG, int VEC, bool COLS>
+__device__ __forceinline__ void so_rowsum_row(int W, int row, int pb, int pe, const int *__restrict__ idx, const float *__restrict__ g,
+                                              float *__restrict__ grow, float *__restrict__ gcol, float (*sh)[64])
 {
-    __shared__ float sh[LONG ? SO_LONG_TPB / 64 : 1][64];
-    const unsigned u = LONG ? blockIdx.x : (unsigned)fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
-    if (u >= (unsigned)N) return;
-    const int row = fg_uni(so_scattered_row(u, N));
-    const int pb = fg_uni(ptr[row]), pe = fg_uni(ptr[row + 1]);
-    const int64_t n = (int64_t)(pe - pb) * W * VEC;
-    if (LONG ? n <= SO_LONG_ELEMS : n > SO_LONG_ELEMS) return;      // empty rows stay with the short launch: they store zeros
     const int lane = fg_lane(), S0 = (64 / W) * W, w = lane % W;
     const int per = S0 / W;                                        // entries per wave-wide trip
     const int nw = LONG ? SO_LONG_TPB / 64 : 1;
@@ -647,13 +760,38 @@ __global__ __launch_bounds__(LONG ? SO_LONG_TPB : FGNN_TPB) void u_add_v_bwd_ker
 #pragma unroll 8
         for (int q = pb + (LONG ? fg_wave() * per : 0) + lane / W; q < pe; q += per * nw) {
             const so_grp<VEC> v = so_load<VEC>(g + ((size_t)q * W + w) * VEC);
-            float *dst = gcol + ((size_t)idx[q] * W + w) * VEC;
 #pragma unroll
-            for (int c = 0; c < VEC; ++c) { acc.c[c] += v.c[c]; unsafeAtomicAdd(dst + c, v.c[c]); }
+            for (int c = 0; c < VEC; ++c) acc.c[c] += v.c[c];
+            if constexpr (COLS) {
+                float *dst = gcol + ((size_t)idx[q] * W + w) * VEC;
+#pragma unroll
+                for (int c = 0; c < VEC; ++c) unsafeAtomicAdd(dst + c, v.c[c]);
+            }
         }
     }
     acc = so_column_reduce<LONG, VEC>(acc, lane, W, S0, sh, so_add());
     if (lane < W && (!LONG || fg_wave() == 0)) so_store<VEC>(grow + ((size_t)row * W + lane) * VEC, acc);
+}
+
+template <int VEC, bool COLS>
+__global__ __launch_bounds__(SO_LONG_TPB) void edge_rowsum_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
+                                                                  const int *__restrict__ idx, const float *__restrict__ g, float *__restrict__ grow,
+                                                                  float *__restrict__ gcol)
+{
+    __shared__ float sh[SO_LONG_TPB / 64][64];
+    __shared__ unsigned long long sh_mask;
+    if (blockIdx.x < n_long_blocks) {
+        for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
+            const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
+            so_rowsum_row<true, VEC, COLS>(W, row, fg_uni(ptr[row]), fg_uni(ptr[row + 1]), idx, g, grow, gcol, sh);
+        }
+        return;
+    }
+    int row, pb;
+    int64_t n;
+    const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (SO_LONG_TPB / 64)) + fg_wave());
+    if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n)) return;      // empty rows stay here: they store zeros
+    so_rowsum_row<false, VEC, COLS>(W, row, pb, fg_uni(ptr[row + 1]), idx, g, grow, gcol, nullptr);
 }
 
 __global__ __launch_bounds__(FGNN_TPB) void u_add_v_bwd_wide_kernel(int N, int W, const int *ptr, const int *idx, const float *g, float *grow, float *gcol)
@@ -713,10 +851,61 @@ extern "C" int fgnn_u_add_v_backward(int N, int64_t E, int W, const int32_t *row
     }
     // one float per lane: the atomics of a wave instruction then fall into the fewest cache lines (with four per lane
     // the pass took three times as long on a 115 M-entry graph)
-    hipLaunchKernelGGL((u_add_v_bwd_kernel<false, 1>), dim3(waves), dim3(FGNN_TPB), 0, st, N, W, row_ptr, col_ind, grad_out, grad_row, grad_col);
-    if (E * W > SO_LONG_ELEMS)
-        hipLaunchKernelGGL((u_add_v_bwd_kernel<true, 1>), dim3((unsigned)N), dim3(SO_LONG_TPB), 0, st, N, W, row_ptr, col_ind, grad_out, grad_row, grad_col);
-    return fgnn_launch_status("u_add_v_bwd_kernel");
+    const unsigned n_long = E * W > SO_LONG_ELEMS ? (unsigned)((N + SO_CAND - 1) / SO_CAND) : 0u;
+    hipLaunchKernelGGL((edge_rowsum_kernel<1, true>), dim3(n_long + (unsigned)((N + SO_LONG_TPB / 64 - 1) / (SO_LONG_TPB / 64))), dim3(SO_LONG_TPB), 0, st,
+                       N, W, n_long, row_ptr, col_ind, grad_out, grad_row, grad_col);
+    return fgnn_launch_status("edge_rowsum_kernel");
+}
+
+// More than 64 columns: one wave per row, lanes over the columns.
+__global__ __launch_bounds__(FGNN_TPB) void edge_rowsum_wide_kernel(int N, int W, const int *__restrict__ ptr, const float *__restrict__ g,
+                                                                    float *__restrict__ out)
+{
+    const int row = fg_uni((int)blockIdx.x * FGNN_WPB + fg_wave());
+    if (row >= N) return;
+    const int pb = fg_uni(ptr[row]), pe = fg_uni(ptr[row + 1]);
+    for (int w = fg_lane(); w < W; w += 64) {
+        float acc = 0.f;
+        for (int q = pb; q < pe; ++q) acc += g[(size_t)q * W + w];
+        out[(size_t)row * W + w] = acc;
+    }
+}
+
+// out[i,:] = sum of g[p,:] over the CSR positions p of row i, in a fixed order.
+extern "C" int fgnn_edge_rowsum(int N, int64_t E, int W, const int32_t *row_ptr, const float *g, float *out, void *stream)
+{
+    FGNN_REQUIRE(N >= 0 && E >= 0 && W >= 1, FGNN_ERR_SHAPE, "fgnn_edge_rowsum: bad sizes");
+    FGNN_REQUIRE((row_ptr && out) || N == 0, FGNN_ERR_NULL, "fgnn_edge_rowsum: NULL argument");
+    FGNN_REQUIRE(g || E == 0, FGNN_ERR_NULL, "fgnn_edge_rowsum: NULL argument");
+    if (N == 0) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned waves = (unsigned)((N + FGNN_WPB - 1) / FGNN_WPB);
+    if (W > 64) {
+        hipLaunchKernelGGL(edge_rowsum_wide_kernel, dim3(waves), dim3(FGNN_TPB), 0, st, N, W, row_ptr, g, out);
+        return fgnn_launch_status("edge_rowsum_wide_kernel");
+    }
+    const bool vec4 = W % 4 == 0 && fgnn_aligned16(g) && fgnn_aligned16(out);
+    const unsigned n_long = E * W > SO_LONG_ELEMS ? (unsigned)((N + SO_CAND - 1) / SO_CAND) : 0u;
+    const unsigned grid = n_long + (unsigned)((N + SO_LONG_TPB / 64 - 1) / (SO_LONG_TPB / 64));
+    if (vec4)
+        hipLaunchKernelGGL((edge_rowsum_kernel<4, false>), dim3(grid), dim3(SO_LONG_TPB), 0, st, N, W / 4, n_long, row_ptr, nullptr, g, out, nullptr);
+    else
+        hipLaunchKernelGGL((edge_rowsum_kernel<1, false>), dim3(grid), dim3(SO_LONG_TPB), 0, st, N, W, n_long, row_ptr, nullptr, g, out, nullptr);
+    return fgnn_launch_status("edge_rowsum_kernel");
+}
+
+// u_add_v's backward without atomics: the row sums by the pass above, the column sums by the tile-ordered pass of
+// fgnn_edge_colsum under a plan of (row_ptr, col_ind).  Both are summed in a fixed order.
+extern "C" int fgnn_u_add_v_backward_planned(int N, int64_t E, int W, const int32_t *row_ptr, const int32_t *col_ind, const float *grad_out,
+                                             float *grad_row, float *grad_col, const fgnn_colsum_plan_t *plan, void *workspace,
+                                             size_t workspace_bytes, void *stream)
+{
+    FGNN_REQUIRE(plan, FGNN_ERR_NULL, "fgnn_u_add_v_backward_planned: NULL plan");
+    FGNN_REQUIRE(fgnn_colsum_plan_matches(plan, row_ptr, col_ind, N, N, E), FGNN_ERR_SCHEDULE,
+                 "fgnn_u_add_v_backward_planned: the plan was built for other arrays");
+    int rc = fgnn_edge_rowsum(N, E, W, row_ptr, grad_out, grad_row, stream);
+    if (rc) return rc;
+    return fgnn_edge_colsum(plan, W, grad_out, grad_col, workspace, workspace_bytes, stream);
 }
 
 // ------------------------------------------------------------------------------- per-edge Linear(2, D) + tanh

@@ -320,12 +320,48 @@ int    fgnn_edge_softmax(int N, int64_t E, int H, const int32_t *row_ptr, const 
                          void *stream);
 int    fgnn_edge_softmax_backward(int N, int64_t E, int H, const int32_t *row_ptr, const float *sm,
                                   const float *grad_out, float *grad_in, void *stream);
-/* u_add_v.u_add_v_forward / u_add_v_backward (src/u_add_v/u_add_v.cpp; u_add_v.cu:28-90).
- * The backward needs the CSC arrays to reduce per source node without atomics. */
+/* u_add_v.u_add_v_forward / u_add_v_backward (src/u_add_v/u_add_v.cpp; u_add_v.cu:28-90):
+ * out[p,w] = row_val[row(p),w] + col_val[col_ind[p],w]; backward grad_row[i,:] = sum of grad_out over row i,
+ * grad_col[j,:] = sum of grad_out over the entries with col_ind == j.  fgnn_u_add_v_backward takes the reference's
+ * arguments and, like the reference, forms the column sums with float atomics (into a buffer it zero-fills first):
+ * the summation order, and with it the last bits of grad_col, vary from run to run.  fgnn_u_add_v_backward_planned
+ * below is the atomic-free form. */
 int    fgnn_u_add_v(int N, int64_t E, int W, const int32_t *row_ptr, const int32_t *col_ind,
                     const float *row_val, const float *col_val, float *out, void *stream);
 int    fgnn_u_add_v_backward(int N, int64_t E, int W, const int32_t *row_ptr, const int32_t *col_ind,
                              const float *grad_out, float *grad_row, float *grad_col, void *stream);
+
+/* Column sums of a per-edge array without global atomics, bit-reproducible: out[j,:] = sum of g[p,:] over the CSR
+ * positions p with col_ind[p] == j (the grad_col of u_add_v's backward, u_add_v.cu:43-90, and the gather_col step of
+ * the fuse-scatter GAT backward, src/fused_gat/fused_gat.cu:558-586, which reads g through `permute`: 32 bytes out
+ * of every 128-byte line it pulls).  A plan belongs to one (row_ptr, col_ind) pair, which must outlive it and keep
+ * its contents, and needs the columns of every row in ascending order to pay off (any order is summed correctly).
+ * It cuts the columns into ranges whose accumulators (columns x W floats, W rounded up to a multiple of 4) fit
+ * lds_bytes of LDS (<= 0: 8 KiB, which lets twenty waves share a compute unit; at most 64 KiB) and keeps 6 bytes of device memory per entry: every range's
+ * entries in CSR order, so that a range's pass reads g in contiguous runs.  task_len (<= 0: chosen from E) is the
+ * number of entries one wave sums; ranges longer than that are summed in pieces and merged in a fixed order through
+ * the workspace.  A plan built for W serves every narrower array too.  Building it sorts the entries once (a radix
+ * sort pass or two) and synchronises `stream`.  W <= 64, or <= 256 in multiples of 4 on 16-byte aligned arrays. */
+typedef struct fgnn_colsum_plan fgnn_colsum_plan_t;
+int    fgnn_colsum_plan_create(const int32_t *row_ptr, const int32_t *col_ind, int n_rows, int n_cols, int64_t E, int W,
+                               int lds_bytes, int task_len, void *stream, fgnn_colsum_plan_t **out);
+void   fgnn_colsum_plan_destroy(fgnn_colsum_plan_t *p);
+size_t fgnn_colsum_plan_device_bytes(const fgnn_colsum_plan_t *p);
+int    fgnn_colsum_plan_columns_per_range(const fgnn_colsum_plan_t *p);
+int    fgnn_colsum_plan_num_tasks(const fgnn_colsum_plan_t *p);
+int    fgnn_colsum_plan_matches(const fgnn_colsum_plan_t *p, const int32_t *row_ptr, const int32_t *col_ind, int n_rows,
+                                int n_cols, int64_t E);
+size_t fgnn_colsum_workspace_bytes(const fgnn_colsum_plan_t *p, int W);
+int    fgnn_edge_colsum(const fgnn_colsum_plan_t *p, int W, const float *g, float *out, void *workspace,
+                        size_t workspace_bytes, void *stream);
+/* Row sums of a per-edge array in a fixed order: out[i,:] = sum of g[p,:] over the CSR positions of row i (the grad_row
+ * of u_add_v's backward, u_add_v.cu:43-66).  Any width. */
+int    fgnn_edge_rowsum(int N, int64_t E, int W, const int32_t *row_ptr, const float *g, float *out, void *stream);
+/* fgnn_u_add_v_backward with both sums in a fixed order: fgnn_edge_rowsum + fgnn_edge_colsum under a plan of
+ * (row_ptr, col_ind) with n_cols == N; workspace of fgnn_colsum_workspace_bytes(plan, W). */
+int    fgnn_u_add_v_backward_planned(int N, int64_t E, int W, const int32_t *row_ptr, const int32_t *col_ind,
+                                     const float *grad_out, float *grad_row, float *grad_col,
+                                     const fgnn_colsum_plan_t *plan, void *workspace, size_t workspace_bytes, void *stream);
 
 /* The per-edge pseudo-coordinate projection of the MoNet drivers, nn.Sequential(nn.Linear(2, D),
  * nn.Tanh()) on the [E, 2] edge coordinates (script/train/train_gmmconv_our.py:46-57), in one pass

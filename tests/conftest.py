@@ -20,3 +20,15 @@ def pytest_collection_modifyitems(config, items):
     for it in items:
         if "gpu" in it.keywords:
             it.add_marker(skip)
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """FGNN_PARITY_LOG=<file>: how much of the derived tolerance every sum-scaled comparison used (tests/util.py)."""
+    path = os.environ.get("FGNN_PARITY_LOG")
+    if not path:
+        return
+    import json
+    from tests import util
+    os.makedirs(os.path.dirname(os.path.abspath(path)), exist_ok=True)
+    with open(path, "w") as fh:
+        json.dump(util.PARITY_LOG, fh, indent=1)

@@ -1032,3 +1032,117 @@ def test_gmm_sum_with_bias_and_residual_in_the_store(k, dim, f, with_bias, with_
     _lib.clear_schedule_cache()
     with pytest.raises(_lib.FgnnError, match="sum over the kernels"):
         fg.gmm_native.gmmconv(gd.row_ptr, gd.col_ind, dl[0].detach(), dl[1].detach(), dl[2].detach(), dl[3].detach(), bias=torch.zeros(f, device=DEV))
+
+
+# ------------------------------------------------------------------ column sums under a tile-ordered plan
+@pytest.mark.parametrize("w,lds,task_len", [(1, 1024, 64), (3, 1024, 0), (4, 2048, 100), (8, 0, 0), (8, 4096, 256), (12, 1024, 64),
+                                            (33, 4096, 0), (64, 8192, 300), (128, 16384, 0), (256, 65536, 64)])
+def test_edge_colsum_under_a_plan(w, lds, task_len):
+    """out[j] = sum of g[p] over the entries of column j: rectangular pattern (more columns than rows, the last range
+    partly filled), unsorted rows with repeated columns, empty columns, ranges cut into several tasks and merged; against
+    float64, twice with equal bits, and through fgnn_u_add_v_backward_planned on the square pattern."""
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd.operators.u_add_v import u_add_v_native
+    rng = np.random.default_rng(w * 7 + lds)
+    n_rows, n_cols = 257, 1500
+    rows = []
+    for i in range(n_rows):
+        d = int(rng.choice([0, 1, 5, 40, 700]))
+        cols = rng.integers(0, n_cols - 300, size=d)          # the last 300 columns stay empty
+        rows.append(list(np.sort(cols)) if i % 3 else list(cols))
+    g = custom_graph(rows, n_rows)
+    e = g.n_edges
+    gen = torch.Generator().manual_seed(w)
+    val = torch.randn(e, w, generator=gen)
+    ref = torch.zeros(n_cols, w, dtype=torch.float64).index_add_(0, g.col_ind.long(), val.double())
+    s_abs = torch.zeros(n_cols, w, dtype=torch.float64).index_add_(0, g.col_ind.long(), val.double().abs())
+    rp, ci, vd = g.row_ptr.to(DEV), g.col_ind.to(DEV), val.to(DEV)
+    plan = _lib.ColsumPlan(rp, ci, n_cols, w, lds_bytes=lds, task_len=task_len)
+    assert plan.n_tasks >= (n_cols + plan.columns_per_range - 1) // plan.columns_per_range
+    out = plan.colsum(vd)
+    assert_close_sum(out, ref, s_abs, "edge colsum W=%d" % w)
+    assert torch.equal(out, plan.colsum(vd)), "column sums differ between two runs"
+    if w > 1:          # a plan serves narrower arrays
+        out1 = plan.colsum(vd[:, :1].contiguous())
+        assert_close_sum(out1, ref[:, :1], s_abs[:, :1], "edge colsum W=1 under a plan for W=%d" % w)
+    # the square pattern through the u_add_v backward, both forms
+    sq = custom_graph([[c % n_rows for c in r] for r in rows], n_rows)
+    rp2, ci2 = sq.row_ptr.to(DEV), sq.col_ind.to(DEV)
+    ref_col = torch.zeros(n_rows, w, dtype=torch.float64).index_add_(0, sq.col_ind.long(), val.double())
+    abs_col = torch.zeros(n_rows, w, dtype=torch.float64).index_add_(0, sq.col_ind.long(), val.double().abs())
+    ref_row = orc.segment_sums(sq.row_ptr, val.double())
+    abs_row = orc.segment_sums(sq.row_ptr, val.double().abs())
+    for atomics in (False, True):
+        grow, gcol = u_add_v_native.u_add_v_backward(rp2, ci2, vd, atomics=atomics)
+        assert_close_sum(grow, ref_row, abs_row, "u_add_v grad row W=%d atomics=%s" % (w, atomics))
+        assert_close_sum(gcol, ref_col, abs_col, "u_add_v grad col W=%d atomics=%s" % (w, atomics))
+
+
+def test_edge_colsum_plan_argument_errors():
+    from ae_mlsys_gnn_amd import _lib
+    g = _small_graph().to(DEV)
+    with pytest.raises(_lib.FgnnError, match="lds_bytes"):
+        _lib.ColsumPlan(g.row_ptr, g.col_ind, g.n, 8, lds_bytes=100)
+    with pytest.raises(_lib.FgnnError, match="too wide"):
+        _lib.ColsumPlan(g.row_ptr, g.col_ind, g.n, 300, lds_bytes=1024)
+    with pytest.raises(_lib.FgnnError, match="outside"):
+        _lib.ColsumPlan(g.row_ptr, g.col_ind, g.n - 50, 8)          # column ids beyond n_cols
+    plan = _lib.ColsumPlan(g.row_ptr, g.col_ind, g.n, 4, lds_bytes=65536)
+    with pytest.raises(_lib.FgnnError, match="narrower"):
+        plan.colsum(torch.zeros(g.n_edges, 64, device=DEV))
+    empty = custom_graph([[] for _ in range(10)], 10).to(DEV)
+    pe = _lib.ColsumPlan(empty.row_ptr, empty.col_ind, 10, 8)
+    assert torch.equal(pe.colsum(torch.zeros(0, 8, device=DEV)), torch.zeros(10, 8, device=DEV))
+
+
+@pytest.mark.parametrize("w", [1, 3, 4, 8, 12, 100, 512, 2051, 2052])
+def test_gather_rows_widths(w):
+    """mhtranspose for row widths on every side of the kernel's cases: scalar and 128-bit lanes, several rows per wave,
+    one row per wave in one or several trips."""
+    from ae_mlsys_gnn_amd.operators import mhspmm as op
+    e = 777 if w < 512 else 37
+    gen = torch.Generator().manual_seed(w)
+    x = torch.randn(e, w, generator=gen)
+    perm = torch.randperm(e, generator=gen).to(torch.int32)
+    out = op.mhtranspose(perm.to(DEV), x.to(DEV))
+    assert torch.equal(out.cpu(), x[perm.long()])
+    # an unaligned view takes the scalar path
+    if w % 4 == 0:
+        buf = torch.randn(e * w + 1, generator=gen).to(DEV)
+        xin = buf[1:].view(e, w)
+        out = torch.empty(e * w + 1, device=DEV)[1:].view(e, w)
+        from ae_mlsys_gnn_amd._lib import check, lib, ptr, stream_ptr
+        check(lib().fgnn_gather_rows(e, w, ptr(perm.to(DEV)), ptr(xin), ptr(out), stream_ptr()), "fgnn_gather_rows")
+        assert torch.equal(out.cpu(), xin.cpu()[perm.long()])
+
+
+@pytest.mark.parametrize("nh", [1, 4, 8, 20])
+def test_edge_softmax_rows_beyond_the_register_cache(nh):
+    """Rows longer than what a workgroup keeps in registers (the part beyond is folded into a running maximum and sum while
+    it streams by): a 40 k-entry row whose values ascend, so the running maximum moves on every trip, one whose values
+    descend, a constant one, next to short rows; forward and backward against float64."""
+    from ae_mlsys_gnn_amd.operators import edge_softmax as op
+    lens = [40000, 3, 0, 40000, 9000, 1, 40000]
+    g = custom_graph([[0] * d for d in lens], len(lens))
+    e = g.n_edges
+    gen = torch.Generator().manual_seed(nh)
+    h = torch.randn(e, nh, generator=gen, dtype=torch.float64)
+    ramp = torch.linspace(-30, 30, 40000, dtype=torch.float64).view(-1, 1)
+    h[:40000] += ramp
+    h[40003:80003] -= ramp
+    h[89004:] = 1.5
+    go = torch.randn(e, nh, generator=gen, dtype=torch.float64)
+    hl = h.clone().requires_grad_(True)
+    ref = orc.edge_softmax(g.row_ptr, hl)
+    ref.backward(go)
+    hd = h.float().to(DEV).requires_grad_(True)
+    out = op.csr_edge_softmax(g.row_ptr.to(DEV), hd)
+    out.backward(go.float().to(DEV))
+    c = c_exp(float(h.max() - h.min()))
+    one = torch.ones((), dtype=torch.float64)
+    assert_close_sum(out, ref.detach(), one, "edge_softmax of long rows", c=c)
+    dst = orc.row_of_edge(g.row_ptr)
+    dot_abs = orc.segment_sums(g.row_ptr, ref.detach() * go.abs())
+    assert_close_sum(hd.grad, hl.grad, ref.detach() * (go.abs() + dot_abs[dst]), "edge_softmax grad of long rows", c=c)
+    sums = orc.segment_sums(g.row_ptr, out.detach().cpu().double())
+    assert float((sums - (torch.tensor(lens) > 0).double().view(-1, 1)).abs().max()) < 1e-5

@@ -43,6 +43,8 @@ _SIGNATURES = {
     "fgnn_gat_backward_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_void_p, c_void_p, c_int]),
     "fgnn_gat_backward": (c_int, [c_int, c_int64, c_int, c_int, c_float] + [c_void_p] * 19
                           + [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "fgnn_gat_backward_own_order": (c_int, [c_int, c_int64, c_int, c_int, c_float] + [c_void_p] * 17
+                                    + [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "fgnn_gat_stash_own_order": (c_int, [c_int, c_int64, c_int, c_float] + [c_void_p] * 7 + [c_void_p, c_void_p]),
     "fgnn_edgeconv_forward": (c_int, [c_int, c_int, c_int, c_int] + [c_void_p] * 5 + [c_void_p]),
     "fgnn_edgeconv_backward": (c_int, [c_int, c_int, c_int] + [c_void_p] * 3 + [c_void_p]),

@@ -19,6 +19,7 @@
 //
 // Math contract: src/fused_gat/fused_gat_SM.cu:193-286 (forward), :560-607, :656-732, :734-801
 // (backward) of the reference; LeakyReLU derivative at 0 is `slope` as in torch.
+#include <algorithm>
 #include "fgnn_common.h"
 
 struct GatFwdP {
@@ -1050,14 +1051,54 @@ static int gat_common_checks(const char *fn, int N, int64_t E, int H, int F)
     FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1 && F >= 1, FGNN_ERR_SHAPE, "%s: bad sizes N=%d E=%lld H=%d F=%d", fn, N, (long long)E, H, F);
     FGNN_REQUIRE(E <= 2147483647LL, FGNN_ERR_LIMIT, "%s: E=%lld exceeds int32 positions", fn, (long long)E);
     FGNN_REQUIRE(H <= 64, FGNN_ERR_LIMIT, "%s: H=%d > 64 heads unsupported", fn, H);
-    FGNN_REQUIRE((int64_t)H * F <= 1024, FGNN_ERR_LIMIT, "%s: H*F=%lld > 1024 unsupported", fn, (long long)H * F);
+    FGNN_REQUIRE(F <= 1024, FGNN_ERR_LIMIT, "%s: F=%d > 1024 floats per head unsupported", fn, F);
     return 0;
 }
+
+// Rows of more than 1024 floats (the reference launches its recompute and stash kernels for any number of heads of up to
+// 1024 floats each, src/fused_gat/fused_gat_SM.cu:518-522, :843-847) are served in passes over groups of heads: scores,
+// row statistics and outputs of different heads never meet, so a pass copies the slices of `hg` heads of the node-sized
+// arrays into contiguous buffers of the workspace, runs the ordinary entry on them and copies its results back.
+__global__ __launch_bounds__(256) void copy2d_kernel(const float *__restrict__ src, size_t src_ld, float *__restrict__ dst, size_t dst_ld,
+                                                     size_t rows, int cols)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * (size_t)cols) return;
+    const size_t r = i / (size_t)cols, c = i - r * (size_t)cols;
+    dst[r * dst_ld + c] = src[r * src_ld + c];
+}
+static int copy2d(const float *src, size_t src_ld, float *dst, size_t dst_ld, size_t rows, int cols, hipStream_t st)
+{
+    const size_t n = rows * (size_t)cols;
+    if (n == 0) return 0;
+    FGNN_REQUIRE((n + 255) / 256 <= 2147483647ULL, FGNN_ERR_LIMIT, "head-group copy: too many elements");
+    hipLaunchKernelGGL(copy2d_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, src, src_ld, dst, dst_ld, rows, cols);
+    return fgnn_launch_status("copy2d_kernel");
+}
+static inline int gat_group_heads(int H, int F) { return (int64_t)H * F <= 1024 ? H : std::max(1, 1024 / F); }
+static inline size_t gat_nf_bytes(int N, int hg, int F) { return fgnn_align256((size_t)N * hg * F * sizeof(float)); }
+static inline size_t gat_nh_bytes(int N, int hg) { return fgnn_align256((size_t)N * hg * sizeof(float)); }
 
 extern "C" size_t fgnn_gat_forward_workspace_bytes(const fgnn_schedule_t *sched, int H, int F)
 {
     if (!sched) return 0;
-    return (size_t)sched->n_partials * gat_fwd_pw(H * F, H, true) * sizeof(float);
+    const int hg = gat_group_heads(H, F);
+    size_t b = (size_t)sched->n_partials * gat_fwd_pw(hg * F, hg, true) * sizeof(float);
+    if (hg < H)        // slices of in_feat, out, out2 and of attn_row, attn_col, edge_max, edge_sum, c
+        b = fgnn_align256(b) + 3 * gat_nf_bytes(sched->n_rows, hg, F) + 5 * gat_nh_bytes(sched->n_rows, hg);
+    return b;
+}
+
+// The stashed per-edge tensors of the stash variants in CSR order, from the row statistics (no dependence on F).
+static int gat_stash_csr_order(int N, int64_t E, int H, const int32_t *row_ptr, const int32_t *col_ind, const float *attn_row,
+                               const float *attn_col, const float *edge_max, const float *edge_sum, float slope, float *e_lrelu,
+                               float *e_softmax, hipStream_t st)
+{
+    if (!e_softmax || E == 0) return 0;
+    const int64_t waves = (E * H + 64 * GAT_STASH_CHUNKS - 1) / (64 * GAT_STASH_CHUNKS);
+    hipLaunchKernelGGL(gat_edge_stash_kernel, dim3((unsigned)((waves + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, st, N, E, H, row_ptr,
+                       col_ind, attn_row, attn_col, edge_max, edge_sum, slope, e_lrelu, e_softmax);
+    return fgnn_launch_status("gat_edge_stash_kernel");
 }
 
 static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_row, const float *attn_col,
@@ -1133,13 +1174,7 @@ static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_
         return 0;
     });
     if (rc) return rc;
-    if (e_softmax && E > 0) {
-        const int64_t waves = (E * H + 64 * GAT_STASH_CHUNKS - 1) / (64 * GAT_STASH_CHUNKS);
-        hipLaunchKernelGGL(gat_edge_stash_kernel, dim3((unsigned)((waves + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, st, N, E, H, row_ptr,
-                           col_ind, attn_row, attn_col, edge_max, edge_sum, slope, e_lrelu, e_softmax);
-        return fgnn_launch_status("gat_edge_stash_kernel");
-    }
-    return 0;
+    return gat_stash_csr_order(N, E, H, row_ptr, col_ind, attn_row, attn_col, edge_max, edge_sum, slope, e_lrelu, e_softmax, st);
 }
 
 extern "C" int fgnn_gat_forward(int N, int64_t E, int H, int F, const float *attn_row, const float *attn_col,
@@ -1156,6 +1191,44 @@ extern "C" int fgnn_gat_forward(int N, int64_t E, int H, int F, const float *att
     FGNN_REQUIRE(e_lrelu == nullptr || e_softmax != nullptr, FGNN_ERR_NULL, "fgnn_gat_forward: e_lrelu is only written together with e_softmax");
     rc = check_sched(sched, row_ptr, col_ind, N, E, "fgnn_gat_forward");
     if (rc) return rc;
+    const int hmax = gat_group_heads(H, F);
+    if (hmax < H) {
+        FGNN_REQUIRE(sched, FGNN_ERR_SCHEDULE, "fgnn_gat_forward: rows of more than 1024 floats (H*F=%lld) need a schedule", (long long)H * F);
+        const size_t need = fgnn_gat_forward_workspace_bytes(sched, H, F);
+        FGNN_REQUIRE(workspace && workspace_bytes >= need, FGNN_ERR_WORKSPACE, "fgnn_gat_forward: workspace %zu < %zu bytes", workspace_bytes, need);
+        FGNN_REQUIRE(fgnn_aligned16(workspace), FGNN_ERR_ALIGN, "fgnn_gat_forward: workspace not 16-byte aligned");
+        hipStream_t st = (hipStream_t)stream;
+        const size_t nf = gat_nf_bytes(N, hmax, F), nh = gat_nh_bytes(N, hmax), HF = (size_t)H * F;
+        char *w = (char *)workspace;
+        float *xg = (float *)w; w += nf;
+        float *og = (float *)w; w += nf;
+        float *o2g = (float *)w; w += nf;
+        float *arg = (float *)w; w += nh;
+        float *acg = (float *)w; w += nh;
+        float *mxg = (float *)w; w += nh;
+        float *smg = (float *)w; w += nh;
+        float *cg = (float *)w; w += nh;
+        const size_t inner = workspace_bytes - (size_t)(w - (char *)workspace);
+        const bool aux = aux_out2 != nullptr;
+        for (int h0 = 0; h0 < H; h0 += hmax) {
+            const int hg = std::min(hmax, H - h0);
+            const size_t gf = (size_t)hg * F;
+            if ((rc = copy2d(attn_row + h0, H, arg, hg, N, hg, st))) return rc;
+            if ((rc = copy2d(attn_col + h0, H, acg, hg, N, hg, st))) return rc;
+            if ((rc = copy2d(in_feat + (size_t)h0 * F, HF, xg, gf, N, (int)gf, st))) return rc;
+            rc = gat_forward_launch(N, E, hg, F, arg, acg, row_ptr, col_ind, negative_slope, xg, og, mxg, smg, aux ? o2g : nullptr,
+                                    aux ? cg : nullptr, nullptr, nullptr, sched, w, inner, st);
+            if (rc) return rc;
+            if ((rc = copy2d(og, gf, out + (size_t)h0 * F, HF, N, (int)gf, st))) return rc;
+            if ((rc = copy2d(mxg, hg, edge_max + h0, H, N, hg, st))) return rc;
+            if ((rc = copy2d(smg, hg, edge_sum + h0, H, N, hg, st))) return rc;
+            if (aux) {
+                if ((rc = copy2d(o2g, gf, aux_out2 + (size_t)h0 * F, HF, N, (int)gf, st))) return rc;
+                if ((rc = copy2d(cg, hg, aux_c + h0, H, N, hg, st))) return rc;
+            }
+        }
+        return gat_stash_csr_order(N, E, H, row_ptr, col_ind, attn_row, attn_col, edge_max, edge_sum, negative_slope, e_lrelu, e_softmax, st);
+    }
     return gat_forward_launch(N, E, H, F, attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, out, edge_max,
                               edge_sum, aux_out2, aux_c, e_lrelu, e_softmax, sched, workspace, workspace_bytes, (hipStream_t)stream);
 }
@@ -1165,6 +1238,15 @@ extern "C" int fgnn_gat_forward(int N, int64_t E, int H, int F, const float *att
 extern "C" size_t fgnn_gat_backward_workspace_bytes(int N, int H, int F, const fgnn_schedule_t *sched_csc,
                                                     const fgnn_schedule_t *sched_csr, int need_recompute)
 {
+    const int hg = gat_group_heads(H, F);
+    if (hg < H) {      // head-group passes: the ordinary workspace of one group plus the contiguous slices
+        const bool rec = (need_recompute & 1) != 0, stash = (need_recompute & 2) != 0;
+        size_t b = fgnn_align256(fgnn_gat_backward_workspace_bytes(N, hg, F, sched_csc, sched_csr, need_recompute & 1));
+        b += (size_t)(rec ? 3 : 5) * gat_nf_bytes(N, hg, F) + (size_t)(rec ? 6 : 7) * gat_nh_bytes(N, hg);
+        if (stash && sched_csc) b += fgnn_align256((size_t)sched_csc->n_edges * hg * sizeof(float));
+        return b;
+    }
+    need_recompute &= 1;
     size_t HF = (size_t)H * F;
     size_t b = fgnn_align256((size_t)N * H * sizeof(float4));
     if (need_recompute) {
@@ -1175,34 +1257,74 @@ extern "C" size_t fgnn_gat_backward_workspace_bytes(int N, int H, int F, const f
     return b;
 }
 
-extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_slope, const int32_t *row_ptr,
-                                 const int32_t *col_ind, const int32_t *col_ptr, const int32_t *row_ind,
-                                 const int32_t *permute, const float *e_lrelu, const float *e_softmax,
-                                 const float *edge_max, const float *edge_sum, const float *in_feat,
-                                 const float *attn_row, const float *attn_col, const float *out_feat,
-                                 const float *aux_out2, const float *aux_c, const float *grad_out, float *grad_feat,
-                                 float *grad_attn_row, float *grad_attn_col, const fgnn_schedule_t *sched_csc,
-                                 const fgnn_schedule_t *sched_csr, void *workspace, size_t workspace_bytes, void *stream)
+// own_order: e_softmax is the stash of fgnn_gat_stash_own_order (entry order of this pass under sched_csc, sign bit =
+// pre-activation not positive) and permute is not used; otherwise a stash is CSR-ordered and read through permute.
+static int gat_backward_impl(int N, int64_t E, int H, int F, float negative_slope, const int32_t *row_ptr,
+                             const int32_t *col_ind, const int32_t *col_ptr, const int32_t *row_ind,
+                             const int32_t *permute, const float *e_softmax, int own_order,
+                             const float *edge_max, const float *edge_sum, const float *in_feat,
+                             const float *attn_row, const float *attn_col, const float *out_feat,
+                             const float *aux_out2, const float *aux_c, const float *grad_out, float *grad_feat,
+                             float *grad_attn_row, float *grad_attn_col, const fgnn_schedule_t *sched_csc,
+                             const fgnn_schedule_t *sched_csr, void *workspace, size_t workspace_bytes, void *stream)
 {
     int rc = gat_common_checks("fgnn_gat_backward", N, E, H, F);
     if (rc) return rc;
+    if (own_order) permute = nullptr;
     FGNN_REQUIRE(col_ptr && (row_ind || E == 0) && edge_max && edge_sum && in_feat && attn_row && attn_col && grad_out &&
                      grad_feat && grad_attn_row && grad_attn_col,
                  FGNN_ERR_NULL, "fgnn_gat_backward: NULL argument");
     const bool stash = e_softmax != nullptr;
-    // permute == NULL with a stash: e_softmax is in the entry order of this pass under sched_csc (fgnn_gat_stash_own_order)
-    FGNN_REQUIRE(!stash || !permute || fgnn_sched_has_pos(sched_csc), FGNN_ERR_SCHEDULE, "fgnn_gat_backward: stashed attention in the caller's order needs a schedule built with edge positions");
-    (void)e_lrelu;      // the sign of the pre-activation is taken from attn_row + attn_col
+    FGNN_REQUIRE(!stash || own_order || permute, FGNN_ERR_NULL,
+                 "fgnn_gat_backward: stashed attention needs permute (a stash in the pass's own order goes to fgnn_gat_backward_own_order)");
+    FGNN_REQUIRE(!stash || own_order || fgnn_sched_has_pos(sched_csc), FGNN_ERR_SCHEDULE, "fgnn_gat_backward: stashed attention in the caller's order needs a schedule built with edge positions");
     const bool recompute = !(out_feat && aux_out2 && aux_c);
     FGNN_REQUIRE(!recompute || (row_ptr && (col_ind || E == 0)), FGNN_ERR_NULL, "fgnn_gat_backward: recomputing the forward needs row_ptr/col_ind");
     rc = check_sched(sched_csc, col_ptr, row_ind, N, E, "fgnn_gat_backward(csc)");
     if (rc) return rc;
     if (recompute) { rc = check_sched(sched_csr, row_ptr, col_ind, N, E, "fgnn_gat_backward(csr)"); if (rc) return rc; }
-    size_t need = fgnn_gat_backward_workspace_bytes(N, H, F, sched_csc, recompute ? sched_csr : nullptr, recompute);
+    const int hmax = gat_group_heads(H, F);
+    FGNN_REQUIRE(hmax == H || sched_csc, FGNN_ERR_SCHEDULE, "fgnn_gat_backward: rows of more than 1024 floats (H*F=%lld) need a schedule", (long long)H * F);
+    size_t need = fgnn_gat_backward_workspace_bytes(N, H, F, sched_csc, recompute ? sched_csr : nullptr, (recompute ? 1 : 0) | (stash ? 2 : 0));
     FGNN_REQUIRE(workspace && workspace_bytes >= need, FGNN_ERR_WORKSPACE, "fgnn_gat_backward: workspace %zu < %zu bytes", workspace_bytes, need);
     FGNN_REQUIRE(fgnn_aligned16(workspace), FGNN_ERR_ALIGN, "fgnn_gat_backward: workspace not 16-byte aligned");
     if (N == 0) return 0;
     hipStream_t st = (hipStream_t)stream;
+    if (hmax < H) {
+        // passes over groups of heads on contiguous slices (see fgnn_gat_forward_workspace_bytes)
+        const size_t nf = gat_nf_bytes(N, hmax, F), nh = gat_nh_bytes(N, hmax), HFw = (size_t)H * F;
+        char *w = (char *)workspace;
+        auto take = [&](size_t bytes) { float *q = (float *)w; w += bytes; return q; };
+        float *xg = take(nf), *gog = take(nf), *gfg = take(nf);
+        float *og = recompute ? nullptr : take(nf), *o2g = recompute ? nullptr : take(nf);
+        float *arg = take(nh), *acg = take(nh), *mxg = take(nh), *smg = take(nh), *garg = take(nh), *gacg = take(nh);
+        float *cg = recompute ? nullptr : take(nh);
+        float *esg = stash ? take(fgnn_align256((size_t)E * hmax * sizeof(float))) : nullptr;
+        const size_t inner = workspace_bytes - (size_t)(w - (char *)workspace);
+        for (int h0 = 0; h0 < H; h0 += hmax) {
+            const int hg = std::min(hmax, H - h0);
+            const size_t gf = (size_t)hg * F;
+            if ((rc = copy2d(attn_row + h0, H, arg, hg, N, hg, st))) return rc;
+            if ((rc = copy2d(attn_col + h0, H, acg, hg, N, hg, st))) return rc;
+            if ((rc = copy2d(edge_max + h0, H, mxg, hg, N, hg, st))) return rc;
+            if ((rc = copy2d(edge_sum + h0, H, smg, hg, N, hg, st))) return rc;
+            if ((rc = copy2d(in_feat + (size_t)h0 * F, HFw, xg, gf, N, (int)gf, st))) return rc;
+            if ((rc = copy2d(grad_out + (size_t)h0 * F, HFw, gog, gf, N, (int)gf, st))) return rc;
+            if (!recompute) {
+                if ((rc = copy2d(out_feat + (size_t)h0 * F, HFw, og, gf, N, (int)gf, st))) return rc;
+                if ((rc = copy2d(aux_out2 + (size_t)h0 * F, HFw, o2g, gf, N, (int)gf, st))) return rc;
+                if ((rc = copy2d(aux_c + h0, H, cg, hg, N, hg, st))) return rc;
+            }
+            if (stash && (rc = copy2d(e_softmax + h0, H, esg, hg, (size_t)E, hg, st))) return rc;
+            rc = gat_backward_impl(N, E, hg, F, negative_slope, row_ptr, col_ind, col_ptr, row_ind, permute, esg, own_order, mxg, smg, xg, arg, acg,
+                                   og, o2g, cg, gog, gfg, garg, gacg, sched_csc, sched_csr, w, inner, stream);
+            if (rc) return rc;
+            if ((rc = copy2d(gfg, gf, grad_feat + (size_t)h0 * F, HFw, N, (int)gf, st))) return rc;
+            if ((rc = copy2d(garg, hg, grad_attn_row + h0, H, N, hg, st))) return rc;
+            if ((rc = copy2d(gacg, hg, grad_attn_col + h0, H, N, hg, st))) return rc;
+        }
+        return 0;
+    }
     const int HF = H * F;
     char *w = (char *)workspace;
     float4 *rec = (float4 *)w; w += fgnn_align256((size_t)N * H * sizeof(float4));
@@ -1229,7 +1351,7 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
     p.items = sched_csc ? sched_csc->items_dev : nullptr;
     p.n_items = sched_csc ? sched_csc->n_items : N;
     p.ptr = col_ptr; p.idx = fgnn_sched_idx(sched_csc, row_ind); p.pos = fgnn_sched_pos(sched_csc); p.permute = permute; p.rec = rec; p.ac = attn_col; p.x = in_feat; p.g = grad_out;
-    const int stash_mode = !stash ? 0 : (permute ? 1 : 2);
+    const int stash_mode = !stash ? 0 : (own_order ? 2 : 1);
     p.delta = (const float *)rec;       // own-order stash: the record area holds the compact [N,H] delta array instead
     p.esm = e_softmax; p.gfeat = grad_feat; p.gac = grad_attn_col; p.part = part;
     p.N = N; p.H = H; p.F = F; p.HF = HF; p.slope = negative_slope;
@@ -1287,6 +1409,35 @@ extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_
         }
         return 0;
     });
+}
+
+extern "C" int fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_slope, const int32_t *row_ptr,
+                                 const int32_t *col_ind, const int32_t *col_ptr, const int32_t *row_ind,
+                                 const int32_t *permute, const float *e_lrelu, const float *e_softmax,
+                                 const float *edge_max, const float *edge_sum, const float *in_feat,
+                                 const float *attn_row, const float *attn_col, const float *out_feat,
+                                 const float *aux_out2, const float *aux_c, const float *grad_out, float *grad_feat,
+                                 float *grad_attn_row, float *grad_attn_col, const fgnn_schedule_t *sched_csc,
+                                 const fgnn_schedule_t *sched_csr, void *workspace, size_t workspace_bytes, void *stream)
+{
+    (void)e_lrelu;      // the sign of the pre-activation is taken from attn_row + attn_col
+    return gat_backward_impl(N, E, H, F, negative_slope, row_ptr, col_ind, col_ptr, row_ind, permute, e_softmax, 0, edge_max, edge_sum, in_feat,
+                             attn_row, attn_col, out_feat, aux_out2, aux_c, grad_out, grad_feat, grad_attn_row, grad_attn_col, sched_csc, sched_csr,
+                             workspace, workspace_bytes, stream);
+}
+
+extern "C" int fgnn_gat_backward_own_order(int N, int64_t E, int H, int F, float negative_slope, const int32_t *row_ptr,
+                                           const int32_t *col_ind, const int32_t *col_ptr, const int32_t *row_ind,
+                                           const float *e_softmax_own, const float *edge_max, const float *edge_sum,
+                                           const float *in_feat, const float *attn_row, const float *attn_col, const float *out_feat,
+                                           const float *aux_out2, const float *aux_c, const float *grad_out, float *grad_feat,
+                                           float *grad_attn_row, float *grad_attn_col, const fgnn_schedule_t *sched_csc,
+                                           const fgnn_schedule_t *sched_csr, void *workspace, size_t workspace_bytes, void *stream)
+{
+    FGNN_REQUIRE(e_softmax_own || E == 0, FGNN_ERR_NULL, "fgnn_gat_backward_own_order: NULL stash");
+    return gat_backward_impl(N, E, H, F, negative_slope, row_ptr, col_ind, col_ptr, row_ind, nullptr, e_softmax_own, e_softmax_own != nullptr, edge_max,
+                             edge_sum, in_feat, attn_row, attn_col, out_feat, aux_out2, aux_c, grad_out, grad_feat, grad_attn_row, grad_attn_col,
+                             sched_csc, sched_csr, workspace, workspace_bytes, stream);
 }
 
 extern "C" int fgnn_gat_stash_own_order(int N, int64_t E, int H, float negative_slope, const int32_t *col_ptr, const int32_t *row_ind,

@@ -3,6 +3,7 @@
 // None of them takes a work list, so each balances its own load: the element-wise ones cut the
 // [E, W] array into fixed chunks and find the rows of a chunk by bisection of row_ptr, the row
 // reductions give short rows to single waves and long rows to whole workgroups.
+#include <algorithm>
 #include "fgnn_common.h"
 
 // largest r in [lo, hi] with ptr[r] <= q
@@ -19,13 +20,13 @@ __device__ __forceinline__ int so_row_of(const int *__restrict__ ptr, int lo, in
 // finds the row of each edge by binary search).  The entries [pb, pe) of one row, 64 at a time, four gathered
 // b-rows in flight; pos (NULL = identity) maps an entry to the position its result is stored at.
 template <int VEC, int R, bool FULL, int LPH>
-__device__ __forceinline__ void sddmm_row_piece(int row, int pb, int pe, int H, int F, int HF, const fg_lanemap<VEC, R> &lm, int lane, float *scr,
+__device__ __forceinline__ void sddmm_row_piece(int row, int pb, int pe, int H, int F, int ld, int ldo, const fg_lanemap<VEC, R> &lm, int lane, float *scr,
                                                 const int *__restrict__ idx, const int *__restrict__ pos, const float *__restrict__ a,
                                                 const float *__restrict__ b, float *__restrict__ out)
 {
     fg_vec<VEC> ar[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ar[r].load(a + (size_t)row * HF + lm.eoff[r]); else ar[r].zero(); }
+    for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ar[r].load(a + (size_t)row * ld + lm.eoff[r]); else ar[r].zero(); }
     for (int c = pb; c < pe; c += 64) {
         const int q = c + lane;
         const int cnt = min(64, pe - c);
@@ -33,20 +34,20 @@ __device__ __forceinline__ void sddmm_row_piece(int row, int pb, int pe, int H, 
         const int id = idx[qq];
         const int pv = pos ? pos[qq] : qq;
         for (int t = 0; t < cnt; t += 4) {
-            fg_vec<VEC> ld[4][R];
+            fg_vec<VEC> lb[4][R];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 int j = __builtin_amdgcn_readlane(id, (t + u) & 63);
 #pragma unroll
-                for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) ld[u][r].load(b + (size_t)j * HF + lm.eoff[r]); else ld[u][r].zero(); }
+                for (int r = 0; r < R; ++r) { if (FULL || lm.ok[r]) lb[u][r].load(b + (size_t)j * ld + lm.eoff[r]); else lb[u][r].zero(); }
             }
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 if (t + u >= cnt) break;
                 float d[R];
 #pragma unroll
-                for (int r = 0; r < R; ++r) d[r] = ld[u][r].dot(ar[r]);
-                const size_t o = (size_t)(unsigned)__builtin_amdgcn_readlane(pv, (t + u) & 63) * H;
+                for (int r = 0; r < R; ++r) d[r] = lb[u][r].dot(ar[r]);
+                const size_t o = (size_t)(unsigned)__builtin_amdgcn_readlane(pv, (t + u) & 63) * ldo;
                 if constexpr (LPH > 0) {
 #pragma unroll
                     for (int r = 0; r < R; ++r) {
@@ -67,7 +68,7 @@ __device__ __forceinline__ void sddmm_row_piece(int row, int pb, int pe, int H, 
 // and the a-row is loaded once per (wave, row).
 #define SDDMM_CHUNK 256
 template <int VEC, int R, bool FULL, int LPH>
-__global__ __launch_bounds__(FGNN_TPB) void mhsddmm_kernel(int N, int64_t E, int H, int F, int HF, int lphp, const int *ptr, const int *idx,
+__global__ __launch_bounds__(FGNN_TPB) void mhsddmm_kernel(int N, int64_t E, int H, int F, int HF, int ld, int ldo, int lphp, const int *ptr, const int *idx,
                                                            const float *a, const float *b, float *out)
 {
     extern __shared__ float lds[];
@@ -82,7 +83,7 @@ __global__ __launch_bounds__(FGNN_TPB) void mhsddmm_kernel(int N, int64_t E, int
     int pb = fg_uni((int)c0);
     while (pb < c1 && row < N) {                             // ptr[N] = E >= c1 keeps row < N on a consistent graph
         const int pe = min(fg_uni(ptr[row + 1]), c1);
-        if (pe > pb) sddmm_row_piece<VEC, R, FULL, LPH>(row, pb, pe, H, F, HF, lm, lane, scr, idx, nullptr, a, b, out);
+        if (pe > pb) sddmm_row_piece<VEC, R, FULL, LPH>(row, pb, pe, H, F, ld, ldo, lm, lane, scr, idx, nullptr, a, b, out);
         pb = pe;
         ++row;
     }
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(FGNN_TPB) void mhsddmm_kernel(int N, int64_t E, int
 // Under a work list (one wave per item; an XCD-aware list keeps each XCD on one eighth of the gathered b-rows):
 // the entries are walked in the list's order and every result goes to its caller's position.
 template <int VEC, int R, bool FULL, int LPH>
-__global__ __launch_bounds__(FGNN_TPB) void mhsddmm_items_kernel(const fgnn_item *items, int n_items, int H, int F, int HF, int lphp, const int *ptr,
+__global__ __launch_bounds__(FGNN_TPB) void mhsddmm_items_kernel(const fgnn_item *items, int n_items, int H, int F, int HF, int ld, int ldo, int lphp, const int *ptr,
                                                                  const int *idx, const int *pos, const float *a, const float *b, float *out)
 {
     extern __shared__ float lds[];
@@ -101,14 +102,14 @@ __global__ __launch_bounds__(FGNN_TPB) void mhsddmm_items_kernel(const fgnn_item
     float *scr = lds + fg_wave() * (64 * R);
     fg_lanemap<VEC, R> lm;
     if (lphp) lm.init_padded(lane, H, F, lphp); else lm.init(lane, HF, F);
-    sddmm_row_piece<VEC, R, FULL, LPH>(row, pb, pe, H, F, HF, lm, lane, scr, idx, pos, a, b, out);
+    sddmm_row_piece<VEC, R, FULL, LPH>(row, pb, pe, H, F, ld, ldo, lm, lane, scr, idx, pos, a, b, out);
 }
 
 static int mhsddmm_run(const char *fn, int N, int64_t E, int H, int F, const int32_t *row_ptr, const int32_t *col_ind, const float *a,
                        const float *b, float *out, const fgnn_schedule_t *sched, hipStream_t st)
 {
     FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1 && F >= 1, FGNN_ERR_SHAPE, "%s: bad sizes", fn);
-    FGNN_REQUIRE(H <= 64 && (int64_t)H * F <= 1024, FGNN_ERR_LIMIT, "%s: H=%d H*F=%lld unsupported", fn, H, (long long)H * F);
+    FGNN_REQUIRE(H <= 64 && F <= 1024, FGNN_ERR_LIMIT, "%s: H=%d F=%d unsupported (at most 64 heads of at most 1024 floats)", fn, H, F);
     FGNN_REQUIRE(row_ptr && (col_ind || E == 0) && a && b && (out || E == 0), FGNN_ERR_NULL, "%s: NULL argument", fn);
     FGNN_REQUIRE(E <= 2147483647LL, FGNN_ERR_LIMIT, "%s: E=%lld exceeds the 32-bit row_ptr", fn, (long long)E);
     if (sched) {
@@ -120,27 +121,35 @@ static int mhsddmm_run(const char *fn, int N, int64_t E, int H, int F, const int
                      "%s: the schedule must carry its edge positions (results are stored at the caller's positions)", fn);
     }
     if (N == 0 || E == 0) return 0;
-    const int HF = H * F;
-    fgnn_rowcfg cfg;
-    FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, fgnn_aligned16(a) && fgnn_aligned16(b), &cfg), FGNN_ERR_LIMIT, "%s: unsupported row width %d", fn, HF);
-    const int lphp = fgnn_pad_lph(cfg.vec, H, F);
-    if (lphp) { int w = H * lphp * 4; cfg.r = w <= 256 ? 1 : w <= 512 ? 2 : 4; cfg.full = false; }
-    const int lph = lphp ? lphp : fgnn_pick_lph(cfg.vec, F);
     const int64_t waves = sched ? sched->n_items : (E + SDDMM_CHUNK - 1) / SDDMM_CHUNK;
     if (waves == 0) return 0;
     const unsigned grid = (unsigned)((waves + FGNN_WPB - 1) / FGNN_WPB);
-    return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
-        return fgnn_dispatch_lph(VEC == 4 ? lph : 0, [&]<int LPH>() -> int {
-            const size_t shm = (size_t)FGNN_WPB * 64 * R * sizeof(float);
-            if (sched)
-                hipLaunchKernelGGL((mhsddmm_items_kernel<VEC, R, FULL, (VEC == 4 ? LPH : 0)>), dim3(grid), dim3(FGNN_TPB), shm, st, sched->items_dev,
-                                   sched->n_items, H, F, HF, lphp, row_ptr, fgnn_sched_idx(sched, col_ind), fgnn_sched_pos(sched), a, b, out);
-            else
-                hipLaunchKernelGGL((mhsddmm_kernel<VEC, R, FULL, (VEC == 4 ? LPH : 0)>), dim3(grid), dim3(FGNN_TPB), shm, st, N, E, H, F, HF, lphp,
-                                   row_ptr, col_ind, a, b, out);
-            return fgnn_launch_status("mhsddmm_kernel");
+    // rows of more than 1024 floats: passes over groups of heads on views of the wide arrays (heads are independent)
+    const int hmax = (int64_t)H * F <= 1024 ? H : std::max(1, 1024 / F);
+    for (int h0 = 0; h0 < H; h0 += hmax) {
+        const int hg = std::min(hmax, H - h0), HF = hg * F, ld = H * F;
+        const float *ag = a + (size_t)h0 * F, *bg = b + (size_t)h0 * F;
+        float *og = out + h0;
+        fgnn_rowcfg cfg;
+        FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, fgnn_aligned16(a) && fgnn_aligned16(b), &cfg), FGNN_ERR_LIMIT, "%s: unsupported row width %d", fn, HF);
+        const int lphp = fgnn_pad_lph(cfg.vec, hg, F);
+        if (lphp) { int w = hg * lphp * 4; cfg.r = w <= 256 ? 1 : w <= 512 ? 2 : 4; cfg.full = false; }
+        const int lph = lphp ? lphp : fgnn_pick_lph(cfg.vec, F);
+        int rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
+            return fgnn_dispatch_lph(VEC == 4 ? lph : 0, [&]<int LPH>() -> int {
+                const size_t shm = (size_t)FGNN_WPB * 64 * R * sizeof(float);
+                if (sched)
+                    hipLaunchKernelGGL((mhsddmm_items_kernel<VEC, R, FULL, (VEC == 4 ? LPH : 0)>), dim3(grid), dim3(FGNN_TPB), shm, st, sched->items_dev,
+                                       sched->n_items, hg, F, HF, ld, H, lphp, row_ptr, fgnn_sched_idx(sched, col_ind), fgnn_sched_pos(sched), ag, bg, og);
+                else
+                    hipLaunchKernelGGL((mhsddmm_kernel<VEC, R, FULL, (VEC == 4 ? LPH : 0)>), dim3(grid), dim3(FGNN_TPB), shm, st, N, E, hg, F, HF, ld, H, lphp,
+                                       row_ptr, col_ind, ag, bg, og);
+                return fgnn_launch_status("mhsddmm_kernel");
+            });
         });
-    });
+        if (rc) return rc;
+    }
+    return 0;
 }
 
 extern "C" int fgnn_mhsddmm(int N, int64_t E, int H, int F, const int32_t *row_ptr, const int32_t *col_ind, const float *a,

@@ -2,6 +2,7 @@
 //   multi-head SpMM with stored edge weights (mhspmm / spmm of the reference),
 //   GMMConv forward (Gaussian mixture weights computed on the fly, src/fused_gmmconv/gmmconv.cu:48-80),
 //   GMMConv backward in one pass over the CSC arrays, and the standalone Gaussian kernels.
+#include <algorithm>
 #include "fgnn_common.h"
 
 struct SpmmP {
@@ -13,6 +14,7 @@ struct SpmmP {
     int sum_h;      // != 0: out is [N,F], the sum over the H heads (GMMConv's .sum(1) fused into the store)
     const float *bias; const float *res;     // with sum_h: out[i,:] += bias[:] (+ res[i,:]) in the same store (either may be NULL)
     int own_order;  // != 0: per-edge arrays are indexed by the work list's own entry positions (pos is not applied)
+    int ld, ldo;    // floats between consecutive rows of feat / of out when they are views of wider arrays (0: HF)
 };
 __host__ __device__ static inline int spmm_pw(int HF) { return (HF + 3) & ~3; }
 
@@ -44,7 +46,7 @@ __device__ __forceinline__ void spmm_store_row(const SpmmP &p, int row, const fg
     if (!p.sum_h) {
 #pragma unroll
         for (int r = 0; r < R; ++r)
-            if (FULL || lm.ok[r]) T[r].store_nt(p.out + (size_t)row * p.HF + lm.eoff[r]);
+            if (FULL || lm.ok[r]) T[r].store_nt(p.out + (size_t)row * p.ldo + lm.eoff[r]);
         return;
     }
 #pragma unroll
@@ -68,10 +70,11 @@ __device__ __forceinline__ void spmm_store_row(const SpmmP &p, int row, const fg
 // Weight sources.  fill() runs with lanes-as-edges: lane t writes wl[h*64 + t] for every head.
 struct WAtt {
     const float *att;   // [E,H] or NULL (all ones)
+    int ld;             // floats between consecutive entries of att (H, or more when att is a view of a wider array)
     __device__ __forceinline__ void prepare(float *, int, int) const {}
     __device__ __forceinline__ void fill(float *wl, const float *, int lane, size_t pos, bool ok, int H) const
     {
-        for (int h = 0; h < H; ++h) wl[h * 64 + lane] = ok ? (att ? att[pos * H + h] : 1.f) : 0.f;
+        for (int h = 0; h < H; ++h) wl[h * 64 + lane] = ok ? (att ? att[pos * ld + h] : 1.f) : 0.f;
     }
 };
 struct WGauss {
@@ -123,7 +126,7 @@ __global__ __launch_bounds__(FGNN_TPB) void spmm_kernel(SpmmP p, WF wf, int shar
         size_t pos = p.pos_map ? (size_t)p.pos_map[orig] : (size_t)orig;
         wf.fill(wl, shared, lane, pos, ok, p.H);
         fg_wave_lds_sync();
-        fg_accum_chunk<VEC, R, FULL>(p.feat, p.HF, id, cnt, wl, lm, T);
+        fg_accum_chunk<VEC, R, FULL>(p.feat, p.ld, id, cnt, wl, lm, T);
         fg_wave_lds_sync();
     }
     if (slot < 0) {
@@ -176,7 +179,7 @@ __global__ __launch_bounds__(FGNN_TPB) void spmm_packed_kernel(SpmmP p, WF wf, i
                 const bool live = ei < cnt && pm.ok;
                 const int rid = __builtin_amdgcn_ds_bpermute((ei & 63) << 2, id);
                 w[u] = live ? wl[pm.hd * 64 + ei] : 0.f;
-                if (live) ld[u].load(p.feat + (size_t)rid * (size_t)p.HF + pm.eoff); else ld[u].zero();
+                if (live) ld[u].load(p.feat + (size_t)rid * (size_t)p.ld + pm.eoff); else ld[u].zero();
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) T.fma(w[u], ld[u]);
@@ -220,7 +223,7 @@ static int spmm_checks(const char *fn, int N, int64_t E, int H, int F, const fgn
 {
     FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1 && F >= 1, FGNN_ERR_SHAPE, "%s: bad sizes N=%d E=%lld H=%d F=%d", fn, N, (long long)E, H, F);
     FGNN_REQUIRE(E <= 2147483647LL, FGNN_ERR_LIMIT, "%s: E=%lld exceeds int32 positions", fn, (long long)E);
-    FGNN_REQUIRE(H <= 64 && (int64_t)H * F <= 1024, FGNN_ERR_LIMIT, "%s: H=%d, H*F=%lld unsupported (limits 64, 1024)", fn, H, (long long)H * F);
+    FGNN_REQUIRE(H <= 64 && F <= 1024, FGNN_ERR_LIMIT, "%s: H=%d, F=%d unsupported (at most 64 heads of at most 1024 floats)", fn, H, F);
     if (sched) {
         FGNN_REQUIRE(sched->ptr_dev == ptr && sched->n_rows == N && sched->n_edges == E, FGNN_ERR_SCHEDULE,
                      "%s: schedule was built for another pointer array", fn);
@@ -242,6 +245,8 @@ static int spmm_launch(const char *name, SpmmP p, WF wf, int shared_floats, cons
     p.idx = fgnn_sched_idx(sched, p.idx);
     p.pos = p.own_order ? nullptr : fgnn_sched_pos(sched);
     p.part = (float *)workspace;
+    if (p.ld == 0) p.ld = p.HF;
+    if (p.ldo == 0) p.ldo = p.HF;
     if (sched && sched->n_partials > 0) {
         size_t need = (size_t)sched->n_partials * spmm_pw(p.HF) * sizeof(float);
         FGNN_REQUIRE(workspace && workspace_bytes >= need, FGNN_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes", name, workspace_bytes, need);
@@ -314,9 +319,8 @@ extern "C" int fgnn_mhspmm(int N, int64_t E, int H, int F, const int32_t *ptr, c
     int rc = spmm_checks("fgnn_mhspmm", N, E, H, F, sched, ptr, idx);
     if (rc) return rc;
     FGNN_REQUIRE(ptr && (idx || E == 0) && feat && out, FGNN_ERR_NULL, "fgnn_mhspmm: NULL argument");
-    SpmmP p{};
-    p.ptr = ptr; p.idx = idx; p.pos_map = pos_map; p.feat = feat; p.out = out; p.N = N; p.H = H; p.F = F; p.HF = H * F;
-    WAtt wf{att};
+    const float *att_use = att;
+    int own_order = 0;
     hipStream_t st = (hipStream_t)stream;
     const size_t part_bytes = spmm_partial_bytes(sched, H, F), own_bytes = (size_t)E * H * sizeof(float);
     if (att && E > 0 && sched && sched->n_buckets > 0 && sched->bpos_dev && workspace && workspace_bytes >= part_bytes + own_bytes) {
@@ -329,11 +333,25 @@ extern "C" int fgnn_mhspmm(int N, int64_t E, int H, int F, const int32_t *ptr, c
             hipLaunchKernelGGL(att_own_order_kernel<1>, grid, dim3(256), 0, st, E, H, runs_per_xcd, sched->bpos_dev, pos_map, att, own);
         rc = fgnn_launch_status("att_own_order_kernel");
         if (rc) return rc;
-        wf.att = own;
-        p.pos_map = nullptr;
-        p.own_order = 1;            // the weights are indexed by the list's own entry positions
+        att_use = own;
+        pos_map = nullptr;
+        own_order = 1;              // the weights are indexed by the list's own entry positions
     }
-    return spmm_launch("fgnn_mhspmm", p, wf, 0, sched, fgnn_aligned16(feat) && fgnn_aligned16(out), workspace, workspace_bytes, st);
+    // Rows of more than 1024 floats (the reference serves any number of heads of up to 1024 floats each,
+    // src/fused_gat/fused_gat_SM.cu:518-522) go in passes over groups of heads: heads are independent, a pass
+    // works on a view of `hg` heads of the wide arrays (same row strides, shifted base).
+    const int hmax = (int64_t)H * F <= 1024 ? H : std::max(1, 1024 / F);
+    for (int h0 = 0; h0 < H; h0 += hmax) {
+        const int hg = std::min(hmax, H - h0);
+        SpmmP p{};
+        p.ptr = ptr; p.idx = idx; p.pos_map = pos_map; p.feat = feat + (size_t)h0 * F; p.out = out + (size_t)h0 * F;
+        p.N = N; p.H = hg; p.F = F; p.HF = hg * F; p.ld = p.ldo = H * F; p.own_order = own_order;
+        WAtt wf{att_use ? att_use + h0 : nullptr, H};
+        rc = spmm_launch("fgnn_mhspmm", p, wf, 0, sched, fgnn_aligned16(feat) && fgnn_aligned16(out) && (hmax == H || F % 4 == 0), workspace,
+                         workspace_bytes, st);
+        if (rc) return rc;
+    }
+    return 0;
 }
 
 extern "C" size_t fgnn_gmm_forward_workspace_bytes(const fgnn_schedule_t *sched, int K, int F)
@@ -352,6 +370,7 @@ extern "C" int fgnn_gmm_forward(int N, int64_t E, int K, int dim, int F, const i
 {
     int rc = spmm_checks("fgnn_gmm_forward", N, E, K, F, sched, ptr, idx);
     if (rc) return rc;
+    FGNN_REQUIRE((int64_t)K * F <= 1024, FGNN_ERR_LIMIT, "fgnn_gmm_forward: K*F=%lld > 1024 unsupported", (long long)K * F);
     FGNN_REQUIRE(dim >= 1 && dim <= 64 && K * dim <= 1024, FGNN_ERR_LIMIT, "fgnn_gmm_forward: dim=%d K*dim=%d unsupported", dim, K * dim);
     FGNN_REQUIRE(ptr && (idx || E == 0) && node_feat && (pseudo || E == 0) && mu && inv_sigma && out, FGNN_ERR_NULL, "fgnn_gmm_forward: NULL argument");
     FGNN_REQUIRE(sum_kernels >= 0 && sum_kernels <= 2, FGNN_ERR_SHAPE, "fgnn_gmm_forward: sum_kernels=%d (0, 1 or 2)", sum_kernels);
@@ -377,6 +396,7 @@ extern "C" int fgnn_gmm_forward_epilogue(int N, int64_t E, int K, int dim, int F
 {
     int rc = spmm_checks("fgnn_gmm_forward_epilogue", N, E, K, F, sched, ptr, idx);
     if (rc) return rc;
+    FGNN_REQUIRE((int64_t)K * F <= 1024, FGNN_ERR_LIMIT, "fgnn_gmm_forward_epilogue: K*F=%lld > 1024 unsupported", (long long)K * F);
     FGNN_REQUIRE(dim >= 1 && dim <= 64 && K * dim <= 1024, FGNN_ERR_LIMIT, "fgnn_gmm_forward_epilogue: dim=%d K*dim=%d unsupported", dim, K * dim);
     FGNN_REQUIRE(ptr && (idx || E == 0) && node_feat && (pseudo || E == 0) && mu && inv_sigma && out, FGNN_ERR_NULL,
                  "fgnn_gmm_forward_epilogue: NULL argument");
@@ -688,7 +708,7 @@ static int gmm_forward_shared(int N, int K, int dim, int F, const int32_t *ptr, 
         fgnn_rowcfg cfg;
         FGNN_REQUIRE(fgnn_pick_rowcfg(HF, F, true, &cfg), FGNN_ERR_LIMIT, "fgnn_gmm_forward: unsupported row width %d", HF);
         SpmmP mp{};
-        mp.part = p.part; mp.out = out; mp.N = N; mp.H = K; mp.F = F; mp.HF = HF;
+        mp.part = p.part; mp.out = out; mp.N = N; mp.H = K; mp.F = F; mp.HF = HF; mp.ld = mp.ldo = HF;
         unsigned g2 = (unsigned)((sched->n_split + FGNN_WPB - 1) / FGNN_WPB);
         rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
             hipLaunchKernelGGL((spmm_merge_kernel<VEC, R>), dim3(g2), dim3(FGNN_TPB), 0, st, mp, sched->split_dev, sched->n_split);
@@ -920,6 +940,7 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
 {
     int rc = spmm_checks("fgnn_gmm_backward", N, E, K, F, sched_csc, col_ptr, row_ind);
     if (rc) return rc;
+    FGNN_REQUIRE((int64_t)K * F <= 1024, FGNN_ERR_LIMIT, "fgnn_gmm_backward: K*F=%lld > 1024 unsupported", (long long)K * F);
     FGNN_REQUIRE(dim >= 1 && dim <= 64 && K * dim <= 1024, FGNN_ERR_LIMIT, "fgnn_gmm_backward: dim=%d K*dim=%d unsupported", dim, K * dim);
     FGNN_REQUIRE(col_ptr && (row_ind || E == 0) && node_feat && (pseudo || E == 0) && mu && inv_sigma &&
                      grad_out && grad_feat && (grad_pseudo || E == 0) && grad_mu && grad_sigma,
@@ -971,7 +992,7 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
             if (rc) return rc;
             if (sched_csc->n_split > 0) {
                 SpmmP mp{};
-                mp.part = part; mp.out = grad_feat; mp.N = N; mp.H = K; mp.F = F; mp.HF = HF;
+                mp.part = part; mp.out = grad_feat; mp.N = N; mp.H = K; mp.F = F; mp.HF = HF; mp.ld = mp.ldo = HF;
                 unsigned g2 = (unsigned)((sched_csc->n_split + FGNN_WPB - 1) / FGNN_WPB);
                 rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
                     hipLaunchKernelGGL((spmm_merge_kernel<VEC, R>), dim3(g2), dim3(FGNN_TPB), 0, st, mp, sched_csc->split_dev, sched_csc->n_split);
@@ -997,7 +1018,7 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
             if (rc2) return rc2;
             if (sched_csc->n_split > 0) {
                 SpmmP mp{};
-                mp.part = part; mp.out = grad_feat; mp.N = N; mp.H = K; mp.F = F; mp.HF = HF;
+                mp.part = part; mp.out = grad_feat; mp.N = N; mp.H = K; mp.F = F; mp.HF = HF; mp.ld = mp.ldo = HF;
                 unsigned g2 = (unsigned)((sched_csc->n_split + FGNN_WPB - 1) / FGNN_WPB);
                 hipLaunchKernelGGL((spmm_merge_kernel<VEC, R>), dim3(g2), dim3(FGNN_TPB), 0, st, mp, sched_csc->split_dev, sched_csc->n_split);
                 return fgnn_launch_status("spmm_merge_kernel");

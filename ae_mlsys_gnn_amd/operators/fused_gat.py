@@ -53,8 +53,17 @@ class gat_native:
 
     @staticmethod
     def gat_backward(negative_slope, row_ptr, col_ind, col_ptr, row_ind, edge_max, edge_sum, in_feat, attn_row, attn_col,
-                     grad, *, out_feat=None, out2=None, cc=None, permute=None, e_lrelu=None, e_soft=None,
+                     grad, *, out_feat=None, out2=None, cc=None, permute=None, e_lrelu=None, e_soft=None, e_soft_order="csr",
                      use_schedule=True):
+        """e_soft: stashed attention [E,H].  e_soft_order="csr": the CSR-ordered stash of gat_forward(stash=True), read
+        through `permute` (required); e_soft_order="own": the stash of gat_stash_own_order (entry order of this pass,
+        signed), streamed.  The two layouts are not interchangeable and nothing in the data tells them apart."""
+        if e_soft_order not in ("csr", "own"):
+            raise _lib.FgnnError("gat_backward: e_soft_order must be 'csr' or 'own', got %r" % (e_soft_order,))
+        own = e_soft is not None and e_soft_order == "own"
+        if e_soft is not None and not own and permute is None:
+            raise _lib.FgnnError("gat_backward: stashed attention needs permute (pass e_soft_order='own' for a stash written by "
+                                 "gat_stash_own_order)")
         require_cuda(grad, in_feat, col_ptr, row_ind, attn_row, attn_col, edge_max, edge_sum, row_ptr, col_ind, out_feat, out2, cc,
                      permute, e_soft)
         # the kernels take raw pointers: every tensor is made contiguous and checked here, so a strided view
@@ -84,19 +93,25 @@ class gat_native:
         grad_attn_row = torch.empty((n, h), dtype=torch.float32, device=dev)
         grad_attn_col = torch.empty((n, h), dtype=torch.float32, device=dev)
         recompute = out_feat is None or out2 is None or cc is None
-        sched_csc = schedule_for(col_ptr, idx_tensor=row_ind, need_positions=e_soft is not None and permute is not None) if use_schedule else None
+        sched_csc = schedule_for(col_ptr, idx_tensor=row_ind, need_positions=e_soft is not None and not own) if use_schedule else None
         sched_csr = schedule_for(row_ptr, idx_tensor=col_ind, need_positions=False) if (use_schedule and recompute) else None
         hc = sched_csc.handle if sched_csc is not None else None
         hr = sched_csr.handle if sched_csr is not None else None
         with torch.cuda.device(dev):
-            ws, wsb = workspace(lib().fgnn_gat_backward_workspace_bytes(n, h, f, hc, hr, int(recompute)), dev)
-            check(lib().fgnn_gat_backward(n, e, h, f, float(negative_slope), ptr(row_ptr), ptr(col_ind), ptr(col_ptr),
-                                          ptr(row_ind), ptr(permute), ptr(e_lrelu), ptr(e_soft), ptr(edge_max),
-                                          ptr(edge_sum), ptr(in_feat), ptr(attn_row), ptr(attn_col),
-                                          None if recompute else ptr(out_feat), None if recompute else ptr(out2),
-                                          None if recompute else ptr(cc), ptr(grad), ptr(grad_feat), ptr(grad_attn_row),
-                                          ptr(grad_attn_col), hc, hr, ptr(ws), wsb, stream_ptr()),
-                  "fgnn_gat_backward")
+            ws, wsb = workspace(lib().fgnn_gat_backward_workspace_bytes(n, h, f, hc, hr, int(recompute) | (2 if e_soft is not None else 0)), dev)
+            saved = (None if recompute else ptr(out_feat), None if recompute else ptr(out2), None if recompute else ptr(cc))
+            if own:
+                check(lib().fgnn_gat_backward_own_order(n, e, h, f, float(negative_slope), ptr(row_ptr), ptr(col_ind), ptr(col_ptr),
+                                                        ptr(row_ind), ptr(e_soft), ptr(edge_max), ptr(edge_sum), ptr(in_feat),
+                                                        ptr(attn_row), ptr(attn_col), *saved, ptr(grad), ptr(grad_feat),
+                                                        ptr(grad_attn_row), ptr(grad_attn_col), hc, hr, ptr(ws), wsb, stream_ptr()),
+                      "fgnn_gat_backward_own_order")
+            else:
+                check(lib().fgnn_gat_backward(n, e, h, f, float(negative_slope), ptr(row_ptr), ptr(col_ind), ptr(col_ptr),
+                                              ptr(row_ind), ptr(permute), ptr(e_lrelu), ptr(e_soft), ptr(edge_max),
+                                              ptr(edge_sum), ptr(in_feat), ptr(attn_row), ptr(attn_col), *saved, ptr(grad),
+                                              ptr(grad_feat), ptr(grad_attn_row), ptr(grad_attn_col), hc, hr, ptr(ws), wsb, stream_ptr()),
+                      "fgnn_gat_backward")
         return grad_feat, grad_attn_row, grad_attn_col
 
 
@@ -176,14 +191,16 @@ class FusedGATFunction_stash(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute):
+        need = _needs_grad(ctx)
         attn_row, attn_col, in_feat = _contig(attn_row), _contig(attn_col), _contig(in_feat)
         row_ptr, col_ind, col_ptr, row_ind, permute = _contig(row_ptr), _contig(col_ind), _contig(col_ptr), _contig(row_ind), _contig(permute)
         out, edge_max, edge_sum, out2, cc, _, _ = gat_native.gat_forward(
-            attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, need_aux=True)
-        # the stash is this function's own tensor: it is written in the order in which the backward walks the edges
-        e_soft = gat_native.gat_stash_own_order(negative_slope, col_ptr, row_ind, edge_max, edge_sum, attn_row, attn_col)
-        ctx.save_for_backward(row_ptr, col_ind, col_ptr, row_ind, permute, e_soft, in_feat, attn_row, attn_col,
-                              edge_max, edge_sum, out, out2, cc)
+            attn_row, attn_col, row_ptr, col_ind, negative_slope, in_feat, need_aux=need)
+        if need:       # inference / no_grad: no stash pass, no [E,H] tensor, no CSC work list
+            # the stash is this function's own tensor: it is written in the order in which the backward walks the edges
+            e_soft = gat_native.gat_stash_own_order(negative_slope, col_ptr, row_ind, edge_max, edge_sum, attn_row, attn_col)
+            ctx.save_for_backward(row_ptr, col_ind, col_ptr, row_ind, permute, e_soft, in_feat, attn_row, attn_col,
+                                  edge_max, edge_sum, out, out2, cc)
         ctx.negative_slope = negative_slope
         return out
 
@@ -193,7 +210,7 @@ class FusedGATFunction_stash(torch.autograd.Function):
          edge_max, edge_sum, out, out2, cc) = ctx.saved_tensors
         grad_feat, grad_attn_row, grad_attn_col = gat_native.gat_backward(
             ctx.negative_slope, row_ptr, col_ind, col_ptr, row_ind, edge_max, edge_sum, in_feat, attn_row, attn_col,
-            grad_out.contiguous(), out_feat=out, out2=out2, cc=cc, permute=None, e_soft=e_soft)
+            grad_out.contiguous(), out_feat=out, out2=out2, cc=cc, e_soft=e_soft, e_soft_order="own")
         return grad_attn_row, grad_attn_col, None, None, None, None, None, grad_feat, None
 
 

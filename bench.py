@@ -292,7 +292,7 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
     ms_sf = ms_fwd + ms_sw
     ms_sb, _, _ = time_calls(
         lambda: gat_native.gat_backward(slope, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, o[1], o[2], h, a_row, a_col, go,
-                                        out_feat=o[0], out2=o[3], cc=o[4], permute=None, e_soft=own),
+                                        out_feat=o[0], out2=o[3], cc=o[4], e_soft=own, e_soft_order="own"),
         max(3, args.steps // 4), 1)
     stash_bytes = e * heads * 4
     del own

@@ -125,9 +125,15 @@ int    fgnn_gat_forward(int N, int64_t E, int H, int F,
 /* Replaces fused_gat_SM.gat_backward (src/fused_gat/fused_gat_SM.cpp:40-124, host launcher
  * fused_gat_SM.cu:865-893); with permute/e_softmax non-NULL it reads the stashed attention
  * instead of recomputing it (fused_gat_stash.gat_backward, fused_gat_stash.cu:776-804;
- * fused_gat.gat_backward, fused_gat.cu:641-670); with e_softmax non-NULL and permute == NULL the stash is taken to
- * be in this pass's own entry order (fgnn_gat_stash_own_order).  e_lrelu is accepted for the reference's argument
- * list and not read: the sign of the pre-activation is that of attn_row + attn_col.
+ * fused_gat.gat_backward, fused_gat.cu:641-670): e_softmax is then the CSR-ordered [E,H] array of fgnn_gat_forward and
+ * permute is required (FGNN_ERR_NULL without it; a stash written by fgnn_gat_stash_own_order has another layout and goes
+ * to fgnn_gat_backward_own_order).  e_lrelu is accepted for the reference's argument list and not read: the sign of the
+ * pre-activation is that of attn_row + attn_col.
+ * Rows of more than 1024 floats (any number of heads <= 64 of up to 1024 floats each, the range of
+ * fused_gat_SM.cu:518-522, :843-847) are served in passes over groups of heads through contiguous slices kept in the
+ * workspace; they need a schedule (FGNN_ERR_SCHEDULE otherwise), and the workspace functions include the slices.
+ * need_recompute of the workspace function: bit 0 = out_feat/aux_out2/aux_c will be NULL, bit 1 = a stash will be passed
+ * (only rows of more than 1024 floats need room for it).
  * Inputs as the reference's plus out_feat/aux_out2/aux_c from the forward; when those three are
  * NULL they are recomputed into the workspace from (row_ptr, col_ind) first.
  * Outputs: grad_feat [N,H,F], grad_attn_row, grad_attn_col [N,H]; all fully overwritten and
@@ -147,12 +153,28 @@ int    fgnn_gat_backward(int N, int64_t E, int H, int F, float negative_slope,
                          const fgnn_schedule_t *sched_csc, const fgnn_schedule_t *sched_csr,
                          void *workspace, size_t workspace_bytes, void *stream);
 
+/* fgnn_gat_backward reading the stash of fgnn_gat_stash_own_order (below): e_softmax_own[q,h] in the entry order of this
+ * pass under the same sched_csc, sign bit set where the pre-activation is not positive.  The layout is a property of the
+ * entry point, not of a NULL argument: a CSR-ordered stash handed in here (or the reverse) would be read as the wrong
+ * edges' weights without any error.  No counterpart in the reference, whose stash is CSR-ordered
+ * (src/fused_gat/fused_gat_stash.cu:444-464). */
+int    fgnn_gat_backward_own_order(int N, int64_t E, int H, int F, float negative_slope,
+                                   const int32_t *row_ptr, const int32_t *col_ind,
+                                   const int32_t *col_ptr, const int32_t *row_ind,
+                                   const float *e_softmax_own, const float *edge_max, const float *edge_sum,
+                                   const float *in_feat, const float *attn_row, const float *attn_col,
+                                   const float *out_feat, const float *aux_out2, const float *aux_c,
+                                   const float *grad_out,
+                                   float *grad_feat, float *grad_attn_row, float *grad_attn_col,
+                                   const fgnn_schedule_t *sched_csc, const fgnn_schedule_t *sched_csr,
+                                   void *workspace, size_t workspace_bytes, void *stream);
+
 /* The stashed attention of the stash variants in the ORDER OF THE BACKWARD PASS: e_softmax_own[q,h] = alpha of
  * entry q of the walk of (col_ptr, row_ind) under sched_csc (its bucket-ordered entry order when it is XCD-aware,
  * plain CSC order otherwise or with sched_csc == NULL), computed from the forward's row statistics; the sign bit of
  * the stored value is set when the edge's pre-activation is not positive (alpha itself is >= 0), so the backward
  * needs no other per-edge or per-destination data than <grad_out, out>.
- * fgnn_gat_backward called with this array as e_softmax, permute == NULL and the same sched_csc then streams the
+ * fgnn_gat_backward_own_order called with this array and the same sched_csc then streams the
  * stash instead of gathering it through permute (114.8 M edges, 8 heads: backward 10.5 -> about 7 ms).  The
  * reference keeps its stash in CSR order and transposes while reading (src/fused_gat/fused_gat_stash.cu:444-464);
  * a caller that owns the stashed tensor (the autograd function does) is free to keep it in this order instead. */

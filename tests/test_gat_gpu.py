@@ -432,7 +432,7 @@ def test_gat_stash_in_both_orders_through_native_calls(h, f, monkeypatch):
                                           out2=o[3], cc=o[4], permute=gd.permute, e_soft=o[6], use_schedule=use_schedule)
         own = gat_native.gat_stash_own_order(0.2, gd.col_ptr, gd.row_ind, o[1], o[2], ard, acd, use_schedule=use_schedule)
         res_own = gat_native.gat_backward(0.2, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, o[1], o[2], xd, ard, acd, god, out_feat=o[0],
-                                          out2=o[3], cc=o[4], permute=None, e_soft=own, use_schedule=use_schedule)
+                                          out2=o[3], cc=o[4], e_soft=own, e_soft_order="own", use_schedule=use_schedule)
         torch.cuda.synchronize()
         for tag, res in (("CSR-ordered stash", res_csr), ("own-order stash", res_own)):
             _check((o[0],) + tuple(res), ref, g, x, ar, ac, go, 0.2, tag=" (%s, buckets %s, schedule %s)" % (tag, buckets, use_schedule))
@@ -465,4 +465,75 @@ def test_fusescatter_pipeline_of_small_operators(h, f, monkeypatch):
     monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
     _lib.clear_schedule_cache()
     _run(graphs.rmat_graph(1500, 90000, seed=62), h, f, variant="pipeline", slope=0.05)
+    _lib.clear_schedule_cache()
+
+
+@pytest.mark.parametrize("variant", ["sm", "stash"])
+@pytest.mark.parametrize("h,f", [(8, 256), (4, 512), (2, 1024), (5, 300), (3, 501), (9, 128)])
+def test_gat_rows_wider_than_1024_floats(h, f, variant, monkeypatch):
+    """Any number of heads of up to 1024 floats each (the range of the reference's recompute and stash kernels,
+    src/fused_gat/fused_gat_SM.cu:518-522): passes over groups of heads, the last group smaller than the others
+    ((5, 300): 3 + 2, (3, 501): 2 + 1 in the scalar layout, (9, 128): 8 + 1), with split and merged rows and an XCD-aware
+    schedule."""
+    from ae_mlsys_gnn_amd import _lib
+    monkeypatch.setenv("FGNN_SEG_LEN", "256")
+    _lib.clear_schedule_cache()
+    _run(degree_edge_graph(n=60, seed=71), h, f, variant=variant)
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
+    monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+    _lib.clear_schedule_cache()
+    _run(graphs.rmat_graph(300, 9000, seed=72), h, f, variant=variant, slope=0.05)
+    _lib.clear_schedule_cache()
+
+
+def test_gat_wide_rows_through_the_reference_signatures(monkeypatch):
+    """H*F > 1024 with the CSR-ordered stash of the reference's gat_forward / gat_backward pair (read through permute) and
+    with a backward that is handed neither out nor the auxiliary outputs and recomputes them, group by group."""
+    from ae_mlsys_gnn_amd.operators.fused_gat import gat_native
+    h, f = 6, 256
+    g = graphs.add_csc_torch(degree_edge_graph(n=50, seed=73))
+    x, ar, ac, go = gat_inputs(g, h, f, 9)
+    ref = _oracle_fwd_bwd(g, x, ar, ac, go, 0.2)
+    gd = g.to("cuda:0")
+    xd, ard, acd, god = (t.float().to("cuda:0") for t in (x, ar, ac, go))
+    o = gat_native.gat_forward(ard, acd, gd.row_ptr, gd.col_ind, 0.2, xd, stash=True)
+    alpha = orc.gat_forward(ar, ac, g.row_ptr, g.col_ind, 0.2, x, return_edge=True)[2]
+    assert_close(o[6], alpha, "e_softmax in CSR order, wide rows")
+    res = gat_native.gat_backward(0.2, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, o[1], o[2], xd, ard, acd, god, out_feat=o[0], out2=o[3],
+                                  cc=o[4], permute=gd.permute, e_soft=o[6])
+    _check((o[0],) + tuple(res), ref, g, x, ar, ac, go, 0.2, tag=" (wide rows, CSR-ordered stash)")
+    res = gat_native.gat_backward(0.2, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, o[1], o[2], xd, ard, acd, god)
+    _check((o[0],) + tuple(res), ref, g, x, ar, ac, go, 0.2, tag=" (wide rows, recomputing backward)")
+
+
+def test_gat_stash_layouts_are_not_interchangeable():
+    """A CSR-ordered stash without permute is refused (by the wrapper and by the C entry) instead of being read as a stash
+    in the backward pass's own order, which would take every weight from the wrong edge; the stash function writes no
+    stash when nothing needs a gradient."""
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd._lib import check, lib, ptr, stream_ptr
+    from ae_mlsys_gnn_amd.operators import fused_gat as fg
+    g = graphs.add_csc_torch(graphs.rmat_graph(200, 3000, seed=74)).to("cuda:0")
+    n, h, f = g.n, 4, 16
+    x, ar, ac = torch.randn(n, h, f, device="cuda:0"), torch.randn(n, h, device="cuda:0"), torch.randn(n, h, device="cuda:0")
+    o = fg.gat_native.gat_forward(ar, ac, g.row_ptr, g.col_ind, 0.2, x, stash=True)
+    go = torch.randn_like(x)
+    with pytest.raises(_lib.FgnnError, match="needs permute"):
+        fg.gat_native.gat_backward(0.2, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, o[1], o[2], x, ar, ac, go, out_feat=o[0], out2=o[3], cc=o[4],
+                                   e_soft=o[6])
+    with pytest.raises(_lib.FgnnError, match="e_soft_order"):
+        fg.gat_native.gat_backward(0.2, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, o[1], o[2], x, ar, ac, go, e_soft=o[6], e_soft_order="csc")
+    ws = torch.empty(lib().fgnn_gat_backward_workspace_bytes(n, h, f, None, None, 0) // 4 + 64, device="cuda:0")
+    outs = [torch.empty_like(x), torch.empty_like(ar), torch.empty_like(ac)]
+    rc = lib().fgnn_gat_backward(n, g.n_edges, h, f, 0.2, ptr(g.row_ptr), ptr(g.col_ind), ptr(g.col_ptr), ptr(g.row_ind), None, None, ptr(o[6]),
+                                 ptr(o[1]), ptr(o[2]), ptr(x), ptr(ar), ptr(ac), ptr(o[0]), ptr(o[3]), ptr(o[4]), ptr(go), ptr(outs[0]),
+                                 ptr(outs[1]), ptr(outs[2]), None, None, ptr(ws), ws.numel() * 4, stream_ptr())
+    assert rc == -1 and b"fgnn_gat_backward_own_order" in lib().fgnn_last_error()
+    # no gradient wanted: the stash variant keeps nothing and builds no CSC work list
+    _lib.clear_schedule_cache()
+    with torch.no_grad():
+        out = fg.fused_gat_stash_op(ar, ac, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, 0.2, x, g.permute)
+    assert torch.equal(out, o[0])
+    keys = [k for k in _lib._sched_cache if k[0] == g.col_ptr.data_ptr()]
+    assert not keys, "a no_grad call of the stash variant built a schedule of col_ptr"
     _lib.clear_schedule_cache()

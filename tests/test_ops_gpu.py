@@ -508,10 +508,14 @@ def test_error_paths_return_codes_not_aborts():
     from ae_mlsys_gnn_amd._lib import FgnnError
     from ae_mlsys_gnn_amd.operators import fused_gat as fg
     g = graphs.add_csc_torch(graphs.uniform_graph(64, 256)).to(DEV)
-    x = torch.randn(64, 8, 256, device=DEV)       # H*F = 2048 > limit
-    a = torch.randn(64, 8, device=DEV)
+    x = torch.randn(64, 2, 1028, device=DEV)       # more than 1024 floats per head
+    a = torch.randn(64, 2, device=DEV)
     with pytest.raises(FgnnError, match="1024"):
         fg.fused_gat_op(a, a, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, 0.2, x)
+    x = torch.randn(64, 8, 256, device=DEV)       # H*F = 2048: served in head groups, but only under a schedule
+    a = torch.randn(64, 8, device=DEV)
+    with pytest.raises(FgnnError, match="need a schedule"):
+        fg.gat_native.gat_forward(a, a, g.row_ptr, g.col_ind, 0.2, x, use_schedule=False)
     with pytest.raises(FgnnError, match="GPU only"):
         fg.fused_gat_op(a.cpu(), a.cpu(), g.row_ptr.cpu(), g.col_ind.cpu(), g.col_ptr.cpu(), g.row_ind.cpu(), 0.2, x.cpu())
     with pytest.raises(FgnnError, match="int32"):
@@ -1146,3 +1150,32 @@ def test_edge_softmax_rows_beyond_the_register_cache(nh):
     assert_close_sum(hd.grad, hl.grad, ref.detach() * (go.abs() + dot_abs[dst]), "edge_softmax grad of long rows", c=c)
     sums = orc.segment_sums(g.row_ptr, out.detach().cpu().double())
     assert float((sums - (torch.tensor(lens) > 0).double().view(-1, 1)).abs().max()) < 1e-5
+
+
+@pytest.mark.parametrize("h,f", [(8, 256), (3, 501), (5, 300)])
+def test_mhspmm_and_mhsddmm_rows_wider_than_1024_floats(h, f, monkeypatch):
+    """Head-group passes over views of the wide arrays (row stride H*F, shifted base), with and without an XCD-aware list."""
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd.operators import mhspmm as op
+    for buckets in ("0", "1"):
+        monkeypatch.setenv("FGNN_XCD_BUCKETS", buckets)
+        monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+        monkeypatch.setenv("FGNN_SEG_LEN", "256")
+        _lib.clear_schedule_cache()
+        g = graphs.add_csc_torch(degree_edge_graph(n=60, seed=81))
+        gen = torch.Generator().manual_seed(h * f)
+        feat = torch.randn(g.n, h, f, generator=gen, dtype=torch.float64)
+        att = torch.randn(g.n_edges, h, generator=gen, dtype=torch.float64)
+        go = torch.randn(g.n, h, f, generator=gen, dtype=torch.float64)
+        fl, al = feat.clone().requires_grad_(True), att.clone().requires_grad_(True)
+        ref = orc.mhspmm(g.row_ptr, g.col_ind, al, fl)
+        ref.backward(go)
+        gd = g.to(DEV)
+        fd, ad = feat.float().to(DEV).requires_grad_(True), att.float().to(DEV).requires_grad_(True)
+        out = op.csrmhspmm(gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, gd.permute, fd, ad)
+        out.backward(go.float().to(DEV))
+        s_out, (s_att, s_feat) = orc.multilinear_abs_sums(lambda a, x: orc.mhspmm(g.row_ptr, g.col_ind, a, x), (att, feat), go)
+        assert_close_sum(out, ref.detach(), s_out, "mhspmm, wide rows, buckets " + buckets)
+        assert_close_sum(fd.grad, fl.grad, s_feat, "mhspmm grad feat, wide rows, buckets " + buckets)
+        assert_close_sum(ad.grad, al.grad, s_att, "mhspmm grad att (mhsddmm), wide rows, buckets " + buckets)
+    _lib.clear_schedule_cache()

@@ -27,17 +27,21 @@ def assert_close(got, ref, what, rtol=RTOL, atol=ATOL):
 # largely cancel) cannot be held to a bar relative to the RESULT: fp32 rounding scales with the sum of
 # the absolute summands S.  Their bar is  rtol*|ref| + max(atol, C_SUM * 2^-24 * S)  with S from the
 # oracle (gat_abs_sums / gmm_abs_sums: elementary products of the inputs, no cancellation inside).
-# C_SUM counts the roundings a summand carries at unit roundoff 2^-24 apart from its exponent: exp2, the
-# 1/sum normalisation, the weight product, the dot product feeding it, the accumulation (partial sums,
-# merges) -- 16 is that count with a factor of ~2 to spare and is not tuned per test.  A weight
-# exp(v) inherits the ABSOLUTE rounding of v as a relative error: forming v and subtracting the maximum
-# are 4 roundings of size 2^-24 * |v|, so operators with an exponential add 4 * max|v| (c_exp).
+# C_SUM stands for the roundings a summand carries at unit roundoff 2^-24 apart from its exponent (exp2, the
+# 1/sum normalisation, the weight product, the dot product feeding it, the accumulation).  A weight
+# exp(v) inherits the ABSOLUTE rounding of v as a relative error, so operators with an exponential add
+# one unit per unit of max|v| (c_exp).  Both constants are set from measurement, not from a worst-case
+# count: every comparison records how much of its allowance it used (PARITY_LOG below), the largest share
+# over the whole suite is 0.38 (sequential per-thread sums of 700 terms) and 0.22 at the benchmark sizes, and
+# the full-size tests assert that no element uses more than half (max_ratio = 0.5).  With the constants of a
+# worst-case count (16 and 4 per unit) no element used more than a tenth.  Not tuned per test.
 EPS32 = 2.0 ** -24
-C_SUM = 16.0
+C_SUM = 4.0
+MAX_RATIO = 0.5
 
 
 def c_exp(max_abs_exponent):
-    return C_SUM + 4.0 * float(max_abs_exponent)
+    return C_SUM + 1.0 * float(max_abs_exponent)
 
 
 # Every assert_close_sum call leaves a record here: how much of the derived allowance the comparison needed.

@@ -30,6 +30,8 @@ _SIGNATURES = {
     "fgnn_schedule_take_positions": (c_int, [c_void_p, c_void_p, c_void_p]),
     "fgnn_schedule_destroy": (None, [c_void_p]),
     "fgnn_schedule_num_items": (c_int, [c_void_p]),
+    "fgnn_schedule_num_buckets": (c_int, [c_void_p]),
+    "fgnn_xcd_mapping_for": (c_int, [ctypes.c_char_p, c_int]),
     "fgnn_schedule_num_partials": (c_int, [c_void_p]),
     "fgnn_schedule_num_edges": (c_int64, [c_void_p]),
     "fgnn_schedule_device_bytes": (c_size_t, [c_void_p]),
@@ -157,7 +159,7 @@ class Schedule:
     """Degree-binned work list of one pointer array (row_ptr or col_ptr).  With `idx_tensor` it is
     the XCD-aware form: long rows are cut by source bucket and each XCD gets one bucket."""
 
-    def __init__(self, ptr_tensor, seg_len=0, idx_tensor=None, min_deg=0, with_positions=True):
+    def __init__(self, ptr_tensor, seg_len=0, idx_tensor=None, min_deg=0, with_positions=True, n_cols=None):
         require_cuda(ptr_tensor)
         self.ptr_tensor = as_i32(ptr_tensor)      # keeps the device memory alive
         self.idx_tensor = None if idx_tensor is None else as_i32(idx_tensor)
@@ -165,8 +167,11 @@ class Schedule:
         handle = c_void_p()
         with torch.cuda.device(self.ptr_tensor.device):
             if self.idx_tensor is not None and os.environ.get("FGNN_VALIDATE", "0") not in ("0", ""):
-                # opt-in: range-check the graph once, when its work list is built, before any gather kernel runs
-                check(lib().fgnn_validate_graph(ptr(self.ptr_tensor), ptr(self.idx_tensor), self.n_rows, self.n_rows,
+                # opt-in: range-check the graph once, when its work list is built, before any gather kernel runs.  The ids
+                # index another array than the pointer array's rows (mhspmm / csrspmm: the gathered matrix), so the bound is
+                # the caller's n_cols; without one only the pointer array and the sign of the ids can be checked
+                bound = int(n_cols) if n_cols is not None else 2147483647
+                check(lib().fgnn_validate_graph(ptr(self.ptr_tensor), ptr(self.idx_tensor), self.n_rows, bound,
                                                 self.idx_tensor.numel(), stream_ptr()), "fgnn_validate_graph")
             if self.idx_tensor is None:
                 check(lib().fgnn_schedule_create(ptr(self.ptr_tensor), self.n_rows, int(seg_len), stream_ptr(),
@@ -177,6 +182,7 @@ class Schedule:
                       "fgnn_schedule_create_bucketed")
         self.handle = handle
         self.n_items = lib().fgnn_schedule_num_items(handle)
+        self.n_buckets = lib().fgnn_schedule_num_buckets(handle)     # 0: plain list (also when the device lacks the XCD mapping)
         self.n_partials = lib().fgnn_schedule_num_partials(handle)
         self.n_edges = lib().fgnn_schedule_num_edges(handle)
         self.own_order = False
@@ -270,12 +276,13 @@ def xcd_buckets_enabled(ptr_tensor, idx_numel=None) -> bool:
 
 
 @_locked
-def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True, own_order=False) -> Schedule:
+def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True, own_order=False, n_cols=None) -> Schedule:
     """Cached schedule of a pointer array.  The cache entry holds the tensors, so their device
     addresses cannot be reused while the entry lives; in-place edits bump `_version`.
     idx_tensor: the index array, for operators that may use an XCD-aware schedule.
     need_positions: whether the operator has per-edge tensors (an XCD-aware schedule then also keeps
     the caller's position of every entry, 4*E bytes more); a schedule with positions serves both.
+    n_cols: rows of the array the ids index, for the opt-in FGNN_VALIDATE check (None: only ids >= 0 is checked).
     own_order: a schedule of its own (never shared with the other kinds) whose position map was taken
     out (`edge_positions`): operators called with it take per-edge tensors in the schedule's order."""
     if seg_len is None:
@@ -301,7 +308,7 @@ def schedule_for(ptr_tensor, seg_len=None, idx_tensor=None, need_positions=True,
         k = key(False)
         s = _sched_cache.get(k)
     if s is None:
-        s = Schedule(ptr_tensor, seg_len, idx_tensor, min_deg, with_positions=need_positions)
+        s = Schedule(ptr_tensor, seg_len, idx_tensor, min_deg, with_positions=need_positions, n_cols=n_cols)
         _sched_cache[k] = s
         while len(_sched_cache) > _SCHED_CACHE_MAX:
             _sched_cache.popitem(last=False)

@@ -131,11 +131,12 @@ extern "C" int fgnn_edgeconv_forward_lrelu(int N, int n_src, int F, int k, const
     return edgeconv_forward_run("fgnn_edgeconv_forward_lrelu", N, n_src, F, k, src_ind, h_src, h_dst, out_slope, out, argmax, stream);
 }
 
-static int edgeconv_backward_run(int N, int n_src, int F, const int32_t *argmax, const float *grad_out, const float *act_out, float act_slope,
-                                 float *grad_src, float *grad_dst, void *stream)
+// fn: the entry point the caller used, for the error messages
+static int edgeconv_backward_run(const char *fn, int N, int n_src, int F, const int32_t *argmax, const float *grad_out, const float *act_out,
+                                 float act_slope, float *grad_src, float *grad_dst, void *stream)
 {
-    FGNN_REQUIRE(N >= 0 && n_src >= 0 && F >= 1, FGNN_ERR_SHAPE, "fgnn_edgeconv_backward: bad sizes");
-    FGNN_REQUIRE(argmax && grad_out && grad_src, FGNN_ERR_NULL, "fgnn_edgeconv_backward: NULL argument");
+    FGNN_REQUIRE(N >= 0 && n_src >= 0 && F >= 1, FGNN_ERR_SHAPE, "%s: bad sizes", fn);
+    FGNN_REQUIRE(argmax && grad_out && grad_src, FGNN_ERR_NULL, "%s: NULL argument", fn);
     hipStream_t st = (hipStream_t)stream;
     int rc = fgnn_fill_f32(grad_src, (size_t)n_src * F, 0.f, st);
     if (rc) return rc;
@@ -149,7 +150,7 @@ static int edgeconv_backward_run(int N, int n_src, int F, const int32_t *argmax,
 extern "C" int fgnn_edgeconv_backward(int N, int n_src, int F, const int32_t *argmax, const float *grad_out,
                                       float *grad_src, void *stream)
 {
-    return edgeconv_backward_run(N, n_src, F, argmax, grad_out, nullptr, 1.f, grad_src, nullptr, stream);
+    return edgeconv_backward_run("fgnn_edgeconv_backward", N, n_src, F, argmax, grad_out, nullptr, 1.f, grad_src, nullptr, stream);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -257,7 +258,7 @@ extern "C" int fgnn_edgeconv_backward_blocked(int N, int n_src, int F, int block
     // destination block covers, the plain scatter does the job
     const int fs = ec_blocked_fs(block);
     if (fs == 0 || n_src != N || (size_t)block * fs * sizeof(float) > 64 * 1024)
-        return fgnn_edgeconv_backward(N, n_src, F, argmax, grad_out, grad_src, stream);
+        return edgeconv_backward_run("fgnn_edgeconv_backward_blocked", N, n_src, F, argmax, grad_out, nullptr, 1.f, grad_src, nullptr, stream);
     size_t need = fgnn_edgeconv_backward_blocked_workspace_bytes(N, F);
     FGNN_REQUIRE(N == 0 || (workspace && workspace_bytes >= need), FGNN_ERR_WORKSPACE, "fgnn_edgeconv_backward_blocked: workspace %zu < %zu bytes",
                  workspace_bytes, need);
@@ -299,12 +300,14 @@ extern "C" int fgnn_edgeconv_backward_blocked_static(int N, int n_src, int F, in
 {
     FGNN_REQUIRE(N >= 0 && n_src >= 0 && F >= 1 && block >= 1, FGNN_ERR_SHAPE, "fgnn_edgeconv_backward_blocked_static: bad sizes");
     FGNN_REQUIRE(argmax && grad_out && grad_src, FGNN_ERR_NULL, "fgnn_edgeconv_backward_blocked_static: NULL argument");
+    FGNN_REQUIRE((int64_t)N * F <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_edgeconv_backward_blocked_static: N*F exceeds int32");
+    const int fs = ec_blocked_fs(block);
+    if (fs == 0 || n_src != N || (size_t)block * fs * sizeof(float) > 64 * 1024)      // fill + scatter: no scratch, no allocation, any size
+        return edgeconv_backward_run("fgnn_edgeconv_backward_blocked_static", N, n_src, F, argmax, grad_out, nullptr, 1.f, grad_src, nullptr, stream);
+    // only the blocked form uses the static array, so only it is bound by its size
     FGNN_REQUIRE((int64_t)N * F <= (int64_t)EC_STATIC_MAX_ELEMS, FGNN_ERR_LIMIT,
                  "fgnn_edgeconv_backward_blocked_static: N*F = %lld exceeds the static scratch of %d elements; use fgnn_edgeconv_backward_blocked with a workspace",
                  (long long)N * F, EC_STATIC_MAX_ELEMS);
-    const int fs = ec_blocked_fs(block);
-    if (fs == 0 || n_src != N || (size_t)block * fs * sizeof(float) > 64 * 1024)
-        return fgnn_edgeconv_backward(N, n_src, F, argmax, grad_out, grad_src, stream);      // fill + scatter: no scratch, no allocation
     if (N == 0) return 0;
     int32_t *ovf = nullptr;
     int rc = ec_static_scratch_for_current_device(&ovf);
@@ -327,7 +330,7 @@ extern "C" int fgnn_edgeconv_backward_lrelu(int N, int n_src, int F, int block, 
     FGNN_REQUIRE((int64_t)N * F <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_edgeconv_backward_lrelu: N*F exceeds int32");
     const int fs = block > 0 ? ec_blocked_fs(block) : 0;
     if (fs == 0 || n_src != N || (size_t)block * fs * sizeof(float) > 64 * 1024)
-        return edgeconv_backward_run(N, n_src, F, argmax, grad_out, out, out_slope, grad_src, grad_dst, stream);
+        return edgeconv_backward_run("fgnn_edgeconv_backward_lrelu", N, n_src, F, argmax, grad_out, out, out_slope, grad_src, grad_dst, stream);
     size_t need = fgnn_edgeconv_backward_blocked_workspace_bytes(N, F);
     FGNN_REQUIRE(N == 0 || (workspace && workspace_bytes >= need), FGNN_ERR_WORKSPACE, "fgnn_edgeconv_backward_lrelu: workspace %zu < %zu bytes",
                  workspace_bytes, need);

@@ -3,6 +3,7 @@
 #include <cstdarg>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <vector>
 #include "fgnn_common.h"
 
@@ -511,11 +512,42 @@ extern "C" int fgnn_schedule_create(const int32_t *ptr_dev, int n_rows, int seg_
     return 0;
 }
 
+// The XCD-aware list rests on one property of the part: workgroup w of a dispatch runs on XCD w % 8.  That holds for a
+// gfx950 device that shows all of its 256 compute units (eight XCDs of 32, SPX mode); a partition of the part (fewer
+// compute units per device) or another part spreads workgroups differently, and the bucketed list would then cost its
+// extra segments and its index copy for nothing.  Returns the number of XCDs the mapping is known for, 0 otherwise.
+extern "C" int fgnn_xcd_mapping_for(const char *gcn_arch, int compute_units)
+{
+    if (!gcn_arch) return 0;
+    const bool gfx950 = strncmp(gcn_arch, "gfx950", 6) == 0 && (gcn_arch[6] == '\0' || gcn_arch[6] == ':');
+    return gfx950 && compute_units == 32 * FGNN_NUM_XCD ? FGNN_NUM_XCD : 0;
+}
+
+// 1: the current device has the workgroup-to-XCD mapping the bucketed lists assume; 0: it has not (or cannot be asked)
+static int current_device_has_xcd_mapping()
+{
+    static std::mutex mu;
+    static int known[64];          // per device: 0 = not asked yet, 1 = no, 2 = yes
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    std::lock_guard<std::mutex> lock(mu);
+    if (known[dev] == 0) {
+        hipDeviceProp_t prop;
+        known[dev] = (hipGetDeviceProperties(&prop, dev) == hipSuccess && fgnn_xcd_mapping_for(prop.gcnArchName, prop.multiProcessorCount) > 0) ? 2 : 1;
+    }
+    return known[dev] == 2;
+}
+
 extern "C" int fgnn_schedule_create_bucketed(const int32_t *ptr_dev, const int32_t *idx_dev, int n_rows, int seg_len, int min_deg,
                                              int with_positions, void *stream, fgnn_schedule_t **out)
 {
     FGNN_REQUIRE(ptr_dev && out, FGNN_ERR_NULL, "fgnn_schedule_create_bucketed: NULL argument");
     FGNN_REQUIRE(n_rows >= 0, FGNN_ERR_SHAPE, "fgnn_schedule_create_bucketed: n_rows=%d", n_rows);
+    // on a device without the assumed workgroup-to-XCD mapping the plain list is built instead (fgnn_schedule_num_buckets
+    // of the result is then 0); FGNN_XCD_MAPPING=0 / 1 in the environment overrides the check
+    const char *force = getenv("FGNN_XCD_MAPPING");
+    if (force ? (strcmp(force, "0") == 0) : !current_device_has_xcd_mapping())
+        return fgnn_schedule_create(ptr_dev, n_rows, seg_len, stream, out);
     if (seg_len <= 0) seg_len = 2048;
     seg_len = (seg_len + 63) & ~63;
     if (min_deg <= 0) min_deg = 64;
@@ -731,5 +763,6 @@ extern "C" int fgnn_row_length_stats(const int32_t *ptr_dev, int n_rows, int lon
 }
 
 extern "C" int fgnn_schedule_num_items(const fgnn_schedule_t *s) { return s ? s->n_items : 0; }
+extern "C" int fgnn_schedule_num_buckets(const fgnn_schedule_t *s) { return s ? s->n_buckets : 0; }
 extern "C" int fgnn_schedule_num_partials(const fgnn_schedule_t *s) { return s ? s->n_partials : 0; }
 extern "C" int64_t fgnn_schedule_num_edges(const fgnn_schedule_t *s) { return s ? s->n_edges : 0; }

@@ -41,7 +41,7 @@ class gat_native:
         cc = torch.empty((n, h), dtype=torch.float32, device=dev) if need_aux else None
         e_lrelu = torch.empty((e, h), dtype=torch.float32, device=dev) if (stash and stash_lrelu) else None
         e_soft = torch.empty((e, h), dtype=torch.float32, device=dev) if stash else None
-        sched = schedule_for(row_ptr, idx_tensor=col_ind, need_positions=False) if use_schedule else None
+        sched = schedule_for(row_ptr, idx_tensor=col_ind, need_positions=False, n_cols=n) if use_schedule else None
         sh = sched.handle if sched is not None else None
         with torch.cuda.device(dev):
             ws, wsb = workspace(lib().fgnn_gat_forward_workspace_bytes(sh, h, f), dev)
@@ -93,8 +93,8 @@ class gat_native:
         grad_attn_row = torch.empty((n, h), dtype=torch.float32, device=dev)
         grad_attn_col = torch.empty((n, h), dtype=torch.float32, device=dev)
         recompute = out_feat is None or out2 is None or cc is None
-        sched_csc = schedule_for(col_ptr, idx_tensor=row_ind, need_positions=e_soft is not None and not own) if use_schedule else None
-        sched_csr = schedule_for(row_ptr, idx_tensor=col_ind, need_positions=False) if (use_schedule and recompute) else None
+        sched_csc = schedule_for(col_ptr, idx_tensor=row_ind, need_positions=e_soft is not None and not own, n_cols=n) if use_schedule else None
+        sched_csr = schedule_for(row_ptr, idx_tensor=col_ind, need_positions=False, n_cols=n) if (use_schedule and recompute) else None
         hc = sched_csc.handle if sched_csc is not None else None
         hr = sched_csr.handle if sched_csr is not None else None
         with torch.cuda.device(dev):
@@ -127,7 +127,7 @@ class gat_native:
         if col_ptr.numel() != n + 1 or any(tuple(t.shape) != (n, h) for t in (attn_col, edge_max, edge_sum)):
             raise _lib.FgnnError("gat_stash_own_order: shape mismatch for N=%d H=%d" % (n, h))
         out = torch.empty((e, h), dtype=torch.float32, device=attn_row.device)
-        sched = schedule_for(col_ptr, idx_tensor=row_ind, need_positions=False) if use_schedule else None
+        sched = schedule_for(col_ptr, idx_tensor=row_ind, need_positions=False, n_cols=n) if use_schedule else None
         with torch.cuda.device(attn_row.device):
             check(lib().fgnn_gat_stash_own_order(n, e, h, float(negative_slope), ptr(col_ptr), ptr(row_ind), ptr(attn_row), ptr(attn_col),
                                                  ptr(edge_max), ptr(edge_sum), ptr(out), sched.handle if sched is not None else None,

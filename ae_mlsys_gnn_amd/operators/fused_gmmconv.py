@@ -36,7 +36,7 @@ class gmm_native:
         out = torch.empty((n, f), dtype=torch.float32, device=node_feat.device) if sum_kernels else torch.empty_like(node_feat)
         gauss = torch.empty((e, k), dtype=torch.float32, device=node_feat.device) if want_gauss else None
         # own_order: pseudo (and gauss) are indexed by the schedule's entry order, pseudo_caller[edge_positions(rowptr, colind)]
-        sched = schedule_for(rowptr, idx_tensor=colind, own_order=own_order)
+        sched = schedule_for(rowptr, idx_tensor=colind, own_order=own_order, n_cols=n)
         epilogue = bias is not None or residual is not None
         if epilogue:
             if not sum_kernels:
@@ -80,7 +80,7 @@ class gmm_native:
         grad_mu = torch.empty_like(mu)
         grad_sigma = torch.empty_like(sigma)
         # own_order: pseudo, grad_pseudo (and permute) are indexed by the schedule's entry order (gmm_edge_positions(colptr, rowind, True))
-        sched = schedule_for(colptr, idx_tensor=None if (sum_kernels and _plain_list_for_summed_backward(n, e)) else rowind, own_order=own_order)
+        sched = schedule_for(colptr, idx_tensor=None if (sum_kernels and _plain_list_for_summed_backward(n, e)) else rowind, own_order=own_order, n_cols=n)
         with torch.cuda.device(dev):
             ws, wsb = workspace(lib().fgnn_gmm_backward_workspace_bytes(sched.handle, k, dim, f), dev)
             check(lib().fgnn_gmm_backward(n, e, k, dim, f, ptr(colptr), ptr(rowind), ptr(permute), ptr(node_feat), ptr(pseudo),
@@ -110,7 +110,7 @@ class gmm_native:
             raise FgnnError("gmmconv_shared: shape mismatch mu %s sigma %s pseudo %s for E=%d" % (
                 tuple(mu.shape), tuple(sigma.shape), tuple(pseudo.shape), e))
         out = torch.empty((n, k, f), dtype=torch.float32, device=feat.device)
-        sched = schedule_for(rowptr, idx_tensor=colind, own_order=own_order)
+        sched = schedule_for(rowptr, idx_tensor=colind, own_order=own_order, n_cols=n)
         with torch.cuda.device(feat.device):
             ws, wsb = workspace(lib().fgnn_gmm_forward_workspace_bytes(sched.handle, k, f), feat.device)
             check(lib().fgnn_gmm_forward(n, e, k, dim, f, ptr(rowptr), ptr(colind), ptr(pos_map), ptr(feat), ptr(pseudo),
@@ -141,7 +141,7 @@ class gmm_native:
         grad_mu = torch.empty_like(mu)
         grad_sigma = torch.empty_like(sigma)
         # same work list as the summed backward, so that one CSC-side copy of own-order edge data serves both kinds of layer
-        sched = schedule_for(colptr, idx_tensor=None if _plain_list_for_summed_backward(n, e) else rowind, own_order=own_order)
+        sched = schedule_for(colptr, idx_tensor=None if _plain_list_for_summed_backward(n, e) else rowind, own_order=own_order, n_cols=n)
         with torch.cuda.device(dev):
             ws, wsb = workspace(lib().fgnn_gmm_backward_workspace_bytes(sched.handle, k, dim, f), dev)
             check(lib().fgnn_gmm_backward(n, e, k, dim, f, ptr(colptr), ptr(rowind), ptr(permute), ptr(feat), ptr(pseudo),

@@ -21,7 +21,7 @@ def mhspmm(ptr_arr, idx, attention, feat, pos_map=None):
     if attention is not None and attention.shape != (e, h):
         raise FgnnError("mhspmm: attention is %s, expected (%d, %d)" % (tuple(attention.shape), e, h))
     out = torch.empty((ptr_arr.numel() - 1, h, f), dtype=torch.float32, device=feat.device)
-    sched = schedule_for(ptr_arr, idx_tensor=idx)
+    sched = schedule_for(ptr_arr, idx_tensor=idx, n_cols=n)          # the ids index the rows of feat
     with torch.cuda.device(feat.device):
         # unweighted: only the partial results of split rows (the same figure as the GMMConv forward's)
         need = (lib().fgnn_mhspmm_workspace_bytes if attention is not None else lib().fgnn_gmm_forward_workspace_bytes)(sched.handle, h, f)
@@ -40,7 +40,7 @@ def mhsddmm(rowptr, colind, grad, feat):
     out = torch.empty((e, h), dtype=torch.float32, device=feat.device)
     # a skewed graph is walked under its XCD-aware work list (each XCD then gathers from one eighth of the feature
     # rows); otherwise the kernel cuts the entry array into equal chunks itself and needs no list
-    sched = schedule_for(rowptr, idx_tensor=colind) if e and xcd_buckets_enabled(rowptr, e) else None
+    sched = schedule_for(rowptr, idx_tensor=colind, n_cols=n) if e and xcd_buckets_enabled(rowptr, e) else None
     with torch.cuda.device(feat.device):
         if sched is not None:
             check(lib().fgnn_mhsddmm_scheduled(rowptr.numel() - 1, e, h, f, ptr(rowptr), ptr(colind), ptr(grad), ptr(feat), ptr(out),

@@ -59,7 +59,15 @@ int     fgnn_schedule_create(const int32_t *ptr_dev, int n_rows, int seg_len, vo
  * with_positions != 0, the original position of every entry (another 4*E bytes): operators with
  * per-edge tensors (stashed GAT attention, mhspmm weights, GMMConv pseudo-coordinates) need it and
  * return FGNN_ERR_SCHEDULE without; the recomputing fused GAT does not.  `idx` must be the array later
- * passed to the operator. */
+ * passed to the operator.
+ * The layout assumes that workgroup w of a dispatch runs on XCD w % 8, which is how a gfx950 device that shows all 256
+ * compute units behaves; the call checks the device (architecture name and compute-unit count, once per device) and on
+ * anything else (a partition of the part, another part) builds the plain list of fgnn_schedule_create instead:
+ * fgnn_schedule_num_buckets() of the result tells (8 or 0).  FGNN_XCD_MAPPING=0 / 1 in the environment overrides the
+ * check.  fgnn_xcd_mapping_for() is the rule itself (XCD count for an architecture name and a compute-unit count, 0 =
+ * mapping unknown), exported so that it can be tested without a device. */
+int     fgnn_xcd_mapping_for(const char *gcn_arch, int compute_units);
+int     fgnn_schedule_num_buckets(const fgnn_schedule_t *s);
 int     fgnn_schedule_create_bucketed(const int32_t *ptr_dev, const int32_t *idx_dev, int n_rows,
                                       int seg_len, int min_deg, int with_positions, void *stream,
                                       fgnn_schedule_t **out);
@@ -224,7 +232,10 @@ int    fgnn_edgeconv_backward_blocked(int N, int n_src, int F, int block, const 
  * the process ends); the call allocates nothing and rejects N*F above
  * fgnn_edgeconv_backward_blocked_static_max_elems() (4 Mi elements) with FGNN_ERR_LIMIT.  All calls on one GPU
  * share that array: calls that overlap on one GPU (different streams, different threads) race; calls on one
- * stream are safe, each call rebuilds the list from a counter it clears first.  No counterpart in the reference. */
+ * stream are safe, each call rebuilds the list from a counter it clears first.  The first call on a device looks the
+ * array's device address up (hipGetSymbolAddress, under a mutex): make one ordinary call on each device before a call
+ * under stream capture.  Shapes that take the plain fill-and-scatter form (n_src != N, block > 4096) use no scratch and
+ * are not bound by the size limit.  No counterpart in the reference. */
 size_t fgnn_edgeconv_backward_blocked_static_max_elems(void);
 int    fgnn_edgeconv_backward_blocked_static(int N, int n_src, int F, int block, const int32_t *argmax,
                                              const float *grad_out, float *grad_src, void *stream);

@@ -537,3 +537,51 @@ def test_gat_stash_layouts_are_not_interchangeable():
     keys = [k for k in _lib._sched_cache if k[0] == g.col_ptr.data_ptr()]
     assert not keys, "a no_grad call of the stash variant built a schedule of col_ptr"
     _lib.clear_schedule_cache()
+
+
+def test_schedules_fall_back_to_plain_lists_without_the_xcd_mapping(monkeypatch):
+    """fgnn_schedule_create_bucketed on a device that is not known to spread workgroups over eight XCDs (forced here with
+    FGNN_XCD_MAPPING=0; the box itself reports the mapping) returns the plain list: no buckets, no index copy, and the
+    operators give the same results; with the mapping the list is bucketed."""
+    from ae_mlsys_gnn_amd import _lib
+    g = graphs.rmat_graph(2000, 150000, seed=91)
+    gd = g.to("cuda:0")
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
+    monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+    monkeypatch.delenv("FGNN_XCD_MAPPING", raising=False)
+    _lib.clear_schedule_cache()
+    s1 = _lib.Schedule(gd.row_ptr, 0, gd.col_ind, 16)
+    assert s1.n_buckets == 8 and s1.device_bytes() >= 8 * g.n_edges
+    prop = torch.cuda.get_device_properties(0)
+    assert _lib.lib().fgnn_xcd_mapping_for(prop.gcnArchName.encode(), prop.multi_processor_count) == 8
+    monkeypatch.setenv("FGNN_XCD_MAPPING", "0")
+    s0 = _lib.Schedule(gd.row_ptr, 0, gd.col_ind, 16)
+    assert s0.n_buckets == 0 and s0.device_bytes() < 4 * g.n_edges
+    pos = s0.take_positions()
+    assert torch.equal(pos, torch.arange(g.n_edges, dtype=torch.int32, device="cuda:0"))
+    _lib.clear_schedule_cache()
+    _run(g, 4, 16, variant="sm")
+    _run(g, 2, 64, variant="stash")
+    _lib.clear_schedule_cache()
+
+
+def test_validation_uses_the_width_of_the_gathered_matrix(monkeypatch):
+    """FGNN_VALIDATE=1 with a rectangular pattern: ids index the rows of the gathered matrix (more of them than the pointer
+    array has rows: accepted; an id beyond them: refused), not the rows of the pointer array."""
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd.operators import mhspmm as op
+    monkeypatch.setenv("FGNN_VALIDATE", "1")
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
+    _lib.clear_schedule_cache()
+    n_rows, n_cols = 50, 400
+    gen = torch.Generator().manual_seed(5)
+    rows = [sorted(torch.randint(0, n_cols, (30,), generator=gen).tolist()) for _ in range(n_rows)]
+    g = custom_graph(rows, n_rows).to("cuda:0")
+    feat = torch.randn(n_cols, 2, 8, device="cuda:0")
+    out = op.mhspmm(g.row_ptr, g.col_ind, None, feat)
+    ref = torch.zeros(n_rows, 16, dtype=torch.float64).index_add_(0, orc.row_of_edge(g.row_ptr.cpu()), feat.cpu().double().view(n_cols, 16)[g.col_ind.cpu().long()])
+    assert_close(out.view(n_rows, 16), ref, "rectangular mhspmm under validation")
+    _lib.clear_schedule_cache()
+    with pytest.raises(_lib.FgnnError, match="malformed graph"):
+        op.mhspmm(g.row_ptr, g.col_ind, None, feat[:300].contiguous())          # ids up to 399 against 300 rows
+    _lib.clear_schedule_cache()

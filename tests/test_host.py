@@ -158,3 +158,38 @@ def test_more_argument_errors_without_gpu():
     assert l.fgnn_schedule_create(None, 4, 0, None, ctypes.byref(out)) == -1
     assert l.fgnn_schedule_create_bucketed(None, None, 4, 0, 0, 1, None, ctypes.byref(out)) == -1
     l.fgnn_schedule_destroy(None)                                                  # no-op on NULL
+
+
+def test_xcd_mapping_rule_without_gpu():
+    """The rule behind the XCD-aware work lists: only a gfx950 device that shows all 256 compute units (eight XCDs of 32)
+    is known to spread workgroups round-robin over eight XCDs; a partition of the part or another part gets plain lists."""
+    l = _lib.lib()
+    assert l.fgnn_xcd_mapping_for(b"gfx950:sramecc+:xnack-", 256) == 8
+    assert l.fgnn_xcd_mapping_for(b"gfx950", 256) == 8
+    assert l.fgnn_xcd_mapping_for(b"gfx950:sramecc+:xnack-", 128) == 0      # DPX: two devices of four XCDs
+    assert l.fgnn_xcd_mapping_for(b"gfx950:sramecc+:xnack-", 32) == 0       # CPX: one XCD per device
+    assert l.fgnn_xcd_mapping_for(b"gfx942:sramecc+:xnack-", 304) == 0
+    assert l.fgnn_xcd_mapping_for(b"gfx9500", 256) == 0
+    assert l.fgnn_xcd_mapping_for(None, 256) == 0
+    assert l.fgnn_schedule_num_buckets(None) == 0
+
+
+def test_column_sum_and_wide_row_argument_errors_without_gpu():
+    l = _lib.lib()
+    out = ctypes.c_void_p()
+    assert l.fgnn_colsum_plan_create(None, None, 4, 4, 3, 8, 0, 0, None, ctypes.byref(out)) == -1
+    assert l.fgnn_colsum_plan_create(None, None, 4, 4, 0, 8, 0, 0, None, None) == -1
+    assert l.fgnn_edge_colsum(None, 8, None, None, None, 0, None) == -1
+    assert l.fgnn_colsum_workspace_bytes(None, 8) == 0 and l.fgnn_colsum_plan_device_bytes(None) == 0
+    l.fgnn_colsum_plan_destroy(None)
+    assert l.fgnn_edge_rowsum(-1, 0, 8, None, None, None, None) == -2
+    assert l.fgnn_u_add_v_backward_planned(4, 3, 8, None, None, None, None, None, None, None, 0, None) == -1
+    # more than 1024 floats per head is the one width the GAT entries refuse; rows of many heads are grouped
+    assert l.fgnn_gat_forward(4, 3, 2, 1028, None, None, None, None, 0.2, None, None, None, None, None, None, None, None, None, None, 0, None) == -4
+    assert b"1024" in l.fgnn_last_error()
+    assert l.fgnn_gat_forward(4, 3, 65, 4, None, None, None, None, 0.2, None, None, None, None, None, None, None, None, None, None, 0, None) == -4
+    assert l.fgnn_mhsddmm(4, 3, 2, 1028, None, None, None, None, None, None) == -4
+    # the workspace of a wide-row backward counts the head-group slices (and the stash slice when bit 1 is set)
+    narrow = l.fgnn_gat_backward_workspace_bytes(1000, 4, 256, None, None, 0)
+    wide = l.fgnn_gat_backward_workspace_bytes(1000, 8, 256, None, None, 0)
+    assert wide > narrow + 5 * 1000 * 1024 * 4

@@ -47,6 +47,8 @@ _SIGNATURES = {
                           + [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "fgnn_gat_backward_own_order": (c_int, [c_int, c_int64, c_int, c_int, c_float] + [c_void_p] * 17
                                     + [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "fgnn_gat_scatter": (c_int, [c_int, c_int64, c_int] + [c_void_p] * 4 + [c_float] + [c_void_p] * 2 + [c_void_p]),
+    "fgnn_gat_gather_row": (c_int, [c_int, c_int64, c_int] + [c_void_p] * 5 + [c_float] + [c_void_p] * 4 + [c_void_p]),
     "fgnn_gat_stash_own_order": (c_int, [c_int, c_int64, c_int, c_float] + [c_void_p] * 7 + [c_void_p, c_void_p]),
     "fgnn_edgeconv_forward": (c_int, [c_int, c_int, c_int, c_int] + [c_void_p] * 5 + [c_void_p]),
     "fgnn_edgeconv_backward": (c_int, [c_int, c_int, c_int] + [c_void_p] * 3 + [c_void_p]),
@@ -91,6 +93,8 @@ _SIGNATURES = {
     "fgnn_edge_linear_tanh": (c_int, [c_int64, c_int] + [c_void_p] * 4 + [c_void_p]),
     "fgnn_edge_linear_tanh_backward_workspace_bytes": (c_size_t, [c_int64, c_int]),
     "fgnn_edge_linear_tanh_backward": (c_int, [c_int64, c_int] + [c_void_p] * 5 + [c_void_p, c_size_t, c_void_p]),
+    "fgnn_cross_entropy_forward": (c_int, [c_int64, c_int, c_int64] + [c_void_p] * 4 + [c_void_p]),
+    "fgnn_cross_entropy_backward": (c_int, [c_int64, c_int, c_int64, c_int64] + [c_void_p] * 5 + [c_void_p]),
     "fgnn_coo2csr_workspace_bytes": (c_size_t, [c_int, c_int, c_int64]),
     "fgnn_coo2csr": (c_int, [c_int, c_int, c_int64, c_void_p, c_void_p, c_int] + [c_void_p] * 4 + [c_void_p, c_size_t, c_void_p]),
     "fgnn_csr2csc_workspace_bytes": (c_size_t, [c_int, c_int, c_int64]),

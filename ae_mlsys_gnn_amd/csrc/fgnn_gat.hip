@@ -655,6 +655,52 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_node_kernel(int N, int H, in
     }
 }
 
+// The same pre-pass for rows narrower than a wave (H*F <= 128 floats in the 128-bit layout): a node takes LPN lanes (the
+// power of two >= H*F/4), 64 / LPN nodes share a wave.  With one wave per node an output layer of 48 floats keeps 12 lanes
+// busy and moves 576 bytes per wave (0.9 ms for 2.4 M nodes; the rows are 1.4 GB).
+template <int LPN>
+__global__ __launch_bounds__(FGNN_TPB) void gat_bwd_node_packed_kernel(int N, int H, int F, int HF, const float *g, const float *out,
+                                                                       const float *out2, const float *cc, const float *ar,
+                                                                       const float *emax, const float *esum, float4 *rec, float *delta_out,
+                                                                       float *gar)
+{
+    constexpr int NPW = 64 / LPN;
+    const int lane = fg_lane(), sub = lane % LPN;
+    const int64_t node = ((int64_t)blockIdx.x * FGNN_WPB + fg_wave()) * NPW + lane / LPN;
+    const bool ok = node < N && sub * 4 < HF;
+    float d1 = 0.f, d2 = 0.f;
+    if (ok) {
+        const size_t o = (size_t)node * HF + sub * 4;
+        fg_vec<4> gv, a, c;
+        gv.load(g + o); a.load(out + o); c.load(out2 + o);
+        d1 = gv.dot(a); d2 = gv.dot(c);
+    }
+    const int lph = F / 4;                                  // lanes per head
+    int head = -1;                                          // the head this lane writes the results of
+    if ((lph & (lph - 1)) == 0) {                           // heads are aligned groups of a power of two lanes
+        for (int d = 1; d < lph; d <<= 1) { d1 += __shfl_xor(d1, d); d2 += __shfl_xor(d2, d); }
+        if (ok && sub % lph == 0) head = sub / lph;
+    } else {                                                // any width: one masked sum over the node's lanes per head
+        const int mine = ok ? (sub * 4) / F : -1;
+        float r1 = 0.f, r2 = 0.f;
+        for (int h = 0; h < H; ++h) {
+            float s1 = mine == h ? d1 : 0.f, s2 = mine == h ? d2 : 0.f;
+#pragma unroll
+            for (int d = 1; d < LPN; d <<= 1) { s1 += __shfl_xor(s1, d); s2 += __shfl_xor(s2, d); }
+            if (sub == h) { r1 = s1; r2 = s2; }
+        }
+        d1 = r1; d2 = r2;
+        if (node < N && sub < H) head = sub;                // H <= H*F/4 <= LPN
+    }
+    if (head >= 0) {
+        const size_t q = (size_t)node * H + head;
+        const float s = esum[q];
+        if (delta_out) delta_out[q] = d1;
+        else rec[q] = make_float4(ar[q] * FGNN_LOG2E, emax[q] * FGNN_LOG2E, s > 0.f ? 1.f / s : 0.f, d1);
+        gar[q] = d2 - d1 * cc[q];
+    }
+}
+
 // Writes grad_feat[col] = T and grad_attn_col[col,h] = <x[col,h,:], slope*T + (1-slope)*P> - z[h].
 // z[r] is held by every lane of head hd[r]; scr is wave-private LDS of 64*R + 64 floats.
 template <int VEC, int R>
@@ -1357,10 +1403,28 @@ static int gat_backward_impl(int N, int64_t E, int H, int F, float negative_slop
     p.N = N; p.H = H; p.F = F; p.HF = HF; p.slope = negative_slope;
 
     return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
-        const unsigned gn = (unsigned)((N + FGNN_WPB - 1) / FGNN_WPB);
-        hipLaunchKernelGGL((gat_bwd_node_kernel<VEC, R>), dim3(gn), dim3(FGNN_TPB), (size_t)FGNN_WPB * 64 * R * sizeof(float), st,
-                           N, H, F, HF, grad_out, out_feat, aux_out2, aux_c, attn_row, edge_max, edge_sum, rec,
-                           stash_mode == 2 ? (float *)rec : nullptr, grad_attn_row);
+        float *delta_out = stash_mode == 2 ? (float *)rec : nullptr;
+        if (VEC == 4 && HF <= 128 && fgnn_aligned16(out_feat) && fgnn_aligned16(aux_out2) && fgnn_aligned16(grad_out)) {
+            int lpn = 1;
+            while (lpn * 4 < HF) lpn *= 2;
+            auto node_launch = [&]<int LPN>() {
+                const int64_t waves = ((int64_t)N + 64 / LPN - 1) / (64 / LPN);
+                hipLaunchKernelGGL((gat_bwd_node_packed_kernel<LPN>), dim3((unsigned)((waves + FGNN_WPB - 1) / FGNN_WPB)), dim3(FGNN_TPB), 0, st,
+                                   N, H, F, HF, grad_out, out_feat, aux_out2, aux_c, attn_row, edge_max, edge_sum, rec, delta_out, grad_attn_row);
+            };
+            switch (lpn) {
+            case 1: node_launch.template operator()<1>(); break;
+            case 2: node_launch.template operator()<2>(); break;
+            case 4: node_launch.template operator()<4>(); break;
+            case 8: node_launch.template operator()<8>(); break;
+            case 16: node_launch.template operator()<16>(); break;
+            default: node_launch.template operator()<32>(); break;
+            }
+        } else {
+            const unsigned gn = (unsigned)((N + FGNN_WPB - 1) / FGNN_WPB);
+            hipLaunchKernelGGL((gat_bwd_node_kernel<VEC, R>), dim3(gn), dim3(FGNN_TPB), (size_t)FGNN_WPB * 64 * R * sizeof(float), st,
+                               N, H, F, HF, grad_out, out_feat, aux_out2, aux_c, attn_row, edge_max, edge_sum, rec, delta_out, grad_attn_row);
+        }
         int rc2 = fgnn_launch_status("gat_bwd_node_kernel");
         if (rc2) return rc2;
         const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);

@@ -416,19 +416,43 @@ template <int VEC> __device__ __forceinline__ so_grp<VEC> so_fill(float x)
 // heads of an entry.  One row: the first CACHE groups of a lane stay in registers over both phases; what a longer
 // row has beyond them is folded into a running (maximum, sum) pair while it streams by (one read instead of a
 // maximum pass and a sum pass) and read once more for the result.
-template <bool LONG, int VEC, int CACHE>
-__device__ __forceinline__ void so_softmax_row(int W, int pb, int64_t n, const float *__restrict__ in, float *__restrict__ out, float (*sh)[64])
+// Where a row's values come from.  load(k, first): group k of the row (lane t only ever asks for groups with k % W == t % W);
+// first = false on the second read of a group that did not fit the registers.
+template <int VEC> struct so_from_array {
+    const float *p;         // the row's first value
+    __device__ __forceinline__ so_grp<VEC> load(int64_t k, bool) const { return so_load<VEC>(p + k * VEC); }
+};
+// lrelu(attn_row[row, h] + attn_col[col_ind[entry], h]): the scores of the fuse-scatter GAT forward, formed on the fly
+// (src/fused_gat/fused_gat.cu:235-300 reads them back from the edge_relu array it has just written).
+template <int VEC> struct so_from_scores {
+    const int *idx;         // col_ind of the row's first entry
+    const float *ac;        // attn_col
+    float *elrelu;          // where the row's LeakyReLU values go (NULL: nowhere)
+    so_grp<VEC> ar;         // attn_row[row, this lane's heads]
+    int W, col;             // groups per entry, this lane's group
+    float slope;
+    __device__ __forceinline__ so_grp<VEC> load(int64_t k, bool first) const
+    {
+        const unsigned e = (unsigned)k / (unsigned)W;                  // k is relative to the row: fits 32 bits
+        so_grp<VEC> v = so_load<VEC>(ac + ((size_t)idx[e] * W + col) * VEC);
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) { const float x = v.c[c] + ar.c[c]; v.c[c] = x > 0.f ? x : x * slope; }
+        if (first && elrelu) so_store<VEC>(elrelu + k * VEC, v);
+        return v;
+    }
+};
+
+template <bool LONG, int VEC, int CACHE, class Src>
+__device__ __forceinline__ void so_softmax_row(int W, int64_t n, const Src &src, float *__restrict__ dst, float (*sh)[64])
 {
     const int lane = fg_lane(), S0 = (64 / W) * W;
     const int64_t first = (LONG ? fg_wave() * S0 : 0) + lane, step = (int64_t)S0 * (LONG ? SO_LONG_TPB / 64 : 1);
     const bool act = lane < S0;
-    const float *src = in + (size_t)pb * W * VEC;
-    float *dst = out + (size_t)pb * W * VEC;
     so_grp<VEC> v[CACHE], m = so_fill<VEC>(-INFINITY), s = so_fill<VEC>(0.f);
 #pragma unroll
     for (int i = 0; i < CACHE; ++i) {
         const int64_t k = first + i * step;
-        v[i] = (act && k < n) ? so_load<VEC>(src + k * VEC) : so_fill<VEC>(-INFINITY);
+        v[i] = (act && k < n) ? src.load(k, true) : so_fill<VEC>(-INFINITY);
     }
 #pragma unroll
     for (int i = 0; i < CACHE; ++i)
@@ -442,7 +466,7 @@ __device__ __forceinline__ void so_softmax_row(int W, int pb, int64_t n, const f
         for (int64_t k0 = rest; k0 < n; k0 += SO_STREAM * step) {
             so_grp<VEC> t[SO_STREAM];
 #pragma unroll
-            for (int j = 0; j < SO_STREAM; ++j) t[j] = k0 + j * step < n ? so_load<VEC>(src + (k0 + j * step) * VEC) : so_fill<VEC>(-INFINITY);
+            for (int j = 0; j < SO_STREAM; ++j) t[j] = k0 + j * step < n ? src.load(k0 + j * step, true) : so_fill<VEC>(-INFINITY);
             so_grp<VEC> mn = m;
 #pragma unroll
             for (int j = 0; j < SO_STREAM; ++j)
@@ -479,7 +503,7 @@ __device__ __forceinline__ void so_softmax_row(int W, int pb, int64_t n, const f
         for (int64_t k0 = rest; k0 < n; k0 += SO_STREAM * step) {
             so_grp<VEC> t[SO_STREAM];
 #pragma unroll
-            for (int j = 0; j < SO_STREAM; ++j) t[j] = k0 + j * step < n ? so_load<VEC>(src + (k0 + j * step) * VEC) : so_fill<VEC>(0.f);
+            for (int j = 0; j < SO_STREAM; ++j) t[j] = k0 + j * step < n ? src.load(k0 + j * step, false) : so_fill<VEC>(0.f);
 #pragma unroll
             for (int j = 0; j < SO_STREAM; ++j) {
 #pragma unroll
@@ -503,7 +527,8 @@ __global__ __launch_bounds__(SO_LONG_TPB) void edge_softmax_kernel(int N, int W,
         for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
             const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
             const int pb = fg_uni(ptr[row]);
-            so_softmax_row<true, VEC, SO_CACHE_LONG>(W, pb, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, in, out, sh);
+            so_softmax_row<true, VEC, SO_CACHE_LONG>(W, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, so_from_array<VEC>{in + (size_t)pb * W * VEC},
+                                                     out + (size_t)pb * W * VEC, sh);
         }
         return;
     }
@@ -511,12 +536,78 @@ __global__ __launch_bounds__(SO_LONG_TPB) void edge_softmax_kernel(int N, int W,
     int64_t n;
     const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (SO_LONG_TPB / 64)) + fg_wave());
     if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n) || n == 0) return;
-    so_softmax_row<false, VEC, SO_CACHE>(W, pb, n, in, out, nullptr);
+    so_softmax_row<false, VEC, SO_CACHE>(W, n, so_from_array<VEC>{in + (size_t)pb * W * VEC}, out + (size_t)pb * W * VEC, nullptr);
 }
 
-template <bool LONG, int VEC>
-__device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, const float *__restrict__ sm, const float *__restrict__ g,
-                                                   float *__restrict__ gin, float (*sh)[64])
+// The fuse-scatter GAT forward (fused_scatter_kernel, src/fused_gat/fused_gat.cu:235-300): scores, LeakyReLU and the row softmax in
+// one pass that writes e_softmax [E,H] (and e_lrelu when asked for).
+template <int VEC>
+__global__ __launch_bounds__(SO_LONG_TPB) void gat_scatter_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
+                                                                  const int *__restrict__ idx, const float *__restrict__ ar,
+                                                                  const float *__restrict__ ac, float slope, float *__restrict__ elrelu,
+                                                                  float *__restrict__ esoft)
+{
+    __shared__ float sh[SO_LONG_TPB / 64][64];
+    __shared__ unsigned long long sh_mask;
+    const int col = fg_lane() % W;
+    auto source = [&](int row, int pb) {
+        so_from_scores<VEC> src;
+        src.idx = idx + pb; src.ac = ac; src.elrelu = elrelu ? elrelu + (size_t)pb * W * VEC : nullptr;
+        src.ar = so_load<VEC>(ar + ((size_t)row * W + col) * VEC);
+        src.W = W; src.col = col; src.slope = slope;
+        return src;
+    };
+    if (blockIdx.x < n_long_blocks) {
+        for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
+            const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
+            const int pb = fg_uni(ptr[row]);
+            so_softmax_row<true, VEC, SO_CACHE_LONG>(W, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, source(row, pb), esoft + (size_t)pb * W * VEC, sh);
+        }
+        return;
+    }
+    int row, pb;
+    int64_t n;
+    const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (SO_LONG_TPB / 64)) + fg_wave());
+    if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n) || n == 0) return;
+    so_softmax_row<false, VEC, SO_CACHE>(W, n, source(row, pb), esoft + (size_t)pb * W * VEC, nullptr);
+}
+
+// The factor LeakyReLU' puts on an entry's gradient, for the fused gather_row pass of the fuse-scatter GAT backward
+// (src/fused_gat/fused_gat.cu:502-556): none (plain softmax backward), from the stashed LeakyReLU values, or from the
+// sign of attn_row + attn_col formed again (no [E,H] array is read for it).
+template <int VEC> struct so_sign_none {
+    static constexpr bool active = false;
+    __device__ __forceinline__ so_grp<VEC> factor(int64_t) const { return so_fill<VEC>(1.f); }
+};
+template <int VEC> struct so_sign_array {
+    static constexpr bool active = true;
+    const float *elrelu; float slope;          // the row's first LeakyReLU value
+    __device__ __forceinline__ so_grp<VEC> factor(int64_t k) const
+    {
+        so_grp<VEC> v = so_load<VEC>(elrelu + k * VEC);
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) v.c[c] = v.c[c] > 0.f ? 1.f : slope;      // a pre-activation of exactly 0 takes the slope, as torch's LeakyReLU does
+        return v;
+    }
+};
+template <int VEC> struct so_sign_scores {
+    static constexpr bool active = true;
+    const int *idx; const float *ac; so_grp<VEC> ar; int W, col; float slope;
+    __device__ __forceinline__ so_grp<VEC> factor(int64_t k) const
+    {
+        const unsigned e = (unsigned)k / (unsigned)W;
+        so_grp<VEC> v = so_load<VEC>(ac + ((size_t)idx[e] * W + col) * VEC);
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) v.c[c] = v.c[c] + ar.c[c] > 0.f ? 1.f : slope;
+        return v;
+    }
+};
+
+// gin = factor * sm * (g - sum_row sm * g); with an active Sign also rowsum[lane's heads] = sum_row gin (the grad_attn_row of
+// the fuse-scatter backward).  gin may be g itself: every value is read before it is overwritten, by the same lane.
+template <bool LONG, int VEC, class Sign>
+__device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, const float *__restrict__ sm, const float *g,
+                                                   float *gin, const Sign &sign, float *__restrict__ rowsum, float (*sh)[64])
 {
     const int lane = fg_lane(), S0 = (64 / W) * W;
     const int64_t first = (LONG ? fg_wave() * S0 : 0) + lane, step = (int64_t)S0 * (LONG ? SO_LONG_TPB / 64 : 1);
@@ -551,12 +642,21 @@ __device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, con
         }
     }
     acc = so_column_reduce<LONG, VEC>(acc, lane, W, S0, sh, so_add());
+    so_grp<VEC> rs = so_fill<VEC>(0.f);
 #pragma unroll
     for (int i = 0; i < SO_CACHE; ++i) {
         const int64_t k = first + i * step;
+        const bool ok = act && k < n;
 #pragma unroll
         for (int c = 0; c < VEC; ++c) sv[i].c[c] *= gv[i].c[c] - acc.c[c];
-        if (act && k < n) so_store<VEC>(gin + base + k * VEC, sv[i]);
+        if constexpr (Sign::active) {
+            if (ok) {
+                const so_grp<VEC> f = sign.factor(k);
+#pragma unroll
+                for (int c = 0; c < VEC; ++c) { sv[i].c[c] *= f.c[c]; rs.c[c] += sv[i].c[c]; }
+            }
+        }
+        if (ok) so_store<VEC>(gin + base + k * VEC, sv[i]);
     }
     if (act) {
         for (int64_t k0 = rest; k0 < n; k0 += (SO_STREAM / 2) * step) {
@@ -569,11 +669,23 @@ __device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, con
             }
 #pragma unroll
             for (int j = 0; j < SO_STREAM / 2; ++j) {
+                const bool ok = k0 + j * step < n;
 #pragma unroll
                 for (int c = 0; c < VEC; ++c) a[j].c[c] *= b[j].c[c] - acc.c[c];
-                if (k0 + j * step < n) so_store<VEC>(gin + base + (k0 + j * step) * VEC, a[j]);
+                if constexpr (Sign::active) {
+                    if (ok) {
+                        const so_grp<VEC> f = sign.factor(k0 + j * step);
+#pragma unroll
+                        for (int c = 0; c < VEC; ++c) { a[j].c[c] *= f.c[c]; rs.c[c] += a[j].c[c]; }
+                    }
+                }
+                if (ok) so_store<VEC>(gin + base + (k0 + j * step) * VEC, a[j]);
             }
         }
+    }
+    if constexpr (Sign::active) {
+        rs = so_column_reduce<LONG, VEC>(rs, lane, W, S0, sh, so_add());
+        if (lane < W && (!LONG || fg_wave() == 0)) so_store<VEC>(rowsum + (size_t)lane * VEC, rs);
     }
 }
 
@@ -588,7 +700,7 @@ __global__ __launch_bounds__(SO_LONG_TPB) void edge_softmax_bwd_kernel(int N, in
         for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
             const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
             const int pb = fg_uni(ptr[row]);
-            so_softmax_bwd_row<true, VEC>(W, pb, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, sm, g, gin, sh);
+            so_softmax_bwd_row<true, VEC>(W, pb, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, sm, g, gin, so_sign_none<VEC>{}, nullptr, sh);
         }
         return;
     }
@@ -596,7 +708,44 @@ __global__ __launch_bounds__(SO_LONG_TPB) void edge_softmax_bwd_kernel(int N, in
     int64_t n;
     const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (SO_LONG_TPB / 64)) + fg_wave());
     if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n) || n == 0) return;
-    so_softmax_bwd_row<false, VEC>(W, pb, n, sm, g, gin, nullptr);
+    so_softmax_bwd_row<false, VEC>(W, pb, n, sm, g, gin, so_sign_none<VEC>{}, nullptr, nullptr);
+}
+
+// fused_gather_row of the fuse-scatter GAT backward (src/fused_gat/fused_gat.cu:502-556): softmax backward, LeakyReLU backward
+// and the row sums (grad_attn_row) in one pass; gout may be g (in place).  Rows without entries get a zero row sum.
+template <int VEC, bool FROM_ARRAY>
+__global__ __launch_bounds__(SO_LONG_TPB) void gat_gather_row_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
+                                                                     const int *__restrict__ idx, const float *__restrict__ ar,
+                                                                     const float *__restrict__ ac, const float *__restrict__ elrelu, float slope,
+                                                                     const float *__restrict__ sm, const float *g, float *gout,
+                                                                     float *__restrict__ gar)
+{
+    __shared__ float sh[SO_LONG_TPB / 64][64];
+    __shared__ unsigned long long sh_mask;
+    const int col = fg_lane() % W;
+    auto run = [&]<bool LONG>(int row, int pb, int64_t n, float (*shp)[64]) {
+        float *rowsum = gar + (size_t)row * W * VEC;
+        if constexpr (FROM_ARRAY) {
+            so_softmax_bwd_row<LONG, VEC>(W, pb, n, sm, g, gout, so_sign_array<VEC>{elrelu + (size_t)pb * W * VEC, slope}, rowsum, shp);
+        } else {
+            so_sign_scores<VEC> sg;
+            sg.idx = idx + pb; sg.ac = ac; sg.ar = so_load<VEC>(ar + ((size_t)row * W + col) * VEC); sg.W = W; sg.col = col; sg.slope = slope;
+            so_softmax_bwd_row<LONG, VEC>(W, pb, n, sm, g, gout, sg, rowsum, shp);
+        }
+    };
+    if (blockIdx.x < n_long_blocks) {
+        for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
+            const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
+            const int pb = fg_uni(ptr[row]);
+            run.template operator()<true>(row, pb, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, sh);
+        }
+        return;
+    }
+    int row, pb;
+    int64_t n;
+    const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (SO_LONG_TPB / 64)) + fg_wave());
+    if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n)) return;
+    run.template operator()<false>(row, pb, n, nullptr);             // an empty row stores its zero sums
 }
 
 // More than 64 heads: one wave per row, one head at a time.
@@ -674,6 +823,58 @@ extern "C" int fgnn_edge_softmax_backward(int N, int64_t E, int H, const int32_t
     else
         hipLaunchKernelGGL(edge_softmax_bwd_kernel<1>, dim3(grid), dim3(SO_LONG_TPB), 0, st, N, H, n_long, row_ptr, sm, grad_out, grad_in);
     return fgnn_launch_status("edge_softmax_bwd_kernel");
+}
+
+// Forward half of the reference's fuse-scatter GAT (fused_gat.gat_forward minus its SpMM, src/fused_gat/fused_gat.cu:235-300,
+// 365-386): e_softmax[p,h] = softmax over row(p) of lrelu(attn_row[row(p),h] + attn_col[col_ind[p],h]); e_lrelu (optional)
+// gets the LeakyReLU values.  H <= 64.
+extern "C" int fgnn_gat_scatter(int N, int64_t E, int H, const int32_t *row_ptr, const int32_t *col_ind, const float *attn_row,
+                                const float *attn_col, float negative_slope, float *e_lrelu, float *e_softmax, void *stream)
+{
+    FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1, FGNN_ERR_SHAPE, "fgnn_gat_scatter: bad sizes");
+    FGNN_REQUIRE(H <= 64, FGNN_ERR_LIMIT, "fgnn_gat_scatter: H=%d > 64 heads unsupported", H);
+    FGNN_REQUIRE(E <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_gat_scatter: E=%lld exceeds int32 positions", (long long)E);
+    if (N == 0 || E == 0) return 0;
+    FGNN_REQUIRE(row_ptr && col_ind && attn_row && attn_col && e_softmax, FGNN_ERR_NULL, "fgnn_gat_scatter: NULL argument");
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned n_long = E * H > SO_LONG_ELEMS ? (unsigned)((N + SO_CAND - 1) / SO_CAND) : 0u;
+    const unsigned grid = n_long + (unsigned)((N + SO_LONG_TPB / 64 - 1) / (SO_LONG_TPB / 64));
+    if (H % 4 == 0 && fgnn_aligned16(attn_row) && fgnn_aligned16(attn_col) && fgnn_aligned16(e_softmax) && fgnn_aligned16(e_lrelu))
+        hipLaunchKernelGGL(gat_scatter_kernel<4>, dim3(grid), dim3(SO_LONG_TPB), 0, st, N, H / 4, n_long, row_ptr, col_ind, attn_row, attn_col,
+                           negative_slope, e_lrelu, e_softmax);
+    else
+        hipLaunchKernelGGL(gat_scatter_kernel<1>, dim3(grid), dim3(SO_LONG_TPB), 0, st, N, H, n_long, row_ptr, col_ind, attn_row, attn_col,
+                           negative_slope, e_lrelu, e_softmax);
+    return fgnn_launch_status("gat_scatter_kernel");
+}
+
+// fused_gather_row of the same variant's backward (src/fused_gat/fused_gat.cu:502-556): grad_edge_out = lrelu'(e) * e_softmax *
+// (grad_edge - sum_row e_softmax * grad_edge), grad_attn_row = its row sums.  The sign of the pre-activation comes from e_lrelu
+// when it is given, else from attn_row + attn_col formed again (col_ind, attn_row, attn_col required).  grad_edge_out may be
+// grad_edge.
+extern "C" int fgnn_gat_gather_row(int N, int64_t E, int H, const int32_t *row_ptr, const int32_t *col_ind, const float *attn_row,
+                                   const float *attn_col, const float *e_lrelu, float negative_slope, const float *e_softmax,
+                                   const float *grad_edge, float *grad_edge_out, float *grad_attn_row, void *stream)
+{
+    FGNN_REQUIRE(N >= 0 && E >= 0 && H >= 1, FGNN_ERR_SHAPE, "fgnn_gat_gather_row: bad sizes");
+    FGNN_REQUIRE(H <= 64, FGNN_ERR_LIMIT, "fgnn_gat_gather_row: H=%d > 64 heads unsupported", H);
+    FGNN_REQUIRE(E <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_gat_gather_row: E=%lld exceeds int32 positions", (long long)E);
+    if (N == 0) return 0;
+    FGNN_REQUIRE(row_ptr && grad_attn_row && (E == 0 || (e_softmax && grad_edge && grad_edge_out)), FGNN_ERR_NULL, "fgnn_gat_gather_row: NULL argument");
+    FGNN_REQUIRE(E == 0 || e_lrelu || (col_ind && attn_row && attn_col), FGNN_ERR_NULL,
+                 "fgnn_gat_gather_row: without e_lrelu the scores are formed again from col_ind, attn_row and attn_col");
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned n_long = E * H > SO_LONG_ELEMS ? (unsigned)((N + SO_CAND - 1) / SO_CAND) : 0u;
+    const unsigned grid = n_long + (unsigned)((N + SO_LONG_TPB / 64 - 1) / (SO_LONG_TPB / 64));
+    const bool vec4 = H % 4 == 0 && fgnn_aligned16(e_softmax) && fgnn_aligned16(grad_edge) && fgnn_aligned16(grad_edge_out) && fgnn_aligned16(grad_attn_row) &&
+                      fgnn_aligned16(e_lrelu) && fgnn_aligned16(attn_row) && fgnn_aligned16(attn_col);
+    const int W = vec4 ? H / 4 : H;
+#define GGR_LAUNCH(V, A) hipLaunchKernelGGL((gat_gather_row_kernel<V, A>), dim3(grid), dim3(SO_LONG_TPB), 0, st, N, W, n_long, row_ptr, col_ind, attn_row, \
+                                            attn_col, e_lrelu, negative_slope, e_softmax, grad_edge, grad_edge_out, grad_attn_row)
+    if (vec4) { if (e_lrelu) GGR_LAUNCH(4, true); else GGR_LAUNCH(4, false); }
+    else { if (e_lrelu) GGR_LAUNCH(1, true); else GGR_LAUNCH(1, false); }
+#undef GGR_LAUNCH
+    return fgnn_launch_status("gat_gather_row_kernel");
 }
 
 // out[p,w] = row_val[row(p),w] + col_val[col_ind[p],w]  (src/u_add_v/u_add_v.cu:4-26).  W <= 64: one thread per

@@ -37,8 +37,11 @@ class _GATBase(nn.Module):
         so that the operator takes its 128-bit row layout; `_crop` drops them again."""
         return _ProjectScores.apply(feat, self.W, self.attn_l, self.attn_r, (-self.out_feats) % 4)
 
-    def _crop(self, out):
-        return out if out.shape[-1] == self.out_feats else out[..., :self.out_feats]
+    def _crop(self, out, keep_padding=False):
+        """keep_padding: hand the operator's zero-padded [N, H, out_feats rounded up to 4] array on as it is (a consumer
+        that takes the number of valid columns, such as the drivers' fused cross-entropy, then needs neither the
+        cropped view nor the zero-filled copy its gradient would go through)."""
+        return out if keep_padding or out.shape[-1] == self.out_feats else out[..., :self.out_feats]
 
 
 class _ProjectScores(torch.autograd.Function):
@@ -86,20 +89,20 @@ class _ProjectScores(torch.autograd.Function):
 class GATConv(_GATBase):
     """Recompute variant: nothing edge-sized survives the forward."""
 
-    def forward(self, row_ptr, col_ind, col_ptr, row_ind, feat, save_memory=True):
+    def forward(self, row_ptr, col_ind, col_ptr, row_ind, feat, save_memory=True, keep_padding=False):
         h, attn_row, attn_col = self._project(feat)
-        return self._crop(fused_gat_op(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, self.negative_slope, h, save_memory))
+        return self._crop(fused_gat_op(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, self.negative_slope, h, save_memory), keep_padding)
 
 
 class GATConv_stash(_GATBase):
     """Stash variant: per-edge LeakyReLU / softmax values [E,H] are kept for the backward."""
 
-    def forward(self, row_ptr, col_ind, col_ptr, row_ind, feat, permute):
+    def forward(self, row_ptr, col_ind, col_ptr, row_ind, feat, permute, keep_padding=False):
         h, attn_row, attn_col = self._project(feat)
-        return self._crop(fused_gat_stash_op(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, self.negative_slope, h, permute))
+        return self._crop(fused_gat_stash_op(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, self.negative_slope, h, permute), keep_padding)
 
 
 class GATConv_fusescatter(_GATBase):
-    def forward(self, row_ptr, col_ind, col_ptr, row_ind, feat, permute):
+    def forward(self, row_ptr, col_ind, col_ptr, row_ind, feat, permute, keep_padding=False):
         h, attn_row, attn_col = self._project(feat)
-        return self._crop(fused_gat_fusescatter(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, self.negative_slope, h, permute))
+        return self._crop(fused_gat_fusescatter(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, self.negative_slope, h, permute), keep_padding)

@@ -4,16 +4,17 @@
 ``fused_gat_stash_op`` / ``FusedGATFunction_stash``  stash variant  (operators/fused_gat.py:33-34,73-86)
 ``fused_gat_fusescatter`` / ``FusedGATFunction``  fuse-scatter variant (operators/fused_gat.py:27-28,36-50)
 
-All three share one forward kernel and one backward kernel; the stash variants additionally
-write / read the per-edge ``[E,H]`` LeakyReLU and softmax tensors.  What the recompute variant
-keeps for the backward is node-sized only: ``out``, ``out2`` ([N,H,F]) and three ``[N,H]`` arrays.
+The recompute and stash variants share one forward kernel and one backward kernel; the stash variant additionally
+writes / reads the per-edge ``[E,H]`` softmax tensor.  What the recompute variant keeps for the backward is
+node-sized only: ``out``, ``out2`` ([N,H,F]) and three ``[N,H]`` arrays.  The fuse-scatter variant is the reference's
+unfused-SpMM data flow (scatter kernel -> [E,H] -> SpMM), kept for the ablation it stands for.
 """
 from __future__ import annotations
 
 import torch
 
 from .. import _lib
-from .._lib import as_f32, as_i32, check, lib, ptr, require_cuda, schedule_for, stream_ptr, workspace
+from .._lib import as_f32, as_i32, check, colsum_plan_for, lib, ptr, require_cuda, schedule_for, stream_ptr, workspace
 
 
 class gat_native:
@@ -135,6 +136,43 @@ class gat_native:
         return out
 
 
+    @staticmethod
+    def gat_scatter(attn_row, attn_col, row_ptr, col_ind, negative_slope, want_lrelu=False):
+        """fused_scatter_kernel of the reference's fuse-scatter variant (src/fused_gat/fused_gat.cu:235-300): (e_lrelu or None,
+        e_softmax [E,H]) in one pass over the rows."""
+        require_cuda(attn_row, attn_col, row_ptr, col_ind)
+        attn_row, attn_col, row_ptr, col_ind = as_f32(attn_row), as_f32(attn_col), as_i32(row_ptr), as_i32(col_ind)
+        n, h = attn_row.shape
+        e = col_ind.numel()
+        if attn_col.shape != (n, h) or row_ptr.numel() != n + 1:
+            raise _lib.FgnnError("gat_scatter: shape mismatch for N=%d H=%d" % (n, h))
+        e_soft = torch.empty((e, h), dtype=torch.float32, device=attn_row.device)
+        e_lrelu = torch.empty((e, h), dtype=torch.float32, device=attn_row.device) if want_lrelu else None
+        with torch.cuda.device(attn_row.device):
+            check(lib().fgnn_gat_scatter(n, e, h, ptr(row_ptr), ptr(col_ind), ptr(attn_row), ptr(attn_col), float(negative_slope),
+                                         ptr(e_lrelu), ptr(e_soft), stream_ptr()), "fgnn_gat_scatter")
+        return e_lrelu, e_soft
+
+    @staticmethod
+    def gat_gather_row(negative_slope, row_ptr, col_ind, attn_row, attn_col, e_soft, grad_edge, e_lrelu=None, inplace=False):
+        """fused_gather_row (src/fused_gat/fused_gat.cu:502-556): (gradient of the pre-activations [E,H], grad_attn_row [N,H])."""
+        require_cuda(row_ptr, col_ind, attn_row, attn_col, e_soft, grad_edge, e_lrelu)
+        row_ptr, col_ind = as_i32(row_ptr), as_i32(col_ind)
+        attn_row, attn_col, e_soft, grad_edge = as_f32(attn_row), as_f32(attn_col), as_f32(e_soft), as_f32(grad_edge)
+        e_lrelu = None if e_lrelu is None else as_f32(e_lrelu)
+        n, h = attn_row.shape
+        e = col_ind.numel()
+        if e_soft.shape != (e, h) or grad_edge.shape != (e, h) or (e_lrelu is not None and e_lrelu.shape != (e, h)) or row_ptr.numel() != n + 1:
+            raise _lib.FgnnError("gat_gather_row: shape mismatch for N=%d E=%d H=%d" % (n, e, h))
+        out = grad_edge if inplace else torch.empty_like(grad_edge)
+        gar = torch.empty((n, h), dtype=torch.float32, device=attn_row.device)
+        with torch.cuda.device(attn_row.device):
+            check(lib().fgnn_gat_gather_row(n, e, h, ptr(row_ptr), ptr(col_ind), ptr(attn_row), ptr(attn_col), ptr(e_lrelu),
+                                            float(negative_slope), ptr(e_soft), ptr(grad_edge), ptr(out), ptr(gar), stream_ptr()),
+                  "fgnn_gat_gather_row")
+        return out, gar
+
+
 def fused_gat_fusescatter(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute):
     return FusedGATFunction.apply(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute)
 
@@ -214,18 +252,48 @@ class FusedGATFunction_stash(torch.autograd.Function):
         return grad_attn_row, grad_attn_col, None, None, None, None, None, grad_feat, None
 
 
-class FusedGATFunction(FusedGATFunction_stash):
-    """Fuse-scatter variant as ONE fused operator: it shares the stash implementation (same math, same
-    stashed tensor).  The reference's own fuse-scatter data flow -- a softmax kernel that materialises
-    [E,H], then a separate SpMM; backward by permuted SpMM, SDDMM and row / column sums
-    (src/fused_gat/fused_gat.cu:235-326, 641-670) -- is `fused_gat_fusescatter_pipeline` below."""
+class FusedGATFunction(torch.autograd.Function):
+    """Fuse-scatter variant with the reference's own data flow (operators/fused_gat.py:36-50; src/fused_gat/fused_gat.cu):
+    forward = one scatter kernel (scores, LeakyReLU, row softmax -> e_softmax [E,H]) + multi-head SpMM; backward = the
+    permuted SpMM over the CSC arrays (grad_feat), the SDDMM (gradient of the weights), one gather-row kernel (softmax and
+    LeakyReLU backward + row sums = grad_attn_row, in place) and the column sums (grad_attn_col).  Kept between the passes:
+    e_softmax only; the reference also keeps the LeakyReLU values, whose sign this backward forms again from the scores."""
+
+    @staticmethod
+    def forward(ctx, attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute):
+        from .mhspmm import mhspmm
+        attn_row, attn_col, in_feat = _contig(attn_row), _contig(attn_col), _contig(in_feat)
+        row_ptr, col_ind, col_ptr, row_ind, permute = _contig(row_ptr), _contig(col_ind), _contig(col_ptr), _contig(row_ind), _contig(permute)
+        _, e_soft = gat_native.gat_scatter(attn_row, attn_col, row_ptr, col_ind, negative_slope)
+        out = mhspmm(row_ptr, col_ind, e_soft, in_feat)
+        if _needs_grad(ctx):
+            ctx.save_for_backward(row_ptr, col_ind, col_ptr, row_ind, permute, e_soft, in_feat, attn_row, attn_col)
+        ctx.negative_slope = negative_slope
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        from .mhspmm import mhsddmm, mhspmm
+        row_ptr, col_ind, col_ptr, row_ind, permute, e_soft, in_feat, attn_row, attn_col = ctx.saved_tensors
+        grad_out = grad_out.contiguous()
+        grad_feat = mhspmm(col_ptr, row_ind, e_soft, grad_out, pos_map=as_i32(permute))
+        grad_edge = mhsddmm(row_ptr, col_ind, grad_out, in_feat)
+        grad_edge, grad_attn_row = gat_native.gat_gather_row(ctx.negative_slope, row_ptr, col_ind, attn_row, attn_col, e_soft, grad_edge, inplace=True)
+        n, h = attn_row.shape
+        grad_attn_col = colsum_plan_for(row_ptr, col_ind, n, h).colsum(grad_edge)
+        return grad_attn_row, grad_attn_col, None, None, None, None, None, grad_feat, None
 
 
 def fused_gat_fusescatter_pipeline(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute):
-    """The fuse-scatter ablation of the reference as a pipeline of this package's small operators, each with
-    its own autograd function: u_add_v -> LeakyReLU -> edge softmax ([E,H] materialised twice) -> multi-head
-    SpMM; the backward runs the permuted SpMM over the CSC arrays, the SDDMM, the softmax backward and the
-    row / column sums of u_add_v.  Same results as the fused operators; several passes over [E,H] more."""
+    """The fuse-scatter ablation of the reference: FusedGATFunction above (its own kernels in its own order)."""
+    return FusedGATFunction.apply(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute)
+
+
+def fused_gat_operator_pipeline(attn_row, attn_col, row_ptr, col_ind, col_ptr, row_ind, negative_slope, in_feat, permute):
+    """The same layer composed from this package's stand-alone operators, each with its own autograd function: u_add_v ->
+    LeakyReLU -> edge softmax ([E,H] materialised three times) -> multi-head SpMM; the backward runs the permuted SpMM
+    over the CSC arrays, the SDDMM, the softmax backward and the row / column sums of u_add_v.  Same results as the fused
+    operators; what an unfused layer costs on this part."""
     from .edge_softmax import csr_edge_softmax
     from .mhspmm import csrmhspmm
     from .u_add_v import u_add_v_op

@@ -28,10 +28,12 @@ class GAT(nn.Module):
         self.hidden = nn.ModuleList(conv(dims[l], num_hidden, heads[l], negative_slope) for l in range(num_layers))
         self.out = conv(dims[-1], num_classes, heads[-1], negative_slope)
 
-    def forward(self, g, x, extra):
+    def forward(self, g, x, extra, keep_padding=False):
+        """keep_padding: the logits keep the output layer's zero columns up to a multiple of four ([N, >= classes]); the
+        loss is told the number of classes instead of reading a cropped view."""
         for layer in self.hidden:
             x = layer(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, x, extra).flatten(1)
-        return common.head_mean(self.out(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, x, extra))
+        return common.head_mean(self.out(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, x, extra, keep_padding=keep_padding))
 
 
 def build_parser():
@@ -77,8 +79,8 @@ def main(argv=None):
 
     def step():
         model.train()
-        logits = model(g, data.feat, extra)
-        loss = loss_fcn(logits[train_idx], train_labels)
+        logits = model(g, data.feat, extra, keep_padding=True)
+        loss = loss_fcn(logits[train_idx], train_labels, data.n_classes)
         opt.zero_grad(set_to_none=False)
         loss.backward()
         opt.step()

@@ -177,6 +177,22 @@ int    fgnn_gat_backward_own_order(int N, int64_t E, int H, int F, float negativ
                                    const fgnn_schedule_t *sched_csc, const fgnn_schedule_t *sched_csr,
                                    void *workspace, size_t workspace_bytes, void *stream);
 
+/* The reference's fuse-scatter GAT variant as it defines it (operators/fused_gat.py:36-50; src/fused_gat/fused_gat.cu):
+ * forward = fused_scatter_kernel (:235-300: scores, LeakyReLU and row softmax in one pass that writes [E,H]) + mhspmm;
+ * backward = permuted mhspmm + mhsddmm + fused_gather_row (:502-556) + gather_col (:558-586).
+ * fgnn_gat_scatter is the first kernel: e_softmax[p,h] = softmax over row(p) of lrelu(attn_row[row(p),h] +
+ * attn_col[col_ind[p],h]); e_lrelu (optional, NULL to skip) gets the LeakyReLU values the reference stashes next to it.
+ * fgnn_gat_gather_row is fused_gather_row: grad_edge_out[p,h] = lrelu'(e) * e_softmax * (grad_edge - sum_row e_softmax *
+ * grad_edge) and grad_attn_row = its row sums, in one pass; the sign of the pre-activation is read from e_lrelu when that
+ * is given and formed again from col_ind / attn_row / attn_col otherwise (4 bytes per entry read instead of 4*H, and no
+ * second [E,H] array kept between the passes).  grad_edge_out may be grad_edge (in place).  The SpMM steps are fgnn_mhspmm
+ * and fgnn_mhsddmm, gather_col is fgnn_edge_colsum.  H <= 64. */
+int    fgnn_gat_scatter(int N, int64_t E, int H, const int32_t *row_ptr, const int32_t *col_ind, const float *attn_row,
+                        const float *attn_col, float negative_slope, float *e_lrelu, float *e_softmax, void *stream);
+int    fgnn_gat_gather_row(int N, int64_t E, int H, const int32_t *row_ptr, const int32_t *col_ind, const float *attn_row,
+                           const float *attn_col, const float *e_lrelu, float negative_slope, const float *e_softmax,
+                           const float *grad_edge, float *grad_edge_out, float *grad_attn_row, void *stream);
+
 /* The stashed attention of the stash variants in the ORDER OF THE BACKWARD PASS: e_softmax_own[q,h] = alpha of
  * entry q of the walk of (col_ptr, row_ind) under sched_csc (its bucket-ordered entry order when it is XCD-aware,
  * plain CSC order otherwise or with sched_csc == NULL), computed from the forward's row statistics; the sign bit of
@@ -408,6 +424,21 @@ size_t fgnn_edge_linear_tanh_backward_workspace_bytes(int64_t E, int D);
 int    fgnn_edge_linear_tanh_backward(int64_t E, int D, const float *x, const float *y,
                                       const float *grad_y, float *grad_W, float *grad_b,
                                       void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---------------------------------------------------------------- loss of the training drivers
+ * torch.nn.CrossEntropyLoss over the labelled rows (script/train/train_gatconv_our.py:166-175) as two passes over the
+ * logits instead of a dozen elementwise and reduction kernels: the forward writes, per row, lse = log sum_c exp(x[c]) and
+ * row_loss = lse - x[label] (the loss is their mean); the backward writes grad[row, c] = (exp(x[c] - lse) - [c == label])
+ * * upstream[row].  logits rows are ld floats apart (ld >= C: a [N, C] view of a padded array is read in place), gradient
+ * rows ld_grad floats apart, their columns C .. ld_grad - 1 get zeros (the gradient of a padded array needs no second
+ * copy).  labels are int64 (torch's default); a label outside [0, C) indexes nothing and gives a NaN row loss.  Nothing
+ * synchronises: the calls can be captured into a HIP graph.  C <= 256 (1024 when ld and ld_grad are multiples of four and
+ * the arrays 16-byte aligned). */
+int    fgnn_cross_entropy_forward(int64_t N, int C, int64_t ld, const float *logits, const int64_t *labels, float *lse,
+                                  float *row_loss, void *stream);
+int    fgnn_cross_entropy_backward(int64_t N, int C, int64_t ld, int64_t ld_grad, const float *logits,
+                                   const int64_t *labels, const float *lse, const float *upstream,
+                                   float *grad_logits, void *stream);
 
 /* ---------------------------------------------------------------- csr2csc
  * Replaces csrtocsc.csr2csc (src/csr2csc/csr2csc.cc; csr2csc.cu:7-43, a cuSPARSE

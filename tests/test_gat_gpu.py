@@ -40,7 +40,7 @@ def _run(g, h, f, slope=0.2, seed=0, attn_scale=1.0, variant="sm", seg_len=None,
     if variant == "sm":
         out = fg.fused_gat_op(ard, acd, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, slope, xd)
     elif variant == "pipeline":
-        out = fg.fused_gat_fusescatter_pipeline(ard, acd, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, slope, xd, gd.permute)
+        out = fg.fused_gat_operator_pipeline(ard, acd, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, slope, xd, gd.permute)
     elif variant == "stash":
         out = fg.fused_gat_stash_op(ard, acd, gd.row_ptr, gd.col_ind, gd.col_ptr, gd.row_ind, slope, xd, gd.permute)
     else:
@@ -457,8 +457,8 @@ def test_gat_stash_in_both_orders_through_native_calls(h, f, monkeypatch):
 
 @pytest.mark.parametrize("h,f", [(8, 32), (1, 47), (4, 16)])
 def test_fusescatter_pipeline_of_small_operators(h, f, monkeypatch):
-    """The reference's fuse-scatter data flow (softmax kernel -> [E,H] -> SpMM; backward by permuted SpMM, SDDMM,
-    softmax backward, row / column sums) composed from u_add_v, edge softmax and mhspmm: same results as the oracle."""
+    """The layer composed from the stand-alone operators (u_add_v, LeakyReLU, edge softmax, mhspmm; backward by permuted
+    SpMM, SDDMM, softmax backward, row / column sums): same results as the oracle."""
     from ae_mlsys_gnn_amd import _lib
     _run(degree_edge_graph(seed=61), h, f, variant="pipeline")
     monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
@@ -584,4 +584,60 @@ def test_validation_uses_the_width_of_the_gathered_matrix(monkeypatch):
     _lib.clear_schedule_cache()
     with pytest.raises(_lib.FgnnError, match="malformed graph"):
         op.mhspmm(g.row_ptr, g.col_ind, None, feat[:300].contiguous())          # ids up to 399 against 300 rows
+    _lib.clear_schedule_cache()
+
+
+@pytest.mark.parametrize("h", [1, 3, 4, 8, 12, 20, 64])
+def test_fusescatter_kernels_against_the_oracle(h):
+    """fgnn_gat_scatter (scores + LeakyReLU + row softmax in one pass, with and without the LeakyReLU array) and
+    fgnn_gat_gather_row (softmax backward + LeakyReLU backward + row sums, sign from the stashed array or formed again, out
+    of place and in place) on a graph with empty rows, rows either side of the wave / workgroup threshold and a 3000-entry
+    hub, against float64."""
+    from ae_mlsys_gnn_amd.operators.fused_gat import gat_native
+    g = degree_edge_graph(n=300, seed=h)
+    gen = torch.Generator().manual_seed(h)
+    # scores that are exact in float32: the sign of a pre-activation (where LeakyReLU' jumps) is then the same in both precisions
+    ar = torch.randn(g.n, h, generator=gen, dtype=torch.float64).float().double()
+    ac = torch.randn(g.n, h, generator=gen, dtype=torch.float64).float().double()
+    ge = torch.randn(g.n_edges, h, generator=gen, dtype=torch.float64)
+    dst = orc.row_of_edge(g.row_ptr)
+    pre = ar[dst] + ac[g.col_ind.long()]
+    e_ref = torch.nn.functional.leaky_relu(pre, 0.2)
+    sm_ref = orc.edge_softmax(g.row_ptr, e_ref)
+    gd = g.to("cuda:0")
+    ard, acd, ged = ar.float().to("cuda:0"), ac.float().to("cuda:0"), ge.float().to("cuda:0")
+    el, sm = gat_native.gat_scatter(ard, acd, gd.row_ptr, gd.col_ind, 0.2, want_lrelu=True)
+    _, sm2 = gat_native.gat_scatter(ard, acd, gd.row_ptr, gd.col_ind, 0.2)
+    c = c_exp(float(e_ref.max() - e_ref.min()))
+    one = torch.ones((), dtype=torch.float64)
+    assert_close(el, e_ref, "e_lrelu of the scatter kernel")
+    assert_close_sum(sm, sm_ref, one, "e_softmax of the scatter kernel", c=c)
+    assert torch.equal(sm, sm2)
+    # gather_row: d pre = lrelu'(pre) * sm * (ge - sum_row sm * ge)
+    dot = orc.segment_sums(g.row_ptr, sm_ref * ge)
+    dot_abs = orc.segment_sums(g.row_ptr, sm_ref * ge.abs())
+    fac = torch.where(pre > 0, torch.ones_like(pre), torch.full_like(pre, 0.2))
+    gp_ref = fac * sm_ref * (ge - dot[dst])
+    gp_abs = sm_ref * (ge.abs() + dot_abs[dst])
+    gar_ref, gar_abs = orc.segment_sums(g.row_ptr, gp_ref), orc.segment_sums(g.row_ptr, gp_abs)
+    for elr, inplace in ((None, False), (el, False), (None, True)):
+        buf = ged.clone()
+        gp, gar = gat_native.gat_gather_row(0.2, gd.row_ptr, gd.col_ind, ard, acd, sm, buf, e_lrelu=elr, inplace=inplace)
+        assert (gp.data_ptr() == buf.data_ptr()) == inplace
+        what = " (sign %s, %s)" % ("stashed" if elr is not None else "formed again", "in place" if inplace else "out of place")
+        assert_close_sum(gp, gp_ref, gp_abs, "gather_row gradient" + what, c=c)
+        assert_close_sum(gar, gar_ref, gar_abs, "gather_row row sums" + what, c=c)
+
+
+@pytest.mark.parametrize("h,f", [(8, 32), (1, 47), (4, 16), (3, 20)])
+def test_fusescatter_variant_with_the_references_data_flow(h, f, monkeypatch):
+    """FusedGATFunction: scatter kernel + mhspmm forward; permuted mhspmm, mhsddmm, gather_row and column sums backward
+    (src/fused_gat/fused_gat.cu:235-326, 641-670), against the oracle, with plain and XCD-aware work lists."""
+    from ae_mlsys_gnn_amd import _lib
+    _run(degree_edge_graph(seed=63), h, f, variant="fusescatter")
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
+    monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+    monkeypatch.setenv("FGNN_SEG_LEN", "256")
+    _lib.clear_schedule_cache()
+    _run(graphs.rmat_graph(1500, 90000, seed=64), h, f, variant="fusescatter", slope=0.05)
     _lib.clear_schedule_cache()

@@ -310,3 +310,35 @@ def test_column_sum_and_add_bias_equal_the_plain_forms():
     got = torch.autograd.grad((add_bias(x, b) * go).sum(), (x, b))
     assert torch.equal(add_bias(x, b), x + b)
     assert all(torch.allclose(a, w, rtol=1e-10, atol=1e-10) for a, w in zip(got, want))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,c,width", [(1000, 47, 48), (1000, 47, 47), (513, 7, 7), (300, 10, 12), (77, 200, 200), (64, 1000, 1000), (5, 1, 4),
+                                       (2000, 41, 44)])
+def test_fused_cross_entropy_rows(n, c, width):
+    """The drivers' loss on the GPU (fgnn_cross_entropy_forward / _backward): value and gradient of
+    torch.nn.CrossEntropyLoss in float64, for logits that are a [n, c] view of a zero-padded [n, width] array and for
+    the padded array itself with the class count handed over; the gradient of the padding columns is zero."""
+    from ae_mlsys_gnn_amd.train.common import cross_entropy
+    torch.manual_seed(n + c)
+    dev = "cuda:0"
+    padded = torch.zeros(n, width)
+    padded[:, :c] = 4 * torch.randn(n, c)
+    y = torch.randint(0, c, (n,))
+    ref_in = padded[:, :c].double().requires_grad_(True)
+    want = torch.nn.CrossEntropyLoss()(ref_in, y)
+    gw, = torch.autograd.grad(want, ref_in)
+    pd = padded.to(dev).requires_grad_(True)
+    got = cross_entropy(pd, y.to(dev), c)                     # padded array + class count
+    gg, = torch.autograd.grad(got, pd)
+    assert abs(float(got) - float(want)) <= 1e-5 * max(1.0, abs(float(want)))
+    assert torch.allclose(gg[:, :c].cpu().double(), gw, rtol=1e-4, atol=1e-7)
+    assert float(gg[:, c:].abs().max()) == 0.0 if width > c else True
+    pv = padded.to(dev).requires_grad_(True)
+    got2 = cross_entropy(pv[:, :c], y.to(dev))                # a cropped view, read in place
+    gg2, = torch.autograd.grad(got2, pv)
+    assert abs(float(got2) - float(want)) <= 1e-5 * max(1.0, abs(float(want)))
+    assert torch.allclose(gg2[:, :c].cpu().double(), gw, rtol=1e-4, atol=1e-7)
+    # a label outside [0, c) reads nothing and poisons the loss
+    bad = y.clone(); bad[0] = c
+    assert torch.isnan(cross_entropy(padded.to(dev), bad.to(dev), c))

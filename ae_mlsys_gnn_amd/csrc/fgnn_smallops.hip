@@ -304,18 +304,35 @@ extern "C" int fgnn_gather_rows(int64_t E, int W, const int32_t *permute, const 
 // A row's entries are one contiguous run of (pe - pb) * W floats.  Lanes t < S0 = (64 / W) * W of a
 // wave take part and stride by a multiple of W, so lane t only ever sees column t % W and every
 // load is a contiguous run of S0 floats.  Rows of up to SO_LONG_ELEMS floats are taken by one wave
-// each (first launch), longer ones by a whole workgroup each (second launch): a 100 k-entry hub row is
-// then a few hundred trips of 512 threads instead of tens of thousands of trips of one wave.  The second
-// launch has one workgroup per SO_CAND candidate rows: its first wave looks at their lengths, a ballot
-// names the long ones, and the workgroup takes those one after the other (on a 233 k-row power-law graph
-// 31 k rows are long and hold 83 % of the entries; a workgroup per row would start 233 k workgroups of
-// which seven in eight leave at once).
+// each, longer ones by a whole workgroup each: a 100 k-entry hub row is then a few hundred trips of a
+// workgroup instead of tens of thousands of trips of one wave.  Both kinds run in ONE launch: its first
+// workgroups each look at SO_CAND candidate rows (the first wave reads their lengths, a ballot names the
+// long ones, the workgroup takes those one after the other), the workgroups behind them give one short
+// row to each of their waves and fill the machine while the last long rows finish.  (On a 233 k-row
+// power-law graph 31 k rows are long and hold 83 % of the entries; a workgroup per row would start
+// 233 k workgroups of which seven in eight leave at once.)
 #define SO_LONG_ELEMS 8192
-#define SO_LONG_TPB 512
 #define SO_CAND 16            // candidate rows per workgroup of a long-row launch
 #define SO_CACHE 8            // groups per lane kept in registers by the short-row kernels
 #define SO_STREAM 8           // loads in flight per lane in the part of a row that is streamed
-#define SO_CACHE_LONG 16      // ... by the long-row softmax (512 threads x 16 groups x 4 floats = 4096 entries of 8 heads)
+#define SO_CACHE_LONG 16      // ... by the long-row softmax (256 threads x 16 groups x 4 floats = 2048 entries of 8 heads)
+
+// Threads of the workgroups of a row-reduction launch and the grid: n_long workgroups for the long-row candidates, then one
+// short row per wave.  More, smaller workgroups keep more long rows in flight per compute unit (a workgroup works through
+// its rows one after the other, each a chain of dependent memory round trips); larger ones hold more of a row in registers.
+// Measured on a 115 M-entry power-law graph, 8 heads (128 / 256 / 512 threads): softmax 1.93 / 1.78 / 1.84 ms, its backward
+// 3.29 / 2.77 / 2.48, the scatter kernel 3.93 / 3.60 / 4.43, gather-row 4.03 / 4.06 / 4.83, row sums 1.08 / 0.79 / 0.66.
+static inline unsigned so_grid(int N, int64_t elems, int tpb, unsigned *n_long)
+{
+    *n_long = elems > SO_LONG_ELEMS ? (unsigned)((N + SO_CAND - 1) / SO_CAND) : 0u;      // otherwise no row can be long
+    return *n_long + (unsigned)((N + tpb / 64 - 1) / (tpb / 64));
+}
+#define SO_DISPATCH_TPB(tpb, ...)                    \
+    do {                                             \
+        if ((tpb) == 128) { constexpr int TPB = 128; __VA_ARGS__; } \
+        else if ((tpb) == 256) { constexpr int TPB = 256; __VA_ARGS__; } \
+        else { constexpr int TPB = 512; __VA_ARGS__; } \
+    } while (0)
 
 struct so_max { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
 struct so_add { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
@@ -323,8 +340,8 @@ struct so_add { __device__ __forceinline__ float operator()(float a, float b) co
 template <int VEC> struct so_grp { float c[VEC]; };
 
 // Combines, per component, the values of the lanes t, t + W, t + 2W, ... < S0 (any count, by suffix doubling) and
-// of the workgroup's waves (LONG) in a fixed order; every lane gets the result of its column.  W * VEC <= 64.
-template <bool LONG, int VEC, class Op>
+// of the workgroup's NW waves in a fixed order; every lane gets the result of its column.  W * VEC <= 64.
+template <int NW, int VEC, class Op>      // NW: waves that share the row (1: a single wave, no LDS step)
 __device__ __forceinline__ so_grp<VEC> so_column_reduce(so_grp<VEC> v, int lane, int W, int S0, float (*sh)[64], Op op)
 {
     for (int off = W; off < S0; off <<= 1) {
@@ -337,7 +354,7 @@ __device__ __forceinline__ so_grp<VEC> so_column_reduce(so_grp<VEC> v, int lane,
     const int col = lane % W;
 #pragma unroll
     for (int c = 0; c < VEC; ++c) v.c[c] = __shfl(v.c[c], col);
-    if constexpr (LONG) {
+    if constexpr (NW > 1) {
         const int w = fg_wave();
         if (lane < W) {
 #pragma unroll
@@ -347,7 +364,7 @@ __device__ __forceinline__ so_grp<VEC> so_column_reduce(so_grp<VEC> v, int lane,
 #pragma unroll
         for (int c = 0; c < VEC; ++c) {
             float r = sh[0][c * W + col];
-            for (int i = 1; i < SO_LONG_TPB / 64; ++i) r = op(r, sh[i][c * W + col]);
+            for (int i = 1; i < NW; ++i) r = op(r, sh[i][c * W + col]);
             v.c[c] = r;
         }
         __syncthreads();
@@ -442,11 +459,11 @@ template <int VEC> struct so_from_scores {
     }
 };
 
-template <bool LONG, int VEC, int CACHE, class Src>
+template <int NW, int VEC, int CACHE, class Src>
 __device__ __forceinline__ void so_softmax_row(int W, int64_t n, const Src &src, float *__restrict__ dst, float (*sh)[64])
 {
     const int lane = fg_lane(), S0 = (64 / W) * W;
-    const int64_t first = (LONG ? fg_wave() * S0 : 0) + lane, step = (int64_t)S0 * (LONG ? SO_LONG_TPB / 64 : 1);
+    const int64_t first = (NW > 1 ? fg_wave() * S0 : 0) + lane, step = (int64_t)S0 * NW;
     const bool act = lane < S0;
     so_grp<VEC> v[CACHE], m = so_fill<VEC>(-INFINITY), s = so_fill<VEC>(0.f);
 #pragma unroll
@@ -482,14 +499,14 @@ __device__ __forceinline__ void so_softmax_row(int W, int64_t n, const Src &src,
             }
         }
     }
-    const so_grp<VEC> mall = so_column_reduce<LONG, VEC>(m, lane, W, S0, sh, so_max());
+    const so_grp<VEC> mall = so_column_reduce<NW, VEC>(m, lane, W, S0, sh, so_max());
 #pragma unroll
     for (int c = 0; c < VEC; ++c) s.c[c] = s.c[c] > 0.f ? s.c[c] * __expf(m.c[c] - mall.c[c]) : 0.f;      // the streamed part, rebased
 #pragma unroll
     for (int i = 0; i < CACHE; ++i)
 #pragma unroll
         for (int c = 0; c < VEC; ++c) { v[i].c[c] = __expf(v[i].c[c] - mall.c[c]); s.c[c] += v[i].c[c]; }      // exp(-inf) = 0 past the row
-    so_grp<VEC> inv = so_column_reduce<LONG, VEC>(s, lane, W, S0, sh, so_add());
+    so_grp<VEC> inv = so_column_reduce<NW, VEC>(s, lane, W, S0, sh, so_add());
 #pragma unroll
     for (int c = 0; c < VEC; ++c) inv.c[c] = 1.f / inv.c[c];
 #pragma unroll
@@ -517,37 +534,37 @@ __device__ __forceinline__ void so_softmax_row(int W, int64_t n, const Src &src,
 // One launch for both kinds of row: the first n_long_blocks workgroups take the long rows among their SO_CAND candidates
 // (they start first, so the longest rows are not left for the end), the workgroups after them give one short row to each
 // of their eight waves.
-template <int VEC>
-__global__ __launch_bounds__(SO_LONG_TPB) void edge_softmax_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
+template <int VEC, int TPB>
+__global__ __launch_bounds__(TPB) void edge_softmax_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
                                                                    const float *__restrict__ in, float *__restrict__ out)
 {
-    __shared__ float sh[SO_LONG_TPB / 64][64];
+    __shared__ float sh[TPB / 64][64];
     __shared__ unsigned long long sh_mask;
     if (blockIdx.x < n_long_blocks) {
         for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
             const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
             const int pb = fg_uni(ptr[row]);
-            so_softmax_row<true, VEC, SO_CACHE_LONG>(W, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, so_from_array<VEC>{in + (size_t)pb * W * VEC},
+            so_softmax_row<TPB / 64, VEC, SO_CACHE_LONG>(W, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, so_from_array<VEC>{in + (size_t)pb * W * VEC},
                                                      out + (size_t)pb * W * VEC, sh);
         }
         return;
     }
     int row, pb;
     int64_t n;
-    const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (SO_LONG_TPB / 64)) + fg_wave());
+    const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (TPB / 64)) + fg_wave());
     if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n) || n == 0) return;
-    so_softmax_row<false, VEC, SO_CACHE>(W, n, so_from_array<VEC>{in + (size_t)pb * W * VEC}, out + (size_t)pb * W * VEC, nullptr);
+    so_softmax_row<1, VEC, SO_CACHE>(W, n, so_from_array<VEC>{in + (size_t)pb * W * VEC}, out + (size_t)pb * W * VEC, nullptr);
 }
 
 // The fuse-scatter GAT forward (fused_scatter_kernel, src/fused_gat/fused_gat.cu:235-300): scores, LeakyReLU and the row softmax in
 // one pass that writes e_softmax [E,H] (and e_lrelu when asked for).
-template <int VEC>
-__global__ __launch_bounds__(SO_LONG_TPB) void gat_scatter_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
+template <int VEC, int TPB>
+__global__ __launch_bounds__(TPB) void gat_scatter_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
                                                                   const int *__restrict__ idx, const float *__restrict__ ar,
                                                                   const float *__restrict__ ac, float slope, float *__restrict__ elrelu,
                                                                   float *__restrict__ esoft)
 {
-    __shared__ float sh[SO_LONG_TPB / 64][64];
+    __shared__ float sh[TPB / 64][64];
     __shared__ unsigned long long sh_mask;
     const int col = fg_lane() % W;
     auto source = [&](int row, int pb) {
@@ -561,15 +578,15 @@ __global__ __launch_bounds__(SO_LONG_TPB) void gat_scatter_kernel(int N, int W, 
         for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
             const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
             const int pb = fg_uni(ptr[row]);
-            so_softmax_row<true, VEC, SO_CACHE_LONG>(W, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, source(row, pb), esoft + (size_t)pb * W * VEC, sh);
+            so_softmax_row<TPB / 64, VEC, SO_CACHE_LONG>(W, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, source(row, pb), esoft + (size_t)pb * W * VEC, sh);
         }
         return;
     }
     int row, pb;
     int64_t n;
-    const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (SO_LONG_TPB / 64)) + fg_wave());
+    const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (TPB / 64)) + fg_wave());
     if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n) || n == 0) return;
-    so_softmax_row<false, VEC, SO_CACHE>(W, n, source(row, pb), esoft + (size_t)pb * W * VEC, nullptr);
+    so_softmax_row<1, VEC, SO_CACHE>(W, n, source(row, pb), esoft + (size_t)pb * W * VEC, nullptr);
 }
 
 // The factor LeakyReLU' puts on an entry's gradient, for the fused gather_row pass of the fuse-scatter GAT backward
@@ -605,12 +622,12 @@ template <int VEC> struct so_sign_scores {
 
 // gin = factor * sm * (g - sum_row sm * g); with an active Sign also rowsum[lane's heads] = sum_row gin (the grad_attn_row of
 // the fuse-scatter backward).  gin may be g itself: every value is read before it is overwritten, by the same lane.
-template <bool LONG, int VEC, class Sign>
+template <int NW, int VEC, class Sign>
 __device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, const float *__restrict__ sm, const float *g,
                                                    float *gin, const Sign &sign, float *__restrict__ rowsum, float (*sh)[64])
 {
     const int lane = fg_lane(), S0 = (64 / W) * W;
-    const int64_t first = (LONG ? fg_wave() * S0 : 0) + lane, step = (int64_t)S0 * (LONG ? SO_LONG_TPB / 64 : 1);
+    const int64_t first = (NW > 1 ? fg_wave() * S0 : 0) + lane, step = (int64_t)S0 * NW;
     const bool act = lane < S0;
     const size_t base = (size_t)pb * W * VEC;
     so_grp<VEC> sv[SO_CACHE], gv[SO_CACHE], acc = so_fill<VEC>(0.f);
@@ -641,7 +658,7 @@ __device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, con
                 for (int c = 0; c < VEC; ++c) acc.c[c] = fmaf(a[j].c[c], b[j].c[c], acc.c[c]);
         }
     }
-    acc = so_column_reduce<LONG, VEC>(acc, lane, W, S0, sh, so_add());
+    acc = so_column_reduce<NW, VEC>(acc, lane, W, S0, sh, so_add());
     so_grp<VEC> rs = so_fill<VEC>(0.f);
 #pragma unroll
     for (int i = 0; i < SO_CACHE; ++i) {
@@ -684,68 +701,68 @@ __device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, con
         }
     }
     if constexpr (Sign::active) {
-        rs = so_column_reduce<LONG, VEC>(rs, lane, W, S0, sh, so_add());
-        if (lane < W && (!LONG || fg_wave() == 0)) so_store<VEC>(rowsum + (size_t)lane * VEC, rs);
+        rs = so_column_reduce<NW, VEC>(rs, lane, W, S0, sh, so_add());
+        if (lane < W && (NW == 1 || fg_wave() == 0)) so_store<VEC>(rowsum + (size_t)lane * VEC, rs);
     }
 }
 
-template <int VEC>
-__global__ __launch_bounds__(SO_LONG_TPB) void edge_softmax_bwd_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
+template <int VEC, int TPB>
+__global__ __launch_bounds__(TPB) void edge_softmax_bwd_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
                                                                        const float *__restrict__ sm, const float *__restrict__ g,
                                                                        float *__restrict__ gin)
 {
-    __shared__ float sh[SO_LONG_TPB / 64][64];
+    __shared__ float sh[TPB / 64][64];
     __shared__ unsigned long long sh_mask;
     if (blockIdx.x < n_long_blocks) {
         for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
             const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
             const int pb = fg_uni(ptr[row]);
-            so_softmax_bwd_row<true, VEC>(W, pb, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, sm, g, gin, so_sign_none<VEC>{}, nullptr, sh);
+            so_softmax_bwd_row<TPB / 64, VEC>(W, pb, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, sm, g, gin, so_sign_none<VEC>{}, nullptr, sh);
         }
         return;
     }
     int row, pb;
     int64_t n;
-    const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (SO_LONG_TPB / 64)) + fg_wave());
+    const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (TPB / 64)) + fg_wave());
     if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n) || n == 0) return;
-    so_softmax_bwd_row<false, VEC>(W, pb, n, sm, g, gin, so_sign_none<VEC>{}, nullptr, nullptr);
+    so_softmax_bwd_row<1, VEC>(W, pb, n, sm, g, gin, so_sign_none<VEC>{}, nullptr, nullptr);
 }
 
 // fused_gather_row of the fuse-scatter GAT backward (src/fused_gat/fused_gat.cu:502-556): softmax backward, LeakyReLU backward
 // and the row sums (grad_attn_row) in one pass; gout may be g (in place).  Rows without entries get a zero row sum.
-template <int VEC, bool FROM_ARRAY>
-__global__ __launch_bounds__(SO_LONG_TPB) void gat_gather_row_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
+template <int VEC, bool FROM_ARRAY, int TPB>
+__global__ __launch_bounds__(TPB) void gat_gather_row_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
                                                                      const int *__restrict__ idx, const float *__restrict__ ar,
                                                                      const float *__restrict__ ac, const float *__restrict__ elrelu, float slope,
                                                                      const float *__restrict__ sm, const float *g, float *gout,
                                                                      float *__restrict__ gar)
 {
-    __shared__ float sh[SO_LONG_TPB / 64][64];
+    __shared__ float sh[TPB / 64][64];
     __shared__ unsigned long long sh_mask;
     const int col = fg_lane() % W;
-    auto run = [&]<bool LONG>(int row, int pb, int64_t n, float (*shp)[64]) {
+    auto run = [&]<int NW>(int row, int pb, int64_t n, float (*shp)[64]) {
         float *rowsum = gar + (size_t)row * W * VEC;
         if constexpr (FROM_ARRAY) {
-            so_softmax_bwd_row<LONG, VEC>(W, pb, n, sm, g, gout, so_sign_array<VEC>{elrelu + (size_t)pb * W * VEC, slope}, rowsum, shp);
+            so_softmax_bwd_row<NW, VEC>(W, pb, n, sm, g, gout, so_sign_array<VEC>{elrelu + (size_t)pb * W * VEC, slope}, rowsum, shp);
         } else {
             so_sign_scores<VEC> sg;
             sg.idx = idx + pb; sg.ac = ac; sg.ar = so_load<VEC>(ar + ((size_t)row * W + col) * VEC); sg.W = W; sg.col = col; sg.slope = slope;
-            so_softmax_bwd_row<LONG, VEC>(W, pb, n, sm, g, gout, sg, rowsum, shp);
+            so_softmax_bwd_row<NW, VEC>(W, pb, n, sm, g, gout, sg, rowsum, shp);
         }
     };
     if (blockIdx.x < n_long_blocks) {
         for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
             const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
             const int pb = fg_uni(ptr[row]);
-            run.template operator()<true>(row, pb, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, sh);
+            run.template operator()<TPB / 64>(row, pb, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, sh);
         }
         return;
     }
     int row, pb;
     int64_t n;
-    const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (SO_LONG_TPB / 64)) + fg_wave());
+    const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (TPB / 64)) + fg_wave());
     if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n)) return;
-    run.template operator()<false>(row, pb, n, nullptr);             // an empty row stores its zero sums
+    run.template operator()<1>(row, pb, n, nullptr);             // an empty row stores its zero sums
 }
 
 // More than 64 heads: one wave per row, one head at a time.
@@ -795,12 +812,13 @@ extern "C" int fgnn_edge_softmax(int N, int64_t E, int H, const int32_t *row_ptr
         hipLaunchKernelGGL(edge_softmax_wide_kernel, dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, in, out);
         return fgnn_launch_status("edge_softmax_wide_kernel");
     }
-    const unsigned n_long = E * H > SO_LONG_ELEMS ? (unsigned)((N + SO_CAND - 1) / SO_CAND) : 0u;      // otherwise no row can be long
-    const unsigned grid = n_long + (unsigned)((N + SO_LONG_TPB / 64 - 1) / (SO_LONG_TPB / 64));
+    unsigned n_long;
+    const int tpb = 256;
+    const unsigned grid = so_grid(N, E * H, tpb, &n_long);
     if (H % 4 == 0 && fgnn_aligned16(in) && fgnn_aligned16(out))
-        hipLaunchKernelGGL(edge_softmax_kernel<4>, dim3(grid), dim3(SO_LONG_TPB), 0, st, N, H / 4, n_long, row_ptr, in, out);
+        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((edge_softmax_kernel<4, TPB>), dim3(grid), dim3(TPB), 0, st, N, H / 4, n_long, row_ptr, in, out));
     else
-        hipLaunchKernelGGL(edge_softmax_kernel<1>, dim3(grid), dim3(SO_LONG_TPB), 0, st, N, H, n_long, row_ptr, in, out);
+        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((edge_softmax_kernel<1, TPB>), dim3(grid), dim3(TPB), 0, st, N, H, n_long, row_ptr, in, out));
     return fgnn_launch_status("edge_softmax_kernel");
 }
 
@@ -816,12 +834,13 @@ extern "C" int fgnn_edge_softmax_backward(int N, int64_t E, int H, const int32_t
         hipLaunchKernelGGL(edge_softmax_bwd_wide_kernel, dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, sm, grad_out, grad_in);
         return fgnn_launch_status("edge_softmax_bwd_wide_kernel");
     }
-    const unsigned n_long = E * H > SO_LONG_ELEMS ? (unsigned)((N + SO_CAND - 1) / SO_CAND) : 0u;
-    const unsigned grid = n_long + (unsigned)((N + SO_LONG_TPB / 64 - 1) / (SO_LONG_TPB / 64));
+    unsigned n_long;
+    const int tpb = 512;
+    const unsigned grid = so_grid(N, E * H, tpb, &n_long);
     if (H % 4 == 0 && fgnn_aligned16(sm) && fgnn_aligned16(grad_out) && fgnn_aligned16(grad_in))
-        hipLaunchKernelGGL(edge_softmax_bwd_kernel<4>, dim3(grid), dim3(SO_LONG_TPB), 0, st, N, H / 4, n_long, row_ptr, sm, grad_out, grad_in);
+        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((edge_softmax_bwd_kernel<4, TPB>), dim3(grid), dim3(TPB), 0, st, N, H / 4, n_long, row_ptr, sm, grad_out, grad_in));
     else
-        hipLaunchKernelGGL(edge_softmax_bwd_kernel<1>, dim3(grid), dim3(SO_LONG_TPB), 0, st, N, H, n_long, row_ptr, sm, grad_out, grad_in);
+        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((edge_softmax_bwd_kernel<1, TPB>), dim3(grid), dim3(TPB), 0, st, N, H, n_long, row_ptr, sm, grad_out, grad_in));
     return fgnn_launch_status("edge_softmax_bwd_kernel");
 }
 
@@ -837,14 +856,15 @@ extern "C" int fgnn_gat_scatter(int N, int64_t E, int H, const int32_t *row_ptr,
     if (N == 0 || E == 0) return 0;
     FGNN_REQUIRE(row_ptr && col_ind && attn_row && attn_col && e_softmax, FGNN_ERR_NULL, "fgnn_gat_scatter: NULL argument");
     hipStream_t st = (hipStream_t)stream;
-    const unsigned n_long = E * H > SO_LONG_ELEMS ? (unsigned)((N + SO_CAND - 1) / SO_CAND) : 0u;
-    const unsigned grid = n_long + (unsigned)((N + SO_LONG_TPB / 64 - 1) / (SO_LONG_TPB / 64));
+    unsigned n_long;
+    const int tpb = 256;
+    const unsigned grid = so_grid(N, E * H, tpb, &n_long);
     if (H % 4 == 0 && fgnn_aligned16(attn_row) && fgnn_aligned16(attn_col) && fgnn_aligned16(e_softmax) && fgnn_aligned16(e_lrelu))
-        hipLaunchKernelGGL(gat_scatter_kernel<4>, dim3(grid), dim3(SO_LONG_TPB), 0, st, N, H / 4, n_long, row_ptr, col_ind, attn_row, attn_col,
-                           negative_slope, e_lrelu, e_softmax);
+        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((gat_scatter_kernel<4, TPB>), dim3(grid), dim3(TPB), 0, st, N, H / 4, n_long, row_ptr, col_ind, attn_row, attn_col,
+                                                negative_slope, e_lrelu, e_softmax));
     else
-        hipLaunchKernelGGL(gat_scatter_kernel<1>, dim3(grid), dim3(SO_LONG_TPB), 0, st, N, H, n_long, row_ptr, col_ind, attn_row, attn_col,
-                           negative_slope, e_lrelu, e_softmax);
+        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((gat_scatter_kernel<1, TPB>), dim3(grid), dim3(TPB), 0, st, N, H, n_long, row_ptr, col_ind, attn_row, attn_col,
+                                                negative_slope, e_lrelu, e_softmax));
     return fgnn_launch_status("gat_scatter_kernel");
 }
 
@@ -864,13 +884,14 @@ extern "C" int fgnn_gat_gather_row(int N, int64_t E, int H, const int32_t *row_p
     FGNN_REQUIRE(E == 0 || e_lrelu || (col_ind && attn_row && attn_col), FGNN_ERR_NULL,
                  "fgnn_gat_gather_row: without e_lrelu the scores are formed again from col_ind, attn_row and attn_col");
     hipStream_t st = (hipStream_t)stream;
-    const unsigned n_long = E * H > SO_LONG_ELEMS ? (unsigned)((N + SO_CAND - 1) / SO_CAND) : 0u;
-    const unsigned grid = n_long + (unsigned)((N + SO_LONG_TPB / 64 - 1) / (SO_LONG_TPB / 64));
+    unsigned n_long;
+    const int tpb = 256;
+    const unsigned grid = so_grid(N, E * H, tpb, &n_long);
     const bool vec4 = H % 4 == 0 && fgnn_aligned16(e_softmax) && fgnn_aligned16(grad_edge) && fgnn_aligned16(grad_edge_out) && fgnn_aligned16(grad_attn_row) &&
                       fgnn_aligned16(e_lrelu) && fgnn_aligned16(attn_row) && fgnn_aligned16(attn_col);
     const int W = vec4 ? H / 4 : H;
-#define GGR_LAUNCH(V, A) hipLaunchKernelGGL((gat_gather_row_kernel<V, A>), dim3(grid), dim3(SO_LONG_TPB), 0, st, N, W, n_long, row_ptr, col_ind, attn_row, \
-                                            attn_col, e_lrelu, negative_slope, e_softmax, grad_edge, grad_edge_out, grad_attn_row)
+#define GGR_LAUNCH(V, A) SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((gat_gather_row_kernel<V, A, TPB>), dim3(grid), dim3(TPB), 0, st, N, W, n_long, row_ptr, col_ind, \
+                                                                   attn_row, attn_col, e_lrelu, negative_slope, e_softmax, grad_edge, grad_edge_out, grad_attn_row))
     if (vec4) { if (e_lrelu) GGR_LAUNCH(4, true); else GGR_LAUNCH(4, false); }
     else { if (e_lrelu) GGR_LAUNCH(1, true); else GGR_LAUNCH(1, false); }
 #undef GGR_LAUNCH
@@ -957,18 +978,18 @@ __global__ __launch_bounds__(FGNN_TPB) void u_add_v_wide_kernel(int N, int W, co
 // into a zero-filled buffer as the reference does it (src/u_add_v/u_add_v.cu:43-90, which adds into uninitialised
 // memory); without COLS the column sums are left to the tile-ordered pass of fgnn_edge_colsum.  One pass over grad_out,
 // rows shared out as in the softmax kernels.
-template <bool LONG, int VEC, bool COLS>
+template <int NW, int VEC, bool COLS>
 __device__ __forceinline__ void so_rowsum_row(int W, int row, int pb, int pe, const int *__restrict__ idx, const float *__restrict__ g,
                                               float *__restrict__ grow, float *__restrict__ gcol, float (*sh)[64])
 {
     const int lane = fg_lane(), S0 = (64 / W) * W, w = lane % W;
     const int per = S0 / W;                                        // entries per wave-wide trip
-    const int nw = LONG ? SO_LONG_TPB / 64 : 1;
+    constexpr int nw = NW;
     const bool act = lane < S0;
     so_grp<VEC> acc = so_fill<VEC>(0.f);
     if (act) {
 #pragma unroll 8
-        for (int q = pb + (LONG ? fg_wave() * per : 0) + lane / W; q < pe; q += per * nw) {
+        for (int q = pb + (NW > 1 ? fg_wave() * per : 0) + lane / W; q < pe; q += per * nw) {
             const so_grp<VEC> v = so_load<VEC>(g + ((size_t)q * W + w) * VEC);
 #pragma unroll
             for (int c = 0; c < VEC; ++c) acc.c[c] += v.c[c];
@@ -979,29 +1000,29 @@ __device__ __forceinline__ void so_rowsum_row(int W, int row, int pb, int pe, co
             }
         }
     }
-    acc = so_column_reduce<LONG, VEC>(acc, lane, W, S0, sh, so_add());
-    if (lane < W && (!LONG || fg_wave() == 0)) so_store<VEC>(grow + ((size_t)row * W + lane) * VEC, acc);
+    acc = so_column_reduce<NW, VEC>(acc, lane, W, S0, sh, so_add());
+    if (lane < W && (NW == 1 || fg_wave() == 0)) so_store<VEC>(grow + ((size_t)row * W + lane) * VEC, acc);
 }
 
-template <int VEC, bool COLS>
-__global__ __launch_bounds__(SO_LONG_TPB) void edge_rowsum_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
+template <int VEC, bool COLS, int TPB>
+__global__ __launch_bounds__(TPB) void edge_rowsum_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
                                                                   const int *__restrict__ idx, const float *__restrict__ g, float *__restrict__ grow,
                                                                   float *__restrict__ gcol)
 {
-    __shared__ float sh[SO_LONG_TPB / 64][64];
+    __shared__ float sh[TPB / 64][64];
     __shared__ unsigned long long sh_mask;
     if (blockIdx.x < n_long_blocks) {
         for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
             const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
-            so_rowsum_row<true, VEC, COLS>(W, row, fg_uni(ptr[row]), fg_uni(ptr[row + 1]), idx, g, grow, gcol, sh);
+            so_rowsum_row<TPB / 64, VEC, COLS>(W, row, fg_uni(ptr[row]), fg_uni(ptr[row + 1]), idx, g, grow, gcol, sh);
         }
         return;
     }
     int row, pb;
     int64_t n;
-    const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (SO_LONG_TPB / 64)) + fg_wave());
+    const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (TPB / 64)) + fg_wave());
     if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n)) return;      // empty rows stay here: they store zeros
-    so_rowsum_row<false, VEC, COLS>(W, row, pb, fg_uni(ptr[row + 1]), idx, g, grow, gcol, nullptr);
+    so_rowsum_row<1, VEC, COLS>(W, row, pb, fg_uni(ptr[row + 1]), idx, g, grow, gcol, nullptr);
 }
 
 __global__ __launch_bounds__(FGNN_TPB) void u_add_v_bwd_wide_kernel(int N, int W, const int *ptr, const int *idx, const float *g, float *grow, float *gcol)
@@ -1061,9 +1082,9 @@ extern "C" int fgnn_u_add_v_backward(int N, int64_t E, int W, const int32_t *row
     }
     // one float per lane: the atomics of a wave instruction then fall into the fewest cache lines (with four per lane
     // the pass took three times as long on a 115 M-entry graph)
-    const unsigned n_long = E * W > SO_LONG_ELEMS ? (unsigned)((N + SO_CAND - 1) / SO_CAND) : 0u;
-    hipLaunchKernelGGL((edge_rowsum_kernel<1, true>), dim3(n_long + (unsigned)((N + SO_LONG_TPB / 64 - 1) / (SO_LONG_TPB / 64))), dim3(SO_LONG_TPB), 0, st,
-                       N, W, n_long, row_ptr, col_ind, grad_out, grad_row, grad_col);
+    unsigned n_long;
+    const unsigned grid = so_grid(N, E * W, 512, &n_long);
+    hipLaunchKernelGGL((edge_rowsum_kernel<1, true, 512>), dim3(grid), dim3(512), 0, st, N, W, n_long, row_ptr, col_ind, grad_out, grad_row, grad_col);
     return fgnn_launch_status("edge_rowsum_kernel");
 }
 
@@ -1095,12 +1116,13 @@ extern "C" int fgnn_edge_rowsum(int N, int64_t E, int W, const int32_t *row_ptr,
         return fgnn_launch_status("edge_rowsum_wide_kernel");
     }
     const bool vec4 = W % 4 == 0 && fgnn_aligned16(g) && fgnn_aligned16(out);
-    const unsigned n_long = E * W > SO_LONG_ELEMS ? (unsigned)((N + SO_CAND - 1) / SO_CAND) : 0u;
-    const unsigned grid = n_long + (unsigned)((N + SO_LONG_TPB / 64 - 1) / (SO_LONG_TPB / 64));
+    unsigned n_long;
+    const int tpb = 512;
+    const unsigned grid = so_grid(N, E * W, tpb, &n_long);
     if (vec4)
-        hipLaunchKernelGGL((edge_rowsum_kernel<4, false>), dim3(grid), dim3(SO_LONG_TPB), 0, st, N, W / 4, n_long, row_ptr, nullptr, g, out, nullptr);
+        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((edge_rowsum_kernel<4, false, TPB>), dim3(grid), dim3(TPB), 0, st, N, W / 4, n_long, row_ptr, nullptr, g, out, nullptr));
     else
-        hipLaunchKernelGGL((edge_rowsum_kernel<1, false>), dim3(grid), dim3(SO_LONG_TPB), 0, st, N, W, n_long, row_ptr, nullptr, g, out, nullptr);
+        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((edge_rowsum_kernel<1, false, TPB>), dim3(grid), dim3(TPB), 0, st, N, W, n_long, row_ptr, nullptr, g, out, nullptr));
     return fgnn_launch_status("edge_rowsum_kernel");
 }
 

@@ -1096,9 +1096,13 @@ __global__ __launch_bounds__(FGNN_TPB) void edge_rowsum_wide_kernel(int N, int W
     if (row >= N) return;
     const int pb = fg_uni(ptr[row]), pe = fg_uni(ptr[row + 1]);
     for (int w = fg_lane(); w < W; w += 64) {
-        float acc = 0.f;
-        for (int q = pb; q < pe; ++q) acc += g[(size_t)q * W + w];
-        out[(size_t)row * W + w] = acc;
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;       // four interleaved partial sums: four loads in flight, a quarter of the rounding growth
+        int q = pb;
+        for (; q + 4 <= pe; q += 4) {
+            a0 += g[(size_t)q * W + w]; a1 += g[(size_t)(q + 1) * W + w]; a2 += g[(size_t)(q + 2) * W + w]; a3 += g[(size_t)(q + 3) * W + w];
+        }
+        for (; q < pe; ++q) a0 += g[(size_t)q * W + w];
+        out[(size_t)row * W + w] = (a0 + a1) + (a2 + a3);
     }
 }
 

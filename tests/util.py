@@ -30,18 +30,19 @@ def assert_close(got, ref, what, rtol=RTOL, atol=ATOL):
 # C_SUM stands for the roundings a summand carries at unit roundoff 2^-24 apart from its exponent (exp2, the
 # 1/sum normalisation, the weight product, the dot product feeding it, the accumulation).  A weight
 # exp(v) inherits the ABSOLUTE rounding of v as a relative error, so operators with an exponential add
-# one unit per unit of max|v| (c_exp).  Both constants are set from measurement, not from a worst-case
-# count: every comparison records how much of its allowance it used (PARITY_LOG below), the largest share
-# over the whole suite is 0.38 (sequential per-thread sums of 700 terms) and 0.22 at the benchmark sizes, and
-# the full-size tests assert that no element uses more than half (max_ratio = 0.5).  With the constants of a
-# worst-case count (16 and 4 per unit) no element used more than a tenth.  Not tuned per test.
+# a quarter of that per unit of max|v| (c_exp).  The constant is set from measurement, not from a worst-case
+# count: every comparison records how much of its allowance it used (PARITY_LOG below); with C_SUM = 2.5 the
+# largest share over the whole suite is 0.39 (a stored-weight SpMM over rows of 1024+ floats) and 0.36 at the
+# benchmark sizes (grad_attn_col of the 1 x 47 output layer on the 64 M-edge graph), and the full-size tests assert
+# that no element uses more than half (MAX_RATIO).  With the constants of a worst-case count (16, and 4 per unit)
+# no element used more than a tenth of its allowance.  Not tuned per test.
 EPS32 = 2.0 ** -24
-C_SUM = 4.0
+C_SUM = 2.5
 MAX_RATIO = 0.5
 
 
 def c_exp(max_abs_exponent):
-    return C_SUM + 1.0 * float(max_abs_exponent)
+    return C_SUM * (1.0 + 0.25 * float(max_abs_exponent))
 
 
 # Every assert_close_sum call leaves a record here: how much of the derived allowance the comparison needed.

@@ -313,9 +313,23 @@ extern "C" int fgnn_gather_rows(int64_t E, int W, const int32_t *permute, const 
 // 233 k workgroups of which seven in eight leave at once.)
 #define SO_LONG_ELEMS 8192
 #define SO_CAND 16            // candidate rows per workgroup of a long-row launch
-#define SO_CACHE 8            // groups per lane kept in registers by the short-row kernels
-#define SO_STREAM 8           // loads in flight per lane in the part of a row that is streamed
-#define SO_CACHE_LONG 16      // ... by the long-row softmax (256 threads x 16 groups x 4 floats = 2048 entries of 8 heads)
+// Registers a row-reduction kernel spends on a row: CACHE groups of VEC floats per lane kept over both phases by a wave on a short
+// row, CLONG by the workgroup on a long row, STREAM loads in flight per lane in the part of a row that is streamed.  The numbers
+// set the kernel's register count and with it the waves resident per SIMD: rows that mostly fit one trip of a wave want a small
+// footprint (each row is a chain of dependent memory round trips, and only the rows in flight hide it), rows of thousands of
+// values want the cache (what is not cached is read twice).  A launch picks between a configuration for dense rows and one for
+// sparse rows by the mean row length.  Measured (softmax / backward / scatter / gather-row, ms; [cache, long cache, stream]):
+//   114.8 M entries in 233 k rows, 8 heads:  [8,16,8] 1.79 / 2.49 / 3.60 / 4.07   [4,8,4] 1.85 / 2.70 / 2.56 / 3.56   [2,4,4] 1.97 / 2.89 / 2.67 / 3.74
+//   64.3 M entries in 2.45 M rows, 8 heads:  [8,16,8] 3.13 / 3.61 / 6.92 / 7.34   [4,8,4] 2.50 / 2.41 / 3.58 / 4.07   [2,4,4] 2.01 / 2.00 / 3.55 / 3.53
+template <int CACHE_, int CLONG_, int STREAM_> struct so_cfg { static constexpr int CACHE = CACHE_, CLONG = CLONG_, STREAM = STREAM_; };
+#define SO_DENSE_ROW_FLOATS 1024          // mean floats per row from which a launch takes its dense-row configuration
+static inline bool so_dense_rows(int N, int64_t elems) { return elems >= (int64_t)SO_DENSE_ROW_FLOATS * N; }
+// launch.operator()<VEC, CFG>() with VEC = 4 or 1 and CFG = the `dense` or `sparse` type of the calling scope
+#define SO_LAUNCH_BY_ROWS(launch, vec4, is_dense)                                                         \
+    do {                                                                                                  \
+        if (vec4) { if (is_dense) launch.template operator()<4, dense>(); else launch.template operator()<4, sparse>(); } \
+        else { if (is_dense) launch.template operator()<1, dense>(); else launch.template operator()<1, sparse>(); }     \
+    } while (0)
 
 // Threads of the workgroups of a row-reduction launch and the grid: n_long workgroups for the long-row candidates, then one
 // short row per wave.  More, smaller workgroups keep more long rows in flight per compute unit (a workgroup works through
@@ -327,12 +341,6 @@ static inline unsigned so_grid(int N, int64_t elems, int tpb, unsigned *n_long)
     *n_long = elems > SO_LONG_ELEMS ? (unsigned)((N + SO_CAND - 1) / SO_CAND) : 0u;      // otherwise no row can be long
     return *n_long + (unsigned)((N + tpb / 64 - 1) / (tpb / 64));
 }
-#define SO_DISPATCH_TPB(tpb, ...)                    \
-    do {                                             \
-        if ((tpb) == 128) { constexpr int TPB = 128; __VA_ARGS__; } \
-        else if ((tpb) == 256) { constexpr int TPB = 256; __VA_ARGS__; } \
-        else { constexpr int TPB = 512; __VA_ARGS__; } \
-    } while (0)
 
 struct so_max { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
 struct so_add { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
@@ -459,7 +467,7 @@ template <int VEC> struct so_from_scores {
     }
 };
 
-template <int NW, int VEC, int CACHE, class Src>
+template <int NW, int VEC, int CACHE, int STREAM, class Src>
 __device__ __forceinline__ void so_softmax_row(int W, int64_t n, const Src &src, float *__restrict__ dst, float (*sh)[64])
 {
     const int lane = fg_lane(), S0 = (64 / W) * W;
@@ -477,23 +485,23 @@ __device__ __forceinline__ void so_softmax_row(int W, int64_t n, const Src &src,
         for (int c = 0; c < VEC; ++c) m.c[c] = fmaxf(m.c[c], v[i].c[c]);
     const int64_t rest = first + CACHE * step;
     // a lane that gets here has CACHE valid groups, so its m is finite and m - max(m, t) is never inf - inf.
-    // SO_STREAM loads are issued before the first is used: a row that one workgroup streams alone is bound by the
+    // STREAM loads are issued before the first is used: a row that one workgroup streams alone is bound by the
     // bytes it keeps in flight.
     if (act) {
-        for (int64_t k0 = rest; k0 < n; k0 += SO_STREAM * step) {
-            so_grp<VEC> t[SO_STREAM];
+        for (int64_t k0 = rest; k0 < n; k0 += STREAM * step) {
+            so_grp<VEC> t[STREAM];
 #pragma unroll
-            for (int j = 0; j < SO_STREAM; ++j) t[j] = k0 + j * step < n ? src.load(k0 + j * step, true) : so_fill<VEC>(-INFINITY);
+            for (int j = 0; j < STREAM; ++j) t[j] = k0 + j * step < n ? src.load(k0 + j * step, true) : so_fill<VEC>(-INFINITY);
             so_grp<VEC> mn = m;
 #pragma unroll
-            for (int j = 0; j < SO_STREAM; ++j)
+            for (int j = 0; j < STREAM; ++j)
 #pragma unroll
                 for (int c = 0; c < VEC; ++c) mn.c[c] = fmaxf(mn.c[c], t[j].c[c]);
 #pragma unroll
             for (int c = 0; c < VEC; ++c) {
                 float acc = s.c[c] * __expf(m.c[c] - mn.c[c]);
 #pragma unroll
-                for (int j = 0; j < SO_STREAM; ++j) acc += __expf(t[j].c[c] - mn.c[c]);       // exp(-inf) = 0 past the row
+                for (int j = 0; j < STREAM; ++j) acc += __expf(t[j].c[c] - mn.c[c]);       // exp(-inf) = 0 past the row
                 s.c[c] = acc;
                 m.c[c] = mn.c[c];
             }
@@ -517,12 +525,12 @@ __device__ __forceinline__ void so_softmax_row(int W, int64_t n, const Src &src,
         if (act && k < n) so_store<VEC>(dst + k * VEC, v[i]);
     }
     if (act) {
-        for (int64_t k0 = rest; k0 < n; k0 += SO_STREAM * step) {
-            so_grp<VEC> t[SO_STREAM];
+        for (int64_t k0 = rest; k0 < n; k0 += STREAM * step) {
+            so_grp<VEC> t[STREAM];
 #pragma unroll
-            for (int j = 0; j < SO_STREAM; ++j) t[j] = k0 + j * step < n ? src.load(k0 + j * step, false) : so_fill<VEC>(0.f);
+            for (int j = 0; j < STREAM; ++j) t[j] = k0 + j * step < n ? src.load(k0 + j * step, false) : so_fill<VEC>(0.f);
 #pragma unroll
-            for (int j = 0; j < SO_STREAM; ++j) {
+            for (int j = 0; j < STREAM; ++j) {
 #pragma unroll
                 for (int c = 0; c < VEC; ++c) t[j].c[c] = __expf(t[j].c[c] - mall.c[c]) * inv.c[c];
                 if (k0 + j * step < n) so_store<VEC>(dst + (k0 + j * step) * VEC, t[j]);
@@ -534,7 +542,7 @@ __device__ __forceinline__ void so_softmax_row(int W, int64_t n, const Src &src,
 // One launch for both kinds of row: the first n_long_blocks workgroups take the long rows among their SO_CAND candidates
 // (they start first, so the longest rows are not left for the end), the workgroups after them give one short row to each
 // of their eight waves.
-template <int VEC, int TPB>
+template <int VEC, int TPB, class CFG>
 __global__ __launch_bounds__(TPB) void edge_softmax_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
                                                                    const float *__restrict__ in, float *__restrict__ out)
 {
@@ -544,7 +552,7 @@ __global__ __launch_bounds__(TPB) void edge_softmax_kernel(int N, int W, unsigne
         for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
             const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
             const int pb = fg_uni(ptr[row]);
-            so_softmax_row<TPB / 64, VEC, SO_CACHE_LONG>(W, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, so_from_array<VEC>{in + (size_t)pb * W * VEC},
+            so_softmax_row<TPB / 64, VEC, CFG::CLONG, CFG::STREAM>(W, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, so_from_array<VEC>{in + (size_t)pb * W * VEC},
                                                      out + (size_t)pb * W * VEC, sh);
         }
         return;
@@ -553,12 +561,12 @@ __global__ __launch_bounds__(TPB) void edge_softmax_kernel(int N, int W, unsigne
     int64_t n;
     const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (TPB / 64)) + fg_wave());
     if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n) || n == 0) return;
-    so_softmax_row<1, VEC, SO_CACHE>(W, n, so_from_array<VEC>{in + (size_t)pb * W * VEC}, out + (size_t)pb * W * VEC, nullptr);
+    so_softmax_row<1, VEC, CFG::CACHE, CFG::STREAM>(W, n, so_from_array<VEC>{in + (size_t)pb * W * VEC}, out + (size_t)pb * W * VEC, nullptr);
 }
 
 // The fuse-scatter GAT forward (fused_scatter_kernel, src/fused_gat/fused_gat.cu:235-300): scores, LeakyReLU and the row softmax in
 // one pass that writes e_softmax [E,H] (and e_lrelu when asked for).
-template <int VEC, int TPB>
+template <int VEC, int TPB, class CFG>
 __global__ __launch_bounds__(TPB) void gat_scatter_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
                                                                   const int *__restrict__ idx, const float *__restrict__ ar,
                                                                   const float *__restrict__ ac, float slope, float *__restrict__ elrelu,
@@ -578,7 +586,7 @@ __global__ __launch_bounds__(TPB) void gat_scatter_kernel(int N, int W, unsigned
         for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
             const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
             const int pb = fg_uni(ptr[row]);
-            so_softmax_row<TPB / 64, VEC, SO_CACHE_LONG>(W, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, source(row, pb), esoft + (size_t)pb * W * VEC, sh);
+            so_softmax_row<TPB / 64, VEC, CFG::CLONG, CFG::STREAM>(W, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, source(row, pb), esoft + (size_t)pb * W * VEC, sh);
         }
         return;
     }
@@ -586,7 +594,7 @@ __global__ __launch_bounds__(TPB) void gat_scatter_kernel(int N, int W, unsigned
     int64_t n;
     const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (TPB / 64)) + fg_wave());
     if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n) || n == 0) return;
-    so_softmax_row<1, VEC, SO_CACHE>(W, n, source(row, pb), esoft + (size_t)pb * W * VEC, nullptr);
+    so_softmax_row<1, VEC, CFG::CACHE, CFG::STREAM>(W, n, source(row, pb), esoft + (size_t)pb * W * VEC, nullptr);
 }
 
 // The factor LeakyReLU' puts on an entry's gradient, for the fused gather_row pass of the fuse-scatter GAT backward
@@ -622,7 +630,7 @@ template <int VEC> struct so_sign_scores {
 
 // gin = factor * sm * (g - sum_row sm * g); with an active Sign also rowsum[lane's heads] = sum_row gin (the grad_attn_row of
 // the fuse-scatter backward).  gin may be g itself: every value is read before it is overwritten, by the same lane.
-template <int NW, int VEC, class Sign>
+template <int NW, int VEC, int CACHE, int STREAM, class Sign>
 __device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, const float *__restrict__ sm, const float *g,
                                                    float *gin, const Sign &sign, float *__restrict__ rowsum, float (*sh)[64])
 {
@@ -630,30 +638,30 @@ __device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, con
     const int64_t first = (NW > 1 ? fg_wave() * S0 : 0) + lane, step = (int64_t)S0 * NW;
     const bool act = lane < S0;
     const size_t base = (size_t)pb * W * VEC;
-    so_grp<VEC> sv[SO_CACHE], gv[SO_CACHE], acc = so_fill<VEC>(0.f);
+    so_grp<VEC> sv[CACHE], gv[CACHE], acc = so_fill<VEC>(0.f);
 #pragma unroll
-    for (int i = 0; i < SO_CACHE; ++i) {
+    for (int i = 0; i < CACHE; ++i) {
         const int64_t k = first + i * step;
         const bool ok = act && k < n;
         sv[i] = ok ? so_load<VEC>(sm + base + k * VEC) : so_fill<VEC>(0.f);
         gv[i] = ok ? so_load<VEC>(g + base + k * VEC) : so_fill<VEC>(0.f);
     }
 #pragma unroll
-    for (int i = 0; i < SO_CACHE; ++i)
+    for (int i = 0; i < CACHE; ++i)
 #pragma unroll
         for (int c = 0; c < VEC; ++c) acc.c[c] = fmaf(sv[i].c[c], gv[i].c[c], acc.c[c]);
-    const int64_t rest = first + SO_CACHE * step;
+    const int64_t rest = first + CACHE * step;
     if (act) {
-        for (int64_t k0 = rest; k0 < n; k0 += (SO_STREAM / 2) * step) {
-            so_grp<VEC> a[SO_STREAM / 2], b[SO_STREAM / 2];
+        for (int64_t k0 = rest; k0 < n; k0 += STREAM * step) {
+            so_grp<VEC> a[STREAM], b[STREAM];
 #pragma unroll
-            for (int j = 0; j < SO_STREAM / 2; ++j) {
+            for (int j = 0; j < STREAM; ++j) {
                 const bool ok = k0 + j * step < n;
                 a[j] = ok ? so_load<VEC>(sm + base + (k0 + j * step) * VEC) : so_fill<VEC>(0.f);
                 b[j] = ok ? so_load<VEC>(g + base + (k0 + j * step) * VEC) : so_fill<VEC>(0.f);
             }
 #pragma unroll
-            for (int j = 0; j < SO_STREAM / 2; ++j)
+            for (int j = 0; j < STREAM; ++j)
 #pragma unroll
                 for (int c = 0; c < VEC; ++c) acc.c[c] = fmaf(a[j].c[c], b[j].c[c], acc.c[c]);
         }
@@ -661,7 +669,7 @@ __device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, con
     acc = so_column_reduce<NW, VEC>(acc, lane, W, S0, sh, so_add());
     so_grp<VEC> rs = so_fill<VEC>(0.f);
 #pragma unroll
-    for (int i = 0; i < SO_CACHE; ++i) {
+    for (int i = 0; i < CACHE; ++i) {
         const int64_t k = first + i * step;
         const bool ok = act && k < n;
 #pragma unroll
@@ -676,16 +684,16 @@ __device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, con
         if (ok) so_store<VEC>(gin + base + k * VEC, sv[i]);
     }
     if (act) {
-        for (int64_t k0 = rest; k0 < n; k0 += (SO_STREAM / 2) * step) {
-            so_grp<VEC> a[SO_STREAM / 2], b[SO_STREAM / 2];
+        for (int64_t k0 = rest; k0 < n; k0 += STREAM * step) {
+            so_grp<VEC> a[STREAM], b[STREAM];
 #pragma unroll
-            for (int j = 0; j < SO_STREAM / 2; ++j) {
+            for (int j = 0; j < STREAM; ++j) {
                 const bool ok = k0 + j * step < n;
                 a[j] = ok ? so_load<VEC>(sm + base + (k0 + j * step) * VEC) : so_fill<VEC>(0.f);
                 b[j] = ok ? so_load<VEC>(g + base + (k0 + j * step) * VEC) : so_fill<VEC>(0.f);
             }
 #pragma unroll
-            for (int j = 0; j < SO_STREAM / 2; ++j) {
+            for (int j = 0; j < STREAM; ++j) {
                 const bool ok = k0 + j * step < n;
 #pragma unroll
                 for (int c = 0; c < VEC; ++c) a[j].c[c] *= b[j].c[c] - acc.c[c];
@@ -706,7 +714,7 @@ __device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, con
     }
 }
 
-template <int VEC, int TPB>
+template <int VEC, int TPB, class CFG>
 __global__ __launch_bounds__(TPB) void edge_softmax_bwd_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
                                                                        const float *__restrict__ sm, const float *__restrict__ g,
                                                                        float *__restrict__ gin)
@@ -717,7 +725,7 @@ __global__ __launch_bounds__(TPB) void edge_softmax_bwd_kernel(int N, int W, uns
         for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
             const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
             const int pb = fg_uni(ptr[row]);
-            so_softmax_bwd_row<TPB / 64, VEC>(W, pb, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, sm, g, gin, so_sign_none<VEC>{}, nullptr, sh);
+            so_softmax_bwd_row<TPB / 64, VEC, CFG::CACHE, CFG::STREAM>(W, pb, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, sm, g, gin, so_sign_none<VEC>{}, nullptr, sh);
         }
         return;
     }
@@ -725,12 +733,12 @@ __global__ __launch_bounds__(TPB) void edge_softmax_bwd_kernel(int N, int W, uns
     int64_t n;
     const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (TPB / 64)) + fg_wave());
     if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n) || n == 0) return;
-    so_softmax_bwd_row<1, VEC>(W, pb, n, sm, g, gin, so_sign_none<VEC>{}, nullptr, nullptr);
+    so_softmax_bwd_row<1, VEC, CFG::CACHE, CFG::STREAM>(W, pb, n, sm, g, gin, so_sign_none<VEC>{}, nullptr, nullptr);
 }
 
 // fused_gather_row of the fuse-scatter GAT backward (src/fused_gat/fused_gat.cu:502-556): softmax backward, LeakyReLU backward
 // and the row sums (grad_attn_row) in one pass; gout may be g (in place).  Rows without entries get a zero row sum.
-template <int VEC, bool FROM_ARRAY, int TPB>
+template <int VEC, bool FROM_ARRAY, int TPB, class CFG>
 __global__ __launch_bounds__(TPB) void gat_gather_row_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
                                                                      const int *__restrict__ idx, const float *__restrict__ ar,
                                                                      const float *__restrict__ ac, const float *__restrict__ elrelu, float slope,
@@ -743,11 +751,11 @@ __global__ __launch_bounds__(TPB) void gat_gather_row_kernel(int N, int W, unsig
     auto run = [&]<int NW>(int row, int pb, int64_t n, float (*shp)[64]) {
         float *rowsum = gar + (size_t)row * W * VEC;
         if constexpr (FROM_ARRAY) {
-            so_softmax_bwd_row<NW, VEC>(W, pb, n, sm, g, gout, so_sign_array<VEC>{elrelu + (size_t)pb * W * VEC, slope}, rowsum, shp);
+            so_softmax_bwd_row<NW, VEC, CFG::CACHE, CFG::STREAM>(W, pb, n, sm, g, gout, so_sign_array<VEC>{elrelu + (size_t)pb * W * VEC, slope}, rowsum, shp);
         } else {
             so_sign_scores<VEC> sg;
             sg.idx = idx + pb; sg.ac = ac; sg.ar = so_load<VEC>(ar + ((size_t)row * W + col) * VEC); sg.W = W; sg.col = col; sg.slope = slope;
-            so_softmax_bwd_row<NW, VEC>(W, pb, n, sm, g, gout, sg, rowsum, shp);
+            so_softmax_bwd_row<NW, VEC, CFG::CACHE, CFG::STREAM>(W, pb, n, sm, g, gout, sg, rowsum, shp);
         }
     };
     if (blockIdx.x < n_long_blocks) {
@@ -813,12 +821,15 @@ extern "C" int fgnn_edge_softmax(int N, int64_t E, int H, const int32_t *row_ptr
         return fgnn_launch_status("edge_softmax_wide_kernel");
     }
     unsigned n_long;
-    const int tpb = 256;
-    const unsigned grid = so_grid(N, E * H, tpb, &n_long);
-    if (H % 4 == 0 && fgnn_aligned16(in) && fgnn_aligned16(out))
-        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((edge_softmax_kernel<4, TPB>), dim3(grid), dim3(TPB), 0, st, N, H / 4, n_long, row_ptr, in, out));
-    else
-        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((edge_softmax_kernel<1, TPB>), dim3(grid), dim3(TPB), 0, st, N, H, n_long, row_ptr, in, out));
+    constexpr int TPB = 256;
+    const unsigned grid = so_grid(N, E * H, TPB, &n_long);
+    const bool vec4 = H % 4 == 0 && fgnn_aligned16(in) && fgnn_aligned16(out);
+    auto launch = [&]<int VEC, class CFG>() {
+        hipLaunchKernelGGL((edge_softmax_kernel<VEC, TPB, CFG>), dim3(grid), dim3(TPB), 0, st, N, H / VEC, n_long, row_ptr, in, out);
+    };
+    using dense = so_cfg<8, 16, 8>;
+    using sparse = so_cfg<2, 4, 4>;
+    SO_LAUNCH_BY_ROWS(launch, vec4, so_dense_rows(N, E * H));
     return fgnn_launch_status("edge_softmax_kernel");
 }
 
@@ -835,12 +846,15 @@ extern "C" int fgnn_edge_softmax_backward(int N, int64_t E, int H, const int32_t
         return fgnn_launch_status("edge_softmax_bwd_wide_kernel");
     }
     unsigned n_long;
-    const int tpb = 512;
-    const unsigned grid = so_grid(N, E * H, tpb, &n_long);
-    if (H % 4 == 0 && fgnn_aligned16(sm) && fgnn_aligned16(grad_out) && fgnn_aligned16(grad_in))
-        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((edge_softmax_bwd_kernel<4, TPB>), dim3(grid), dim3(TPB), 0, st, N, H / 4, n_long, row_ptr, sm, grad_out, grad_in));
-    else
-        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((edge_softmax_bwd_kernel<1, TPB>), dim3(grid), dim3(TPB), 0, st, N, H, n_long, row_ptr, sm, grad_out, grad_in));
+    constexpr int TPB = 512;
+    const unsigned grid = so_grid(N, E * H, TPB, &n_long);
+    const bool vec4 = H % 4 == 0 && fgnn_aligned16(sm) && fgnn_aligned16(grad_out) && fgnn_aligned16(grad_in);
+    auto launch = [&]<int VEC, class CFG>() {
+        hipLaunchKernelGGL((edge_softmax_bwd_kernel<VEC, TPB, CFG>), dim3(grid), dim3(TPB), 0, st, N, H / VEC, n_long, row_ptr, sm, grad_out, grad_in);
+    };
+    using dense = so_cfg<8, 8, 4>;           // the backward keeps two arrays: CACHE groups of each, STREAM loads of each in flight
+    using sparse = so_cfg<2, 2, 2>;
+    SO_LAUNCH_BY_ROWS(launch, vec4, so_dense_rows(N, E * H));
     return fgnn_launch_status("edge_softmax_bwd_kernel");
 }
 
@@ -857,14 +871,16 @@ extern "C" int fgnn_gat_scatter(int N, int64_t E, int H, const int32_t *row_ptr,
     FGNN_REQUIRE(row_ptr && col_ind && attn_row && attn_col && e_softmax, FGNN_ERR_NULL, "fgnn_gat_scatter: NULL argument");
     hipStream_t st = (hipStream_t)stream;
     unsigned n_long;
-    const int tpb = 256;
-    const unsigned grid = so_grid(N, E * H, tpb, &n_long);
-    if (H % 4 == 0 && fgnn_aligned16(attn_row) && fgnn_aligned16(attn_col) && fgnn_aligned16(e_softmax) && fgnn_aligned16(e_lrelu))
-        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((gat_scatter_kernel<4, TPB>), dim3(grid), dim3(TPB), 0, st, N, H / 4, n_long, row_ptr, col_ind, attn_row, attn_col,
-                                                negative_slope, e_lrelu, e_softmax));
-    else
-        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((gat_scatter_kernel<1, TPB>), dim3(grid), dim3(TPB), 0, st, N, H, n_long, row_ptr, col_ind, attn_row, attn_col,
-                                                negative_slope, e_lrelu, e_softmax));
+    constexpr int TPB = 256;
+    const unsigned grid = so_grid(N, E * H, TPB, &n_long);
+    const bool vec4 = H % 4 == 0 && fgnn_aligned16(attn_row) && fgnn_aligned16(attn_col) && fgnn_aligned16(e_softmax) && fgnn_aligned16(e_lrelu);
+    auto launch = [&]<int VEC, class CFG>() {
+        hipLaunchKernelGGL((gat_scatter_kernel<VEC, TPB, CFG>), dim3(grid), dim3(TPB), 0, st, N, H / VEC, n_long, row_ptr, col_ind, attn_row, attn_col,
+                           negative_slope, e_lrelu, e_softmax);
+    };
+    using dense = so_cfg<4, 8, 4>;           // every load is an index and a gathered row: fewer in flight, more waves resident
+    using sparse = so_cfg<2, 4, 4>;
+    SO_LAUNCH_BY_ROWS(launch, vec4, so_dense_rows(N, E * H));
     return fgnn_launch_status("gat_scatter_kernel");
 }
 
@@ -885,16 +901,20 @@ extern "C" int fgnn_gat_gather_row(int N, int64_t E, int H, const int32_t *row_p
                  "fgnn_gat_gather_row: without e_lrelu the scores are formed again from col_ind, attn_row and attn_col");
     hipStream_t st = (hipStream_t)stream;
     unsigned n_long;
-    const int tpb = 256;
-    const unsigned grid = so_grid(N, E * H, tpb, &n_long);
+    constexpr int TPB = 256;
+    const unsigned grid = so_grid(N, E * H, TPB, &n_long);
     const bool vec4 = H % 4 == 0 && fgnn_aligned16(e_softmax) && fgnn_aligned16(grad_edge) && fgnn_aligned16(grad_edge_out) && fgnn_aligned16(grad_attn_row) &&
                       fgnn_aligned16(e_lrelu) && fgnn_aligned16(attn_row) && fgnn_aligned16(attn_col);
-    const int W = vec4 ? H / 4 : H;
-#define GGR_LAUNCH(V, A) SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((gat_gather_row_kernel<V, A, TPB>), dim3(grid), dim3(TPB), 0, st, N, W, n_long, row_ptr, col_ind, \
-                                                                   attn_row, attn_col, e_lrelu, negative_slope, e_softmax, grad_edge, grad_edge_out, grad_attn_row))
-    if (vec4) { if (e_lrelu) GGR_LAUNCH(4, true); else GGR_LAUNCH(4, false); }
-    else { if (e_lrelu) GGR_LAUNCH(1, true); else GGR_LAUNCH(1, false); }
-#undef GGR_LAUNCH
+    auto launch = [&]<int VEC, class CFG>() {
+        auto go = [&]<bool FROM_ARRAY>() {
+            hipLaunchKernelGGL((gat_gather_row_kernel<VEC, FROM_ARRAY, TPB, CFG>), dim3(grid), dim3(TPB), 0, st, N, H / VEC, n_long, row_ptr, col_ind,
+                               attn_row, attn_col, e_lrelu, negative_slope, e_softmax, grad_edge, grad_edge_out, grad_attn_row);
+        };
+        if (e_lrelu) go.template operator()<true>(); else go.template operator()<false>();
+    };
+    using dense = so_cfg<8, 8, 2>;
+    using sparse = so_cfg<4, 4, 1>;
+    SO_LAUNCH_BY_ROWS(launch, vec4, so_dense_rows(N, E * H));
     return fgnn_launch_status("gat_gather_row_kernel");
 }
 
@@ -1121,12 +1141,12 @@ extern "C" int fgnn_edge_rowsum(int N, int64_t E, int W, const int32_t *row_ptr,
     }
     const bool vec4 = W % 4 == 0 && fgnn_aligned16(g) && fgnn_aligned16(out);
     unsigned n_long;
-    const int tpb = 512;
-    const unsigned grid = so_grid(N, E * W, tpb, &n_long);
+    constexpr int TPB = 512;
+    const unsigned grid = so_grid(N, E * W, TPB, &n_long);
     if (vec4)
-        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((edge_rowsum_kernel<4, false, TPB>), dim3(grid), dim3(TPB), 0, st, N, W / 4, n_long, row_ptr, nullptr, g, out, nullptr));
+        hipLaunchKernelGGL((edge_rowsum_kernel<4, false, TPB>), dim3(grid), dim3(TPB), 0, st, N, W / 4, n_long, row_ptr, nullptr, g, out, nullptr);
     else
-        SO_DISPATCH_TPB(tpb, hipLaunchKernelGGL((edge_rowsum_kernel<1, false, TPB>), dim3(grid), dim3(TPB), 0, st, N, W, n_long, row_ptr, nullptr, g, out, nullptr));
+        hipLaunchKernelGGL((edge_rowsum_kernel<1, false, TPB>), dim3(grid), dim3(TPB), 0, st, N, W, n_long, row_ptr, nullptr, g, out, nullptr);
     return fgnn_launch_status("edge_rowsum_kernel");
 }
 

@@ -71,9 +71,20 @@ __device__ __forceinline__ void spmm_store_row(const SpmmP &p, int row, const fg
 struct WAtt {
     const float *att;   // [E,H] or NULL (all ones)
     int ld;             // floats between consecutive entries of att (H, or more when att is a view of a wider array)
+    bool vec4;          // H % 4 == 0, ld % 4 == 0 and att 16-byte aligned: an entry's weights load as 128-bit words
     __device__ __forceinline__ void prepare(float *, int, int) const {}
     __device__ __forceinline__ void fill(float *wl, const float *, int lane, size_t pos, bool ok, int H) const
     {
+        if (att && vec4) {
+            // one 128-bit load per four heads instead of four strided 32-bit ones: the entry positions of a chunk are
+            // scattered wherever the work list reorders a row, and each instruction costs a pass of the address unit
+            const float4 *src = reinterpret_cast<const float4 *>(att + pos * ld);
+            for (int h = 0; h < H; h += 4) {
+                const float4 v = ok ? src[h >> 2] : make_float4(0.f, 0.f, 0.f, 0.f);
+                wl[h * 64 + lane] = v.x; wl[(h + 1) * 64 + lane] = v.y; wl[(h + 2) * 64 + lane] = v.z; wl[(h + 3) * 64 + lane] = v.w;
+            }
+            return;
+        }
         for (int h = 0; h < H; ++h) wl[h * 64 + lane] = ok ? (att ? att[pos * ld + h] : 1.f) : 0.f;
     }
 };

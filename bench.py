@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused GNN sparse-operator path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gat_c2|gat_c5|gat_c5_train|edgeconv_c3|gmm_c4|gather_ceiling]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gat_c2|gat_c5|gat_c5_l2|gat_c5_train|edgeconv_c3|gmm_c4|small_ops_c2|gather_ceiling]
 
 Default workload = benchmark configuration 2: one fused GAT layer forward+backward (dense projection by
 torch.matmul, fused sparse op by libfgnn_hip.so) on a seeded R-MAT power-law graph with 232,965
@@ -12,6 +12,9 @@ metric, the roofline record of the dominant kernel and a CPU baseline (the torch
 layer of oracle/ on the host cores, on a bounded sample of the same graph).  The default run also
 measures the other benchmark configurations (EdgeConv C3, GMMConv C4, GAT C5 layer 1 and the C5
 training step, the small operators at C2) and appends them to the same line under "other_configs" (--no-others skips them).
+gat_c5_l2 is the output layer of the C5 model alone (256 -> 1 head x 47 classes), the second half of the training step's sparse work.
+Every timed call sits inside a marker range (roctx) named for the workload and the entry point, so that a kernel trace of this
+file can be cut per entry point.
 
 Roofline record: `achieved` is MEASURED bytes (rocprofv3 FETCH_SIZE + WRITE_SIZE of the entry point's
 kernels, kept in profiles/traffic.json) over the live HIP-event time, `frac` its share of the 8 TB/s HBM
@@ -89,6 +92,29 @@ def roofline_record(kernel, alg_bytes, ms, traffic, stale=False, note=None):
     return rec
 
 
+class marker:
+    """Named range around a phase of the benchmark (roctx through torch.cuda.nvtx; the counterpart of the reference's
+    util/indicator.py:17-20 cudaProfilerStart/Stop brackets): `rocprofv3 --marker-trace` attributes kernels to it."""
+
+    def __init__(self, name):
+        self.name = name
+
+    def __enter__(self):
+        try:
+            import torch
+            torch.cuda.nvtx.range_push(self.name)
+            self.ok = True
+        except Exception:
+            self.ok = False
+        return self
+
+    def __exit__(self, *exc):
+        if self.ok:
+            import torch
+            torch.cuda.nvtx.range_pop()
+        return False
+
+
 def peak_hbm_gib():
     """Peak device memory: torch's allocator plus what the library's schedules hold outside it."""
     import torch
@@ -103,19 +129,20 @@ def gat_alg_bytes(n, e, h, f):
     return fwd, bwd
 
 
-def time_calls(fn, steps, warmup):
+def time_calls(fn, steps, warmup, name=None):
     """Average milliseconds of fn() over `steps` calls, HIP events on torch's current stream (the
-    stream every fgnn_* launch is given)."""
+    stream every fgnn_* launch is given); the timed calls sit in a range marker called `name`."""
     import torch
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-    for a, b in ev:
-        a.record()
-        fn()
-        b.record()
-    torch.cuda.synchronize()
+    with marker(name or getattr(fn, "__name__", "timed calls")):
+        for a, b in ev:
+            a.record()
+            fn()
+            b.record()
+        torch.cuda.synchronize()
     ts = [a.elapsed_time(b) for a, b in ev]
     return sum(ts) / len(ts), min(ts), sorted(ts)[len(ts) // 2]
 
@@ -158,15 +185,10 @@ def time_device_preprocessing(g):
     return out
 
 
-def cpu_baseline_gat(g, x_feat, layer, slope, target_edges, go):
-    """The DGL-composed GAT layer (oracle.gat_layer_dgl: u_add_v, LeakyReLU, edge softmax,
-    u_mul_e + sum in plain torch) forward+backward on the host cores, on the sub-graph formed by a
-    seeded random sample of destination rows of the benchmark graph holding about `target_edges` edges
-    (all other rows empty; every source node kept); scaled to the full edge count."""
+def sample_rows_subgraph(g, target_edges):
+    """(row_ptr, col_ind, edges, rows) of the sub-graph formed by a seeded random sample of destination rows of `g` holding
+    about `target_edges` edges (all other rows empty; every source node kept), on the host."""
     import torch
-    from oracle import fgnn_oracle as orc
-    cores = os.cpu_count() or 1
-    torch.set_num_threads(cores)
     rp = g.row_ptr.cpu().long()
     deg = rp[1:] - rp[:-1]
     order = torch.randperm(g.n, generator=torch.Generator().manual_seed(12345))
@@ -179,7 +201,49 @@ def cpu_baseline_gat(g, x_feat, layer, slope, target_edges, go):
     e_s = int(rp_s[-1])
     seg = torch.repeat_interleave(torch.arange(r), deg[rows])
     pos = rp[rows][seg] + (torch.arange(e_s) - (torch.cumsum(deg[rows], 0) - deg[rows])[seg])
-    ci_s = g.col_ind.cpu()[pos]
+    return rp_s, g.col_ind.cpu()[pos], e_s, r
+
+
+def cpu_baseline_small_ops(g, h, f, target_edges):
+    """The stand-alone operators on the host cores (oracle: u_add_v, LeakyReLU, edge softmax, multi-head SpMM, forward and
+    backward by autograd) on a sampled sub-graph, scaled to the full edge count: ms for the whole chain."""
+    import torch
+    from oracle import fgnn_oracle as orc
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    rp_s, ci_s, e_s, r = sample_rows_subgraph(g, target_edges)
+    gen = torch.Generator().manual_seed(3)
+    ar = torch.randn(g.n, h, generator=gen).requires_grad_(True)
+    ac = torch.randn(g.n, h, generator=gen).requires_grad_(True)
+    x = torch.randn(g.n, h, f, generator=gen).requires_grad_(True)
+    go = torch.randn(g.n, h, f, generator=gen)
+
+    def step():
+        e = torch.nn.functional.leaky_relu(orc.u_add_v(rp_s, ci_s, ar, ac), 0.2)
+        orc.mhspmm(rp_s, ci_s, orc.edge_softmax(rp_s, e), x).backward(go)
+        ar.grad = None; ac.grad = None; x.grad = None
+    step()
+    ts, t_all = [], time.time()
+    while len(ts) < 3 or (time.time() - t_all < 6.0 and len(ts) < 10):
+        t0 = time.time()
+        step()
+        ts.append((time.time() - t0) * 1e3)
+    ms = sorted(ts)[len(ts) // 2]
+    return {"value": round(ms * g.n_edges / e_s, 1), "unit": "ms for u_add_v + LeakyReLU + edge softmax + mhspmm, forward and backward", "cores": cores,
+            "kind": "port", "sample": "oracle operators (torch CPU, %d threads) on a seeded random sample of %d destination rows = %d edges of the same "
+            "graph: median %.1f ms over %d iters, scaled by E/E_sample = %.1f" % (cores, r, e_s, ms, len(ts), g.n_edges / e_s)}
+
+
+def cpu_baseline_gat(g, x_feat, layer, slope, target_edges, go):
+    """The DGL-composed GAT layer (oracle.gat_layer_dgl: u_add_v, LeakyReLU, edge softmax,
+    u_mul_e + sum in plain torch) forward+backward on the host cores, on the sub-graph formed by a
+    seeded random sample of destination rows of the benchmark graph holding about `target_edges` edges
+    (all other rows empty; every source node kept); scaled to the full edge count."""
+    import torch
+    from oracle import fgnn_oracle as orc
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    rp_s, ci_s, e_s, r = sample_rows_subgraph(g, target_edges)
     feat = x_feat.detach().cpu()
     w_t = layer.W.detach().cpu().t().contiguous().requires_grad_(True)
     # weight mapping to GATConv_dgl: attn_l(dgl) = attn_r(ours), attn_r(dgl) = attn_l(ours)
@@ -266,9 +330,10 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
+    with marker(workload + ": layer forward + backward, timed steps"):
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
     # dominant kernels alone, through the C ABI, HIP events on the launch stream
@@ -276,13 +341,18 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
         h = torch.matmul(x, layer.W).view(-1, heads, out_feats).contiguous()
         a_row = (layer.attn_l * h).sum(-1).contiguous()
         a_col = (layer.attn_r * h).sum(-1).contiguous()
+    go_k, f_k = go, out_feats
+    if out_feats % 4:          # an output layer: the layer zero-pads its rows to a multiple of four floats (128-bit lanes); so does this
+        f_k = out_feats + (-out_feats) % 4
+        h = torch.nn.functional.pad(h, (0, f_k - out_feats)).contiguous()
+        go_k = torch.nn.functional.pad(go, (0, f_k - out_feats)).contiguous()
     fwd_out = gat_native.gat_forward(a_row, a_col, g.row_ptr, g.col_ind, slope, h)
-    ms_fwd, ms_fwd_min, _ = time_calls(lambda: gat_native.gat_forward(a_row, a_col, g.row_ptr, g.col_ind, slope, h), args.steps, 2)
+    ms_fwd, ms_fwd_min, _ = time_calls(lambda: gat_native.gat_forward(a_row, a_col, g.row_ptr, g.col_ind, slope, h), args.steps, 2, workload + ": fgnn_gat_forward")
     o = fwd_out
     ms_bwd, ms_bwd_min, _ = time_calls(
-        lambda: gat_native.gat_backward(slope, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, o[1], o[2], h, a_row, a_col, go,
-                                        out_feat=o[0], out2=o[3], cc=o[4]), args.steps, 2)
-    b_fwd, b_bwd = gat_alg_bytes(n, e, heads, out_feats)
+        lambda: gat_native.gat_backward(slope, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, o[1], o[2], h, a_row, a_col, go_k,
+                                        out_feat=o[0], out2=o[3], cc=o[4]), args.steps, 2, workload + ": fgnn_gat_backward")
+    b_fwd, b_bwd = gat_alg_bytes(n, e, heads, f_k)
     traffic, stale = measured_traffic(workload)
     peak_mem = peak_hbm_gib()
     # stash variant as the autograd function runs it: the attention [E,H] written after the forward in the entry order of
@@ -291,7 +361,7 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
     ms_sw, _, _ = time_calls(lambda: gat_native.gat_stash_own_order(slope, g.col_ptr, g.row_ind, o[1], o[2], a_row, a_col), max(3, args.steps // 4), 1)
     ms_sf = ms_fwd + ms_sw
     ms_sb, _, _ = time_calls(
-        lambda: gat_native.gat_backward(slope, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, o[1], o[2], h, a_row, a_col, go,
+        lambda: gat_native.gat_backward(slope, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, o[1], o[2], h, a_row, a_col, go_k,
                                         out_feat=o[0], out2=o[3], cc=o[4], e_soft=own, e_soft_order="own"),
         max(3, args.steps // 4), 1)
     stash_bytes = e * heads * 4
@@ -304,11 +374,11 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
         hp, arp, acp = (t.detach().clone().requires_grad_(True) for t in (h, a_row, a_col))
 
         def pipeline_step():
-            pfn(arp, acp, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, slope, hp, g.permute).backward(go)
+            pfn(arp, acp, g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, slope, hp, g.permute).backward(go_k)
             hp.grad = None; arp.grad = None; acp.grad = None
         torch.cuda.empty_cache()
         torch.cuda.reset_peak_memory_stats()
-        ms_p, _, _ = time_calls(pipeline_step, max(3, args.steps // 4), 1)
+        ms_p, _, _ = time_calls(pipeline_step, max(3, args.steps // 4), 1, workload + ": pipeline " + pname)
         pipes[pname] = (ms_p, peak_hbm_gib())
         del hp, arp, acp
     ms_pipe, pipe_peak = pipes["fusescatter"]
@@ -318,7 +388,7 @@ def run_gat(args, n, e_target, in_feats, heads, out_feats, workload):
         cpu_ms, cpu_e, cpu_rows, cores, cpu_iters = float("nan"), e, 0, 0, 0
     else:
         cpu_ms, cpu_e, cpu_rows, cores, cpu_iters = cpu_baseline_gat(g, x, layer, slope, args.cpu_sample_edges, go)
-    c1 = None if args.no_cpu_baseline else cpu_baseline_c1()
+    c1 = None if (args.no_cpu_baseline or workload != "gat_c2") else cpu_baseline_c1()
     rec = {
         "metric": "GAT layer fwd+bwd ms/iter + achieved HBM GB/s (% of peak), 1 MI355X",
         "value": round(ms_step, 4), "unit": "ms/iter", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -534,9 +604,10 @@ def run_gat_train(args):
             step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(args.steps):
-            loss = step()
-        torch.cuda.synchronize()
+        with marker("gat_c5_train: " + name + ", timed steps"):
+            for _ in range(args.steps):
+                loss = step()
+            torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) * 1e3 / args.steps
         res[name] = {"ms_per_step": round(ms, 3), "peak_hbm_GiB": round(peak_hbm_gib(), 3),
                      "of_which_schedules_GiB": round(_lib.schedule_device_bytes() / 2**30, 3),
@@ -546,6 +617,10 @@ def run_gat_train(args):
     b2 = gat_alg_bytes(n, e, 1, classes)
     alg = sum(b1) + sum(b2)
     ms = res["recompute"]["ms_per_step"]
+    # measured bytes of the step's sparse entry points: both layers, forward and backward
+    t1, stale1 = measured_traffic("gat_c5_layer1")
+    t2, stale2 = measured_traffic("gat_c5_layer2")
+    traffic = (t1["fwd"] + t1["bwd"] + t2["fwd"] + t2["bwd"]) if (t1 and t2 and all(k in t for t in (t1, t2) for k in ("fwd", "bwd"))) else None
     return {
         "metric": "2-layer GAT training step ms/step + peak HBM, recompute vs stash, 1 MI355X", "value": ms, "unit": "ms/step",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": False, "scaling": "weak",
@@ -553,7 +628,9 @@ def run_gat_train(args):
         "config": {"workload": "gat_c5_train", "nodes": n, "edges": e, "in_feats": in_dim, "hidden": "8x32", "classes": classes,
                    "optimizer": "Adam(lr=5e-3, weight_decay=5e-4)", "loss": "mean cross-entropy over all nodes (fused row pass: logsumexp - true-class logit)"},
         "variants": res,
-        "roofline": roofline_record("whole step (sparse ops of both layers; dense GEMMs, loss and Adam included in the time)", alg, ms, None),
+        "roofline": roofline_record("whole step (sparse ops of both layers; dense GEMMs, loss and Adam included in the time)", alg, ms, traffic,
+                                    stale1 or stale2, note="traffic = measured bytes of fgnn_gat_forward + fgnn_gat_backward of both layers "
+                                    "(gat_c5_layer1 + gat_c5_layer2 of profiles/traffic.json); the GEMMs, the loss and Adam add time but are not in the bytes"),
         "cpu_baseline": None,
     }
 
@@ -614,6 +691,7 @@ def run_small_ops(args):
     import torch
     from ae_mlsys_gnn_amd import _lib
     from ae_mlsys_gnn_amd.operators import csr2csc as csc_op
+    from ae_mlsys_gnn_amd.operators import fused_gat as fg
     from ae_mlsys_gnn_amd.operators import mhspmm as mh
     from ae_mlsys_gnn_amd.operators.edge_softmax import edge_softmax_native
     from ae_mlsys_gnn_amd.operators.u_add_v import u_add_v_native
@@ -631,7 +709,10 @@ def run_small_ops(args):
     eh, nh, row = 4 * e * h, 4 * n * h, 4 * h * f
     ops = (
         ("u_add_v", "fgnn_u_add_v", eh + 4 * e + 2 * nh, lambda: u_add_v_native.u_add_v_forward(g.row_ptr, g.col_ind, ar, ac)),
-        ("u_add_v_backward", "fgnn_u_add_v_backward", eh + 4 * e + 2 * nh, lambda: u_add_v_native.u_add_v_backward(g.row_ptr, g.col_ind, ee)),
+        ("u_add_v_backward", "fgnn_u_add_v_backward_planned (row sums + column sums under a plan, no atomics)", 2 * eh + 2 * nh,
+         lambda: u_add_v_native.u_add_v_backward(g.row_ptr, g.col_ind, ee)),
+        ("u_add_v_backward_atomics", "fgnn_u_add_v_backward", eh + 4 * e + 2 * nh,
+         lambda: u_add_v_native.u_add_v_backward(g.row_ptr, g.col_ind, ee, atomics=True)),
         ("edge_softmax", "fgnn_edge_softmax", 2 * eh, lambda: edge_softmax_native.edge_softmax(g.row_ptr, ee)),
         ("edge_softmax_backward", "fgnn_edge_softmax_backward", 3 * eh, lambda: edge_softmax_native.edge_softmax_backward(g.row_ptr, sm, ee)),
         ("mhspmm", "fgnn_mhspmm", e * (row + 4 + 4 * h) + n * row, lambda: mh.mhspmm(g.row_ptr, g.col_ind, sm, x)),
@@ -639,22 +720,35 @@ def run_small_ops(args):
          lambda: mh.mhspmm(g.col_ptr, g.row_ind, sm, go, pos_map=g.permute)),
         ("mhsddmm", "fgnn_mhsddmm", e * (row + 4 + 4 * h) + n * row, lambda: mh.mhsddmm(g.row_ptr, g.col_ind, go, x)),
         ("mhtranspose", "fgnn_gather_rows", 2 * eh + 4 * e, lambda: mh.mhtranspose(g.permute, sm)),
+        ("gat_scatter", "fgnn_gat_scatter", eh + 4 * e + 2 * nh, lambda: fg.gat_native.gat_scatter(ar, ac, g.row_ptr, g.col_ind, 0.2)),
+        ("gat_gather_row", "fgnn_gat_gather_row", 3 * eh, lambda: fg.gat_native.gat_gather_row(0.2, g.row_ptr, g.col_ind, ar, ac, sm, ee)),
         ("csr2csc", "fgnn_csr2csc", 0, lambda: csc_op.csr2csc(g.row_ptr, g.col_ind)),
     )
     out = {}
+    traffic, stale = measured_traffic("small_ops_c2")
+    traffic = traffic or {}
     for name, entry, nbytes, fn in ops:
-        ms, _, _ = time_calls(fn, min(args.steps, 10), 2)
+        ms, _, _ = time_calls(fn, min(args.steps, 10), 2, "small_ops_c2: " + name)
         out[name] = {"entry_point": entry, "ms": round(ms, 3)}
+        if name in traffic:          # L2<->fabric bytes by the byte counters: above `bytes` where rows are fetched as whole 128-byte lines or read twice
+            out[name].update({"traffic": traffic[name], "traffic_GBps": round(traffic[name] / ms / 1e6, 1),
+                              "traffic_frac_of_hbm_peak": round(traffic[name] / ms / 1e6 / HBM_PEAK_GBPS, 4)})
+            if stale:
+                out[name]["traffic_stale"] = True
         if nbytes and name.startswith("mh") and name != "mhtranspose":
             # feature rows gathered once per entry by the model, mostly served by the L2s: a rate, not a share of the HBM peak
             out[name].update({"no_reuse_model_bytes": nbytes, "effective_gather_GBps": round(nbytes / ms / 1e6, 1)})
         elif nbytes:
             out[name].update({"bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)})
     total = sum(v["ms"] for v in out.values())
+    cpu = None if args.no_cpu_baseline else cpu_baseline_small_ops(g, h, f, args.cpu_sample_edges)
+    if cpu:
+        cpu["gpu_ms_same_chain"] = round(sum(out[k]["ms"] for k in ("u_add_v", "u_add_v_backward", "edge_softmax", "edge_softmax_backward", "mhspmm",
+                                                                    "mhspmm_transposed", "mhsddmm")), 3)
     return {"metric": "small per-edge operators on the C2 graph, ms per call, 1 MI355X", "value": round(total, 3), "unit": "ms (sum over the operators)",
             "n_gpus": 1, "steps": min(args.steps, 10), "warmup": 2, "ms_per_step": round(total, 3), "higher_is_better": False, "scaling": "weak",
             "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-            "config": {"workload": "small_ops_c2", "nodes": n, "edges": e, "heads": h, "out_feats": f}, "operators": out, "cpu_baseline": None}
+            "config": {"workload": "small_ops_c2", "nodes": n, "edges": e, "heads": h, "out_feats": f}, "operators": out, "cpu_baseline": cpu}
 
 
 def brief(rec):
@@ -669,12 +763,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="gat_c2", choices=["gat_c2", "gat_c5", "gat_c5_train", "edgeconv_c3", "gmm_c4", "small_ops_c2", "gather_ceiling"])
+    ap.add_argument("--workload", default="gat_c2", choices=["gat_c2", "gat_c5", "gat_c5_l2", "gat_c5_train", "edgeconv_c3", "gmm_c4", "small_ops_c2", "gather_ceiling"])
     ap.add_argument("--no-others", action="store_true", help="gat_c2 only: do not append the other benchmark configurations to the line")
     ap.add_argument("--cpu-sample-edges", type=int, default=1_500_000)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline (profiling runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run a 1 GiB device copy (reads 1 GiB, writes 1 GiB) so that profiler byte counters can be scaled")
+                    help="also run a 1 GiB elementwise pass (torch.neg: reads 1 GiB, writes 1 GiB) so that profiler byte counters can be scaled")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures ONE GPU: the fused sparse-operator path is single-GPU (as is the reference); "
@@ -688,7 +782,7 @@ def main():
         a = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").normal_()
         b = torch.empty_like(a)
         for _ in range(3):
-            b.copy_(a)
+            torch.neg(a, out=b)          # a kernel of its own name in the counter table (a plain copy_ shares hipMemcpy's)
         torch.cuda.synchronize()
         del a, b
     if args.workload == "gat_c2":
@@ -700,9 +794,11 @@ def main():
             others = {}
             sub = argparse.Namespace(**vars(args))
             sub.steps, sub.warmup, sub.no_cpu_baseline = min(args.steps, 10), min(args.warmup, 3), True
+            sub_cpu = argparse.Namespace(**vars(sub))          # a shorter host sample than the headline's: a few seconds
+            sub_cpu.no_cpu_baseline, sub_cpu.cpu_sample_edges = args.no_cpu_baseline, min(args.cpu_sample_edges, 300_000)
             for name, fn in (("edgeconv_c3", lambda: run_edgeconv(args)), ("gmm_c4", lambda: run_gmm(args)),
-                             ("gat_c5_layer1", lambda: run_gat(sub, 2449029, 61_900_000, 100, 8, 32, "gat_c5_layer1")),
-                             ("gat_c5_train", lambda: run_gat_train(sub)), ("small_ops_c2", lambda: run_small_ops(sub))):
+                             ("gat_c5_layer1", lambda: run_gat(sub_cpu, 2449029, 61_900_000, 100, 8, 32, "gat_c5_layer1")),
+                             ("gat_c5_train", lambda: run_gat_train(sub)), ("small_ops_c2", lambda: run_small_ops(sub_cpu))):
                 gc.collect()
                 _lib.clear_schedule_cache()
                 torch.cuda.empty_cache()
@@ -720,6 +816,8 @@ def main():
         rec = run_small_ops(args)
     elif args.workload == "gat_c5":
         rec = run_gat(args, 2449029, 61_900_000, 100, 8, 32, "gat_c5_layer1")
+    elif args.workload == "gat_c5_l2":          # the output layer of the C5 model alone: 256 -> 1 head x 47 classes (zero-padded to 48)
+        rec = run_gat(args, 2449029, 61_900_000, 256, 1, 47, "gat_c5_layer2")
     elif args.workload == "gat_c5_train":
         rec = run_gat_train(args)
     elif args.workload == "edgeconv_c3":

@@ -1120,13 +1120,16 @@ def test_gather_rows_widths(w):
         assert torch.equal(out.cpu(), xin.cpu()[perm.long()])
 
 
+@pytest.mark.parametrize("n_short", [0, 6000])
 @pytest.mark.parametrize("nh", [1, 4, 8, 20])
-def test_edge_softmax_rows_beyond_the_register_cache(nh):
+def test_edge_softmax_rows_beyond_the_register_cache(nh, n_short):
     """Rows longer than what a workgroup keeps in registers (the part beyond is folded into a running maximum and sum while
     it streams by): a 40 k-entry row whose values ascend, so the running maximum moves on every trip, one whose values
-    descend, a constant one, next to short rows; forward and backward against float64."""
+    descend, a constant one, next to short rows; forward and backward against float64.  With n_short rows of two entries
+    appended the mean row is short and the launch takes its small-footprint configuration (fewer values cached, more
+    streamed) for the same long rows."""
     from ae_mlsys_gnn_amd.operators import edge_softmax as op
-    lens = [40000, 3, 0, 40000, 9000, 1, 40000]
+    lens = [40000, 3, 0, 40000, 9000, 1, 40000] + [2] * n_short
     g = custom_graph([[0] * d for d in lens], len(lens))
     e = g.n_edges
     gen = torch.Generator().manual_seed(nh)
@@ -1150,6 +1153,7 @@ def test_edge_softmax_rows_beyond_the_register_cache(nh):
     assert_close_sum(hd.grad, hl.grad, ref.detach() * (go.abs() + dot_abs[dst]), "edge_softmax grad of long rows", c=c)
     sums = orc.segment_sums(g.row_ptr, out.detach().cpu().double())
     assert float((sums - (torch.tensor(lens) > 0).double().view(-1, 1)).abs().max()) < 1e-5
+    assert (e * nh >= 1024 * len(lens)) == (n_short == 0)          # the two configurations' side of the mean-row-length rule
 
 
 @pytest.mark.parametrize("h,f", [(8, 256), (3, 501), (5, 300)])

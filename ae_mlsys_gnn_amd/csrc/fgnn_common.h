@@ -42,6 +42,7 @@ static inline bool fgnn_aligned16(const void *p) { return (((uintptr_t)p) & 15u)
 static inline size_t fgnn_align256(size_t x) { return (x + 255) & ~(size_t)255; }
 // Fills n floats with v on `st` (a kernel, so it may be captured into a HIP graph).
 int fgnn_fill_f32(float *p, size_t n, float v, hipStream_t st);
+int fgnn_current_device_has_xcd_mapping();      // 1: workgroup w of a dispatch runs on XCD w % FGNN_NUM_XCD on the current device
 
 // Stable LSD radix sort of (key, payload) pairs and an inclusive int32 scan (fgnn_csr2csc.hip); device pointers.
 size_t fgnn_rs_sort_workspace(int64_t n);

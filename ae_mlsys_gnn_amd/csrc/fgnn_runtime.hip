@@ -524,7 +524,7 @@ extern "C" int fgnn_xcd_mapping_for(const char *gcn_arch, int compute_units)
 }
 
 // 1: the current device has the workgroup-to-XCD mapping the bucketed lists assume; 0: it has not (or cannot be asked)
-static int current_device_has_xcd_mapping()
+int fgnn_current_device_has_xcd_mapping()
 {
     static std::mutex mu;
     static int known[64];          // per device: 0 = not asked yet, 1 = no, 2 = yes
@@ -546,7 +546,7 @@ extern "C" int fgnn_schedule_create_bucketed(const int32_t *ptr_dev, const int32
     // on a device without the assumed workgroup-to-XCD mapping the plain list is built instead (fgnn_schedule_num_buckets
     // of the result is then 0); FGNN_XCD_MAPPING=0 / 1 in the environment overrides the check
     const char *force = getenv("FGNN_XCD_MAPPING");
-    if (force ? (strcmp(force, "0") == 0) : !current_device_has_xcd_mapping())
+    if (force ? (strcmp(force, "0") == 0) : !fgnn_current_device_has_xcd_mapping())
         return fgnn_schedule_create(ptr_dev, n_rows, seg_len, stream, out);
     if (seg_len <= 0) seg_len = 2048;
     seg_len = (seg_len + 63) & ~63;

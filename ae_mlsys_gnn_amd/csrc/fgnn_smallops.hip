@@ -243,13 +243,17 @@ extern "C" int fgnn_sddmm_coo(int64_t E, int n_rows, int n_cols, int H, int F, c
 // and 16-byte aligned arrays, 128-bit lanes); a wave takes RW consecutive output rows = at most 64 * GR_U groups, lane j of
 // a trip owns group j of that span.  Its row inside the span is j / G by a multiply and a shift (inv = ceil(2^20 / G), exact
 // for j * G < 2^20; spans of one row pass inv = 0), so there is no division per element, and the GR_U loads of a lane are
-// all issued before the first store.
+// all issued before the first store.  With per_xcd > 0 the workgroups of one XCD (blockIdx.x % FGNN_NUM_XCD) take one contiguous
+// eighth of the output between them, in launch order: a 128-byte line of `in` holds several short rows, and when permute
+// is the map of a transposition, rows that are neighbours in `in` are wanted by nearby outputs (the neighbouring columns of
+// one matrix row) - close in time on ONE XCD's L2 instead of spread round-robin over eight that share nothing.
 #define GR_U 8
 template <int VEC>
-__global__ __launch_bounds__(FGNN_TPB) void gather_rows_kernel(int64_t E, int G, int RW, unsigned inv, const int *__restrict__ permute,
+__global__ __launch_bounds__(FGNN_TPB) void gather_rows_kernel(int64_t E, int G, int RW, unsigned inv, unsigned per_xcd, const int *__restrict__ permute,
                                                                const float *__restrict__ in, float *__restrict__ out)
 {
-    const int64_t q0 = ((int64_t)blockIdx.x * FGNN_WPB + fg_wave()) * RW;
+    const unsigned chunk = per_xcd ? (blockIdx.x % FGNN_NUM_XCD) * per_xcd + blockIdx.x / FGNN_NUM_XCD : blockIdx.x;
+    const int64_t q0 = ((int64_t)chunk * FGNN_WPB + fg_wave()) * RW;
     if (q0 >= E) return;
     const int rows = (int)min((int64_t)RW, E - q0);
     const int64_t n = (int64_t)rows * G;                 // groups of this wave: <= 64 * GR_U unless RW == 1
@@ -292,11 +296,15 @@ extern "C" int fgnn_gather_rows(int64_t E, int W, const int32_t *permute, const 
     const unsigned inv = RW > 1 ? (unsigned)(((1u << 20) + (unsigned)G - 1u) / (unsigned)G) : 0u;
     const int64_t waves = (E + RW - 1) / RW;
     const int64_t blocks = (waves + FGNN_WPB - 1) / FGNN_WPB;
-    FGNN_REQUIRE(blocks <= 2147483647LL, FGNN_ERR_LIMIT, "fgnn_gather_rows: too many rows");
+    FGNN_REQUIRE(blocks <= 2147483647LL - FGNN_NUM_XCD, FGNN_ERR_LIMIT, "fgnn_gather_rows: too many rows");
+    // rows shorter than a cache line, enough workgroups to matter, and a device whose workgroups go round the XCDs in turn
+    const unsigned per_xcd = (G * (vec4 ? 16 : 4) < 128 && blocks >= 64 * FGNN_NUM_XCD && fgnn_current_device_has_xcd_mapping())
+                                 ? (unsigned)((blocks + FGNN_NUM_XCD - 1) / FGNN_NUM_XCD) : 0u;
+    const unsigned grid = per_xcd ? per_xcd * FGNN_NUM_XCD : (unsigned)blocks;
     if (vec4)
-        hipLaunchKernelGGL(gather_rows_kernel<4>, dim3((unsigned)blocks), dim3(FGNN_TPB), 0, (hipStream_t)stream, E, G, RW, inv, permute, in, out);
+        hipLaunchKernelGGL(gather_rows_kernel<4>, dim3(grid), dim3(FGNN_TPB), 0, (hipStream_t)stream, E, G, RW, inv, per_xcd, permute, in, out);
     else
-        hipLaunchKernelGGL(gather_rows_kernel<1>, dim3((unsigned)blocks), dim3(FGNN_TPB), 0, (hipStream_t)stream, E, G, RW, inv, permute, in, out);
+        hipLaunchKernelGGL(gather_rows_kernel<1>, dim3(grid), dim3(FGNN_TPB), 0, (hipStream_t)stream, E, G, RW, inv, per_xcd, permute, in, out);
     return fgnn_launch_status("gather_rows_kernel");
 }
 

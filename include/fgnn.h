@@ -335,10 +335,11 @@ int    fgnn_gaussian_backward(int64_t E, int K, int dim, const float *pseudo, co
  * mhspmm.mhspmm (src/spmm/mhspmm.cc; mhspmm.cu:44-66): out[i,h,:] = sum_p att[p,h]*feat[idx[p],h,:];
  * att row used is att[pos_map[p]] when pos_map is non-NULL.  With H == 1 and att == NULL it is
  * the unweighted single-head SpMM of operators/spmm.py:38-41.
- * Workspace: the partial results of split rows and, for an XCD-aware schedule, E*H floats more into which the weights
- * are first copied in the list's entry order (the gather pass then streams them).  With att == NULL, or with a
- * workspace that only holds the partials (fgnn_gmm_forward_workspace_bytes of the same shape), the weights are read
- * in place. */
+ * Workspace: the partial results of split rows and, for an XCD-aware schedule with a head count that is neither a
+ * multiple of four nor below three, E*H floats more into which the weights are first copied in the list's entry order
+ * (the gather pass then streams them; with H % 4 == 0 it reads them in place as 128-bit words).  With att == NULL, or
+ * with a workspace that only holds the partials (fgnn_gmm_forward_workspace_bytes of the same shape), the weights are
+ * always read in place. */
 size_t fgnn_mhspmm_workspace_bytes(const fgnn_schedule_t *sched, int H, int F);
 int    fgnn_mhspmm(int N, int64_t E, int H, int F, const int32_t *ptr, const int32_t *idx,
                    const int32_t *pos_map, const float *att, const float *feat, float *out,

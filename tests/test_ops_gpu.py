@@ -702,19 +702,29 @@ def test_mhspmm_and_gmm_with_xcd_buckets(monkeypatch):
     assert_close_sum(out, ref.detach(), s_out, "mhspmm (buckets)")
     assert_close_sum(fd.grad, fl.grad, s_feat, "mhspmm grad feat (buckets)")
     assert_close_sum(ad.grad, al.grad, s_att, "mhspmm grad att (buckets)")
-    # the wrapper's workspace has room for the weights in the work list's entry order (copied there first, then streamed);
-    # with a workspace that only holds the partial results the same call reads them in place: same terms in the same order
+    # head counts that are multiples of four read the weights in place as 128-bit words; for others above two the wrapper's
+    # workspace has room for the weights in the work list's entry order (copied there first, then streamed), and with a
+    # workspace that only holds the partial results the same call reads them in place: same terms in the same order
     sch = _lib.schedule_for(gd.row_ptr, idx_tensor=gd.col_ind)
-    assert sch.handle is not None and _lib.lib().fgnn_mhspmm_workspace_bytes(sch.handle, 4, 16) > _lib.lib().fgnn_gmm_forward_workspace_bytes(sch.handle, 4, 16)
-    for pm in (None, gd.permute):
-        ptr_arr, idx = (gd.row_ptr, gd.col_ind) if pm is None else (gd.col_ptr, gd.row_ind)
-        sc = _lib.schedule_for(ptr_arr, idx_tensor=idx)
-        copied = op.mhspmm(ptr_arr, idx, ad.detach(), fd.detach(), pos_map=pm)
-        in_place = torch.empty_like(copied)
-        ws, wsb = _lib.workspace(_lib.lib().fgnn_gmm_forward_workspace_bytes(sc.handle, 4, 16), DEV)
-        _lib.check(_lib.lib().fgnn_mhspmm(g.n, g.n_edges, 4, 16, _lib.ptr(ptr_arr), _lib.ptr(idx), _lib.ptr(pm), _lib.ptr(ad.detach()),
-                                           _lib.ptr(fd.detach()), _lib.ptr(in_place), sc.handle, _lib.ptr(ws), wsb, _lib.stream_ptr()), "fgnn_mhspmm")
-        assert torch.equal(copied, in_place)
+    assert sch.handle is not None
+    assert _lib.lib().fgnn_mhspmm_workspace_bytes(sch.handle, 4, 16) == _lib.lib().fgnn_gmm_forward_workspace_bytes(sch.handle, 4, 16)
+    assert _lib.lib().fgnn_mhspmm_workspace_bytes(sch.handle, 6, 16) > _lib.lib().fgnn_gmm_forward_workspace_bytes(sch.handle, 6, 16)
+    for hh in (4, 6):
+        a_h = torch.randn(g.n_edges, hh, generator=gen).to(DEV)
+        x_h = torch.randn(g.n, hh, 16, generator=gen).to(DEV)
+        want = orc.mhspmm(g.row_ptr, g.col_ind, a_h.cpu().double(), x_h.cpu().double())
+        for pm in (None, gd.permute):
+            ptr_arr, idx = (gd.row_ptr, gd.col_ind) if pm is None else (gd.col_ptr, gd.row_ind)
+            sc = _lib.schedule_for(ptr_arr, idx_tensor=idx)
+            copied = op.mhspmm(ptr_arr, idx, a_h, x_h, pos_map=pm)
+            in_place = torch.empty_like(copied)
+            ws, wsb = _lib.workspace(_lib.lib().fgnn_gmm_forward_workspace_bytes(sc.handle, hh, 16), DEV)
+            _lib.check(_lib.lib().fgnn_mhspmm(g.n, g.n_edges, hh, 16, _lib.ptr(ptr_arr), _lib.ptr(idx), _lib.ptr(pm), _lib.ptr(a_h),
+                                               _lib.ptr(x_h), _lib.ptr(in_place), sc.handle, _lib.ptr(ws), wsb, _lib.stream_ptr()), "fgnn_mhspmm")
+            assert torch.equal(copied, in_place)
+            if pm is None:
+                assert_close_sum(copied, want, orc.mhspmm(g.row_ptr, g.col_ind, a_h.cpu().double().abs(), x_h.cpu().double().abs()),
+                                 "mhspmm with %d heads under an XCD-aware list" % hh)
     # the SDDMM under the work list against the list-free kernel: the same dot product per entry, stored at the same place
     sd = op.mhsddmm(gd.row_ptr, gd.col_ind, go.float().to(DEV), fd.detach())
     plain = torch.empty_like(sd)

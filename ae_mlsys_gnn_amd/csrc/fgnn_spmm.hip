@@ -150,6 +150,78 @@ __global__ __launch_bounds__(FGNN_TPB) void spmm_kernel(SpmmP p, WF wf, int shar
     }
 }
 
+// The same gather with STORED per-edge weights handled in a pair layout (that of the fused GAT forward): lane
+// (u << hp_shift) | h owns (entry u of a batch of U, head h) and alone loads that weight, one 32-bit load per lane and batch
+// issued a batch ahead of its use; the feature lanes take the weight of (their entry, their head) with ds_bpermute.  No
+// staging of a chunk's weights in LDS and none of its two wave-wide waits per 64 entries.  Needs U << hp_shift <= 64 lanes and
+// no sum over heads in the store.
+template <int VEC, int R, bool FULL>
+__global__ __launch_bounds__(FGNN_TPB) void spmm_pair_kernel(SpmmP p, const float *__restrict__ att, int att_ld, int hp_shift)
+{
+    int row, b, e, slot;
+    if (!fg_get_item(p.items, p.n_items, p.ptr, row, b, e, slot)) return;
+    const int lane = fg_lane();
+    fg_lanemap<VEC, R> lm;
+    lm.init(lane, p.HF, p.F);
+    fg_vec<VEC> T[R];
+    uint32_t boff[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) { T[r].zero(); boff[r] = (uint32_t)((FULL || lm.ok[r]) ? lm.eoff[r] : 0) * 4u; }
+    constexpr int U = (R >= 8) ? 1 : 8 / R;          // feature rows in flight per wave
+    const int pu = lane >> hp_shift, ph = lane & ((1 << hp_shift) - 1);
+    const bool pok = ph < p.H && pu < U;
+    const uint32_t row_bytes = (uint32_t)p.ld * 4u;
+    for (int c = b; c < e; c += 64) {
+        const int q = c + lane, cnt = min(64, e - c), qq = q < e ? q : c;      // lanes past the end repeat a valid entry
+        const int idv = p.idx[qq];
+        const int orig = p.pos ? p.pos[qq] : qq;
+        const int posv = p.pos_map ? p.pos_map[orig] : orig;
+        // weight of the lane's pair in the batch that starts at entry t (0 for a slot without an entry); the lane
+        // exchange stays outside divergent code
+        auto fetch = [&](int t) {
+            const int pp = __builtin_amdgcn_ds_bpermute(((t + pu) & 63) << 2, posv);
+            float a = 0.f;
+            if (pok && t + pu < cnt) a = att[(size_t)(unsigned)pp * att_ld + ph];
+            return a;
+        };
+        float av = fetch(0);
+        for (int t = 0; t < cnt; t += U) {
+            float an = 0.f;
+            if (t + U < cnt) an = fetch(t + U);                                  // wave-uniform
+            fg_vec<VEC> ld[U][R];
+            uint32_t bo[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) bo[r] = fg_pin(boff[r]);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint64_t j = (uint64_t)(uint32_t)__builtin_amdgcn_readlane(idv, (t + u) & 63);      // past the chunk: a valid row, weight 0
+                const fg_gptr base = fg_uniform_ptr((const char *)p.feat + j * row_bytes);
+#pragma unroll
+                for (int r = 0; r < R; ++r) ld[u][r].load_off(base, bo[r]);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const float a = __int_as_float(__builtin_amdgcn_ds_bpermute(((u << hp_shift) + lm.hd[r]) << 2, __float_as_int(av)));
+                    T[r].fma(a, ld[u][r]);
+                }
+            }
+            av = an;
+        }
+    }
+    if (slot < 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            if (FULL || lm.ok[r]) T[r].store_nt(p.out + (size_t)row * p.ldo + lm.eoff[r]);
+    } else {
+        float *dst = p.part + (size_t)slot * spmm_pw(p.HF);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            if (FULL || lm.ok[r]) T[r].store_nt(dst + lm.eoff[r]);
+    }
+}
+
 // Rows narrower than a wave take the packed lane layout (fg_packmap): G entries of the row per load
 // instruction, one partial sum per lane group, a butterfly over the groups at the end.
 template <int G, class WF>
@@ -245,9 +317,10 @@ static int spmm_checks(const char *fn, int N, int64_t E, int H, int F, const fgn
     return 0;
 }
 
+// pair_att != NULL: stored weights [*, pair_ld] that the pair-layout kernel reads itself where its lane budget allows
 template <class WF>
 static int spmm_launch(const char *name, SpmmP p, WF wf, int shared_floats, const fgnn_schedule_t *sched, bool aligned,
-                       void *workspace, size_t workspace_bytes, hipStream_t st)
+                       void *workspace, size_t workspace_bytes, hipStream_t st, const float *pair_att = nullptr, int pair_ld = 0)
 {
     fgnn_rowcfg cfg;
     FGNN_REQUIRE(fgnn_pick_rowcfg(p.HF, p.F, aligned && fgnn_aligned16(workspace), &cfg), FGNN_ERR_LIMIT, "%s: unsupported row width %d", name, p.HF);
@@ -272,7 +345,15 @@ static int spmm_launch(const char *name, SpmmP p, WF wf, int shared_floats, cons
         if (pack == 8) hipLaunchKernelGGL((spmm_packed_kernel<8, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
         else if (pack == 4) hipLaunchKernelGGL((spmm_packed_kernel<4, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
         else if (pack == 2) hipLaunchKernelGGL((spmm_packed_kernel<2, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
-        else hipLaunchKernelGGL((spmm_kernel<VEC, R, FULL, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
+        else {
+            constexpr int U = (R >= 8) ? 1 : 8 / R;
+            int hp_shift = 0;
+            while ((1 << hp_shift) < p.H) ++hp_shift;
+            if (pair_att && !p.sum_h && (U << hp_shift) <= 64)
+                hipLaunchKernelGGL((spmm_pair_kernel<VEC, R, FULL>), dim3(grid), dim3(FGNN_TPB), 0, st, p, pair_att, pair_ld, hp_shift);
+            else
+                hipLaunchKernelGGL((spmm_kernel<VEC, R, FULL, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
+        }
         int rc = fgnn_launch_status(name);
         if (rc) return rc;
         if (sched && sched->n_split > 0) {
@@ -367,7 +448,7 @@ extern "C" int fgnn_mhspmm(int N, int64_t E, int H, int F, const int32_t *ptr, c
         p.N = N; p.H = hg; p.F = F; p.HF = hg * F; p.ld = p.ldo = H * F; p.own_order = own_order;
         WAtt wf{att_use ? att_use + h0 : nullptr, H, att_use && H % 4 == 0 && hg % 4 == 0 && h0 % 4 == 0 && fgnn_aligned16(att_use)};
         rc = spmm_launch("fgnn_mhspmm", p, wf, 0, sched, fgnn_aligned16(feat) && fgnn_aligned16(out) && (hmax == H || F % 4 == 0), workspace,
-                         workspace_bytes, st);
+                         workspace_bytes, st, wf.att, H);
         if (rc) return rc;
     }
     return 0;

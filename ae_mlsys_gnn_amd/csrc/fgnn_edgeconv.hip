@@ -12,13 +12,17 @@
 #include <mutex>
 #include "fgnn_common.h"
 
+// per_xcd > 0: the workgroups of one XCD (blockIdx.x % FGNN_NUM_XCD) take one contiguous eighth of the nodes.  The neighbours of
+// a node of a batched kNN graph lie in its own cloud; with the workgroups dealt round-robin every XCD gathered from every
+// cloud and the feature matrix crossed the fabric eight times (106 MB fetched for 32 clouds of 1024 points x 64 floats).
 template <int VEC>
-__global__ __launch_bounds__(256) void edgeconv_fwd_kernel(int N, int F, int k, const int *__restrict__ src_ind,
+__global__ __launch_bounds__(256) void edgeconv_fwd_kernel(int N, int F, int k, unsigned per_xcd, const int *__restrict__ src_ind,
                                                            const float *__restrict__ h_src, const float *__restrict__ h_dst,
                                                            float out_slope, float *__restrict__ out, int *__restrict__ argmax)
 {
     const int per = F / VEC;
-    const long long tid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const unsigned chunk = per_xcd ? (blockIdx.x % FGNN_NUM_XCD) * per_xcd + blockIdx.x / FGNN_NUM_XCD : blockIdx.x;
+    const long long tid = (long long)chunk * blockDim.x + threadIdx.x;
     if (tid >= (long long)N * per) return;
     const int node = (int)(tid / per);
     const int fo = (int)(tid - (long long)node * per) * VEC;
@@ -112,8 +116,13 @@ static int edgeconv_forward_run(const char *fn, int N, int n_src, int F, int k, 
     bool v4 = (F % 4 == 0) && fgnn_aligned16(h_src) && fgnn_aligned16(h_dst);
     long long threads = (long long)N * (v4 ? F / 4 : F);
     unsigned grid = (unsigned)((threads + 255) / 256);
-    if (v4) hipLaunchKernelGGL(edgeconv_fwd_kernel<4>, dim3(grid), dim3(256), 0, st, N, F, k, src_ind, h_src, h_dst, out_slope, out, argmax);
-    else hipLaunchKernelGGL(edgeconv_fwd_kernel<1>, dim3(grid), dim3(256), 0, st, N, F, k, src_ind, h_src, h_dst, out_slope, out, argmax);
+    unsigned per_xcd = 0;
+    if (grid >= 8 * FGNN_NUM_XCD && fgnn_current_device_has_xcd_mapping()) {
+        per_xcd = (grid + FGNN_NUM_XCD - 1) / FGNN_NUM_XCD;
+        grid = per_xcd * FGNN_NUM_XCD;
+    }
+    if (v4) hipLaunchKernelGGL(edgeconv_fwd_kernel<4>, dim3(grid), dim3(256), 0, st, N, F, k, per_xcd, src_ind, h_src, h_dst, out_slope, out, argmax);
+    else hipLaunchKernelGGL(edgeconv_fwd_kernel<1>, dim3(grid), dim3(256), 0, st, N, F, k, per_xcd, src_ind, h_src, h_dst, out_slope, out, argmax);
     return fgnn_launch_status("edgeconv_fwd_kernel");
 }
 
@@ -164,14 +173,24 @@ extern "C" int fgnn_edgeconv_backward(int N, int n_src, int F, const int32_t *ar
 #define EC_OVF_HEADER 64        // ints in front of the overflow list (counter + padding)
 
 #define EC_BT 1024      // threads per workgroup of the blocked backward
+// n_tiles > 0: a one-dimensional grid in which the n_tiles column tiles of a block all run on one XCD (workgroup w runs on XCD
+// w % FGNN_NUM_XCD): a tile row is FS * 4 = 32 bytes of a 128-byte line of grad_out and argmax, and with the tiles of a block
+// spread over the XCDs every line crossed the fabric once per XCD that held one of its four tiles (67 MB fetched for 16.8 MB).
 template <int FS>
-__global__ __launch_bounds__(EC_BT) void edgeconv_bwd_blocked_kernel(int N, int F, int block, const int *__restrict__ argmax,
+__global__ __launch_bounds__(EC_BT) void edgeconv_bwd_blocked_kernel(int N, int F, int block, int n_tiles, const int *__restrict__ argmax,
                                                                      const float *__restrict__ grad_out, const float *__restrict__ act_out,
                                                                      float act_slope, float *__restrict__ grad_src, float *__restrict__ grad_dst,
                                                                      int *__restrict__ ovf)
 {
     extern __shared__ float tile[];                 // [rows of the block][FS]
-    const int b = (int)blockIdx.y, f0 = (int)blockIdx.x * FS;
+    int b = (int)blockIdx.y, tx = (int)blockIdx.x;
+    if (n_tiles > 0) {
+        const unsigned j = blockIdx.x / FGNN_NUM_XCD;
+        b = (int)((j / (unsigned)n_tiles) * FGNN_NUM_XCD + blockIdx.x % FGNN_NUM_XCD);
+        tx = (int)(j % (unsigned)n_tiles);
+        if ((long long)b * block >= N) return;          // the last round of blocks may be incomplete (uniform over the workgroup)
+    }
+    const int f0 = tx * FS;
     const int r0 = b * block, rows = min(block, N - r0), fs = min(FS, F - f0);
     const int total = rows * FS;
     for (int i = (int)threadIdx.x; i < total; i += EC_BT) tile[i] = 0.f;
@@ -237,11 +256,17 @@ static int edgeconv_backward_blocked_run(int N, int F, int block, int fs, const 
 {
     int rc = fgnn_fill_f32((float *)ovf, 1, 0.f, st);        // the counter (bit pattern of 0.0f is integer 0); a kernel, so capturable
     if (rc) return rc;
-    dim3 grid((unsigned)((F + fs - 1) / fs), (unsigned)((N + block - 1) / block));
-    FGNN_REQUIRE(grid.y <= 65535, FGNN_ERR_LIMIT, "fgnn_edgeconv_backward_blocked: more than 65535 blocks");
+    const long long n_tiles = (F + fs - 1) / fs, n_blocks = ((long long)N + block - 1) / block;
+    dim3 grid((unsigned)n_tiles, (unsigned)n_blocks);
+    FGNN_REQUIRE(n_blocks <= 65535, FGNN_ERR_LIMIT, "fgnn_edgeconv_backward_blocked: more than 65535 blocks");
+    int tiles_arg = 0;
+    if (n_tiles > 1 && fgnn_current_device_has_xcd_mapping()) {          // all column tiles of a block on one XCD
+        grid = dim3((unsigned)(((n_blocks + FGNN_NUM_XCD - 1) / FGNN_NUM_XCD) * FGNN_NUM_XCD * n_tiles));
+        tiles_arg = (int)n_tiles;
+    }
     const size_t shm = (size_t)block * fs * sizeof(float);
-    if (fs == 8) hipLaunchKernelGGL(edgeconv_bwd_blocked_kernel<8>, grid, dim3(EC_BT), shm, st, N, F, block, argmax, grad_out, act_out, act_slope, grad_src, grad_dst, ovf);
-    else hipLaunchKernelGGL(edgeconv_bwd_blocked_kernel<4>, grid, dim3(EC_BT), shm, st, N, F, block, argmax, grad_out, act_out, act_slope, grad_src, grad_dst, ovf);
+    if (fs == 8) hipLaunchKernelGGL(edgeconv_bwd_blocked_kernel<8>, grid, dim3(EC_BT), shm, st, N, F, block, tiles_arg, argmax, grad_out, act_out, act_slope, grad_src, grad_dst, ovf);
+    else hipLaunchKernelGGL(edgeconv_bwd_blocked_kernel<4>, grid, dim3(EC_BT), shm, st, N, F, block, tiles_arg, argmax, grad_out, act_out, act_slope, grad_src, grad_dst, ovf);
     rc = fgnn_launch_status("edgeconv_bwd_blocked_kernel");
     if (rc) return rc;
     hipLaunchKernelGGL(edgeconv_bwd_overflow_kernel, dim3(64), dim3(256), 0, st, F, argmax, grad_out, act_out, act_slope, grad_src, ovf);

@@ -46,16 +46,20 @@ __device__ __forceinline__ void sddmm_row_piece(int row, int pb, int pe, int H, 
             const int pv = pos ? pos[qq] : qq;
             for (int t = 0; t < cnt; t += EB) {
                 float keep = 0.f;
-                fg_vec<VEC> lb[EB];                                   // all rows of the batch in flight
+                constexpr int UL = EB < 4 ? EB : 4;                   // gathered rows in flight (eight: same time, 12 % more L2 misses)
 #pragma unroll
-                for (int u = 0; u < EB; ++u) {
-                    const int j = __builtin_amdgcn_readlane(id, (t + u) & 63);      // past the chunk: a valid row, result not stored
-                    if (FULL || lm.ok[0]) lb[u].load(b + (size_t)j * ld + lm.eoff[0]); else lb[u].zero();
-                }
+                for (int t4 = 0; t4 < EB; t4 += UL) {
+                    fg_vec<VEC> lb[UL];
 #pragma unroll
-                for (int u = 0; u < EB; ++u) {
-                    const float sum = fg_group_sum<LPH>(lb[u].dot(ar[0]));
-                    keep = sub == u ? sum : keep;
+                    for (int u = 0; u < UL; ++u) {
+                        const int j = __builtin_amdgcn_readlane(id, (t + t4 + u) & 63);      // past the chunk: a valid row, result not stored
+                        if (FULL || lm.ok[0]) lb[u].load(b + (size_t)j * ld + lm.eoff[0]); else lb[u].zero();
+                    }
+#pragma unroll
+                    for (int u = 0; u < UL; ++u) {
+                        const float sum = fg_group_sum<LPH>(lb[u].dot(ar[0]));
+                        keep = sub == t4 + u ? sum : keep;
+                    }
                 }
                 const float v = __int_as_float(__builtin_amdgcn_ds_bpermute(osrc, __float_as_int(keep)));
                 const int po = __builtin_amdgcn_ds_bpermute(((t + ou) & 63) << 2, pv);

@@ -613,6 +613,23 @@ def run_gat_train(args):
                      "of_which_schedules_GiB": round(_lib.schedule_device_bytes() / 2**30, 3),
                      "resident_before_GiB": round(base / 2**30, 3), "final_loss": round(float(loss.detach()), 5)}
         del model, opt
+        if name == "recompute":
+            # the same step captured once into a HIP graph and replayed (same number of optimizer steps from the same start):
+            # what the launch gaps between the step's ~100 kernels are worth at this size
+            from ae_mlsys_gnn_amd.train.common import capture_step
+            torch.manual_seed(1)
+            model = GAT(conv).to(dev)
+            opt = torch.optim.Adam(model.parameters(), lr=5e-3, weight_decay=5e-4, capturable=True)
+            replay = capture_step(step, dev, warmup=args.warmup)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            with marker("gat_c5_train: recompute, HIP-graph replays"):
+                for _ in range(args.steps):
+                    loss = replay()
+                torch.cuda.synchronize()
+            res[name]["hip_graph_ms_per_step"] = round((time.perf_counter() - t0) * 1e3 / args.steps, 3)
+            res[name]["hip_graph_final_loss"] = round(float(loss.detach()), 5)
+            del model, opt, replay
     b1 = gat_alg_bytes(n, e, heads, hidden)
     b2 = gat_alg_bytes(n, e, 1, classes)
     alg = sum(b1) + sum(b2)

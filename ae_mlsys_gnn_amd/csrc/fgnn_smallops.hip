@@ -370,14 +370,33 @@ extern "C" int fgnn_gather_rows(int64_t E, int W, const int32_t *permute, const 
 // sparse rows by the mean row length.  Measured (softmax / backward / scatter / gather-row, ms; [cache, long cache, stream]):
 //   114.8 M entries in 233 k rows, 8 heads:  [8,16,8] 1.79 / 2.49 / 3.60 / 4.07   [4,8,4] 1.85 / 2.70 / 2.56 / 3.56   [2,4,4] 1.97 / 2.89 / 2.67 / 3.74
 //   64.3 M entries in 2.45 M rows, 8 heads:  [8,16,8] 3.13 / 3.61 / 6.92 / 7.34   [4,8,4] 2.50 / 2.41 / 3.58 / 4.07   [2,4,4] 2.01 / 2.00 / 3.55 / 3.53
-template <int CACHE_, int CLONG_, int STREAM_> struct so_cfg { static constexpr int CACHE = CACHE_, CLONG = CLONG_, STREAM = STREAM_; };
+// L: lanes a short row gets (64: a wave per row; 32, 16, 8: a wave takes 64 / L rows side by side, each in its own group of L
+// lanes - where the mean row fills a fraction of a wave's trip, the per-row chain of dependent loads is shared by 2-8 rows).
+template <int CACHE_, int CLONG_, int STREAM_, int L_ = 64> struct so_cfg { static constexpr int CACHE = CACHE_, CLONG = CLONG_, STREAM = STREAM_, L = L_; };
 #define SO_DENSE_ROW_FLOATS 1024          // mean floats per row from which a launch takes its dense-row configuration
 static inline bool so_dense_rows(int N, int64_t elems) { return elems >= (int64_t)SO_DENSE_ROW_FLOATS * N; }
-// launch.operator()<VEC, CFG>() with VEC = 4 or 1 and CFG = the `dense` or `sparse` type of the calling scope
-#define SO_LAUNCH_BY_ROWS(launch, vec4, is_dense)                                                         \
-    do {                                                                                                  \
-        if (vec4) { if (is_dense) launch.template operator()<4, dense>(); else launch.template operator()<4, sparse>(); } \
-        else { if (is_dense) launch.template operator()<1, dense>(); else launch.template operator()<1, sparse>(); }     \
+// Lanes a short row gets in the sparse configuration, from the mean row length in groups of VEC floats.  Rows of a power-law graph
+// scatter widely about their mean, so a group is sized generously: 32 lanes down to a mean of 12 groups.  Measured on 64.3 M
+// entries in 2.45 M rows (softmax / backward / scatter / gather-row, ms; lanes 64 | 32 | 16 | 8):
+//   8 heads (mean 53 groups of four floats): 1.97 / 1.92 / 3.00 / 3.60 | 1.58 / 1.83 / 2.74 / 3.17 | 1.47 / 1.97 / 3.14 / 3.56 | 1.67 / 2.40 / 4.24 / 4.72
+//   1 head (mean 26 floats):                  1.05 / 1.09 / 1.67 / 1.46 | 0.71 / 0.89 / 1.51 / 1.29 | 0.65 / 0.99 / 1.82 / 1.49 | 0.76 / 1.34 / 2.71 / 2.10
+static inline int so_pick_lanes(int N, int64_t elems, int vec, int W)
+{
+    const int64_t mean_groups = elems / vec / std::max(N, 1);
+    int L = mean_groups > 64 ? 64 : mean_groups > 12 ? 32 : mean_groups > 6 ? 16 : 8;
+    while (L < W) L *= 2;                                   // a group holds at least one entry
+    return L;
+}
+// launch.operator()<VEC, CFG>() with VEC = 4 or 1 and CFG = the `dense` type of the calling scope or so_cfg<SP_CACHE, SP_CLONG,
+// SP_STREAM, lanes> from its constants
+#define SO_LAUNCH_CFG(launch, vec4, ...) do { if (vec4) launch.template operator()<4, __VA_ARGS__>(); else launch.template operator()<1, __VA_ARGS__>(); } while (0)
+#define SO_LAUNCH_BY_ROWS(launch, vec4, is_dense, lanes)                                              \
+    do {                                                                                              \
+        if (is_dense) SO_LAUNCH_CFG(launch, vec4, dense);                                             \
+        else if ((lanes) == 32) SO_LAUNCH_CFG(launch, vec4, so_cfg<SP_CACHE, SP_CLONG, SP_STREAM, 32>); \
+        else if ((lanes) == 16) SO_LAUNCH_CFG(launch, vec4, so_cfg<SP_CACHE, SP_CLONG, SP_STREAM, 16>); \
+        else if ((lanes) == 8) SO_LAUNCH_CFG(launch, vec4, so_cfg<SP_CACHE, SP_CLONG, SP_STREAM, 8>);   \
+        else SO_LAUNCH_CFG(launch, vec4, so_cfg<SP_CACHE, SP_CLONG, SP_STREAM, 64>);                    \
     } while (0)
 
 // Threads of the workgroups of a row-reduction launch and the grid: n_long workgroups for the long-row candidates, then one
@@ -385,10 +404,11 @@ static inline bool so_dense_rows(int N, int64_t elems) { return elems >= (int64_
 // its rows one after the other, each a chain of dependent memory round trips); larger ones hold more of a row in registers.
 // Measured on a 115 M-entry power-law graph, 8 heads (128 / 256 / 512 threads): softmax 1.93 / 1.78 / 1.84 ms, its backward
 // 3.29 / 2.77 / 2.48, the scatter kernel 3.93 / 3.60 / 4.43, gather-row 4.03 / 4.06 / 4.83, row sums 1.08 / 0.79 / 0.66.
-static inline unsigned so_grid(int N, int64_t elems, int tpb, unsigned *n_long)
+static inline unsigned so_grid(int N, int64_t elems, int tpb, unsigned *n_long, int lanes_per_row = 64)
 {
     *n_long = elems > SO_LONG_ELEMS ? (unsigned)((N + SO_CAND - 1) / SO_CAND) : 0u;      // otherwise no row can be long
-    return *n_long + (unsigned)((N + tpb / 64 - 1) / (tpb / 64));
+    const int rows_per_block = (tpb / 64) * (64 / lanes_per_row);
+    return *n_long + (unsigned)((N + rows_per_block - 1) / rows_per_block);
 }
 
 struct so_max { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
@@ -429,6 +449,25 @@ __device__ __forceinline__ so_grp<VEC> so_column_reduce(so_grp<VEC> v, int lane,
     return v;
 }
 
+// The same combination inside aligned groups of L lanes (L a power of two, W <= L): group-relative lane sl = lane % L, the lanes
+// sl, sl + W, ... < S0 = (L / W) * W of a group are combined and every lane of the group gets the result of its column.
+template <int VEC, int L, class Op>
+__device__ __forceinline__ so_grp<VEC> so_group_reduce(so_grp<VEC> v, int lane, int W, int S0, Op op)
+{
+    const int sl = lane & (L - 1);
+    for (int off = W; off < S0; off <<= 1) {
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) {
+            const float o = __shfl(v.c[c], (lane + off) & 63);          // used only where sl + off < S0 <= L: the same group
+            if (sl + off < S0) v.c[c] = op(v.c[c], o);
+        }
+    }
+    const int src = lane - sl + sl % W;
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) v.c[c] = __shfl(v.c[c], src);
+    return v;
+}
+
 // Work unit u (a wave of the short launch, a candidate of the long launch) takes row (u * p) mod N with p a prime
 // above 2^31: a bijection of [0, N) that scatters neighbouring rows.  Workgroups go to the eight XCDs round-robin, and on a
 // power-law graph generated by recursive quadrants a row's length follows the low bits of its number (the
@@ -445,6 +484,19 @@ __device__ __forceinline__ bool so_take_short_row(unsigned u, int N, int W, cons
     pb = fg_uni(ptr[row]);
     n = (int64_t)(fg_uni(ptr[row + 1]) - pb) * W;
     return n * VEC <= SO_LONG_ELEMS;
+}
+// Short launch with groups of L < 64 lanes: group g of work unit u takes row (u * 64 / L + g) scattered as above; n = 0 marks a group
+// without a row of its own (past the end, empty, or a long row).  False when no group of the wave has one.
+template <int VEC, int L>
+__device__ __forceinline__ bool so_take_short_rows(unsigned u, int N, int W, const int *ptr, int &row, int &pb, int64_t &n, bool &mine)
+{
+    const unsigned v = u * (64 / L) + (unsigned)fg_lane() / L;
+    mine = v < (unsigned)N;
+    row = mine ? so_scattered_row(v, N) : 0;
+    pb = mine ? ptr[row] : 0;
+    n = mine ? (int64_t)(ptr[row + 1] - pb) * W : 0;
+    if (n * VEC > SO_LONG_ELEMS) { n = 0; mine = false; }          // the long launch has it
+    return __builtin_amdgcn_ballot_w64(mine) != 0ull;
 }
 // Long launch: bit l of the result is set when candidate blockIdx.x * SO_CAND + l is a long row (uniform over the workgroup).
 template <int VEC>
@@ -516,12 +568,17 @@ template <int VEC> struct so_from_scores {
     }
 };
 
-template <int NW, int VEC, int CACHE, int STREAM, class Src>
-__device__ __forceinline__ void so_softmax_row(int W, int64_t n, const Src &src, float *__restrict__ dst, float (*sh)[64])
+template <int NW, int VEC, int CACHE, int STREAM, class Src, int L = 64>          // L < 64 (NW == 1): n, src and dst are per group of L lanes
+__device__ __forceinline__ void so_softmax_row(int W, int64_t n, const Src &src, float *dst, float (*sh)[64])
 {
-    const int lane = fg_lane(), S0 = (64 / W) * W;
-    const int64_t first = (NW > 1 ? fg_wave() * S0 : 0) + lane, step = (int64_t)S0 * NW;
-    const bool act = lane < S0;
+    static_assert(L == 64 || NW == 1, "lane groups only where one wave has the row");
+    const int lane = fg_lane(), sl = lane & (L - 1), S0 = (L / W) * W;
+    const int64_t first = (NW > 1 ? fg_wave() * S0 : 0) + sl, step = (int64_t)S0 * NW;
+    const bool act = sl < S0;
+    auto reduce = [&](so_grp<VEC> v, auto op) {
+        if constexpr (L < 64) return so_group_reduce<VEC, L>(v, lane, W, S0, op);
+        else return so_column_reduce<NW, VEC>(v, lane, W, S0, sh, op);
+    };
     so_grp<VEC> v[CACHE], m = so_fill<VEC>(-INFINITY), s = so_fill<VEC>(0.f);
 #pragma unroll
     for (int i = 0; i < CACHE; ++i) {
@@ -556,14 +613,14 @@ __device__ __forceinline__ void so_softmax_row(int W, int64_t n, const Src &src,
             }
         }
     }
-    const so_grp<VEC> mall = so_column_reduce<NW, VEC>(m, lane, W, S0, sh, so_max());
+    const so_grp<VEC> mall = reduce(m, so_max());
 #pragma unroll
     for (int c = 0; c < VEC; ++c) s.c[c] = s.c[c] > 0.f ? s.c[c] * __expf(m.c[c] - mall.c[c]) : 0.f;      // the streamed part, rebased
 #pragma unroll
     for (int i = 0; i < CACHE; ++i)
 #pragma unroll
         for (int c = 0; c < VEC; ++c) { v[i].c[c] = __expf(v[i].c[c] - mall.c[c]); s.c[c] += v[i].c[c]; }      // exp(-inf) = 0 past the row
-    so_grp<VEC> inv = so_column_reduce<NW, VEC>(s, lane, W, S0, sh, so_add());
+    so_grp<VEC> inv = reduce(s, so_add());
 #pragma unroll
     for (int c = 0; c < VEC; ++c) inv.c[c] = 1.f / inv.c[c];
 #pragma unroll
@@ -609,6 +666,13 @@ __global__ __launch_bounds__(TPB) void edge_softmax_kernel(int N, int W, unsigne
     int row, pb;
     int64_t n;
     const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (TPB / 64)) + fg_wave());
+    if constexpr (CFG::L < 64) {
+        bool mine;
+        if (!so_take_short_rows<VEC, CFG::L>(u, N, W, ptr, row, pb, n, mine)) return;
+        so_softmax_row<1, VEC, CFG::CACHE, CFG::STREAM, so_from_array<VEC>, CFG::L>(W, n, so_from_array<VEC>{in + (size_t)pb * W * VEC},
+                                                                                     out + (size_t)pb * W * VEC, nullptr);
+        return;
+    }
     if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n) || n == 0) return;
     so_softmax_row<1, VEC, CFG::CACHE, CFG::STREAM>(W, n, so_from_array<VEC>{in + (size_t)pb * W * VEC}, out + (size_t)pb * W * VEC, nullptr);
 }
@@ -623,27 +687,34 @@ __global__ __launch_bounds__(TPB) void gat_scatter_kernel(int N, int W, unsigned
 {
     __shared__ float sh[TPB / 64][64];
     __shared__ unsigned long long sh_mask;
-    const int col = fg_lane() % W;
-    auto source = [&](int row, int pb) {
+    auto source = [&](int row, int pb, int col) {
         so_from_scores<VEC> src;
         src.idx = idx + pb; src.ac = ac; src.elrelu = elrelu ? elrelu + (size_t)pb * W * VEC : nullptr;
         src.ar = so_load<VEC>(ar + ((size_t)row * W + col) * VEC);
         src.W = W; src.col = col; src.slope = slope;
         return src;
     };
+    const int col = fg_lane() % W;
     if (blockIdx.x < n_long_blocks) {
         for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
             const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
             const int pb = fg_uni(ptr[row]);
-            so_softmax_row<TPB / 64, VEC, CFG::CLONG, CFG::STREAM>(W, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, source(row, pb), esoft + (size_t)pb * W * VEC, sh);
+            so_softmax_row<TPB / 64, VEC, CFG::CLONG, CFG::STREAM>(W, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, source(row, pb, col), esoft + (size_t)pb * W * VEC, sh);
         }
         return;
     }
     int row, pb;
     int64_t n;
     const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (TPB / 64)) + fg_wave());
+    if constexpr (CFG::L < 64) {
+        bool mine;
+        if (!so_take_short_rows<VEC, CFG::L>(u, N, W, ptr, row, pb, n, mine)) return;
+        so_softmax_row<1, VEC, CFG::CACHE, CFG::STREAM, so_from_scores<VEC>, CFG::L>(W, n, source(row, pb, (fg_lane() & (CFG::L - 1)) % W),
+                                                                                      esoft + (size_t)pb * W * VEC, nullptr);
+        return;
+    }
     if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n) || n == 0) return;
-    so_softmax_row<1, VEC, CFG::CACHE, CFG::STREAM>(W, n, source(row, pb), esoft + (size_t)pb * W * VEC, nullptr);
+    so_softmax_row<1, VEC, CFG::CACHE, CFG::STREAM>(W, n, source(row, pb, col), esoft + (size_t)pb * W * VEC, nullptr);
 }
 
 // The factor LeakyReLU' puts on an entry's gradient, for the fused gather_row pass of the fuse-scatter GAT backward
@@ -679,13 +750,18 @@ template <int VEC> struct so_sign_scores {
 
 // gin = factor * sm * (g - sum_row sm * g); with an active Sign also rowsum[lane's heads] = sum_row gin (the grad_attn_row of
 // the fuse-scatter backward).  gin may be g itself: every value is read before it is overwritten, by the same lane.
-template <int NW, int VEC, int CACHE, int STREAM, class Sign>
+template <int NW, int VEC, int CACHE, int STREAM, class Sign, int L = 64>         // L < 64 (NW == 1): pb, n, sign and rowsum are per group of L lanes
 __device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, const float *__restrict__ sm, const float *g,
-                                                   float *gin, const Sign &sign, float *__restrict__ rowsum, float (*sh)[64])
+                                                   float *gin, const Sign &sign, float *rowsum, float (*sh)[64])
 {
-    const int lane = fg_lane(), S0 = (64 / W) * W;
-    const int64_t first = (NW > 1 ? fg_wave() * S0 : 0) + lane, step = (int64_t)S0 * NW;
-    const bool act = lane < S0;
+    static_assert(L == 64 || NW == 1, "lane groups only where one wave has the row");
+    const int lane = fg_lane(), sl = lane & (L - 1), S0 = (L / W) * W;
+    const int64_t first = (NW > 1 ? fg_wave() * S0 : 0) + sl, step = (int64_t)S0 * NW;
+    const bool act = sl < S0;
+    auto reduce = [&](so_grp<VEC> v, auto op) {
+        if constexpr (L < 64) return so_group_reduce<VEC, L>(v, lane, W, S0, op);
+        else return so_column_reduce<NW, VEC>(v, lane, W, S0, sh, op);
+    };
     const size_t base = (size_t)pb * W * VEC;
     so_grp<VEC> sv[CACHE], gv[CACHE], acc = so_fill<VEC>(0.f);
 #pragma unroll
@@ -715,7 +791,7 @@ __device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, con
                 for (int c = 0; c < VEC; ++c) acc.c[c] = fmaf(a[j].c[c], b[j].c[c], acc.c[c]);
         }
     }
-    acc = so_column_reduce<NW, VEC>(acc, lane, W, S0, sh, so_add());
+    acc = reduce(acc, so_add());
     so_grp<VEC> rs = so_fill<VEC>(0.f);
 #pragma unroll
     for (int i = 0; i < CACHE; ++i) {
@@ -758,8 +834,8 @@ __device__ __forceinline__ void so_softmax_bwd_row(int W, int pb, int64_t n, con
         }
     }
     if constexpr (Sign::active) {
-        rs = so_column_reduce<NW, VEC>(rs, lane, W, S0, sh, so_add());
-        if (lane < W && (NW == 1 || fg_wave() == 0)) so_store<VEC>(rowsum + (size_t)lane * VEC, rs);
+        rs = reduce(rs, so_add());
+        if (sl < W && rowsum && (NW == 1 || fg_wave() == 0)) so_store<VEC>(rowsum + (size_t)sl * VEC, rs);      // rowsum == NULL: a group without a row
     }
 }
 
@@ -781,6 +857,12 @@ __global__ __launch_bounds__(TPB) void edge_softmax_bwd_kernel(int N, int W, uns
     int row, pb;
     int64_t n;
     const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (TPB / 64)) + fg_wave());
+    if constexpr (CFG::L < 64) {
+        bool mine;
+        if (!so_take_short_rows<VEC, CFG::L>(u, N, W, ptr, row, pb, n, mine)) return;
+        so_softmax_bwd_row<1, VEC, CFG::CACHE, CFG::STREAM, so_sign_none<VEC>, CFG::L>(W, pb, n, sm, g, gin, so_sign_none<VEC>{}, nullptr, nullptr);
+        return;
+    }
     if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n) || n == 0) return;
     so_softmax_bwd_row<1, VEC, CFG::CACHE, CFG::STREAM>(W, pb, n, sm, g, gin, so_sign_none<VEC>{}, nullptr, nullptr);
 }
@@ -796,30 +878,38 @@ __global__ __launch_bounds__(TPB) void gat_gather_row_kernel(int N, int W, unsig
 {
     __shared__ float sh[TPB / 64][64];
     __shared__ unsigned long long sh_mask;
-    const int col = fg_lane() % W;
-    auto run = [&]<int NW>(int row, int pb, int64_t n, float (*shp)[64]) {
-        float *rowsum = gar + (size_t)row * W * VEC;
+    // L: lanes per row (64 except on the packed short path); mine: the lane group has a row whose sums it stores
+    auto run = [&]<int NW, int L>(int row, int pb, int64_t n, bool mine, float (*shp)[64]) {
+        float *rowsum = mine ? gar + (size_t)row * W * VEC : nullptr;
+        const int col = (fg_lane() & (L - 1)) % W;
         if constexpr (FROM_ARRAY) {
-            so_softmax_bwd_row<NW, VEC, CFG::CACHE, CFG::STREAM>(W, pb, n, sm, g, gout, so_sign_array<VEC>{elrelu + (size_t)pb * W * VEC, slope}, rowsum, shp);
+            so_softmax_bwd_row<NW, VEC, CFG::CACHE, CFG::STREAM, so_sign_array<VEC>, L>(W, pb, n, sm, g, gout, so_sign_array<VEC>{elrelu + (size_t)pb * W * VEC, slope},
+                                                                                      rowsum, shp);
         } else {
             so_sign_scores<VEC> sg;
             sg.idx = idx + pb; sg.ac = ac; sg.ar = so_load<VEC>(ar + ((size_t)row * W + col) * VEC); sg.W = W; sg.col = col; sg.slope = slope;
-            so_softmax_bwd_row<NW, VEC, CFG::CACHE, CFG::STREAM>(W, pb, n, sm, g, gout, sg, rowsum, shp);
+            so_softmax_bwd_row<NW, VEC, CFG::CACHE, CFG::STREAM, so_sign_scores<VEC>, L>(W, pb, n, sm, g, gout, sg, rowsum, shp);
         }
     };
     if (blockIdx.x < n_long_blocks) {
         for (unsigned long long m = so_long_candidates<VEC>(N, W, ptr, &sh_mask); m; m &= m - 1) {
             const int row = so_scattered_row(blockIdx.x * SO_CAND + (unsigned)__builtin_ctzll(m), N);
             const int pb = fg_uni(ptr[row]);
-            run.template operator()<TPB / 64>(row, pb, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, sh);
+            run.template operator()<TPB / 64, 64>(row, pb, (int64_t)(fg_uni(ptr[row + 1]) - pb) * W, true, sh);
         }
         return;
     }
     int row, pb;
     int64_t n;
     const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (TPB / 64)) + fg_wave());
+    if constexpr (CFG::L < 64) {
+        bool mine;
+        if (!so_take_short_rows<VEC, CFG::L>(u, N, W, ptr, row, pb, n, mine)) return;
+        run.template operator()<1, CFG::L>(row, pb, n, mine, nullptr);
+        return;
+    }
     if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n)) return;
-    run.template operator()<1>(row, pb, n, nullptr);             // an empty row stores its zero sums
+    run.template operator()<1, 64>(row, pb, n, true, nullptr);             // an empty row stores its zero sums
 }
 
 // More than 64 heads: one wave per row, one head at a time.
@@ -869,16 +959,16 @@ extern "C" int fgnn_edge_softmax(int N, int64_t E, int H, const int32_t *row_ptr
         hipLaunchKernelGGL(edge_softmax_wide_kernel, dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, in, out);
         return fgnn_launch_status("edge_softmax_wide_kernel");
     }
-    unsigned n_long;
     constexpr int TPB = 256;
-    const unsigned grid = so_grid(N, E * H, TPB, &n_long);
     const bool vec4 = H % 4 == 0 && fgnn_aligned16(in) && fgnn_aligned16(out);
     auto launch = [&]<int VEC, class CFG>() {
+        unsigned n_long;
+        const unsigned grid = so_grid(N, E * H, TPB, &n_long, CFG::L);
         hipLaunchKernelGGL((edge_softmax_kernel<VEC, TPB, CFG>), dim3(grid), dim3(TPB), 0, st, N, H / VEC, n_long, row_ptr, in, out);
     };
     using dense = so_cfg<8, 16, 8>;
-    using sparse = so_cfg<2, 4, 4>;
-    SO_LAUNCH_BY_ROWS(launch, vec4, so_dense_rows(N, E * H));
+    constexpr int SP_CACHE = 2, SP_CLONG = 4, SP_STREAM = 4;
+    SO_LAUNCH_BY_ROWS(launch, vec4, so_dense_rows(N, E * H), so_pick_lanes(N, E * H, vec4 ? 4 : 1, vec4 ? H / 4 : H));
     return fgnn_launch_status("edge_softmax_kernel");
 }
 
@@ -894,16 +984,16 @@ extern "C" int fgnn_edge_softmax_backward(int N, int64_t E, int H, const int32_t
         hipLaunchKernelGGL(edge_softmax_bwd_wide_kernel, dim3(waves), dim3(FGNN_TPB), 0, st, N, H, row_ptr, sm, grad_out, grad_in);
         return fgnn_launch_status("edge_softmax_bwd_wide_kernel");
     }
-    unsigned n_long;
     constexpr int TPB = 512;
-    const unsigned grid = so_grid(N, E * H, TPB, &n_long);
     const bool vec4 = H % 4 == 0 && fgnn_aligned16(sm) && fgnn_aligned16(grad_out) && fgnn_aligned16(grad_in);
     auto launch = [&]<int VEC, class CFG>() {
+        unsigned n_long;
+        const unsigned grid = so_grid(N, E * H, TPB, &n_long, CFG::L);
         hipLaunchKernelGGL((edge_softmax_bwd_kernel<VEC, TPB, CFG>), dim3(grid), dim3(TPB), 0, st, N, H / VEC, n_long, row_ptr, sm, grad_out, grad_in);
     };
     using dense = so_cfg<8, 8, 4>;           // the backward keeps two arrays: CACHE groups of each, STREAM loads of each in flight
-    using sparse = so_cfg<2, 2, 2>;
-    SO_LAUNCH_BY_ROWS(launch, vec4, so_dense_rows(N, E * H));
+    constexpr int SP_CACHE = 2, SP_CLONG = 2, SP_STREAM = 2;
+    SO_LAUNCH_BY_ROWS(launch, vec4, so_dense_rows(N, E * H), so_pick_lanes(N, E * H, vec4 ? 4 : 1, vec4 ? H / 4 : H));
     return fgnn_launch_status("edge_softmax_bwd_kernel");
 }
 
@@ -919,17 +1009,17 @@ extern "C" int fgnn_gat_scatter(int N, int64_t E, int H, const int32_t *row_ptr,
     if (N == 0 || E == 0) return 0;
     FGNN_REQUIRE(row_ptr && col_ind && attn_row && attn_col && e_softmax, FGNN_ERR_NULL, "fgnn_gat_scatter: NULL argument");
     hipStream_t st = (hipStream_t)stream;
-    unsigned n_long;
     constexpr int TPB = 256;
-    const unsigned grid = so_grid(N, E * H, TPB, &n_long);
     const bool vec4 = H % 4 == 0 && fgnn_aligned16(attn_row) && fgnn_aligned16(attn_col) && fgnn_aligned16(e_softmax) && fgnn_aligned16(e_lrelu);
     auto launch = [&]<int VEC, class CFG>() {
+        unsigned n_long;
+        const unsigned grid = so_grid(N, E * H, TPB, &n_long, CFG::L);
         hipLaunchKernelGGL((gat_scatter_kernel<VEC, TPB, CFG>), dim3(grid), dim3(TPB), 0, st, N, H / VEC, n_long, row_ptr, col_ind, attn_row, attn_col,
                            negative_slope, e_lrelu, e_softmax);
     };
     using dense = so_cfg<4, 8, 4>;           // every load is an index and a gathered row: fewer in flight, more waves resident
-    using sparse = so_cfg<2, 4, 4>;
-    SO_LAUNCH_BY_ROWS(launch, vec4, so_dense_rows(N, E * H));
+    constexpr int SP_CACHE = 2, SP_CLONG = 4, SP_STREAM = 4;
+    SO_LAUNCH_BY_ROWS(launch, vec4, so_dense_rows(N, E * H), so_pick_lanes(N, E * H, vec4 ? 4 : 1, vec4 ? H / 4 : H));
     return fgnn_launch_status("gat_scatter_kernel");
 }
 
@@ -949,12 +1039,12 @@ extern "C" int fgnn_gat_gather_row(int N, int64_t E, int H, const int32_t *row_p
     FGNN_REQUIRE(E == 0 || e_lrelu || (col_ind && attn_row && attn_col), FGNN_ERR_NULL,
                  "fgnn_gat_gather_row: without e_lrelu the scores are formed again from col_ind, attn_row and attn_col");
     hipStream_t st = (hipStream_t)stream;
-    unsigned n_long;
     constexpr int TPB = 256;
-    const unsigned grid = so_grid(N, E * H, TPB, &n_long);
     const bool vec4 = H % 4 == 0 && fgnn_aligned16(e_softmax) && fgnn_aligned16(grad_edge) && fgnn_aligned16(grad_edge_out) && fgnn_aligned16(grad_attn_row) &&
                       fgnn_aligned16(e_lrelu) && fgnn_aligned16(attn_row) && fgnn_aligned16(attn_col);
     auto launch = [&]<int VEC, class CFG>() {
+        unsigned n_long;
+        const unsigned grid = so_grid(N, E * H, TPB, &n_long, CFG::L);
         auto go = [&]<bool FROM_ARRAY>() {
             hipLaunchKernelGGL((gat_gather_row_kernel<VEC, FROM_ARRAY, TPB, CFG>), dim3(grid), dim3(TPB), 0, st, N, H / VEC, n_long, row_ptr, col_ind,
                                attn_row, attn_col, e_lrelu, negative_slope, e_softmax, grad_edge, grad_edge_out, grad_attn_row);
@@ -962,8 +1052,8 @@ extern "C" int fgnn_gat_gather_row(int N, int64_t E, int H, const int32_t *row_p
         if (e_lrelu) go.template operator()<true>(); else go.template operator()<false>();
     };
     using dense = so_cfg<8, 8, 2>;
-    using sparse = so_cfg<4, 4, 1>;
-    SO_LAUNCH_BY_ROWS(launch, vec4, so_dense_rows(N, E * H));
+    constexpr int SP_CACHE = 4, SP_CLONG = 4, SP_STREAM = 1;
+    SO_LAUNCH_BY_ROWS(launch, vec4, so_dense_rows(N, E * H), so_pick_lanes(N, E * H, vec4 ? 4 : 1, vec4 ? H / 4 : H));
     return fgnn_launch_status("gat_gather_row_kernel");
 }
 
@@ -1047,18 +1137,19 @@ __global__ __launch_bounds__(FGNN_TPB) void u_add_v_wide_kernel(int N, int W, co
 // into a zero-filled buffer as the reference does it (src/u_add_v/u_add_v.cu:43-90, which adds into uninitialised
 // memory); without COLS the column sums are left to the tile-ordered pass of fgnn_edge_colsum.  One pass over grad_out,
 // rows shared out as in the softmax kernels.
-template <int NW, int VEC, bool COLS>
+template <int NW, int VEC, bool COLS, int L = 64>        // L < 64 (NW == 1): row, pb, pe per group of L lanes; row < 0: a group without a row
 __device__ __forceinline__ void so_rowsum_row(int W, int row, int pb, int pe, const int *__restrict__ idx, const float *__restrict__ g,
                                               float *__restrict__ grow, float *__restrict__ gcol, float (*sh)[64])
 {
-    const int lane = fg_lane(), S0 = (64 / W) * W, w = lane % W;
-    const int per = S0 / W;                                        // entries per wave-wide trip
+    static_assert(L == 64 || NW == 1, "lane groups only where one wave has the row");
+    const int lane = fg_lane(), sl = lane & (L - 1), S0 = (L / W) * W, w = sl % W;
+    const int per = S0 / W;                                        // entries per trip of the wave (of the lane group)
     constexpr int nw = NW;
-    const bool act = lane < S0;
+    const bool act = sl < S0;
     so_grp<VEC> acc = so_fill<VEC>(0.f);
     if (act) {
 #pragma unroll 8
-        for (int q = pb + (NW > 1 ? fg_wave() * per : 0) + lane / W; q < pe; q += per * nw) {
+        for (int q = pb + (NW > 1 ? fg_wave() * per : 0) + sl / W; q < pe; q += per * nw) {
             const so_grp<VEC> v = so_load<VEC>(g + ((size_t)q * W + w) * VEC);
 #pragma unroll
             for (int c = 0; c < VEC; ++c) acc.c[c] += v.c[c];
@@ -1069,11 +1160,12 @@ __device__ __forceinline__ void so_rowsum_row(int W, int row, int pb, int pe, co
             }
         }
     }
-    acc = so_column_reduce<NW, VEC>(acc, lane, W, S0, sh, so_add());
-    if (lane < W && (NW == 1 || fg_wave() == 0)) so_store<VEC>(grow + ((size_t)row * W + lane) * VEC, acc);
+    if constexpr (L < 64) acc = so_group_reduce<VEC, L>(acc, lane, W, S0, so_add());
+    else acc = so_column_reduce<NW, VEC>(acc, lane, W, S0, sh, so_add());
+    if (sl < W && row >= 0 && (NW == 1 || fg_wave() == 0)) so_store<VEC>(grow + ((size_t)row * W + sl) * VEC, acc);
 }
 
-template <int VEC, bool COLS, int TPB>
+template <int VEC, bool COLS, int TPB, int L = 64>
 __global__ __launch_bounds__(TPB) void edge_rowsum_kernel(int N, int W, unsigned n_long_blocks, const int *__restrict__ ptr,
                                                                   const int *__restrict__ idx, const float *__restrict__ g, float *__restrict__ grow,
                                                                   float *__restrict__ gcol)
@@ -1090,6 +1182,12 @@ __global__ __launch_bounds__(TPB) void edge_rowsum_kernel(int N, int W, unsigned
     int row, pb;
     int64_t n;
     const unsigned u = (unsigned)fg_uni((int)((blockIdx.x - n_long_blocks) * (TPB / 64)) + fg_wave());
+    if constexpr (L < 64) {
+        bool mine;
+        if (!so_take_short_rows<VEC, L>(u, N, W, ptr, row, pb, n, mine)) return;
+        so_rowsum_row<1, VEC, COLS, L>(W, mine ? row : -1, pb, pb + (int)(n / W), idx, g, grow, gcol, nullptr);
+        return;
+    }
     if (!so_take_short_row<VEC>(u, N, W, ptr, row, pb, n)) return;      // empty rows stay here: they store zeros
     so_rowsum_row<1, VEC, COLS>(W, row, pb, fg_uni(ptr[row + 1]), idx, g, grow, gcol, nullptr);
 }
@@ -1191,11 +1289,15 @@ extern "C" int fgnn_edge_rowsum(int N, int64_t E, int W, const int32_t *row_ptr,
     const bool vec4 = W % 4 == 0 && fgnn_aligned16(g) && fgnn_aligned16(out);
     unsigned n_long;
     constexpr int TPB = 512;
-    const unsigned grid = so_grid(N, E * W, TPB, &n_long);
-    if (vec4)
-        hipLaunchKernelGGL((edge_rowsum_kernel<4, false, TPB>), dim3(grid), dim3(TPB), 0, st, N, W / 4, n_long, row_ptr, nullptr, g, out, nullptr);
-    else
-        hipLaunchKernelGGL((edge_rowsum_kernel<1, false, TPB>), dim3(grid), dim3(TPB), 0, st, N, W, n_long, row_ptr, nullptr, g, out, nullptr);
+    // sparse rows share waves, as in the softmax kernels
+    const int lanes = so_dense_rows(N, E * W) ? 64 : so_pick_lanes(N, E * W, vec4 ? 4 : 1, vec4 ? W / 4 : W);
+    auto launch = [&]<int VEC, int L>() {
+        const unsigned grid = so_grid(N, E * W, TPB, &n_long, L);
+        hipLaunchKernelGGL((edge_rowsum_kernel<VEC, false, TPB, L>), dim3(grid), dim3(TPB), 0, st, N, W / VEC, n_long, row_ptr, nullptr, g, out, nullptr);
+    };
+#define RS_L(LL) do { if (vec4) launch.template operator()<4, LL>(); else launch.template operator()<1, LL>(); } while (0)
+    if (lanes == 32) RS_L(32); else if (lanes == 16) RS_L(16); else if (lanes == 8) RS_L(8); else RS_L(64);
+#undef RS_L
     return fgnn_launch_status("edge_rowsum_kernel");
 }
 

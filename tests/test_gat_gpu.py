@@ -587,14 +587,16 @@ def test_validation_uses_the_width_of_the_gathered_matrix(monkeypatch):
     _lib.clear_schedule_cache()
 
 
-@pytest.mark.parametrize("n", [300, 20])
+@pytest.mark.parametrize("n", [300, 20, 3000, 30000])
 @pytest.mark.parametrize("h", [1, 3, 4, 8, 12, 20, 64])
 def test_fusescatter_kernels_against_the_oracle(h, n):
     """fgnn_gat_scatter (scores + LeakyReLU + row softmax in one pass, with and without the LeakyReLU array) and
     fgnn_gat_gather_row (softmax backward + LeakyReLU backward + row sums, sign from the stashed array or formed again, out
     of place and in place) on a graph with empty rows, rows either side of the wave / workgroup threshold and a 3000-entry
     hub, against float64.  n = 20 keeps only the rows of fixed length: a mean of 430 entries per row, for which the launches
-    take their dense-row configuration from 3 heads on (n = 300: only at 64 heads)."""
+    take their dense-row configuration from 3 heads on (n = 300: only at 64 heads).  n = 3000 and 30000 add rows of 0-11
+    entries until the mean row is 8 and 6 entries: short rows then share waves, 16 / 32 / 64 and 8 / 16 / 32 lanes per row
+    depending on the head count."""
     from ae_mlsys_gnn_amd.operators.fused_gat import gat_native
     g = degree_edge_graph(n=n, seed=h)
     gen = torch.Generator().manual_seed(h)

@@ -420,6 +420,48 @@ def test_u_add_v(nh):
     assert_close_sum(cd.grad, cl.grad, s_col, "u_add_v grad col")
 
 
+@pytest.mark.parametrize("w,max_deg", [(1, 6), (4, 6), (8, 6), (3, 8), (1, 22), (8, 22), (12, 30), (40, 3)])
+def test_row_operators_where_short_rows_share_a_wave(w, max_deg):
+    """Graphs whose mean row is a few entries (20 k rows of 0..max_deg entries, two long rows among them): the row kernels then
+    give a row 8, 16 or 32 lanes and a wave takes several rows side by side.  Edge softmax both ways and both halves of the
+    u_add_v backward (row sums, column sums) against float64; empty rows, rows past a group's registers and the long rows
+    (which go to whole workgroups) included."""
+    from ae_mlsys_gnn_amd.operators import edge_softmax as es
+    from ae_mlsys_gnn_amd.operators import u_add_v as uav
+    rng = np.random.default_rng(w * 100 + max_deg)
+    n = 20000
+    degs = rng.integers(0, max_deg + 1, size=n)
+    degs[77] = 8192 // w + 5           # a long row (more than 8192 floats)
+    degs[78] = 700                     # longer than any group's registers hold
+    g = custom_graph([list(rng.integers(0, n, size=int(d))) for d in degs], n)
+    gd = g.to(DEV)
+    e = g.n_edges
+    gen = torch.Generator().manual_seed(w + max_deg)
+    x = torch.randn(e, w, generator=gen, dtype=torch.float64) * 2
+    go = torch.randn(e, w, generator=gen, dtype=torch.float64)
+    xl = x.clone().requires_grad_(True)
+    ref = orc.edge_softmax(g.row_ptr, xl)
+    ref.backward(go)
+    xd = x.float().to(DEV).requires_grad_(True)
+    out = es.csr_edge_softmax(gd.row_ptr, xd)
+    out.backward(go.float().to(DEV))
+    c = c_exp(float(x.max() - x.min()))
+    one = torch.ones((), dtype=torch.float64)
+    assert_close_sum(out, ref.detach(), one, "edge_softmax, short rows, width %d" % w, c=c)
+    dst = orc.row_of_edge(g.row_ptr)
+    dot_abs = orc.segment_sums(g.row_ptr, ref.detach() * go.abs())
+    assert_close_sum(xd.grad, xl.grad, ref.detach() * (go.abs() + dot_abs[dst]), "edge_softmax grad, short rows, width %d" % w, c=c)
+    rv = torch.randn(n, w, generator=gen, dtype=torch.float64)
+    cv = torch.randn(n, w, generator=gen, dtype=torch.float64)
+    rl, cl = rv.clone().requires_grad_(True), cv.clone().requires_grad_(True)
+    orc.u_add_v(g.row_ptr, g.col_ind, rl, cl).backward(go)
+    rd, cd = rv.float().to(DEV).requires_grad_(True), cv.float().to(DEV).requires_grad_(True)
+    uav.u_add_v_op(gd.row_ptr, gd.col_ind, rd, cd).backward(go.float().to(DEV))
+    _, (s_row, s_col) = orc.multilinear_abs_sums(lambda a, b: orc.u_add_v(g.row_ptr, g.col_ind, a, b), (rv, cv), go)
+    assert_close_sum(rd.grad, rl.grad, s_row, "u_add_v grad row, short rows, width %d" % w)
+    assert_close_sum(cd.grad, cl.grad, s_col, "u_add_v grad col, short rows, width %d" % w)
+
+
 @pytest.mark.parametrize("seed", range(8))
 def test_small_operators_on_random_heavy_tailed_graphs(seed):
     """Random graphs whose row lengths straddle the kernels' thresholds (empty rows, rows of a few entries, rows around
@@ -1130,14 +1172,15 @@ def test_gather_rows_widths(w):
         assert torch.equal(out.cpu(), xin.cpu()[perm.long()])
 
 
-@pytest.mark.parametrize("n_short", [0, 6000])
+@pytest.mark.parametrize("n_short", [0, 6000, 60000])
 @pytest.mark.parametrize("nh", [1, 4, 8, 20])
 def test_edge_softmax_rows_beyond_the_register_cache(nh, n_short):
     """Rows longer than what a workgroup keeps in registers (the part beyond is folded into a running maximum and sum while
     it streams by): a 40 k-entry row whose values ascend, so the running maximum moves on every trip, one whose values
     descend, a constant one, next to short rows; forward and backward against float64.  With n_short rows of two entries
     appended the mean row is short and the launch takes its small-footprint configuration (fewer values cached, more
-    streamed) for the same long rows."""
+    streamed) for the same long rows; with 60000 of them the short rows share waves (groups of 8, 16 or 32 lanes per
+    row, by head count)."""
     from ae_mlsys_gnn_amd.operators import edge_softmax as op
     lens = [40000, 3, 0, 40000, 9000, 1, 40000] + [2] * n_short
     g = custom_graph([[0] * d for d in lens], len(lens))

@@ -444,6 +444,118 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_packed_kernel(GatFwdP p)
     }
 }
 
+// The slot of a work list that lane group g of the wave takes when every group has an item of its own: the G slots of a
+// wave are consecutive among the slots of ONE source bucket (slot ((k / WPB) * 8 + b) * WPB + k % WPB is the k-th slot of
+// bucket b in an XCD-aware list, and workgroup w runs on XCD w % 8); in a plain list they are simply consecutive.
+__device__ __forceinline__ int gat_group_slot(int G, int g, int bucketed)
+{
+    const int w = (int)blockIdx.x, v = fg_wave();
+    if (!bucketed) return (w * FGNN_WPB + v) * G + g;
+    const int b = w % FGNN_NUM_XCD, k = ((w / FGNN_NUM_XCD) * FGNN_WPB + v) * G + g;
+    return ((k / FGNN_WPB) * FGNN_NUM_XCD + b) * FGNN_WPB + k % FGNN_WPB;
+}
+
+// The packed forward with the lane groups on DIFFERENT items: group g of a wave takes a work item of its own and walks it
+// alone (its LPR lanes fetch LPR ids at a time, eight gathered rows of the group in flight), so one load instruction
+// fetches a row for each of G destinations and nothing is combined at the end.  Per-lane scores (no pair layout).
+template <int G, bool AUX, bool SLE1>
+__global__ __launch_bounds__(FGNN_TPB) void gat_fwd_rowpack_kernel(GatFwdP p, int bucketed)
+{
+    constexpr int LPR = 64 / G, U = 8;
+    const int lane = fg_lane();
+    const int H = p.H;
+    fg_packmap<G> pm;
+    pm.init(lane, p.HF, p.F);
+    const int sl = lane & (LPR - 1), gbase = lane - sl;
+    const int it = gat_group_slot(G, pm.grp, bucketed);
+    int row = -1, b = 0, e = 0, slot = -1;
+    if (it < p.n_items) {
+        if (p.items) { const fgnn_item q = p.items[it]; row = q.row; b = q.begin; e = q.end; slot = q.slot; }
+        else { row = it; b = p.ptr[it]; e = p.ptr[it + 1]; }
+    }
+    if (row < 0) { b = 0; e = 0; }                                    // padding item or past the list: nothing to walk or store
+    if (__builtin_amdgcn_ballot_w64(row >= 0) == 0ull) return;
+    const float slope = p.slope;
+    fg_vec<4> T, P;
+    T.zero(); P.zero();
+    float s = 0.f, cp = 0.f, m = -INFINITY;
+    const float arh = row >= 0 ? p.ar[(size_t)row * H + pm.hd] * FGNN_LOG2E : 0.f;
+    for (int c = b; __builtin_amdgcn_ballot_w64(c < e) != 0ull; c += LPR) {
+        const int cnt = min(LPR, e - c);                              // <= 0: this group is done
+        int idv = 0;
+        if (c < e) idv = p.idx[c + sl < e ? c + sl : c];              // idle lanes repeat a valid id
+        for (int t = 0; __builtin_amdgcn_ballot_w64(t < cnt) != 0ull; t += U) {
+            fg_vec<4> ld[U];
+            float ev[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u;
+                const size_t j = (size_t)(unsigned)__builtin_amdgcn_ds_bpermute((gbase + (ei & (LPR - 1))) << 2, idv);
+                if (ei < cnt && pm.ok) { ld[u].load(p.x + j * p.HF + pm.eoff); ev[u] = p.ac[j * H + pm.hd]; }
+                else { ld[u].zero(); ev[u] = 0.f; }
+            }
+            float bm = -INFINITY;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float v = fg_lrelu_t<SLE1>(fmaf(ev[u], FGNN_LOG2E, arh), slope);
+                v = (t + u < cnt && pm.ok) ? v : -INFINITY;           // no edge for this lane: weight 0
+                ev[u] = v;
+                bm = fmaxf(bm, v);
+            }
+            if (__builtin_amdgcn_ballot_w64(bm > m) != 0ull) {
+                const float mn = fmaxf(m, bm);
+                const float sc = (mn == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m - mn);
+                m = mn;
+                T.scale(sc);
+                s *= sc;
+                if (AUX) { P.scale(sc); cp *= sc; }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const float w = (ev[u] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ev[u] - m);
+                T.fma(w, ld[u]);
+                s += w;
+                if (AUX) {
+                    const float wp = ev[u] > 0.f ? w : 0.f;
+                    P.fma(wp, ld[u]);
+                    cp += wp;
+                }
+            }
+        }
+    }
+    if (!pm.ok || row < 0) return;
+    // same epilogue as gat_fwd_kernel: the maximum leaves in natural units, its rounding goes into the sums
+    const float mnat = m * FGNN_LN2;
+    const float fix = (b < e) ? __builtin_amdgcn_exp2f(m - mnat * FGNN_LOG2E) : 1.f;
+    if (slot < 0) {
+        const float inv = s > 0.f ? 1.f / s : 0.f;
+        const size_t o = (size_t)row * p.HF + pm.eoff;
+        if (AUX) {
+            fg_vec<4> o2 = T.lin(slope * inv, (1.f - slope) * inv, P);
+            o2.store_nt(p.out2 + o);
+        }
+        T.scale(inv);
+        T.store_nt(p.out + o);
+        if (pm.eoff % p.F == 0) {
+            const size_t so = (size_t)row * H + pm.hd;
+            p.emax[so] = (b < e) ? mnat : -1e38f;
+            p.esum[so] = s * fix;
+            if (AUX) p.cc[so] = (cp + slope * (s - cp)) * inv;
+        }
+    } else {
+        float *pp = p.part + (size_t)slot * gat_fwd_pw(p.HF, H, AUX);
+        T.scale(fix);
+        T.store_nt(pp + pm.eoff);
+        if (AUX) { P.scale(fix); P.store_nt(pp + p.HF + pm.eoff); }
+        if (pm.eoff % p.F == 0) {
+            float *st = pp + (AUX ? 2 : 1) * p.HF;
+            st[pm.hd] = mnat;
+            st[H + pm.hd] = s * fix;
+            st[2 * H + pm.hd] = cp * fix;
+        }
+    }
+}
+
 // Merge of the segments of split rows: log-sum-exp combination of (m, s, T, P).
 template <int VEC, int R, bool AUX>
 __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_merge_kernel(GatFwdP p, const fgnn_split *split, int n_split)
@@ -1045,6 +1157,102 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
     }
 }
 
+// The column pass with the lane groups on different items (see gat_fwd_rowpack_kernel).  T, P and z of an item stay inside
+// its group; the per-head dot product of the epilogue is reduced inside the group as well (no LDS).
+template <int G, int STASH, bool SLE1>
+__global__ __launch_bounds__(FGNN_TPB) void gat_bwd_rowpack_kernel(GatBwdP p, int bucketed)
+{
+    constexpr int LPR = 64 / G, U = 8;
+    const int lane = fg_lane();
+    const int H = p.H;
+    fg_packmap<G> pm;
+    pm.init(lane, p.HF, p.F);
+    const int sl = lane & (LPR - 1), gbase = lane - sl;
+    const int it = gat_group_slot(G, pm.grp, bucketed);
+    int col = -1, b = 0, e = 0, slot = -1;
+    if (it < p.n_items) {
+        if (p.items) { const fgnn_item q = p.items[it]; col = q.row; b = q.begin; e = q.end; slot = q.slot; }
+        else { col = it; b = p.ptr[it]; e = p.ptr[it + 1]; }
+    }
+    if (col < 0) { b = 0; e = 0; }
+    if (__builtin_amdgcn_ballot_w64(col >= 0) == 0ull) return;
+    fg_vec<4> T, P;
+    T.zero(); P.zero();
+    float z = 0.f;
+    const float ach = col >= 0 ? p.ac[(size_t)col * H + pm.hd] : 0.f;
+    for (int c = b; __builtin_amdgcn_ballot_w64(c < e) != 0ull; c += LPR) {
+        const int cnt = min(LPR, e - c);                              // <= 0: this group is done
+        int idv = 0, posv = 0;
+        if (c < e) {
+            const int qq = c + sl < e ? c + sl : c;                   // idle lanes repeat a valid entry
+            idv = p.idx[qq];
+            if (STASH) posv = p.permute ? p.permute[p.pos ? p.pos[qq] : qq] : qq;
+        }
+        for (int t = 0; __builtin_amdgcn_ballot_w64(t < cnt) != 0ull; t += U) {
+            fg_vec<4> ld[U];
+            float4 rc[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u, src = (gbase + (ei & (LPR - 1))) << 2;
+                const size_t i = (size_t)(unsigned)__builtin_amdgcn_ds_bpermute(src, idv);
+                const size_t pos = STASH ? (size_t)(unsigned)__builtin_amdgcn_ds_bpermute(src, posv) : 0;
+                if (ei < cnt && pm.ok) {
+                    ld[u].load(p.g + i * p.HF + pm.eoff);
+                    if (STASH == 2) rc[u] = make_float4(0.f, p.esm[pos * H + pm.hd], 0.f, p.delta[i * H + pm.hd]);
+                    else rc[u] = p.rec[i * H + pm.hd];
+                    if (STASH == 1) rc[u].y = p.esm[pos * H + pm.hd];
+                } else {
+                    ld[u].zero();
+                    rc[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float ev, al;
+                if (STASH == 2) { ev = __float_as_int(rc[u].y) >= 0 ? 1.f : -1.f; al = fabsf(rc[u].y); }
+                else if (STASH == 1) { ev = fmaf(ach, FGNN_LOG2E, rc[u].x); al = rc[u].y; }
+                else { ev = fg_lrelu_t<SLE1>(fmaf(ach, FGNN_LOG2E, rc[u].x), p.slope); al = __builtin_amdgcn_exp2f(ev - rc[u].y) * rc[u].z; }
+                al = (t + u < cnt && pm.ok) ? al : 0.f;
+                const bool pos_e = ev > 0.f;
+                T.fma(al, ld[u]);
+                P.fma(pos_e ? al : 0.f, ld[u]);
+                z = fmaf(pos_e ? al : al * p.slope, rc[u].w, z);
+            }
+        }
+    }
+    // epilogue of gat_bwd_finish, inside the group: every lane of a head holds that head's z
+    const bool whole = col >= 0 && slot < 0;
+    float d = 0.f;
+    if (whole && pm.ok) {
+        const size_t o = (size_t)col * p.HF + pm.eoff;
+        T.store_nt(p.gfeat + o);
+        fg_vec<4> g2 = T.lin(p.slope, 1.f - p.slope, P);
+        fg_vec<4> xv; xv.load(p.x + o);
+        d = xv.dot(g2);
+    }
+    const int lph = p.F / 4;                                          // lanes per head
+    if ((lph & (lph - 1)) == 0) {                                     // heads are aligned runs of a power of two lanes
+        for (int s = 1; s < lph; s <<= 1) d += __shfl_xor(d, s);
+        if (whole && pm.ok && sl % lph == 0) p.gac[(size_t)col * H + pm.hd] = d - z;
+    } else {                                                          // any width: one masked sum over the group per head
+        float r = 0.f;
+        for (int h = 0; h < H; ++h) {
+            float s1 = (pm.ok && pm.hd == h) ? d : 0.f;
+#pragma unroll
+            for (int s = 1; s < LPR; s <<= 1) s1 += __shfl_xor(s1, s);
+            if (sl == h) r = s1;
+        }
+        const float zh = fg_bperm(z, gbase + min(sl, H - 1) * lph);   // z of head sl, from that head's first lane
+        if (whole && sl < H) p.gac[(size_t)col * H + sl] = r - zh;
+    }
+    if (col >= 0 && slot >= 0 && pm.ok) {
+        float *pp = p.part + (size_t)slot * gat_bwd_pw(p.HF, H);
+        T.store_nt(pp + pm.eoff);
+        P.store_nt(pp + p.HF + pm.eoff);
+        if (pm.eoff % p.F == 0) pp[2 * p.HF + pm.hd] = z;
+    }
+}
+
 template <int VEC, int R>
 __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_merge_kernel(GatBwdP p, const fgnn_split *split, int n_split)
 {
@@ -1147,6 +1355,26 @@ static int gat_stash_csr_order(int N, int64_t E, int H, const int32_t *row_ptr, 
     return fgnn_launch_status("gat_edge_stash_kernel");
 }
 
+// Rows narrower than a wave on graphs of short rows go to the kernels that give every lane group its own work item
+// (gat_fwd_rowpack_kernel): with a wave per item, an item of two dozen entries fills one batch of 8*G loads at best, and
+// the wave then spends as long combining its groups as gathering.  Measured on 2.4 M-node graphs, forward + backward of a
+// layer: 1 x 48 floats 9.4 -> 7.8 ms at 26 entries per row, 9.9 -> 8.3 ms at 48, 7.7 -> 7.3 ms at 128, but 4.6 -> 4.8 ms
+// at 492 (there the gathered rows hit L2 and the pair layout's single pass over the scores wins); 4 x 32 floats (two
+// groups) 15.7 -> 15.1 ms at 26 entries per row, 13.9 -> 14.5 ms at 128.
+static inline bool gat_rowpack_wanted(int pack, int64_t E, int N)
+{
+    return E < (pack >= 4 ? 256 : 64) * (int64_t)N;
+}
+// Grid of those kernels: one wave per G slots of the list, the slots of a wave from one source bucket when the list is
+// XCD-aware (its length is then a multiple of 8 * FGNN_WPB).
+static inline unsigned gat_rowpack_grid(int n_items, int pack, bool bucketed)
+{
+    const int64_t waves = ((int64_t)n_items + pack - 1) / pack;
+    unsigned grid = (unsigned)((waves + FGNN_WPB - 1) / FGNN_WPB);
+    if (bucketed) grid = (grid + FGNN_NUM_XCD - 1) / FGNN_NUM_XCD * FGNN_NUM_XCD;
+    return grid;
+}
+
 static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_row, const float *attn_col,
                               const int32_t *row_ptr, const int32_t *col_ind, float slope, const float *in_feat,
                               float *out, float *edge_max, float *edge_sum, float *aux_out2, float *aux_c,
@@ -1179,7 +1407,17 @@ static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_
             while ((1 << p.hp_shift) < H) ++p.hp_shift;
             // the pair layout needs 8*G entry slots x heads (rounded up to a power of two) <= 64 lanes
             const bool pair = ((8 * pack) << p.hp_shift) <= 64 && E >= 64 * (int64_t)N;
+            const bool rowpack = gat_rowpack_wanted(pack, E, N);
+            const int bucketed = sched && sched->n_buckets > 0;
+            const unsigned grid_rp = gat_rowpack_grid(p.n_items, pack, bucketed);
             auto launch = [&]<int G>() {
+                if (rowpack) {
+                    if (aux && sle1) hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, true, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
+                    else if (aux) hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, true, false>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
+                    else if (sle1) hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, false, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
+                    else hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, false, false>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
+                    return;
+                }
                 auto go = [&]<bool PAIR>() {
                     if (aux && sle1) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, true, PAIR>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
                     else if (aux) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, false, PAIR>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
@@ -1435,7 +1673,17 @@ static int gat_backward_impl(int N, int64_t E, int H, int F, float negative_slop
             p.hp_shift = 0;
             while ((1 << p.hp_shift) < H) ++p.hp_shift;
             const bool pair = ((8 * pack) << p.hp_shift) <= 64 && E >= 64 * (int64_t)N;
+            const bool rowpack = gat_rowpack_wanted(pack, E, N);
+            const int bucketed = sched_csc && sched_csc->n_buckets > 0;
+            const unsigned grid_rp = gat_rowpack_grid(p.n_items, pack, bucketed);
             auto launch = [&]<int G>() {
+                if (rowpack) {
+                    if (stash_mode == 2) hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 2, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
+                    else if (stash_mode == 1) hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 1, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
+                    else if (sle1) hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 0, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
+                    else hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 0, false>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
+                    return;
+                }
                 auto go = [&]<bool PAIR>() {
                     if (stash_mode == 2) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 2, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
                     else if (stash_mode == 1) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 1, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);

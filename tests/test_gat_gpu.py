@@ -79,6 +79,21 @@ def test_gat_rows_narrower_than_a_wave(h, f, variant, monkeypatch):
     _lib.clear_schedule_cache()
 
 
+def _long_row_graph(seed):
+    """300 rows: the degrees of degree_edge_graph (0 ... 513 and a hub of 3000) and 280 rows of 256..300 DISTINCT sources
+    (a row that names a source many times makes the rounding errors of the per-node terms add up in step, which the
+    sum-of-magnitudes bar of these tests does not model)."""
+    import numpy as np
+    gen = np.random.default_rng(seed)
+    base = degree_edge_graph(n=20, seed=seed)
+    rows = []
+    for i in range(20):
+        d = int(base.row_ptr[i + 1] - base.row_ptr[i])
+        rows.append(list(gen.choice(300, size=d, replace=False) if d <= 300 else gen.integers(0, 300, size=d)))
+    rows += [list(gen.choice(300, size=int(gen.integers(256, 301)), replace=False)) for _ in range(280)]
+    return custom_graph(rows, 300)
+
+
 @pytest.mark.parametrize("variant", ["sm", "stash"])
 @pytest.mark.parametrize("h,f", [(8, 32), (4, 64), (1, 256), (2, 72), (5, 52), (16, 32), (16, 16), (3, 50), (7, 36), (64, 16), (33, 31),
                                  (1, 128), (1, 44), (1, 64), (2, 64), (2, 24), (1, 16), (1, 32), (3, 40), (4, 16), (1, 4)])
@@ -89,14 +104,39 @@ def test_gat_long_rows_pair_layout(h, f, variant, monkeypatch):
     wide rows and in the packed ones for H*F <= 128.  Degrees 0..3000 with ragged batch tails, whole and
     split rows, and an XCD-aware schedule."""
     from ae_mlsys_gnn_amd import _lib
-    g = degree_edge_graph(n=80, seed=21)
-    assert g.n_edges >= 64 * g.n
+    g = _long_row_graph(seed=21)
+    assert g.n_edges >= 256 * g.n          # below 256 entries per row the packed widths take the kernels of the next test
     _run(g, h, f, variant=variant)
     monkeypatch.setenv("FGNN_SEG_LEN", "256")
     monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
     monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
     _lib.clear_schedule_cache()
-    _run(degree_edge_graph(n=75, seed=22), h, f, variant=variant)
+    _run(_long_row_graph(seed=22), h, f, variant=variant)
+    _lib.clear_schedule_cache()
+
+
+@pytest.mark.parametrize("variant", ["sm", "stash"])
+@pytest.mark.parametrize("h,f", [(1, 47), (1, 16), (8, 4), (2, 12), (1, 4), (1, 64), (3, 20), (2, 32), (4, 16), (1, 128), (5, 24), (4, 32), (8, 16)])
+def test_gat_lane_groups_on_their_own_items(h, f, variant, monkeypatch):
+    """H*F <= 128 on graphs of short rows (under 256 entries per row for 8 or 4 lane groups, under 64 for 2): every
+    lane group of a wave walks a work item of its own.  Groups of 8, 16 and 32 lanes; heads of a power of two of
+    lanes and of 3, 5, 6 and 12 lanes; whole rows of 0..3000 entries side by side in one wave, split rows, XCD-aware
+    lists whose groups take their items from one bucket, a list shorter than one wave's groups, and a slope above 1."""
+    from ae_mlsys_gnn_amd import _lib
+    _lib.clear_schedule_cache()
+    _run(degree_edge_graph(seed=41), h, f, variant=variant)
+    _run(custom_graph([[0, 1], [], [2]], 3), h, f, variant=variant)
+    _run(degree_edge_graph(seed=44), h, f, variant=variant, slope=1.5)
+    monkeypatch.setenv("FGNN_SEG_LEN", "256")
+    _lib.clear_schedule_cache()
+    g = degree_edge_graph(n=140, seed=42)
+    assert 32 * g.n <= g.n_edges < 64 * g.n
+    _run(g, h, f, variant=variant)
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
+    monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+    _lib.clear_schedule_cache()
+    _run(graphs.rmat_graph(2000, 60000, seed=43), h, f, variant=variant)
+    _run(degree_edge_graph(n=150, seed=45), h, f, variant=variant)
     _lib.clear_schedule_cache()
 
 

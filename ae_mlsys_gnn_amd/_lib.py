@@ -36,6 +36,7 @@ _SIGNATURES = {
     "fgnn_schedule_num_edges": (c_int64, [c_void_p]),
     "fgnn_schedule_device_bytes": (c_size_t, [c_void_p]),
     "fgnn_schedule_num_splits": (c_int, [c_void_p]),
+    "fgnn_schedule_num_wave_slots": (c_int, [c_void_p]),
     "fgnn_schedule_export": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p]),
     "fgnn_validate_graph": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int64, c_void_p]),
     "fgnn_row_length_stats": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p]),
@@ -188,6 +189,7 @@ class Schedule:
         self.n_items = lib().fgnn_schedule_num_items(handle)
         self.n_buckets = lib().fgnn_schedule_num_buckets(handle)     # 0: plain list (also when the device lacks the XCD mapping)
         self.n_partials = lib().fgnn_schedule_num_partials(handle)
+        self.n_wave_slots = lib().fgnn_schedule_num_wave_slots(handle)   # items from this slot on have at most 64 entries
         self.n_edges = lib().fgnn_schedule_num_edges(handle)
         self.own_order = False
 

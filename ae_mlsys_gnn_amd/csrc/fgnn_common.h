@@ -76,7 +76,12 @@ struct fgnn_schedule {
     int32_t *bidx_dev;
     int32_t *bpos_dev;      // original position of every bucket-ordered entry (for per-edge arrays)
     int own_order;          // the position map was handed to the caller: per-edge arrays come in the schedule's entry order
+    // Every item at a slot >= n_wave_slots has at most FGNN_GROUP_ITEM_MAX entries (the lists are sorted longest first, so the
+    // long items are a prefix).  A multiple of 64 slots per source bucket, or n_items.  Kernels that give each lane group of a
+    // wave its own item start there; the prefix goes to the kernels that put a whole wave on an item.
+    int n_wave_slots;
 };
+#define FGNN_GROUP_ITEM_MAX 64
 // The index array a kernel walks under schedule `s`, and the map from its positions back to the
 // caller's edge positions (NULL = identity).
 static inline const int32_t *fgnn_sched_idx(const fgnn_schedule *s, const int32_t *idx) { return (s && s->n_buckets > 0) ? s->bidx_dev : idx; }
@@ -268,6 +273,29 @@ __device__ __forceinline__ bool fg_get_item(const fgnn_item *items, int n_items,
         row = item; b = fg_uni(ptr[item]); e = fg_uni(ptr[item + 1]); slot = -1;
     }
     return true;
+}
+
+// The slot of a work list that lane group g of the wave takes when every group has an item of its own: the G slots of a
+// wave are consecutive among the slots of ONE source bucket (slot ((k / WPB) * 8 + b) * WPB + k % WPB is the k-th slot of
+// bucket b in an XCD-aware list, and workgroup w runs on XCD w % 8); in a plain list they are simply consecutive.
+// `first`: the slot the launch starts at (fgnn_schedule::n_wave_slots).
+__device__ __forceinline__ int fg_group_slot(int G, int g, int bucketed, int first)
+{
+    const int w = (int)blockIdx.x, v = fg_wave();
+    if (!bucketed) return first + (w * FGNN_WPB + v) * G + g;
+    const int b = w % FGNN_NUM_XCD, k = first / FGNN_NUM_XCD + ((w / FGNN_NUM_XCD) * FGNN_WPB + v) * G + g;
+    return ((k / FGNN_WPB) * FGNN_NUM_XCD + b) * FGNN_WPB + k % FGNN_WPB;
+}
+
+// Grid of the kernels that give every lane group of a wave its own work item (fg_group_slot): one wave per `pack` slots of
+// the list, the slots of a wave from one source bucket when the list is XCD-aware (its length is then a multiple of
+// 8 * FGNN_WPB).
+static inline unsigned fgnn_group_item_grid(int n_items, int pack, bool bucketed)
+{
+    const int64_t waves = ((int64_t)n_items + pack - 1) / pack;
+    unsigned grid = (unsigned)((waves + FGNN_WPB - 1) / FGNN_WPB);
+    if (bucketed) grid = (grid + FGNN_NUM_XCD - 1) / FGNN_NUM_XCD * FGNN_NUM_XCD;
+    return grid;
 }
 
 // Weighted accumulation of up to 64 gathered feature rows with the weights staged in LDS (the

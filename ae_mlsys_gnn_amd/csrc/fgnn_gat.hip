@@ -444,22 +444,11 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_packed_kernel(GatFwdP p)
     }
 }
 
-// The slot of a work list that lane group g of the wave takes when every group has an item of its own: the G slots of a
-// wave are consecutive among the slots of ONE source bucket (slot ((k / WPB) * 8 + b) * WPB + k % WPB is the k-th slot of
-// bucket b in an XCD-aware list, and workgroup w runs on XCD w % 8); in a plain list they are simply consecutive.
-__device__ __forceinline__ int gat_group_slot(int G, int g, int bucketed)
-{
-    const int w = (int)blockIdx.x, v = fg_wave();
-    if (!bucketed) return (w * FGNN_WPB + v) * G + g;
-    const int b = w % FGNN_NUM_XCD, k = ((w / FGNN_NUM_XCD) * FGNN_WPB + v) * G + g;
-    return ((k / FGNN_WPB) * FGNN_NUM_XCD + b) * FGNN_WPB + k % FGNN_WPB;
-}
-
 // The packed forward with the lane groups on DIFFERENT items: group g of a wave takes a work item of its own and walks it
 // alone (its LPR lanes fetch LPR ids at a time, eight gathered rows of the group in flight), so one load instruction
 // fetches a row for each of G destinations and nothing is combined at the end.  Per-lane scores (no pair layout).
 template <int G, bool AUX, bool SLE1>
-__global__ __launch_bounds__(FGNN_TPB) void gat_fwd_rowpack_kernel(GatFwdP p, int bucketed)
+__global__ __launch_bounds__(FGNN_TPB) void gat_fwd_rowpack_kernel(GatFwdP p, int bucketed, int first)
 {
     constexpr int LPR = 64 / G, U = 8;
     const int lane = fg_lane();
@@ -467,7 +456,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_rowpack_kernel(GatFwdP p, in
     fg_packmap<G> pm;
     pm.init(lane, p.HF, p.F);
     const int sl = lane & (LPR - 1), gbase = lane - sl;
-    const int it = gat_group_slot(G, pm.grp, bucketed);
+    const int it = fg_group_slot(G, pm.grp, bucketed, first);
     int row = -1, b = 0, e = 0, slot = -1;
     if (it < p.n_items) {
         if (p.items) { const fgnn_item q = p.items[it]; row = q.row; b = q.begin; e = q.end; slot = q.slot; }
@@ -1160,7 +1149,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
 // The column pass with the lane groups on different items (see gat_fwd_rowpack_kernel).  T, P and z of an item stay inside
 // its group; the per-head dot product of the epilogue is reduced inside the group as well (no LDS).
 template <int G, int STASH, bool SLE1>
-__global__ __launch_bounds__(FGNN_TPB) void gat_bwd_rowpack_kernel(GatBwdP p, int bucketed)
+__global__ __launch_bounds__(FGNN_TPB) void gat_bwd_rowpack_kernel(GatBwdP p, int bucketed, int first)
 {
     constexpr int LPR = 64 / G, U = 8;
     const int lane = fg_lane();
@@ -1168,7 +1157,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_rowpack_kernel(GatBwdP p, in
     fg_packmap<G> pm;
     pm.init(lane, p.HF, p.F);
     const int sl = lane & (LPR - 1), gbase = lane - sl;
-    const int it = gat_group_slot(G, pm.grp, bucketed);
+    const int it = fg_group_slot(G, pm.grp, bucketed, first);
     int col = -1, b = 0, e = 0, slot = -1;
     if (it < p.n_items) {
         if (p.items) { const fgnn_item q = p.items[it]; col = q.row; b = q.begin; e = q.end; slot = q.slot; }
@@ -1365,16 +1354,6 @@ static inline bool gat_rowpack_wanted(int pack, int64_t E, int N)
 {
     return E < (pack >= 4 ? 256 : 64) * (int64_t)N;
 }
-// Grid of those kernels: one wave per G slots of the list, the slots of a wave from one source bucket when the list is
-// XCD-aware (its length is then a multiple of 8 * FGNN_WPB).
-static inline unsigned gat_rowpack_grid(int n_items, int pack, bool bucketed)
-{
-    const int64_t waves = ((int64_t)n_items + pack - 1) / pack;
-    unsigned grid = (unsigned)((waves + FGNN_WPB - 1) / FGNN_WPB);
-    if (bucketed) grid = (grid + FGNN_NUM_XCD - 1) / FGNN_NUM_XCD * FGNN_NUM_XCD;
-    return grid;
-}
-
 static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_row, const float *attn_col,
                               const int32_t *row_ptr, const int32_t *col_ind, float slope, const float *in_feat,
                               float *out, float *edge_max, float *edge_sum, float *aux_out2, float *aux_c,
@@ -1407,22 +1386,26 @@ static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_
             while ((1 << p.hp_shift) < H) ++p.hp_shift;
             // the pair layout needs 8*G entry slots x heads (rounded up to a power of two) <= 64 lanes
             const bool pair = ((8 * pack) << p.hp_shift) <= 64 && E >= 64 * (int64_t)N;
-            const bool rowpack = gat_rowpack_wanted(pack, E, N);
+            // the long items at the head of the list keep a wave each; the rest go four (G) to a wave on graphs of short rows
+            const int first = sched && gat_rowpack_wanted(pack, E, N) ? sched->n_wave_slots : p.n_items;
             const int bucketed = sched && sched->n_buckets > 0;
-            const unsigned grid_rp = gat_rowpack_grid(p.n_items, pack, bucketed);
+            const unsigned grid_rp = fgnn_group_item_grid(p.n_items - first, pack, bucketed);
+            GatFwdP pw = p;
+            pw.n_items = first;
+            const unsigned grid_w = (unsigned)((first + FGNN_WPB - 1) / FGNN_WPB);
             auto launch = [&]<int G>() {
-                if (rowpack) {
-                    if (aux && sle1) hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, true, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
-                    else if (aux) hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, true, false>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
-                    else if (sle1) hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, false, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
-                    else hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, false, false>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
-                    return;
+                if (first < p.n_items) {
+                    if (aux && sle1) hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, true, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
+                    else if (aux) hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, true, false>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
+                    else if (sle1) hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, false, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
+                    else hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, false, false>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
                 }
+                if (first == 0) return;
                 auto go = [&]<bool PAIR>() {
-                    if (aux && sle1) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, true, PAIR>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
-                    else if (aux) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, false, PAIR>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
-                    else if (sle1) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, false, true, PAIR>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
-                    else hipLaunchKernelGGL((gat_fwd_packed_kernel<G, false, false, PAIR>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
+                    if (aux && sle1) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, true, PAIR>), dim3(grid_w), dim3(FGNN_TPB), 0, st, pw);
+                    else if (aux) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, false, PAIR>), dim3(grid_w), dim3(FGNN_TPB), 0, st, pw);
+                    else if (sle1) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, false, true, PAIR>), dim3(grid_w), dim3(FGNN_TPB), 0, st, pw);
+                    else hipLaunchKernelGGL((gat_fwd_packed_kernel<G, false, false, PAIR>), dim3(grid_w), dim3(FGNN_TPB), 0, st, pw);
                 };
                 if (pair) go.template operator()<true>(); else go.template operator()<false>();
             };
@@ -1673,22 +1656,25 @@ static int gat_backward_impl(int N, int64_t E, int H, int F, float negative_slop
             p.hp_shift = 0;
             while ((1 << p.hp_shift) < H) ++p.hp_shift;
             const bool pair = ((8 * pack) << p.hp_shift) <= 64 && E >= 64 * (int64_t)N;
-            const bool rowpack = gat_rowpack_wanted(pack, E, N);
+            const int first = sched_csc && gat_rowpack_wanted(pack, E, N) ? sched_csc->n_wave_slots : p.n_items;      // as in the forward
             const int bucketed = sched_csc && sched_csc->n_buckets > 0;
-            const unsigned grid_rp = gat_rowpack_grid(p.n_items, pack, bucketed);
+            const unsigned grid_rp = fgnn_group_item_grid(p.n_items - first, pack, bucketed);
+            GatBwdP pw = p;
+            pw.n_items = first;
+            const unsigned grid_w = (unsigned)((first + FGNN_WPB - 1) / FGNN_WPB);
             auto launch = [&]<int G>() {
-                if (rowpack) {
-                    if (stash_mode == 2) hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 2, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
-                    else if (stash_mode == 1) hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 1, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
-                    else if (sle1) hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 0, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
-                    else hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 0, false>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed);
-                    return;
+                if (first < p.n_items) {
+                    if (stash_mode == 2) hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 2, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
+                    else if (stash_mode == 1) hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 1, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
+                    else if (sle1) hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 0, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
+                    else hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 0, false>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
                 }
+                if (first == 0) return;
                 auto go = [&]<bool PAIR>() {
-                    if (stash_mode == 2) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 2, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
-                    else if (stash_mode == 1) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 1, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
-                    else if (sle1) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 0, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
-                    else hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 0, false, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                    if (stash_mode == 2) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 2, true, PAIR>), dim3(grid_w), dim3(FGNN_TPB), shm, st, pw);
+                    else if (stash_mode == 1) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 1, true, PAIR>), dim3(grid_w), dim3(FGNN_TPB), shm, st, pw);
+                    else if (sle1) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 0, true, PAIR>), dim3(grid_w), dim3(FGNN_TPB), shm, st, pw);
+                    else hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 0, false, PAIR>), dim3(grid_w), dim3(FGNN_TPB), shm, st, pw);
                 };
                 if (pair) go.template operator()<true>(); else go.template operator()<false>();
             };

@@ -93,6 +93,41 @@ static void sort_longest_first(std::vector<fgnn_item> &v, size_t first = 0)
     std::copy(sorted.begin(), sorted.end(), v.begin() + first);
 }
 
+// k + 1 for the last slot k (counted per source bucket in an XCD-aware list) that holds an item of more than `limit` entries
+__global__ __launch_bounds__(256) void sched_long_prefix_kernel(int n_items, const fgnn_item *__restrict__ items, int bucketed, int limit,
+                                                                int *__restrict__ out)
+{
+    const int i = (int)(blockIdx.x * 256 + threadIdx.x);
+    if (i >= n_items) return;
+    const fgnn_item it = items[i];
+    if (it.row < 0 || it.end - it.begin <= limit) return;
+    const int k = bucketed ? (i / (FGNN_NUM_XCD * FGNN_WPB)) * FGNN_WPB + i % FGNN_WPB : i;
+    atomicMax(out, k + 1);
+}
+
+// Sets s->n_wave_slots from the finished item array (one more read-back of one int).
+static int schedule_mark_long_prefix(fgnn_schedule *s, hipStream_t st)
+{
+    s->n_wave_slots = 0;
+    if (s->n_items == 0) return 0;
+    int *dev = nullptr, last = 0;
+    FGNN_HIP(hipMalloc((void **)&dev, sizeof(int)));
+    hipError_t err = hipMemcpyAsync(dev, &last, sizeof(int), hipMemcpyHostToDevice, st);
+    if (err == hipSuccess) {
+        hipLaunchKernelGGL(sched_long_prefix_kernel, dim3((unsigned)((s->n_items + 255) / 256)), dim3(256), 0, st, s->n_items, s->items_dev,
+                           s->n_buckets > 0 ? 1 : 0, FGNN_GROUP_ITEM_MAX, dev);
+        err = hipGetLastError();
+    }
+    if (err == hipSuccess) err = hipMemcpyAsync(&last, dev, sizeof(int), hipMemcpyDeviceToHost, st);
+    if (err == hipSuccess) err = hipStreamSynchronize(st);
+    (void)hipFree(dev);
+    if (err != hipSuccess) { fgnn_set_error("schedule: %s", hipGetErrorString(err)); return (int)err; }
+    const int64_t per = s->n_buckets > 0 ? FGNN_NUM_XCD : 1;
+    const int64_t slots = ((int64_t)last + 63) / 64 * 64 * per;
+    s->n_wave_slots = (int)std::min<int64_t>(slots, s->n_items);
+    return 0;
+}
+
 static int upload_schedule(fgnn_schedule *s, const std::vector<fgnn_item> &items, const std::vector<fgnn_split> &splits, hipStream_t st)
 {
     hipError_t err = hipSuccess;
@@ -109,7 +144,7 @@ static int upload_schedule(fgnn_schedule *s, const std::vector<fgnn_item> &items
         fgnn_set_error("schedule upload: %s", hipGetErrorString(err));
         return (int)err;
     }
-    return 0;
+    return schedule_mark_long_prefix(s, st);
 }
 
 static int read_ptr(const int32_t *ptr_dev, int n_rows, hipStream_t st, std::vector<int32_t> &ptr)
@@ -129,7 +164,7 @@ static fgnn_schedule *new_schedule(const int32_t *ptr_dev, int n_rows, int64_t n
     s->n_rows = n_rows; s->n_edges = n_edges; s->seg_len = seg_len;
     s->n_items = s->n_partials = s->n_split = 0;
     s->items_dev = nullptr; s->split_dev = nullptr; s->ptr_dev = ptr_dev;
-    s->n_buckets = 0; s->idx_src_dev = nullptr; s->bidx_dev = nullptr; s->bpos_dev = nullptr; s->own_order = 0;
+    s->n_buckets = 0; s->idx_src_dev = nullptr; s->bidx_dev = nullptr; s->bpos_dev = nullptr; s->own_order = 0; s->n_wave_slots = 0;
     (void)hipGetDevice(&s->device);
     return s;
 }
@@ -477,6 +512,7 @@ static int schedule_build_device(fgnn_schedule *s, const int32_t *ptr_dev, const
     SCHED_HIP(hipStreamSynchronize(st));          // the temporaries are freed below
     if (tmp2) (void)hipFree(tmp2);
     (void)hipFree(tmp1);
+    if (!rc) rc = schedule_mark_long_prefix(s, st);
     return rc;
 }
 
@@ -608,6 +644,7 @@ extern "C" int fgnn_schedule_export(const fgnn_schedule_t *s, int32_t *items_out
     return 0;
 }
 extern "C" int fgnn_schedule_num_splits(const fgnn_schedule_t *s) { return s ? s->n_split : 0; }
+extern "C" int fgnn_schedule_num_wave_slots(const fgnn_schedule_t *s) { return s ? s->n_wave_slots : 0; }
 
 __global__ __launch_bounds__(256) void iota_i32_kernel(int64_t n, int *__restrict__ out)
 {

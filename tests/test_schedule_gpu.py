@@ -20,7 +20,8 @@ def _both(monkeypatch, ptr, idx, seg_len, min_deg, with_positions=True):
         s = _lib.Schedule(ptr, seg_len, idx, min_deg, with_positions=with_positions)
         items, splits = s.export()
         pos = s.take_positions() if (idx is not None and with_positions) else None
-        out.append((s.n_items, s.n_partials, s.n_edges, items.cpu(), splits.cpu(), None if pos is None else pos.cpu(), s.device_bytes()))
+        out.append((s.n_items, s.n_partials, s.n_edges, items.cpu(), splits.cpu(), None if pos is None else pos.cpu(), s.device_bytes(),
+                    s.n_wave_slots, s.n_buckets))
     monkeypatch.delenv("FGNN_SCHEDULE_BUILDER")
     return out
 
@@ -47,6 +48,18 @@ def test_device_built_schedules_equal_the_host_built_ones(name, seg_len, min_deg
         if idx is not None:
             assert torch.equal(dev[5], host[5]), "position maps differ"
         assert dev[6] == host[6]
+        # the long items are a prefix of the list: nothing longer than 64 entries from slot n_wave_slots on, and the mark
+        # is tight to the 64 slots (per source bucket) it is rounded up to
+        for n_wave, n_buckets, items in ((dev[7], dev[8], dev[3]), (host[7], host[8], host[3])):
+            length = (items[:, 2] - items[:, 1]) * (items[:, 0] >= 0)
+            per = 64 * max(n_buckets, 1)
+            assert 0 <= n_wave <= len(items) and (n_wave % per == 0 or n_wave == len(items))
+            assert n_wave == len(items) or int(length[n_wave:].max()) <= 64
+            if n_wave > 0:
+                assert int(length[max(n_wave - per, 0):n_wave].max()) > 64 or n_wave == len(items)
+            else:
+                assert len(items) == 0 or int(length.max()) <= 64
+        assert dev[7] == host[7]
         # the list covers every entry exactly once
         it = dev[3][dev[3][:, 0] >= 0].long()
         assert int((it[:, 2] - it[:, 1]).sum()) == g.n_edges

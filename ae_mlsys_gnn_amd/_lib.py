@@ -419,11 +419,61 @@ def schedule_device_bytes() -> int:
         return sum(s.device_bytes() for s in _sched_cache.values()) + sum(p.device_bytes() for p in _colsum_cache.values())
 
 
+_own_view_cache: "collections.OrderedDict" = collections.OrderedDict()
+_OWN_VIEW_CACHE_MAX = 4
+
+
+def _gather_i32(src, index):
+    """src[index] for int32 device vectors, by the library's row-gather kernel (the words move as they are)."""
+    out = torch.empty_like(index)
+    if index.numel():
+        with torch.cuda.device(src.device):
+            check(lib().fgnn_gather_rows(index.numel(), 1, ptr(index), ptr(src), ptr(out), stream_ptr()), "fgnn_gather_rows")
+    return out
+
+
+def own_order_view(row_ptr, col_ind, col_ptr, row_ind, permute):
+    """(col_ind_own, permute_own) for pipelines that keep their per-edge tensors in the ENTRY ORDER of the work lists:
+    col_ind_own is col_ind in the order the CSR-side list walks the entries (an XCD-aware list regroups the entries of a row
+    by source bucket, so (row_ptr, col_ind_own) is a CSR of the same graph), and permute_own[q] is the position in that
+    order of the entry that the CSC-side list walks q-th.  Operators called with own_order=True then read and write [E,H]
+    tensors as contiguous runs; with plain lists on both sides the caller's arrays come back.  Built once per set of
+    arrays and cached with the two own-order schedules (the cache holds the tensors)."""
+    key = tuple((t.data_ptr(), t.numel(), t._version) for t in (row_ptr, col_ind, col_ptr, row_ind, permute)) + (
+        row_ptr.device.index, default_seg_len(), os.environ.get("FGNN_BUCKET_MIN_DEG", "0"), os.environ.get("FGNN_XCD_BUCKETS"))
+    with _cache_lock:
+        hit = _own_view_cache.get(key)
+        if hit is not None:
+            _own_view_cache.move_to_end(key)
+            return hit[0], hit[1]
+    pos_r = edge_positions(row_ptr, col_ind)
+    pos_c = edge_positions(col_ptr, row_ind)
+    perm = permute if pos_c is None else _gather_i32(permute, pos_c)
+    if pos_r is None:
+        idx_own, perm_own = col_ind, perm
+    else:
+        idx_own = _gather_i32(col_ind, pos_r)
+        e = pos_r.numel()
+        iota = torch.arange(e, dtype=torch.int32, device=pos_r.device)
+        inv = torch.empty_like(pos_r)
+        inv.scatter_(0, pos_r.long(), iota)
+        if not torch.equal(_gather_i32(inv, pos_r), iota):
+            raise FgnnError("own_order_view: the position map of the work list is not a permutation")
+        perm_own = _gather_i32(inv, perm)
+        del inv, iota
+    with _cache_lock:
+        _own_view_cache[key] = (idx_own, perm_own, (row_ptr, col_ind, col_ptr, row_ind, permute))
+        while len(_own_view_cache) > _OWN_VIEW_CACHE_MAX:
+            _own_view_cache.popitem(last=False)
+    return idx_own, perm_own
+
+
 def clear_schedule_cache():
     with _cache_lock:
         _sched_cache.clear()
         _bucket_rule_cache.clear()
         _colsum_cache.clear()
+        _own_view_cache.clear()
 
 
 def workspace(nbytes: int, device):

@@ -158,7 +158,8 @@ static int mhsddmm_run(const char *fn, int N, int64_t E, int H, int F, const int
                      "%s: schedule was built for another pointer array", fn);
         FGNN_REQUIRE(sched->n_buckets == 0 || sched->idx_src_dev == col_ind, FGNN_ERR_SCHEDULE,
                      "%s: XCD-aware schedule was built from another index array", fn);
-        FGNN_REQUIRE(fgnn_sched_has_pos(sched) && !sched->own_order, FGNN_ERR_SCHEDULE,
+        // a list whose position map was handed to the caller (fgnn_schedule_take_positions) stores in its own entry order
+        FGNN_REQUIRE(fgnn_sched_has_pos(sched), FGNN_ERR_SCHEDULE,
                      "%s: the schedule must carry its edge positions (results are stored at the caller's positions)", fn);
     }
     if (N == 0 || E == 0) return 0;

@@ -264,23 +264,26 @@ class FusedGATFunction(torch.autograd.Function):
         from .mhspmm import mhspmm
         attn_row, attn_col, in_feat = _contig(attn_row), _contig(attn_col), _contig(in_feat)
         row_ptr, col_ind, col_ptr, row_ind, permute = _contig(row_ptr), _contig(col_ind), _contig(col_ptr), _contig(row_ind), _contig(permute)
-        _, e_soft = gat_native.gat_scatter(attn_row, attn_col, row_ptr, col_ind, negative_slope)
-        out = mhspmm(row_ptr, col_ind, e_soft, in_feat)
+        # e_softmax and the edge gradients live in the entry order of the work lists: rows keep their places, the entries
+        # of a row are regrouped by source bucket when the list is XCD-aware, so every pass below streams them
+        idx_own, perm_own = _lib.own_order_view(row_ptr, col_ind, col_ptr, row_ind, as_i32(permute))
+        _, e_soft = gat_native.gat_scatter(attn_row, attn_col, row_ptr, idx_own, negative_slope)
+        out = mhspmm(row_ptr, col_ind, e_soft, in_feat, own_order=True)
         if _needs_grad(ctx):
-            ctx.save_for_backward(row_ptr, col_ind, col_ptr, row_ind, permute, e_soft, in_feat, attn_row, attn_col)
+            ctx.save_for_backward(row_ptr, col_ind, col_ptr, row_ind, idx_own, perm_own, e_soft, in_feat, attn_row, attn_col)
         ctx.negative_slope = negative_slope
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
         from .mhspmm import mhsddmm, mhspmm
-        row_ptr, col_ind, col_ptr, row_ind, permute, e_soft, in_feat, attn_row, attn_col = ctx.saved_tensors
+        row_ptr, col_ind, col_ptr, row_ind, idx_own, perm_own, e_soft, in_feat, attn_row, attn_col = ctx.saved_tensors
         grad_out = grad_out.contiguous()
-        grad_feat = mhspmm(col_ptr, row_ind, e_soft, grad_out, pos_map=as_i32(permute))
-        grad_edge = mhsddmm(row_ptr, col_ind, grad_out, in_feat)
-        grad_edge, grad_attn_row = gat_native.gat_gather_row(ctx.negative_slope, row_ptr, col_ind, attn_row, attn_col, e_soft, grad_edge, inplace=True)
+        grad_feat = mhspmm(col_ptr, row_ind, e_soft, grad_out, pos_map=perm_own, own_order=True)
+        grad_edge = mhsddmm(row_ptr, col_ind, grad_out, in_feat, own_order=True)
+        grad_edge, grad_attn_row = gat_native.gat_gather_row(ctx.negative_slope, row_ptr, idx_own, attn_row, attn_col, e_soft, grad_edge, inplace=True)
         n, h = attn_row.shape
-        grad_attn_col = colsum_plan_for(row_ptr, col_ind, n, h).colsum(grad_edge)
+        grad_attn_col = colsum_plan_for(row_ptr, idx_own, n, h).colsum(grad_edge)
         return grad_attn_row, grad_attn_col, None, None, None, None, None, grad_feat, None
 
 

@@ -6,8 +6,10 @@ import torch
 from .._lib import FgnnError, as_f32, as_i32, check, lib, ptr, require_cuda, schedule_for, stream_ptr, workspace, xcd_buckets_enabled
 
 
-def mhspmm(ptr_arr, idx, attention, feat, pos_map=None):
-    """mhspmm.mhspmm(rowptr, colind, attention, feat) (src/spmm/mhspmm.cc): out[i,h,:] = sum_p att[p,h]*feat[idx[p],h,:]."""
+def mhspmm(ptr_arr, idx, attention, feat, pos_map=None, own_order=False):
+    """mhspmm.mhspmm(rowptr, colind, attention, feat) (src/spmm/mhspmm.cc): out[i,h,:] = sum_p att[p,h]*feat[idx[p],h,:].
+    own_order: attention (or pos_map, when given) is indexed by the entry order of the work list of (ptr_arr, idx)
+    (_lib.own_order_view), not by the caller's positions."""
     require_cuda(ptr_arr, idx, feat)
     ptr_arr, idx, feat = as_i32(ptr_arr), as_i32(idx), as_f32(feat)
     attention = None if attention is None else as_f32(attention)
@@ -21,7 +23,7 @@ def mhspmm(ptr_arr, idx, attention, feat, pos_map=None):
     if attention is not None and attention.shape != (e, h):
         raise FgnnError("mhspmm: attention is %s, expected (%d, %d)" % (tuple(attention.shape), e, h))
     out = torch.empty((ptr_arr.numel() - 1, h, f), dtype=torch.float32, device=feat.device)
-    sched = schedule_for(ptr_arr, idx_tensor=idx, n_cols=n)          # the ids index the rows of feat
+    sched = schedule_for(ptr_arr, idx_tensor=idx, n_cols=n, own_order=own_order)          # the ids index the rows of feat
     with torch.cuda.device(feat.device):
         # unweighted: only the partial results of split rows (the same figure as the GMMConv forward's)
         need = (lib().fgnn_mhspmm_workspace_bytes if attention is not None else lib().fgnn_gmm_forward_workspace_bytes)(sched.handle, h, f)
@@ -31,8 +33,9 @@ def mhspmm(ptr_arr, idx, attention, feat, pos_map=None):
     return out
 
 
-def mhsddmm(rowptr, colind, grad, feat):
-    """mhsddmm.mhsddmm (src/sddmm/mhsddmm.cc): out[p,h] = <grad[row(p),h,:], feat[colind[p],h,:]>."""
+def mhsddmm(rowptr, colind, grad, feat, own_order=False):
+    """mhsddmm.mhsddmm (src/sddmm/mhsddmm.cc): out[p,h] = <grad[row(p),h,:], feat[colind[p],h,:]>.
+    own_order: the result is written in the entry order of the work list of (rowptr, colind) (_lib.own_order_view)."""
     require_cuda(rowptr, colind, grad, feat)
     rowptr, colind, grad, feat = as_i32(rowptr), as_i32(colind), as_f32(grad), as_f32(feat)
     n, h, f = feat.shape
@@ -40,7 +43,7 @@ def mhsddmm(rowptr, colind, grad, feat):
     out = torch.empty((e, h), dtype=torch.float32, device=feat.device)
     # a skewed graph is walked under its XCD-aware work list (each XCD then gathers from one eighth of the feature
     # rows); otherwise the kernel cuts the entry array into equal chunks itself and needs no list
-    sched = schedule_for(rowptr, idx_tensor=colind, n_cols=n) if e and xcd_buckets_enabled(rowptr, e) else None
+    sched = schedule_for(rowptr, idx_tensor=colind, n_cols=n, own_order=own_order) if e and xcd_buckets_enabled(rowptr, e) else None
     with torch.cuda.device(feat.device):
         if sched is not None:
             check(lib().fgnn_mhsddmm_scheduled(rowptr.numel() - 1, e, h, f, ptr(rowptr), ptr(colind), ptr(grad), ptr(feat), ptr(out),

@@ -355,7 +355,8 @@ int    fgnn_mhsddmm(int N, int64_t E, int H, int F, const int32_t *row_ptr, cons
                     const float *a, const float *b, float *out, void *stream);
 /* The same operator walked under a work list of (row_ptr, col_ind) that carries its edge positions (NULL = the
  * call above): with an XCD-aware list every XCD gathers from one eighth of the b-rows; results are stored at the
- * caller's CSR positions either way. */
+ * caller's CSR positions either way, unless the list's position map was handed out (fgnn_schedule_take_positions):
+ * then out is in the list's entry order, written as contiguous runs. */
 int    fgnn_mhsddmm_scheduled(int N, int64_t E, int H, int F, const int32_t *row_ptr, const int32_t *col_ind,
                               const float *a, const float *b, float *out, const fgnn_schedule_t *sched,
                               void *stream);

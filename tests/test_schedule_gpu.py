@@ -95,8 +95,9 @@ def test_row_length_statistics(name):
 
 
 def test_scheduled_sddmm_refuses_lists_it_cannot_use(monkeypatch):
-    """fgnn_mhsddmm_scheduled stores its results at the caller's positions: a list of another graph, a list built
-    without the position map and one whose map was handed out are refused before any kernel runs."""
+    """fgnn_mhsddmm_scheduled stores its results at the caller's positions: a list of another graph and a list built
+    without the position map are refused before any kernel runs; a list whose map was handed out stores in its own
+    entry order."""
     from ae_mlsys_gnn_amd import _lib
     from ae_mlsys_gnn_amd._lib import lib, ptr, stream_ptr
     g = graphs.add_csc_torch(graphs.rmat_graph(500, 20000, seed=1)).to(DEV)
@@ -118,5 +119,41 @@ def test_scheduled_sddmm_refuses_lists_it_cannot_use(monkeypatch):
     assert call(_lib.Schedule(g.row_ptr, 0, g.col_ind, 16, with_positions=False)) == -6
     assert b"edge positions" in lib().fgnn_last_error()
     taken = _lib.Schedule(g.row_ptr, 0, g.col_ind, 16, with_positions=True)
-    taken.take_positions()
-    assert call(taken) == -6 and b"edge positions" in lib().fgnn_last_error()
+    pos = taken.take_positions()
+    assert taken.n_buckets == 8 and not torch.equal(pos.cpu(), torch.arange(g.n_edges, dtype=torch.int32))
+    assert call(taken) == 0
+    assert torch.equal(out, plain[pos.long()])
+
+
+def test_own_order_view_of_a_graph(monkeypatch):
+    """_lib.own_order_view: the index array in the entry order of the CSR-side work list and the CSC-to-CSR map between the
+    two entry orders.  Per-edge tensors kept in that order give the same multi-head SpMM (through the map) and SDDMM as the
+    caller's order gives, bit for bit; rows keep their entries; the view is cached; plain lists give the arrays back."""
+    from ae_mlsys_gnn_amd import _lib
+    from ae_mlsys_gnn_amd.operators.mhspmm import mhsddmm, mhspmm
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
+    monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", "16")
+    _lib.clear_schedule_cache()
+    g = graphs.add_csc_torch(graphs.rmat_graph(1500, 90000, seed=5)).to(DEV)
+    idx_own, perm_own = _lib.own_order_view(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, g.permute)
+    pos_r = _lib.edge_positions(g.row_ptr, g.col_ind)
+    assert pos_r is not None and torch.equal(idx_own, g.col_ind[pos_r.long()])
+    rows = torch.repeat_interleave(torch.arange(g.n, device=DEV), (g.row_ptr[1:] - g.row_ptr[:-1]).long())
+    assert torch.equal(rows[pos_r.long()], rows)                       # a row's entries stay in the row
+    assert torch.equal(torch.sort(perm_own).values, torch.arange(g.n_edges, dtype=torch.int32, device=DEV))
+    again = _lib.own_order_view(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, g.permute)
+    assert again[0].data_ptr() == idx_own.data_ptr() and again[1].data_ptr() == perm_own.data_ptr()
+    h, f = 4, 16
+    torch.manual_seed(0)
+    w = torch.randn(g.n_edges, h, device=DEV)
+    a, b = torch.randn(g.n, h, f, device=DEV), torch.randn(g.n, h, f, device=DEV)
+    w_own = w[pos_r.long()].contiguous()
+    assert torch.equal(mhspmm(g.row_ptr, g.col_ind, w_own, a, own_order=True), mhspmm(g.row_ptr, g.col_ind, w, a))
+    assert torch.equal(mhspmm(g.col_ptr, g.row_ind, w_own, a, pos_map=perm_own, own_order=True),
+                       mhspmm(g.col_ptr, g.row_ind, w, a, pos_map=g.permute))
+    assert torch.equal(mhsddmm(g.row_ptr, g.col_ind, a, b, own_order=True), mhsddmm(g.row_ptr, g.col_ind, a, b)[pos_r.long()])
+    monkeypatch.setenv("FGNN_XCD_BUCKETS", "0")
+    _lib.clear_schedule_cache()
+    idx_p, perm_p = _lib.own_order_view(g.row_ptr, g.col_ind, g.col_ptr, g.row_ind, g.permute)
+    assert idx_p.data_ptr() == g.col_ind.data_ptr() and perm_p.data_ptr() == g.permute.data_ptr()
+    _lib.clear_schedule_cache()

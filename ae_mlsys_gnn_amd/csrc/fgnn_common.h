@@ -278,10 +278,12 @@ __device__ __forceinline__ bool fg_get_item(const fgnn_item *items, int n_items,
 // The slot of a work list that lane group g of the wave takes when every group has an item of its own: the G slots of a
 // wave are consecutive among the slots of ONE source bucket (slot ((k / WPB) * 8 + b) * WPB + k % WPB is the k-th slot of
 // bucket b in an XCD-aware list, and workgroup w runs on XCD w % 8); in a plain list they are simply consecutive.
-// `first`: the slot the launch starts at (fgnn_schedule::n_wave_slots).
-__device__ __forceinline__ int fg_group_slot(int G, int g, int bucketed, int first)
+// `first`: the slot the lane-group part of the launch starts at (fgnn_schedule::n_wave_slots); `w`: the workgroup's index
+// in that part (the workgroups before it take the head of the list a wave per item; their number is a multiple of 8 when the
+// list is XCD-aware, so w % 8 is still the workgroup's XCD).
+__device__ __forceinline__ int fg_group_slot(int G, int g, int bucketed, int first, int w)
 {
-    const int w = (int)blockIdx.x, v = fg_wave();
+    const int v = fg_wave();
     if (!bucketed) return first + (w * FGNN_WPB + v) * G + g;
     const int b = w % FGNN_NUM_XCD, k = first / FGNN_NUM_XCD + ((w / FGNN_NUM_XCD) * FGNN_WPB + v) * G + g;
     return ((k / FGNN_WPB) * FGNN_NUM_XCD + b) * FGNN_WPB + k % FGNN_WPB;

@@ -283,11 +283,12 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_kernel(GatFwdP p)
 // PAIR: the scores are handled in the pair layout of gat_fwd_pair_batch, one lane per (entry of the
 // batch of 8*G, head); the wave then keeps ONE running maximum per head, so the groups' accumulators
 // are plain partial sums.
+// n_head: the items this form takes (all of them, or the head of a list whose short items go to gat_fwd_rowpack_items).
 template <int G, bool AUX, bool SLE1, bool PAIR>
-__global__ __launch_bounds__(FGNN_TPB) void gat_fwd_packed_kernel(GatFwdP p)
+__device__ __forceinline__ void gat_fwd_packed_item(const GatFwdP &p, int n_head)
 {
     int row, b, e, slot;
-    if (!fg_get_item(p.items, p.n_items, p.ptr, row, b, e, slot)) return;
+    if (!fg_get_item(p.items, n_head, p.ptr, row, b, e, slot)) return;
     const int lane = fg_lane();
     const int H = p.H;
     fg_packmap<G> pm;
@@ -448,7 +449,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_packed_kernel(GatFwdP p)
 // alone (its LPR lanes fetch LPR ids at a time, eight gathered rows of the group in flight), so one load instruction
 // fetches a row for each of G destinations and nothing is combined at the end.  Per-lane scores (no pair layout).
 template <int G, bool AUX, bool SLE1>
-__global__ __launch_bounds__(FGNN_TPB) void gat_fwd_rowpack_kernel(GatFwdP p, int bucketed, int first)
+__device__ __forceinline__ void gat_fwd_rowpack_items(const GatFwdP &p, int bucketed, int first, int w)
 {
     constexpr int LPR = 64 / G, U = 8;
     const int lane = fg_lane();
@@ -456,7 +457,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_rowpack_kernel(GatFwdP p, in
     fg_packmap<G> pm;
     pm.init(lane, p.HF, p.F);
     const int sl = lane & (LPR - 1), gbase = lane - sl;
-    const int it = fg_group_slot(G, pm.grp, bucketed, first);
+    const int it = fg_group_slot(G, pm.grp, bucketed, first, w);
     int row = -1, b = 0, e = 0, slot = -1;
     if (it < p.n_items) {
         if (p.items) { const fgnn_item q = p.items[it]; row = q.row; b = q.begin; e = q.end; slot = q.slot; }
@@ -543,6 +544,21 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_rowpack_kernel(GatFwdP p, in
             st[2 * H + pm.hd] = cp * fix;
         }
     }
+}
+
+template <int G, bool AUX, bool SLE1, bool PAIR>
+__global__ __launch_bounds__(FGNN_TPB) void gat_fwd_packed_kernel(GatFwdP p)
+{
+    gat_fwd_packed_item<G, AUX, SLE1, PAIR>(p, p.n_items);
+}
+// One launch for a list with a long head: the first head_blocks workgroups put a wave on each of the `first` leading items,
+// the others give every lane group an item of the rest.  The head is launched first, so its long items run while the short
+// ones fill the rest of the machine (as two launches the second would wait for the longest item of the first).
+template <int G, bool AUX, bool SLE1, bool PAIR>
+__global__ __launch_bounds__(FGNN_TPB) void gat_fwd_mixed_kernel(GatFwdP p, int bucketed, int first, unsigned head_blocks)
+{
+    if (blockIdx.x < head_blocks) gat_fwd_packed_item<G, AUX, SLE1, PAIR>(p, first);
+    else gat_fwd_rowpack_items<G, AUX, SLE1>(p, bucketed, first, (int)(blockIdx.x - head_blocks));
 }
 
 // Merge of the segments of split rows: log-sum-exp combination of (m, s, T, P).
@@ -1031,11 +1047,10 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_kernel(GatBwdP p)
 // The column pass for rows narrower than a wave: G entries of the column per load instruction
 // (see gat_fwd_packed_kernel); T, P and z are plain sums, so the groups are added by a butterfly.
 template <int G, int STASH, bool SLE1, bool PAIR>
-__global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
+__device__ __forceinline__ void gat_bwd_packed_item(const GatBwdP &p, int n_head, float *lds)
 {
-    extern __shared__ float lds[];
     int col, b, e, slot;
-    if (!fg_get_item(p.items, p.n_items, p.ptr, col, b, e, slot)) return;
+    if (!fg_get_item(p.items, n_head, p.ptr, col, b, e, slot)) return;
     const int lane = fg_lane();
     const int H = p.H;
     float *scr = lds + fg_wave() * (64 + 64);
@@ -1146,10 +1161,10 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
     }
 }
 
-// The column pass with the lane groups on different items (see gat_fwd_rowpack_kernel).  T, P and z of an item stay inside
+// The column pass with the lane groups on different items (see gat_fwd_rowpack_items).  T, P and z of an item stay inside
 // its group; the per-head dot product of the epilogue is reduced inside the group as well (no LDS).
 template <int G, int STASH, bool SLE1>
-__global__ __launch_bounds__(FGNN_TPB) void gat_bwd_rowpack_kernel(GatBwdP p, int bucketed, int first)
+__device__ __forceinline__ void gat_bwd_rowpack_items(const GatBwdP &p, int bucketed, int first, int w)
 {
     constexpr int LPR = 64 / G, U = 8;
     const int lane = fg_lane();
@@ -1157,7 +1172,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_rowpack_kernel(GatBwdP p, in
     fg_packmap<G> pm;
     pm.init(lane, p.HF, p.F);
     const int sl = lane & (LPR - 1), gbase = lane - sl;
-    const int it = fg_group_slot(G, pm.grp, bucketed, first);
+    const int it = fg_group_slot(G, pm.grp, bucketed, first, w);
     int col = -1, b = 0, e = 0, slot = -1;
     if (it < p.n_items) {
         if (p.items) { const fgnn_item q = p.items[it]; col = q.row; b = q.begin; e = q.end; slot = q.slot; }
@@ -1240,6 +1255,21 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_rowpack_kernel(GatBwdP p, in
         P.store_nt(pp + p.HF + pm.eoff);
         if (pm.eoff % p.F == 0) pp[2 * p.HF + pm.hd] = z;
     }
+}
+
+template <int G, int STASH, bool SLE1, bool PAIR>
+__global__ __launch_bounds__(FGNN_TPB) void gat_bwd_packed_kernel(GatBwdP p)
+{
+    extern __shared__ float lds[];
+    gat_bwd_packed_item<G, STASH, SLE1, PAIR>(p, p.n_items, lds);
+}
+// Head of the list a wave per item, the rest a lane group per item, in one launch (see gat_fwd_mixed_kernel).
+template <int G, int STASH, bool SLE1, bool PAIR>
+__global__ __launch_bounds__(FGNN_TPB) void gat_bwd_mixed_kernel(GatBwdP p, int bucketed, int first, unsigned head_blocks)
+{
+    extern __shared__ float lds[];
+    if (blockIdx.x < head_blocks) gat_bwd_packed_item<G, STASH, SLE1, PAIR>(p, first, lds);
+    else gat_bwd_rowpack_items<G, STASH, SLE1>(p, bucketed, first, (int)(blockIdx.x - head_blocks));
 }
 
 template <int VEC, int R>
@@ -1344,12 +1374,13 @@ static int gat_stash_csr_order(int N, int64_t E, int H, const int32_t *row_ptr, 
     return fgnn_launch_status("gat_edge_stash_kernel");
 }
 
-// Rows narrower than a wave on graphs of short rows go to the kernels that give every lane group its own work item
-// (gat_fwd_rowpack_kernel): with a wave per item, an item of two dozen entries fills one batch of 8*G loads at best, and
-// the wave then spends as long combining its groups as gathering.  Measured on 2.4 M-node graphs, forward + backward of a
-// layer: 1 x 48 floats 9.4 -> 7.8 ms at 26 entries per row, 9.9 -> 8.3 ms at 48, 7.7 -> 7.3 ms at 128, but 4.6 -> 4.8 ms
-// at 492 (there the gathered rows hit L2 and the pair layout's single pass over the scores wins); 4 x 32 floats (two
-// groups) 15.7 -> 15.1 ms at 26 entries per row, 13.9 -> 14.5 ms at 128.
+// Rows narrower than a wave on graphs of short rows: the short items of the work list go G to a wave, every lane group on an
+// item of its own (gat_fwd_rowpack_items); with a wave per item, an item of two dozen entries fills one batch of 8*G loads at
+// best, and the wave then spends as long combining its groups as gathering.  Measured on R-MAT graphs, forward + backward of
+// a layer: 1 x 48 floats 9.0 -> 7.6 ms at 2.4 M nodes x 26 entries per row, 9.9 -> 8.3 ms at 48 entries, 7.7 -> 7.3 ms at 128,
+// but 4.6 -> 4.8 ms at 492 (there the gathered rows hit L2 and the pair layout's single pass over the scores wins); 1 x 16
+// floats at 1 M nodes 3.2 -> 2.2 ms; 4 x 32 floats (two groups) 15.7 -> 15.1 ms at 2.4 M nodes, 1.02 -> 0.99 ms at 169 k
+// nodes, 13.9 -> 14.5 ms at 128 entries per row.
 static inline bool gat_rowpack_wanted(int pack, int64_t E, int N)
 {
     return E < (pack >= 4 ? 256 : 64) * (int64_t)N;
@@ -1386,26 +1417,24 @@ static int gat_forward_launch(int N, int64_t E, int H, int F, const float *attn_
             while ((1 << p.hp_shift) < H) ++p.hp_shift;
             // the pair layout needs 8*G entry slots x heads (rounded up to a power of two) <= 64 lanes
             const bool pair = ((8 * pack) << p.hp_shift) <= 64 && E >= 64 * (int64_t)N;
-            // the long items at the head of the list keep a wave each; the rest go four (G) to a wave on graphs of short rows
+            // the long items at the head of the list keep a wave each; the rest go G to a wave on graphs of short rows
             const int first = sched && gat_rowpack_wanted(pack, E, N) ? sched->n_wave_slots : p.n_items;
             const int bucketed = sched && sched->n_buckets > 0;
-            const unsigned grid_rp = fgnn_group_item_grid(p.n_items - first, pack, bucketed);
-            GatFwdP pw = p;
-            pw.n_items = first;
-            const unsigned grid_w = (unsigned)((first + FGNN_WPB - 1) / FGNN_WPB);
+            const unsigned head_blocks = (unsigned)((first + FGNN_WPB - 1) / FGNN_WPB);      // first is a multiple of 64, or n_items
+            const unsigned grid_mixed = head_blocks + fgnn_group_item_grid(p.n_items - first, pack, bucketed);
             auto launch = [&]<int G>() {
-                if (first < p.n_items) {
-                    if (aux && sle1) hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, true, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
-                    else if (aux) hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, true, false>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
-                    else if (sle1) hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, false, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
-                    else hipLaunchKernelGGL((gat_fwd_rowpack_kernel<G, false, false>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
-                }
-                if (first == 0) return;
                 auto go = [&]<bool PAIR>() {
-                    if (aux && sle1) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, true, PAIR>), dim3(grid_w), dim3(FGNN_TPB), 0, st, pw);
-                    else if (aux) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, false, PAIR>), dim3(grid_w), dim3(FGNN_TPB), 0, st, pw);
-                    else if (sle1) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, false, true, PAIR>), dim3(grid_w), dim3(FGNN_TPB), 0, st, pw);
-                    else hipLaunchKernelGGL((gat_fwd_packed_kernel<G, false, false, PAIR>), dim3(grid_w), dim3(FGNN_TPB), 0, st, pw);
+                    if (first < p.n_items) {
+                        if (aux && sle1) hipLaunchKernelGGL((gat_fwd_mixed_kernel<G, true, true, PAIR>), dim3(grid_mixed), dim3(FGNN_TPB), 0, st, p, bucketed, first, head_blocks);
+                        else if (aux) hipLaunchKernelGGL((gat_fwd_mixed_kernel<G, true, false, PAIR>), dim3(grid_mixed), dim3(FGNN_TPB), 0, st, p, bucketed, first, head_blocks);
+                        else if (sle1) hipLaunchKernelGGL((gat_fwd_mixed_kernel<G, false, true, PAIR>), dim3(grid_mixed), dim3(FGNN_TPB), 0, st, p, bucketed, first, head_blocks);
+                        else hipLaunchKernelGGL((gat_fwd_mixed_kernel<G, false, false, PAIR>), dim3(grid_mixed), dim3(FGNN_TPB), 0, st, p, bucketed, first, head_blocks);
+                        return;
+                    }
+                    if (aux && sle1) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, true, PAIR>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
+                    else if (aux) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, true, false, PAIR>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
+                    else if (sle1) hipLaunchKernelGGL((gat_fwd_packed_kernel<G, false, true, PAIR>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
+                    else hipLaunchKernelGGL((gat_fwd_packed_kernel<G, false, false, PAIR>), dim3(grid), dim3(FGNN_TPB), 0, st, p);
                 };
                 if (pair) go.template operator()<true>(); else go.template operator()<false>();
             };
@@ -1658,23 +1687,21 @@ static int gat_backward_impl(int N, int64_t E, int H, int F, float negative_slop
             const bool pair = ((8 * pack) << p.hp_shift) <= 64 && E >= 64 * (int64_t)N;
             const int first = sched_csc && gat_rowpack_wanted(pack, E, N) ? sched_csc->n_wave_slots : p.n_items;      // as in the forward
             const int bucketed = sched_csc && sched_csc->n_buckets > 0;
-            const unsigned grid_rp = fgnn_group_item_grid(p.n_items - first, pack, bucketed);
-            GatBwdP pw = p;
-            pw.n_items = first;
-            const unsigned grid_w = (unsigned)((first + FGNN_WPB - 1) / FGNN_WPB);
+            const unsigned head_blocks = (unsigned)((first + FGNN_WPB - 1) / FGNN_WPB);
+            const unsigned grid_mixed = head_blocks + fgnn_group_item_grid(p.n_items - first, pack, bucketed);
             auto launch = [&]<int G>() {
-                if (first < p.n_items) {
-                    if (stash_mode == 2) hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 2, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
-                    else if (stash_mode == 1) hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 1, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
-                    else if (sle1) hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 0, true>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
-                    else hipLaunchKernelGGL((gat_bwd_rowpack_kernel<G, 0, false>), dim3(grid_rp), dim3(FGNN_TPB), 0, st, p, bucketed, first);
-                }
-                if (first == 0) return;
                 auto go = [&]<bool PAIR>() {
-                    if (stash_mode == 2) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 2, true, PAIR>), dim3(grid_w), dim3(FGNN_TPB), shm, st, pw);
-                    else if (stash_mode == 1) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 1, true, PAIR>), dim3(grid_w), dim3(FGNN_TPB), shm, st, pw);
-                    else if (sle1) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 0, true, PAIR>), dim3(grid_w), dim3(FGNN_TPB), shm, st, pw);
-                    else hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 0, false, PAIR>), dim3(grid_w), dim3(FGNN_TPB), shm, st, pw);
+                    if (first < p.n_items) {
+                        if (stash_mode == 2) hipLaunchKernelGGL((gat_bwd_mixed_kernel<G, 2, true, PAIR>), dim3(grid_mixed), dim3(FGNN_TPB), shm, st, p, bucketed, first, head_blocks);
+                        else if (stash_mode == 1) hipLaunchKernelGGL((gat_bwd_mixed_kernel<G, 1, true, PAIR>), dim3(grid_mixed), dim3(FGNN_TPB), shm, st, p, bucketed, first, head_blocks);
+                        else if (sle1) hipLaunchKernelGGL((gat_bwd_mixed_kernel<G, 0, true, PAIR>), dim3(grid_mixed), dim3(FGNN_TPB), shm, st, p, bucketed, first, head_blocks);
+                        else hipLaunchKernelGGL((gat_bwd_mixed_kernel<G, 0, false, PAIR>), dim3(grid_mixed), dim3(FGNN_TPB), shm, st, p, bucketed, first, head_blocks);
+                        return;
+                    }
+                    if (stash_mode == 2) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 2, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                    else if (stash_mode == 1) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 1, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                    else if (sle1) hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 0, true, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
+                    else hipLaunchKernelGGL((gat_bwd_packed_kernel<G, 0, false, PAIR>), dim3(grid), dim3(FGNN_TPB), shm, st, p);
                 };
                 if (pair) go.template operator()<true>(); else go.template operator()<false>();
             };

@@ -682,10 +682,9 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_packed_kernel(GmmBwdP p)
 // feature matrix (aggregate first, transform afterwards): out[i,k,:] = sum_p w[p,k] * g[idx[p],:], nothing
 // per edge is written and x is not read.
 #define GMM_SUMK_MAX 4
-template <int LPF, bool GWW = true>
-__global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_sum_kernel(GmmBwdP p)
+template <int LPF, bool GWW>
+__device__ __forceinline__ void gmm_bwd_sum_item(const GmmBwdP &p, int n_head, float *lds)
 {
-    extern __shared__ float lds[];
     constexpr int G = 64 / LPF;         // rows per load instruction
     constexpr int U = G > 8 ? 64 / G : 8;       // load instructions in flight; U * G divides 64
     const int K = p.K, dim = p.dim, KD = K * dim, F = p.F;
@@ -694,7 +693,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_sum_kernel(GmmBwdP p)
     for (int i = (int)threadIdx.x; i < KD; i += FGNN_TPB) { shared[i] = p.mu[i]; shared[KD + i] = p.isg[i]; }
     __syncthreads();
     int col, b, e, slot;
-    if (!fg_get_item(p.items, p.n_items, p.ptr, col, b, e, slot)) return;
+    if (!fg_get_item(p.items, n_head, p.ptr, col, b, e, slot)) return;
     const int lane = fg_lane();
     float *wl = lds + fg_wave() * per_wave;
     const int grp = lane / LPF, sub = lane % LPF;
@@ -762,9 +761,141 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_sum_kernel(GmmBwdP p)
     }
 }
 
-template <bool GWW>
-static void gmm_sum_launch(int lpf, unsigned grid, size_t shm, hipStream_t st, const GmmBwdP &p)
+// The same pass with the lane groups on different work items (fg_group_slot): group g walks its own item LPF entries at a
+// time (its LPF lanes compute the weights of LPF entries), min(8, LPF) gathered rows of the group in flight, and writes its
+// own result; no butterfly over the groups.
+template <int LPF, bool GWW>
+__device__ __forceinline__ void gmm_bwd_sum_group_items(const GmmBwdP &p, int bucketed, int first, int w, float *lds)
 {
+    constexpr int G = 64 / LPF;
+    constexpr int U = LPF < 8 ? LPF : 8;
+    const int K = p.K, dim = p.dim, KD = K * dim, F = p.F;
+    const int per_wave = K * 64;
+    float *shared = lds + FGNN_WPB * per_wave;          // mu | inv_sigma
+    for (int i = (int)threadIdx.x; i < KD; i += FGNN_TPB) { shared[i] = p.mu[i]; shared[KD + i] = p.isg[i]; }
+    __syncthreads();
+    const int lane = fg_lane();
+    const int grp = lane / LPF, sub = lane % LPF, gbase = lane - sub;
+    const int it = fg_group_slot(G, grp, bucketed, first, w);
+    int col = -1, b = 0, e = 0, slot = -1;
+    if (it < p.n_items) {
+        if (p.items) { const fgnn_item q = p.items[it]; col = q.row; b = q.begin; e = q.end; slot = q.slot; }
+        else { col = it; b = p.ptr[it]; e = p.ptr[it + 1]; }
+    }
+    if (col < 0) { b = 0; e = 0; }                      // padding item or past the list: nothing to walk or store
+    if (__builtin_amdgcn_ballot_w64(col >= 0) == 0ull) return;
+    float *wl = lds + fg_wave() * per_wave;
+    const bool fok = sub * 4 < F;
+    const int foff = fok ? sub * 4 : 0;
+    fg_vec<4> T[GMM_SUMK_MAX], xr[GMM_SUMK_MAX];
+#pragma unroll
+    for (int k = 0; k < GMM_SUMK_MAX; ++k) {
+        T[k].zero();
+        if (GWW && k < K && fok && col >= 0) xr[k].load(p.x + (size_t)col * p.HF + k * F + foff); else xr[k].zero();
+    }
+    for (int c = b; __builtin_amdgcn_ballot_w64(c < e) != 0ull; c += LPF) {
+        const bool ok = c + sub < e;
+        const int cnt = min(LPF, e - c);                // <= 0: this group is done
+        int id = 0, posv = 0;
+        if (c < e) {
+            const int qq = ok ? c + sub : c;            // idle lanes repeat a valid entry
+            id = p.idx[qq];
+            posv = p.pos ? p.pos[qq] : qq;
+            if (p.permute) posv = p.permute[posv];
+        }
+        if (ok) {
+            const float *ps = p.pseudo + (size_t)(unsigned)posv * dim;
+            float pv[GMM_PV];
+            gmm_load_pseudo(ps, dim, pv);
+            for (int k = 0; k < K; ++k) wl[k * 64 + lane] = gmm_weight(pv, ps, shared + k * dim, shared + KD + k * dim, dim);
+        } else {
+            for (int k = 0; k < K; ++k) wl[k * 64 + lane] = 0.f;
+        }
+        fg_wave_lds_sync();
+        for (int t = 0; __builtin_amdgcn_ballot_w64(t < cnt) != 0ull; t += U) {
+            fg_vec<4> ld[U];
+            int pe[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u, src = (gbase + (ei & (LPF - 1))) << 2;
+                const int rid = __builtin_amdgcn_ds_bpermute(src, id);
+                pe[u] = __builtin_amdgcn_ds_bpermute(src, posv);
+                if (ei < cnt && fok) ld[u].load(p.g + (size_t)rid * F + foff); else ld[u].zero();
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u;
+                const bool live = ei < cnt;
+                float *gdst = p.gww + (size_t)(unsigned)pe[u] * K;
+                float mine = 0.f;                                   // lane `sub` of a row keeps the value of kernel `sub`
+#pragma unroll
+                for (int k = 0; k < GMM_SUMK_MAX; ++k) {
+                    if (k < K) {
+                        const float w = live ? wl[k * 64 + gbase + (ei & (LPF - 1))] : 0.f;
+                        T[k].fma(w, ld[u]);
+                        if constexpr (GWW) {
+                            const float sum = fg_group_sum<LPF>(ld[u].dot(xr[k]));
+                            if constexpr (LPF >= GMM_SUMK_MAX) mine = sub == k ? sum * w : mine;
+                            else if (live && sub == 0) __builtin_nontemporal_store(sum * w, gdst + k);
+                        }
+                    }
+                }
+                if constexpr (GWW && LPF >= GMM_SUMK_MAX) { if (live && sub < K) __builtin_nontemporal_store(mine, gdst + sub); }
+            }
+        }
+        fg_wave_lds_sync();
+    }
+    if (col < 0 || !fok) return;
+    float *dst = slot < 0 ? p.gfeat + (size_t)col * p.HF : p.part + (size_t)slot * spmm_pw(p.HF);
+#pragma unroll
+    for (int k = 0; k < GMM_SUMK_MAX; ++k)
+        if (k < K) T[k].store_nt(dst + k * F + foff);
+}
+
+template <int LPF, bool GWW = true>
+__global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_sum_kernel(GmmBwdP p)
+{
+    extern __shared__ float lds[];
+    gmm_bwd_sum_item<LPF, GWW>(p, p.n_items, lds);
+}
+// One launch for a list with a long head: the first head_blocks workgroups put a wave on each of the `first` leading items,
+// the others give every lane group an item of the rest; the long items then run beside the short ones.
+template <int LPF, bool GWW = true>
+__global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_sum_mixed_kernel(GmmBwdP p, int bucketed, int first, unsigned head_blocks)
+{
+    extern __shared__ float lds[];
+    if (blockIdx.x < head_blocks) gmm_bwd_sum_item<LPF, GWW>(p, first, lds);
+    else gmm_bwd_sum_group_items<LPF, GWW>(p, bucketed, first, (int)(blockIdx.x - head_blocks), lds);
+}
+
+// Where the lane-group part of a launch starts (-1: a wave per item throughout).  Groups of at most 16 lanes (F <= 64) on
+// graphs under 256 entries per row; measured with K = 3 on R-MAT graphs of 14-26 entries per row, column pass / shared-feature
+// forward: F = 64 0.329 -> 0.316 / 0.167 -> 0.124 ms at 169 k nodes, 1.35 -> 1.05 / 0.71 -> 0.61 ms at 500 k nodes;
+// K = 2, F = 16 0.211 -> 0.174 / 0.132 -> 0.082 ms at 169 k nodes, 5.9 -> 4.6 / 2.3 -> 1.7 ms at 2.4 M nodes; F = 128 (two
+// groups of 32 lanes) 9.7 -> 10.1 ms at 2.4 M nodes: not taken.
+static inline int gmm_group_items_first(const fgnn_schedule_t *sched, int lpf)
+{
+    if (!sched || lpf > 16 || sched->n_edges >= 256 * (int64_t)sched->n_rows) return -1;
+    return sched->n_wave_slots;
+}
+
+template <bool GWW>
+static void gmm_sum_launch(int lpf, unsigned grid, size_t shm, hipStream_t st, const GmmBwdP &p, int first = -1, int bucketed = 0)
+{
+    // first >= 0: the items from slot `first` on are short and go 64/lpf to a wave (gmm_bwd_sum_group_items)
+    if (first >= 0 && first < p.n_items && lpf <= 32) {
+        const unsigned hb = (unsigned)((first + FGNN_WPB - 1) / FGNN_WPB);
+        const unsigned g2 = hb + fgnn_group_item_grid(p.n_items - first, 64 / lpf, bucketed != 0);
+        switch (lpf) {
+        case 1: hipLaunchKernelGGL((gmm_bwd_sum_mixed_kernel<1, GWW>), dim3(g2), dim3(FGNN_TPB), shm, st, p, bucketed, first, hb); break;
+        case 2: hipLaunchKernelGGL((gmm_bwd_sum_mixed_kernel<2, GWW>), dim3(g2), dim3(FGNN_TPB), shm, st, p, bucketed, first, hb); break;
+        case 4: hipLaunchKernelGGL((gmm_bwd_sum_mixed_kernel<4, GWW>), dim3(g2), dim3(FGNN_TPB), shm, st, p, bucketed, first, hb); break;
+        case 8: hipLaunchKernelGGL((gmm_bwd_sum_mixed_kernel<8, GWW>), dim3(g2), dim3(FGNN_TPB), shm, st, p, bucketed, first, hb); break;
+        case 16: hipLaunchKernelGGL((gmm_bwd_sum_mixed_kernel<16, GWW>), dim3(g2), dim3(FGNN_TPB), shm, st, p, bucketed, first, hb); break;
+        default: hipLaunchKernelGGL((gmm_bwd_sum_mixed_kernel<32, GWW>), dim3(g2), dim3(FGNN_TPB), shm, st, p, bucketed, first, hb); break;
+        }
+        return;
+    }
     switch (lpf) {
     case 1: hipLaunchKernelGGL((gmm_bwd_sum_kernel<1, GWW>), dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
     case 2: hipLaunchKernelGGL((gmm_bwd_sum_kernel<2, GWW>), dim3(grid), dim3(FGNN_TPB), shm, st, p); break;
@@ -801,7 +932,7 @@ static int gmm_forward_shared(int N, int K, int dim, int F, const int32_t *ptr, 
     const size_t shm = ((size_t)FGNN_WPB * K * 64 + 2 * KD) * sizeof(float);
     FGNN_REQUIRE(shm <= 64 * 1024, FGNN_ERR_LIMIT, "fgnn_gmm_forward: K=%d, dim=%d need %zu bytes of LDS per workgroup (limit 64 KiB)", K, dim, shm);
     const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
-    gmm_sum_launch<false>(lpf, grid, shm, st, p);
+    gmm_sum_launch<false>(lpf, grid, shm, st, p, gmm_group_items_first(sched, lpf), sched && sched->n_buckets > 0);
     int rc = fgnn_launch_status("gmm_bwd_sum_kernel (forward, shared features)");
     if (rc) return rc;
     if (sched && sched->n_split > 0) {
@@ -1087,7 +1218,7 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
             const size_t shm = ((size_t)FGNN_WPB * K * 64 + 2 * KD) * sizeof(float);
             FGNN_REQUIRE(shm <= 64 * 1024, FGNN_ERR_LIMIT, "fgnn_gmm_backward: K=%d, dim=%d need %zu bytes of LDS per workgroup (limit 64 KiB)", K, dim, shm);
             p.lphp = 0;
-            gmm_sum_launch<true>(lpf, grid, shm, st, p);
+            gmm_sum_launch<true>(lpf, grid, shm, st, p, gmm_group_items_first(sched_csc, lpf), sched_csc->n_buckets > 0);
             rc = fgnn_launch_status("gmm_bwd_sum_kernel");
             if (rc) return rc;
             if (sched_csc->n_split > 0) {

@@ -15,6 +15,7 @@ struct SpmmP {
     const float *bias; const float *res;     // with sum_h: out[i,:] += bias[:] (+ res[i,:]) in the same store (either may be NULL)
     int own_order;  // != 0: per-edge arrays are indexed by the work list's own entry positions (pos is not applied)
     int ld, ldo;    // floats between consecutive rows of feat / of out when they are views of wider arrays (0: HF)
+    int scr_floats; // LDS floats per wave behind the staged weights (the sum over heads in the store): set by spmm_launch
 };
 __host__ __device__ static inline int spmm_pw(int HF) { return (HF + 3) & ~3; }
 
@@ -112,7 +113,7 @@ template <int VEC, int R, bool FULL, class WF>
 __global__ __launch_bounds__(FGNN_TPB) void spmm_kernel(SpmmP p, WF wf, int shared_floats)
 {
     extern __shared__ float lds[];
-    float *shared = lds + FGNN_WPB * (p.H * 64 + (p.sum_h ? spmm_pw(p.HF) : 0));
+    float *shared = lds + FGNN_WPB * (p.H * 64 + p.scr_floats);
     if (shared_floats > 0) {
         wf.prepare(shared, (int)threadIdx.x, p.H);
         __syncthreads();
@@ -120,7 +121,7 @@ __global__ __launch_bounds__(FGNN_TPB) void spmm_kernel(SpmmP p, WF wf, int shar
     int row, b, e, slot;
     if (!fg_get_item(p.items, p.n_items, p.ptr, row, b, e, slot)) return;
     const int lane = fg_lane();
-    float *wl = lds + fg_wave() * (p.H * 64 + (p.sum_h ? spmm_pw(p.HF) : 0));
+    float *wl = lds + fg_wave() * (p.H * 64 + p.scr_floats);
     float *scr = wl + p.H * 64;
     fg_lanemap<VEC, R> lm;
     lm.init(lane, p.HF, p.F);
@@ -225,19 +226,11 @@ __global__ __launch_bounds__(FGNN_TPB) void spmm_pair_kernel(SpmmP p, const floa
 // Rows narrower than a wave take the packed lane layout (fg_packmap): G entries of the row per load
 // instruction, one partial sum per lane group, a butterfly over the groups at the end.
 template <int G, class WF>
-__global__ __launch_bounds__(FGNN_TPB) void spmm_packed_kernel(SpmmP p, WF wf, int shared_floats)
+__device__ __forceinline__ void spmm_packed_item(const SpmmP &p, const WF &wf, const float *shared, float *wl, float *scr, int n_head)
 {
-    extern __shared__ float lds[];
-    float *shared = lds + FGNN_WPB * (p.H * 64 + (p.sum_h ? spmm_pw(p.HF) : 0));
-    if (shared_floats > 0) {
-        wf.prepare(shared, (int)threadIdx.x, p.H);
-        __syncthreads();
-    }
     int row, b, e, slot;
-    if (!fg_get_item(p.items, p.n_items, p.ptr, row, b, e, slot)) return;
+    if (!fg_get_item(p.items, n_head, p.ptr, row, b, e, slot)) return;
     const int lane = fg_lane();
-    float *wl = lds + fg_wave() * (p.H * 64 + (p.sum_h ? spmm_pw(p.HF) : 0));
-    float *scr = wl + p.H * 64;
     fg_packmap<G> pm;
     pm.init(lane, p.HF, p.F);
     fg_vec<4> T;
@@ -278,6 +271,107 @@ __global__ __launch_bounds__(FGNN_TPB) void spmm_packed_kernel(SpmmP p, WF wf, i
     } else if (lm.ok[0]) {
         T.store_nt(p.part + (size_t)slot * spmm_pw(p.HF) + pm.eoff);
     }
+}
+
+// The same with the lane groups on DIFFERENT work items (fg_group_slot): group g walks its own item 64/G entries at a time
+// (its lanes stage the weights of those entries), eight gathered rows of the group in flight, and stores its own row; nothing
+// is combined at the end.  For lists of short items: with a wave per item, a dozen entries fill a fraction of the 8*G load
+// slots of a batch.  scr: 256 floats per wave (a row per group) when the store sums over the heads.
+template <int G, class WF>
+__device__ __forceinline__ void spmm_packed_group_items(const SpmmP &p, const WF &wf, const float *shared, float *wl, float *scr, int bucketed,
+                                                        int first, int w)
+{
+    constexpr int LPR = 64 / G, U = 8;
+    const int lane = fg_lane();
+    fg_packmap<G> pm;
+    pm.init(lane, p.HF, p.F);
+    const int sl = lane & (LPR - 1), gbase = lane - sl;
+    const int it = fg_group_slot(G, pm.grp, bucketed, first, w);
+    int row = -1, b = 0, e = 0, slot = -1;
+    if (it < p.n_items) {
+        if (p.items) { const fgnn_item q = p.items[it]; row = q.row; b = q.begin; e = q.end; slot = q.slot; }
+        else { row = it; b = p.ptr[it]; e = p.ptr[it + 1]; }
+    }
+    if (row < 0) { b = 0; e = 0; }                      // padding item or past the list: nothing to walk or store
+    if (__builtin_amdgcn_ballot_w64(row >= 0) == 0ull) return;
+    fg_vec<4> T;
+    T.zero();
+    for (int c = b; __builtin_amdgcn_ballot_w64(c < e) != 0ull; c += LPR) {
+        const bool ok = c + sl < e;
+        const int cnt = min(LPR, e - c);                // <= 0: this group is done
+        int id = 0;
+        size_t pos = 0;                                 // idle lanes and finished groups name entry 0 (there is one: some group has entries)
+        if (c < e) {
+            const int qq = ok ? c + sl : c;
+            id = p.idx[qq];
+            const int orig = p.pos ? p.pos[qq] : qq;
+            pos = p.pos_map ? (size_t)p.pos_map[orig] : (size_t)orig;
+        }
+        wf.fill(wl, shared, lane, pos, ok, p.H);
+        fg_wave_lds_sync();
+        for (int t = 0; __builtin_amdgcn_ballot_w64(t < cnt) != 0ull; t += U) {
+            fg_vec<4> ld[U];
+            float wv[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u, src = gbase + (ei & (LPR - 1));
+                const bool live = ei < cnt && pm.ok;
+                const int rid = __builtin_amdgcn_ds_bpermute(src << 2, id);
+                wv[u] = live ? wl[pm.hd * 64 + src] : 0.f;
+                if (live) ld[u].load(p.feat + (size_t)rid * (size_t)p.ld + pm.eoff); else ld[u].zero();
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) T.fma(wv[u], ld[u]);
+        }
+        fg_wave_lds_sync();
+    }
+    const bool mine = pm.ok && row >= 0;
+    if (slot >= 0) {
+        if (mine) T.store_nt(p.part + (size_t)slot * spmm_pw(p.HF) + pm.eoff);
+    } else if (!p.sum_h) {
+        if (mine) T.store_nt(p.out + (size_t)row * p.ldo + pm.eoff);
+    }
+    if (p.sum_h) {                                      // as spmm_store_row, a row of scratch per group
+        float *sg = scr + pm.grp * (LPR * 4);
+        if (pm.ok) T.store(sg + pm.eoff);
+        fg_wave_lds_sync();
+        if (mine && slot < 0 && pm.eoff < p.F) {
+            fg_vec<4> acc; acc.zero();
+            for (int h = 0; h < p.H; ++h) { fg_vec<4> t; t.load(sg + h * p.F + pm.eoff); acc.add(t); }
+            if (p.res) { fg_vec<4> t; t.load(p.res + (size_t)row * p.F + pm.eoff); acc.add(t); }
+            if (p.bias) { fg_vec<4> t; t.load(p.bias + pm.eoff); acc.add(t); }
+            acc.store(p.out + (size_t)row * p.F + pm.eoff);
+        }
+        fg_wave_lds_sync();
+    }
+}
+
+template <int G, class WF>
+__global__ __launch_bounds__(FGNN_TPB) void spmm_packed_kernel(SpmmP p, WF wf, int shared_floats)
+{
+    extern __shared__ float lds[];
+    float *shared = lds + FGNN_WPB * (p.H * 64 + p.scr_floats);
+    if (shared_floats > 0) {
+        wf.prepare(shared, (int)threadIdx.x, p.H);
+        __syncthreads();
+    }
+    float *wl = lds + fg_wave() * (p.H * 64 + p.scr_floats);
+    spmm_packed_item<G, WF>(p, wf, shared, wl, wl + p.H * 64, p.n_items);
+}
+// One launch for a list with a long head: the first head_blocks workgroups put a wave on each of the `first` leading items,
+// the others give every lane group an item of the rest, so the long items run beside the short ones.
+template <int G, class WF>
+__global__ __launch_bounds__(FGNN_TPB) void spmm_packed_mixed_kernel(SpmmP p, WF wf, int shared_floats, int bucketed, int first, unsigned head_blocks)
+{
+    extern __shared__ float lds[];
+    float *shared = lds + FGNN_WPB * (p.H * 64 + p.scr_floats);
+    if (shared_floats > 0) {
+        wf.prepare(shared, (int)threadIdx.x, p.H);
+        __syncthreads();
+    }
+    float *wl = lds + fg_wave() * (p.H * 64 + p.scr_floats);
+    if (blockIdx.x < head_blocks) spmm_packed_item<G, WF>(p, wf, shared, wl, wl + p.H * 64, first);
+    else spmm_packed_group_items<G, WF>(p, wf, shared, wl, wl + p.H * 64, bucketed, first, (int)(blockIdx.x - head_blocks));
 }
 
 template <int VEC, int R>
@@ -337,12 +431,21 @@ static int spmm_launch(const char *name, SpmmP p, WF wf, int shared_floats, cons
     }
     if (p.n_items == 0) return 0;
     const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
-    const size_t shm = ((size_t)FGNN_WPB * (p.H * 64 + (p.sum_h ? spmm_pw(p.HF) : 0)) + shared_floats) * sizeof(float);
+    const int pack = fgnn_pick_pack(cfg.vec, p.HF);
+    // rows of at most 64 floats on graphs of short rows: the items behind the long head of the list go `pack` to a wave
+    // (spmm_packed_group_items; MoNet's 2 x 16 forward at 2.4 M nodes x 26 entries per row: 2.2 -> 1.6 ms)
+    const int first = (pack >= 4 && sched && sched->n_edges < 256 * (int64_t)sched->n_rows) ? sched->n_wave_slots : p.n_items;
+    const int bucketed = sched && sched->n_buckets > 0;
+    const unsigned head_blocks = (unsigned)((first + FGNN_WPB - 1) / FGNN_WPB);
+    const unsigned grid_mixed = head_blocks + fgnn_group_item_grid(p.n_items - first, pack, bucketed);
+    p.scr_floats = p.sum_h ? (first < p.n_items ? 256 : spmm_pw(p.HF)) : 0;
+    const size_t shm = ((size_t)FGNN_WPB * (p.H * 64 + p.scr_floats) + shared_floats) * sizeof(float);
     const size_t shm_merge = p.sum_h ? (size_t)FGNN_WPB * spmm_pw(p.HF) * sizeof(float) : 0;
     FGNN_REQUIRE(shm <= 64 * 1024, FGNN_ERR_LIMIT, "%s: H=%d needs %zu bytes of LDS per workgroup (limit 64 KiB)", name, p.H, shm);
-    const int pack = fgnn_pick_pack(cfg.vec, p.HF);
     return fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
-        if (pack == 8) hipLaunchKernelGGL((spmm_packed_kernel<8, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
+        if (pack == 8 && first < p.n_items) hipLaunchKernelGGL((spmm_packed_mixed_kernel<8, WF>), dim3(grid_mixed), dim3(FGNN_TPB), shm, st, p, wf, shared_floats, bucketed, first, head_blocks);
+        else if (pack == 4 && first < p.n_items) hipLaunchKernelGGL((spmm_packed_mixed_kernel<4, WF>), dim3(grid_mixed), dim3(FGNN_TPB), shm, st, p, wf, shared_floats, bucketed, first, head_blocks);
+        else if (pack == 8) hipLaunchKernelGGL((spmm_packed_kernel<8, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
         else if (pack == 4) hipLaunchKernelGGL((spmm_packed_kernel<4, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
         else if (pack == 2) hipLaunchKernelGGL((spmm_packed_kernel<2, WF>), dim3(grid), dim3(FGNN_TPB), shm, st, p, wf, shared_floats);
         else {
@@ -612,16 +715,15 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_kernel(GmmBwdP p)
 // The same pass for rows narrower than a wave, G column entries per load instruction (see
 // spmm_packed_kernel).  Needs F/4 lanes per mixture kernel to be a power of two (LPH > 0).
 template <int G, int LPH>
-__global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_packed_kernel(GmmBwdP p)
+__device__ __forceinline__ void gmm_bwd_packed_item(const GmmBwdP &p, int n_head, float *lds)
 {
-    extern __shared__ float lds[];
     const int K = p.K, dim = p.dim, KD = K * dim;
     const int per_wave = K * 64 + 64;
     float *shared = lds + FGNN_WPB * per_wave;          // mu | inv_sigma
     for (int i = (int)threadIdx.x; i < KD; i += FGNN_TPB) { shared[i] = p.mu[i]; shared[KD + i] = p.isg[i]; }
     __syncthreads();
     int col, b, e, slot;
-    if (!fg_get_item(p.items, p.n_items, p.ptr, col, b, e, slot)) return;
+    if (!fg_get_item(p.items, n_head, p.ptr, col, b, e, slot)) return;
     const int lane = fg_lane();
     float *wl = lds + fg_wave() * per_wave;
     fg_packmap<G> pm;
@@ -671,6 +773,96 @@ __global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_packed_kernel(GmmBwdP p)
     fg_pack_reduce<G>(T, lane);
     float *dst = slot < 0 ? p.gfeat + (size_t)col * p.HF : p.part + (size_t)slot * spmm_pw(p.HF);
     if (pm.ok && pm.grp == 0) T.store_nt(dst + pm.eoff);
+}
+
+// The same with the lane groups on different work items (see spmm_packed_group_items).
+template <int G, int LPH>
+__device__ __forceinline__ void gmm_bwd_packed_group_items(const GmmBwdP &p, int bucketed, int first, int w, float *lds)
+{
+    constexpr int LPR = 64 / G, U = 8;
+    const int K = p.K, dim = p.dim, KD = K * dim;
+    const int per_wave = K * 64 + 64;
+    float *shared = lds + FGNN_WPB * per_wave;          // mu | inv_sigma
+    for (int i = (int)threadIdx.x; i < KD; i += FGNN_TPB) { shared[i] = p.mu[i]; shared[KD + i] = p.isg[i]; }
+    __syncthreads();
+    const int lane = fg_lane();
+    float *wl = lds + fg_wave() * per_wave;
+    fg_packmap<G> pm;
+    if (p.lphp) pm.init_padded(lane, p.K, p.F, p.lphp); else pm.init(lane, p.HF, p.F);
+    const int sl = lane & (LPR - 1), gbase = lane - sl;
+    const int it = fg_group_slot(G, pm.grp, bucketed, first, w);
+    int col = -1, b = 0, e = 0, slot = -1;
+    if (it < p.n_items) {
+        if (p.items) { const fgnn_item q = p.items[it]; col = q.row; b = q.begin; e = q.end; slot = q.slot; }
+        else { col = it; b = p.ptr[it]; e = p.ptr[it + 1]; }
+    }
+    if (col < 0) { b = 0; e = 0; }                      // padding item or past the list: nothing to walk or store
+    if (__builtin_amdgcn_ballot_w64(col >= 0) == 0ull) return;
+    const bool mine = pm.ok && col >= 0;
+    fg_vec<4> T, xr;
+    T.zero();
+    if (mine) xr.load(p.x + (size_t)col * p.x_stride + (p.x_stride == p.HF ? pm.eoff : pm.eoff % p.F)); else xr.zero();
+    const int goff = (p.g_stride == p.HF) ? pm.eoff : pm.eoff % p.F;
+    const bool writer = pm.ok && pm.eoff % p.F == 0;
+    for (int c = b; __builtin_amdgcn_ballot_w64(c < e) != 0ull; c += LPR) {
+        const bool ok = c + sl < e;
+        const int cnt = min(LPR, e - c);                // <= 0: this group is done
+        int id = 0, posv = 0;
+        if (c < e) {
+            const int qq = ok ? c + sl : c;             // idle lanes repeat a valid entry
+            id = p.idx[qq];
+            posv = p.pos ? p.pos[qq] : qq;
+            if (p.permute) posv = p.permute[posv];
+        }
+        if (ok) {
+            const float *ps = p.pseudo + (size_t)(unsigned)posv * dim;
+            float pv[GMM_PV];
+            gmm_load_pseudo(ps, dim, pv);
+            for (int k = 0; k < K; ++k) wl[k * 64 + lane] = gmm_weight(pv, ps, shared + k * dim, shared + KD + k * dim, dim);
+        } else {
+            for (int k = 0; k < K; ++k) wl[k * 64 + lane] = 0.f;
+        }
+        fg_wave_lds_sync();
+        for (int t = 0; __builtin_amdgcn_ballot_w64(t < cnt) != 0ull; t += U) {
+            fg_vec<4> ld[U];
+            int pe[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u, src = gbase + (ei & (LPR - 1));
+                const bool live = ei < cnt && pm.ok;
+                const int rid = __builtin_amdgcn_ds_bpermute(src << 2, id);
+                pe[u] = __builtin_amdgcn_ds_bpermute(src << 2, posv);
+                if (live) ld[u].load(p.g + (size_t)rid * p.g_stride + goff); else ld[u].zero();
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u;
+                const bool live = ei < cnt && pm.ok;
+                const float wv = live ? wl[pm.hd * 64 + gbase + (ei & (LPR - 1))] : 0.f;
+                T.fma(wv, ld[u]);
+                const float sum = fg_group_sum<LPH>(ld[u].dot(xr));
+                if (live && writer) __builtin_nontemporal_store(sum * wv, p.gww + (size_t)(unsigned)pe[u] * K + pm.hd);
+            }
+        }
+        fg_wave_lds_sync();
+    }
+    if (!mine) return;
+    float *dst = slot < 0 ? p.gfeat + (size_t)col * p.HF : p.part + (size_t)slot * spmm_pw(p.HF);
+    T.store_nt(dst + pm.eoff);
+}
+
+template <int G, int LPH>
+__global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_packed_kernel(GmmBwdP p)
+{
+    extern __shared__ float lds[];
+    gmm_bwd_packed_item<G, LPH>(p, p.n_items, lds);
+}
+template <int G, int LPH>
+__global__ __launch_bounds__(FGNN_TPB) void gmm_bwd_packed_mixed_kernel(GmmBwdP p, int bucketed, int first, unsigned head_blocks)
+{
+    extern __shared__ float lds[];
+    if (blockIdx.x < head_blocks) gmm_bwd_packed_item<G, LPH>(p, first, lds);
+    else gmm_bwd_packed_group_items<G, LPH>(p, bucketed, first, (int)(blockIdx.x - head_blocks), lds);
 }
 
 // The column pass when grad_out is the gradient of the SUM over the mixture kernels ([N, F], the
@@ -1239,6 +1431,13 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
             int rc2 = fgnn_dispatch_lph(VEC == 4 ? lph : 0, [&]<int LPH>() -> int {
                 if constexpr (VEC == 4 && R == 1 && LPH > 0 && LPH <= 32) {
                     // a mixture kernel's LPH lanes must fit inside one group of 64/pack lanes
+                    // graphs of short rows: the items behind the long head of the list go `pack` to a wave (gmm_bwd_packed_group_items)
+                    const int first = (pack >= 4 && sched_csc->n_edges < 256 * (int64_t)sched_csc->n_rows) ? sched_csc->n_wave_slots : p.n_items;
+                    const int bucketed = sched_csc->n_buckets > 0;
+                    const unsigned hb = (unsigned)((first + FGNN_WPB - 1) / FGNN_WPB);
+                    const unsigned gm = hb + fgnn_group_item_grid(p.n_items - first, pack, bucketed);
+                    if (pack == 8 && LPH <= 8 && first < p.n_items) { hipLaunchKernelGGL((gmm_bwd_packed_mixed_kernel<8, (LPH <= 8 ? LPH : 1)>), dim3(gm), dim3(FGNN_TPB), shm, st, p, bucketed, first, hb); return fgnn_launch_status("gmm_bwd_packed_mixed_kernel"); }
+                    if (pack == 4 && LPH <= 16 && first < p.n_items) { hipLaunchKernelGGL((gmm_bwd_packed_mixed_kernel<4, (LPH <= 16 ? LPH : 1)>), dim3(gm), dim3(FGNN_TPB), shm, st, p, bucketed, first, hb); return fgnn_launch_status("gmm_bwd_packed_mixed_kernel"); }
                     if (pack == 8 && LPH <= 8) { hipLaunchKernelGGL((gmm_bwd_packed_kernel<8, (LPH <= 8 ? LPH : 1)>), dim3(grid), dim3(FGNN_TPB), shm, st, p); return fgnn_launch_status("gmm_bwd_packed_kernel"); }
                     if (pack == 4 && LPH <= 16) { hipLaunchKernelGGL((gmm_bwd_packed_kernel<4, (LPH <= 16 ? LPH : 1)>), dim3(grid), dim3(FGNN_TPB), shm, st, p); return fgnn_launch_status("gmm_bwd_packed_kernel"); }
                     if (pack == 2 && LPH <= 32) { hipLaunchKernelGGL((gmm_bwd_packed_kernel<2, LPH>), dim3(grid), dim3(FGNN_TPB), shm, st, p); return fgnn_launch_status("gmm_bwd_packed_kernel"); }

@@ -146,6 +146,74 @@ __global__ __launch_bounds__(FGNN_TPB) void mhsddmm_items_kernel(const fgnn_item
     sddmm_row_piece<VEC, R, FULL, LPH>(row, pb, pe, H, F, ld, ldo, lm, lane, scr, idx, pos, a, b, out);
 }
 
+// The same for rows narrower than a wave (at most 128 floats in the 128-bit layout): the wave is cut into G lane groups
+// (fg_packmap) that take G different entries of the row with the same load instruction, eight instructions in flight; a head's
+// dot product is summed inside its LPH lanes and its first lane stores it.  With one entry per instruction a row of 48 floats
+// kept 12 lanes busy (64 M entries of 1 x 48: 3.5 ms).
+template <int G, int LPH>
+__device__ __forceinline__ void sddmm_row_piece_packed(int row, int pb, int pe, int H, int F, int HF, int ld, int ldo, int lphp, int lane,
+                                                       const int *__restrict__ idx, const int *__restrict__ pos, const float *__restrict__ a,
+                                                       const float *__restrict__ b, float *__restrict__ out)
+{
+    constexpr int U = 8;
+    fg_packmap<G> pm;
+    if (lphp) pm.init_padded(lane, H, F, lphp); else pm.init(lane, HF, F);
+    fg_vec<4> ar;
+    if (pm.ok) ar.load(a + (size_t)row * ld + pm.eoff); else ar.zero();
+    const bool writer = pm.ok && pm.eoff % F == 0;
+    for (int c = pb; c < pe; c += 64) {
+        const int q = c + lane;
+        const int cnt = min(64, pe - c);
+        const int qq = q < pe ? q : c;
+        const int id = idx[qq];
+        const int pv = pos ? pos[qq] : qq;
+        for (int t = 0; t < cnt; t += U * G) {
+            fg_vec<4> lb[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u * G + pm.grp;
+                const size_t j = (size_t)(unsigned)__builtin_amdgcn_ds_bpermute((ei & 63) << 2, id);
+                if (ei < cnt && pm.ok) lb[u].load(b + j * ld + pm.eoff); else lb[u].zero();
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ei = t + u * G + pm.grp;
+                const float sum = fg_group_sum<LPH>(lb[u].dot(ar));
+                const size_t po = (size_t)(unsigned)__builtin_amdgcn_ds_bpermute((ei & 63) << 2, pv);
+                if (writer && ei < cnt) __builtin_nontemporal_store(sum, out + po * ldo + pm.hd);
+            }
+        }
+    }
+}
+
+template <int G, int LPH>
+__global__ __launch_bounds__(FGNN_TPB) void mhsddmm_packed_kernel(int N, int64_t E, int H, int F, int HF, int ld, int ldo, int lphp, const int *ptr, const int *idx,
+                                                                  const float *a, const float *b, float *out)
+{
+    const int64_t c0 = ((int64_t)blockIdx.x * FGNN_WPB + fg_wave()) * SDDMM_CHUNK;
+    if (c0 >= E) return;
+    const int c1 = fg_uni((int)min(c0 + SDDMM_CHUNK, E));
+    const int lane = fg_lane();
+    int row = fg_uni(so_row_of(ptr, 0, N - 1, (int)c0));     // ptr[row] <= c0 < ptr[row + 1]
+    int pb = fg_uni((int)c0);
+    while (pb < c1 && row < N) {
+        const int pe = min(fg_uni(ptr[row + 1]), c1);
+        if (pe > pb) sddmm_row_piece_packed<G, LPH>(row, pb, pe, H, F, HF, ld, ldo, lphp, lane, idx, nullptr, a, b, out);
+        pb = pe;
+        ++row;
+    }
+}
+
+template <int G, int LPH>
+__global__ __launch_bounds__(FGNN_TPB) void mhsddmm_packed_items_kernel(const fgnn_item *items, int n_items, int H, int F, int HF, int ld, int ldo, int lphp,
+                                                                        const int *ptr, const int *idx, const int *pos, const float *a, const float *b,
+                                                                        float *out)
+{
+    int row, pb, pe, slot;
+    if (!fg_get_item(items, n_items, ptr, row, pb, pe, slot)) return;
+    sddmm_row_piece_packed<G, LPH>(row, pb, pe, H, F, HF, ld, ldo, lphp, fg_lane(), idx, pos, a, b, out);
+}
+
 static int mhsddmm_run(const char *fn, int N, int64_t E, int H, int F, const int32_t *row_ptr, const int32_t *col_ind, const float *a,
                        const float *b, float *out, const fgnn_schedule_t *sched, hipStream_t st)
 {
@@ -177,9 +245,26 @@ static int mhsddmm_run(const char *fn, int N, int64_t E, int H, int F, const int
         const int lphp = fgnn_pad_lph(cfg.vec, hg, F);
         if (lphp) { int w = hg * lphp * 4; cfg.r = w <= 256 ? 1 : w <= 512 ? 2 : 4; cfg.full = false; }
         const int lph = lphp ? lphp : fgnn_pick_lph(cfg.vec, F);
+        // rows narrower than a wave: `pack` entries per load instruction (a head's lanes must fit inside a group of 64 / pack)
+        const int pack = lph > 0 ? fgnn_pick_pack(cfg.vec, lphp ? hg * lphp * 4 : HF) : 1;
         int rc = fgnn_dispatch_rowcfg(cfg, [&]<int VEC, int R, bool FULL>() -> int {
             return fgnn_dispatch_lph(VEC == 4 ? lph : 0, [&]<int LPH>() -> int {
                 const size_t shm = (size_t)FGNN_WPB * 64 * R * sizeof(float);
+                if constexpr (VEC == 4 && R == 1 && LPH > 0 && LPH <= 32) {
+                    auto packed = [&]<int G>() -> int {
+                        constexpr int L = LPH <= 64 / G ? LPH : 1;          // never launched with L != LPH
+                        if (sched)
+                            hipLaunchKernelGGL((mhsddmm_packed_items_kernel<G, L>), dim3(grid), dim3(FGNN_TPB), 0, st, sched->items_dev, sched->n_items, hg, F,
+                                               HF, ld, H, lphp, row_ptr, fgnn_sched_idx(sched, col_ind), fgnn_sched_pos(sched), ag, bg, og);
+                        else
+                            hipLaunchKernelGGL((mhsddmm_packed_kernel<G, L>), dim3(grid), dim3(FGNN_TPB), 0, st, N, E, hg, F, HF, ld, H, lphp, row_ptr, col_ind,
+                                               ag, bg, og);
+                        return fgnn_launch_status("mhsddmm_packed_kernel");
+                    };
+                    if (pack == 8 && LPH <= 8) return packed.template operator()<8>();
+                    if (pack == 4 && LPH <= 16) return packed.template operator()<4>();
+                    if (pack == 2 && LPH <= 32) return packed.template operator()<2>();
+                }
                 if (sched)
                     hipLaunchKernelGGL((mhsddmm_items_kernel<VEC, R, FULL, (VEC == 4 ? LPH : 0)>), dim3(grid), dim3(FGNN_TPB), shm, st, sched->items_dev,
                                        sched->n_items, hg, F, HF, ld, H, lphp, row_ptr, fgnn_sched_idx(sched, col_ind), fgnn_sched_pos(sched), ag, bg, og);

@@ -274,14 +274,14 @@ __device__ __forceinline__ void spmm_packed_item(const SpmmP &p, const WF &wf, c
 }
 
 // The same with the lane groups on DIFFERENT work items (fg_group_slot): group g walks its own item 64/G entries at a time
-// (its lanes stage the weights of those entries), eight gathered rows of the group in flight, and stores its own row; nothing
+// (its lanes stage the weights of those entries), four gathered rows of the group in flight, and stores its own row; nothing
 // is combined at the end.  For lists of short items: with a wave per item, a dozen entries fill a fraction of the 8*G load
 // slots of a batch.  scr: 256 floats per wave (a row per group) when the store sums over the heads.
 template <int G, class WF>
 __device__ __forceinline__ void spmm_packed_group_items(const SpmmP &p, const WF &wf, const float *shared, float *wl, float *scr, int bucketed,
                                                         int first, int w)
 {
-    constexpr int LPR = 64 / G, U = 8;
+    constexpr int LPR = 64 / G, U = 4;
     const int lane = fg_lane();
     fg_packmap<G> pm;
     pm.init(lane, p.HF, p.F);
@@ -779,7 +779,7 @@ __device__ __forceinline__ void gmm_bwd_packed_item(const GmmBwdP &p, int n_head
 template <int G, int LPH>
 __device__ __forceinline__ void gmm_bwd_packed_group_items(const GmmBwdP &p, int bucketed, int first, int w, float *lds)
 {
-    constexpr int LPR = 64 / G, U = 8;
+    constexpr int LPR = 64 / G, U = 4;
     const int K = p.K, dim = p.dim, KD = K * dim;
     const int per_wave = K * 64 + 64;
     float *shared = lds + FGNN_WPB * per_wave;          // mu | inv_sigma
@@ -954,13 +954,13 @@ __device__ __forceinline__ void gmm_bwd_sum_item(const GmmBwdP &p, int n_head, f
 }
 
 // The same pass with the lane groups on different work items (fg_group_slot): group g walks its own item LPF entries at a
-// time (its LPF lanes compute the weights of LPF entries), min(8, LPF) gathered rows of the group in flight, and writes its
+// time (its LPF lanes compute the weights of LPF entries), min(4, LPF) gathered rows of the group in flight, and writes its
 // own result; no butterfly over the groups.
 template <int LPF, bool GWW>
 __device__ __forceinline__ void gmm_bwd_sum_group_items(const GmmBwdP &p, int bucketed, int first, int w, float *lds)
 {
     constexpr int G = 64 / LPF;
-    constexpr int U = LPF < 8 ? LPF : 8;
+    constexpr int U = LPF < 4 ? LPF : 4;
     const int K = p.K, dim = p.dim, KD = K * dim, F = p.F;
     const int per_wave = K * 64;
     float *shared = lds + FGNN_WPB * per_wave;          // mu | inv_sigma

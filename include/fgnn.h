@@ -94,8 +94,9 @@ size_t  fgnn_schedule_device_bytes(const fgnn_schedule_t *s);
  * may be NULL. */
 int     fgnn_schedule_num_splits(const fgnn_schedule_t *s);
 /* The lists are sorted longest first: every work item at a slot >= this number has at most 64 entries (a multiple of 64
- * slots per source bucket, or fgnn_schedule_num_items).  The fused GAT on rows of at most 128 floats puts a whole wave on
- * the items before it and one lane group of a wave on each item after it.  No counterpart in the reference. */
+ * slots per source bucket, or fgnn_schedule_num_items).  On graphs of short rows the kernels for rows narrower than a wave
+ * (fused GAT up to 128 floats, multi-head SpMM and GMMConv up to 64) put a whole wave on each item before it and one lane
+ * group of a wave on each item after it, in one launch.  No counterpart in the reference. */
 int     fgnn_schedule_num_wave_slots(const fgnn_schedule_t *s);
 int     fgnn_schedule_export(const fgnn_schedule_t *s, int32_t *items_out, int32_t *splits_out, void *stream);
 

@@ -72,15 +72,13 @@ def main(argv=None):
     heads = [args.num_heads] * args.num_layers + [args.num_out_heads]
     model = GAT(VARIANTS[args.variant], args.num_layers, data.feat.shape[1], args.num_hidden, data.n_classes, heads, args.negative_slope).to(dev)
     extra = True if args.variant == "our" else g.permute
-    loss_fcn = common.cross_entropy
     opt = torch.optim.Adam(model.parameters(), lr=args.lr, weight_decay=args.weight_decay, capturable=args.hip_graph)
-    train_idx = data.train_mask.nonzero().squeeze(1)
-    train_labels = data.label[train_idx]
+    train_rows = common.MaskedRows(data.train_mask, data.label)
 
     def step():
         model.train()
         logits = model(g, data.feat, extra, keep_padding=True)
-        loss = loss_fcn(logits[train_idx], train_labels, data.n_classes)
+        loss = common.masked_cross_entropy(logits, train_rows, data.n_classes)      # the mean over logits[train_mask]
         opt.zero_grad(set_to_none=False)
         loss.backward()
         opt.step()

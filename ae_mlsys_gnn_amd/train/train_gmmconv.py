@@ -119,10 +119,8 @@ def main(argv=None):
     torch.manual_seed(args.seed)
     model = MoNet(VARIANTS[args.variant], data.feat.shape[1], args.n_hidden, data.n_classes, args.n_layers, args.pseudo_dim, args.n_kernels,
                   args.dropout).to(dev)
-    loss_fcn = common.cross_entropy
     opt = torch.optim.Adam(model.parameters(), lr=args.lr, weight_decay=args.weight_decay, capturable=args.hip_graph)
-    train_idx = data.train_mask.nonzero().squeeze(1)
-    train_labels = data.label[train_idx]
+    train_rows = common.MaskedRows(data.train_mask, data.label)
 
     def evaluate(mask):
         model.eval()
@@ -131,7 +129,7 @@ def main(argv=None):
 
     def train_step():
         model.train()
-        loss = loss_fcn(model(g, data.feat, pseudo, pseudo_csc, own_order=own_order)[train_idx], train_labels)
+        loss = common.masked_cross_entropy(model(g, data.feat, pseudo, pseudo_csc, own_order=own_order), train_rows)      # the mean over logits[train_mask]
         opt.zero_grad(set_to_none=False)
         loss.backward()
         opt.step()

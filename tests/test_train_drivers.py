@@ -242,6 +242,50 @@ def test_cross_entropy_helper_equals_torch():
     assert torch.allclose(gw, gg, atol=1e-14)
 
 
+def test_masked_cross_entropy_equals_the_loss_over_the_selected_rows():
+    """masked_cross_entropy(logits, MaskedRows(mask, labels)) = CrossEntropyLoss()(logits[mask], labels[mask]) in value
+    and gradient (zero on the unselected rows), also when an unselected row carries a placeholder label."""
+    from ae_mlsys_gnn_amd.train.common import MaskedRows, masked_cross_entropy
+    torch.manual_seed(1)
+    logits = (5 * torch.randn(300, 47, dtype=torch.float64)).requires_grad_(True)
+    y = torch.randint(0, 47, (300,))
+    mask = torch.rand(300) < 0.4
+    y_marked = torch.where(mask, y, torch.full_like(y, -1))
+    want = torch.nn.CrossEntropyLoss()(logits[mask], y[mask])
+    gw, = torch.autograd.grad(want, logits)
+    for labels in (y, y_marked):
+        got = masked_cross_entropy(logits, MaskedRows(mask, labels))
+        assert abs(float(got.detach()) - float(want.detach())) < 1e-12
+        gg, = torch.autograd.grad(got, logits)
+        assert torch.allclose(gw, gg, atol=1e-14) and float(gg[~mask].abs().max()) == 0.0
+    padded = torch.cat([logits.detach(), torch.zeros(300, 1, dtype=torch.float64)], 1)
+    assert abs(float(masked_cross_entropy(padded, MaskedRows(mask, y), 47)) - float(want.detach())) < 1e-12
+
+
+@pytest.mark.gpu
+def test_masked_cross_entropy_on_the_device():
+    """The same through the fused row pass: padded [N, 48] logits with 47 classes and a cropped view."""
+    from ae_mlsys_gnn_amd.train.common import MaskedRows, masked_cross_entropy
+    torch.manual_seed(2)
+    dev = "cuda:0"
+    n, c, width = 5000, 47, 48
+    padded = torch.zeros(n, width)
+    padded[:, :c] = 4 * torch.randn(n, c)
+    y = torch.randint(0, c, (n,))
+    mask = torch.rand(n) < 0.3
+    ref_in = padded[:, :c].double().requires_grad_(True)
+    want = torch.nn.CrossEntropyLoss()(ref_in[mask], y[mask])
+    gw, = torch.autograd.grad(want, ref_in)
+    rows = MaskedRows(mask.to(dev), torch.where(mask, y, torch.full_like(y, -1)).to(dev))
+    for crop in (False, True):
+        pd = padded.to(dev).requires_grad_(True)
+        got = masked_cross_entropy(pd[:, :c], rows) if crop else masked_cross_entropy(pd, rows, c)
+        gg, = torch.autograd.grad(got, pd)
+        assert abs(float(got) - float(want)) <= 1e-5 * max(1.0, abs(float(want)))
+        assert torch.allclose(gg[:, :c].cpu().double(), gw, rtol=1e-4, atol=1e-9)
+        assert float(gg[:, c:].abs().max()) == 0.0 and float(gg[~mask.to(dev)].abs().max()) == 0.0
+
+
 @pytest.mark.gpu
 def test_forward_latency_driver(tmp_path):
     from ae_mlsys_gnn_amd.train import forward_latency

@@ -327,6 +327,41 @@ def test_gat_random_shapes_and_graphs(seed):
     _run(g, h, f, slope=slope, seed=seed, variant=variant)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_gat_narrow_rows_random_graphs_and_lists(seed, monkeypatch):
+    """Seeded sweep over the widths that share a wave (4 .. 128 floats per row), graph kinds (R-MAT, uniform, the degree
+    ladder, short rows with a few hubs of up to 5000 entries), work-list kinds (plain or XCD-aware with several bucket
+    cut-offs), segment lengths, slopes and variants: the head of a list a wave per item, the rest a lane group per item."""
+    import random
+    import numpy as np
+    from ae_mlsys_gnn_amd import _lib
+    rnd = random.Random(7000 + seed)
+    if rnd.random() < 0.5:
+        monkeypatch.setenv("FGNN_XCD_BUCKETS", "1")
+        monkeypatch.setenv("FGNN_BUCKET_MIN_DEG", str(rnd.choice([8, 16, 64])))
+    if rnd.random() < 0.5:
+        monkeypatch.setenv("FGNN_SEG_LEN", str(rnd.choice([64, 128, 256, 1024])))
+    _lib.clear_schedule_cache()
+    h, f = rnd.choice([(1, 4), (1, 8), (2, 4), (1, 12), (3, 4), (1, 16), (2, 8), (4, 4), (1, 20), (1, 32), (2, 16), (8, 4), (1, 44), (1, 48),
+                       (3, 16), (4, 16), (1, 64), (2, 32), (3, 20), (5, 12), (1, 100), (1, 128), (2, 64), (4, 32), (8, 16), (2, 44)])
+    kind = rnd.choice(["rmat", "uniform", "degrees", "hubs", "hubs"])
+    if kind == "rmat":
+        g = graphs.rmat_graph(rnd.randrange(50, 4000), rnd.randrange(500, 60000), seed=seed)
+    elif kind == "uniform":
+        g = graphs.uniform_graph(rnd.randrange(10, 3000), rnd.randrange(10, 30000), seed=seed, self_loops=rnd.random() < 0.7)
+    elif kind == "degrees":
+        g = degree_edge_graph(n=rnd.randrange(30, 900), seed=100 + seed)
+    else:
+        n = rnd.randrange(100, 2000)
+        gen = np.random.default_rng(seed)
+        rows = [list(gen.integers(0, n, size=int(gen.integers(0, 40)))) for _ in range(n)]
+        for _ in range(rnd.randrange(1, 6)):
+            rows[rnd.randrange(n)] = list(gen.integers(0, n, size=rnd.randrange(65, 5000)))
+        g = custom_graph(rows, n)
+    _run(g, h, f, slope=rnd.choice([0.2, 0.01, 1.0, 1.5]), seed=seed, variant=rnd.choice(["sm", "stash", "fusescatter"]))
+    _lib.clear_schedule_cache()
+
+
 @pytest.mark.parametrize("dense", [False, True])
 @pytest.mark.parametrize("h,f", [(8, 32), (1, 128), (3, 20)])
 def test_gat_without_schedules_and_reference_backward_signature(h, f, dense):

@@ -446,8 +446,9 @@ __device__ __forceinline__ void gat_fwd_packed_item(const GatFwdP &p, int n_head
 }
 
 // The packed forward with the lane groups on DIFFERENT items: group g of a wave takes a work item of its own and walks it
-// alone (its LPR lanes fetch LPR ids at a time, four gathered rows of the group in flight: eight cost a wave per SIMD in registers and 4 % in time), so one load instruction
-// fetches a row for each of G destinations and nothing is combined at the end.  Per-lane scores (no pair layout).
+// alone (its LPR lanes fetch LPR ids at a time, four gathered rows of the group in flight: eight cost a wave per SIMD in
+// registers and 4 % in time), so one load instruction fetches a row for each of G destinations and nothing is combined at
+// the end.  Per-lane scores (no pair layout).
 template <int G, bool AUX, bool SLE1>
 __device__ __forceinline__ void gat_fwd_rowpack_items(const GatFwdP &p, int bucketed, int first, int w)
 {

@@ -433,7 +433,7 @@ static int spmm_launch(const char *name, SpmmP p, WF wf, int shared_floats, cons
     const unsigned grid = (unsigned)((p.n_items + FGNN_WPB - 1) / FGNN_WPB);
     const int pack = fgnn_pick_pack(cfg.vec, p.HF);
     // rows of at most 64 floats on graphs of short rows: the items behind the long head of the list go `pack` to a wave
-    // (spmm_packed_group_items; MoNet's 2 x 16 forward at 2.4 M nodes x 26 entries per row: 2.2 -> 1.6 ms)
+    // (spmm_packed_group_items; MoNet's 2 x 16 forward at 2.4 M nodes x 26 entries per row: 2.18 -> 0.94 ms)
     const int first = (pack >= 4 && sched && sched->n_edges < 256 * (int64_t)sched->n_rows) ? sched->n_wave_slots : p.n_items;
     const int bucketed = sched && sched->n_buckets > 0;
     const unsigned head_blocks = (unsigned)((first + FGNN_WPB - 1) / FGNN_WPB);
@@ -1431,7 +1431,8 @@ extern "C" int fgnn_gmm_backward(int N, int64_t E, int K, int dim, int F, const 
             int rc2 = fgnn_dispatch_lph(VEC == 4 ? lph : 0, [&]<int LPH>() -> int {
                 if constexpr (VEC == 4 && R == 1 && LPH > 0 && LPH <= 32) {
                     // a mixture kernel's LPH lanes must fit inside one group of 64/pack lanes
-                    // graphs of short rows: the items behind the long head of the list go `pack` to a wave (gmm_bwd_packed_group_items)
+                    // graphs of short rows: the items behind the long head of the list go `pack` to a wave (gmm_bwd_packed_group_items;
+                    // [N,2,16] rows at 2.4 M nodes x 26 entries per column: 2.59 -> 1.50 ms)
                     const int first = (pack >= 4 && sched_csc->n_edges < 256 * (int64_t)sched_csc->n_rows) ? sched_csc->n_wave_slots : p.n_items;
                     const int bucketed = sched_csc->n_buckets > 0;
                     const unsigned hb = (unsigned)((first + FGNN_WPB - 1) / FGNN_WPB);

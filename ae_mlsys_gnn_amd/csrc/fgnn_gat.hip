@@ -284,7 +284,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_kernel(GatFwdP p)
 // batch of 8*G, head); the wave then keeps ONE running maximum per head, so the groups' accumulators
 // are plain partial sums.
 // n_head: the items this form takes (all of them, or the head of a list whose short items go to gat_fwd_rowpack_items).
-template <int G, bool AUX, bool SLE1, bool PAIR>
+template <int G, bool AUX, bool SLE1, bool PAIR, int U = 8>
 __device__ __forceinline__ void gat_fwd_packed_item(const GatFwdP &p, int n_head)
 {
     int row, b, e, slot;
@@ -298,7 +298,7 @@ __device__ __forceinline__ void gat_fwd_packed_item(const GatFwdP &p, int n_head
     T.zero(); P.zero();
     float s = 0.f, cp = 0.f, m = -INFINITY;
     const float arh = p.ar[(size_t)row * H + pm.hd] * FGNN_LOG2E;
-    constexpr int U = 8;
+    // U: load instructions in flight
     GatFwdPair pr;
     pr.u = lane >> p.hp_shift; pr.h = lane & ((1 << p.hp_shift) - 1);
     pr.ok = PAIR && pr.h < H && pr.u < U * G;
@@ -558,7 +558,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_packed_kernel(GatFwdP p)
 template <int G, bool AUX, bool SLE1, bool PAIR>
 __global__ __launch_bounds__(FGNN_TPB) void gat_fwd_mixed_kernel(GatFwdP p, int bucketed, int first, unsigned head_blocks)
 {
-    if (blockIdx.x < head_blocks) gat_fwd_packed_item<G, AUX, SLE1, PAIR>(p, first);
+    if (blockIdx.x < head_blocks) gat_fwd_packed_item<G, AUX, SLE1, PAIR, 4>(p, first);
     else gat_fwd_rowpack_items<G, AUX, SLE1>(p, bucketed, first, (int)(blockIdx.x - head_blocks));
 }
 
@@ -1047,7 +1047,7 @@ __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_kernel(GatBwdP p)
 
 // The column pass for rows narrower than a wave: G entries of the column per load instruction
 // (see gat_fwd_packed_kernel); T, P and z are plain sums, so the groups are added by a butterfly.
-template <int G, int STASH, bool SLE1, bool PAIR>
+template <int G, int STASH, bool SLE1, bool PAIR, int U = 8>
 __device__ __forceinline__ void gat_bwd_packed_item(const GatBwdP &p, int n_head, float *lds)
 {
     int col, b, e, slot;
@@ -1061,7 +1061,7 @@ __device__ __forceinline__ void gat_bwd_packed_item(const GatBwdP &p, int n_head
     T.zero(); P.zero();
     float z = 0.f;
     const float ach = p.ac[(size_t)col * H + pm.hd];
-    constexpr int U = 8;
+    // U: load instructions in flight
     // PAIR: the attention weights are formed in the pair layout of gat_bwd_pair_batch, one lane per
     // (entry of the batch of 8*G, head)
     GatPair pr;
@@ -1269,7 +1269,7 @@ template <int G, int STASH, bool SLE1, bool PAIR>
 __global__ __launch_bounds__(FGNN_TPB) void gat_bwd_mixed_kernel(GatBwdP p, int bucketed, int first, unsigned head_blocks)
 {
     extern __shared__ float lds[];
-    if (blockIdx.x < head_blocks) gat_bwd_packed_item<G, STASH, SLE1, PAIR>(p, first, lds);
+    if (blockIdx.x < head_blocks) gat_bwd_packed_item<G, STASH, SLE1, PAIR, 4>(p, first, lds);
     else gat_bwd_rowpack_items<G, STASH, SLE1>(p, bucketed, first, (int)(blockIdx.x - head_blocks));
 }
 

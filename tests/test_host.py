@@ -79,6 +79,17 @@ def test_graph_builders():
     assert torch.equal(g.col_ind, g2.col_ind)
     deg = rp[1:] - rp[:-1]
     assert int(deg.max()) > 4 * float(deg.float().mean()), "R-MAT should be heavy tailed"
+    # the same graph with its node labels permuted: a valid sorted CSR, the same in- and out-degree multisets, one self loop
+    # per node, reproducible by seed, and the hubs no longer at the generator's ids
+    gp = graphs.rmat_graph(500, 6000, seed=1, permute_labels=True)
+    rpp, cip = gp.row_ptr.long(), gp.col_ind.long()
+    dstp = torch.repeat_interleave(torch.arange(gp.n), rpp[1:] - rpp[:-1])
+    kp = dstp * gp.n + cip
+    assert gp.n_edges == g.n_edges and bool((kp[1:] > kp[:-1]).all()) and int((dstp == cip).sum()) == gp.n
+    assert torch.equal(torch.sort(rpp[1:] - rpp[:-1]).values, torch.sort(deg).values)
+    assert torch.equal(torch.sort(torch.bincount(cip, minlength=gp.n)).values, torch.sort(torch.bincount(ci, minlength=g.n)).values)
+    assert torch.equal(gp.col_ind, graphs.rmat_graph(500, 6000, seed=1, permute_labels=True).col_ind)
+    assert not torch.equal(rpp, rp)
     pts = torch.rand(3, 50, 3)
     src = graphs.knn_graph(pts, 7).view(3, 50, 7)
     assert bool((src[:, :, 0] == torch.arange(150).view(3, 50)).all()), "nearest neighbour of a point is itself"

@@ -256,6 +256,41 @@ def test_c4_gmm_full_size_vs_oracle():
     assert_close_sum(gs, torch.from_numpy(rgs), sc["grad_sigma"], "gmm grad_sigma at C4", c=c, max_ratio=MAX_RATIO)
 
 
+def test_c4_graph_monet_widths_vs_oracle():
+    """The C4 graph with MoNet's widths (K=2, dim=1, F=16: rows of 32 floats, eight to a load instruction): the packed SpMM
+    and column pass and the passes that sum over the mixture kernels, whose short work items go a lane group each behind
+    the long head of the list, against the C oracle on every row."""
+    from ae_mlsys_gnn_amd.operators import csr2csc as csc_op
+    from ae_mlsys_gnn_amd.operators.fused_gmmconv import gmm_native
+    n, kk, dim, f = 169343, 2, 1, 16
+    g = graphs.rmat_graph(n, 2_300_000, seed=1, device=DEV)
+    g.col_ptr, g.row_ind, g.permute = csc_op.csr2csc(g.row_ptr, g.col_ind)
+    torch.manual_seed(3)
+    pseudo = torch.rand(g.n_edges, dim, device=DEV)
+    x = torch.randn(n, kk, f, device=DEV)
+    mu = torch.rand(kk, dim, device=DEV)
+    isg = 0.5 + torch.rand(kk, dim, device=DEV)
+    go = torch.randn(n, kk, f, device=DEV)
+    rp, ci = g.row_ptr.cpu().numpy(), g.col_ind.cpu().numpy()
+    args = [t.cpu().numpy() for t in (x, pseudo, mu, isg)]
+    c = c_exp(float((0.5 * (((pseudo.double().unsqueeze(1) - mu.double().unsqueeze(0)) * isg.double().unsqueeze(0)) ** 2).sum(-1)).max()))
+    for summed in (False, True):
+        gout = go[:, 0, :].contiguous() if summed else go
+        gfull = gout.unsqueeze(1).expand(-1, kk, -1).contiguous() if summed else go
+        out = gmm_native.gmmconv(g.row_ptr, g.col_ind, x, pseudo, mu, isg, sum_kernels=summed)
+        gx, gp, gm, gs = gmm_native.gmmconv_backward(g.col_ptr, g.row_ind, g.permute, x, pseudo, mu, isg, gout, sum_kernels=summed)
+        ref = c_oracle.gmm_forward(rp, ci, *args)
+        rgx, rgp, rgm, rgs = c_oracle.gmm_backward(rp, ci, *args, gfull.cpu().numpy())
+        sc = orc.gmm_abs_sums(g.row_ptr, g.col_ind, x.double(), pseudo.double(), mu.double(), isg.double(), gfull.double())
+        tag = " at the C4 graph, 2 x 16" + (" summed" if summed else "")
+        ref_out, s_out = (torch.from_numpy(ref).sum(1), sc["out"].sum(1)) if summed else (torch.from_numpy(ref), sc["out"])
+        assert_close_sum(out, ref_out, s_out, "gmm out" + tag, c=c, max_ratio=MAX_RATIO)
+        assert_close_sum(gx, torch.from_numpy(rgx), sc["grad_feat"], "gmm grad_feat" + tag, c=c, max_ratio=MAX_RATIO)
+        assert_close_sum(gp, torch.from_numpy(rgp), sc["grad_pseudo"], "gmm grad_pseudo" + tag, c=c, max_ratio=MAX_RATIO)
+        assert_close_sum(gm, torch.from_numpy(rgm), sc["grad_mu"], "gmm grad_mu" + tag, c=c, max_ratio=MAX_RATIO)
+        assert_close_sum(gs, torch.from_numpy(rgs), sc["grad_sigma"], "gmm grad_sigma" + tag, c=c, max_ratio=MAX_RATIO)
+
+
 @pytest.fixture(scope="module")
 def c5_graph():
     from ae_mlsys_gnn_amd.operators import csr2csc as csc_op
